@@ -1,0 +1,606 @@
+"""TEST INFRASTRUCTURE -- NOT PART OF THE PRODUCT.
+
+Restatement of the reference's host-side training step as it runs on its CPU backend:
+  * Tape / Variable                     packages/autograd/src/tape.ts:29-201
+  * differentiable ops + CPU fallbacks  packages/autograd/src/ops.ts:99-974
+  * initGPT / transformerBlock / gptForward (the NON-flash branch cpu_ref takes)
+                                        packages/model/src/gpt.ts:73-151, 220-333, 344-427
+  * AdamW.stepParamEntries              packages/train/src/optimizers.ts:54-115
+  * LR schedule, grad-norm, clip        packages/train/src/trainer.ts:1088-1096,1150-1159,1297,
+                                        1332-1349,1650-1656,1761-1784
+  * no-decay set                        apps/cli/src/commands/train.ts:319-331
+All tensor arithmetic goes through oracle.ref.CpuRef (C loops).  cpu_ref exposes none of the
+optional fused backend ops, so every op below takes the fallback branch the reference takes.
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass, field
+from typing import Callable, Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+
+from . import ref
+from .ref import TD, CpuRef, SeededRng, shape_size
+
+
+# ---- tape.ts ------------------------------------------------------------------------------------
+
+class Variable:
+    _next = 0
+
+    def __init__(self, data: TD, requiresGrad: bool = False):
+        self.id = Variable._next
+        Variable._next += 1
+        self.data = data
+        self.grad: Optional[TD] = None
+        self.requiresGrad = requiresGrad
+
+
+class Tape:
+    def __init__(self):
+        self.entries = []
+
+    def record(self, output, inputs, backward):
+        self.entries.append((output, inputs, backward))
+
+    def backward(self, loss: Variable, B: CpuRef, initialGrad: Optional[TD] = None):
+        """tape.ts:60-157 without the release bookkeeping (CPU arrays are garbage collected)."""
+        loss.grad = initialGrad if initialGrad is not None else B.ones(loss.data.shape, loss.data.dtype)
+        for output, inputs, bw in reversed(self.entries):
+            outGrad = output.grad
+            if outGrad is None:
+                continue
+            needs = None
+            if any(not v.requiresGrad for v in inputs):
+                needs = [v.requiresGrad for v in inputs]
+            grads = bw(outGrad, B, needs)
+            for inp, g in zip(inputs, grads):
+                if g is None or not inp.requiresGrad:
+                    continue
+                if inp.grad is not None:
+                    inp.grad = B.add(inp.grad, g)       # tape.ts:121-123 (no addInplace on cpu_ref)
+                else:
+                    inp.grad = B.clone(g)               # tape.ts:126
+            output.grad = None
+
+    def clear(self):
+        for output, _, _ in self.entries:
+            output.grad = None
+        self.entries = []
+
+
+@dataclass
+class Ctx:
+    tape: Tape
+    backend: CpuRef
+
+
+def _record(ctx: Ctx, data: TD, inputs, backward) -> Variable:
+    out = Variable(data, True)
+    ctx.tape.record(out, inputs, backward)
+    return out
+
+
+# ---- ops.ts -------------------------------------------------------------------------------------
+
+def _reduce_broadcast(B: CpuRef, grad: TD, target: Tuple[int, ...]) -> TD:
+    """ops.ts:878-900."""
+    if tuple(grad.shape) == tuple(target):
+        return grad
+    if len(target) == 0 or (len(target) == 1 and target[0] == 1 and len(grad.shape) > 1):
+        return B.sum(grad)
+    result = grad
+    while len(result.shape) > len(target):
+        result = B.sum(result, 0)
+    for i in range(len(target)):
+        if target[i] == 1 and result.shape[i] != 1:
+            result = B.sum(result, i, True)
+    return result
+
+
+def _broadcast_to(B: CpuRef, t: TD, target: Tuple[int, ...]) -> TD:
+    """ops.ts:903-929."""
+    if tuple(t.shape) == tuple(target):
+        return t
+    src = t.data.reshape(t.shape if len(t.shape) else (1,))
+    out = np.broadcast_to(src, target).astype(np.float32).reshape(-1).copy()
+    return TD(tuple(target), t.dtype, out)
+
+
+def add(ctx, a, b):
+    sa, sb = a.data.shape, b.data.shape
+    return _record(ctx, ctx.backend.add(a.data, b.data), [a, b],
+                   lambda g, B, n: [_reduce_broadcast(B, g, sa), _reduce_broadcast(B, g, sb)])
+
+
+def sub(ctx, a, b):
+    sa, sb = a.data.shape, b.data.shape
+
+    def bw(g, B, n):
+        negG = B.neg(g)
+        return [_reduce_broadcast(B, g, sa), _reduce_broadcast(B, negG, sb)]
+    return _record(ctx, ctx.backend.sub(a.data, b.data), [a, b], bw)
+
+
+def mul(ctx, a, b):
+    ad, bd = a.data, b.data
+
+    def bw(g, B, n):
+        return [_reduce_broadcast(B, B.mul(g, bd), ad.shape), _reduce_broadcast(B, B.mul(g, ad), bd.shape)]
+    return _record(ctx, ctx.backend.mul(ad, bd), [a, b], bw)
+
+
+def div(ctx, a, b):
+    ad, bd = a.data, b.data
+
+    def bw(g, B, n):
+        ga = B.div(g, bd)
+        gb = B.neg(B.div(B.mul(g, ad), B.mul(bd, bd)))
+        return [_reduce_broadcast(B, ga, ad.shape), _reduce_broadcast(B, gb, bd.shape)]
+    return _record(ctx, ctx.backend.div(ad, bd), [a, b], bw)
+
+
+def scale(ctx, a, s):
+    return _record(ctx, ctx.backend.scale(a.data, s), [a], lambda g, B, n: [B.scale(g, s)])
+
+
+def neg(ctx, a):
+    return _record(ctx, ctx.backend.neg(a.data), [a], lambda g, B, n: [B.neg(g)])
+
+
+def matmul(ctx, a, b):
+    """ops.ts:165-189 (no matmulTransposedA on cpu_ref)."""
+    ad, bd = a.data, b.data
+
+    def bw(g, B, needs):
+        ga = gb = None
+        if needs is None or needs[0]:
+            ga = B.matmul(g, B.transpose(bd, len(bd.shape) - 2, len(bd.shape) - 1))
+        if needs is None or needs[1]:
+            gb = B.matmul(B.transpose(ad, len(ad.shape) - 2, len(ad.shape) - 1), g)
+        return [ga, gb]
+    return _record(ctx, ctx.backend.matmul(ad, bd), [a, b], bw)
+
+
+def matmulTransposed(ctx, a, b):
+    """ops.ts:197-234, fallback branch: transpose(b) then matmul; dB = transpose(g) @ a."""
+    ad, bd = a.data, b.data
+    B0 = ctx.backend
+    tB = B0.transpose(bd, len(bd.shape) - 2, len(bd.shape) - 1)
+
+    def bw(g, B, needs):
+        ga = gb = None
+        if needs is None or needs[0]:
+            ga = B.matmul(g, bd)
+        if needs is None or needs[1]:
+            gb = B.matmul(B.transpose(g, len(g.shape) - 2, len(g.shape) - 1), ad)
+        return [ga, gb]
+    return _record(ctx, B0.matmul(ad, tB), [a, b], bw)
+
+
+def matmulTransposedGelu(ctx, a, b):
+    """ops.ts:426-487, fallback branches."""
+    ad, bd = a.data, b.data
+    B0 = ctx.backend
+    tB = B0.transpose(bd, len(bd.shape) - 2, len(bd.shape) - 1)
+    mm = B0.matmul(ad, tB)
+
+    def bw(g, B, needs):
+        dMM = ref.gelu_backward(mm, g, fused=True)
+        ga = gb = None
+        if needs is None or needs[0]:
+            ga = B.matmul(dMM, bd)
+        if needs is None or needs[1]:
+            gb = B.matmul(B.transpose(dMM, len(dMM.shape) - 2, len(dMM.shape) - 1), ad)
+        return [ga, gb]
+    return _record(ctx, B0.gelu(mm), [a, b], bw)
+
+
+def sum_(ctx, a, axis=None, keepdims=False):
+    sa = a.data.shape
+    return _record(ctx, ctx.backend.sum(a.data, axis, keepdims), [a], lambda g, B, n: [_broadcast_to(B, g, sa)])
+
+
+def mean(ctx, a, axis=None, keepdims=False):
+    sa = a.data.shape
+    n_ = sa[axis + len(sa) if axis is not None and axis < 0 else axis] if axis is not None else shape_size(sa)
+    return _record(ctx, ctx.backend.mean(a.data, axis, keepdims), [a],
+                   lambda g, B, n: [B.scale(_broadcast_to(B, g, sa), 1 / n_)])
+
+
+def exp(ctx, a):
+    out = ctx.backend.exp(a.data)
+    return _record(ctx, out, [a], lambda g, B, n: [B.mul(g, out)])
+
+
+def log(ctx, a):
+    ad = a.data
+    return _record(ctx, ctx.backend.log(ad), [a], lambda g, B, n: [B.div(g, ad)])
+
+
+def relu(ctx, a):
+    ad = a.data
+    return _record(ctx, ctx.backend.relu(ad), [a], lambda g, B, n: [ref.relu_backward(ad, g)])
+
+
+def clamp(ctx, a, lo, hi):
+    ad = a.data
+    return _record(ctx, ctx.backend.clamp(ad, lo, hi), [a], lambda g, B, n: [ref.clamp_backward(ad, g, lo, hi)])
+
+
+def softCap(ctx, a, cap):
+    """ops.ts:329-340: composed tanh via exp(2x/cap) clamped to [-80, 80]."""
+    xs = scale(ctx, a, 2 / cap)
+    xc = clamp(ctx, xs, -80, 80)
+    e2x = exp(ctx, xc)
+    ones = Variable(ctx.backend.ones(e2x.data.shape, e2x.data.dtype), False)
+    numer = sub(ctx, e2x, ones)
+    denom = add(ctx, e2x, ones)
+    return scale(ctx, div(ctx, numer, denom), cap)
+
+
+def silu(ctx, a):
+    ad = a.data
+    return _record(ctx, ctx.backend.silu(ad), [a], lambda g, B, n: [ref.silu_backward(ad, g)])
+
+
+def siluMul(ctx, a, b):
+    """ops.ts:364-399 fallback: silu(a)*b; da = siluBackwardCPU(a, g*b), db = g*silu(a)."""
+    ad, bd = a.data, b.data
+    B0 = ctx.backend
+    sa = B0.silu(ad)
+
+    def bw(g, B, n):
+        ga = B.mul(g, bd)
+        return [ref.silu_backward(ad, ga), B.mul(g, sa)]
+    return _record(ctx, B0.mul(sa, bd), [a, b], bw)
+
+
+def gelu(ctx, a):
+    ad = a.data
+    return _record(ctx, ctx.backend.gelu(ad), [a], lambda g, B, n: [ref.gelu_backward(ad, g, fused=False)])
+
+
+def embedding(ctx, weight, indices: TD):
+    wd = weight.data
+    return _record(ctx, ctx.backend.embedding(wd, indices), [weight],
+                   lambda g, B, n: [ref.embedding_backward(indices, g, wd.shape[0])])
+
+
+def layerNorm(ctx, x, weight, bias, eps):
+    xd, wd = x.data, weight.data
+    return _record(ctx, ctx.backend.layerNorm(xd, wd, bias.data, eps), [x, weight, bias],
+                   lambda g, B, n: list(ref.layernorm_backward(xd, wd, g, eps)))
+
+
+def softmax(ctx, a, axis=None):
+    """ops.ts:688-700."""
+    out = ctx.backend.softmax(a.data, axis)
+
+    def bw(g, B, n):
+        sg = B.mul(out, g)
+        sumSg = B.sum(sg, -1 if axis is None else axis, True)
+        diff = B.sub(g, _broadcast_to(B, sumSg, out.shape))
+        return [B.mul(out, diff)]
+    return _record(ctx, out, [a], bw)
+
+
+def crossEntropy(ctx, logits, targets: TD):
+    ld = logits.data
+    return _record(ctx, ctx.backend.crossEntropy(ld, targets), [logits],
+                   lambda g, B, n: [ref.cross_entropy_backward(ld, targets, float(g.data[0]))])
+
+
+def slice_(ctx, a, starts, ends):
+    """ops.ts:775-809, zero-pad fallback (equals scatterSlice: same zero-filled placement)."""
+    orig = tuple(a.data.shape)
+    return _record(ctx, ctx.backend.slice(a.data, starts, ends), [a],
+                   lambda g, B, n: [B.scatterSlice(g, orig, starts, ends)])
+
+
+def sliceQkv(ctx, a):
+    rows, cols3 = a.data.shape
+    D = cols3 // 3
+    return (slice_(ctx, a, [0, 0], [rows, D]), slice_(ctx, a, [0, D], [rows, 2 * D]),
+            slice_(ctx, a, [0, 2 * D], [rows, 3 * D]))
+
+
+def reshape(ctx, a, shape):
+    orig = a.data.shape
+    return _record(ctx, ctx.backend.reshape(a.data, shape), [a], lambda g, B, n: [B.reshape(g, orig)])
+
+
+def transpose(ctx, a, d0, d1):
+    return _record(ctx, ctx.backend.transpose(a.data, d0, d1), [a], lambda g, B, n: [B.transpose(g, d0, d1)])
+
+
+def residualDropoutAdd(ctx, residual, projected, p, training):
+    if not training or p == 0:
+        return add(ctx, residual, projected)        # ops.ts:624
+    raise NotImplementedError("dropout > 0 is outside the measured configurations")
+
+
+# ---- gpt.ts -------------------------------------------------------------------------------------
+
+@dataclass
+class ModelConfig:
+    vocabSize: int
+    blockSize: int
+    nLayer: int
+    nEmbd: int
+    nHead: int
+    dropout: float = 0.0
+    ffnActivation: str = "gelu"
+    ffnDim: Optional[int] = None
+    softCap: Optional[float] = None
+
+
+def _init_weight(rng: SeededRng, shape, std) -> Variable:
+    return Variable(TD(tuple(shape), "f32", rng.fill_gauss(shape_size(shape), std)), True)
+
+
+def initGPT(cfg: ModelConfig, B: CpuRef, rng: SeededRng) -> dict:
+    """gpt.ts:73-151.  Draw order: wte, wpe, per layer (mlp weights FIRST, then wqkv, wo), lmHead."""
+    V, T, L, Cc = cfg.vocabSize, cfg.blockSize, cfg.nLayer, cfg.nEmbd
+    act = cfg.ffnActivation or "gelu"
+    std = 0.02
+    wte = _init_weight(rng, [V, Cc], std)
+    wpe = _init_weight(rng, [T, Cc], std)
+    ffn = cfg.ffnDim or (math.ceil((8 / 3) * Cc / 64) * 64 if act == "swiglu" else 4 * Cc)
+    layers = []
+    for _ in range(L):
+        if act == "swiglu":
+            mlp = {"fc_gate": _init_weight(rng, [ffn, Cc], std), "fc_up": _init_weight(rng, [ffn, Cc], std),
+                   "fc_proj": _init_weight(rng, [Cc, ffn], std / math.sqrt(2 * L))}
+        else:
+            mlp = {"fc1": _init_weight(rng, [ffn, Cc], std), "fc2": _init_weight(rng, [Cc, ffn], std / math.sqrt(2 * L))}
+            if act == "universal":
+                mlp["act_gate"] = Variable(B.full([1, ffn], 1.0), True)
+                mlp["act_skip"] = Variable(B.full([1, ffn], 0.0), True)
+            elif act == "kan_spline":
+                for k, v in (("kan_c0", 0.5), ("kan_c1", 0.0), ("kan_c2", 0.5), ("kan_c3", 0.0), ("kan_c4", 0.0)):
+                    mlp[k] = Variable(B.full([1, ffn], v), True)
+        layers.append({
+            "ln1": {"weight": Variable(B.ones([Cc]), True), "bias": Variable(B.zeros([Cc]), True)},
+            "attn": {"wqkv": _init_weight(rng, [3 * Cc, Cc], std), "wo": _init_weight(rng, [Cc, Cc], std / math.sqrt(2 * L))},
+            "ln2": {"weight": Variable(B.ones([Cc]), True), "bias": Variable(B.zeros([Cc]), True)},
+            "mlp": mlp,
+        })
+    lnF = {"weight": Variable(B.ones([Cc]), True), "bias": Variable(B.zeros([Cc]), True)}
+    lmHead = _init_weight(rng, [V, Cc], std)
+    return {"wte": wte, "wpe": wpe, "layers": layers, "lnF": lnF, "lmHead": lmHead}
+
+
+def collectParamEntries(params: dict) -> List[Tuple[str, Variable]]:
+    """gpt.ts:433-468."""
+    e = [("wte", params["wte"]), ("wpe", params["wpe"]), ("lmHead", params["lmHead"]),
+         ("lnF.weight", params["lnF"]["weight"]), ("lnF.bias", params["lnF"]["bias"])]
+    for i, l in enumerate(params["layers"]):
+        e += [(f"layer.{i}.ln1.weight", l["ln1"]["weight"]), (f"layer.{i}.ln1.bias", l["ln1"]["bias"]),
+              (f"layer.{i}.attn.wqkv", l["attn"]["wqkv"]), (f"layer.{i}.attn.wo", l["attn"]["wo"]),
+              (f"layer.{i}.ln2.weight", l["ln2"]["weight"]), (f"layer.{i}.ln2.bias", l["ln2"]["bias"])]
+        m = l["mlp"]
+        if "fc_gate" in m:
+            e += [(f"layer.{i}.mlp.fc_gate", m["fc_gate"]), (f"layer.{i}.mlp.fc_up", m["fc_up"]),
+                  (f"layer.{i}.mlp.fc_proj", m["fc_proj"])]
+        else:
+            e += [(f"layer.{i}.mlp.fc1", m["fc1"]), (f"layer.{i}.mlp.fc2", m["fc2"])]
+        for k in ("act_gate", "act_skip", "kan_c0", "kan_c1", "kan_c2", "kan_c3", "kan_c4"):
+            if k in m:
+                e.append((f"layer.{i}.mlp.{k}", m[k]))
+    return e
+
+
+def _transformer_block(ctx, x, layer, cfg: ModelConfig, Bt, T, mask: TD, training):
+    """gpt.ts:220-333, the branch taken when backend.flashAttention is absent (cpu_ref)."""
+    H, Cc = cfg.nHead, cfg.nEmbd
+    D = Cc // H
+    ln1 = layerNorm(ctx, x, layer["ln1"]["weight"], layer["ln1"]["bias"], 1e-5)
+    qkv = matmulTransposed(ctx, reshape(ctx, ln1, [Bt * T, Cc]), layer["attn"]["wqkv"])
+    qF, kF, vF = sliceQkv(ctx, qkv)
+    q = reshape(ctx, qF, [Bt, T, Cc])
+    k = reshape(ctx, kF, [Bt, T, Cc])
+    v = reshape(ctx, vF, [Bt, T, Cc])
+    cap = cfg.softCap if cfg.softCap is not None else 30.0
+    qH = transpose(ctx, reshape(ctx, q, [Bt, T, H, D]), 1, 2)
+    kH = transpose(ctx, reshape(ctx, k, [Bt, T, H, D]), 1, 2)
+    vH = transpose(ctx, reshape(ctx, v, [Bt, T, H, D]), 1, 2)
+    kT = transpose(ctx, kH, 2, 3)
+    raw = scale(ctx, matmul(ctx, qH, kT), 1 / math.sqrt(D))
+    scores = softCap(ctx, raw, cap)
+    masked = Variable(ctx.backend.maskedFill(scores.data, mask, -1e9), True)
+    ctx.tape.record(masked, [scores], lambda g, B, n: [B.maskedFill(g, mask, 0)])
+    att = softmax(ctx, masked, -1)
+    out = matmul(ctx, att, vH)           # dropout p=0 is the identity (ops.ts:574)
+    concat = reshape(ctx, transpose(ctx, out, 1, 2), [Bt * T, Cc])
+    proj = reshape(ctx, matmulTransposed(ctx, concat, layer["attn"]["wo"]), [Bt, T, Cc])
+    x = residualDropoutAdd(ctx, x, proj, cfg.dropout, training)
+
+    ln2 = layerNorm(ctx, x, layer["ln2"]["weight"], layer["ln2"]["bias"], 1e-5)
+    flat = reshape(ctx, ln2, [Bt * T, Cc])
+    act = cfg.ffnActivation or "gelu"
+    m = layer["mlp"]
+    if act == "swiglu":
+        gate = matmulTransposed(ctx, flat, m["fc_gate"])
+        up = matmulTransposed(ctx, flat, m["fc_up"])
+        mlpH = matmulTransposed(ctx, siluMul(ctx, gate, up), m["fc_proj"])
+    elif act == "universal":
+        h = matmulTransposed(ctx, flat, m["fc1"])
+        h_act = add(ctx, mul(ctx, silu(ctx, h), m["act_gate"]), mul(ctx, h, m["act_skip"]))
+        mlpH = matmulTransposed(ctx, h_act, m["fc2"])
+    elif act == "kan_spline":
+        h = matmulTransposed(ctx, flat, m["fc1"])
+        hs = mul(ctx, silu(ctx, h), m["kan_c0"])
+        hr = mul(ctx, relu(ctx, h), m["kan_c1"])
+        hg = mul(ctx, gelu(ctx, h), m["kan_c2"])
+        hi = mul(ctx, h, m["kan_c3"])
+        hq = mul(ctx, mul(ctx, h, h), m["kan_c4"])
+        h_act = add(ctx, add(ctx, add(ctx, add(ctx, hs, hr), hg), hi), hq)
+        mlpH = matmulTransposed(ctx, h_act, m["fc2"])
+    elif act == "silu":
+        mlpH = matmulTransposed(ctx, silu(ctx, matmulTransposed(ctx, flat, m["fc1"])), m["fc2"])
+    elif act == "relu":
+        mlpH = matmulTransposed(ctx, relu(ctx, matmulTransposed(ctx, flat, m["fc1"])), m["fc2"])
+    else:
+        mlpH = matmulTransposed(ctx, matmulTransposedGelu(ctx, flat, m["fc1"]), m["fc2"])
+    return residualDropoutAdd(ctx, x, reshape(ctx, mlpH, [Bt, T, Cc]), cfg.dropout, training)
+
+
+def gptForward(cfg: ModelConfig, params: dict, B: CpuRef, tape: Tape, tokens: TD, targets: Optional[TD] = None,
+               training: bool = False):
+    """gpt.ts:344-427."""
+    ctx = Ctx(tape, B)
+    Bt, T = tokens.shape
+    tok = embedding(ctx, params["wte"], tokens)
+    pos = TD((Bt, T), "i32", np.tile(np.arange(T, dtype=np.int32), Bt))
+    x = add(ctx, tok, embedding(ctx, params["wpe"], pos))
+    mask = B.causalMask(T)
+    for layer in params["layers"]:
+        x = _transformer_block(ctx, x, layer, cfg, Bt, T, mask, training)
+    x = layerNorm(ctx, x, params["lnF"]["weight"], params["lnF"]["bias"], 1e-5)
+    flat = reshape(ctx, x, [Bt * T, cfg.nEmbd])
+    logits = reshape(ctx, matmulTransposed(ctx, flat, params["lmHead"]), [Bt, T, cfg.vocabSize])
+    loss = None
+    if targets is not None:
+        tf = TD((Bt * T,), "i32", targets.data)
+        loss = crossEntropy(ctx, reshape(ctx, logits, [Bt * T, cfg.vocabSize]), tf)
+    return logits, loss
+
+
+# ---- optimizers.ts / trainer.ts -----------------------------------------------------------------
+
+def no_decay_names(nLayer: int) -> set:
+    """apps/cli/src/commands/train.ts:319-331 ("lmHead.weight" never matches -> lmHead IS decayed)."""
+    s = {"wte", "wpe", "lnF.weight", "lnF.bias", "lmHead.weight"}
+    for i in range(nLayer):
+        s |= {f"layer.{i}.ln1.weight", f"layer.{i}.ln1.bias", f"layer.{i}.ln2.weight", f"layer.{i}.ln2.bias"}
+    return s
+
+
+class AdamW:
+    """optimizers.ts:21-115 (CPU loop branch)."""
+
+    def __init__(self, lr=3e-4, beta1=0.9, beta2=0.999, eps=1e-8, weightDecay=0.01, noDecayNames=None):
+        self.lr, self.beta1, self.beta2, self.eps, self.wd = lr, beta1, beta2, eps, weightDecay
+        self.noDecay = noDecayNames or set()
+        self._step = 0
+        self._b1p = 1.0
+        self._b2p = 1.0
+        self.m: Dict[str, np.ndarray] = {}
+        self.v: Dict[str, np.ndarray] = {}
+
+    def setLr(self, lr):
+        self.lr = lr
+
+    def stepParamEntries(self, entries, gradScale=1.0):
+        self._step += 1
+        self._b1p *= self.beta1
+        self._b2p *= self.beta2
+        bc1, bc2 = 1 - self._b1p, 1 - self._b2p
+        for name, var in entries:
+            if var.grad is None:
+                continue
+            if name not in self.m:
+                self.m[name] = np.zeros(var.data.data.size, dtype=np.float32)
+                self.v[name] = np.zeros(var.data.data.size, dtype=np.float32)
+            wd = 0.0 if name in self.noDecay else self.wd
+            ref.adamw_step(var.data, var.grad, self.m[name], self.v[name], self.lr, self.beta1, self.beta2,
+                           self.eps, wd, bc1, bc2, gradScale)
+
+
+@dataclass
+class TrainConfig:
+    iters: int = 1
+    lr: float = 3e-4
+    lrMin: float = 0.0
+    warmupIters: int = 0
+    beta1: float = 0.9
+    beta2: float = 0.95
+    eps: float = 1e-8
+    weightDecay: float = 0.1
+    gradClip: float = 1.0
+    gradAccumSteps: int = 1
+
+
+def lr_at(tc: TrainConfig, step: int) -> float:
+    """trainer.ts:1088-1096,1150-1159 (runtimeLrScale = 1)."""
+    warmup = tc.warmupIters if tc.warmupIters > 0 else (0 if tc.warmupIters < 0 else min(2000, tc.iters // 5))
+    lrMin = tc.lr / 10 if (tc.lrMin or 0) == 0 else tc.lrMin
+    denom = max(1, tc.iters - warmup)
+    if step < warmup:
+        base = lrMin + (tc.lr - lrMin) * (step + 1) / warmup
+    else:
+        decay = (step - warmup) / denom
+        base = lrMin + (tc.lr - lrMin) * 0.5 * (1 + math.cos(math.pi * decay))
+    return max(lrMin * 0.1, base)
+
+
+@dataclass
+class StepResult:
+    loss: float
+    gradNorm: float
+    clipCoef: float
+    lr: float
+
+
+class Trainer:
+    """The arithmetic of one optimizer step of train() (trainer.ts:1146-1784); telemetry omitted."""
+
+    def __init__(self, cfg: ModelConfig, tc: TrainConfig, seed: int = 0):
+        self.cfg, self.tc = cfg, tc
+        self.B = CpuRef()
+        self.rng = SeededRng(seed)
+        self.params = initGPT(cfg, self.B, self.rng)
+        self.entries = collectParamEntries(self.params)
+        self.opt = AdamW(tc.lr, tc.beta1, tc.beta2, tc.eps, tc.weightDecay, no_decay_names(cfg.nLayer))
+        self.tape = Tape()
+        self.step_idx = 0
+
+    def forward_backward(self, inputs: TD, targets: TD) -> float:
+        _, loss = gptForward(self.cfg, self.params, self.B, self.tape, inputs, targets, True)
+        self.tape.backward(loss, self.B)
+        val = float(loss.data.data[0])
+        self.tape.clear()
+        return val
+
+    def step(self, batches: Sequence[Tuple[TD, TD]]) -> StepResult:
+        tc = self.tc
+        lr = lr_at(tc, self.step_idx)
+        self.opt.setLr(lr)
+        accum = len(batches)
+        loss_val = 0.0
+        if accum == 1:
+            loss_val = self.forward_backward(*batches[0])
+        else:  # trainer.ts:1208-1223: f32 scale by 1/accum then f32 add
+            acc = None
+            for inp, tgt in batches:
+                lv = TD((), "f32", np.array([self.forward_backward(inp, tgt)], dtype=np.float32))
+                s = self.B.scale(lv, 1 / accum)
+                acc = s if acc is None else self.B.add(acc, s)
+            loss_val = float(acc.data[0])
+        gradScale = 1.0 / accum
+        sq = 0.0
+        for _, v in self.entries:
+            if v.grad is not None:
+                sq += ref.sum_sq(v.grad)
+        gradNorm = math.sqrt(sq) * abs(gradScale)
+        clip, eff = 1.0, gradScale
+        if tc.gradClip > 0 and gradNorm > tc.gradClip:
+            clip = tc.gradClip / gradNorm
+            eff *= clip
+        self.opt.stepParamEntries(self.entries, eff)
+        for _, v in self.entries:
+            v.grad = None
+        self.step_idx += 1
+        return StepResult(loss_val, gradNorm, clip, lr)
+
+
+def synthetic_batch(seed: int, Bt: int, T: int, vocab: int) -> Tuple[TD, TD]:
+    """Uniform token ids: rng=SeededRng(seed); B*(T+1) draws floor(next()*vocab); row b takes draws
+    [b*(T+1), (b+1)*(T+1)); inputs = first T, targets = last T (shift by one, as data.ts:110-114)."""
+    rng = SeededRng(seed)
+    u = rng.fill_uniform(Bt * (T + 1))
+    ids = np.floor(u * vocab).astype(np.int32).reshape(Bt, T + 1)
+    return (TD((Bt, T), "i32", np.ascontiguousarray(ids[:, :T]).reshape(-1)),
+            TD((Bt, T), "i32", np.ascontiguousarray(ids[:, 1:]).reshape(-1)))

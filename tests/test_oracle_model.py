@@ -1,0 +1,192 @@
+"""Pins the oracle's model-level restatement (RNG stream, init order, full forward/backward, trainer
+step arithmetic) against independent computations: a big-int Python xorshift, PyTorch float64
+autograd of the same network, and closed forms.  No GPU."""
+import math
+
+import numpy as np
+import torch
+import torch.nn.functional as F
+
+from oracle import ref
+from oracle import ref_model as rm
+
+
+def _py_rng_stream(seed, n):
+    """Independent restatement of the int32 xorshift in arbitrary-precision ints
+    (packages/core/src/rng.ts:13-50)."""
+    M = 0xFFFFFFFF
+
+    def i32(x):
+        x &= M
+        return x - (1 << 32) if x >> 31 else x
+    s0, s1 = i32(seed), i32(seed ^ 0xDEADBEEF)
+    out = []
+    for i in range(n + 20):
+        a, b = s0 & M, s1 & M
+        s0 = i32(b)
+        a ^= (a << 23) & M
+        a ^= a >> 17
+        a ^= b
+        a ^= b >> 26
+        s1 = i32(a)
+        if i >= 20:
+            out.append(((s0 + s1) & M) / 4294967296.0)
+    return out
+
+
+def test_rng_integer_stream_bit_exact():
+    for seed in (0, 1, 42, 123, -7, 2**31 - 1):
+        r = ref.SeededRng(seed)
+        got = [r.next() for _ in range(500)]
+        assert got == _py_rng_stream(seed, 500)
+        assert all(0 <= v < 1 for v in got)
+    assert ref.SeededRng(1).next() != ref.SeededRng(2).next()      # rng.test.ts:32-38
+
+
+def test_rng_gauss_polar_with_spare():
+    r = ref.SeededRng(42)
+    u = iter(_py_rng_stream(42, 4000))
+    want = []
+    while len(want) < 1000:
+        while True:
+            a, b = next(u) * 2 - 1, next(u) * 2 - 1
+            s = a * a + b * b
+            if not (s >= 1 or s == 0):
+                break
+        m = math.sqrt(-2.0 * math.log(s) / s)
+        want += [a * m, b * m]
+    got = [r.nextGauss() for _ in range(1000)]
+    assert np.allclose(got, want, rtol=1e-15, atol=0)
+    assert abs(np.mean([ref.SeededRng(42).nextGauss() for _ in range(1)])) < 10
+    r2 = ref.SeededRng(42)
+    assert abs(sum(r2.nextGauss() for _ in range(10000)) / 10000) < 0.1   # rng.test.ts:24-30
+
+
+def test_init_order_and_std():
+    cfg = rm.ModelConfig(vocabSize=11, blockSize=5, nLayer=2, nEmbd=8, nHead=2)
+    p = rm.initGPT(cfg, ref.CpuRef(), ref.SeededRng(0))
+    r = ref.SeededRng(0)
+    C_, Fd, L = 8, 32, 2
+    draws = lambda n, std: r.fill_gauss(n, std)
+    assert np.array_equal(p["wte"].data.data, draws(11 * C_, 0.02))
+    assert np.array_equal(p["wpe"].data.data, draws(5 * C_, 0.02))
+    for l in p["layers"]:   # mlp is built before the attention weights (gpt.ts:89-144)
+        assert np.array_equal(l["mlp"]["fc1"].data.data, draws(Fd * C_, 0.02))
+        assert np.array_equal(l["mlp"]["fc2"].data.data, draws(C_ * Fd, 0.02 / math.sqrt(2 * L)))
+        assert np.array_equal(l["attn"]["wqkv"].data.data, draws(3 * C_ * C_, 0.02))
+        assert np.array_equal(l["attn"]["wo"].data.data, draws(C_ * C_, 0.02 / math.sqrt(2 * L)))
+        assert np.all(l["ln1"]["weight"].data.data == 1) and np.all(l["ln2"]["bias"].data.data == 0)
+    assert np.array_equal(p["lmHead"].data.data, draws(11 * C_, 0.02))
+    names = [n for n, _ in rm.collectParamEntries(p)]
+    assert names[:5] == ["wte", "wpe", "lmHead", "lnF.weight", "lnF.bias"]
+    assert names[5:13] == [f"layer.0.{s}" for s in ("ln1.weight", "ln1.bias", "attn.wqkv", "attn.wo", "ln2.weight",
+                                                   "ln2.bias", "mlp.fc1", "mlp.fc2")]
+    assert "lmHead" not in rm.no_decay_names(2) and "wte" in rm.no_decay_names(2)
+
+
+def _torch_forward(cfg, P, tokens, targets, cap=30.0):
+    """The same network in PyTorch float64 (library ops; independent of the oracle's loops)."""
+    Bt, T = tokens.shape
+    H, Cc = cfg.nHead, cfg.nEmbd
+    D = Cc // H
+    x = P["wte"][tokens] + P["wpe"][torch.arange(T)][None]
+    mask = torch.triu(torch.ones(T, T, dtype=torch.bool), 1)
+    for i in range(cfg.nLayer):
+        g = lambda s: P[f"layer.{i}.{s}"]
+        h = F.layer_norm(x, (Cc,), g("ln1.weight"), g("ln1.bias"), 1e-5)
+        qkv = h.reshape(Bt * T, Cc) @ g("attn.wqkv").T
+        q, k, v = [t.reshape(Bt, T, H, D).transpose(1, 2) for t in qkv.split(Cc, dim=1)]
+        s = (q @ k.transpose(2, 3)) / math.sqrt(D)
+        s = cap * torch.tanh(s / cap)
+        s = s.masked_fill(mask, -1e9)
+        a = torch.softmax(s, -1) @ v
+        x = x + (a.transpose(1, 2).reshape(Bt * T, Cc) @ g("attn.wo").T).reshape(Bt, T, Cc)
+        h = F.layer_norm(x, (Cc,), g("ln2.weight"), g("ln2.bias"), 1e-5).reshape(Bt * T, Cc)
+        act = cfg.ffnActivation
+        if act == "swiglu":
+            hh = F.silu(h @ g("mlp.fc_gate").T) * (h @ g("mlp.fc_up").T)
+            m = hh @ g("mlp.fc_proj").T
+        else:
+            pre = h @ g("mlp.fc1").T
+            if act == "gelu":
+                hh = F.gelu(pre, approximate="tanh")
+            elif act == "silu":
+                hh = F.silu(pre)
+            elif act == "relu":
+                hh = F.relu(pre)
+            elif act == "universal":
+                hh = F.silu(pre) * g("mlp.act_gate") + pre * g("mlp.act_skip")
+            else:
+                hh = (F.silu(pre) * g("mlp.kan_c0") + F.relu(pre) * g("mlp.kan_c1") + F.gelu(pre, approximate="tanh") * g("mlp.kan_c2")
+                      + pre * g("mlp.kan_c3") + pre * pre * g("mlp.kan_c4"))
+            m = hh @ g("mlp.fc2").T
+        x = x + m.reshape(Bt, T, Cc)
+    x = F.layer_norm(x, (Cc,), P["lnF.weight"], P["lnF.bias"], 1e-5)
+    logits = x.reshape(Bt * T, Cc) @ P["lmHead"].T
+    return logits, F.cross_entropy(logits, targets.reshape(-1))
+
+
+def _check_model(act, seed):
+    cfg = rm.ModelConfig(vocabSize=29, blockSize=12, nLayer=2, nEmbd=16, nHead=4, ffnActivation=act)
+    Bm = ref.CpuRef()
+    params = rm.initGPT(cfg, Bm, ref.SeededRng(seed))
+    entries = rm.collectParamEntries(params)
+    rs = np.random.RandomState(seed)
+    for _, v in entries:       # perturb so LN weights/biases and gates are generic
+        v.data.data += (rs.randn(v.data.data.size) * 0.05).astype(np.float32)
+    inp, tgt = rm.synthetic_batch(seed + 1, 3, 12, 29)
+    tape = rm.Tape()
+    logits, loss = rm.gptForward(cfg, params, Bm, tape, inp, tgt, True)
+    tape.backward(loss, Bm)
+    P = {n: torch.tensor(v.data.data.astype(np.float64)).reshape(v.data.shape).requires_grad_() for n, v in entries}
+    tl, tloss = _torch_forward(cfg, P, torch.tensor(inp.data.astype(np.int64)).reshape(3, 12),
+                               torch.tensor(tgt.data.astype(np.int64)).reshape(3, 12))
+    tloss.backward()
+    assert abs(float(loss.data.data[0]) - tloss.item()) < 2e-6
+    assert np.max(np.abs(logits.data.data - tl.detach().numpy().reshape(-1))) < 2e-6
+    for n, v in entries:
+        want = P[n].grad.numpy().reshape(-1)
+        got = v.grad.data.astype(np.float64)
+        assert np.max(np.abs(got - want)) <= 2e-6 * (1 + np.max(np.abs(want))), n
+
+
+def test_full_model_forward_backward_vs_torch_f64_gelu():
+    _check_model("gelu", 0)
+
+
+def test_full_model_forward_backward_vs_torch_f64_custom_activations():
+    for act in ("swiglu", "universal", "kan_spline", "silu", "relu"):
+        _check_model(act, 3)
+
+
+def test_lr_schedule_closed_form():
+    tc = rm.TrainConfig(iters=50, lr=3e-4)
+    assert abs(rm.lr_at(tc, 0) - (3e-5 + 2.7e-4 * 1 / 10)) < 1e-18            # warm-up = min(2000, 50//5) = 10
+    assert abs(rm.lr_at(tc, 9) - 3e-4) < 1e-18
+    assert abs(rm.lr_at(tc, 30) - (3e-5 + 2.7e-4 * 0.5 * (1 + math.cos(math.pi * 20 / 40)))) < 1e-18
+    assert abs(rm.lr_at(rm.TrainConfig(iters=1, lr=3e-4), 0) - 3e-4) < 1e-18  # no warm-up at iters=1
+
+
+def test_trainer_step_clip_identity_and_initial_loss():
+    cfg = rm.ModelConfig(vocabSize=64, blockSize=16, nLayer=2, nEmbd=32, nHead=4)
+    tr = rm.Trainer(cfg, rm.TrainConfig(iters=1), seed=0)
+    before = {n: v.data.data.copy() for n, v in tr.entries}
+    r = tr.step([rm.synthetic_batch(1, 2, 16, 64)])
+    assert abs(r.loss - math.log(64)) < 0.05                # uniform prediction at std-0.02 init
+    assert r.gradNorm > 1.0 and abs(r.clipCoef * r.gradNorm - 1.0) < 1e-12      # post-clip norm == clip
+    # step 1 from m=v=0: |dp| <= lr * (1 + wd*|p|); sign(dp) = -sign(g) for no-decay tensors
+    for n, v in tr.entries:
+        d = v.data.data - before[n]
+        assert np.all(np.abs(d) <= 3e-4 * (1 + 0.1 * np.abs(before[n])) + 2e-8), n
+
+
+def test_grad_accumulation_scales_by_one_over_k():
+    cfg = rm.ModelConfig(vocabSize=32, blockSize=8, nLayer=1, nEmbd=16, nHead=2)
+    b1, b2 = rm.synthetic_batch(5, 2, 8, 32), rm.synthetic_batch(6, 2, 8, 32)
+    tr = rm.Trainer(cfg, rm.TrainConfig(iters=1, gradClip=0.0), seed=1)
+    r = tr.step([b1, b2])
+    tr1 = rm.Trainer(cfg, rm.TrainConfig(iters=1, gradClip=0.0), seed=1)
+    l1 = tr1.forward_backward(*b1); l2 = tr1.forward_backward(*b2)
+    assert abs(r.loss - (l1 + l2) / 2) < 1e-6              # gpu-perf.test.ts:303-321: sum(loss_i)/K
+    sq = sum(ref.sum_sq(v.grad) for _, v in tr1.entries)
+    assert abs(r.gradNorm - math.sqrt(sq) * 0.5) < 1e-9
