@@ -1,0 +1,90 @@
+// Shared host/device helpers for libalpha_hip (gfx950 only, wave64).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_bf16.h>
+#include <stdint.h>
+#include <stddef.h>
+#include "../../include/alpha_hip.h"
+
+namespace ah {
+
+// ---- host-side context (defined in runtime.hip) -------------------------------------------------
+hipStream_t stream();
+bool        ready();
+int32_t     fail(int32_t code, const char *fmt, ...);
+int32_t     hip_fail(hipError_t e, const char *what);
+void        count_op();
+int         num_cus();
+// Scratch for two-stage reductions: a library-owned device buffer of at least `bytes` bytes that stays
+// valid until the next call that asks for scratch on the same stream (calls are stream-ordered).
+void       *scratch(size_t bytes);
+
+#define AH_REQUIRE_READY() do { if (!ah::ready()) return ah::fail(AH_ERR_STATE, "%s: ah_init has not been called", __func__); } while (0)
+#define AH_HIP(expr) do { hipError_t _e = (expr); if (_e != hipSuccess) return ah::hip_fail(_e, #expr); } while (0)
+#define AH_ARG(cond, ...) do { if (!(cond)) return ah::fail(AH_ERR_ARG, __VA_ARGS__); } while (0)
+#define AH_LAUNCH_CHECK() do { hipError_t _e = hipGetLastError(); if (_e != hipSuccess) return ah::hip_fail(_e, __func__); ah::count_op(); } while (0)
+
+template <class T> static inline T *dp(ah_ptr p) { return reinterpret_cast<T *>(static_cast<uintptr_t>(p)); }
+static inline bool aligned16(ah_ptr p) { return (p & 15u) == 0; }
+static inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// ---- device helpers -----------------------------------------------------------------------------
+typedef __hip_bfloat16 bf16;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint16_t h) { return __uint_as_float(((uint32_t)h) << 16); }
+// round-to-nearest-even f32 -> bf16 bits (NaN kept quiet)
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  return (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
+}
+
+template <class T> struct Io;
+template <> struct Io<float> {
+  static __device__ __forceinline__ float ld(const float *p, size_t i) { return p[i]; }
+  static __device__ __forceinline__ void  st(float *p, size_t i, float v) { p[i] = v; }
+};
+template <> struct Io<uint16_t> {   // bf16 storage
+  static __device__ __forceinline__ float ld(const uint16_t *p, size_t i) { return bf16_bits_to_f32(p[i]); }
+  static __device__ __forceinline__ void  st(uint16_t *p, size_t i, float v) { p[i] = f32_to_bf16_bits(v); }
+};
+
+// wave64 butterfly reductions
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ double wave_sum_d(double v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+
+// tanh-approximation GELU and its derivative (cpu_ref.ts:422-427; ops.ts:405-417)
+__device__ __forceinline__ float gelu_f(float x) {
+  const float k = 0.7978845608028654f;
+  return 0.5f * x * (1.0f + tanhf(k * (x + 0.044715f * x * x * x)));
+}
+__device__ __forceinline__ float gelu_grad_f(float x) {
+  const float k = 0.7978845608028654f;
+  float t = tanhf(k * (x + 0.044715f * x * x * x));
+  float sech2 = 1.0f - t * t;
+  float dinner = k * (1.0f + 3.0f * 0.044715f * x * x);
+  return 0.5f * (1.0f + t) + 0.5f * x * sech2 * dinner;
+}
+
+}  // namespace ah

@@ -1,0 +1,510 @@
+// Element-wise and data-movement kernels (HBM-bound; coalesced, float4 where alignment allows).
+#include "common.h"
+
+using namespace ah;
+
+namespace {
+
+constexpr int TPB = 256;
+
+inline int grid_for(uint64_t work_items) {
+  int64_t blocks = cdiv((int64_t)work_items, TPB);
+  int64_t cap = (int64_t)num_cus() * 16;
+  if (blocks > cap) blocks = cap;
+  if (blocks < 1) blocks = 1;
+  return (int)blocks;
+}
+
+// ---- functors -----------------------------------------------------------------------------------
+struct BinOp {
+  int op;
+  __device__ __forceinline__ float operator()(float x, float y) const {
+    switch (op) { case AH_ADD: return x + y; case AH_SUB: return x - y; case AH_MUL: return x * y; default: return x / y; }
+  }
+};
+struct UnOp {
+  int op; float p0, p1;
+  __device__ __forceinline__ float operator()(float x) const {
+    switch (op) {
+      case AH_NEG: return -x;
+      case AH_EXP: return expf(x);
+      case AH_LOG: return logf(x);
+      case AH_SQRT: return sqrtf(x);
+      case AH_POW: return powf(x, p0);
+      case AH_SCALE: return x * p0;
+      case AH_CLAMP: return fmaxf(p0, fminf(p1, x));
+      case AH_GELU: return gelu_f(x);
+      case AH_RELU: return x > 0.f ? x : 0.f;
+      case AH_SILU: return x / (1.0f + expf(-x));
+      default: return tanhf(x / p0) * p0;     // AH_SOFTCAP
+    }
+  }
+};
+struct UnBwd {
+  int op; float p0, p1;
+  __device__ __forceinline__ float operator()(float x, float g) const {
+    switch (op) {
+      case AH_GELU_BWD: return g * gelu_grad_f(x);
+      case AH_RELU_BWD: return x > 0.f ? g : 0.f;
+      case AH_SILU_BWD: { float s = 1.0f / (1.0f + expf(-x)); return g * (s * (1.0f + x * (1.0f - s))); }
+      case AH_CLAMP_BWD: return (x > p0 && x < p1) ? g : 0.f;
+      default: { float t = tanhf(x / p0); return g * (1.0f - t * t); }   // AH_SOFTCAP_BWD
+    }
+  }
+};
+
+template <class F>
+__global__ void k_unary(const float *__restrict__ x, float *__restrict__ out, uint64_t n, F f, int vec) {
+  uint64_t tid = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x, stride = (uint64_t)gridDim.x * blockDim.x;
+  if (vec) {
+    uint64_t n4 = n >> 2;
+    for (uint64_t i = tid; i < n4; i += stride) {
+      float4 v = reinterpret_cast<const float4 *>(x)[i];
+      v.x = f(v.x); v.y = f(v.y); v.z = f(v.z); v.w = f(v.w);
+      reinterpret_cast<float4 *>(out)[i] = v;
+    }
+    for (uint64_t i = (n4 << 2) + tid; i < n; i += stride) out[i] = f(x[i]);
+  } else {
+    for (uint64_t i = tid; i < n; i += stride) out[i] = f(x[i]);
+  }
+}
+template <class F>
+__global__ void k_binary(const float *__restrict__ a, const float *__restrict__ b, float *__restrict__ out,
+                         uint64_t n, F f, int vec) {
+  uint64_t tid = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x, stride = (uint64_t)gridDim.x * blockDim.x;
+  if (vec) {
+    uint64_t n4 = n >> 2;
+    for (uint64_t i = tid; i < n4; i += stride) {
+      float4 u = reinterpret_cast<const float4 *>(a)[i], v = reinterpret_cast<const float4 *>(b)[i], r;
+      r.x = f(u.x, v.x); r.y = f(u.y, v.y); r.z = f(u.z, v.z); r.w = f(u.w, v.w);
+      reinterpret_cast<float4 *>(out)[i] = r;
+    }
+    for (uint64_t i = (n4 << 2) + tid; i < n; i += stride) out[i] = f(a[i], b[i]);
+  } else {
+    for (uint64_t i = tid; i < n; i += stride) out[i] = f(a[i], b[i]);
+  }
+}
+
+struct Dims6 { int64_t shape[6]; int64_t sa[6]; int64_t sb[6]; int nd; };
+
+__global__ void k_binary_bcast(const float *__restrict__ a, const float *__restrict__ b, float *__restrict__ out,
+                               uint64_t n, Dims6 d, BinOp f) {
+  uint64_t tid = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x, stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t i = tid; i < n; i += stride) {
+    uint64_t rem = i; int64_t ia = 0, ib = 0;
+    for (int k = d.nd - 1; k >= 0; k--) {
+      uint64_t c = rem % (uint64_t)d.shape[k]; rem /= (uint64_t)d.shape[k];
+      ia += (int64_t)c * d.sa[k]; ib += (int64_t)c * d.sb[k];
+    }
+    out[i] = f(a[ia], b[ib]);
+  }
+}
+
+// generic strided gather: out[i] = src[offset + sum(coord_k * stride_k)] over `shape`
+struct Gather6 { int64_t shape[6]; int64_t stride[6]; int64_t offset; int nd; };
+__global__ void k_gather(const uint32_t *__restrict__ src, uint32_t *__restrict__ out, uint64_t n, Gather6 d) {
+  uint64_t tid = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x, stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t i = tid; i < n; i += stride) {
+    uint64_t rem = i; int64_t s = d.offset;
+    for (int k = d.nd - 1; k >= 0; k--) {
+      uint64_t c = rem % (uint64_t)d.shape[k]; rem /= (uint64_t)d.shape[k];
+      s += (int64_t)c * d.stride[k];
+    }
+    out[i] = src[s];
+  }
+}
+// generic strided scatter: dst[offset + sum(coord_k*stride_k)] = src[i]
+__global__ void k_scatter(const uint32_t *__restrict__ src, uint32_t *__restrict__ dst, uint64_t n, Gather6 d) {
+  uint64_t tid = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x, stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t i = tid; i < n; i += stride) {
+    uint64_t rem = i; int64_t s = d.offset;
+    for (int k = d.nd - 1; k >= 0; k--) {
+      uint64_t c = rem % (uint64_t)d.shape[k]; rem /= (uint64_t)d.shape[k];
+      s += (int64_t)c * d.stride[k];
+    }
+    dst[s] = src[i];
+  }
+}
+
+// 32x32 LDS-tiled transpose of the last two dims of [batch, R, C] (coalesced both ways)
+__global__ void k_transpose_last2(const uint32_t *__restrict__ in, uint32_t *__restrict__ out, int64_t R, int64_t C) {
+  __shared__ uint32_t tile[32][33];
+  int64_t b = blockIdx.z;
+  const uint32_t *src = in + b * R * C;
+  uint32_t *dst = out + b * R * C;
+  int64_t c0 = (int64_t)blockIdx.x * 32, r0 = (int64_t)blockIdx.y * 32;
+  for (int j = threadIdx.y; j < 32; j += blockDim.y) {
+    int64_t r = r0 + j, c = c0 + threadIdx.x;
+    if (r < R && c < C) tile[j][threadIdx.x] = src[r * C + c];
+  }
+  __syncthreads();
+  for (int j = threadIdx.y; j < 32; j += blockDim.y) {
+    int64_t c = c0 + j, r = r0 + threadIdx.x;
+    if (r < R && c < C) dst[c * R + r] = tile[threadIdx.x][j];
+  }
+}
+
+template <class T>
+__global__ void k_fill(T *__restrict__ p, T v, uint64_t n) {
+  uint64_t tid = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x, stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t i = tid; i < n; i += stride) p[i] = v;
+}
+
+__global__ void k_axpy(float *__restrict__ a, const float *__restrict__ b, float s, uint64_t n) {
+  uint64_t tid = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x, stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t i = tid; i < n; i += stride) a[i] += b[i] * s;
+}
+
+__global__ void k_silu_mul(const float *__restrict__ a, const float *__restrict__ b, float *__restrict__ out, uint64_t n) {
+  uint64_t tid = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x, stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t i = tid; i < n; i += stride) { float x = a[i]; out[i] = x / (1.0f + expf(-x)) * b[i]; }
+}
+__global__ void k_silu_mul_bwd(const float *__restrict__ a, const float *__restrict__ b, const float *__restrict__ g,
+                               float *__restrict__ da, float *__restrict__ db, uint64_t n) {
+  uint64_t tid = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x, stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t i = tid; i < n; i += stride) {
+    float x = a[i], s = 1.0f / (1.0f + expf(-x)), gi = g[i];
+    da[i] = gi * b[i] * (s * (1.0f + x * (1.0f - s)));
+    db[i] = gi * (x * s);
+  }
+}
+__global__ void k_residual_dropout_add(const float *__restrict__ r, const float *__restrict__ p, const float *__restrict__ m,
+                                       float *__restrict__ out, uint64_t n) {
+  uint64_t tid = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x, stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t i = tid; i < n; i += stride) out[i] = r[i] + (m ? p[i] * m[i] : p[i]);
+}
+// u32-wrapping variant of the reference's splitmix-style hash (packages/helios/src/kernels/nn.ts:5600-5748)
+__global__ void k_dropout_mask(float *__restrict__ out, uint64_t n, uint32_t seed, uint32_t counter, float p, float keep) {
+  uint64_t tid = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x, stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t i = tid; i < n; i += stride) {
+    uint32_t h = seed + counter * 2654435761u + (uint32_t)i * 2246822519u;
+    h = (h ^ (h >> 16)) * 0x85ebca6bu;
+    h = (h ^ (h >> 13)) * 0xc2b2ae35u;
+    h = h ^ (h >> 16);
+    float x = (float)((double)h / 4294967296.0);
+    out[i] = x > p ? keep : 0.f;
+  }
+}
+__global__ void k_masked_fill(const float *__restrict__ a, const float *__restrict__ mask, float *__restrict__ out,
+                              uint64_t n, uint64_t mask_n, float value) {
+  uint64_t tid = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x, stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t i = tid; i < n; i += stride) out[i] = (mask[i % mask_n] != 0.f) ? value : a[i];
+}
+__global__ void k_causal_mask(float *__restrict__ out, int64_t size) {
+  uint64_t n = (uint64_t)size * size;
+  uint64_t tid = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x, stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t i = tid; i < n; i += stride) out[i] = ((int64_t)(i % size) > (int64_t)(i / size)) ? -INFINITY : 0.f;
+}
+
+__device__ __forceinline__ uint16_t f32_to_f16_bits(float f) { _Float16 h = (_Float16)f; uint16_t u; __builtin_memcpy(&u, &h, 2); return u; }
+__device__ __forceinline__ float f16_bits_to_f32(uint16_t u) { _Float16 h; __builtin_memcpy(&h, &u, 2); return (float)h; }
+
+__global__ void k_cast(const void *__restrict__ src, int sd, void *__restrict__ dst, int dd, uint64_t n) {
+  uint64_t tid = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x, stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t i = tid; i < n; i += stride) {
+    float v;
+    if (sd == AH_F32) v = ((const float *)src)[i];
+    else if (sd == AH_BF16) v = bf16_bits_to_f32(((const uint16_t *)src)[i]);
+    else if (sd == AH_F16) v = f16_bits_to_f32(((const uint16_t *)src)[i]);
+    else v = (float)((const int32_t *)src)[i];
+    if (dd == AH_F32) ((float *)dst)[i] = v;
+    else if (dd == AH_BF16) ((uint16_t *)dst)[i] = f32_to_bf16_bits(v);
+    else if (dd == AH_F16) ((uint16_t *)dst)[i] = f32_to_f16_bits(v);
+    else ((int32_t *)dst)[i] = (int32_t)v;
+  }
+}
+
+__global__ void k_check_finite(const float *__restrict__ x, uint64_t n, float *__restrict__ flag) {
+  uint64_t tid = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x, stride = (uint64_t)gridDim.x * blockDim.x;
+  bool bad = false;
+  for (uint64_t i = tid; i < n; i += stride) {
+    uint32_t u = __float_as_uint(x[i]);
+    bad |= ((u & 0x7f800000u) == 0x7f800000u);
+  }
+  if (__any(bad) && (threadIdx.x & 63) == 0) *flag = 1.0f;   // every writer stores the same value
+}
+
+inline bool vec_ok(uint64_t n, ah_ptr a, ah_ptr b, ah_ptr c) {
+  (void)n;
+  return aligned16(a) && aligned16(b) && aligned16(c);
+}
+
+void row_major_strides(int nd, const int64_t *shape, int64_t *st) {
+  int64_t s = 1;
+  for (int i = nd - 1; i >= 0; i--) { st[i] = s; s *= shape[i]; }
+}
+int64_t prod(int nd, const int64_t *shape) { int64_t s = 1; for (int i = 0; i < nd; i++) s *= shape[i]; return s; }
+
+}  // namespace
+
+extern "C" {
+
+int32_t ah_fill_f32(ah_ptr dst, float value, uint64_t n) {
+  AH_REQUIRE_READY();
+  if (n == 0) return AH_OK;
+  AH_ARG(dst != 0, "ah_fill_f32: null dst");
+  hipLaunchKernelGGL(k_fill<float>, dim3(grid_for(n)), dim3(TPB), 0, stream(), dp<float>(dst), value, n);
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+int32_t ah_fill_i32(ah_ptr dst, int32_t value, uint64_t n) {
+  AH_REQUIRE_READY();
+  if (n == 0) return AH_OK;
+  AH_ARG(dst != 0, "ah_fill_i32: null dst");
+  hipLaunchKernelGGL(k_fill<int32_t>, dim3(grid_for(n)), dim3(TPB), 0, stream(), dp<int32_t>(dst), value, n);
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+
+int32_t ah_binary(int32_t op, ah_ptr a, ah_ptr b, ah_ptr out, uint64_t n) {
+  AH_REQUIRE_READY();
+  AH_ARG(op >= AH_ADD && op <= AH_DIV, "ah_binary: bad op %d", op);
+  if (n == 0) return AH_OK;
+  AH_ARG(a && b && out, "ah_binary: null operand");
+  int vec = vec_ok(n, a, b, out);
+  hipLaunchKernelGGL(k_binary<BinOp>, dim3(grid_for(vec ? n / 4 + 1 : n)), dim3(TPB), 0, stream(),
+                     dp<const float>(a), dp<const float>(b), dp<float>(out), n, BinOp{op}, vec);
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+
+int32_t ah_binary_broadcast(int32_t op, ah_ptr a, ah_ptr b, ah_ptr out, int32_t nd, const int64_t *shape,
+                            const int64_t *stride_a, const int64_t *stride_b) {
+  AH_REQUIRE_READY();
+  AH_ARG(op >= AH_ADD && op <= AH_DIV, "ah_binary_broadcast: bad op %d", op);
+  AH_ARG(nd >= 0 && nd <= 6, "ah_binary_broadcast: nd %d > 6", nd);
+  Dims6 d; d.nd = nd;
+  for (int i = 0; i < nd; i++) { d.shape[i] = shape[i]; d.sa[i] = stride_a[i]; d.sb[i] = stride_b[i]; }
+  uint64_t n = (uint64_t)prod(nd, shape);
+  if (n == 0) return AH_OK;
+  AH_ARG(a && b && out, "ah_binary_broadcast: null operand");
+  hipLaunchKernelGGL(k_binary_bcast, dim3(grid_for(n)), dim3(TPB), 0, stream(), dp<const float>(a), dp<const float>(b),
+                     dp<float>(out), n, d, BinOp{op});
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+
+int32_t ah_unary(int32_t op, ah_ptr x, ah_ptr out, uint64_t n, float p0, float p1) {
+  AH_REQUIRE_READY();
+  AH_ARG(op >= AH_NEG && op <= AH_SOFTCAP, "ah_unary: bad op %d", op);
+  if (n == 0) return AH_OK;
+  AH_ARG(x && out, "ah_unary: null operand");
+  int vec = vec_ok(n, x, x, out);
+  hipLaunchKernelGGL(k_unary<UnOp>, dim3(grid_for(vec ? n / 4 + 1 : n)), dim3(TPB), 0, stream(), dp<const float>(x),
+                     dp<float>(out), n, UnOp{op, p0, p1}, vec);
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+
+int32_t ah_add_inplace(ah_ptr a, ah_ptr b, uint64_t n) { return ah_binary(AH_ADD, a, b, a, n); }
+int32_t ah_scale_inplace(ah_ptr a, float s, uint64_t n) { return ah_unary(AH_SCALE, a, a, n, s, 0.f); }
+int32_t ah_axpy_inplace(ah_ptr a, ah_ptr b, float s, uint64_t n) {
+  AH_REQUIRE_READY();
+  if (n == 0) return AH_OK;
+  AH_ARG(a && b, "ah_axpy_inplace: null operand");
+  hipLaunchKernelGGL(k_axpy, dim3(grid_for(n)), dim3(TPB), 0, stream(), dp<float>(a), dp<const float>(b), s, n);
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+
+int32_t ah_unary_bwd(int32_t op, ah_ptr x, ah_ptr grad_out, ah_ptr out, uint64_t n, float p0, float p1) {
+  AH_REQUIRE_READY();
+  AH_ARG(op >= AH_GELU_BWD && op <= AH_SOFTCAP_BWD, "ah_unary_bwd: bad op %d", op);
+  if (n == 0) return AH_OK;
+  AH_ARG(x && grad_out && out, "ah_unary_bwd: null operand");
+  int vec = vec_ok(n, x, grad_out, out);
+  hipLaunchKernelGGL(k_binary<UnBwd>, dim3(grid_for(vec ? n / 4 + 1 : n)), dim3(TPB), 0, stream(), dp<const float>(x),
+                     dp<const float>(grad_out), dp<float>(out), n, UnBwd{op, p0, p1}, vec);
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+
+int32_t ah_silu_mul(ah_ptr a, ah_ptr b, ah_ptr out, uint64_t n) {
+  AH_REQUIRE_READY();
+  if (n == 0) return AH_OK;
+  AH_ARG(a && b && out, "ah_silu_mul: null operand");
+  hipLaunchKernelGGL(k_silu_mul, dim3(grid_for(n)), dim3(TPB), 0, stream(), dp<const float>(a), dp<const float>(b), dp<float>(out), n);
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+int32_t ah_silu_mul_bwd(ah_ptr a, ah_ptr b, ah_ptr g, ah_ptr da, ah_ptr db, uint64_t n) {
+  AH_REQUIRE_READY();
+  if (n == 0) return AH_OK;
+  AH_ARG(a && b && g && da && db, "ah_silu_mul_bwd: null operand");
+  hipLaunchKernelGGL(k_silu_mul_bwd, dim3(grid_for(n)), dim3(TPB), 0, stream(), dp<const float>(a), dp<const float>(b),
+                     dp<const float>(g), dp<float>(da), dp<float>(db), n);
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+int32_t ah_residual_dropout_add(ah_ptr residual, ah_ptr projected, ah_ptr mask, ah_ptr out, uint64_t n) {
+  AH_REQUIRE_READY();
+  if (n == 0) return AH_OK;
+  AH_ARG(residual && projected && out, "ah_residual_dropout_add: null operand");
+  hipLaunchKernelGGL(k_residual_dropout_add, dim3(grid_for(n)), dim3(TPB), 0, stream(), dp<const float>(residual),
+                     dp<const float>(projected), dp<const float>(mask), dp<float>(out), n);
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+int32_t ah_dropout_mask(ah_ptr out, uint64_t n, int32_t seed, int32_t counter, float p) {
+  AH_REQUIRE_READY();
+  if (n == 0) return AH_OK;
+  AH_ARG(out != 0, "ah_dropout_mask: null out");
+  AH_ARG(p >= 0.f && p < 1.f, "ah_dropout_mask: p must be in [0,1)");
+  hipLaunchKernelGGL(k_dropout_mask, dim3(grid_for(n)), dim3(TPB), 0, stream(), dp<float>(out), n, (uint32_t)seed,
+                     (uint32_t)counter, p, 1.0f / (1.0f - p));
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+int32_t ah_masked_fill(ah_ptr a, ah_ptr mask, ah_ptr out, uint64_t n, uint64_t mask_n, float value) {
+  AH_REQUIRE_READY();
+  if (n == 0) return AH_OK;
+  AH_ARG(a && mask && out && mask_n > 0, "ah_masked_fill: null operand or empty mask");
+  hipLaunchKernelGGL(k_masked_fill, dim3(grid_for(n)), dim3(TPB), 0, stream(), dp<const float>(a), dp<const float>(mask),
+                     dp<float>(out), n, mask_n, value);
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+int32_t ah_causal_mask(ah_ptr out, int64_t size) {
+  AH_REQUIRE_READY();
+  if (size <= 0) return AH_OK;
+  AH_ARG(out != 0, "ah_causal_mask: null out");
+  hipLaunchKernelGGL(k_causal_mask, dim3(grid_for((uint64_t)size * size)), dim3(TPB), 0, stream(), dp<float>(out), size);
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+int32_t ah_cast(ah_ptr src, int32_t sd, ah_ptr dst, int32_t dd, uint64_t n) {
+  AH_REQUIRE_READY();
+  AH_ARG(sd >= AH_F32 && sd <= AH_F16 && dd >= AH_F32 && dd <= AH_F16, "ah_cast: bad dtype");
+  if (n == 0) return AH_OK;
+  AH_ARG(src && dst, "ah_cast: null operand");
+  hipLaunchKernelGGL(k_cast, dim3(grid_for(n)), dim3(TPB), 0, stream(), dp<const void>(src), sd, dp<void>(dst), dd, n);
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+int32_t ah_check_finite(ah_ptr x, uint64_t n, ah_ptr out_flag) {
+  AH_REQUIRE_READY();
+  AH_ARG(out_flag != 0, "ah_check_finite: null out");
+  int32_t rc = ah_fill_f32(out_flag, 0.f, 1);
+  if (rc) return rc;
+  if (n == 0) return AH_OK;
+  AH_ARG(x != 0, "ah_check_finite: null x");
+  hipLaunchKernelGGL(k_check_finite, dim3(grid_for(n)), dim3(TPB), 0, stream(), dp<const float>(x), n, dp<float>(out_flag));
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+
+int32_t ah_transpose(ah_ptr a, ah_ptr out, int32_t nd, const int64_t *shape, int32_t d0, int32_t d1) {
+  AH_REQUIRE_READY();
+  AH_ARG(nd >= 1 && nd <= 6, "ah_transpose: nd %d out of range", nd);
+  if (d0 < 0) d0 += nd;
+  if (d1 < 0) d1 += nd;
+  AH_ARG(d0 >= 0 && d0 < nd && d1 >= 0 && d1 < nd, "ah_transpose: axis out of range for ndim %d", nd);
+  uint64_t n = (uint64_t)prod(nd, shape);
+  if (n == 0) return AH_OK;
+  AH_ARG(a && out, "ah_transpose: null operand");
+  if (d0 == d1) return ah_copy(out, a, n * 4);
+  if (d0 > d1) { int t = d0; d0 = d1; d1 = t; }
+  if (d0 == nd - 2 && d1 == nd - 1) {
+    int64_t R = shape[nd - 2], C = shape[nd - 1], batch = (int64_t)(n / (uint64_t)(R * C));
+    if (batch <= 65535) {
+      dim3 grid((unsigned)cdiv(C, 32), (unsigned)cdiv(R, 32), (unsigned)batch);
+      hipLaunchKernelGGL(k_transpose_last2, grid, dim3(32, 8), 0, stream(), dp<const uint32_t>(a), dp<uint32_t>(out), R, C);
+      AH_LAUNCH_CHECK();
+      return AH_OK;
+    }
+  }
+  // out[i] over the transposed shape gathers from a with swapped strides
+  int64_t st[6]; row_major_strides(nd, shape, st);
+  Gather6 g; g.nd = nd; g.offset = 0;
+  for (int i = 0; i < nd; i++) { g.shape[i] = shape[i]; g.stride[i] = st[i]; }
+  { int64_t t = g.shape[d0]; g.shape[d0] = g.shape[d1]; g.shape[d1] = t; t = g.stride[d0]; g.stride[d0] = g.stride[d1]; g.stride[d1] = t; }
+  hipLaunchKernelGGL(k_gather, dim3(grid_for(n)), dim3(TPB), 0, stream(), dp<const uint32_t>(a), dp<uint32_t>(out), n, g);
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+
+int32_t ah_slice(ah_ptr a, ah_ptr out, int32_t nd, const int64_t *shape, const int64_t *starts, const int64_t *ends) {
+  AH_REQUIRE_READY();
+  AH_ARG(nd >= 1 && nd <= 6, "ah_slice: nd %d out of range", nd);
+  int64_t st[6]; row_major_strides(nd, shape, st);
+  Gather6 g; g.nd = nd; g.offset = 0;
+  for (int i = 0; i < nd; i++) {
+    AH_ARG(starts[i] >= 0 && ends[i] <= shape[i] && starts[i] <= ends[i], "ah_slice: range [%lld,%lld) outside dim %d of size %lld",
+           (long long)starts[i], (long long)ends[i], i, (long long)shape[i]);
+    g.shape[i] = ends[i] - starts[i]; g.stride[i] = st[i]; g.offset += starts[i] * st[i];
+  }
+  uint64_t n = (uint64_t)prod(nd, g.shape);
+  if (n == 0) return AH_OK;
+  AH_ARG(a && out, "ah_slice: null operand");
+  hipLaunchKernelGGL(k_gather, dim3(grid_for(n)), dim3(TPB), 0, stream(), dp<const uint32_t>(a), dp<uint32_t>(out), n, g);
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+
+int32_t ah_scatter_slice(ah_ptr grad, ah_ptr out, int32_t nd, const int64_t *gshape, const int64_t *orig, const int64_t *starts) {
+  AH_REQUIRE_READY();
+  AH_ARG(nd >= 1 && nd <= 6, "ah_scatter_slice: nd %d out of range", nd);
+  int64_t st[6]; row_major_strides(nd, orig, st);
+  Gather6 g; g.nd = nd; g.offset = 0;
+  for (int i = 0; i < nd; i++) {
+    AH_ARG(starts[i] >= 0 && starts[i] + gshape[i] <= orig[i], "ah_scatter_slice: slice does not fit dim %d", i);
+    g.shape[i] = gshape[i]; g.stride[i] = st[i]; g.offset += starts[i] * st[i];
+  }
+  uint64_t total = (uint64_t)prod(nd, orig), n = (uint64_t)prod(nd, gshape);
+  if (total == 0) return AH_OK;
+  AH_ARG(out != 0, "ah_scatter_slice: null out");
+  int32_t rc = ah_fill_f32(out, 0.f, total);
+  if (rc) return rc;
+  if (n == 0) return AH_OK;
+  AH_ARG(grad != 0, "ah_scatter_slice: null grad");
+  hipLaunchKernelGGL(k_scatter, dim3(grid_for(n)), dim3(TPB), 0, stream(), dp<const uint32_t>(grad), dp<uint32_t>(out), n, g);
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+
+int32_t ah_cat_part(ah_ptr src, ah_ptr dst, int32_t nd, const int64_t *src_shape, const int64_t *dst_shape, int32_t axis,
+                    int64_t axis_offset) {
+  AH_REQUIRE_READY();
+  AH_ARG(nd >= 1 && nd <= 6, "ah_cat_part: nd %d out of range", nd);
+  if (axis < 0) axis += nd;
+  AH_ARG(axis >= 0 && axis < nd, "ah_cat_part: axis out of range");
+  int64_t st[6]; row_major_strides(nd, dst_shape, st);
+  Gather6 g; g.nd = nd; g.offset = axis_offset * st[axis];
+  for (int i = 0; i < nd; i++) {
+    if (i != axis) AH_ARG(src_shape[i] == dst_shape[i], "cat: shape mismatch at dim %d", i);
+    g.shape[i] = src_shape[i]; g.stride[i] = st[i];
+  }
+  AH_ARG(axis_offset >= 0 && axis_offset + src_shape[axis] <= dst_shape[axis], "ah_cat_part: operand does not fit");
+  uint64_t n = (uint64_t)prod(nd, src_shape);
+  if (n == 0) return AH_OK;
+  AH_ARG(src && dst, "ah_cat_part: null operand");
+  hipLaunchKernelGGL(k_scatter, dim3(grid_for(n)), dim3(TPB), 0, stream(), dp<const uint32_t>(src), dp<uint32_t>(dst), n, g);
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+
+int32_t ah_slice_qkv(ah_ptr qkv, ah_ptr q, ah_ptr k, ah_ptr v, int64_t rows, int64_t d) {
+  int64_t shape[2] = {rows, 3 * d};
+  ah_ptr outs[3] = {q, k, v};
+  for (int i = 0; i < 3; i++) {
+    int64_t s[2] = {0, i * d}, e[2] = {rows, (i + 1) * d};
+    int32_t rc = ah_slice(qkv, outs[i], 2, shape, s, e);
+    if (rc) return rc;
+  }
+  return AH_OK;
+}
+
+int32_t ah_broadcast(ah_ptr a, ah_ptr out, int32_t nd, const int64_t *out_shape, const int64_t *stride_a) {
+  AH_REQUIRE_READY();
+  AH_ARG(nd >= 0 && nd <= 6, "ah_broadcast: nd %d out of range", nd);
+  Gather6 g; g.nd = nd; g.offset = 0;
+  for (int i = 0; i < nd; i++) { g.shape[i] = out_shape[i]; g.stride[i] = stride_a[i]; }
+  uint64_t n = (uint64_t)prod(nd, out_shape);
+  if (n == 0) return AH_OK;
+  AH_ARG(a && out, "ah_broadcast: null operand");
+  hipLaunchKernelGGL(k_gather, dim3(grid_for(n)), dim3(TPB), 0, stream(), dp<const uint32_t>(a), dp<uint32_t>(out), n, g);
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+
+}  // extern "C"

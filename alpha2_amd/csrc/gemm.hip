@@ -1,0 +1,378 @@
+// GEMM on the gfx950 matrix cores.
+//   fp32 (parity mode): v_mfma_f32_32x32x2_f32, 128x128x16 LDS tiles, 4 waves (2x2) of 64x64.
+//   bf16 (fast mode)  : v_mfma_f32_32x32x16_bf16, BMxBNx32 LDS tiles double-buffered, fp32 accumulate.
+// All three operand layouts the training step needs are handled (NN: dX = G W, NT: Y = X W^T,
+// TN: dW = G^T X).  Epilogues fuse GELU (+ saved pre-activation), the residual add, gradient
+// accumulation and the GELU derivative.
+#include "common.h"
+
+using namespace ah;
+
+namespace {
+
+struct GemmArgs {
+  const void *a, *b;
+  void *c;
+  const void *aux;     // EPI_RESIDUAL: f32 [M,N]; EPI_GELU_BWD: pre-activation (C dtype)
+  void *aux_out;       // EPI_GELU: pre-activation out (C dtype)
+  int M, N, K;
+  int64_t lda, ldb, ldc;
+  int64_t sa, sb, sc;  // batch strides (elements)
+  int epi;
+};
+
+template <class OUT>
+__device__ __forceinline__ void epilogue_store(const GemmArgs &g, int64_t cbase, int row, int col, float acc) {
+  if (row >= g.M || col >= g.N) return;
+  int64_t idx = cbase + (int64_t)row * g.ldc + col;
+  OUT *c = (OUT *)g.c;
+  switch (g.epi) {
+    case AH_EPI_NONE: Io<OUT>::st(c, idx, acc); break;
+    case AH_EPI_ACCUM: Io<OUT>::st(c, idx, Io<OUT>::ld(c, idx) + acc); break;
+    case AH_EPI_GELU: Io<OUT>::st((OUT *)g.aux_out, idx, acc); Io<OUT>::st(c, idx, gelu_f(acc)); break;
+    case AH_EPI_RESIDUAL: Io<OUT>::st(c, idx, acc + ((const float *)g.aux)[idx]); break;
+    default: Io<OUT>::st(c, idx, acc * gelu_grad_f(Io<OUT>::ld((const OUT *)g.aux, idx))); break;   // GELU_BWD
+  }
+}
+
+// ================================================================ fp32 MFMA kernel
+// LDS tiles are k-major: As[k][m], Bs[k][n]; a lane of the 32x32x2 MFMA reads As[2*kk + lane/32][m0 + lane%32].
+constexpr int F_BM = 128, F_BN = 128, F_BK = 16, F_PAD = 4;
+
+// Load a [rows x F_BK] tile of an operand into registers (2 float4 per thread).
+//   KCONTIG = true : memory is [row][k] (k contiguous), thread -> (row = t/4 + 64*i, kq = t%4)
+//   KCONTIG = false: memory is [k][row] (row contiguous), thread -> (k = t/32 + 8*i, r4 = t%32)
+template <bool KCONTIG>
+__device__ __forceinline__ void f32_load_tile(const float *__restrict__ base, int64_t ld, int row0, int k0, int rows, int K,
+                                              bool vec, float4 (&v)[2]) {
+  int t = threadIdx.x;
+#pragma unroll
+  for (int i = 0; i < 2; i++) {
+    int r, k;
+    if (KCONTIG) { r = row0 + (t >> 2) + 64 * i; k = k0 + (t & 3) * 4; }
+    else { k = k0 + (t >> 5) + 8 * i; r = row0 + (t & 31) * 4; }
+    float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (KCONTIG) {
+      if (r < rows) {
+        const float *p = base + (int64_t)r * ld + k;
+        if (vec && k + 3 < K) x = *reinterpret_cast<const float4 *>(p);
+        else { if (k < K) x.x = p[0]; if (k + 1 < K) x.y = p[1]; if (k + 2 < K) x.z = p[2]; if (k + 3 < K) x.w = p[3]; }
+      }
+    } else {
+      if (k < K) {
+        const float *p = base + (int64_t)k * ld + r;
+        if (vec && r + 3 < rows) x = *reinterpret_cast<const float4 *>(p);
+        else { if (r < rows) x.x = p[0]; if (r + 1 < rows) x.y = p[1]; if (r + 2 < rows) x.z = p[2]; if (r + 3 < rows) x.w = p[3]; }
+      }
+    }
+    v[i] = x;
+  }
+}
+template <bool KCONTIG>
+__device__ __forceinline__ void f32_store_tile(float (*s)[F_BM + F_PAD], const float4 (&v)[2]) {
+  int t = threadIdx.x;
+#pragma unroll
+  for (int i = 0; i < 2; i++) {
+    if (KCONTIG) {
+      int r = (t >> 2) + 64 * i, k = (t & 3) * 4;
+      s[k + 0][r] = v[i].x; s[k + 1][r] = v[i].y; s[k + 2][r] = v[i].z; s[k + 3][r] = v[i].w;
+    } else {
+      int k = (t >> 5) + 8 * i, r = (t & 31) * 4;
+      *reinterpret_cast<float4 *>(&s[k][r]) = v[i];
+    }
+  }
+}
+
+template <int LAYOUT, class OUT>
+__global__ __launch_bounds__(256) void k_gemm_f32(GemmArgs g, int vec_a, int vec_b) {
+  __shared__ __attribute__((aligned(16))) float As[2][F_BK][F_BM + F_PAD];
+  __shared__ __attribute__((aligned(16))) float Bs[2][F_BK][F_BN + F_PAD];
+  constexpr bool A_KC = (LAYOUT != AH_GEMM_TN);     // A is [M][K] except for TN ([K][M])
+  constexpr bool B_KC = (LAYOUT == AH_GEMM_NT);     // B is [N][K] only for NT
+  int bz = blockIdx.z;
+  const float *A = (const float *)g.a + (int64_t)bz * g.sa;
+  const float *B = (const float *)g.b + (int64_t)bz * g.sb;
+  int64_t cbase = (int64_t)bz * g.sc;
+  int m0 = blockIdx.y * F_BM, n0 = blockIdx.x * F_BN;
+  int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+  int lr = lane & 31, lk = lane >> 5;
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
+
+  float4 ra[2], rb[2];
+  int nt = (g.K + F_BK - 1) / F_BK;
+  f32_load_tile<A_KC>(A, g.lda, m0, 0, g.M, g.K, vec_a, ra);
+  f32_load_tile<B_KC>(B, g.ldb, n0, 0, g.N, g.K, vec_b, rb);
+  f32_store_tile<A_KC>(As[0], ra);
+  f32_store_tile<B_KC>(Bs[0], rb);
+  __syncthreads();
+  for (int t = 0; t < nt; t++) {
+    int cur = t & 1;
+    if (t + 1 < nt) {
+      f32_load_tile<A_KC>(A, g.lda, m0, (t + 1) * F_BK, g.M, g.K, vec_a, ra);
+      f32_load_tile<B_KC>(B, g.ldb, n0, (t + 1) * F_BK, g.N, g.K, vec_b, rb);
+    }
+#pragma unroll
+    for (int kk = 0; kk < F_BK / 2; kk++) {
+      float a0 = As[cur][2 * kk + lk][wm + lr], a1 = As[cur][2 * kk + lk][wm + 32 + lr];
+      float b0 = Bs[cur][2 * kk + lk][wn + lr], b1 = Bs[cur][2 * kk + lk][wn + 32 + lr];
+      acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
+      acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
+      acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
+      acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+    }
+    if (t + 1 < nt) {
+      f32_store_tile<A_KC>(As[cur ^ 1], ra);
+      f32_store_tile<B_KC>(Bs[cur ^ 1], rb);
+    }
+    __syncthreads();
+  }
+  // accumulator element e of a 32x32 tile: row = 8*(e/4) + 4*(lane/32) + e%4, col = lane%32
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int e = 0; e < 16; e++) {
+        int row = m0 + wm + 32 * i + 8 * (e >> 2) + 4 * lk + (e & 3);
+        int col = n0 + wn + 32 * j + lr;
+        epilogue_store<OUT>(g, cbase, row, col, acc[i][j][e]);
+      }
+}
+
+// ================================================================ bf16 MFMA kernel (NT operands)
+// Both operands are [rows][K] with K contiguous.  LDS tiles are [rows][BK] with an 80-byte row pitch
+// (32 bf16 + 8 pad) so the 16-byte fragment reads of 8 consecutive rows hit 8 distinct bank groups.
+// A lane of v_mfma_f32_32x32x16_bf16 supplies, for row lane%32, the 8 k-values 8*(lane/32)..+7.
+constexpr int H_BK = 32, H_PITCH = 40;   // in bf16 elements
+
+template <int ROWS>
+__device__ __forceinline__ void h_load_tile(const uint16_t *__restrict__ base, int64_t ld, int row0, int k0, int rows, int K,
+                                            uint4 (&v)[ROWS / 64]) {
+  // ROWS x 32 bf16 = ROWS*4 chunks of 16 bytes; 256 threads -> ROWS/64 chunks each.
+  int t = threadIdx.x;
+#pragma unroll
+  for (int i = 0; i < ROWS / 64; i++) {
+    int r = row0 + (t >> 2) + 64 * i, k = k0 + (t & 3) * 8;
+    uint4 x = make_uint4(0, 0, 0, 0);
+    if (r < rows && k < K) x = *reinterpret_cast<const uint4 *>(base + (int64_t)r * ld + k);   // K % 8 == 0 is required
+    v[i] = x;
+  }
+}
+template <int ROWS>
+__device__ __forceinline__ void h_store_tile(uint16_t *s, const uint4 (&v)[ROWS / 64]) {
+  int t = threadIdx.x;
+#pragma unroll
+  for (int i = 0; i < ROWS / 64; i++) {
+    int r = (t >> 2) + 64 * i, k = (t & 3) * 8;
+    *reinterpret_cast<uint4 *>(s + r * H_PITCH + k) = v[i];
+  }
+}
+
+// BM x BN block tile, 4 waves as WGM x WGN grid; each wave owns (BM/WGM) x (BN/WGN).
+template <int BM, int BN, int WGM, int WGN, class OUT>
+__global__ __launch_bounds__(256) void k_gemm_bf16_nt(GemmArgs g) {
+  constexpr int WM = BM / WGM, WN = BN / WGN, TM = WM / 32, TN = WN / 32;
+  extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+  uint16_t *As = smem;                                   // [2][BM][H_PITCH]
+  uint16_t *Bs = smem + 2 * BM * H_PITCH;                // [2][BN][H_PITCH]
+  int bz = blockIdx.z;
+  const uint16_t *A = (const uint16_t *)g.a + (int64_t)bz * g.sa;
+  const uint16_t *B = (const uint16_t *)g.b + (int64_t)bz * g.sb;
+  int64_t cbase = (int64_t)bz * g.sc;
+  // Tile order: consecutive blocks walk down M inside one N column so the B (weight) tile stays hot in L2.
+  int tiles_m = (g.M + BM - 1) / BM;
+  int bid = blockIdx.x;
+  int m0 = (bid % tiles_m) * BM, n0 = (bid / tiles_m) * BN;
+  int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  int wm = (wave / WGN) * WM, wn = (wave % WGN) * WN;
+  int lr = lane & 31, lk = lane >> 5;
+
+  f32x16 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
+
+  uint4 ra[BM / 64], rb[BN / 64];
+  int nt = (g.K + H_BK - 1) / H_BK;
+  h_load_tile<BM>(A, g.lda, m0, 0, g.M, g.K, ra);
+  h_load_tile<BN>(B, g.ldb, n0, 0, g.N, g.K, rb);
+  h_store_tile<BM>(As, ra);
+  h_store_tile<BN>(Bs, rb);
+  __syncthreads();
+  for (int t = 0; t < nt; t++) {
+    int cur = t & 1;
+    if (t + 1 < nt) {
+      h_load_tile<BM>(A, g.lda, m0, (t + 1) * H_BK, g.M, g.K, ra);
+      h_load_tile<BN>(B, g.ldb, n0, (t + 1) * H_BK, g.N, g.K, rb);
+    }
+    const uint16_t *as = As + cur * BM * H_PITCH, *bs = Bs + cur * BN * H_PITCH;
+#pragma unroll
+    for (int kk = 0; kk < H_BK / 16; kk++) {
+      bf16x8 fa[TM], fb[TN];
+#pragma unroll
+      for (int i = 0; i < TM; i++) fa[i] = *reinterpret_cast<const bf16x8 *>(as + (wm + 32 * i + lr) * H_PITCH + kk * 16 + lk * 8);
+#pragma unroll
+      for (int j = 0; j < TN; j++) fb[j] = *reinterpret_cast<const bf16x8 *>(bs + (wn + 32 * j + lr) * H_PITCH + kk * 16 + lk * 8);
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    }
+    if (t + 1 < nt) {
+      h_store_tile<BM>(As + (cur ^ 1) * BM * H_PITCH, ra);
+      h_store_tile<BN>(Bs + (cur ^ 1) * BN * H_PITCH, rb);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int e = 0; e < 16; e++) {
+        int row = m0 + wm + 32 * i + 8 * (e >> 2) + 4 * lk + (e & 3);
+        int col = n0 + wn + 32 * j + lr;
+        epilogue_store<OUT>(g, cbase, row, col, acc[i][j][e]);
+      }
+}
+
+// 16-bit [R][C] -> [C][R] through a 64x64 LDS tile (used to bring NN / TN operands into NT form)
+__global__ void k_transpose_u16(const uint16_t *__restrict__ in, int64_t ld_in, uint16_t *__restrict__ out, int64_t ld_out, int R, int C) {
+  __shared__ uint16_t tile[64][66];
+  int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+  for (int j = threadIdx.y; j < 64; j += blockDim.y) {
+    int r = r0 + j, c = c0 + threadIdx.x;
+    tile[j][threadIdx.x] = (r < R && c < C) ? in[(int64_t)r * ld_in + c] : (uint16_t)0;
+  }
+  __syncthreads();
+  for (int j = threadIdx.y; j < 64; j += blockDim.y) {
+    int c = c0 + j, r = r0 + threadIdx.x;
+    if (r < R && c < C) out[(int64_t)c * ld_out + r] = tile[threadIdx.x][j];
+  }
+}
+
+template <int BM, int BN, int WGM, int WGN>
+int32_t launch_bf16_nt(const GemmArgs &ga, int batch, int out_dtype) {
+  size_t lds = sizeof(uint16_t) * 2 * (size_t)(BM + BN) * H_PITCH;
+  int64_t tiles = cdiv(ga.M, BM) * cdiv(ga.N, BN);
+  dim3 grid((unsigned)tiles, 1, (unsigned)batch);
+  if (out_dtype == AH_F32) {
+    auto kfn = k_gemm_bf16_nt<BM, BN, WGM, WGN, float>;
+    if (lds > 64 * 1024) AH_HIP(hipFuncSetAttribute((const void *)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(kfn, grid, dim3(256), lds, stream(), ga);
+  } else {
+    auto kfn = k_gemm_bf16_nt<BM, BN, WGM, WGN, uint16_t>;
+    if (lds > 64 * 1024) AH_HIP(hipFuncSetAttribute((const void *)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(kfn, grid, dim3(256), lds, stream(), ga);
+  }
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+
+int32_t run_bf16_nt(const GemmArgs &ga, int batch, int out_dtype) {
+  // Tile choice: the largest tile that still yields at least ~2 waves of blocks over the CUs.
+  int64_t cus = num_cus();
+  auto blocks = [&](int bm, int bn) { return cdiv(ga.M, bm) * cdiv(ga.N, bn) * batch; };
+  if (ga.M >= 256 && ga.N >= 256 && blocks(256, 256) >= 2 * cus) return launch_bf16_nt<256, 256, 2, 2>(ga, batch, out_dtype);
+  if (ga.M >= 256 && ga.N >= 128 && blocks(256, 128) >= cus) return launch_bf16_nt<256, 128, 2, 2>(ga, batch, out_dtype);
+  return launch_bf16_nt<128, 128, 2, 2>(ga, batch, out_dtype);
+}
+
+template <int LAYOUT>
+int32_t launch_f32(const GemmArgs &ga, int batch, int out_dtype, int vec_a, int vec_b) {
+  dim3 grid((unsigned)cdiv(ga.N, F_BN), (unsigned)cdiv(ga.M, F_BM), (unsigned)batch);
+  if (out_dtype == AH_F32) hipLaunchKernelGGL((k_gemm_f32<LAYOUT, float>), grid, dim3(256), 0, stream(), ga, vec_a, vec_b);
+  else hipLaunchKernelGGL((k_gemm_f32<LAYOUT, uint16_t>), grid, dim3(256), 0, stream(), ga, vec_a, vec_b);
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t ah_gemm(const AhGemm *p) {
+  AH_REQUIRE_READY();
+  AH_ARG(p != nullptr, "ah_gemm: null descriptor");
+  const AhGemm &q = *p;
+  AH_ARG(q.layout >= AH_GEMM_NN && q.layout <= AH_GEMM_TN, "ah_gemm: bad layout %d", q.layout);
+  AH_ARG(q.in_dtype == AH_F32 || q.in_dtype == AH_BF16, "ah_gemm: operands must be f32 or bf16");
+  AH_ARG(q.out_dtype == AH_F32 || q.out_dtype == AH_BF16, "ah_gemm: output must be f32 or bf16");
+  AH_ARG(q.epilogue >= AH_EPI_NONE && q.epilogue <= AH_EPI_GELU_BWD, "ah_gemm: bad epilogue %d", q.epilogue);
+  AH_ARG(q.m >= 0 && q.n >= 0 && q.k >= 0 && q.batch >= 0, "ah_gemm: negative extent");
+  AH_ARG(q.m < (1ll << 31) && q.n < (1ll << 31) && q.k < (1ll << 31) && q.batch <= 65535, "ah_gemm: extent too large");
+  if (q.m == 0 || q.n == 0 || q.batch == 0) return AH_OK;
+  AH_ARG(q.c != 0, "ah_gemm: null C");
+  AH_ARG(q.k == 0 || (q.a != 0 && q.b != 0), "ah_gemm: null operand");
+  // minimum leading dimensions for the stated layout
+  int64_t a_cols = q.layout == AH_GEMM_TN ? q.m : q.k, b_cols = q.layout == AH_GEMM_NT ? q.k : q.n;
+  AH_ARG(q.lda >= a_cols && q.ldb >= b_cols && q.ldc >= q.n, "matmul shape mismatch: lda/ldb/ldc (%lld,%lld,%lld) too small for m=%lld n=%lld k=%lld",
+         (long long)q.lda, (long long)q.ldb, (long long)q.ldc, (long long)q.m, (long long)q.n, (long long)q.k);
+  if (q.epilogue == AH_EPI_GELU || q.epilogue == AH_EPI_RESIDUAL || q.epilogue == AH_EPI_GELU_BWD)
+    AH_ARG(q.aux != 0, "ah_gemm: epilogue %d needs aux", q.epilogue);
+
+  GemmArgs ga;
+  ga.a = dp<const void>(q.a); ga.b = dp<const void>(q.b); ga.c = dp<void>(q.c);
+  ga.aux = dp<const void>(q.aux); ga.aux_out = dp<void>(q.aux);
+  ga.M = (int)q.m; ga.N = (int)q.n; ga.K = (int)q.k;
+  ga.lda = q.lda; ga.ldb = q.ldb; ga.ldc = q.ldc;
+  ga.sa = q.stride_a; ga.sb = q.stride_b; ga.sc = q.stride_c;
+  ga.epi = q.epilogue;
+  int batch = (int)q.batch;
+
+  if (q.in_dtype == AH_F32) {
+    int vec_a = aligned16(q.a) && (q.lda % 4 == 0) && (q.stride_a % 4 == 0);
+    int vec_b = aligned16(q.b) && (q.ldb % 4 == 0) && (q.stride_b % 4 == 0);
+    switch (q.layout) {
+      case AH_GEMM_NN: return launch_f32<AH_GEMM_NN>(ga, batch, q.out_dtype, vec_a, vec_b);
+      case AH_GEMM_NT: return launch_f32<AH_GEMM_NT>(ga, batch, q.out_dtype, vec_a, vec_b);
+      default: return launch_f32<AH_GEMM_TN>(ga, batch, q.out_dtype, vec_a, vec_b);
+    }
+  }
+
+  // bf16: the MFMA kernel consumes K-contiguous operands; bring the others into that form.
+  AH_ARG(batch == 1 || q.layout == AH_GEMM_NT, "ah_gemm: batched bf16 is supported for the NT layout only");
+  AH_ARG(q.k % 8 == 0, "ah_gemm: bf16 contraction length %lld must be a multiple of 8", (long long)q.k);
+  ah_ptr ta = 0, tb = 0;
+  int32_t rc = AH_OK;
+  if (q.layout == AH_GEMM_TN) {           // A is [K][M] -> [M][K]
+    int64_t ldt = (q.k + 7) & ~7ll;
+    rc = ah_alloc((uint64_t)q.m * ldt * 2, &ta);
+    if (rc) return rc;
+    hipLaunchKernelGGL(k_transpose_u16, dim3((unsigned)cdiv(q.m, 64), (unsigned)cdiv(q.k, 64)), dim3(64, 4), 0, stream(),
+                       (const uint16_t *)ga.a, q.lda, dp<uint16_t>(ta), ldt, (int)q.k, (int)q.m);
+    AH_LAUNCH_CHECK();
+    ga.a = dp<const void>(ta); ga.lda = ldt;
+  }
+  if (q.layout != AH_GEMM_NT) {           // B is [K][N] -> [N][K]
+    int64_t ldt = (q.k + 7) & ~7ll;
+    rc = ah_alloc((uint64_t)q.n * ldt * 2, &tb);
+    if (rc) { if (ta) ah_free(ta); return rc; }
+    hipLaunchKernelGGL(k_transpose_u16, dim3((unsigned)cdiv(q.n, 64), (unsigned)cdiv(q.k, 64)), dim3(64, 4), 0, stream(),
+                       (const uint16_t *)ga.b, q.ldb, dp<uint16_t>(tb), ldt, (int)q.k, (int)q.n);
+    AH_LAUNCH_CHECK();
+    ga.b = dp<const void>(tb); ga.ldb = ldt;
+  }
+  if (!(((uintptr_t)ga.a & 15u) == 0 && ((uintptr_t)ga.b & 15u) == 0 && ga.lda % 8 == 0 && ga.ldb % 8 == 0 && ga.sa % 8 == 0 && ga.sb % 8 == 0)) {
+    if (ta) ah_free(ta);
+    if (tb) ah_free(tb);
+    return fail(AH_ERR_ARG, "ah_gemm: bf16 operands need 16-byte aligned rows (lda, ldb, batch strides multiples of 8)");
+  }
+  rc = run_bf16_nt(ga, batch, q.out_dtype);
+  if (ta) ah_free(ta);       // stream-ordered: reusable only by later work
+  if (tb) ah_free(tb);
+  return rc;
+}
+
+}  // extern "C"

@@ -1,0 +1,394 @@
+// Bandwidth-bound neural-network kernels: embedding gather / scatter-add, LayerNorm forward and
+// backward, softmax-cross-entropy forward and backward.  One wave64 owns one row; rows live in
+// registers between the statistics pass and the write, so each tensor is read once.
+#include "common.h"
+
+using namespace ah;
+
+namespace {
+
+constexpr int TPB = 256;
+constexpr int WPB = TPB / 64;
+
+// ---------------------------------------------------------------- embedding
+template <class OUT>
+__global__ void k_embedding(const float *__restrict__ w, const int32_t *__restrict__ idx, OUT *__restrict__ out,
+                            int64_t n_idx, int64_t dim, int64_t vocab) {
+  int64_t row = blockIdx.x * (int64_t)WPB + (threadIdx.x >> 6);
+  if (row >= n_idx) return;
+  int lane = threadIdx.x & 63;
+  int64_t r = idx[row];
+  bool ok = r >= 0 && r < vocab;                 // an out-of-range id yields a zero row instead of a fault
+  const float *src = w + (ok ? r : 0) * dim;
+  OUT *dst = out + row * dim;
+  for (int64_t j = lane; j < dim; j += 64) Io<OUT>::st(dst, j, ok ? src[j] : 0.f);
+}
+__global__ void k_embedding_tok_pos(const float *__restrict__ wte, const float *__restrict__ wpe, const int32_t *__restrict__ tok,
+                                    float *__restrict__ out, int64_t n_idx, int64_t T, int64_t dim, int64_t vocab) {
+  int64_t row = blockIdx.x * (int64_t)WPB + (threadIdx.x >> 6);
+  if (row >= n_idx) return;
+  int lane = threadIdx.x & 63;
+  int64_t r = tok[row];
+  bool ok = r >= 0 && r < vocab;
+  const float *a = wte + (ok ? r : 0) * dim, *b = wpe + (row % T) * dim;
+  float *dst = out + row * dim;
+  if ((dim & 3) == 0) {
+    for (int64_t j = lane; j < (dim >> 2); j += 64) {
+      float4 u = reinterpret_cast<const float4 *>(a)[j], v = reinterpret_cast<const float4 *>(b)[j];
+      if (!ok) u = make_float4(0, 0, 0, 0);
+      reinterpret_cast<float4 *>(dst)[j] = make_float4(u.x + v.x, u.y + v.y, u.z + v.z, u.w + v.w);
+    }
+  } else {
+    for (int64_t j = lane; j < dim; j += 64) dst[j] = (ok ? a[j] : 0.f) + b[j];
+  }
+}
+// scatter-add with hardware f32 atomics (the reference's GPU kernel uses CAS-loop atomics:
+// packages/helios/src/kernels/nn.ts:5300-5345); summation order is not fixed.
+__global__ void k_embedding_bwd(const int32_t *__restrict__ idx, const float *__restrict__ g, float *__restrict__ gw,
+                                int64_t n_idx, int64_t dim, int64_t vocab) {
+  int64_t row = blockIdx.x * (int64_t)WPB + (threadIdx.x >> 6);
+  if (row >= n_idx) return;
+  int lane = threadIdx.x & 63;
+  int64_t r = idx[row];
+  if (r < 0 || r >= vocab) return;
+  const float *src = g + row * dim;
+  float *dst = gw + r * dim;
+  for (int64_t j = lane; j < dim; j += 64) unsafeAtomicAdd(dst + j, src[j]);
+}
+__global__ void k_pos_embedding_bwd(const float *__restrict__ g, float *__restrict__ gw, int64_t batch, int64_t td, int accumulate) {
+  int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+  if (i >= td) return;
+  float s = accumulate ? gw[i] : 0.f;
+  for (int64_t b = 0; b < batch; b++) s += g[b * td + i];
+  gw[i] = s;
+}
+
+// ---------------------------------------------------------------- LayerNorm
+// NV = float4 per lane held in registers (row length <= 256*NV); NV == 0: generic re-reading path.
+template <int NV, class OUT>
+__global__ void k_layernorm(const float *__restrict__ x, const float *__restrict__ w, const float *__restrict__ b,
+                            OUT *__restrict__ out, int64_t rows, int dim, float eps) {
+  int64_t row = blockIdx.x * (int64_t)WPB + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  int lane = threadIdx.x & 63;
+  const float *xr = x + row * (int64_t)dim;
+  OUT *orow = out + row * (int64_t)dim;
+  float inv_dim = 1.0f / (float)dim;
+  if constexpr (NV > 0) {
+    int nv = dim >> 2;
+    float4 v[NV > 0 ? NV : 1];
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+      int j = lane + 64 * i;
+      v[i] = j < nv ? reinterpret_cast<const float4 *>(xr)[j] : make_float4(0, 0, 0, 0);
+      s += (v[i].x + v[i].y) + (v[i].z + v[i].w);
+    }
+    float mean = wave_sum(s) * inv_dim;
+    float q = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+      int j = lane + 64 * i;
+      if (j < nv) {
+        float a = v[i].x - mean, c = v[i].y - mean, d = v[i].z - mean, e = v[i].w - mean;
+        q += (a * a + c * c) + (d * d + e * e);
+      }
+    }
+    float rstd = 1.0f / sqrtf(wave_sum(q) * inv_dim + eps);
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+      int j = lane + 64 * i;
+      if (j < nv) {
+        float4 ww = reinterpret_cast<const float4 *>(w)[j], bb = reinterpret_cast<const float4 *>(b)[j];
+        float o0 = (v[i].x - mean) * rstd * ww.x + bb.x, o1 = (v[i].y - mean) * rstd * ww.y + bb.y;
+        float o2 = (v[i].z - mean) * rstd * ww.z + bb.z, o3 = (v[i].w - mean) * rstd * ww.w + bb.w;
+        Io<OUT>::st(orow, 4 * j + 0, o0); Io<OUT>::st(orow, 4 * j + 1, o1);
+        Io<OUT>::st(orow, 4 * j + 2, o2); Io<OUT>::st(orow, 4 * j + 3, o3);
+      }
+    }
+  } else {
+    float s = 0.f;
+    for (int j = lane; j < dim; j += 64) s += xr[j];
+    float mean = wave_sum(s) * inv_dim;
+    float q = 0.f;
+    for (int j = lane; j < dim; j += 64) { float d = xr[j] - mean; q += d * d; }
+    float rstd = 1.0f / sqrtf(wave_sum(q) * inv_dim + eps);
+    for (int j = lane; j < dim; j += 64) Io<OUT>::st(orow, j, (xr[j] - mean) * rstd * w[j] + b[j]);
+  }
+}
+
+// Backward.  Each wave walks rows r = wave_global, += total_waves; per row it recomputes mean / rstd,
+// writes dx (+ residual gradient), and adds g*xhat and g into per-lane column accumulators.  The four
+// waves of a block then combine through LDS into one partial row of dw/db per block; a second kernel
+// sums the partials column-wise in fixed order (deterministic, no [rows, dim] temporaries).
+template <class G>
+__global__ void k_layernorm_bwd(const float *__restrict__ x, const float *__restrict__ w, const G *__restrict__ g,
+                                const float *__restrict__ res, float *__restrict__ dx, float *__restrict__ part_dw,
+                                float *__restrict__ part_db, int64_t rows, int dim, float eps) {
+  extern __shared__ float sh[];      // [2][WPB][dim]
+  int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  float *my_dw = sh + (size_t)wave * dim, *my_db = sh + (size_t)(WPB + wave) * dim;
+  for (int j = lane; j < dim; j += 64) { my_dw[j] = 0.f; my_db[j] = 0.f; }
+  float inv_dim = 1.0f / (float)dim;
+  int64_t stride = (int64_t)gridDim.x * WPB;
+  for (int64_t row = blockIdx.x * (int64_t)WPB + wave; row < rows; row += stride) {
+    const float *xr = x + row * (int64_t)dim;
+    const G *gr = g + row * (int64_t)dim;
+    float s = 0.f;
+    for (int j = lane; j < dim; j += 64) s += xr[j];
+    float mean = wave_sum(s) * inv_dim;
+    float q = 0.f;
+    for (int j = lane; j < dim; j += 64) { float d = xr[j] - mean; q += d * d; }
+    float rstd = 1.0f / sqrtf(wave_sum(q) * inv_dim + eps);
+    float s1 = 0.f, s2 = 0.f;
+    for (int j = lane; j < dim; j += 64) {
+      float gv = Io<G>::ld(gr, j), xh = (xr[j] - mean) * rstd, dy = gv * w[j];
+      s1 += dy; s2 += dy * xh;
+      my_dw[j] += gv * xh; my_db[j] += gv;
+    }
+    s1 = wave_sum(s1); s2 = wave_sum(s2);
+    for (int j = lane; j < dim; j += 64) {
+      float gv = Io<G>::ld(gr, j), xh = (xr[j] - mean) * rstd, dy = gv * w[j];
+      float d = rstd * (dy - (s1 + xh * s2) * inv_dim);
+      if (res) d += res[row * (int64_t)dim + j];
+      dx[row * (int64_t)dim + j] = d;
+    }
+  }
+  __syncthreads();
+  for (int j = threadIdx.x; j < dim; j += blockDim.x) {
+    float a = 0.f, c = 0.f;
+    for (int k = 0; k < WPB; k++) { a += sh[(size_t)k * dim + j]; c += sh[(size_t)(WPB + k) * dim + j]; }
+    part_dw[(size_t)blockIdx.x * dim + j] = a;
+    part_db[(size_t)blockIdx.x * dim + j] = c;
+  }
+}
+__global__ void k_colsum_partials(const float *__restrict__ part_dw, const float *__restrict__ part_db, int nparts, int dim,
+                                  float *__restrict__ dw, float *__restrict__ db, int accumulate) {
+  int j = blockIdx.x * blockDim.x + threadIdx.x;
+  if (j >= dim) return;
+  double a = 0, c = 0;
+  for (int p = 0; p < nparts; p++) { a += part_dw[(size_t)p * dim + j]; c += part_db[(size_t)p * dim + j]; }
+  dw[j] = (accumulate ? dw[j] : 0.f) + (float)a;
+  db[j] = (accumulate ? db[j] : 0.f) + (float)c;
+}
+
+// ---------------------------------------------------------------- softmax cross-entropy
+__device__ __forceinline__ void online_merge(float &m, float &s, float m2, float s2) {
+  float nm = fmaxf(m, m2);
+  if (nm == -INFINITY) { m = nm; s = 0.f; return; }
+  s = s * expf(m - nm) + s2 * expf(m2 - nm);
+  m = nm;
+}
+// one block per row: single read of the row with an online (max, sum-exp) pair per thread
+template <class T>
+__global__ void k_ce_fwd(const T *__restrict__ logits, const int32_t *__restrict__ targets, float *__restrict__ row_loss,
+                         float *__restrict__ lse_out, int64_t c) {
+  __shared__ float shm[WPB], shs[WPB];
+  int64_t row = blockIdx.x;
+  const T *p = logits + row * c;
+  float m = -INFINITY, s = 0.f;
+  for (int64_t j = threadIdx.x; j < c; j += blockDim.x) {
+    float v = Io<T>::ld(p, j);
+    if (v > m) { s = s * expf(m - v) + 1.0f; m = v; } else { s += expf(v - m); }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) online_merge(m, s, __shfl_xor(m, off, 64), __shfl_xor(s, off, 64));
+  int wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  if (lane == 0) { shm[wv] = m; shs[wv] = s; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int k = 1; k < WPB; k++) online_merge(m, s, shm[k], shs[k]);
+    float lse = m + logf(s);
+    int32_t t = targets[row];
+    float picked = (t >= 0 && t < c) ? Io<T>::ld(p, t) : lse;     // an out-of-range target contributes 0 loss
+    row_loss[row] = lse - picked;
+    if (lse_out) lse_out[row] = lse;
+  }
+}
+__global__ void k_mean_rows(const float *__restrict__ v, int64_t n, float *__restrict__ out) {
+  __shared__ double sh[WPB];
+  double s = 0;
+  for (int64_t i = threadIdx.x; i < n; i += blockDim.x) s += (double)v[i];
+  s = wave_sum_d(s);
+  if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = s;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    double t = 0;
+    for (int k = 0; k < WPB; k++) t += sh[k];
+    out[0] = (float)(t / (double)n);
+  }
+}
+template <class T>
+__global__ void k_ce_bwd(const T *__restrict__ logits, const int32_t *__restrict__ targets, const float *__restrict__ lse,
+                         const float *__restrict__ g, float g_mul, T *__restrict__ out, int64_t n, int64_t c) {
+  int64_t row = blockIdx.y;
+  float scale = (g ? g[0] : 1.0f) * g_mul / (float)n;
+  float l = lse[row];
+  int32_t t = targets[row];
+  const T *p = logits + row * c;
+  T *q = out + row * c;
+  for (int64_t j = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; j < c; j += (int64_t)gridDim.x * blockDim.x) {
+    float prob = expf(Io<T>::ld(p, j) - l);
+    Io<T>::st(q, j, (prob - (j == t ? 1.0f : 0.0f)) * scale);
+  }
+}
+
+}  // namespace
+
+template <class OUT>
+static int32_t launch_ln(ah_ptr x, ah_ptr w, ah_ptr b, ah_ptr out, int64_t rows, int64_t dim, float eps) {
+  dim3 grid((unsigned)cdiv(rows, WPB)), blk(TPB);
+  bool vec = (dim % 4 == 0) && dim <= 2048 && aligned16(x) && aligned16(w) && aligned16(b);
+  int nvl = vec ? (int)cdiv(dim / 4, 64) : 0;
+#define LN_CASE(NV) hipLaunchKernelGGL((k_layernorm<NV, OUT>), grid, blk, 0, stream(), dp<const float>(x), dp<const float>(w), dp<const float>(b), dp<OUT>(out), rows, (int)dim, eps)
+  switch (nvl) {
+    case 1: LN_CASE(1); break;
+    case 2: LN_CASE(2); break;
+    case 3: LN_CASE(3); break;
+    case 4: LN_CASE(4); break;
+    case 5: case 6: LN_CASE(6); break;
+    case 7: case 8: LN_CASE(8); break;
+    default: LN_CASE(0); break;
+  }
+#undef LN_CASE
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+
+extern "C" {
+
+int32_t ah_embedding(ah_ptr weight, ah_ptr idx, ah_ptr out, int64_t n_idx, int64_t dim, int64_t vocab, int32_t out_dtype) {
+  AH_REQUIRE_READY();
+  AH_ARG(out_dtype == AH_F32 || out_dtype == AH_BF16, "ah_embedding: out dtype must be f32 or bf16");
+  if (n_idx == 0 || dim == 0) return AH_OK;
+  AH_ARG(weight && idx && out, "ah_embedding: null operand");
+  dim3 grid((unsigned)cdiv(n_idx, WPB));
+  if (out_dtype == AH_F32)
+    hipLaunchKernelGGL(k_embedding<float>, grid, dim3(TPB), 0, stream(), dp<const float>(weight), dp<const int32_t>(idx), dp<float>(out), n_idx, dim, vocab);
+  else
+    hipLaunchKernelGGL(k_embedding<uint16_t>, grid, dim3(TPB), 0, stream(), dp<const float>(weight), dp<const int32_t>(idx), dp<uint16_t>(out), n_idx, dim, vocab);
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+
+int32_t ah_embedding_tok_pos(ah_ptr wte, ah_ptr wpe, ah_ptr tok, ah_ptr out, int64_t n_idx, int64_t T, int64_t dim, int64_t vocab) {
+  AH_REQUIRE_READY();
+  if (n_idx == 0 || dim == 0) return AH_OK;
+  AH_ARG(wte && wpe && tok && out && T > 0, "ah_embedding_tok_pos: null operand");
+  AH_ARG(aligned16(wte) && aligned16(wpe) && aligned16(out), "ah_embedding_tok_pos: operands must be 16-byte aligned");
+  hipLaunchKernelGGL(k_embedding_tok_pos, dim3((unsigned)cdiv(n_idx, WPB)), dim3(TPB), 0, stream(), dp<const float>(wte),
+                     dp<const float>(wpe), dp<const int32_t>(tok), dp<float>(out), n_idx, T, dim, vocab);
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+
+int32_t ah_embedding_bwd(ah_ptr idx, ah_ptr grad_out, ah_ptr grad_w, int64_t n_idx, int64_t dim, int64_t vocab, int32_t accumulate) {
+  AH_REQUIRE_READY();
+  AH_ARG(grad_w != 0 || vocab * dim == 0, "ah_embedding_bwd: null grad_w");
+  if (!accumulate) { int32_t rc = ah_fill_f32(grad_w, 0.f, (uint64_t)(vocab * dim)); if (rc) return rc; }
+  if (n_idx == 0 || dim == 0) return AH_OK;
+  AH_ARG(idx && grad_out, "ah_embedding_bwd: null operand");
+  hipLaunchKernelGGL(k_embedding_bwd, dim3((unsigned)cdiv(n_idx, WPB)), dim3(TPB), 0, stream(), dp<const int32_t>(idx),
+                     dp<const float>(grad_out), dp<float>(grad_w), n_idx, dim, vocab);
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+
+int32_t ah_pos_embedding_bwd(ah_ptr grad_out, ah_ptr grad_wpe, int64_t batch, int64_t T, int64_t dim, int32_t accumulate) {
+  AH_REQUIRE_READY();
+  int64_t td = T * dim;
+  if (td == 0) return AH_OK;
+  AH_ARG(grad_out && grad_wpe, "ah_pos_embedding_bwd: null operand");
+  hipLaunchKernelGGL(k_pos_embedding_bwd, dim3((unsigned)cdiv(td, TPB)), dim3(TPB), 0, stream(), dp<const float>(grad_out),
+                     dp<float>(grad_wpe), batch, td, accumulate);
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+
+int32_t ah_layernorm(ah_ptr x, ah_ptr w, ah_ptr b, ah_ptr out, int64_t rows, int64_t dim, float eps, int32_t out_dtype) {
+  AH_REQUIRE_READY();
+  AH_ARG(out_dtype == AH_F32 || out_dtype == AH_BF16, "ah_layernorm: out dtype must be f32 or bf16");
+  if (rows == 0 || dim == 0) return AH_OK;
+  AH_ARG(x && w && b && out, "ah_layernorm: null operand");
+  AH_ARG(dim < (int64_t(1) << 30), "ah_layernorm: row too long");
+  return out_dtype == AH_F32 ? launch_ln<float>(x, w, b, out, rows, dim, eps) : launch_ln<uint16_t>(x, w, b, out, rows, dim, eps);
+}
+
+int32_t ah_layernorm_bwd(ah_ptr x, ah_ptr w, ah_ptr grad_out, int32_t grad_dtype, ah_ptr residual_grad, ah_ptr dx, ah_ptr dw,
+                         ah_ptr db, int64_t rows, int64_t dim, float eps, int32_t accumulate) {
+  AH_REQUIRE_READY();
+  AH_ARG(grad_dtype == AH_F32 || grad_dtype == AH_BF16, "ah_layernorm_bwd: grad dtype must be f32 or bf16");
+  if (dim == 0) return AH_OK;
+  AH_ARG(dw && db, "ah_layernorm_bwd: null dw/db");
+  if (rows == 0) {
+    if (!accumulate) { int32_t rc = ah_fill_f32(dw, 0.f, (uint64_t)dim); if (rc) return rc; return ah_fill_f32(db, 0.f, (uint64_t)dim); }
+    return AH_OK;
+  }
+  AH_ARG(x && w && grad_out && dx, "ah_layernorm_bwd: null operand");
+  size_t lds = sizeof(float) * 2 * WPB * (size_t)dim;
+  AH_ARG(lds <= 160 * 1024, "ah_layernorm_bwd: dim %lld too large for the LDS column accumulators", (long long)dim);
+  int nblk = (int)cdiv(rows, WPB * 8);            // >= 8 rows per wave amortises the partial write
+  int cap = num_cus() * 2;
+  if (nblk > cap) nblk = cap;
+  if (nblk < 1) nblk = 1;
+  float *part = (float *)scratch(sizeof(float) * 2 * (size_t)nblk * (size_t)dim);
+  if (!part) return fail(AH_ERR_OOM, "ah_layernorm_bwd: no scratch");
+  float *part_dw = part, *part_db = part + (size_t)nblk * dim;
+  if (grad_dtype == AH_F32)
+    hipLaunchKernelGGL(k_layernorm_bwd<float>, dim3(nblk), dim3(TPB), lds, stream(), dp<const float>(x), dp<const float>(w),
+                       dp<const float>(grad_out), dp<const float>(residual_grad), dp<float>(dx), part_dw, part_db, rows, (int)dim, eps);
+  else
+    hipLaunchKernelGGL(k_layernorm_bwd<uint16_t>, dim3(nblk), dim3(TPB), lds, stream(), dp<const float>(x), dp<const float>(w),
+                       dp<const uint16_t>(grad_out), dp<const float>(residual_grad), dp<float>(dx), part_dw, part_db, rows, (int)dim, eps);
+  AH_LAUNCH_CHECK();
+  hipLaunchKernelGGL(k_colsum_partials, dim3((unsigned)cdiv(dim, TPB)), dim3(TPB), 0, stream(), part_dw, part_db, nblk, (int)dim,
+                     dp<float>(dw), dp<float>(db), accumulate);
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+
+int32_t ah_cross_entropy(ah_ptr logits, int32_t dtype, ah_ptr targets, ah_ptr loss_out, ah_ptr lse_out, int64_t n, int64_t c) {
+  AH_REQUIRE_READY();
+  AH_ARG(dtype == AH_F32 || dtype == AH_BF16, "ah_cross_entropy: logits dtype must be f32 or bf16");
+  AH_ARG(loss_out != 0, "ah_cross_entropy: null loss_out");
+  AH_ARG(n > 0 && c > 0, "ah_cross_entropy: empty logits [%lld, %lld]", (long long)n, (long long)c);
+  AH_ARG(logits && targets, "ah_cross_entropy: null operand");
+  AH_ARG(n < (int64_t(1) << 31), "ah_cross_entropy: too many rows");
+  float *rows = (float *)scratch(sizeof(float) * (size_t)n);
+  if (!rows) return fail(AH_ERR_OOM, "ah_cross_entropy: no scratch");
+  if (dtype == AH_F32)
+    hipLaunchKernelGGL(k_ce_fwd<float>, dim3((unsigned)n), dim3(TPB), 0, stream(), dp<const float>(logits), dp<const int32_t>(targets), rows, dp<float>(lse_out), c);
+  else
+    hipLaunchKernelGGL(k_ce_fwd<uint16_t>, dim3((unsigned)n), dim3(TPB), 0, stream(), dp<const uint16_t>(logits), dp<const int32_t>(targets), rows, dp<float>(lse_out), c);
+  AH_LAUNCH_CHECK();
+  hipLaunchKernelGGL(k_mean_rows, dim3(1), dim3(TPB), 0, stream(), rows, n, dp<float>(loss_out));
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+
+int32_t ah_cross_entropy_bwd(ah_ptr logits, int32_t dtype, ah_ptr targets, ah_ptr lse, ah_ptr g_scalar, float g_mul, ah_ptr dlogits,
+                             int64_t n, int64_t c) {
+  AH_REQUIRE_READY();
+  AH_ARG(dtype == AH_F32 || dtype == AH_BF16, "ah_cross_entropy_bwd: dtype must be f32 or bf16");
+  if (n == 0 || c == 0) return AH_OK;
+  AH_ARG(logits && targets && lse && dlogits, "ah_cross_entropy_bwd: null operand");
+  AH_ARG(n <= 65535 * 1024ll, "ah_cross_entropy_bwd: too many rows");
+  unsigned gx = (unsigned)cdiv(c, TPB * 8);
+  if (gx < 1) gx = 1;
+  // gridDim.y is limited to 65535: fold rows beyond that by launching in row chunks
+  for (int64_t r0 = 0; r0 < n; r0 += 65535) {
+    int64_t nr = n - r0 < 65535 ? n - r0 : 65535;
+    size_t esz = dtype == AH_F32 ? 4 : 2;
+    ah_ptr lg = logits + (uint64_t)(r0 * c) * esz, dl = dlogits + (uint64_t)(r0 * c) * esz;
+    if (dtype == AH_F32)
+      hipLaunchKernelGGL(k_ce_bwd<float>, dim3(gx, (unsigned)nr), dim3(TPB), 0, stream(), dp<const float>(lg),
+                         dp<const int32_t>(targets) + r0, dp<const float>(lse) + r0, dp<const float>(g_scalar), g_mul, dp<float>(dl), n, c);
+    else
+      hipLaunchKernelGGL(k_ce_bwd<uint16_t>, dim3(gx, (unsigned)nr), dim3(TPB), 0, stream(), dp<const uint16_t>(lg),
+                         dp<const int32_t>(targets) + r0, dp<const float>(lse) + r0, dp<const float>(g_scalar), g_mul, dp<uint16_t>(dl), n, c);
+    AH_LAUNCH_CHECK();
+  }
+  return AH_OK;
+}
+
+}  // extern "C"

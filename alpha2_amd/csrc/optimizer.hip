@@ -1,0 +1,87 @@
+// Fused AdamW and the device-side clip coefficient (packages/train/src/optimizers.ts:76-92;
+// packages/train/src/trainer.ts:1650-1656).  Single pass: 4 f32 reads + 3 f32 writes per element
+// (+ one bf16 write when a shadow copy for the next step's MFMA operands is requested).
+#include "common.h"
+
+using namespace ah;
+
+namespace {
+
+constexpr int TPB = 256;
+
+__device__ __forceinline__ void adam_one(float &p, float g, float &m, float &v, const AhAdamW &h, float gs) {
+  g *= gs;
+  if (h.weight_decay > 0.f) p -= h.lr * h.weight_decay * p;
+  m = h.beta1 * m + (1.0f - h.beta1) * g;
+  v = h.beta2 * v + (1.0f - h.beta2) * g * g;
+  float mh = m / h.bc1, vh = v / h.bc2;
+  p -= h.lr * mh / (sqrtf(vh) + h.eps);
+}
+
+__global__ void k_adamw(float *__restrict__ p, const float *__restrict__ g, float *__restrict__ m, float *__restrict__ v,
+                        uint64_t n, AhAdamW h, const AhAdamW *__restrict__ dev_h, const float *__restrict__ dev_scale,
+                        uint16_t *__restrict__ shadow, int vec) {
+  if (dev_h) { float wd = h.weight_decay; h = *dev_h; h.weight_decay = wd; }   // weight decay stays per tensor
+  float gs = h.grad_scale * (dev_scale ? dev_scale[0] : 1.0f);
+  uint64_t tid = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x, stride = (uint64_t)gridDim.x * blockDim.x;
+  uint64_t start = 0;
+  if (vec) {
+    uint64_t n4 = n >> 2;
+    for (uint64_t i = tid; i < n4; i += stride) {
+      float4 pp = reinterpret_cast<float4 *>(p)[i], gg = reinterpret_cast<const float4 *>(g)[i];
+      float4 mm = reinterpret_cast<float4 *>(m)[i], vv = reinterpret_cast<float4 *>(v)[i];
+      adam_one(pp.x, gg.x, mm.x, vv.x, h, gs); adam_one(pp.y, gg.y, mm.y, vv.y, h, gs);
+      adam_one(pp.z, gg.z, mm.z, vv.z, h, gs); adam_one(pp.w, gg.w, mm.w, vv.w, h, gs);
+      reinterpret_cast<float4 *>(p)[i] = pp; reinterpret_cast<float4 *>(m)[i] = mm; reinterpret_cast<float4 *>(v)[i] = vv;
+      if (shadow) {
+        uint2 s; s.x = pack_bf16x2(pp.x, pp.y); s.y = pack_bf16x2(pp.z, pp.w);
+        reinterpret_cast<uint2 *>(shadow)[i] = s;
+      }
+    }
+    start = n4 << 2;
+  }
+  for (uint64_t i = start + tid; i < n; i += stride) {
+    float pp = p[i], mm = m[i], vv = v[i];
+    adam_one(pp, g[i], mm, vv, h, gs);
+    p[i] = pp; m[i] = mm; v[i] = vv;
+    if (shadow) shadow[i] = f32_to_bf16_bits(pp);
+  }
+}
+
+__global__ void k_clip_coef(const float *__restrict__ sumsq, float grad_scale, float clip, float *__restrict__ out) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) {
+    float norm = sqrtf(sumsq[0]) * fabsf(grad_scale);
+    out[0] = (clip > 0.f && norm > clip) ? clip / norm : 1.0f;
+    out[1] = norm;
+  }
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t ah_adamw(ah_ptr p, ah_ptr g, ah_ptr m, ah_ptr v, uint64_t n, const AhAdamW *h, ah_ptr dev_hyper, ah_ptr dev_scale,
+                 ah_ptr bf16_shadow) {
+  AH_REQUIRE_READY();
+  AH_ARG(h != nullptr, "ah_adamw: null hyper-parameters");
+  if (n == 0) return AH_OK;
+  AH_ARG(p && g && m && v, "ah_adamw: null operand");
+  int vec = aligned16(p) && aligned16(g) && aligned16(m) && aligned16(v) && ((bf16_shadow & 7u) == 0);
+  int64_t blocks = cdiv((int64_t)(vec ? n / 4 + 1 : n), TPB);
+  int64_t cap = (int64_t)num_cus() * 16;
+  if (blocks > cap) blocks = cap;
+  hipLaunchKernelGGL(k_adamw, dim3((unsigned)blocks), dim3(TPB), 0, stream(), dp<float>(p), dp<const float>(g), dp<float>(m),
+                     dp<float>(v), n, *h, dp<const AhAdamW>(dev_hyper), dp<const float>(dev_scale), dp<uint16_t>(bf16_shadow), vec);
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+
+int32_t ah_clip_coef(ah_ptr sumsq, float grad_scale, float clip, ah_ptr out2) {
+  AH_REQUIRE_READY();
+  AH_ARG(sumsq && out2, "ah_clip_coef: null operand");
+  hipLaunchKernelGGL(k_clip_coef, dim3(1), dim3(64), 0, stream(), dp<const float>(sumsq), grad_scale, clip, dp<float>(out2));
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,269 @@
+/*
+ * alpha_hip.h -- flat C ABI of libalpha_hip.so, the MI355X (gfx950) compute backend for the GPT
+ * training step of alpha2.  This is the seam a Bun-FFI / N-API / ctypes shim binds; it replaces the
+ * reference's only native seam, the N-API addon `helios_vk.c` (export table
+ * packages/helios/native/helios_vk.c:4403-4432, typed in packages/helios/src/device.ts:17-39), and
+ * provides one entry point per operation of the reference's `Backend` interface
+ * (packages/core/src/interfaces.ts:38-151) that the training step reaches.
+ *
+ * Conventions
+ *   - Every function returns int32 status, 0 = OK; ah_last_error() gives the message.  No C++
+ *     exception crosses this boundary.  (Reference: napi_throw_error, helios_vk.c:3367,3405.)
+ *   - Device memory is named by opaque uint64 handles that ARE device addresses; a handle plus a
+ *     byte offset is a valid operand (views).  Only handles returned by ah_alloc may be freed.
+ *   - Tensors are row-major contiguous unless a leading-dimension argument says otherwise.
+ *   - One caller thread.  All work is enqueued on one persistent HIP stream in call order;
+ *     ah_sync, ah_download and ah_event_elapsed_ms are the only blocking calls.
+ *   - dtype codes: AH_F32 activations/params/grads, AH_BF16 internal fast-mode storage,
+ *     AH_I32 indices, AH_F16 storage-only cast target (the reference's Dtype has no bf16:
+ *     packages/core/src/types.ts:6).
+ */
+#ifndef ALPHA_HIP_H
+#define ALPHA_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef uint64_t ah_ptr;
+
+enum { AH_F32 = 0, AH_BF16 = 1, AH_I32 = 2, AH_F16 = 3 };
+
+enum {
+  AH_OK = 0,
+  AH_ERR_HIP = 1,        /* a HIP runtime call failed */
+  AH_ERR_ARG = 2,        /* shape / dtype / alignment mismatch (reference: thrown Error, cpu_ref.ts:172-182) */
+  AH_ERR_STATE = 3,      /* not initialised, or call illegal while a graph is being captured */
+  AH_ERR_OOM = 4,
+  AH_ERR_UNSUPPORTED = 5
+};
+
+/* ---- device / lifetime.  Replaces initDevice / destroy / waitIdle (helios_vk.c:4405-4425). ---- */
+typedef struct {
+  char     name[128];
+  char     arch[32];          /* "gfx950..." */
+  int32_t  compute_units;
+  int32_t  wavefront;
+  int32_t  clock_khz;
+  int32_t  lds_bytes_per_block;
+  uint64_t hbm_bytes;
+} AhDeviceInfo;
+
+int32_t     ah_init(int32_t device);
+int32_t     ah_shutdown(void);
+const char *ah_last_error(void);
+int32_t     ah_device_info(AhDeviceInfo *out);
+int32_t     ah_sync(void);
+
+/* ---- buffers.  Replaces createBuffer / uploadBuffer / fillBuffer / readBuffer / destroyBuffer
+ *      (helios_vk.c:4407-4412).  Frees are stream-ordered: a freed block is only ever reused by
+ *      work enqueued later on the same stream. ---- */
+int32_t ah_alloc(uint64_t bytes, ah_ptr *out);
+int32_t ah_free(ah_ptr p);
+int32_t ah_upload(ah_ptr dst, const void *host, uint64_t bytes);      /* host buffer borrowed for the call only */
+int32_t ah_download(void *host, ah_ptr src, uint64_t bytes);          /* blocks until data has landed */
+int32_t ah_copy(ah_ptr dst, ah_ptr src, uint64_t bytes);              /* device to device */
+int32_t ah_fill_f32(ah_ptr dst, float value, uint64_t n);
+int32_t ah_fill_i32(ah_ptr dst, int32_t value, uint64_t n);
+
+/* Counters the reference trainer polls through gpuMemStats()/gpuOpsThisStep/resetStepOps
+ * (packages/train/src/trainer.ts:1003-1032,1821-1843,1915). */
+typedef struct {
+  uint64_t live_allocs;
+  uint64_t live_bytes;
+  uint64_t pool_blocks;
+  uint64_t pool_bytes;
+  uint64_t device_mallocs;      /* hipMalloc calls so far */
+  uint64_t ops_launched;        /* kernels enqueued since ah_reset_op_count */
+  uint64_t graphs_live;
+} AhStats;
+int32_t ah_stats(AhStats *out);
+int32_t ah_reset_op_count(void);
+int32_t ah_trim_pool(void);      /* purgeBufferPools (trainer.ts:1012): return cached blocks to the driver */
+
+/* ---- whole-step capture.  Replaces batchBegin / batchSubmit / batchExecuteAll
+ *      (helios_vk.c:4414-4419): everything enqueued between begin and end becomes one hipGraph.
+ *      Blocks allocated while capturing belong to the graph until ah_graph_destroy. ---- */
+int32_t ah_graph_begin(void);
+int32_t ah_graph_end(uint64_t *out_graph);
+int32_t ah_graph_launch(uint64_t graph);
+int32_t ah_graph_destroy(uint64_t graph);
+
+/* ---- timing on the library stream.  Replaces gpuTime (helios_vk.c:3448). ---- */
+int32_t ah_event_create(uint64_t *out_event);
+int32_t ah_event_record(uint64_t event);
+int32_t ah_event_elapsed_ms(uint64_t start, uint64_t stop, float *out_ms);   /* blocks on `stop` */
+int32_t ah_event_destroy(uint64_t event);
+
+/* ---- element-wise, f32.  Backend.add/sub/mul/div/neg/exp/log/sqrt/pow/scale/clamp/gelu/relu/silu
+ *      (interfaces.ts:49-73; cpu_ref.ts:150-164,334-360,422-435). ---- */
+enum { AH_ADD = 0, AH_SUB = 1, AH_MUL = 2, AH_DIV = 3 };
+enum { AH_NEG = 0, AH_EXP = 1, AH_LOG = 2, AH_SQRT = 3, AH_POW = 4, AH_SCALE = 5, AH_CLAMP = 6,
+       AH_GELU = 7, AH_RELU = 8, AH_SILU = 9, AH_SOFTCAP = 10 };
+/* same-shape binary */
+int32_t ah_binary(int32_t op, ah_ptr a, ah_ptr b, ah_ptr out, uint64_t n);
+/* NumPy-broadcast binary: out has `nd` dims `shape`; a/b element strides per dim (0 = broadcast)
+ * (packages/core/src/broadcast.ts:13-65). nd <= 6. */
+int32_t ah_binary_broadcast(int32_t op, ah_ptr a, ah_ptr b, ah_ptr out, int32_t nd,
+                            const int64_t *shape, const int64_t *stride_a, const int64_t *stride_b);
+int32_t ah_unary(int32_t op, ah_ptr x, ah_ptr out, uint64_t n, float p0, float p1);
+/* in place: Backend.addInplace / scaleInplace (interfaces.ts:113-114) */
+int32_t ah_add_inplace(ah_ptr a, ah_ptr b, uint64_t n);
+int32_t ah_scale_inplace(ah_ptr a, float s, uint64_t n);
+/* a[i] += b[i] * s  -- loss accumulation over micro-steps (trainer.ts:1208-1223) without a temporary */
+int32_t ah_axpy_inplace(ah_ptr a, ah_ptr b, float s, uint64_t n);
+
+/* backward element-wise: Backend.geluBackward/reluBackward/siluBackward/clampBackward/
+ * softCapBackward/siluMul/siluMulBackward (interfaces.ts:96-106; CPU fallbacks ops.ts:284-417) */
+enum { AH_GELU_BWD = 0, AH_RELU_BWD = 1, AH_SILU_BWD = 2, AH_CLAMP_BWD = 3, AH_SOFTCAP_BWD = 4 };
+int32_t ah_unary_bwd(int32_t op, ah_ptr x, ah_ptr grad_out, ah_ptr out, uint64_t n, float p0, float p1);
+int32_t ah_silu_mul(ah_ptr a, ah_ptr b, ah_ptr out, uint64_t n);
+int32_t ah_silu_mul_bwd(ah_ptr a, ah_ptr b, ah_ptr grad_out, ah_ptr da, ah_ptr db, uint64_t n);
+/* Backend.residualDropoutAdd: out = residual + projected*mask (interfaces.ts:110; mask may be 0 = no dropout) */
+int32_t ah_residual_dropout_add(ah_ptr residual, ah_ptr projected, ah_ptr mask, ah_ptr out, uint64_t n);
+/* Backend.dropoutMask: u32-wrapping splitmix hash of (seed, counter, i) > p ? 1/(1-p) : 0
+ * (interfaces.ts:125; packages/helios/src/kernels/nn.ts:5600-5748) */
+int32_t ah_dropout_mask(ah_ptr out, uint64_t n, int32_t seed, int32_t counter, float p);
+/* Backend.maskedFill with the mask tiled by i % mask_n (cpu_ref.ts:891-911) */
+int32_t ah_masked_fill(ah_ptr a, ah_ptr mask, ah_ptr out, uint64_t n, uint64_t mask_n, float value);
+/* Backend.causalMask (cpu_ref.ts:880-889) */
+int32_t ah_causal_mask(ah_ptr out, int64_t size);
+/* Backend.castDtype f32<->f16 storage cast (interfaces.ts:139) and the internal f32<->bf16 cast */
+int32_t ah_cast(ah_ptr src, int32_t src_dtype, ah_ptr dst, int32_t dst_dtype, uint64_t n);
+/* Backend.checkFinite -> one f32: 0.0 all finite, 1.0 otherwise (interfaces.ts:146) */
+int32_t ah_check_finite(ah_ptr x, uint64_t n, ah_ptr out_flag);
+
+/* ---- data movement, 4-byte elements.  Backend.transpose/slice/scatterSlice/cat/sliceQkv/broadcast
+ *      (cpu_ref.ts:578-694; interfaces.ts:117-136). nd <= 6. ---- */
+int32_t ah_transpose(ah_ptr a, ah_ptr out, int32_t nd, const int64_t *shape, int32_t dim0, int32_t dim1);
+int32_t ah_slice(ah_ptr a, ah_ptr out, int32_t nd, const int64_t *shape, const int64_t *starts, const int64_t *ends);
+/* zero-fills `out` (orig_shape) and places grad at [starts, starts+gshape) */
+int32_t ah_scatter_slice(ah_ptr grad, ah_ptr out, int32_t nd, const int64_t *gshape, const int64_t *orig_shape,
+                         const int64_t *starts);
+/* copies `src` (src_shape) into `dst` (dst_shape) at offset `axis_offset` along `axis` -- one call per cat() operand */
+int32_t ah_cat_part(ah_ptr src, ah_ptr dst, int32_t nd, const int64_t *src_shape, const int64_t *dst_shape,
+                    int32_t axis, int64_t axis_offset);
+int32_t ah_slice_qkv(ah_ptr qkv, ah_ptr q, ah_ptr k, ah_ptr v, int64_t rows, int64_t d);
+int32_t ah_broadcast(ah_ptr a, ah_ptr out, int32_t nd, const int64_t *out_shape, const int64_t *stride_a);
+
+/* ---- reductions, f32.  Backend.sum/mean/softmax/logSoftmax/argmax (cpu_ref.ts:260-330,437-541,
+ *      698-756), sumOfSquares/totalSumOfSquares (interfaces.ts:144-145). The tensor is viewed as
+ *      [outer, dim, inner] with the reduced axis in the middle. ---- */
+int32_t ah_sum_axis(ah_ptr a, ah_ptr out, int64_t outer, int64_t dim, int64_t inner, int32_t mean);
+int32_t ah_sum_all(ah_ptr a, ah_ptr out, uint64_t n, int32_t mean);
+int32_t ah_softmax(ah_ptr a, ah_ptr out, int64_t outer, int64_t dim, int64_t inner, int32_t log_softmax);
+/* first maximum wins, NaN never selected, i32 result: bit-exact with cpu_ref.ts:698-756 */
+int32_t ah_argmax(ah_ptr a, ah_ptr out_i32, int64_t outer, int64_t dim, int64_t inner);
+/* out[0] (f32) = sum of x^2 over n elements; deterministic two-stage f64 reduction */
+int32_t ah_sum_sq(ah_ptr x, uint64_t n, ah_ptr out);
+/* softmax backward: s*(g - sum(g*s)) over the last dim (ops.ts:688-700), rows x dim */
+int32_t ah_softmax_bwd(ah_ptr s, ah_ptr g, ah_ptr out, int64_t rows, int64_t dim);
+
+/* ---- nn.  Backend.embedding / embeddingBackward (cpu_ref.ts:364-385; ops.ts:491-507),
+ *      layerNorm / layerNormBackward (cpu_ref.ts:387-420; ops.ts:509-571),
+ *      crossEntropy / crossEntropyBackward (cpu_ref.ts:543-563; ops.ts:702-729). ---- */
+int32_t ah_embedding(ah_ptr weight, ah_ptr idx_i32, ah_ptr out, int64_t n_idx, int64_t dim, int64_t vocab,
+                     int32_t out_dtype);
+/* out[i] = wte[tok[i]] + wpe[i % T]  -- tok+pos embedding and the add of gpt.ts:362-379 in one pass */
+int32_t ah_embedding_tok_pos(ah_ptr wte, ah_ptr wpe, ah_ptr tok_i32, ah_ptr out, int64_t n_idx, int64_t T,
+                             int64_t dim, int64_t vocab);
+/* grad_w[vocab,dim] = scatter-add of grad_out rows (zero-filled first unless accumulate != 0) */
+int32_t ah_embedding_bwd(ah_ptr idx_i32, ah_ptr grad_out, ah_ptr grad_w, int64_t n_idx, int64_t dim,
+                         int64_t vocab, int32_t accumulate);
+/* grad_wpe[T,dim] (+)= sum over the batch of grad_out[b,t,:]  (positions are 0..T-1 per row) */
+int32_t ah_pos_embedding_bwd(ah_ptr grad_out, ah_ptr grad_wpe, int64_t batch, int64_t T, int64_t dim,
+                             int32_t accumulate);
+int32_t ah_layernorm(ah_ptr x, ah_ptr w, ah_ptr b, ah_ptr out, int64_t rows, int64_t dim, float eps,
+                     int32_t out_dtype);
+/* dx (+= residual_grad when that handle is non-zero), dw, db.  dw/db are deterministic column sums;
+ * accumulate != 0 adds them into existing dw/db (gradient accumulation). grad_out dtype f32 or bf16. */
+int32_t ah_layernorm_bwd(ah_ptr x, ah_ptr w, ah_ptr grad_out, int32_t grad_dtype, ah_ptr residual_grad,
+                         ah_ptr dx, ah_ptr dw, ah_ptr db, int64_t rows, int64_t dim, float eps,
+                         int32_t accumulate);
+/* loss[0] = mean_i (logsumexp(logits[i,:]) - logits[i,target[i]]); lse[N] kept for backward (0 = skip) */
+int32_t ah_cross_entropy(ah_ptr logits, int32_t logits_dtype, ah_ptr targets_i32, ah_ptr loss_out, ah_ptr lse_out,
+                         int64_t n, int64_t c);
+/* dlogits = (softmax - onehot) * g[0] * g_mul / N; g_scalar = device f32 (0 = use 1.0); may run in place */
+int32_t ah_cross_entropy_bwd(ah_ptr logits, int32_t dtype, ah_ptr targets_i32, ah_ptr lse, ah_ptr g_scalar,
+                             float g_mul, ah_ptr dlogits, int64_t n, int64_t c);
+
+/* ---- GEMM on MFMA.  Backend.matmul / matmulTransposed / matmulTransposedA (cpu_ref.ts:166-258;
+ *      interfaces.ts:111-112; autograd use ops.ts:197-234).  C[M,N] = op(A) * op(B):
+ *        AH_GEMM_NN: A[M,K] * B[K,N]      (matmul;            dX = G * W)
+ *        AH_GEMM_NT: A[M,K] * B[N,K]^T    (matmulTransposed;  Y = X * W^T)
+ *        AH_GEMM_TN: A[K,M]^T * B[K,N]    (matmulTransposedA; dW = G^T * X)
+ *      f32 operands -> fp32 MFMA (parity mode); bf16 operands -> bf16 MFMA with fp32 accumulation.
+ *      lda/ldb/ldc are row strides in elements.  batch > 1 repeats with the given element strides
+ *      (0 = operand shared across the batch).
+ *      Epilogues: AH_EPI_NONE; AH_EPI_ACCUM  C += acc (gradient accumulation);
+ *      AH_EPI_GELU  C = gelu(acc), aux (same dtype/ld as C) = acc  (matmulTransposedGelu, ops.ts:426-487);
+ *      AH_EPI_RESIDUAL  C = acc + aux (aux f32 [M,N], ld = ldc) (residual add of gpt.ts:280-281);
+ *      AH_EPI_GELU_BWD  C = acc * gelu'(aux) (aux = saved pre-activation, dtype of C). ---- */
+enum { AH_GEMM_NN = 0, AH_GEMM_NT = 1, AH_GEMM_TN = 2 };
+enum { AH_EPI_NONE = 0, AH_EPI_ACCUM = 1, AH_EPI_GELU = 2, AH_EPI_RESIDUAL = 3, AH_EPI_GELU_BWD = 4 };
+typedef struct {
+  int32_t layout;            /* AH_GEMM_* */
+  int32_t in_dtype;          /* AH_F32 or AH_BF16 (both operands) */
+  int32_t out_dtype;         /* AH_F32 or AH_BF16 */
+  int32_t epilogue;          /* AH_EPI_* */
+  int64_t m, n, k;
+  int64_t lda, ldb, ldc;
+  int64_t batch;
+  int64_t stride_a, stride_b, stride_c;
+  ah_ptr  a, b, c, aux;
+} AhGemm;
+int32_t ah_gemm(const AhGemm *g);
+
+/* ---- fused causal flash attention.  Backend.flashAttention / flashAttentionBackward
+ *      (interfaces.ts:127-135; kernel semantics packages/helios/src/kernels/attention.ts:1-586):
+ *      s = (q.k)*scale; s = cap*tanh(s/cap) if cap > 0; keys after the query masked; online softmax;
+ *      O = P V; LSE = m + log(l).  Element (b, h, t, d) of Q lives at q + b*q_sb + h*q_sh + t*q_st + d
+ *      (same strides for K, V; o_* for O and dO; dq/dk/dv use the q strides), so both the reference's
+ *      [B*H, T, D] contract and a [B*T, 3C] QKV projection read in place are expressible.
+ *      LSE is [B, H, T] f32.  head_dim in {32, 64, 128}. ---- */
+typedef struct {
+  int32_t dtype;             /* AH_F32 (fp32 MFMA) or AH_BF16 */
+  int32_t batch, heads, seq, head_dim;
+  int64_t q_sb, q_sh, q_st;
+  int64_t k_sb, k_sh, k_st;
+  int64_t v_sb, v_sh, v_st;
+  int64_t o_sb, o_sh, o_st;
+  float   scale, soft_cap;
+  ah_ptr  q, k, v, o, lse;
+  ah_ptr  d_o, dq, dk, dv;   /* backward only; dq/dk/dv share the strides of q/k/v */
+} AhFlash;
+int32_t ah_flash_fwd(const AhFlash *f);
+int32_t ah_flash_bwd(const AhFlash *f);
+
+/* ---- optimizer.  Backend.adamwStep (interfaces.ts:149-150; CPU loop optimizers.ts:76-92). ---- */
+typedef struct {
+  float lr, beta1, beta2, eps, weight_decay, bc1, bc2, grad_scale;
+} AhAdamW;
+/* In place on p, m, v (f32).  `dev_scale` (0 or a device f32) multiplies grad_scale on the device, so a
+ * clip coefficient computed by ah_clip_coef never visits the host.  `dev_hyper` (0 or a device AhAdamW)
+ * overrides `h` with values read on the device: a captured graph then follows per-step lr / bias
+ * corrections written by ah_upload between launches.  `bf16_shadow` (0 or bf16[n]) receives the updated
+ * parameters rounded to bf16 for the next step's MFMA operands. */
+int32_t ah_adamw(ah_ptr p, ah_ptr g, ah_ptr m, ah_ptr v, uint64_t n, const AhAdamW *h, ah_ptr dev_hyper,
+                 ah_ptr dev_scale, ah_ptr bf16_shadow);
+/* out[0] = clip / (sqrt(sumsq[0]) * |grad_scale|) if that norm exceeds clip, else 1  (trainer.ts:1650-1656);
+ * out[1] = the norm itself. */
+int32_t ah_clip_coef(ah_ptr sumsq, float grad_scale, float clip, ah_ptr out2);
+
+/* ---- host-side SeededRng (packages/core/src/rng.ts:6-68): int32 xorshift pair, 20 warm-up draws,
+ *      next() = ((s0+s1)>>>0)/2^32, polar Box-Muller with a cached spare.  Pure host code (no device work);
+ *      here so that parameter initialisation (packages/model/src/gpt.ts:53-59,73-151) draws the reference's
+ *      stream at native speed. ---- */
+typedef struct { int32_t s0, s1; int32_t has_spare; int32_t _pad; double spare; } AhRng;
+int32_t ah_rng_seed(AhRng *r, int32_t seed);
+int32_t ah_rng_next(AhRng *r, double *out);
+int32_t ah_rng_next_gauss(AhRng *r, double *out);
+int32_t ah_rng_fill_gauss_f32(AhRng *r, float *out, uint64_t n, double std);   /* out[i] = (float)(nextGauss()*std) */
+int32_t ah_rng_fill_uniform_f64(AhRng *r, double *out, uint64_t n);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ALPHA_HIP_H */

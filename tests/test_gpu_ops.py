@@ -1,0 +1,380 @@
+"""Per-op parity of the HIP kernels (called through the C ABI via HipBackend) against the CPU oracle on the same
+seeded inputs.  Bar: bit-exact for integer / index / pure data-movement results; rel 1e-4 (tests/util.py) for fp32."""
+import math
+
+import numpy as np
+import pytest
+
+from oracle import ref
+from oracle import ref_model as rm
+from tests.util import assert_close
+
+pytestmark = pytest.mark.gpu
+
+O = ref.CpuRef()
+
+
+@pytest.fixture(scope="module")
+def B():
+    from alpha2_amd import HipBackend
+    return HipBackend(0)
+
+
+def dev(B, arr, dtype="f32"):
+    from alpha2_amd import TensorData
+    arr = np.asarray(arr)
+    return TensorData(arr.shape, dtype, arr)
+
+
+def orc(arr):
+    arr = np.asarray(arr)
+    return ref.f32(arr) if arr.dtype != np.int32 else ref.i32(arr)
+
+
+rs = np.random.RandomState(7)
+
+
+def test_reference_known_answers_on_device(B, golden):
+    g = golden["tensor.test.ts"]
+    c = g["matmul_2x2"]
+    assert [round(float(v)) for v in B.matmul(B.fromArray(c["a"], c["shape"]), B.fromArray(c["b"], c["shape"])).data] == c["expect"]
+    c = g["softmax_row"]
+    assert abs(float(B.softmax(B.fromArray(c["x"], c["shape"]), -1).data.sum()) - 1.0) < 1e-5
+    c = g["gelu"]
+    out = B.gelu(B.fromArray(c["x"], [3])).data
+    assert abs(out[0]) < 5e-4 and abs(out[1] - c["expect1"]) < 5e-3
+    c = g["embedding"]
+    out = B.embedding(B.fromArray(c["weight"], c["wshape"]), B.fromArray(c["indices"], [2], "i32"))
+    assert out.shape == (2, 2) and np.allclose(out.data, c["expect"], atol=5e-3)
+    c = g["layerNorm"]
+    out = B.layerNorm(B.fromArray(c["x"], c["shape"]), B.ones([2]), B.zeros([2]), c["eps"]).data
+    assert abs(out[0] + out[1]) < 5e-4 and abs(out[2] + out[3]) < 5e-4
+    c = g["crossEntropy"]
+    loss = B.crossEntropy(B.fromArray(c["logits"], c["shape"]), B.fromArray(c["targets"], [2], "i32"))
+    assert loss.data.size == 1 and loss.data[0] < c["less_than"]
+    c = g["causalMask"]
+    m = B.causalMask(c["size"]).data
+    assert all(m[i] == 0 for i in c["zero_at"]) and all(m[i] == -np.inf for i in c["neg_inf_at"])
+    c = g["transpose"]
+    t = B.transpose(B.fromArray(c["a"], c["shape"]), 0, 1)
+    assert list(t.shape) == c["expect_shape"] and [round(float(v)) for v in t.data] == c["expect"]
+    c = g["reshape"]
+    r = B.reshape(B.fromArray(c["a"], c["shape"]), c["to"])
+    assert list(r.shape) == c["to"] and list(r.data) == c["expect"]
+    assert B.sum(B.fromArray(g["sum_all"]["a"], [3])).data[0] == g["sum_all"]["expect"]
+    c = g["sum_axis0"]
+    s = B.sum(B.fromArray(c["a"], c["shape"]), 0)
+    assert s.shape == (2,) and [round(float(v)) for v in s.data] == c["expect"]
+    c = g["add"]
+    assert list(B.add(B.fromArray(c["a"], [3]), B.fromArray(c["b"], [3])).data) == c["expect"]
+    assert list(B.zeros([2, 3]).data) == [0] * 6 and list(B.ones([3]).data) == [1, 1, 1]
+    cf = golden["gpu-perf.test.ts"]["checkFinite"]
+    for case in cf["cases"]:
+        x = np.array([float(v) for v in case["x"]], dtype=np.float32)
+        assert B.checkFinite(dev(B, x)).data[0] == case["expect"]
+    big = (np.arange(cf["large"]["size"]) * cf["large"]["step"]).astype(np.float32)
+    assert B.checkFinite(dev(B, big)).data[0] == 0.0
+    big[-1] = np.nan
+    assert B.checkFinite(dev(B, big)).data[0] == 1.0
+    la = golden["gpu-perf.test.ts"]["loss_accum"]
+    acc = None
+    for v in la["losses"]:
+        s = B.scale(B.fromArray([v], [1]), 1 / la["accumSteps"])
+        acc = s if acc is None else B.add(acc, s)
+    assert abs(acc.data[0] - sum(la["losses"]) / la["accumSteps"]) < 5e-5
+    nan = B.add(B.scale(B.fromArray([float("nan")], [1]), 0.25), B.fromArray([0.5], [1]))
+    assert math.isnan(nan.data[0])
+
+
+@pytest.mark.parametrize("n", [1, 5, 1024, 100003])
+def test_elementwise_vs_oracle(B, n):
+    x = (rs.randn(n) * 2).astype(np.float32)
+    y = (rs.randn(n) + 3).astype(np.float32)
+    for name in ("add", "sub", "mul", "div"):
+        assert_close(getattr(B, name)(dev(B, x), dev(B, y)).data, getattr(O, name)(orc(x), orc(y)).data, what=name)
+    for name in ("neg", "exp", "gelu", "relu", "silu"):
+        assert_close(getattr(B, name)(dev(B, x)).data, getattr(O, name)(orc(x)).data, what=name)
+    xp = np.abs(x) + 0.1
+    for name in ("log", "sqrt"):
+        assert_close(getattr(B, name)(dev(B, xp)).data, getattr(O, name)(orc(xp)).data, what=name)
+    assert_close(B.pow(dev(B, xp), 2.5).data, O.pow(orc(xp), 2.5).data, what="pow")
+    assert_close(B.scale(dev(B, x), -0.37).data, O.scale(orc(x), -0.37).data, what="scale")
+    assert np.array_equal(B.clamp(dev(B, x), -0.5, 1.25).data, O.clamp(orc(x), -0.5, 1.25).data)
+    g = rs.randn(n).astype(np.float32)
+    assert_close(B.geluBackward(dev(B, x), dev(B, g)).data, ref.gelu_backward(orc(x), orc(g), fused=True).data, what="geluBackward")
+    assert_close(B.siluBackward(dev(B, x), dev(B, g)).data, ref.silu_backward(orc(x), orc(g)).data, what="siluBackward")
+    assert np.array_equal(B.reluBackward(dev(B, x), dev(B, g)).data, ref.relu_backward(orc(x), orc(g)).data)
+    assert np.array_equal(B.clampBackward(dev(B, x), dev(B, g), -0.7, 0.9).data, ref.clamp_backward(orc(x), orc(g), -0.7, 0.9).data)
+    # softCap: tanh(x/cap)*cap against the oracle's composed exp form (ops.ts:329-340)
+    tape = rm.Tape(); ctx = rm.Ctx(tape, O)
+    xv = rm.Variable(orc(x * 20), True)
+    sc = rm.softCap(ctx, xv, 30.0)
+    assert_close(B.softCap(dev(B, x * 20), 30.0).data, sc.data.data, what="softCap")
+    tape.backward(sc, O, orc(g))
+    assert_close(B.softCapBackward(dev(B, g), dev(B, x * 20), 30.0).data, xv.grad.data, what="softCapBackward")
+    a, b = dev(B, x), dev(B, y)
+    B.addInplace(a, b)
+    assert_close(a.data, O.add(orc(x), orc(y)).data, what="addInplace")
+    B.scaleInplace(a, 0.5)
+    assert_close(a.data, O.scale(O.add(orc(x), orc(y)), 0.5).data, what="scaleInplace")
+    sm = B.siluMul(dev(B, x), dev(B, y))
+    assert_close(sm.data, O.mul(O.silu(orc(x)), orc(y)).data, what="siluMul")
+    da, db = B.siluMulBackward(dev(B, x), dev(B, y), dev(B, g))
+    assert_close(da.data, ref.silu_backward(orc(x), O.mul(orc(g), orc(y))).data, what="siluMulBackward.da")
+    assert_close(db.data, O.mul(orc(g), O.silu(orc(x))).data, what="siluMulBackward.db")
+    assert_close(B.residualDropoutAdd(dev(B, x), dev(B, y), dev(B, g)).data, O.add(orc(x), O.mul(orc(y), orc(g))).data, what="rda")
+
+
+def test_empty_tensors(B):
+    e = dev(B, np.zeros((0, 4), np.float32))
+    assert B.add(e, e).data.size == 0 and B.gelu(e).data.size == 0
+    assert B.sum(dev(B, np.zeros((0,), np.float32))).data[0] == 0.0
+
+
+def test_broadcast_binary_and_errors(B):
+    a, b = rs.randn(2, 1, 4).astype(np.float32), (rs.randn(3, 1) + 3).astype(np.float32)
+    for name in ("add", "sub", "mul", "div"):
+        got, want = getattr(B, name)(dev(B, a), dev(B, b)), getattr(O, name)(orc(a), orc(b))
+        assert got.shape == want.shape
+        assert_close(got.data, want.data, what=name)
+    with pytest.raises(ValueError):
+        B.add(dev(B, rs.randn(2, 3).astype(np.float32)), dev(B, rs.randn(4).astype(np.float32)))
+    # [BT,F] * [1,F] -- the per-channel gate of the universal / kan_spline activations
+    h, gate = rs.randn(37, 24).astype(np.float32), rs.randn(1, 24).astype(np.float32)
+    assert_close(B.mul(dev(B, h), dev(B, gate)).data, O.mul(orc(h), orc(gate)).data)
+    t = B.broadcast(dev(B, gate), (5, 24))
+    assert np.array_equal(t.data.reshape(5, 24), np.broadcast_to(gate, (5, 24)))
+
+
+def test_reductions_vs_oracle(B):
+    a = rs.randn(3, 40, 5).astype(np.float32)
+    assert_close(B.sum(dev(B, a)).data, O.sum(orc(a)).data)
+    assert_close(B.mean(dev(B, a)).data, O.mean(orc(a)).data)
+    for ax in (0, 1, 2, -1):
+        for keep in (False, True):
+            got, want = B.sum(dev(B, a), ax, keep), O.sum(orc(a), ax, keep)
+            assert got.shape == want.shape
+            assert_close(got.data, want.data, what=f"sum{ax}")
+            assert_close(B.mean(dev(B, a), ax, keep).data, O.mean(orc(a), ax, keep).data, what=f"mean{ax}")
+    big = rs.randn(1_000_003).astype(np.float32)
+    assert_close(B.sum(dev(B, big)).data, O.sum(orc(big)).data, rel=1e-5)
+    wide = rs.randn(5000, 3).astype(np.float32)        # many short strided lines
+    assert_close(B.sum(dev(B, wide), 0).data, O.sum(orc(wide), 0).data)
+    assert_close(B.sumOfSquares(dev(B, big)).data, [ref.sum_sq(orc(big))], rel=1e-6)
+    parts = [rs.randn(n).astype(np.float32) for n in (1, 7, 4096, 33333)]
+    assert_close(B.totalSumOfSquares([dev(B, p) for p in parts]).data, [sum(ref.sum_sq(orc(p)) for p in parts)], rel=1e-6)
+
+
+def test_softmax_family_vs_oracle(B):
+    a = (rs.randn(3, 5, 300) * 4).astype(np.float32)
+    for ax in (0, 1, 2):
+        assert_close(B.softmax(dev(B, a), ax).data, O.softmax(orc(a), ax).data, what=f"softmax{ax}")
+        assert_close(B.logSoftmax(dev(B, a), ax).data, O.logSoftmax(orc(a), ax).data, what=f"logSoftmax{ax}")
+    s = O.softmax(orc(a), -1)
+    g = rs.randn(*a.shape).astype(np.float32)
+    tape = rm.Tape(); ctx = rm.Ctx(tape, O)
+    av = rm.Variable(orc(a), True)
+    tape.backward(rm.softmax(ctx, av, -1), O, orc(g))
+    assert_close(B.softmaxBackward(dev(B, s.data.reshape(a.shape)), dev(B, g)).data, av.grad.data, what="softmaxBackward")
+
+
+def test_argmax_bit_exact(B):
+    a = np.array([[1, 5, 5, 2], [np.nan, 3, 3, -1], [-np.inf, -np.inf, -np.inf, -np.inf]], dtype=np.float32)
+    assert list(B.argmax(dev(B, a), 1).data) == list(O.argmax(orc(a), 1).data) == [1, 1, 0]
+    assert int(B.argmax(dev(B, a)).data[0]) == int(O.argmax(orc(a)).data[0])
+    r = np.round(rs.randn(64, 50304) * 3, 1).astype(np.float32)       # rounded: many exact ties per row
+    assert np.array_equal(B.argmax(dev(B, r), -1).data, O.argmax(orc(r), -1).data)
+    r2 = np.round(rs.randn(70, 9, 33) * 2, 1).astype(np.float32)
+    for ax in (0, 1, 2):
+        got = B.argmax(dev(B, r2), ax)
+        assert got.dtype == "i32" and np.array_equal(got.data, O.argmax(orc(r2), ax).data)
+
+
+def test_data_movement_bit_exact(B):
+    a = rs.randn(2, 3, 4, 5).astype(np.float32)
+    for d0, d1 in ((1, 2), (0, 3), (2, 3), (-1, -2), (0, 1)):
+        got, want = B.transpose(dev(B, a), d0, d1), O.transpose(orc(a), d0, d1)
+        assert got.shape == want.shape and np.array_equal(got.data, want.data)
+    big = rs.randn(3, 70, 130).astype(np.float32)
+    assert np.array_equal(B.transpose(dev(B, big), 1, 2).data, O.transpose(orc(big), 1, 2).data)
+    s = B.slice(dev(B, a), [0, 1, 1, 2], [2, 3, 3, 5])
+    assert np.array_equal(s.data, O.slice(orc(a), [0, 1, 1, 2], [2, 3, 3, 5]).data)
+    sc = B.scatterSlice(s, a.shape, [0, 1, 1, 2], [2, 3, 3, 5])
+    assert np.array_equal(sc.data, O.scatterSlice(O.slice(orc(a), [0, 1, 1, 2], [2, 3, 3, 5]), a.shape, [0, 1, 1, 2], [2, 3, 3, 5]).data)
+    c = B.cat([dev(B, a), dev(B, a[:, :, :2])], 2)
+    assert np.array_equal(c.data, O.cat([orc(a), orc(a[:, :, :2])], 2).data)
+    with pytest.raises(ValueError):
+        B.cat([dev(B, a), dev(B, a[:, :2])], 2)
+    qkv = rs.randn(9, 24).astype(np.float32)
+    q, k, v = B.sliceQkv(dev(B, qkv))
+    assert np.array_equal(q.data.reshape(9, 8), qkv[:, :8]) and np.array_equal(v.data.reshape(9, 8), qkv[:, 16:])
+    r = B.reshape(dev(B, a), (6, 20))
+    assert r.shape == (6, 20) and np.array_equal(r.data, a.reshape(-1))
+    with pytest.raises(ValueError):
+        B.reshape(dev(B, a), (7, 20))
+    m = B.causalMask(5)
+    assert np.array_equal(m.data, O.causalMask(5).data)
+    x = rs.randn(2, 3, 5, 5).astype(np.float32)
+    assert np.array_equal(B.maskedFill(dev(B, x), m, -1e9).data, O.maskedFill(orc(x), O.causalMask(5), -1e9).data)
+    cl = B.clone(dev(B, a))
+    assert np.array_equal(cl.data, a.reshape(-1))
+    h = B.castDtype(dev(B, a), "f16")
+    assert h.dtype == "f16" and np.array_equal(h.data.view(np.float16), a.reshape(-1).astype(np.float16))
+    assert_close(B.castDtype(h, "f32").data, a.reshape(-1).astype(np.float16).astype(np.float32), rel=0)
+
+
+def test_embedding_fwd_bwd(B):
+    V, D = 257, 48
+    w = rs.randn(V, D).astype(np.float32)
+    idx = rs.randint(0, V, (4, 33)).astype(np.int32)
+    idx[0, :8] = 5                          # collisions
+    g = rs.randn(4, 33, D).astype(np.float32)
+    out = B.embedding(dev(B, w), dev(B, idx, "i32"))
+    assert out.shape == (4, 33, D) and np.array_equal(out.data, O.embedding(orc(w), orc(idx)).data)   # gather is bit exact
+    gw = B.embeddingBackward(dev(B, idx, "i32"), dev(B, g), V)
+    assert_close(gw.data, ref.embedding_backward(orc(idx), orc(g), V).data, what="embeddingBackward")
+
+
+@pytest.mark.parametrize("rows,dim", [(1, 2), (7, 48), (1024, 128), (333, 768), (5, 1000), (3, 4096)])
+def test_layernorm_fwd_bwd(B, rows, dim):
+    x = (rs.randn(rows, dim) * 2 + 0.5).astype(np.float32)
+    w, b_, g = rs.randn(dim).astype(np.float32), rs.randn(dim).astype(np.float32), rs.randn(rows, dim).astype(np.float32)
+    assert_close(B.layerNorm(dev(B, x), dev(B, w), dev(B, b_), 1e-5).data, O.layerNorm(orc(x), orc(w), orc(b_), 1e-5).data, what="ln")
+    r = B.layerNormBackward(dev(B, x), dev(B, w), dev(B, g), 1e-5)
+    dx, dw, db = ref.layernorm_backward(orc(x), orc(w), orc(g), 1e-5)
+    assert_close(r["dx"].data, dx.data, what="ln.dx")
+    assert_close(r["dw"].data, dw.data, what="ln.dw")
+    assert_close(r["db"].data, db.data, what="ln.db")
+
+
+@pytest.mark.parametrize("n,c", [(2, 3), (11, 37), (128, 256), (16, 50304)])
+def test_cross_entropy_fwd_bwd(B, n, c):
+    lg = (rs.randn(n, c) * 3).astype(np.float32)
+    tg = rs.randint(0, c, n).astype(np.int32)
+    lgd, tgd = dev(B, lg), dev(B, tg, "i32")
+    loss = B.crossEntropy(lgd, tgd)
+    assert loss.shape == ()
+    assert_close(loss.data, O.crossEntropy(orc(lg), orc(tg)).data, what="ce")
+    gs = dev(B, np.array([0.7], np.float32))
+    assert_close(B.crossEntropyBackward(lgd, tgd, gs).data, ref.cross_entropy_backward(orc(lg), orc(tg), 0.7).data, what="ce.bwd")
+    fresh = dev(B, lg)                      # backward without a preceding forward on the same object
+    assert_close(B.crossEntropyBackward(fresh, tgd, gs).data, ref.cross_entropy_backward(orc(lg), orc(tg), 0.7).data, what="ce.bwd2")
+
+
+@pytest.mark.parametrize("M,K,N", [(2, 2, 2), (33, 19, 47), (64, 64, 64), (128, 128, 128), (256, 256, 256), (1024, 128, 384), (130, 515, 257)])
+def test_gemm_f32_all_layouts(B, M, K, N):
+    a, b = rs.randn(M, K).astype(np.float32), rs.randn(K, N).astype(np.float32)
+    want = O.matmul(orc(a), orc(b)).data
+    assert_close(B.matmul(dev(B, a), dev(B, b)).data, want, what="matmul")
+    bt = np.ascontiguousarray(b.T)
+    assert_close(B.matmulTransposed(dev(B, a), dev(B, bt)).data, want, what="matmulTransposed")
+    at = np.ascontiguousarray(a.T)
+    assert_close(B.matmulTransposedA(dev(B, at), dev(B, b)).data, want, what="matmulTransposedA")
+    with pytest.raises(ValueError):
+        B.matmul(dev(B, a), dev(B, rs.randn(K + 1, N).astype(np.float32)))
+
+
+def test_gemm_f32_batched_and_broadcast(B):
+    a, b = rs.randn(2, 3, 40, 16).astype(np.float32), rs.randn(2, 3, 16, 24).astype(np.float32)
+    assert_close(B.matmul(dev(B, a), dev(B, b)).data, O.matmul(orc(a), orc(b)).data)
+    b1 = rs.randn(16, 24).astype(np.float32)
+    got = B.matmul(dev(B, a), dev(B, b1))
+    assert got.shape == (2, 3, 40, 24)
+    assert_close(got.data, O.matmul(orc(a), orc(b1)).data)
+    b2 = rs.randn(3, 16, 24).astype(np.float32)          # mixed broadcast [2,3] x [3]
+    assert_close(B.matmul(dev(B, a), dev(B, b2)).data, O.matmul(orc(a), orc(b2)).data)
+    bt = np.ascontiguousarray(np.swapaxes(b, 2, 3))
+    assert_close(B.matmulTransposed(dev(B, a), dev(B, bt)).data, O.matmul(orc(a), orc(b)).data)
+    g = rs.randn(2, 3, 40, 24).astype(np.float32)
+    want = O.matmul(O.transpose(orc(a), 2, 3), orc(g)).data
+    assert_close(B.matmulTransposedA(dev(B, a), dev(B, g)).data, want)
+
+
+def _oracle_attention(q, k, v, do, scale, cap):
+    """[BH,T,D] attention through the oracle's own op chain (gpt.ts:255-279) and tape."""
+    tape = rm.Tape(); ctx = rm.Ctx(tape, O)
+    T = q.shape[1]
+    qv, kv, vv = (rm.Variable(orc(x), True) for x in (q, k, v))
+    s = rm.scale(ctx, rm.matmul(ctx, qv, rm.transpose(ctx, kv, 1, 2)), scale)
+    if cap > 0:
+        s = rm.softCap(ctx, s, cap)
+    mask = O.causalMask(T)
+    masked = rm.Variable(O.maskedFill(s.data, mask, -1e9), True)
+    tape.record(masked, [s], lambda g, Bk, n: [Bk.maskedFill(g, mask, 0)])
+    att = rm.softmax(ctx, masked, -1)
+    out = rm.matmul(ctx, att, vv)
+    lse = np.log(np.sum(np.exp(masked.data.data.reshape(-1, T).astype(np.float64)), -1))
+    tape.backward(out, O, orc(do))
+    return out.data.data, lse, qv.grad.data, kv.grad.data, vv.grad.data
+
+
+@pytest.mark.parametrize("BH,T,D,cap", [(2, 64, 32, 30.0), (3, 100, 64, 0.0), (2, 129, 64, 30.0), (1, 256, 128, 30.0), (2, 1, 32, 0.0)])
+def test_flash_attention_f32_vs_materialised(B, BH, T, D, cap):
+    q, k, v, do = (rs.randn(BH, T, D).astype(np.float32) for _ in range(4))
+    scale = 1 / math.sqrt(D)
+    want_o, want_lse, dq, dk, dv = _oracle_attention(q, k, v, do, scale, cap)
+    Q, K, V = dev(B, q), dev(B, k), dev(B, v)
+    r = B.flashAttention(Q, K, V, T, scale, cap)
+    assert r["output"].shape == (BH, T, D) and r["lse"].shape == (BH, T)
+    assert_close(r["output"].data, want_o, what="flash.O")
+    assert_close(r["lse"].data, want_lse, what="flash.LSE")
+    g = B.flashAttentionBackward(Q, K, V, r["output"], dev(B, do), r["lse"], T, scale, cap)
+    assert_close(g["dQ"].data, dq, what="flash.dQ")
+    assert_close(g["dK"].data, dk, what="flash.dK")
+    assert_close(g["dV"].data, dv, what="flash.dV")
+
+
+def test_adamw_vs_oracle_and_reference_gradscale_identity(B, golden):
+    n = 100003
+    p0, g = rs.randn(n).astype(np.float32), rs.randn(n).astype(np.float32)
+    p, m, v = dev(B, p0), dev(B, np.zeros(n, np.float32)), dev(B, np.zeros(n, np.float32))
+    po, mo, vo = orc(p0), np.zeros(n, np.float32), np.zeros(n, np.float32)
+    b1p = b2p = 1.0
+    for _ in range(3):
+        b1p *= 0.9; b2p *= 0.95
+        B.adamwStep(p, dev(B, g), m, v, 3e-4, 0.9, 0.95, 1e-8, 0.1, 1 - b1p, 1 - b2p, 0.5)
+        ref.adamw_step(po, orc(g), mo, vo, 3e-4, 0.9, 0.95, 1e-8, 0.1, 1 - b1p, 1 - b2p, 0.5)
+    assert_close(p.data, po.data, rel=1e-6, what="adamw.p")
+    assert_close(m.data, mo, what="adamw.m")
+    assert_close(v.data, vo, what="adamw.v")
+    c = golden["optimizer.test.ts"]["adamw_gradscale"]      # optimizer.test.ts:23-45 on the device
+
+    def run(prescale):
+        pp, gg = dev(B, np.array(c["p"], np.float32)), np.array(c["g"], np.float32)
+        gs = c["gradScale"]
+        if prescale:
+            gg, gs = gg * np.float32(gs), 1.0
+        B.adamwStep(pp, dev(B, gg), dev(B, np.zeros(4, np.float32)), dev(B, np.zeros(4, np.float32)), c["lr"], c["beta1"], c["beta2"],
+                    c["eps"], c["weightDecay"], 1 - c["beta1"], 1 - c["beta2"], gs)
+        return pp.data
+    assert np.max(np.abs(run(False) - run(True))) < 1e-7
+
+
+def test_graph_capture_replays_match_eager(B):
+    import ctypes as C
+    from alpha2_amd import _ffi as ffi
+    lib = B.lib
+    x = dev(B, rs.randn(512, 256).astype(np.float32)); w = dev(B, rs.randn(128, 256).astype(np.float32))
+    acc = B.zeros((512, 128))
+    B._ptr(x), B._ptr(w)
+
+    def body():
+        y = B.matmulTransposed(x, w)
+        z = B.gelu(y)
+        B.addInplace(acc, z)
+        for t in (y, z):
+            B.releaseGpuTensor(t)
+    body()                                   # eager warm-up fills the pool
+    B.syncGpu()
+    ffi.check(lib.ah_graph_begin())
+    body()
+    gid = C.c_uint64()
+    ffi.check(lib.ah_graph_end(C.byref(gid)))
+    want = O.gelu(O.matmul(orc(x.data.reshape(512, 256)), O.transpose(orc(w.data.reshape(128, 256)), 0, 1))).data
+    for i in range(2, 6):                    # replays interleaved with eager work and syncs
+        ffi.check(lib.ah_graph_launch(gid.value))
+        tmp = B.scale(acc, 1.0 / i)          # eager op between replays
+        B.syncGpu()
+        assert_close(tmp.data, want, what=f"replay {i}")
+        B.releaseGpuTensor(tmp)
+    ffi.check(lib.ah_graph_destroy(gid.value))
