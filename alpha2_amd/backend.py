@@ -670,6 +670,44 @@ class HipBackend:
         check(self.lib.ah_flash_bwd(C.byref(f)))
         return {"dQ": dQ, "dK": dK, "dV": dV}
 
+    def _qkv_desc(self, qkv: TensorData, Bt, T, H, scale, softCap, store) -> ffi.AhFlash:
+        rows, c3 = qkv.shape
+        Cc = c3 // 3
+        D = Cc // H
+        if rows != Bt * T or Cc * 3 != c3 or D * H != Cc:
+            raise ValueError(f"attentionQkv: qkv {qkv.shape} does not match B={Bt}, T={T}, H={H}")
+        f = ffi.AhFlash()
+        f.dtype, f.batch, f.heads, f.seq, f.head_dim = ffi.DTYPE_CODE[store], Bt, H, T, D
+        for p in ("q", "k", "v"):
+            setattr(f, p + "_sb", T * c3), setattr(f, p + "_sh", D), setattr(f, p + "_st", c3)
+        f.o_sb, f.o_sh, f.o_st = T * Cc, D, Cc
+        f.scale, f.soft_cap = scale, softCap
+        return f
+
+    def attentionQkv(self, qkv: TensorData, Bt: int, T: int, nHead: int, scale: float, softCap: float) -> dict:
+        """Causal multi-head attention on a fused [B*T, 3C] projection, heads addressed through strides; the output is
+        [B*T, C] with heads merged.  Same function as the chain at packages/model/src/gpt.ts:255-279."""
+        Cc = qkv.shape[1] // 3
+        f = self._qkv_desc(qkv, Bt, T, nHead, scale, softCap, qkv.store)
+        esz = ffi.DTYPE_BYTES[qkv.store]
+        out = self._new((Bt * T, Cc), "f32", qkv.store)
+        lse = self._new((Bt * nHead, T))
+        base = self._ptr(qkv)
+        f.q, f.k, f.v, f.o, f.lse = base, base + Cc * esz, base + 2 * Cc * esz, out._buf.ptr, lse._buf.ptr
+        check(self.lib.ah_flash_fwd(C.byref(f)))
+        return {"output": out, "lse": lse}
+
+    def attentionQkvBackward(self, qkv, out, dOut, lse, Bt, T, nHead, scale, softCap) -> TensorData:
+        Cc = qkv.shape[1] // 3
+        f = self._qkv_desc(qkv, Bt, T, nHead, scale, softCap, qkv.store)
+        esz = ffi.DTYPE_BYTES[qkv.store]
+        dqkv = self._new(qkv.shape, "f32", qkv.store)
+        base, dbase = self._ptr(qkv), dqkv._buf.ptr
+        f.q, f.k, f.v, f.o, f.lse = base, base + Cc * esz, base + 2 * Cc * esz, self._ptr(out), self._ptr(lse)
+        f.d_o, f.dq, f.dk, f.dv = self._ptr(dOut), dbase, dbase + Cc * esz, dbase + 2 * Cc * esz
+        check(self.lib.ah_flash_bwd(C.byref(f)))
+        return dqkv
+
     # ------------------------------------------------------------------ reductions / optimizer
     def sumOfSquares(self, data: TensorData) -> TensorData:
         self._f32(data)

@@ -1,0 +1,159 @@
+"""Model-level parity on the GPU: the HipBackend-driven forward / backward / AdamW step against the CPU oracle's
+restatement of the reference trainer, on identical seeded parameters and token batches (fp32 parity mode)."""
+import gc
+import math
+
+import numpy as np
+import pytest
+
+from oracle import ref
+from oracle import ref_model as rm
+from tests.util import assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def B():
+    from alpha2_amd import HipBackend
+    return HipBackend(0)
+
+
+def _both(B, cfg_kw, tc_kw, seed=0):
+    from alpha2_amd.model import ModelConfig
+    from alpha2_amd.train import TrainConfig, Trainer
+    dev = Trainer(B, ModelConfig(**cfg_kw), TrainConfig(**tc_kw), seed=seed)
+    orc = rm.Trainer(rm.ModelConfig(**{k: v for k, v in cfg_kw.items() if k != "attention"}),
+                     rm.TrainConfig(**{k: v for k, v in tc_kw.items() if k in rm.TrainConfig.__dataclass_fields__}), seed=seed)
+    for (n1, v1), (n2, v2) in zip(dev.entries, orc.entries):        # same names, same order, same initial values
+        assert n1 == n2 and np.array_equal(v1.data.data, v2.data.data), n1
+    return dev, orc
+
+
+@pytest.mark.parametrize("attention", ["heads", "unfused"])
+def test_forward_backward_grads_match_oracle(B, attention):
+    from alpha2_amd.autograd import Tape
+    from alpha2_amd.model import gptForward
+    from alpha2_amd.train import syntheticBatch
+    cfg = dict(vocabSize=61, blockSize=24, nLayer=2, nEmbd=64, nHead=2 if attention == "heads" else 4, attention=attention)
+    dev, orc = _both(B, cfg, dict(iters=1))
+    inp, tgt = syntheticBatch(3, 3, 24, 61)
+    oi, ot = rm.synthetic_batch(3, 3, 24, 61)
+    assert np.array_equal(inp.data, oi.data) and np.array_equal(tgt.data, ot.data)       # token ids: bit exact
+    tape = Tape()
+    r = gptForward(dev.cfg, dev.params, B, tape, inp, tgt, True)
+    otape = rm.Tape()
+    ologits, oloss = rm.gptForward(orc.cfg, orc.params, orc.B, otape, oi, ot, True)
+    assert_close(r["logits"].data.data, ologits.data.data, what="logits")
+    assert_close(r["loss"].data.data, oloss.data.data, what="loss")
+    tape.backward(r["loss"], B)
+    otape.backward(oloss, orc.B)
+    for (n, v), (_, ov) in zip(dev.entries, orc.entries):
+        assert_close(v.grad.data, ov.grad.data, what=f"grad {n}")
+
+
+@pytest.mark.parametrize("act", ["swiglu", "universal", "kan_spline", "silu", "relu"])
+def test_custom_activation_models_match_oracle(B, act):
+    from alpha2_amd.autograd import Tape
+    from alpha2_amd.model import gptForward
+    from alpha2_amd.train import syntheticBatch
+    cfg = dict(vocabSize=40, blockSize=16, nLayer=1, nEmbd=64, nHead=2, ffnActivation=act)
+    dev, orc = _both(B, cfg, dict(iters=1), seed=5)
+    rs = np.random.RandomState(1)
+    for (n, v), (_, ov) in zip(dev.entries, orc.entries):           # generic gates / coefficients
+        d = (rs.randn(v.data.size) * 0.05).astype(np.float32)
+        v.data.data = v.data.data + d
+        ov.data.data += d
+    inp, tgt = syntheticBatch(9, 2, 16, 40)
+    oi, ot = rm.synthetic_batch(9, 2, 16, 40)
+    tape, otape = Tape(), rm.Tape()
+    r = gptForward(dev.cfg, dev.params, B, tape, inp, tgt, True)
+    _, oloss = rm.gptForward(orc.cfg, orc.params, orc.B, otape, oi, ot, True)
+    assert_close(r["loss"].data.data, oloss.data.data, what="loss")
+    tape.backward(r["loss"], B, B.releaseGpuTensor)
+    otape.backward(oloss, orc.B)
+    for (n, v), (_, ov) in zip(dev.entries, orc.entries):
+        assert_close(v.grad.data, ov.grad.data, what=f"grad {n}")
+
+
+def test_tiny_char_gpt_one_step_matches_oracle(B):
+    """The reference's CPU-runnable configuration: vocab 256, d 128, 4 layers, 4 heads, B=8 x T=128, AdamW 3e-4,
+    betas (0.9, 0.95), wd 0.1, clip 1.0, seed 0 parameters, seed 1 tokens."""
+    from alpha2_amd.train import syntheticBatch
+    cfg = dict(vocabSize=256, blockSize=128, nLayer=4, nEmbd=128, nHead=4)
+    dev, orc = _both(B, cfg, dict(iters=1))
+    r = dev.step([syntheticBatch(1, 8, 128, 256)])
+    o = orc.step([rm.synthetic_batch(1, 8, 128, 256)])
+    assert abs(r.loss - o.loss) <= 1e-4 * abs(o.loss)
+    assert abs(r.gradNorm - o.gradNorm) <= 1e-4 * o.gradNorm
+    assert abs(r.clipCoef - o.clipCoef) <= 1e-4 and r.lr == o.lr
+    assert abs(o.loss - math.log(256)) < 0.1
+    for (n, v), (_, ov) in zip(dev.entries, orc.entries):
+        # step 1 of Adam moves every entry by lr*g/(|g|+eps): entries whose gradient cancels to ~eps are ill-conditioned
+        assert_close(v.data.data, ov.data.data, rel=1e-5, what=f"param {n} after step", outlier_frac=max(1e-3, 2.5 / v.data.size),
+                     outlier_abs=0.1 * 3e-4)
+        m, mo = dev.optimizer._m[n].data, orc.opt.m[n]
+        assert_close(m, mo, what=f"adam m {n}")
+    del o
+    gc.collect()
+    st = B.gpuMemStats()
+    assert st["liveAllocs"] >= 3 * len(dev.entries)              # params + m + v are resident ...
+
+
+def test_loss_parity_over_steps_with_accumulation(B):
+    """Step loss within 1e-3 relative over a run (warm-up + cosine schedule, clip, 2 micro-batches)."""
+    from alpha2_amd.train import syntheticBatch
+    cfg = dict(vocabSize=96, blockSize=32, nLayer=2, nEmbd=64, nHead=2)
+    tc = dict(iters=12, gradAccumSteps=2)
+    dev, orc = _both(B, cfg, tc, seed=2)
+    live = None
+    for s in range(12):
+        db = [syntheticBatch(100 + 2 * s + i, 4, 32, 96) for i in range(2)]
+        ob = [rm.synthetic_batch(100 + 2 * s + i, 4, 32, 96) for i in range(2)]
+        r, o = dev.step(db), orc.step(ob)
+        assert abs(r.loss - o.loss) <= 1e-3 * abs(o.loss), (s, r.loss, o.loss)
+        assert abs(r.gradNorm - o.gradNorm) <= 1e-3 * o.gradNorm and abs(r.lr - o.lr) < 1e-15
+        gc.collect()                                       # tensors of earlier tests may still be awaiting collection
+        n = B.gpuMemStats()["liveAllocs"]
+        if s >= 1:
+            assert n <= live, "live allocations must not grow from step to step"
+        live = n
+    assert r.loss < math.log(96)
+
+
+def test_activation_checkpointing_matches_plain(B):
+    from alpha2_amd.autograd import Tape
+    from alpha2_amd.model import ModelConfig, collectParamEntries, gptForward, initGPT
+    from alpha2_amd.rng import SeededRng
+    from alpha2_amd.train import syntheticBatch
+    cfg = ModelConfig(vocabSize=50, blockSize=16, nLayer=2, nEmbd=64, nHead=2)
+    out = []
+    for ck in (False, True):
+        params = initGPT(cfg, B, SeededRng(4))
+        tape = Tape()
+        inp, tgt = syntheticBatch(8, 2, 16, 50)
+        r = gptForward(cfg, params, B, tape, inp, tgt, True, ck, False, None, B.releaseGpuTensor)
+        loss = float(r["loss"].data.data[0])
+        tape.backward(r["loss"], B, B.releaseGpuTensor)
+        out.append((loss, [v.grad.data.copy() for _, v in collectParamEntries(params)]))
+    assert abs(out[0][0] - out[1][0]) < 1e-6
+    for a, b in zip(out[0][1], out[1][1]):
+        assert_close(b, a, rel=1e-5)
+
+
+def test_reference_flash_layout_is_exposed_and_differs(B):
+    """The reference reshapes [B,T,C] -> [B*H,T,D] without a head transpose when a backend exposes flashAttention
+    (gpt.ts:248-254); that path is available as attention="reference-flash" and is NOT the cpu_ref function."""
+    from alpha2_amd.autograd import Tape
+    from alpha2_amd.model import ModelConfig, gptForward, initGPT
+    from alpha2_amd.rng import SeededRng
+    from alpha2_amd.train import syntheticBatch
+    losses = {}
+    for mode in ("heads", "reference-flash"):
+        cfg = ModelConfig(vocabSize=50, blockSize=16, nLayer=2, nEmbd=64, nHead=2, attention=mode)
+        params = initGPT(cfg, B, SeededRng(4))
+        for l in params["layers"]:
+            l["attn"]["wqkv"].data.data = l["attn"]["wqkv"].data.data * 20        # make attention matter
+        inp, tgt = syntheticBatch(8, 2, 16, 50)
+        losses[mode] = float(gptForward(cfg, params, B, Tape(), inp, tgt, True)["loss"].data.data[0])
+    assert math.isfinite(losses["reference-flash"]) and abs(losses["heads"] - losses["reference-flash"]) > 1e-6

@@ -242,7 +242,8 @@ def test_layernorm_fwd_bwd(B, rows, dim):
     assert_close(B.layerNorm(dev(B, x), dev(B, w), dev(B, b_), 1e-5).data, O.layerNorm(orc(x), orc(w), orc(b_), 1e-5).data, what="ln")
     r = B.layerNormBackward(dev(B, x), dev(B, w), dev(B, g), 1e-5)
     dx, dw, db = ref.layernorm_backward(orc(x), orc(w), orc(g), 1e-5)
-    assert_close(r["dx"].data, dx.data, what="ln.dx")
+    term = float(np.max(np.abs(g * w)) / np.sqrt(np.min(x.var(-1)) + 1e-5))      # size of the terms dx is a difference of
+    assert_close(r["dx"].data, dx.data, what="ln.dx", scale=term if dim < 8 else 0.0)
     assert_close(r["dw"].data, dw.data, what="ln.dw")
     assert_close(r["db"].data, db.data, what="ln.db")
 
@@ -319,8 +320,10 @@ def test_flash_attention_f32_vs_materialised(B, BH, T, D, cap):
     assert_close(r["output"].data, want_o, what="flash.O")
     assert_close(r["lse"].data, want_lse, what="flash.LSE")
     g = B.flashAttentionBackward(Q, K, V, r["output"], dev(B, do), r["lse"], T, scale, cap)
-    assert_close(g["dQ"].data, dq, what="flash.dQ")
-    assert_close(g["dK"].data, dk, what="flash.dK")
+    # dS = P*(dP - delta) cancels exactly when a row sees a single key: floor the bound at the size of its terms
+    term = float(np.abs(np.einsum("bqd,bkd->bqk", do, v)).max() * max(np.abs(k).max(), np.abs(q).max()) * scale)
+    assert_close(g["dQ"].data, dq, what="flash.dQ", scale=term if T < 4 else 0.0)
+    assert_close(g["dK"].data, dk, what="flash.dK", scale=term if T < 4 else 0.0)
     assert_close(g["dV"].data, dv, what="flash.dV")
 
 

@@ -2,9 +2,10 @@
 import numpy as np
 
 
-def assert_close(got, want, rel=1e-4, what=""):
+def assert_close(got, want, rel=1e-4, what="", scale=0.0, outlier_frac=0.0, outlier_abs=0.0):
     """The parity bar for fp32 ops: |got - want| <= rel * (|want| + rms(want)) element-wise, i.e. 1e-4 relative with
-    the tensor's own scale as the floor for entries near zero."""
+    the tensor's own scale as the floor for entries near zero.  `scale` raises that floor to the magnitude of the
+    terms that cancel when the result is a small difference of large numbers (e.g. LayerNorm dx on a 2-wide row)."""
     got = np.asarray(got, dtype=np.float64).reshape(-1)
     want = np.asarray(want, dtype=np.float64).reshape(-1)
     assert got.shape == want.shape, (what, got.shape, want.shape)
@@ -16,6 +17,12 @@ def assert_close(got, want, rel=1e-4, what=""):
         return
     rms = float(np.sqrt(np.mean(w * w)))
     err = np.abs(g - w)
-    bound = rel * (np.abs(w) + rms) + 1e-30
+    bound = rel * (np.abs(w) + max(rms, scale)) + 1e-30
     bad = err > bound
+    if outlier_frac > 0.0:
+        # ill-conditioned entries (e.g. Adam's g/(|g|+eps) where a gradient cancels to ~eps): a bounded fraction may
+        # miss the tight bound but must stay within `outlier_abs`
+        assert bad.mean() <= outlier_frac and (not bad.any() or err[bad].max() <= outlier_abs), \
+            f"{what}: {int(bad.sum())}/{g.size} outliers, worst {err.max():.3e} (allowed {outlier_frac:.1e} of entries within {outlier_abs:.1e})"
+        return
     assert not bad.any(), f"{what}: {int(bad.sum())}/{g.size} outside rel {rel}; worst err {err.max():.3e} (rms {rms:.3e})"
