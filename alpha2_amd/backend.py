@@ -272,7 +272,36 @@ class HipBackend:
     def _gemm(self, layout, a_ptr, b_ptr, c_ptr, m, n, k, lda, ldb, ldc, batch=1, sa=0, sb=0, sc=0, in_dtype=ffi.F32,
               out_dtype=ffi.F32, epilogue=ffi.EPI_NONE, aux=0):
         g = ffi.AhGemm(layout, in_dtype, out_dtype, epilogue, m, n, k, lda, ldb, ldc, batch, sa, sb, sc, a_ptr, b_ptr, c_ptr, aux)
+        timed = getattr(self, "_timed", None)
+        if timed is None:
+            check(self.lib.ah_gemm(C.byref(g)))
+            return
+        e0, e1 = self._event(), self._event()
+        check(self.lib.ah_event_record(e0))
         check(self.lib.ah_gemm(C.byref(g)))
+        check(self.lib.ah_event_record(e1))
+        timed.append({"kind": "gemm", "layout": layout, "dtype": in_dtype, "m": m, "n": n, "k": k, "batch": batch,
+                      "flops": 2.0 * m * n * k * batch, "e0": e0, "e1": e1})
+
+    def _event(self) -> int:
+        ev = C.c_uint64()
+        check(self.lib.ah_event_create(C.byref(ev)))
+        return ev.value
+
+    def startTiming(self):
+        """Bracket every GEMM launch with HIP events on the library stream until stopTiming()."""
+        self._timed = []
+
+    def stopTiming(self) -> list:
+        """Returns one record per launch with its duration in milliseconds (blocks until the work has finished)."""
+        recs, self._timed = self._timed or [], None
+        ms = C.c_float()
+        for r in recs:
+            check(self.lib.ah_event_elapsed_ms(r["e0"], r["e1"], C.byref(ms)))
+            r["ms"] = ms.value
+            for e in (r.pop("e0"), r.pop("e1")):
+                check(self.lib.ah_event_destroy(e))
+        return recs
 
     def _batched(self, a: TensorData, b: TensorData, a_mat, b_mat):
         """Resolve broadcast batch dims (cpu_ref.ts:184-243).  Returns (batch_shape, batch, stride_a, stride_b)

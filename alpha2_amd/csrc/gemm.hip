@@ -4,36 +4,12 @@
 // All three operand layouts the training step needs are handled (NN: dX = G W, NT: Y = X W^T,
 // TN: dW = G^T X).  Epilogues fuse GELU (+ saved pre-activation), the residual add, gradient
 // accumulation and the GELU derivative.
-#include "common.h"
+#include "gemm_common.h"
+#include <cstdlib>
 
 using namespace ah;
 
 namespace {
-
-struct GemmArgs {
-  const void *a, *b;
-  void *c;
-  const void *aux;     // EPI_RESIDUAL: f32 [M,N]; EPI_GELU_BWD: pre-activation (C dtype)
-  void *aux_out;       // EPI_GELU: pre-activation out (C dtype)
-  int M, N, K;
-  int64_t lda, ldb, ldc;
-  int64_t sa, sb, sc;  // batch strides (elements)
-  int epi;
-};
-
-template <class OUT>
-__device__ __forceinline__ void epilogue_store(const GemmArgs &g, int64_t cbase, int row, int col, float acc) {
-  if (row >= g.M || col >= g.N) return;
-  int64_t idx = cbase + (int64_t)row * g.ldc + col;
-  OUT *c = (OUT *)g.c;
-  switch (g.epi) {
-    case AH_EPI_NONE: Io<OUT>::st(c, idx, acc); break;
-    case AH_EPI_ACCUM: Io<OUT>::st(c, idx, Io<OUT>::ld(c, idx) + acc); break;
-    case AH_EPI_GELU: Io<OUT>::st((OUT *)g.aux_out, idx, acc); Io<OUT>::st(c, idx, gelu_f(acc)); break;
-    case AH_EPI_RESIDUAL: Io<OUT>::st(c, idx, acc + ((const float *)g.aux)[idx]); break;
-    default: Io<OUT>::st(c, idx, acc * gelu_grad_f(Io<OUT>::ld((const OUT *)g.aux, idx))); break;   // GELU_BWD
-  }
-}
 
 // ================================================================ fp32 MFMA kernel
 // LDS tiles are k-major: As[k][m], Bs[k][n]; a lane of the 32x32x2 MFMA reads As[2*kk + lane/32][m0 + lane%32].
@@ -83,8 +59,8 @@ __device__ __forceinline__ void f32_store_tile(float (*s)[F_BM + F_PAD], const f
   }
 }
 
-template <int LAYOUT, class OUT>
-__global__ __launch_bounds__(256) void k_gemm_f32(GemmArgs g, int vec_a, int vec_b) {
+template <int LAYOUT, int EPI, class OUT>
+__global__ __launch_bounds__(256) void k_gemm_f32(GemmArgs g, int vec_a, int vec_b, int vec_c) {
   __shared__ __attribute__((aligned(16))) float As[2][F_BK][F_BM + F_PAD];
   __shared__ __attribute__((aligned(16))) float Bs[2][F_BK][F_BN + F_PAD];
   constexpr bool A_KC = (LAYOUT != AH_GEMM_TN);     // A is [M][K] except for TN ([K][M])
@@ -123,10 +99,11 @@ __global__ __launch_bounds__(256) void k_gemm_f32(GemmArgs g, int vec_a, int vec
     for (int kk = 0; kk < F_BK / 2; kk++) {
       float a0 = As[cur][2 * kk + lk][wm + lr], a1 = As[cur][2 * kk + lk][wm + 32 + lr];
       float b0 = Bs[cur][2 * kk + lk][wn + lr], b1 = Bs[cur][2 * kk + lk][wn + 32 + lr];
-      acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
-      acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
-      acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
-      acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+      // operands swapped: the accumulator holds C^T tiles (rows = n, columns = m)
+      acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(b0, a0, acc[0][0], 0, 0, 0);
+      acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(b1, a0, acc[0][1], 0, 0, 0);
+      acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(b0, a1, acc[1][0], 0, 0, 0);
+      acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(b1, a1, acc[1][1], 0, 0, 0);
     }
     if (t + 1 < nt) {
       f32_store_tile<A_KC>(As[cur ^ 1], ra);
@@ -134,16 +111,16 @@ __global__ __launch_bounds__(256) void k_gemm_f32(GemmArgs g, int vec_a, int vec
     }
     __syncthreads();
   }
-  // accumulator element e of a 32x32 tile: row = 8*(e/4) + 4*(lane/32) + e%4, col = lane%32
+  // accumulator element e of a (transposed) 32x32 tile: n = 8*(e/4) + 4*(lane/32) + e%4, m = lane%32
 #pragma unroll
   for (int i = 0; i < 2; i++)
 #pragma unroll
     for (int j = 0; j < 2; j++)
 #pragma unroll
-      for (int e = 0; e < 16; e++) {
-        int row = m0 + wm + 32 * i + 8 * (e >> 2) + 4 * lk + (e & 3);
-        int col = n0 + wn + 32 * j + lr;
-        epilogue_store<OUT>(g, cbase, row, col, acc[i][j][e]);
+      for (int q = 0; q < 4; q++) {
+        int row = m0 + wm + 32 * i + lr;
+        int col = n0 + wn + 32 * j + 8 * q + 4 * lk;
+        epilogue4<EPI, OUT>(g, cbase, row, col, acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3], vec_c);
       }
 }
 
@@ -177,8 +154,8 @@ __device__ __forceinline__ void h_store_tile(uint16_t *s, const uint4 (&v)[ROWS 
 }
 
 // BM x BN block tile, 4 waves as WGM x WGN grid; each wave owns (BM/WGM) x (BN/WGN).
-template <int BM, int BN, int WGM, int WGN, class OUT>
-__global__ __launch_bounds__(256) void k_gemm_bf16_nt(GemmArgs g) {
+template <int BM, int BN, int WGM, int WGN, int EPI, class OUT>
+__global__ __launch_bounds__(256) void k_gemm_bf16_nt(GemmArgs g, int vec_c) {
   constexpr int WM = BM / WGM, WN = BN / WGN, TM = WM / 32, TN = WN / 32;
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
   uint16_t *As = smem;                                   // [2][BM][H_PITCH]
@@ -227,7 +204,7 @@ __global__ __launch_bounds__(256) void k_gemm_bf16_nt(GemmArgs g) {
 #pragma unroll
       for (int i = 0; i < TM; i++)
 #pragma unroll
-        for (int j = 0; j < TN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+        for (int j = 0; j < TN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[j], fa[i], acc[i][j], 0, 0, 0);   // C^T tile
     }
     if (t + 1 < nt) {
       h_store_tile<BM>(As + (cur ^ 1) * BM * H_PITCH, ra);
@@ -240,10 +217,10 @@ __global__ __launch_bounds__(256) void k_gemm_bf16_nt(GemmArgs g) {
 #pragma unroll
     for (int j = 0; j < TN; j++)
 #pragma unroll
-      for (int e = 0; e < 16; e++) {
-        int row = m0 + wm + 32 * i + 8 * (e >> 2) + 4 * lk + (e & 3);
-        int col = n0 + wn + 32 * j + lr;
-        epilogue_store<OUT>(g, cbase, row, col, acc[i][j][e]);
+      for (int q = 0; q < 4; q++) {
+        int row = m0 + wm + 32 * i + lr;
+        int col = n0 + wn + 32 * j + 8 * q + 4 * lk;
+        epilogue4<EPI, OUT>(g, cbase, row, col, acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3], vec_c);
       }
 }
 
@@ -262,40 +239,50 @@ __global__ void k_transpose_u16(const uint16_t *__restrict__ in, int64_t ld_in, 
   }
 }
 
-template <int BM, int BN, int WGM, int WGN>
-int32_t launch_bf16_nt(const GemmArgs &ga, int batch, int out_dtype) {
+template <int BM, int BN, int WGM, int WGN, int EPI, class OUT>
+int32_t launch_bf16_nt_t(const GemmArgs &ga, int batch, int vec_c) {
   size_t lds = sizeof(uint16_t) * 2 * (size_t)(BM + BN) * H_PITCH;
   int64_t tiles = cdiv(ga.M, BM) * cdiv(ga.N, BN);
   dim3 grid((unsigned)tiles, 1, (unsigned)batch);
-  if (out_dtype == AH_F32) {
-    auto kfn = k_gemm_bf16_nt<BM, BN, WGM, WGN, float>;
-    if (lds > 64 * 1024) AH_HIP(hipFuncSetAttribute((const void *)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    hipLaunchKernelGGL(kfn, grid, dim3(256), lds, stream(), ga);
-  } else {
-    auto kfn = k_gemm_bf16_nt<BM, BN, WGM, WGN, uint16_t>;
-    if (lds > 64 * 1024) AH_HIP(hipFuncSetAttribute((const void *)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    hipLaunchKernelGGL(kfn, grid, dim3(256), lds, stream(), ga);
+  auto kfn = k_gemm_bf16_nt<BM, BN, WGM, WGN, EPI, OUT>;
+  if (lds > 64 * 1024) {
+    static bool raised = false;      // per instantiation: the attribute only needs setting once
+    if (!raised) { AH_HIP(hipFuncSetAttribute((const void *)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); raised = true; }
   }
+  hipLaunchKernelGGL(kfn, grid, dim3(256), lds, stream(), ga, vec_c);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
-
-int32_t run_bf16_nt(const GemmArgs &ga, int batch, int out_dtype) {
-  // Tile choice: the largest tile that still yields at least ~2 waves of blocks over the CUs.
-  int64_t cus = num_cus();
-  auto blocks = [&](int bm, int bn) { return cdiv(ga.M, bm) * cdiv(ga.N, bn) * batch; };
-  if (ga.M >= 256 && ga.N >= 256 && blocks(256, 256) >= 2 * cus) return launch_bf16_nt<256, 256, 2, 2>(ga, batch, out_dtype);
-  if (ga.M >= 256 && ga.N >= 128 && blocks(256, 128) >= cus) return launch_bf16_nt<256, 128, 2, 2>(ga, batch, out_dtype);
-  return launch_bf16_nt<128, 128, 2, 2>(ga, batch, out_dtype);
+int32_t run_bf16_nt(const GemmArgs &ga, int batch, int out_dtype, int vec_c) {
+  // Fallback kernel for shapes the direct kernel does not take (K % 64 != 0, unaligned C): one tile size.
+  bool f32 = out_dtype == AH_F32;
+  switch (ga.epi) {
+    case AH_EPI_NONE: return f32 ? launch_bf16_nt_t<128, 128, 2, 2, AH_EPI_NONE, float>(ga, batch, vec_c)
+                                 : launch_bf16_nt_t<128, 128, 2, 2, AH_EPI_NONE, uint16_t>(ga, batch, vec_c);
+    case AH_EPI_ACCUM: return launch_bf16_nt_t<128, 128, 2, 2, AH_EPI_ACCUM, float>(ga, batch, vec_c);
+    case AH_EPI_RESIDUAL: return launch_bf16_nt_t<128, 128, 2, 2, AH_EPI_RESIDUAL, float>(ga, batch, vec_c);
+    case AH_EPI_GELU: return launch_bf16_nt_t<128, 128, 2, 2, AH_EPI_GELU, uint16_t>(ga, batch, vec_c);
+    default: return launch_bf16_nt_t<128, 128, 2, 2, AH_EPI_GELU_BWD, uint16_t>(ga, batch, vec_c);
+  }
 }
 
-template <int LAYOUT>
-int32_t launch_f32(const GemmArgs &ga, int batch, int out_dtype, int vec_a, int vec_b) {
+template <int LAYOUT, int EPI, class OUT>
+int32_t launch_f32_t(const GemmArgs &ga, int batch, int vec_a, int vec_b, int vec_c) {
   dim3 grid((unsigned)cdiv(ga.N, F_BN), (unsigned)cdiv(ga.M, F_BM), (unsigned)batch);
-  if (out_dtype == AH_F32) hipLaunchKernelGGL((k_gemm_f32<LAYOUT, float>), grid, dim3(256), 0, stream(), ga, vec_a, vec_b);
-  else hipLaunchKernelGGL((k_gemm_f32<LAYOUT, uint16_t>), grid, dim3(256), 0, stream(), ga, vec_a, vec_b);
+  hipLaunchKernelGGL((k_gemm_f32<LAYOUT, EPI, OUT>), grid, dim3(256), 0, stream(), ga, vec_a, vec_b, vec_c);
   AH_LAUNCH_CHECK();
   return AH_OK;
+}
+template <int LAYOUT>
+int32_t launch_f32(const GemmArgs &ga, int batch, int out_dtype, int vec_a, int vec_b, int vec_c) {
+  switch (ga.epi) {
+    case AH_EPI_NONE: return out_dtype == AH_F32 ? launch_f32_t<LAYOUT, AH_EPI_NONE, float>(ga, batch, vec_a, vec_b, vec_c)
+                                                 : launch_f32_t<LAYOUT, AH_EPI_NONE, uint16_t>(ga, batch, vec_a, vec_b, vec_c);
+    case AH_EPI_ACCUM: return launch_f32_t<LAYOUT, AH_EPI_ACCUM, float>(ga, batch, vec_a, vec_b, vec_c);
+    case AH_EPI_GELU: return launch_f32_t<LAYOUT, AH_EPI_GELU, float>(ga, batch, vec_a, vec_b, vec_c);
+    case AH_EPI_RESIDUAL: return launch_f32_t<LAYOUT, AH_EPI_RESIDUAL, float>(ga, batch, vec_a, vec_b, vec_c);
+    default: return launch_f32_t<LAYOUT, AH_EPI_GELU_BWD, float>(ga, batch, vec_a, vec_b, vec_c);
+  }
 }
 
 }  // namespace
@@ -321,6 +308,10 @@ int32_t ah_gemm(const AhGemm *p) {
          (long long)q.lda, (long long)q.ldb, (long long)q.ldc, (long long)q.m, (long long)q.n, (long long)q.k);
   if (q.epilogue == AH_EPI_GELU || q.epilogue == AH_EPI_RESIDUAL || q.epilogue == AH_EPI_GELU_BWD)
     AH_ARG(q.aux != 0, "ah_gemm: epilogue %d needs aux", q.epilogue);
+  // epilogue / output-type combinations: NONE -> f32 or bf16; ACCUM, RESIDUAL -> f32; GELU, GELU_BWD -> the operand type
+  bool combo = q.epilogue == AH_EPI_NONE || ((q.epilogue == AH_EPI_ACCUM || q.epilogue == AH_EPI_RESIDUAL) && q.out_dtype == AH_F32) ||
+               ((q.epilogue == AH_EPI_GELU || q.epilogue == AH_EPI_GELU_BWD) && q.out_dtype == q.in_dtype);
+  if (!combo) return fail(AH_ERR_UNSUPPORTED, "ah_gemm: epilogue %d with operands of dtype %d and output dtype %d is not provided", q.epilogue, q.in_dtype, q.out_dtype);
 
   GemmArgs ga;
   ga.a = dp<const void>(q.a); ga.b = dp<const void>(q.b); ga.c = dp<void>(q.c);
@@ -329,21 +320,35 @@ int32_t ah_gemm(const AhGemm *p) {
   ga.lda = q.lda; ga.ldb = q.ldb; ga.ldc = q.ldc;
   ga.sa = q.stride_a; ga.sb = q.stride_b; ga.sc = q.stride_c;
   ga.epi = q.epilogue;
+  ga.ksplit = (int)q.k; ga.nsplit = 1;
   int batch = (int)q.batch;
 
+  // 4-wide epilogue accesses need 16-byte (f32) / 8-byte (bf16) aligned rows of C and aux
+  int osz = q.out_dtype == AH_F32 ? 4 : 2;
+  int vec_c = ((q.c % (4 * osz)) == 0) && (q.ldc % 4 == 0) && (q.stride_c % 4 == 0);
+  if (q.epilogue == AH_EPI_RESIDUAL) vec_c = vec_c && (q.aux % 16 == 0);
+  if (q.epilogue == AH_EPI_GELU || q.epilogue == AH_EPI_GELU_BWD) vec_c = vec_c && (q.aux % (4 * osz) == 0);
   if (q.in_dtype == AH_F32) {
     int vec_a = aligned16(q.a) && (q.lda % 4 == 0) && (q.stride_a % 4 == 0);
     int vec_b = aligned16(q.b) && (q.ldb % 4 == 0) && (q.stride_b % 4 == 0);
     switch (q.layout) {
-      case AH_GEMM_NN: return launch_f32<AH_GEMM_NN>(ga, batch, q.out_dtype, vec_a, vec_b);
-      case AH_GEMM_NT: return launch_f32<AH_GEMM_NT>(ga, batch, q.out_dtype, vec_a, vec_b);
-      default: return launch_f32<AH_GEMM_TN>(ga, batch, q.out_dtype, vec_a, vec_b);
+      case AH_GEMM_NN: return launch_f32<AH_GEMM_NN>(ga, batch, q.out_dtype, vec_a, vec_b, vec_c);
+      case AH_GEMM_NT: return launch_f32<AH_GEMM_NT>(ga, batch, q.out_dtype, vec_a, vec_b, vec_c);
+      default: return launch_f32<AH_GEMM_TN>(ga, batch, q.out_dtype, vec_a, vec_b, vec_c);
     }
   }
 
-  // bf16: the MFMA kernel consumes K-contiguous operands; bring the others into that form.
-  AH_ARG(batch == 1 || q.layout == AH_GEMM_NT, "ah_gemm: batched bf16 is supported for the NT layout only");
   AH_ARG(q.k % 8 == 0, "ah_gemm: bf16 contraction length %lld must be a multiple of 8", (long long)q.k);
+  {
+    // direct kernel: every operand row (k-contiguous) or row group (k-major) must be 16-byte addressable
+    bool akm = q.layout == AH_GEMM_TN, bkm = q.layout != AH_GEMM_NT;
+    bool ok = aligned16(q.a) && aligned16(q.b) && q.lda % 8 == 0 && q.ldb % 8 == 0 && q.stride_a % 8 == 0 && q.stride_b % 8 == 0 &&
+              (!akm || q.m % 8 == 0) && (!bkm || q.n % 8 == 0);
+    ok = ok && vec_c && q.k % 64 == 0;
+    if (ok) return ah::gemm_bf16_direct(ga, q.layout, batch, q.out_dtype);
+  }
+  // fallback for unaligned shapes: bring the operands into K-contiguous form with explicit transposes
+  AH_ARG(batch == 1 || q.layout == AH_GEMM_NT, "ah_gemm: batched bf16 with unaligned operands is supported for the NT layout only");
   ah_ptr ta = 0, tb = 0;
   int32_t rc = AH_OK;
   if (q.layout == AH_GEMM_TN) {           // A is [K][M] -> [M][K]
@@ -369,7 +374,7 @@ int32_t ah_gemm(const AhGemm *p) {
     if (tb) ah_free(tb);
     return fail(AH_ERR_ARG, "ah_gemm: bf16 operands need 16-byte aligned rows (lda, ldb, batch strides multiples of 8)");
   }
-  rc = run_bf16_nt(ga, batch, q.out_dtype);
+  rc = run_bf16_nt(ga, batch, q.out_dtype, vec_c);
   if (ta) ah_free(ta);       // stream-ordered: reusable only by later work
   if (tb) ah_free(tb);
   return rc;

@@ -1,0 +1,70 @@
+// Shared between the GEMM translation units: argument block and the fused epilogues.
+#pragma once
+#include "common.h"
+
+namespace ah {
+
+struct GemmArgs {
+  const void *a, *b;
+  void *c;
+  const void *aux;     // EPI_RESIDUAL: f32 [M,N]; EPI_GELU_BWD: pre-activation (C dtype)
+  void *aux_out;       // EPI_GELU: pre-activation out (C dtype)
+  int M, N, K;
+  int64_t lda, ldb, ldc;
+  int64_t sa, sb, sc;  // batch strides (elements)
+  int epi;
+  int ksplit, nsplit;  // split-K (bf16 direct kernel only): K elements per split, number of splits (1 = off)
+};
+
+// Epilogue for 4 consecutive columns (col..col+3) of one row: the MFMA operands are swapped (acc = B-frag x A-frag)
+// so that an accumulator's 4 consecutive registers are 4 consecutive COLUMNS of C; a lane then moves 16 bytes (f32)
+// or 8 bytes (bf16) per access and the 2 half-waves of a row group fill 32 contiguous bytes.
+template <int EPI, class OUT>
+__device__ __forceinline__ void epilogue4(const GemmArgs &g, int64_t cbase, int row, int col, float v0, float v1, float v2, float v3, bool vec) {
+  if (row >= g.M || col >= g.N) return;
+  int64_t idx = cbase + (int64_t)row * g.ldc + col;
+  OUT *c = (OUT *)g.c;
+  float v[4] = {v0, v1, v2, v3};
+  if (vec && col + 3 < g.N) {
+    if (EPI == AH_EPI_ACCUM) {
+      if (sizeof(OUT) == 4) { float4 o = *reinterpret_cast<const float4 *>((const float *)g.c + idx); v[0] += o.x; v[1] += o.y; v[2] += o.z; v[3] += o.w; }
+      else { uint2 o = *reinterpret_cast<const uint2 *>((const uint16_t *)g.c + idx);
+             v[0] += bf16_bits_to_f32(o.x & 0xffff); v[1] += bf16_bits_to_f32(o.x >> 16); v[2] += bf16_bits_to_f32(o.y & 0xffff); v[3] += bf16_bits_to_f32(o.y >> 16); }
+    } else if (EPI == AH_EPI_RESIDUAL) {
+      float4 o = *reinterpret_cast<const float4 *>((const float *)g.aux + idx);
+      v[0] += o.x; v[1] += o.y; v[2] += o.z; v[3] += o.w;
+    } else if (EPI == AH_EPI_GELU_BWD) {
+      float x[4];
+      if (sizeof(OUT) == 4) { float4 o = *reinterpret_cast<const float4 *>((const float *)g.aux + idx); x[0] = o.x; x[1] = o.y; x[2] = o.z; x[3] = o.w; }
+      else { uint2 o = *reinterpret_cast<const uint2 *>((const uint16_t *)g.aux + idx);
+             x[0] = bf16_bits_to_f32(o.x & 0xffff); x[1] = bf16_bits_to_f32(o.x >> 16); x[2] = bf16_bits_to_f32(o.y & 0xffff); x[3] = bf16_bits_to_f32(o.y >> 16); }
+#pragma unroll
+      for (int i = 0; i < 4; i++) v[i] *= gelu_grad_f(x[i]);
+    } else if (EPI == AH_EPI_GELU) {
+      if (sizeof(OUT) == 4) *reinterpret_cast<float4 *>((float *)g.aux_out + idx) = make_float4(v[0], v[1], v[2], v[3]);
+      else *reinterpret_cast<uint2 *>((uint16_t *)g.aux_out + idx) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+#pragma unroll
+      for (int i = 0; i < 4; i++) v[i] = gelu_f(v[i]);
+    }
+    if (sizeof(OUT) == 4) *reinterpret_cast<float4 *>((float *)g.c + idx) = make_float4(v[0], v[1], v[2], v[3]);
+    else *reinterpret_cast<uint2 *>((uint16_t *)g.c + idx) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+    return;
+  }
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    if (col + i < g.N) {
+      float a = v[i];
+      if (EPI == AH_EPI_ACCUM) a += Io<OUT>::ld(c, idx + i);
+      else if (EPI == AH_EPI_RESIDUAL) a += ((const float *)g.aux)[idx + i];
+      else if (EPI == AH_EPI_GELU_BWD) a *= gelu_grad_f(Io<OUT>::ld((const OUT *)g.aux, idx + i));
+      else if (EPI == AH_EPI_GELU) { Io<OUT>::st((OUT *)g.aux_out, idx + i, a); a = gelu_f(a); }
+      Io<OUT>::st(c, idx + i, a);
+    }
+  }
+}
+
+
+// gemm_bf16.hip
+int32_t gemm_bf16_direct(const GemmArgs &ga, int layout, int batch, int out_dtype);
+
+}  // namespace ah

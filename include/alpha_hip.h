@@ -200,7 +200,9 @@ int32_t ah_cross_entropy_bwd(ah_ptr logits, int32_t dtype, ah_ptr targets_i32, a
  *      Epilogues: AH_EPI_NONE; AH_EPI_ACCUM  C += acc (gradient accumulation);
  *      AH_EPI_GELU  C = gelu(acc), aux (same dtype/ld as C) = acc  (matmulTransposedGelu, ops.ts:426-487);
  *      AH_EPI_RESIDUAL  C = acc + aux (aux f32 [M,N], ld = ldc) (residual add of gpt.ts:280-281);
- *      AH_EPI_GELU_BWD  C = acc * gelu'(aux) (aux = saved pre-activation, dtype of C). ---- */
+ *      AH_EPI_GELU_BWD  C = acc * gelu'(aux) (aux = saved pre-activation, dtype of C).
+ *      Provided combinations: NONE -> f32 or bf16 output; ACCUM and RESIDUAL -> f32 output; GELU and GELU_BWD ->
+ *      output of the operand type.  Anything else returns AH_ERR_UNSUPPORTED. ---- */
 enum { AH_GEMM_NN = 0, AH_GEMM_NT = 1, AH_GEMM_TN = 2 };
 enum { AH_EPI_NONE = 0, AH_EPI_ACCUM = 1, AH_EPI_GELU = 2, AH_EPI_RESIDUAL = 3, AH_EPI_GELU_BWD = 4 };
 typedef struct {

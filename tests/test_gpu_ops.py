@@ -381,3 +381,95 @@ def test_graph_capture_replays_match_eager(B):
         assert_close(tmp.data, want, what=f"replay {i}")
         B.releaseGpuTensor(tmp)
     ffi.check(lib.ah_graph_destroy(gid.value))
+
+
+def _bf16_round(x):
+    """round-to-nearest-even to bf16, returned as f32 values and as raw u16 bits"""
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    u = (u + 0x7FFF + ((u >> 16) & 1)) >> 16
+    bits = u.astype(np.uint16)
+    return (bits.astype(np.uint32) << 16).view(np.float32).reshape(np.shape(x)), bits.reshape(np.shape(x))
+
+
+def _raw_gemm(B, layout, a, b, m, n, k, in_dtype, out_dtype, epi=0, aux=None, c_init=None):
+    """ah_gemm through the C ABI on raw buffers; returns C (f32 values) and aux-out if the epilogue writes one."""
+    import ctypes as C
+    from alpha2_amd import TensorData, _ffi as ffi
+
+    def up(arr, store):
+        if store == ffi.BF16:
+            t = TensorData(arr.shape, "f16", _bf16_round(arr)[1])      # 2-byte container for the raw bits
+        else:
+            t = TensorData(arr.shape, "f32", arr)
+        return t, B._ptr(t)
+    ta, pa = up(a, in_dtype)
+    tb, pb = up(b, in_dtype)
+    cinit = np.zeros((m, n), np.float32) if c_init is None else c_init
+    tc, pc = up(cinit, out_dtype)
+    paux = 0
+    if aux is not None:
+        taux, paux = up(aux, ffi.F32 if epi == ffi.EPI_RESIDUAL else out_dtype)
+    elif epi == ffi.EPI_GELU:
+        taux, paux = up(np.zeros((m, n), np.float32), out_dtype)
+    lda = a.shape[1]
+    ldb = b.shape[1]
+    g = ffi.AhGemm(layout, in_dtype, out_dtype, epi, m, n, k, lda, ldb, n, 1, 0, 0, 0, pa, pb, pc, paux)
+    ffi.check(B.lib.ah_gemm(C.byref(g)))
+
+    def down(t, store):
+        B._dirty(t)
+        raw = t.data
+        return (raw.astype(np.uint32) << 16).view(np.float32) if store == ffi.BF16 else raw
+    out = down(tc, out_dtype).reshape(m, n)
+    aux_out = down(taux, out_dtype).reshape(m, n) if epi == ffi.EPI_GELU else None
+    return out, aux_out
+
+
+@pytest.mark.parametrize("in_bf16,out_bf16", [(False, False), (True, False), (True, True)])
+@pytest.mark.parametrize("M,N,K", [(128, 128, 64), (256, 384, 96), (300, 200, 72), (1024, 768, 256)])
+def test_gemm_layouts_epilogues_dtypes(B, in_bf16, out_bf16, M, N, K):
+    from alpha2_amd import _ffi as ffi
+    idt, odt = (ffi.BF16 if in_bf16 else ffi.F32), (ffi.BF16 if out_bf16 else ffi.F32)
+    a, b = rs.randn(M, K).astype(np.float32), rs.randn(N, K).astype(np.float32)
+    if in_bf16:
+        a, b = _bf16_round(a)[0], _bf16_round(b)[0]
+    want = O.matmul(orc(a), O.transpose(orc(b), 0, 1)).data.reshape(M, N)
+    rel = 1e-4 if not out_bf16 else 2.0 ** -7            # a bf16 result carries 8 significant bits
+
+    def cmp(got, ref_, what):
+        assert_close(got, ref_, rel=rel, what=what)
+    cmp(_raw_gemm(B, ffi.GEMM_NT, a, b, M, N, K, idt, odt)[0], want, "NT")
+    cmp(_raw_gemm(B, ffi.GEMM_NN, a, np.ascontiguousarray(b.T), M, N, K, idt, odt)[0], want, "NN")
+    cmp(_raw_gemm(B, ffi.GEMM_TN, np.ascontiguousarray(a.T), np.ascontiguousarray(b.T), M, N, K, idt, odt)[0], want, "TN")
+    # provided combinations: ACCUM / RESIDUAL write f32; GELU / GELU_BWD write the operand type
+    if not out_bf16:
+        c0 = rs.randn(M, N).astype(np.float32)
+        cmp(_raw_gemm(B, ffi.GEMM_NT, a, b, M, N, K, idt, odt, ffi.EPI_ACCUM, c_init=c0)[0], want + c0, "ACCUM")
+        cmp(_raw_gemm(B, ffi.GEMM_TN, np.ascontiguousarray(a.T), np.ascontiguousarray(b.T), M, N, K, idt, odt, ffi.EPI_ACCUM, c_init=c0)[0],
+            want + c0, "TN ACCUM")
+        res = rs.randn(M, N).astype(np.float32)
+        cmp(_raw_gemm(B, ffi.GEMM_NT, a, b, M, N, K, idt, odt, ffi.EPI_RESIDUAL, aux=res)[0], want + res, "RESIDUAL")
+    if in_bf16 == out_bf16:
+        got, pre = _raw_gemm(B, ffi.GEMM_NT, a, b, M, N, K, idt, odt, ffi.EPI_GELU)
+        cmp(pre, want, "GELU.pre")
+        cmp(got, O.gelu(orc(want)).data.reshape(M, N), "GELU")
+        pre_act = rs.randn(M, N).astype(np.float32)
+        if out_bf16:
+            pre_act = _bf16_round(pre_act)[0]
+        gb = ref.gelu_backward(orc(pre_act), orc(want), fused=True).data.reshape(M, N)
+        cmp(_raw_gemm(B, ffi.GEMM_NN, a, np.ascontiguousarray(b.T), M, N, K, idt, odt, ffi.EPI_GELU_BWD, aux=pre_act)[0], gb, "GELU_BWD")
+    else:
+        import ctypes as C
+        g = ffi.AhGemm(ffi.GEMM_NT, idt, odt, ffi.EPI_GELU, M, N, K, K, K, N, 1, 0, 0, 0, 1 << 20, 1 << 20, 1 << 20, 1 << 20)
+        assert B.lib.ah_gemm(C.byref(g)) == 5 and b"not provided" in B.lib.ah_last_error()
+
+
+def test_gemm_bf16_split_k_weight_gradient(B):
+    """dW = G^T X with a long token axis and few output tiles takes the split-K path (atomic f32 partial sums)."""
+    from alpha2_amd import _ffi as ffi
+    Kc, M, N = 4096, 256, 128
+    g_, x = _bf16_round(rs.randn(Kc, M).astype(np.float32) * 0.1)[0], _bf16_round(rs.randn(Kc, N).astype(np.float32))[0]
+    want = O.matmul(O.transpose(orc(g_), 0, 1), orc(x)).data.reshape(M, N)
+    assert_close(_raw_gemm(B, ffi.GEMM_TN, g_, x, M, N, Kc, ffi.BF16, ffi.F32)[0], want, what="split-K NONE")
+    c0 = rs.randn(M, N).astype(np.float32)
+    assert_close(_raw_gemm(B, ffi.GEMM_TN, g_, x, M, N, Kc, ffi.BF16, ffi.F32, ffi.EPI_ACCUM, c_init=c0)[0], want + c0, what="split-K ACCUM")
