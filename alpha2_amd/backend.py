@@ -610,6 +610,14 @@ class HipBackend:
         check(self.lib.ah_cast(self._ptr(a), ffi.DTYPE_CODE[a.store], out._buf.ptr, ffi.DTYPE_CODE[dtype], a.size))
         return out
 
+    def castStore(self, a: TensorData, store: str) -> TensorData:
+        """Internal storage cast f32 <-> bf16 (the tensor stays "f32" to callers: packages/core/src/types.ts:6 has no bf16)."""
+        if a.store == store:
+            return a
+        out = self._new(a.shape, a.dtype, store)
+        check(self.lib.ah_cast(self._ptr(a), ffi.DTYPE_CODE[a.store], out._buf.ptr, ffi.DTYPE_CODE[store], a.size))
+        return out
+
     # ------------------------------------------------------------------ utility
     def argmax(self, a: TensorData, axis=None) -> TensorData:
         self._f32(a)
@@ -683,17 +691,17 @@ class HipBackend:
         return f
 
     def flashAttention(self, Q, K, V, T, scale, softCap) -> dict:
-        self._f32(Q, K, V)
         f = self._flash_desc(Q, K, V, T, scale, softCap)
-        out, lse = self._new(Q.shape), self._new((Q.shape[0], T))
+        f.dtype = ffi.DTYPE_CODE[Q.store]
+        out, lse = self._new(Q.shape, "f32", Q.store), self._new((Q.shape[0], T))
         f.q, f.k, f.v, f.o, f.lse = self._ptr(Q), self._ptr(K), self._ptr(V), out._buf.ptr, lse._buf.ptr
         check(self.lib.ah_flash_fwd(C.byref(f)))
         return {"output": out, "lse": lse}
 
     def flashAttentionBackward(self, Q, K, V, O, dO, lse, T, scale, softCap) -> dict:
-        self._f32(Q, K, V, O, dO, lse)
         f = self._flash_desc(Q, K, V, T, scale, softCap)
-        dQ, dK, dV = self._new(Q.shape), self._new(Q.shape), self._new(Q.shape)
+        f.dtype = ffi.DTYPE_CODE[Q.store]
+        dQ, dK, dV = (self._new(Q.shape, "f32", Q.store) for _ in range(3))
         f.q, f.k, f.v, f.o, f.lse = self._ptr(Q), self._ptr(K), self._ptr(V), self._ptr(O), self._ptr(lse)
         f.d_o, f.dq, f.dk, f.dv = self._ptr(dO), dQ._buf.ptr, dK._buf.ptr, dV._buf.ptr
         check(self.lib.ah_flash_bwd(C.byref(f)))

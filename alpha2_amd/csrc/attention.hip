@@ -13,23 +13,11 @@
 // An accumulator element e of a 32x32 tile sits at row 8*(e/4) + 4*(lane/32) + e%4, column lane%32, and
 // MFMA number (j, r) of a 32-deep contraction contracts rows {8j + r, 8j + 4 + r}: half lane/32 = h owns
 // row 8j + 4h + r in the accumulator and must supply exactly that row as operand -> no data movement.
-#include "common.h"
+#include "attention_common.h"
 
 using namespace ah;
 
 namespace {
-
-struct FlashArgs {
-  const void *q, *k, *v;
-  void *o;
-  float *lse;
-  const void *d_o;
-  void *dq, *dk, *dv;
-  float *delta;            // [B, H, T] rowsum(dO * O)
-  int B, H, T;
-  int64_t q_sb, q_sh, q_st, k_sb, k_sh, k_st, v_sb, v_sh, v_st, o_sb, o_sh, o_st;
-  float scale, cap;
-};
 
 constexpr int BC = 32;     // rows of the streamed tile per iteration
 constexpr int WAVES = 4;   // 4 waves x 32 owned rows = 128 rows per block
@@ -298,13 +286,14 @@ __global__ __launch_bounds__(256) void k_flash_dkv_f32(FlashArgs a) {
 
 int32_t check(const AhFlash *f, bool bwd, FlashArgs &a) {
   AH_ARG(f != nullptr, "flash attention: null descriptor");
-  AH_ARG(f->dtype == AH_F32, "flash attention: dtype %d not supported by this build (f32 only)", f->dtype);
+  AH_ARG(f->dtype == AH_F32 || f->dtype == AH_BF16, "flash attention: dtype %d must be f32 or bf16", f->dtype);
   AH_ARG(f->head_dim == 32 || f->head_dim == 64 || f->head_dim == 128, "flash attention: head_dim %d not in {32, 64, 128}", f->head_dim);
   AH_ARG(f->batch >= 0 && f->heads >= 0 && f->seq >= 0, "flash attention: negative extent");
   AH_ARG((int64_t)f->batch * f->heads <= 65535, "flash attention: batch*heads %lld exceeds 65535", (long long)f->batch * f->heads);
   AH_ARG(f->q && f->k && f->v && f->o && f->lse, "flash attention: null operand");
   const int64_t st[] = {f->q_sb, f->q_sh, f->q_st, f->k_sb, f->k_sh, f->k_st, f->v_sb, f->v_sh, f->v_st, f->o_sb, f->o_sh, f->o_st};
-  for (int64_t s : st) AH_ARG(s % 4 == 0 && s >= 0, "flash attention: strides must be non-negative multiples of 4 elements");
+  const int64_t sm = f->dtype == AH_BF16 ? 8 : 4;        // rows are moved in 16-byte pieces
+  for (int64_t s : st) AH_ARG(s % sm == 0 && s >= 0, "flash attention: strides must be non-negative multiples of 16 bytes");
   AH_ARG(f->q_st >= f->head_dim && f->k_st >= f->head_dim && f->v_st >= f->head_dim && f->o_st >= f->head_dim,
          "flash attention: row stride smaller than head_dim");
   AH_ARG(aligned16(f->q) && aligned16(f->k) && aligned16(f->v) && aligned16(f->o), "flash attention: operands must be 16-byte aligned");
@@ -359,6 +348,7 @@ int32_t ah_flash_fwd(const AhFlash *f) {
   int32_t rc = check(f, false, a);
   if (rc) return rc;
   if (a.B * a.H == 0 || a.T == 0) return AH_OK;
+  if (f->dtype == AH_BF16) return flash_fwd_bf16(a, f->head_dim);
   switch (f->head_dim) {
     case 32: return run_fwd<32>(a);
     case 64: return run_fwd<64>(a);
@@ -372,6 +362,7 @@ int32_t ah_flash_bwd(const AhFlash *f) {
   int32_t rc = check(f, true, a);
   if (rc) return rc;
   if (a.B * a.H == 0 || a.T == 0) return AH_OK;
+  if (f->dtype == AH_BF16) return flash_bwd_bf16(a, f->head_dim);
   switch (f->head_dim) {
     case 32: return run_bwd<32>(a);
     case 64: return run_bwd<64>(a);

@@ -1,0 +1,420 @@
+// bf16 causal flash attention (fp32 accumulation) on v_mfma_f32_32x32x16_bf16, forward and backward.
+//
+// Same arrangement as the fp32 kernels: the index a wave owns (32 queries in forward / dQ, 32 keys in dK/dV) is
+// the accumulator COLUMN, so softmax statistics are per-lane scalars and the probabilities feed the second product
+// straight from registers.  A 32x32 accumulator holds rows 8j + 4h + r (j = 0..3, r = 0..3, h = lane/32); as the B
+// operand of a 16-deep MFMA, half h supplies 8 k-slots, and slot i of MFMA m is taken to mean streamed row
+// 16m + 8(i/4) + 4h + i%4 -- exactly the rows that half holds in accumulator registers 8m..8m+7.  The other operand
+// must use the same slot order; it is read from the [row][d] LDS tile with ds_read_b64_tr_b16, whose 16-lane groups
+// may address any four rows, so no transposed copy of V (or K, Q, dO in the backward kernels) is ever made.
+//
+// One block = 4 waves = 128 owned rows; the streamed operand moves in 64-row tiles, register-prefetched one tile
+// ahead and double-buffered in LDS (one barrier per 64 rows).
+#include "attention_common.h"
+
+using namespace ah;
+
+namespace {
+
+constexpr int ST = 64;       // streamed rows per LDS tile
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) bf16x4 lds_v4;
+
+template <int D> struct Geo {
+  static constexpr int PITCH = D + 16;                 // bf16 elements; (D+16)*2 bytes = 32 mod 128 for D in {32,64,128}... see tile_frag_t
+  static constexpr int ELEMS = ST * PITCH;
+  static constexpr int CHUNKS = ST * D / 8 / 256;      // 16-byte chunks per thread per tile (D=32: 1, 64: 2, 128: 4)
+};
+
+__device__ __forceinline__ float softcap_f(float s, float cap, float inv_cap) {
+  // cap * tanh(s / cap) with tanh(x) = 1 - 2 / (exp(2x) + 1): one exp and one reciprocal
+  if (cap <= 0.f) return s;
+  float e = __expf(2.0f * s * inv_cap);
+  return cap * (1.0f - 2.0f * __frcp_rn(e + 1.0f));
+}
+
+// global -> registers: rows [row0, row0+64) of a [T][D] operand with row stride st (elements); rows >= T read as zero
+template <int D>
+__device__ __forceinline__ void tile_load(const uint16_t *__restrict__ base, int64_t st, int row0, int T, u32x4 (&v)[Geo<D>::CHUNKS]) {
+#pragma unroll
+  for (int i = 0; i < Geo<D>::CHUNKS; i++) {
+    int c = threadIdx.x + 256 * i, r = c / (D / 8), c8 = c % (D / 8);
+    u32x4 x = {0u, 0u, 0u, 0u};
+    if (row0 + r < T) x = *reinterpret_cast<const u32x4 *>(base + (int64_t)(row0 + r) * st + c8 * 8);
+    v[i] = x;
+  }
+}
+template <int D>
+__device__ __forceinline__ void tile_store(uint16_t *s, const u32x4 (&v)[Geo<D>::CHUNKS]) {
+#pragma unroll
+  for (int i = 0; i < Geo<D>::CHUNKS; i++) {
+    int c = threadIdx.x + 256 * i, r = c / (D / 8), c8 = c % (D / 8);
+    *reinterpret_cast<u32x4 *>(s + r * Geo<D>::PITCH + c8 * 8) = v[i];
+  }
+}
+// A/B fragment with the tile ROW as the MFMA row/column (k = feature d): rows r0 + lane%32, d = 16*ks + 8*(lane/32)..
+template <int D>
+__device__ __forceinline__ bf16x8 tile_frag(const uint16_t *s, int r0, int ks, int lane) {
+  return *reinterpret_cast<const bf16x8 *>(s + (r0 + (lane & 31)) * Geo<D>::PITCH + ks * 16 + (lane >> 5) * 8);
+}
+// A fragment with the feature d as the MFMA row (k = tile row, in the accumulator's slot order): features
+// 32*db + lane%32, k-slot i of this half = tile row r0 + 16m + 8(i/4) + 4(lane/32) + i%4.
+template <int D>
+__device__ __forceinline__ bf16x8 tile_frag_t(const uint16_t *s, int r0, int m, int db, int lane) {
+  int j = lane & 15, g = lane >> 4, lk = g >> 1;
+  const uint16_t *p = s + (r0 + 16 * m + 4 * lk + (j >> 2)) * Geo<D>::PITCH + 32 * db + 16 * (g & 1) + 4 * (j & 3);
+  bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_v4 *)p);
+  bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_v4 *)(p + 8 * Geo<D>::PITCH));
+  return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+}
+// accumulator registers 8m..8m+7 -> bf16 B operand of MFMA m
+__device__ __forceinline__ bf16x8 acc_to_b(const f32x16 &s, int m) {
+  bf16x8 r;
+#pragma unroll
+  for (int i = 0; i < 8; i++) r[i] = (__bf16)s[8 * m + i];
+  return r;
+}
+// this lane's row of a [T][D] operand as B fragments (k = d): one 16-byte global load per 16 features
+template <int D>
+__device__ __forceinline__ void row_frags(const uint16_t *__restrict__ base, int64_t st, int row, bool live, int lane, bf16x8 (&f)[D / 16]) {
+#pragma unroll
+  for (int ks = 0; ks < D / 16; ks++) {
+    u32x4 x = {0u, 0u, 0u, 0u};
+    if (live) x = *reinterpret_cast<const u32x4 *>(base + (int64_t)row * st + ks * 16 + (lane >> 5) * 8);
+    f[ks] = __builtin_bit_cast(bf16x8, x);
+  }
+}
+// O^T-style accumulators (rows = features 32db + 8j + 4h + r, column = owned row) -> bf16 row-major store
+template <int D>
+__device__ __forceinline__ void store_rows(uint16_t *__restrict__ dst, const f32x16 (&acc)[D / 32], float mul, int lane) {
+  int lk = lane >> 5;
+#pragma unroll
+  for (int db = 0; db < D / 32; db++)
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      uint2 w = make_uint2(pack_bf16x2(acc[db][4 * j] * mul, acc[db][4 * j + 1] * mul), pack_bf16x2(acc[db][4 * j + 2] * mul, acc[db][4 * j + 3] * mul));
+      *reinterpret_cast<uint2 *>(dst + 32 * db + 8 * j + 4 * lk) = w;
+    }
+}
+
+// ------------------------------------------------------------------------------------------ forward
+template <int D>
+__global__ __launch_bounds__(256) void k_flash_fwd_bf16(FlashArgs a) {
+  constexpr int DB = D / 32, KS = D / 16;
+  __shared__ __attribute__((aligned(16))) uint16_t Ks[2][Geo<D>::ELEMS], Vs[2][Geo<D>::ELEMS];
+  int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
+  int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 31, lk = lane >> 5;
+  int q0 = blockIdx.x * 128 + wave * 32, qi = q0 + lr;
+  const uint16_t *Q = (const uint16_t *)a.q + b * a.q_sb + h * a.q_sh;
+  const uint16_t *K = (const uint16_t *)a.k + b * a.k_sb + h * a.k_sh;
+  const uint16_t *V = (const uint16_t *)a.v + b * a.v_sb + h * a.v_sh;
+  float inv_cap = a.cap > 0.f ? 1.0f / a.cap : 0.f;
+
+  bf16x8 qf[KS];
+  row_frags<D>(Q, a.q_st, qi, qi < a.T, lane, qf);
+  f32x16 o[DB];
+#pragma unroll
+  for (int d = 0; d < DB; d++)
+#pragma unroll
+    for (int e = 0; e < 16; e++) o[d][e] = 0.f;
+  float m = -INFINITY, l = 0.f;
+
+  int kv_end = min(a.T, (int)(blockIdx.x + 1) * 128);            // causal: keys < kv_end
+  int ntile = (kv_end + ST - 1) / ST;
+  u32x4 rk[Geo<D>::CHUNKS], rv[Geo<D>::CHUNKS];
+  tile_load<D>(K, a.k_st, 0, a.T, rk);
+  tile_load<D>(V, a.v_st, 0, a.T, rv);
+  tile_store<D>(Ks[0], rk);
+  tile_store<D>(Vs[0], rv);
+  __syncthreads();
+  for (int it = 0; it < ntile; it++) {
+    int cur = it & 1;
+    if (it + 1 < ntile) {
+      tile_load<D>(K, a.k_st, (it + 1) * ST, a.T, rk);
+      tile_load<D>(V, a.v_st, (it + 1) * ST, a.T, rv);
+    }
+#pragma unroll
+    for (int sub = 0; sub < ST / 32; sub++) {
+      int kv0 = it * ST + sub * 32;
+      if (kv0 <= q0 + 31) {                                        // otherwise the sub-tile is in this wave's future
+        f32x16 s;
+#pragma unroll
+        for (int e = 0; e < 16; e++) s[e] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++)
+          s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tile_frag<D>(Ks[cur], sub * 32, ks, lane), qf[ks], s, 0, 0, 0);   // S^T[kv, q]
+        float tmax = -INFINITY;
+#pragma unroll
+        for (int e = 0; e < 16; e++) {
+          int kv = kv0 + 8 * (e >> 2) + 4 * lk + (e & 3);
+          float x = softcap_f(s[e] * a.scale, a.cap, inv_cap);
+          x = (kv > qi || kv >= a.T) ? -INFINITY : x;
+          s[e] = x;
+          tmax = fmaxf(tmax, x);
+        }
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+        float m_new = fmaxf(m, tmax);
+        float m_use = m_new == -INFINITY ? 0.f : m_new;
+        float alpha = __expf(m - m_use);
+        float psum = 0.f;
+#pragma unroll
+        for (int e = 0; e < 16; e++) { float p = __expf(s[e] - m_use); s[e] = p; psum += p; }
+        psum += __shfl_xor(psum, 32, 64);
+        l = l * alpha + psum;
+        m = m_new;
+        bf16x8 pb0 = acc_to_b(s, 0), pb1 = acc_to_b(s, 1);
+#pragma unroll
+        for (int d = 0; d < DB; d++) {
+#pragma unroll
+          for (int e = 0; e < 16; e++) o[d][e] *= alpha;
+          o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tile_frag_t<D>(Vs[cur], sub * 32, 0, d, lane), pb0, o[d], 0, 0, 0);   // O^T[d, q]
+          o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tile_frag_t<D>(Vs[cur], sub * 32, 1, d, lane), pb1, o[d], 0, 0, 0);
+        }
+      }
+    }
+    if (it + 1 < ntile) {
+      tile_store<D>(Ks[cur ^ 1], rk);
+      tile_store<D>(Vs[cur ^ 1], rv);
+    }
+    __syncthreads();
+  }
+  if (qi < a.T) {
+    float inv_l = l > 0.f ? 1.0f / l : 0.f;
+    store_rows<D>((uint16_t *)a.o + b * a.o_sb + h * a.o_sh + (int64_t)qi * a.o_st, o, inv_l, lane);
+    if (lk == 0) a.lse[((int64_t)b * a.H + h) * a.T + qi] = m + __logf(l);
+  }
+}
+
+// delta[b,h,t] = sum_d dO[t,d] * O[t,d]   (one wave per row)
+template <int D>
+__global__ void k_flash_delta_bf16(FlashArgs a) {
+  int64_t row = blockIdx.x * (int64_t)(blockDim.x >> 6) + (threadIdx.x >> 6);
+  int64_t total = (int64_t)a.B * a.H * a.T;
+  if (row >= total) return;
+  int lane = threadIdx.x & 63;
+  int t = (int)(row % a.T), h = (int)((row / a.T) % a.H), b = (int)(row / ((int64_t)a.T * a.H));
+  const uint16_t *O = (const uint16_t *)a.o + b * a.o_sb + h * a.o_sh + (int64_t)t * a.o_st;
+  const uint16_t *dO = (const uint16_t *)a.d_o + b * a.o_sb + h * a.o_sh + (int64_t)t * a.o_st;
+  float s = 0.f;
+  for (int d = lane; d < D; d += 64) s += bf16_bits_to_f32(O[d]) * bf16_bits_to_f32(dO[d]);
+  s = wave_sum(s);
+  if (lane == 0) a.delta[row] = s;
+}
+
+// ------------------------------------------------------------------------------------------ dQ
+template <int D>
+__global__ __launch_bounds__(256) void k_flash_dq_bf16(FlashArgs a) {
+  constexpr int DB = D / 32, KS = D / 16;
+  __shared__ __attribute__((aligned(16))) uint16_t Ks[2][Geo<D>::ELEMS], Vs[2][Geo<D>::ELEMS];
+  int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
+  int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 31, lk = lane >> 5;
+  int q0 = blockIdx.x * 128 + wave * 32, qi = q0 + lr;
+  const uint16_t *Q = (const uint16_t *)a.q + b * a.q_sb + h * a.q_sh;
+  const uint16_t *K = (const uint16_t *)a.k + b * a.k_sb + h * a.k_sh;
+  const uint16_t *V = (const uint16_t *)a.v + b * a.v_sb + h * a.v_sh;
+  const uint16_t *dO = (const uint16_t *)a.d_o + b * a.o_sb + h * a.o_sh;
+  float inv_cap = a.cap > 0.f ? 1.0f / a.cap : 0.f;
+  bool live = qi < a.T;
+  bf16x8 qf[KS], dof[KS];
+  row_frags<D>(Q, a.q_st, qi, live, lane, qf);
+  row_frags<D>(dO, a.o_st, qi, live, lane, dof);
+  int64_t srow = ((int64_t)b * a.H + h) * a.T + qi;
+  float lse = live ? a.lse[srow] : 0.f, delta = live ? a.delta[srow] : 0.f;
+  f32x16 dq[DB];
+#pragma unroll
+  for (int d = 0; d < DB; d++)
+#pragma unroll
+    for (int e = 0; e < 16; e++) dq[d][e] = 0.f;
+
+  int kv_end = min(a.T, (int)(blockIdx.x + 1) * 128);
+  int ntile = (kv_end + ST - 1) / ST;
+  u32x4 rk[Geo<D>::CHUNKS], rv[Geo<D>::CHUNKS];
+  tile_load<D>(K, a.k_st, 0, a.T, rk);
+  tile_load<D>(V, a.v_st, 0, a.T, rv);
+  tile_store<D>(Ks[0], rk);
+  tile_store<D>(Vs[0], rv);
+  __syncthreads();
+  for (int it = 0; it < ntile; it++) {
+    int cur = it & 1;
+    if (it + 1 < ntile) {
+      tile_load<D>(K, a.k_st, (it + 1) * ST, a.T, rk);
+      tile_load<D>(V, a.v_st, (it + 1) * ST, a.T, rv);
+    }
+#pragma unroll
+    for (int sub = 0; sub < ST / 32; sub++) {
+      int kv0 = it * ST + sub * 32;
+      if (kv0 <= q0 + 31) {
+        f32x16 s, dp;
+#pragma unroll
+        for (int e = 0; e < 16; e++) { s[e] = 0.f; dp[e] = 0.f; }
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+          s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tile_frag<D>(Ks[cur], sub * 32, ks, lane), qf[ks], s, 0, 0, 0);     // S^T[kv, q]
+          dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tile_frag<D>(Vs[cur], sub * 32, ks, lane), dof[ks], dp, 0, 0, 0);  // dP^T[kv, q]
+        }
+#pragma unroll
+        for (int e = 0; e < 16; e++) {
+          int kv = kv0 + 8 * (e >> 2) + 4 * lk + (e & 3);
+          float sc = softcap_f(s[e] * a.scale, a.cap, inv_cap);
+          float p = (kv > qi || kv >= a.T || !live) ? 0.f : __expf(sc - lse);
+          float ds = p * (dp[e] - delta);
+          if (a.cap > 0.f) { float t = sc * inv_cap; ds *= (1.0f - t * t); }
+          s[e] = ds * a.scale;
+        }
+        bf16x8 b0 = acc_to_b(s, 0), b1 = acc_to_b(s, 1);
+#pragma unroll
+        for (int d = 0; d < DB; d++) {                             // dQ^T[d, q] += K^T[d, kv] dS^T[kv, q]
+          dq[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tile_frag_t<D>(Ks[cur], sub * 32, 0, d, lane), b0, dq[d], 0, 0, 0);
+          dq[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tile_frag_t<D>(Ks[cur], sub * 32, 1, d, lane), b1, dq[d], 0, 0, 0);
+        }
+      }
+    }
+    if (it + 1 < ntile) {
+      tile_store<D>(Ks[cur ^ 1], rk);
+      tile_store<D>(Vs[cur ^ 1], rv);
+    }
+    __syncthreads();
+  }
+  if (live) store_rows<D>((uint16_t *)a.dq + b * a.q_sb + h * a.q_sh + (int64_t)qi * a.q_st, dq, 1.0f, lane);
+}
+
+// ------------------------------------------------------------------------------------------ dK, dV
+template <int D>
+__global__ __launch_bounds__(256) void k_flash_dkv_bf16(FlashArgs a) {
+  constexpr int DB = D / 32, KS = D / 16;
+  __shared__ __attribute__((aligned(16))) uint16_t Qs[2][Geo<D>::ELEMS], dOs[2][Geo<D>::ELEMS];
+  __shared__ float Ls[2][ST], Ds[2][ST];
+  int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
+  int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 31, lk = lane >> 5;
+  int kv_blk0 = blockIdx.x * 128, kv0 = kv_blk0 + wave * 32, kvi = kv0 + lr;
+  const uint16_t *Q = (const uint16_t *)a.q + b * a.q_sb + h * a.q_sh;
+  const uint16_t *K = (const uint16_t *)a.k + b * a.k_sb + h * a.k_sh;
+  const uint16_t *V = (const uint16_t *)a.v + b * a.v_sb + h * a.v_sh;
+  const uint16_t *dO = (const uint16_t *)a.d_o + b * a.o_sb + h * a.o_sh;
+  float inv_cap = a.cap > 0.f ? 1.0f / a.cap : 0.f;
+  bool live = kvi < a.T;
+  bf16x8 kf[KS], vf[KS];
+  row_frags<D>(K, a.k_st, kvi, live, lane, kf);
+  row_frags<D>(V, a.v_st, kvi, live, lane, vf);
+  f32x16 dk[DB], dv[DB];
+#pragma unroll
+  for (int d = 0; d < DB; d++)
+#pragma unroll
+    for (int e = 0; e < 16; e++) { dk[d][e] = 0.f; dv[d][e] = 0.f; }
+
+  int64_t srow0 = ((int64_t)b * a.H + h) * a.T;
+  int q_first = (kv_blk0 / ST) * ST;                               // causal: queries at or after this block's first key
+  int ntile = (a.T - q_first + ST - 1) / ST;
+  u32x4 rq[Geo<D>::CHUNKS], rdo[Geo<D>::CHUNKS];
+  float rl = 0.f, rd = 0.f;
+  auto load_stats = [&](int q_base) {
+    if (threadIdx.x < ST) {
+      int qi = q_base + threadIdx.x;
+      rl = qi < a.T ? a.lse[srow0 + qi] : 0.f;
+      rd = qi < a.T ? a.delta[srow0 + qi] : 0.f;
+    }
+  };
+  tile_load<D>(Q, a.q_st, q_first, a.T, rq);
+  tile_load<D>(dO, a.o_st, q_first, a.T, rdo);
+  load_stats(q_first);
+  tile_store<D>(Qs[0], rq);
+  tile_store<D>(dOs[0], rdo);
+  if (threadIdx.x < ST) { Ls[0][threadIdx.x] = rl; Ds[0][threadIdx.x] = rd; }
+  __syncthreads();
+  for (int it = 0; it < ntile; it++) {
+    int cur = it & 1;
+    if (it + 1 < ntile) {
+      tile_load<D>(Q, a.q_st, q_first + (it + 1) * ST, a.T, rq);
+      tile_load<D>(dO, a.o_st, q_first + (it + 1) * ST, a.T, rdo);
+      load_stats(q_first + (it + 1) * ST);
+    }
+#pragma unroll
+    for (int sub = 0; sub < ST / 32; sub++) {
+      int qs = q_first + it * ST + sub * 32;
+      if (qs + 31 >= kv0 && qs < a.T) {                            // otherwise every query of the sub-tile precedes this wave's keys
+        f32x16 s, dp;
+#pragma unroll
+        for (int e = 0; e < 16; e++) { s[e] = 0.f; dp[e] = 0.f; }
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {                          // rows = queries, columns = this wave's keys
+          s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tile_frag<D>(Qs[cur], sub * 32, ks, lane), kf[ks], s, 0, 0, 0);
+          dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tile_frag<D>(dOs[cur], sub * 32, ks, lane), vf[ks], dp, 0, 0, 0);
+        }
+        f32x16 pm;
+#pragma unroll
+        for (int e = 0; e < 16; e++) {
+          int qr = sub * 32 + 8 * (e >> 2) + 4 * lk + (e & 3), qi = q_first + it * ST + qr;
+          float sc = softcap_f(s[e] * a.scale, a.cap, inv_cap);
+          float p = (kvi > qi || qi >= a.T || !live) ? 0.f : __expf(sc - Ls[cur][qr]);
+          float ds = p * (dp[e] - Ds[cur][qr]);
+          if (a.cap > 0.f) { float t = sc * inv_cap; ds *= (1.0f - t * t); }
+          pm[e] = p;
+          s[e] = ds * a.scale;
+        }
+        bf16x8 p0 = acc_to_b(pm, 0), p1 = acc_to_b(pm, 1), d0 = acc_to_b(s, 0), d1 = acc_to_b(s, 1);
+#pragma unroll
+        for (int d = 0; d < DB; d++) {
+          dv[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tile_frag_t<D>(dOs[cur], sub * 32, 0, d, lane), p0, dv[d], 0, 0, 0);   // dV^T[d, kv]
+          dv[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tile_frag_t<D>(dOs[cur], sub * 32, 1, d, lane), p1, dv[d], 0, 0, 0);
+          dk[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tile_frag_t<D>(Qs[cur], sub * 32, 0, d, lane), d0, dk[d], 0, 0, 0);    // dK^T[d, kv]
+          dk[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tile_frag_t<D>(Qs[cur], sub * 32, 1, d, lane), d1, dk[d], 0, 0, 0);
+        }
+      }
+    }
+    if (it + 1 < ntile) {
+      tile_store<D>(Qs[cur ^ 1], rq);
+      tile_store<D>(dOs[cur ^ 1], rdo);
+      if (threadIdx.x < ST) { Ls[cur ^ 1][threadIdx.x] = rl; Ds[cur ^ 1][threadIdx.x] = rd; }
+    }
+    __syncthreads();
+  }
+  if (live) {
+    store_rows<D>((uint16_t *)a.dk + b * a.k_sb + h * a.k_sh + (int64_t)kvi * a.k_st, dk, 1.0f, lane);
+    store_rows<D>((uint16_t *)a.dv + b * a.v_sb + h * a.v_sh + (int64_t)kvi * a.v_st, dv, 1.0f, lane);
+  }
+}
+
+template <int D>
+int32_t run_fwd(const FlashArgs &a) {
+  dim3 grid((unsigned)cdiv(a.T, 128), (unsigned)(a.B * a.H));
+  hipLaunchKernelGGL(k_flash_fwd_bf16<D>, grid, dim3(256), 0, stream(), a);
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+template <int D>
+int32_t run_bwd(FlashArgs &a) {
+  int64_t rows = (int64_t)a.B * a.H * a.T;
+  ah_ptr delta = 0;
+  int32_t rc = ah_alloc((uint64_t)rows * 4, &delta);
+  if (rc) return rc;
+  a.delta = dp<float>(delta);
+  hipLaunchKernelGGL(k_flash_delta_bf16<D>, dim3((unsigned)cdiv(rows, 4)), dim3(256), 0, stream(), a);
+  AH_LAUNCH_CHECK();
+  dim3 grid((unsigned)cdiv(a.T, 128), (unsigned)(a.B * a.H));
+  hipLaunchKernelGGL(k_flash_dq_bf16<D>, grid, dim3(256), 0, stream(), a);
+  AH_LAUNCH_CHECK();
+  hipLaunchKernelGGL(k_flash_dkv_bf16<D>, grid, dim3(256), 0, stream(), a);
+  AH_LAUNCH_CHECK();
+  return ah_free(delta);
+}
+
+}  // namespace
+
+namespace ah {
+
+int32_t flash_fwd_bf16(const FlashArgs &a, int head_dim) {
+  switch (head_dim) {
+    case 32: return run_fwd<32>(a);
+    case 64: return run_fwd<64>(a);
+    default: return run_fwd<128>(a);
+  }
+}
+int32_t flash_bwd_bf16(FlashArgs &a, int head_dim) {
+  switch (head_dim) {
+    case 32: return run_bwd<32>(a);
+    case 64: return run_bwd<64>(a);
+    default: return run_bwd<128>(a);
+  }
+}
+
+}  // namespace ah

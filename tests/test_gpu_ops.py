@@ -473,3 +473,30 @@ def test_gemm_bf16_split_k_weight_gradient(B):
     assert_close(_raw_gemm(B, ffi.GEMM_TN, g_, x, M, N, Kc, ffi.BF16, ffi.F32)[0], want, what="split-K NONE")
     c0 = rs.randn(M, N).astype(np.float32)
     assert_close(_raw_gemm(B, ffi.GEMM_TN, g_, x, M, N, Kc, ffi.BF16, ffi.F32, ffi.EPI_ACCUM, c_init=c0)[0], want + c0, what="split-K ACCUM")
+
+
+@pytest.mark.parametrize("BH,T,D,cap", [(2, 64, 32, 30.0), (3, 100, 64, 0.0), (2, 129, 64, 30.0), (2, 320, 64, 30.0), (1, 256, 128, 30.0), (2, 1, 64, 0.0)])
+def test_flash_attention_bf16_vs_materialised(B, BH, T, D, cap):
+    """bf16 operands, fp32 accumulation.  Inputs are bf16-exact so the oracle sees the same numbers; the kernel rounds P and
+    dS to bf16 before the second product and its outputs to bf16, so the bar is bf16 resolution (2^-7 of the tensor scale)."""
+    q, k, v, do = (_bf16_round(rs.randn(BH, T, D).astype(np.float32))[0] for _ in range(4))
+    scale = 1 / math.sqrt(D)
+    want_o, want_lse, dq, dk, dv = _oracle_attention(q, k, v, do, scale, cap)
+    Q, K, V, dO = (B.castStore(dev(B, x), "bf16") for x in (q, k, v, do))
+    r = B.flashAttention(Q, K, V, T, scale, cap)
+    assert r["output"].store == "bf16"
+    rel = 2.0 ** -6
+    assert_close(r["output"].data, want_o, rel=rel, what="flash16.O")
+    assert_close(r["lse"].data, want_lse, rel=1e-4, what="flash16.LSE")
+    g = B.flashAttentionBackward(Q, K, V, r["output"], dO, r["lse"], T, scale, cap)
+    term = float(np.abs(np.einsum("bqd,bkd->bqk", do, v)).max() * max(np.abs(k).max(), np.abs(q).max()) * scale)
+    # sums of bf16-rounded products: a few entries in a thousand may sit a little outside the element-wise bound
+    def loose(x):
+        return dict(outlier_frac=2e-3, outlier_abs=0.1 * float(np.sqrt(np.mean(np.square(x)))) + 1e-6)
+    if T < 4:
+        assert_close(g["dQ"].data, dq, rel=rel, what="flash16.dQ", scale=term)
+        assert_close(g["dK"].data, dk, rel=rel, what="flash16.dK", scale=term)
+    else:
+        assert_close(g["dQ"].data, dq, rel=rel, what="flash16.dQ", **loose(dq))
+        assert_close(g["dK"].data, dk, rel=rel, what="flash16.dK", **loose(dk))
+    assert_close(g["dV"].data, dv, rel=rel, what="flash16.dV", **loose(dv))
