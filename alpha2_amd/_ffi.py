@@ -90,7 +90,7 @@ SIGNATURES = {
     "ah_embedding_bwd": [u64, u64, u64, i64, i64, i64, i32],
     "ah_pos_embedding_bwd": [u64, u64, i64, i64, i64, i32],
     "ah_layernorm": [u64, u64, u64, u64, i64, i64, f32, i32],
-    "ah_layernorm_bwd": [u64, u64, u64, i32, u64, u64, u64, u64, i64, i64, f32, i32],
+    "ah_layernorm_bwd": [u64, u64, u64, i32, u64, u64, u64, u64, u64, i64, i64, f32, i32],
     "ah_cross_entropy": [u64, i32, u64, u64, u64, i64, i64],
     "ah_cross_entropy_bwd": [u64, i32, u64, u64, u64, f32, u64, i64, i64],
     "ah_gemm": [C.POINTER(AhGemm)],

@@ -491,7 +491,7 @@ class HipBackend:
         self._f32(x, weight, gradOutput)
         dim = x.shape[-1]
         dx, dw, db = self._new(x.shape), self._new(weight.shape), self._new(weight.shape)
-        check(self.lib.ah_layernorm_bwd(self._ptr(x), self._ptr(weight), self._ptr(gradOutput), ffi.F32, 0, dx._buf.ptr, dw._buf.ptr,
+        check(self.lib.ah_layernorm_bwd(self._ptr(x), self._ptr(weight), self._ptr(gradOutput), ffi.F32, 0, dx._buf.ptr, 0, dw._buf.ptr,
                                         db._buf.ptr, x.size // max(1, dim), dim, eps, 0))
         return {"dx": dx, "dw": dw, "db": db}
 

@@ -123,7 +123,7 @@ __global__ void k_layernorm(const float *__restrict__ x, const float *__restrict
 // sums the partials column-wise in fixed order (deterministic, no [rows, dim] temporaries).
 template <class G>
 __global__ void k_layernorm_bwd(const float *__restrict__ x, const float *__restrict__ w, const G *__restrict__ g,
-                                const float *__restrict__ res, float *__restrict__ dx, float *__restrict__ part_dw,
+                                const float *__restrict__ res, float *__restrict__ dx, uint16_t *__restrict__ dx16, float *__restrict__ part_dw,
                                 float *__restrict__ part_db, int64_t rows, int dim, float eps) {
   extern __shared__ float sh[];      // [2][WPB][dim]
   int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -152,6 +152,7 @@ __global__ void k_layernorm_bwd(const float *__restrict__ x, const float *__rest
       float d = rstd * (dy - (s1 + xh * s2) * inv_dim);
       if (res) d += res[row * (int64_t)dim + j];
       dx[row * (int64_t)dim + j] = d;
+      if (dx16) dx16[row * (int64_t)dim + j] = f32_to_bf16_bits(d);
     }
   }
   __syncthreads();
@@ -314,8 +315,8 @@ int32_t ah_layernorm(ah_ptr x, ah_ptr w, ah_ptr b, ah_ptr out, int64_t rows, int
   return out_dtype == AH_F32 ? launch_ln<float>(x, w, b, out, rows, dim, eps) : launch_ln<uint16_t>(x, w, b, out, rows, dim, eps);
 }
 
-int32_t ah_layernorm_bwd(ah_ptr x, ah_ptr w, ah_ptr grad_out, int32_t grad_dtype, ah_ptr residual_grad, ah_ptr dx, ah_ptr dw,
-                         ah_ptr db, int64_t rows, int64_t dim, float eps, int32_t accumulate) {
+int32_t ah_layernorm_bwd(ah_ptr x, ah_ptr w, ah_ptr grad_out, int32_t grad_dtype, ah_ptr residual_grad, ah_ptr dx, ah_ptr dx_bf16,
+                         ah_ptr dw, ah_ptr db, int64_t rows, int64_t dim, float eps, int32_t accumulate) {
   AH_REQUIRE_READY();
   AH_ARG(grad_dtype == AH_F32 || grad_dtype == AH_BF16, "ah_layernorm_bwd: grad dtype must be f32 or bf16");
   if (dim == 0) return AH_OK;
@@ -336,10 +337,10 @@ int32_t ah_layernorm_bwd(ah_ptr x, ah_ptr w, ah_ptr grad_out, int32_t grad_dtype
   float *part_dw = part, *part_db = part + (size_t)nblk * dim;
   if (grad_dtype == AH_F32)
     hipLaunchKernelGGL(k_layernorm_bwd<float>, dim3(nblk), dim3(TPB), lds, stream(), dp<const float>(x), dp<const float>(w),
-                       dp<const float>(grad_out), dp<const float>(residual_grad), dp<float>(dx), part_dw, part_db, rows, (int)dim, eps);
+                       dp<const float>(grad_out), dp<const float>(residual_grad), dp<float>(dx), dp<uint16_t>(dx_bf16), part_dw, part_db, rows, (int)dim, eps);
   else
     hipLaunchKernelGGL(k_layernorm_bwd<uint16_t>, dim3(nblk), dim3(TPB), lds, stream(), dp<const float>(x), dp<const float>(w),
-                       dp<const uint16_t>(grad_out), dp<const float>(residual_grad), dp<float>(dx), part_dw, part_db, rows, (int)dim, eps);
+                       dp<const uint16_t>(grad_out), dp<const float>(residual_grad), dp<float>(dx), dp<uint16_t>(dx_bf16), part_dw, part_db, rows, (int)dim, eps);
   AH_LAUNCH_CHECK();
   hipLaunchKernelGGL(k_colsum_partials, dim3((unsigned)cdiv(dim, TPB)), dim3(TPB), 0, stream(), part_dw, part_db, nblk, (int)dim,
                      dp<float>(dw), dp<float>(db), accumulate);

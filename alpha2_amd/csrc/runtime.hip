@@ -42,8 +42,14 @@ struct Context {
   // staging
   void *pinned = nullptr;
   size_t pinned_bytes = 0;
+  // ring of small pinned slots: uploads of a few bytes (per-step hyper-parameters) need no stream sync
+  char *ring = nullptr;
+  unsigned ring_next = 0;
+  hipEvent_t ring_ev[2] = {nullptr, nullptr};
 };
 Context g;
+
+constexpr unsigned RING_SLOTS = 256, RING_SLOT_BYTES = 256;
 
 size_t round_size(size_t b) {
   if (b == 0) b = 1;
@@ -102,6 +108,9 @@ int32_t ah_init(int32_t device) {
   AH_HIP(hipMalloc(&g.scratch, g.scratch_bytes));
   g.pinned_bytes = size_t(64) << 20;
   AH_HIP(hipHostMalloc(&g.pinned, g.pinned_bytes, hipHostMallocDefault));
+  AH_HIP(hipHostMalloc((void **)&g.ring, RING_SLOTS * RING_SLOT_BYTES, hipHostMallocDefault));
+  AH_HIP(hipEventCreateWithFlags(&g.ring_ev[0], hipEventDisableTiming));
+  AH_HIP(hipEventCreateWithFlags(&g.ring_ev[1], hipEventDisableTiming));
   g.device = device;
   g.inited = true;
   g.err[0] = 0;
@@ -125,6 +134,9 @@ int32_t ah_shutdown(void) {
   g.capture_pool.clear();
   if (g.scratch) (void)hipFree(g.scratch);
   if (g.pinned) (void)hipHostFree(g.pinned);
+  if (g.ring) (void)hipHostFree(g.ring);
+  if (g.ring_ev[0]) (void)hipEventDestroy(g.ring_ev[0]);
+  if (g.ring_ev[1]) (void)hipEventDestroy(g.ring_ev[1]);
   (void)hipStreamDestroy(g.stream);
   g = Context();
   return AH_OK;
@@ -205,6 +217,18 @@ int32_t ah_upload(ah_ptr dst, const void *host, uint64_t bytes) {
   if (g.capturing) return fail(AH_ERR_STATE, "ah_upload: illegal while a graph is being captured");
   if (bytes == 0) return AH_OK;
   AH_ARG(dst != 0 && host != nullptr, "ah_upload: null pointer");
+  if (bytes <= RING_SLOT_BYTES) {
+    // Small upload: copy into the next pinned ring slot and enqueue; no wait.  An event per half of the ring
+    // guarantees a slot's previous copy has completed before the slot is overwritten.
+    unsigned slot = g.ring_next % RING_SLOTS, half = slot / (RING_SLOTS / 2);
+    if (slot % (RING_SLOTS / 2) == 0 && g.ring_next >= RING_SLOTS) AH_HIP(hipEventSynchronize(g.ring_ev[half]));
+    char *p = g.ring + (size_t)slot * RING_SLOT_BYTES;
+    memcpy(p, host, bytes);
+    AH_HIP(hipMemcpyAsync(dp<void>(dst), p, bytes, hipMemcpyHostToDevice, g.stream));
+    if (slot % (RING_SLOTS / 2) == RING_SLOTS / 2 - 1) AH_HIP(hipEventRecord(g.ring_ev[half], g.stream));
+    g.ring_next++;
+    return AH_OK;
+  }
   // Stage through pinned memory so the caller's buffer is free again when this returns.
   const char *src = (const char *)host;
   uint64_t off = 0;

@@ -1,0 +1,358 @@
+"""Fast-mode training step: the same GPT step as `train.Trainer` (packages/train/src/trainer.ts:1146-1784 driving
+packages/model/src/gpt.ts:344-427), scheduled by hand on flat device arenas, bf16 activations and bf16 shadow weights
+for the MFMA operands, fp32 master weights / gradients / Adam moments, and captured once into a hipGraph that is
+replayed every step.
+
+Differences from the op-by-op path are layout and fusion only; the arithmetic is the same function:
+  * tok+pos embedding and their add are one kernel; the residual adds are GEMM epilogues; GELU (+ saved
+    pre-activation) and its derivative are GEMM epilogues; attention reads Q, K, V in place out of the [BT, 3C]
+    projection and writes merged heads;
+  * parameters, gradients and Adam moments each live in ONE arena ordered [decayed | not decayed], so the gradient
+    norm is one reduction and AdamW is two launches; the clip coefficient never visits the host
+    (trainer.ts:1650-1656 computes it on the host from a read-back norm);
+  * per-step scalars (lr, bias corrections) are read by the AdamW kernel from a small device struct written before
+    each replay, so the captured graph follows the LR schedule.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import math
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Tuple
+
+import numpy as np
+
+from . import _ffi as ffi
+from ._ffi import check
+from .backend import HipBackend, TensorData, shapeSize
+from .model import ModelConfig, collectParamEntries, ffn_dim, initGPT
+from .train import TrainConfig, lrAt, noDecayNames
+
+F32, BF16 = ffi.F32, ffi.BF16
+
+
+def _align(n: int, a: int = 64) -> int:
+    return (n + a - 1) // a * a
+
+
+@dataclass
+class StepStats:
+    loss: float
+    gradNorm: float
+    clipCoef: float
+    lr: float
+
+
+class FusedTrainer:
+    def __init__(self, backend: HipBackend, cfg: ModelConfig, tc: TrainConfig, batch: int, seed: int = 0, use_graph: bool = True,
+                 accum: int = 1, params: Optional[dict] = None):
+        if (cfg.ffnActivation or "gelu") != "gelu" or cfg.dropout != 0:
+            raise ValueError("FusedTrainer schedules the default GELU block without dropout; use train.Trainer for the variants")
+        self.B, self.lib, self.cfg, self.tc = backend, backend.lib, cfg, tc
+        self.batch, self.T, self.accum, self.use_graph = batch, cfg.blockSize, accum, use_graph
+        self.C, self.H, self.L, self.V, self.F = cfg.nEmbd, cfg.nHead, cfg.nLayer, cfg.vocabSize, ffn_dim(cfg)
+        self.D = self.C // self.H
+        if self.D not in (32, 64, 128) or self.C % 8 or self.F % 64 or self.C % 64 or self.V % 8:
+            raise ValueError("FusedTrainer needs head_dim in {32,64,128}, nEmbd and ffnDim multiples of 64, vocab multiple of 8")
+        self.BT = batch * self.T
+        self.cap = cfg.softCap if cfg.softCap is not None else 30.0
+        self._bufs: List[int] = []
+        self._graph = None
+        self._timed = None
+        self._snap = None
+        self.stepIdx = 0
+        self._b1p = self._b2p = 1.0
+
+        # ---- parameters: reference initialisation order (gpt.ts:73-151), then packed [decayed | not decayed]
+        if params is None:
+            from .rng import SeededRng
+            params = initGPT(cfg, backend, SeededRng(seed))
+        self.entries = collectParamEntries(params)
+        nodecay = noDecayNames(cfg.nLayer)
+        order = [e for e in self.entries if e[0] not in nodecay] + [e for e in self.entries if e[0] in nodecay]
+        self.off: Dict[str, int] = {}
+        pos = 0
+        for name, var in order:
+            if name in nodecay and "_split" not in self.off:
+                self.off["_split"] = pos
+            self.off[name] = pos
+            pos += _align(var.data.size)
+        self.off.setdefault("_split", pos)
+        self.nparam = pos
+        host = np.zeros(pos, dtype=np.float32)
+        for name, var in order:
+            host[self.off[name]:self.off[name] + var.data.size] = var.data.data
+        self.P, self.G, self.M, self.Vm = (self._alloc(pos * 4) for _ in range(4))
+        self.Pb = self._alloc(pos * 2)
+        check(self.lib.ah_upload(self.P, host.ctypes.data_as(C.c_void_p), host.nbytes))
+        for buf in (self.G, self.M, self.Vm):
+            check(self.lib.ah_fill_f32(buf, 0.0, pos))
+        check(self.lib.ah_cast(self.P, F32, self.Pb, BF16, pos))
+        self.shapes = {name: var.data.shape for name, var in self.entries}
+
+        # ---- activations (all shapes are static, so every buffer is allocated once)
+        BT, Cc, Fd, V = self.BT, self.C, self.F, self.V
+        a = self._alloc
+        self.tok, self.tgt = a(BT * 4), a(BT * 4)
+        self.x = [a(BT * Cc * 4) for _ in range(self.L + 1)]            # residual stream entering layer l (f32)
+        self.xmid = [a(BT * Cc * 4) for _ in range(self.L)]
+        self.ln1 = [a(BT * Cc * 2) for _ in range(self.L)]
+        self.qkv = [a(BT * 3 * Cc * 2) for _ in range(self.L)]
+        self.att = [a(BT * Cc * 2) for _ in range(self.L)]
+        self.lse = [a(batch * self.H * self.T * 4) for _ in range(self.L)]
+        self.ln2 = [a(BT * Cc * 2) for _ in range(self.L)]
+        self.hpre = [a(BT * Fd * 2) for _ in range(self.L)]
+        self.hact = [a(BT * Fd * 2) for _ in range(self.L)]
+        self.lnf, self.logits, self.rowlse = a(BT * Cc * 2), a(BT * V * 2), a(BT * 4)
+        self.dx = [a(BT * Cc * 4), a(BT * Cc * 4)]
+        self.dxb, self.dlnb, self.datt = a(BT * Cc * 2), a(BT * Cc * 2), a(BT * Cc * 2)
+        self.dh, self.dqkv = a(BT * Fd * 2), a(BT * 3 * Cc * 2)
+        self.loss, self.sumsq, self.clip = a(4), a(4), a(8)
+        self.hyper = a(ffi.C.sizeof(ffi.AhAdamW))
+        self.loss_hist_cap = 4096
+        self.loss_hist, self.norm_hist = a(self.loss_hist_cap * 4), a(self.loss_hist_cap * 8)
+        self._batches: List[Tuple[int, int]] = []
+
+    # ------------------------------------------------------------------ helpers
+    def _alloc(self, nbytes: int) -> int:
+        p = C.c_uint64()
+        check(self.lib.ah_alloc(max(16, nbytes), C.byref(p)))
+        self._bufs.append(p.value)
+        return p.value
+
+    def p(self, name: str, bf16: bool = False) -> int:
+        return (self.Pb + self.off[name] * 2) if bf16 else (self.P + self.off[name] * 4)
+
+    def g(self, name: str) -> int:
+        return self.G + self.off[name] * 4
+
+    def _gemm(self, layout, a, b, c, m, n, k, lda, ldb, ldc, out=BF16, epi=ffi.EPI_NONE, aux=0):
+        g = ffi.AhGemm(layout, BF16, out, epi, m, n, k, lda, ldb, ldc, 1, 0, 0, 0, a, b, c, aux)
+        if self._timed is None:
+            check(self.lib.ah_gemm(C.byref(g)))
+            return
+        e0, e1 = self.B._event(), self.B._event()
+        check(self.lib.ah_event_record(e0))
+        check(self.lib.ah_gemm(C.byref(g)))
+        check(self.lib.ah_event_record(e1))
+        self._timed.append({"kind": "gemm", "layout": layout, "m": m, "n": n, "k": k, "flops": 2.0 * m * n * k, "e0": e0, "e1": e1})
+
+    def _flash(self, l: int, bwd: bool):
+        Cc, T, D = self.C, self.T, self.D
+        f = ffi.AhFlash()
+        f.dtype, f.batch, f.heads, f.seq, f.head_dim = BF16, self.batch, self.H, T, D
+        for nm in ("q", "k", "v"):
+            setattr(f, nm + "_sb", T * 3 * Cc), setattr(f, nm + "_sh", D), setattr(f, nm + "_st", 3 * Cc)
+        f.o_sb, f.o_sh, f.o_st = T * Cc, D, Cc
+        f.scale, f.soft_cap = 1 / math.sqrt(D), self.cap
+        q = self.qkv[l]
+        f.q, f.k, f.v, f.o, f.lse = q, q + Cc * 2, q + 2 * Cc * 2, self.att[l], self.lse[l]
+        if bwd:
+            d = self.dqkv
+            f.d_o, f.dq, f.dk, f.dv = self.datt, d, d + Cc * 2, d + 2 * Cc * 2
+        t0 = None
+        if self._timed is not None:
+            t0 = self.B._event()
+            check(self.lib.ah_event_record(t0))
+        check((self.lib.ah_flash_bwd if bwd else self.lib.ah_flash_fwd)(C.byref(f)))
+        if t0 is not None:
+            t1 = self.B._event()
+            check(self.lib.ah_event_record(t1))
+            fl = 4.0 * self.batch * self.H * T * T * D * (2 if bwd else 1)
+            self._timed.append({"kind": "flash_bwd" if bwd else "flash_fwd", "flops": fl, "e0": t0, "e1": t1})
+
+    # ------------------------------------------------------------------ the step
+    def _forward_backward(self, first_micro: bool):
+        lib, BT, Cc, Fd, V, L = self.lib, self.BT, self.C, self.F, self.V, self.L
+        NN, NT, TN = ffi.GEMM_NN, ffi.GEMM_NT, ffi.GEMM_TN
+        acc = 0 if first_micro else 1
+        wepi = ffi.EPI_NONE if first_micro else ffi.EPI_ACCUM
+        check(lib.ah_embedding_tok_pos(self.p("wte"), self.p("wpe"), self.tok, self.x[0], BT, self.T, Cc, V))
+        for l in range(L):
+            pre = f"layer.{l}."
+            check(lib.ah_layernorm(self.x[l], self.p(pre + "ln1.weight"), self.p(pre + "ln1.bias"), self.ln1[l], BT, Cc, 1e-5, BF16))
+            self._gemm(NT, self.ln1[l], self.p(pre + "attn.wqkv", True), self.qkv[l], BT, 3 * Cc, Cc, Cc, Cc, 3 * Cc)
+            self._flash(l, False)
+            self._gemm(NT, self.att[l], self.p(pre + "attn.wo", True), self.xmid[l], BT, Cc, Cc, Cc, Cc, Cc, F32, ffi.EPI_RESIDUAL, self.x[l])
+            check(lib.ah_layernorm(self.xmid[l], self.p(pre + "ln2.weight"), self.p(pre + "ln2.bias"), self.ln2[l], BT, Cc, 1e-5, BF16))
+            self._gemm(NT, self.ln2[l], self.p(pre + "mlp.fc1", True), self.hact[l], BT, Fd, Cc, Cc, Cc, Fd, BF16, ffi.EPI_GELU, self.hpre[l])
+            self._gemm(NT, self.hact[l], self.p(pre + "mlp.fc2", True), self.x[l + 1], BT, Cc, Fd, Fd, Fd, Cc, F32, ffi.EPI_RESIDUAL, self.xmid[l])
+        check(lib.ah_layernorm(self.x[L], self.p("lnF.weight"), self.p("lnF.bias"), self.lnf, BT, Cc, 1e-5, BF16))
+        self._gemm(NT, self.lnf, self.p("lmHead", True), self.logits, BT, V, Cc, Cc, Cc, V)
+        check(lib.ah_cross_entropy(self.logits, BF16, self.tgt, self.loss, self.rowlse, BT, V))
+        check(lib.ah_cross_entropy_bwd(self.logits, BF16, self.tgt, self.rowlse, 0, 1.0, self.logits, BT, V))     # dlogits in place
+
+        self._gemm(NN, self.logits, self.p("lmHead", True), self.dlnb, BT, Cc, V, V, Cc, Cc)
+        self._gemm(TN, self.logits, self.lnf, self.g("lmHead"), V, Cc, BT, V, Cc, Cc, F32, wepi)
+        cur = 0
+        check(lib.ah_layernorm_bwd(self.x[L], self.p("lnF.weight"), self.dlnb, BF16, 0, self.dx[cur], self.dxb, self.g("lnF.weight"),
+                                   self.g("lnF.bias"), BT, Cc, 1e-5, acc))
+        for l in reversed(range(L)):
+            pre = f"layer.{l}."
+            # MLP: x_out = x_mid + fc2(gelu(fc1(ln2(x_mid))))
+            self._gemm(NN, self.dxb, self.p(pre + "mlp.fc2", True), self.dh, BT, Fd, Cc, Cc, Fd, Fd, BF16, ffi.EPI_GELU_BWD, self.hpre[l])
+            self._gemm(TN, self.dxb, self.hact[l], self.g(pre + "mlp.fc2"), Cc, Fd, BT, Cc, Fd, Fd, F32, wepi)
+            self._gemm(NN, self.dh, self.p(pre + "mlp.fc1", True), self.dlnb, BT, Cc, Fd, Fd, Cc, Cc)
+            self._gemm(TN, self.dh, self.ln2[l], self.g(pre + "mlp.fc1"), Fd, Cc, BT, Fd, Cc, Cc, F32, wepi)
+            check(lib.ah_layernorm_bwd(self.xmid[l], self.p(pre + "ln2.weight"), self.dlnb, BF16, self.dx[cur], self.dx[cur ^ 1], self.dxb,
+                                       self.g(pre + "ln2.weight"), self.g(pre + "ln2.bias"), BT, Cc, 1e-5, acc))
+            cur ^= 1
+            # attention: x_mid = x_in + wo(attn(wqkv(ln1(x_in))))
+            self._gemm(NN, self.dxb, self.p(pre + "attn.wo", True), self.datt, BT, Cc, Cc, Cc, Cc, Cc)
+            self._gemm(TN, self.dxb, self.att[l], self.g(pre + "attn.wo"), Cc, Cc, BT, Cc, Cc, Cc, F32, wepi)
+            self._flash(l, True)
+            self._gemm(NN, self.dqkv, self.p(pre + "attn.wqkv", True), self.dlnb, BT, Cc, 3 * Cc, 3 * Cc, Cc, Cc)
+            self._gemm(TN, self.dqkv, self.ln1[l], self.g(pre + "attn.wqkv"), 3 * Cc, Cc, BT, 3 * Cc, Cc, Cc, F32, wepi)
+            check(lib.ah_layernorm_bwd(self.x[l], self.p(pre + "ln1.weight"), self.dlnb, BF16, self.dx[cur], self.dx[cur ^ 1], self.dxb,
+                                       self.g(pre + "ln1.weight"), self.g(pre + "ln1.bias"), BT, Cc, 1e-5, acc))
+            cur ^= 1
+        check(lib.ah_embedding_bwd(self.tok, self.dx[cur], self.g("wte"), BT, Cc, V, acc))
+        check(lib.ah_pos_embedding_bwd(self.dx[cur], self.g("wpe"), self.batch, self.T, Cc, acc))
+
+    def _optimizer(self):
+        lib, tc = self.lib, self.tc
+        split = self.off["_split"]
+        check(lib.ah_sum_sq(self.G, self.nparam, self.sumsq))               # arena padding is zero and stays zero
+        check(lib.ah_clip_coef(self.sumsq, 1.0 / self.accum, tc.gradClip, self.clip))
+        h = ffi.AhAdamW(tc.lr, tc.beta1, tc.beta2, tc.eps, tc.weightDecay, 1.0, 1.0, 1.0 / self.accum)
+        if split > 0:
+            check(lib.ah_adamw(self.P, self.G, self.M, self.Vm, split, C.byref(h), self.hyper, self.clip, self.Pb))
+        h.weight_decay = 0.0
+        n2 = self.nparam - split
+        if n2 > 0:
+            check(lib.ah_adamw(self.P + split * 4, self.G + split * 4, self.M + split * 4, self.Vm + split * 4, n2, C.byref(h), self.hyper,
+                               self.clip, self.Pb + split * 2))
+
+    def _whole_step(self):
+        self._forward_backward(True)
+        self._optimizer()
+
+    def set_batch(self, inputs: TensorData, targets: TensorData):
+        """Make one [B, T] token batch resident; step() then trains on it until another is set."""
+        self.add_batch(inputs, targets)
+        self._use_batch(len(self._batches) - 1)
+
+    def add_batch(self, inputs: TensorData, targets: TensorData) -> int:
+        n = self.BT * 4
+        ti, tt = self._alloc(n), self._alloc(n)
+        a, b = np.ascontiguousarray(inputs.data, dtype=np.int32), np.ascontiguousarray(targets.data, dtype=np.int32)
+        if a.size != self.BT or b.size != self.BT:
+            raise ValueError(f"batch must be [{self.batch}, {self.T}]")
+        check(self.lib.ah_upload(ti, a.ctypes.data_as(C.c_void_p), n))
+        check(self.lib.ah_upload(tt, b.ctypes.data_as(C.c_void_p), n))
+        self._batches.append((ti, tt))
+        return len(self._batches) - 1
+
+    def _use_batch(self, i: int):
+        ti, tt = self._batches[i]
+        check(self.lib.ah_copy(self.tok, ti, self.BT * 4))
+        check(self.lib.ah_copy(self.tgt, tt, self.BT * 4))
+
+    def _write_hyper(self) -> float:
+        tc = self.tc
+        lr = lrAt(tc, self.stepIdx)
+        self._b1p *= tc.beta1
+        self._b2p *= tc.beta2
+        h = ffi.AhAdamW(lr, tc.beta1, tc.beta2, tc.eps, tc.weightDecay, 1 - self._b1p, 1 - self._b2p, 1.0 / self.accum)
+        check(self.lib.ah_upload(self.hyper, C.byref(h), C.sizeof(h)))
+        return lr
+
+    def step(self, batch_index: Optional[int] = None) -> int:
+        """Enqueue one optimizer step (no host synchronisation); returns the step index whose loss / grad-norm can be
+        read later with history()."""
+        if batch_index is not None:
+            self._use_batch(batch_index)
+        elif not self._batches:
+            raise RuntimeError("no batch set")
+        self._write_hyper()
+        if self.accum != 1:
+            raise NotImplementedError("micro-batch accumulation runs through step_accum()")
+        if self.use_graph:
+            if self._graph is None:
+                self.prepare()
+                self._whole_step()                       # eager once: fills the allocator pool, raises any argument error
+                self.B.syncGpu()
+                self._restore_after_warm_step()
+                check(self.lib.ah_graph_begin())
+                try:
+                    self._whole_step()
+                finally:
+                    gid = C.c_uint64()
+                    check(self.lib.ah_graph_end(C.byref(gid)))
+                self._graph = gid.value
+            check(self.lib.ah_graph_launch(self._graph))
+        else:
+            self._whole_step()
+        i = self.stepIdx % self.loss_hist_cap
+        check(self.lib.ah_copy(self.loss_hist + i * 4, self.loss, 4))
+        check(self.lib.ah_copy(self.norm_hist + i * 8, self.clip, 8))
+        self.stepIdx += 1
+        return self.stepIdx - 1
+
+    def _restore_after_warm_step(self):
+        """The eager run that precedes capture must not count as a training step: put parameters and moments back."""
+        check(self.lib.ah_copy(self.P, self._snap[0], self.nparam * 4))
+        check(self.lib.ah_copy(self.M, self._snap[1], self.nparam * 4))
+        check(self.lib.ah_copy(self.Vm, self._snap[2], self.nparam * 4))
+        check(self.lib.ah_cast(self.P, F32, self.Pb, BF16, self.nparam))
+        for s in self._snap:
+            check(self.lib.ah_free(s))
+            self._bufs.remove(s)
+        self._snap = None
+
+    def prepare(self):
+        """Snapshot state ahead of the warm-up run inside the first step()."""
+        self._snap = [self._alloc(self.nparam * 4) for _ in range(3)]
+        for dst, src in zip(self._snap, (self.P, self.M, self.Vm)):
+            check(self.lib.ah_copy(dst, src, self.nparam * 4))
+
+    def history(self, first: int, count: int) -> List[StepStats]:
+        """Blocks; loss, gradient norm and clip coefficient of steps [first, first+count)."""
+        self.B.syncGpu()
+        out = []
+        lo, nm = np.empty(self.loss_hist_cap, np.float32), np.empty(self.loss_hist_cap * 2, np.float32)
+        check(self.lib.ah_download(lo.ctypes.data_as(C.c_void_p), self.loss_hist, lo.nbytes))
+        check(self.lib.ah_download(nm.ctypes.data_as(C.c_void_p), self.norm_hist, nm.nbytes))
+        for s in range(first, first + count):
+            i = s % self.loss_hist_cap
+            out.append(StepStats(float(lo[i]), float(nm[2 * i + 1]), float(nm[2 * i]), lrAt(self.tc, s)))
+        return out
+
+    def timed_step(self) -> list:
+        """One eager step with every GEMM and attention launch bracketed by HIP events on the library stream."""
+        self.B.syncGpu()
+        self._write_hyper()
+        self._timed = []
+        self._whole_step()
+        recs, self._timed = self._timed, None
+        ms = C.c_float()
+        for r in recs:
+            check(self.lib.ah_event_elapsed_ms(r["e0"], r["e1"], C.byref(ms)))
+            r["ms"] = ms.value
+            for e in (r.pop("e0"), r.pop("e1")):
+                check(self.lib.ah_event_destroy(e))
+        self.stepIdx += 1
+        return recs
+
+    def param(self, name: str) -> np.ndarray:
+        n = shapeSize(self.shapes[name])
+        out = np.empty(n, np.float32)
+        self.B.syncGpu()
+        check(self.lib.ah_download(out.ctypes.data_as(C.c_void_p), self.p(name), n * 4))
+        return out
+
+    def grad(self, name: str) -> np.ndarray:
+        n = shapeSize(self.shapes[name])
+        out = np.empty(n, np.float32)
+        self.B.syncGpu()
+        check(self.lib.ah_download(out.ctypes.data_as(C.c_void_p), self.g(name), n * 4))
+        return out
+
+    def close(self):
+        self.B.syncGpu()
+        if self._graph is not None:
+            check(self.lib.ah_graph_destroy(self._graph))
+            self._graph = None
+        for b in self._bufs:
+            self.lib.ah_free(b)
+        self._bufs = []

@@ -178,9 +178,10 @@ int32_t ah_pos_embedding_bwd(ah_ptr grad_out, ah_ptr grad_wpe, int64_t batch, in
 int32_t ah_layernorm(ah_ptr x, ah_ptr w, ah_ptr b, ah_ptr out, int64_t rows, int64_t dim, float eps,
                      int32_t out_dtype);
 /* dx (+= residual_grad when that handle is non-zero), dw, db.  dw/db are deterministic column sums;
- * accumulate != 0 adds them into existing dw/db (gradient accumulation). grad_out dtype f32 or bf16. */
+ * accumulate != 0 adds them into existing dw/db (gradient accumulation). grad_out dtype f32 or bf16.
+ * dx_bf16 (0 = none) also receives dx rounded to bf16, the operand of the next backward GEMMs. */
 int32_t ah_layernorm_bwd(ah_ptr x, ah_ptr w, ah_ptr grad_out, int32_t grad_dtype, ah_ptr residual_grad,
-                         ah_ptr dx, ah_ptr dw, ah_ptr db, int64_t rows, int64_t dim, float eps,
+                         ah_ptr dx, ah_ptr dx_bf16, ah_ptr dw, ah_ptr db, int64_t rows, int64_t dim, float eps,
                          int32_t accumulate);
 /* loss[0] = mean_i (logsumexp(logits[i,:]) - logits[i,target[i]]); lse[N] kept for backward (0 = skip) */
 int32_t ah_cross_entropy(ah_ptr logits, int32_t logits_dtype, ah_ptr targets_i32, ah_ptr loss_out, ah_ptr lse_out,
