@@ -163,14 +163,105 @@ __global__ void k_layernorm_bwd(const float *__restrict__ x, const float *__rest
     part_db[(size_t)blockIdx.x * dim + j] = c;
   }
 }
+// column sums of the per-block partials: 32 columns per block, 8 row slices per column, fixed summation order
 __global__ void k_colsum_partials(const float *__restrict__ part_dw, const float *__restrict__ part_db, int nparts, int dim,
                                   float *__restrict__ dw, float *__restrict__ db, int accumulate) {
-  int j = blockIdx.x * blockDim.x + threadIdx.x;
-  if (j >= dim) return;
+  __shared__ double sa[8][33], sc[8][33];
+  int cx = threadIdx.x & 31, sl = threadIdx.x >> 5, j = blockIdx.x * 32 + cx;
   double a = 0, c = 0;
-  for (int p = 0; p < nparts; p++) { a += part_dw[(size_t)p * dim + j]; c += part_db[(size_t)p * dim + j]; }
-  dw[j] = (accumulate ? dw[j] : 0.f) + (float)a;
-  db[j] = (accumulate ? db[j] : 0.f) + (float)c;
+  if (j < dim)
+    for (int p = sl; p < nparts; p += 8) { a += part_dw[(size_t)p * dim + j]; c += part_db[(size_t)p * dim + j]; }
+  sa[sl][cx] = a; sc[sl][cx] = c;
+  __syncthreads();
+  if (sl == 0 && j < dim) {
+    for (int k = 1; k < 8; k++) { a += sa[k][cx]; c += sc[k][cx]; }
+    dw[j] = (accumulate ? dw[j] : 0.f) + (float)a;
+    db[j] = (accumulate ? db[j] : 0.f) + (float)c;
+  }
+}
+
+// Register-resident LayerNorm backward for rows of up to 256*NV floats (dim % 4 == 0): x, g and the residual gradient
+// are each read once; dw / db accumulate in per-lane registers over all rows a wave walks.
+template <class G> __device__ __forceinline__ float4 ld4(const G *p, int j);
+template <> __device__ __forceinline__ float4 ld4<float>(const float *p, int j) { return reinterpret_cast<const float4 *>(p)[j]; }
+template <> __device__ __forceinline__ float4 ld4<uint16_t>(const uint16_t *p, int j) {
+  uint2 u = reinterpret_cast<const uint2 *>(p)[j];
+  return make_float4(bf16_bits_to_f32(u.x & 0xffff), bf16_bits_to_f32(u.x >> 16), bf16_bits_to_f32(u.y & 0xffff), bf16_bits_to_f32(u.y >> 16));
+}
+template <int NV, class G>
+__global__ __launch_bounds__(256) void k_layernorm_bwd_vec(const float *__restrict__ x, const float *__restrict__ w, const G *__restrict__ g,
+                                                           const float *__restrict__ res, float *__restrict__ dx, uint16_t *__restrict__ dx16,
+                                                           float *__restrict__ part_dw, float *__restrict__ part_db, int64_t rows, int dim, float eps) {
+  extern __shared__ float sh[];      // [2][WPB][dim]
+  int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nv = dim >> 2;
+  float inv_dim = 1.0f / (float)dim;
+  float4 wv[NV], adw[NV], adb[NV];
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    int j = lane + 64 * i;
+    wv[i] = j < nv ? reinterpret_cast<const float4 *>(w)[j] : make_float4(0, 0, 0, 0);
+    adw[i] = make_float4(0, 0, 0, 0); adb[i] = make_float4(0, 0, 0, 0);
+  }
+  int64_t stride = (int64_t)gridDim.x * WPB;
+  for (int64_t row = blockIdx.x * (int64_t)WPB + wave; row < rows; row += stride) {
+    const float *xr = x + row * (int64_t)dim;
+    const G *gr = g + row * (int64_t)dim;
+    float4 xv[NV], gv[NV];
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+      int j = lane + 64 * i;
+      bool ok = j < nv;
+      xv[i] = ok ? reinterpret_cast<const float4 *>(xr)[j] : make_float4(0, 0, 0, 0);
+      gv[i] = ok ? ld4<G>(gr, j) : make_float4(0, 0, 0, 0);
+      s += (xv[i].x + xv[i].y) + (xv[i].z + xv[i].w);
+    }
+    float mean = wave_sum(s) * inv_dim, q = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; i++)
+      if (lane + 64 * i < nv) {
+        float a = xv[i].x - mean, b = xv[i].y - mean, c = xv[i].z - mean, d = xv[i].w - mean;
+        q += (a * a + b * b) + (c * c + d * d);
+      }
+    float rstd = 1.0f / sqrtf(wave_sum(q) * inv_dim + eps), s1 = 0.f, s2 = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; i++) {       // xv becomes xhat; out-of-range lanes hold g = w = 0 and contribute nothing
+      xv[i].x = (xv[i].x - mean) * rstd; xv[i].y = (xv[i].y - mean) * rstd; xv[i].z = (xv[i].z - mean) * rstd; xv[i].w = (xv[i].w - mean) * rstd;
+      float d0 = gv[i].x * wv[i].x, d1 = gv[i].y * wv[i].y, d2 = gv[i].z * wv[i].z, d3 = gv[i].w * wv[i].w;
+      s1 += (d0 + d1) + (d2 + d3);
+      s2 += (d0 * xv[i].x + d1 * xv[i].y) + (d2 * xv[i].z + d3 * xv[i].w);
+      adw[i].x += gv[i].x * xv[i].x; adw[i].y += gv[i].y * xv[i].y; adw[i].z += gv[i].z * xv[i].z; adw[i].w += gv[i].w * xv[i].w;
+      adb[i].x += gv[i].x; adb[i].y += gv[i].y; adb[i].z += gv[i].z; adb[i].w += gv[i].w;
+    }
+    s1 = wave_sum(s1) * inv_dim; s2 = wave_sum(s2) * inv_dim;
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+      int j = lane + 64 * i;
+      if (j < nv) {
+        float4 d;
+        d.x = rstd * (gv[i].x * wv[i].x - (s1 + xv[i].x * s2)); d.y = rstd * (gv[i].y * wv[i].y - (s1 + xv[i].y * s2));
+        d.z = rstd * (gv[i].z * wv[i].z - (s1 + xv[i].z * s2)); d.w = rstd * (gv[i].w * wv[i].w - (s1 + xv[i].w * s2));
+        if (res) { float4 r = reinterpret_cast<const float4 *>(res + row * (int64_t)dim)[j]; d.x += r.x; d.y += r.y; d.z += r.z; d.w += r.w; }
+        reinterpret_cast<float4 *>(dx + row * (int64_t)dim)[j] = d;
+        if (dx16) reinterpret_cast<uint2 *>(dx16 + row * (int64_t)dim)[j] = make_uint2(pack_bf16x2(d.x, d.y), pack_bf16x2(d.z, d.w));
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    int j = lane + 64 * i;
+    if (j < nv) {
+      reinterpret_cast<float4 *>(sh + (size_t)wave * dim)[j] = adw[i];
+      reinterpret_cast<float4 *>(sh + (size_t)(WPB + wave) * dim)[j] = adb[i];
+    }
+  }
+  __syncthreads();
+  for (int j = threadIdx.x; j < dim; j += blockDim.x) {
+    float a = 0.f, c = 0.f;
+    for (int k = 0; k < WPB; k++) { a += sh[(size_t)k * dim + j]; c += sh[(size_t)(WPB + k) * dim + j]; }
+    part_dw[(size_t)blockIdx.x * dim + j] = a;
+    part_db[(size_t)blockIdx.x * dim + j] = c;
+  }
 }
 
 // ---------------------------------------------------------------- softmax cross-entropy
@@ -188,7 +279,24 @@ __global__ void k_ce_fwd(const T *__restrict__ logits, const int32_t *__restrict
   int64_t row = blockIdx.x;
   const T *p = logits + row * c;
   float m = -INFINITY, s = 0.f;
-  for (int64_t j = threadIdx.x; j < c; j += blockDim.x) {
+  constexpr int VW = 16 / sizeof(T);                    // elements per 16-byte load
+  int64_t nvec = ((((uintptr_t)p) & 15u) == 0) ? c / VW : 0;
+  for (int64_t j = threadIdx.x; j < nvec; j += blockDim.x) {
+    uint4 u = reinterpret_cast<const uint4 *>(p)[j];
+    float v[VW];
+    if (sizeof(T) == 4) { v[0] = __uint_as_float(u.x); v[1] = __uint_as_float(u.y); v[2] = __uint_as_float(u.z); v[VW - 1] = __uint_as_float(u.w); }
+    else {
+      v[0] = bf16_bits_to_f32(u.x & 0xffff); v[1] = bf16_bits_to_f32(u.x >> 16); v[2] = bf16_bits_to_f32(u.y & 0xffff); v[3] = bf16_bits_to_f32(u.y >> 16);
+      v[VW - 4] = bf16_bits_to_f32(u.z & 0xffff); v[VW - 3] = bf16_bits_to_f32(u.z >> 16); v[VW - 2] = bf16_bits_to_f32(u.w & 0xffff); v[VW - 1] = bf16_bits_to_f32(u.w >> 16);
+    }
+    float vm = v[0];
+#pragma unroll
+    for (int i = 1; i < VW; i++) vm = fmaxf(vm, v[i]);
+    if (vm > m) { s *= __expf(m - vm); m = vm; }
+#pragma unroll
+    for (int i = 0; i < VW; i++) s += __expf(v[i] - m);
+  }
+  for (int64_t j = nvec * VW + threadIdx.x; j < c; j += blockDim.x) {
     float v = Io<T>::ld(p, j);
     if (v > m) { s = s * expf(m - v) + 1.0f; m = v; } else { s += expf(v - m); }
   }
@@ -228,6 +336,21 @@ __global__ void k_ce_bwd(const T *__restrict__ logits, const int32_t *__restrict
   int32_t t = targets[row];
   const T *p = logits + row * c;
   T *q = out + row * c;
+  if (sizeof(T) == 2 && (c & 7) == 0 && (((uintptr_t)logits | (uintptr_t)out) & 15u) == 0) {      // bf16: 8 classes per 16-byte access
+    for (int64_t j8 = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; j8 < (c >> 3); j8 += (int64_t)gridDim.x * blockDim.x) {
+      uint4 u = reinterpret_cast<const uint4 *>(p)[j8];
+      uint32_t in[4] = {u.x, u.y, u.z, u.w}, o[4];
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        int64_t j = j8 * 8 + 2 * i;
+        float a = (__expf(bf16_bits_to_f32(in[i] & 0xffff) - l) - (j == t ? 1.0f : 0.0f)) * scale;
+        float b = (__expf(bf16_bits_to_f32(in[i] >> 16) - l) - (j + 1 == t ? 1.0f : 0.0f)) * scale;
+        o[i] = pack_bf16x2(a, b);
+      }
+      reinterpret_cast<uint4 *>(q)[j8] = make_uint4(o[0], o[1], o[2], o[3]);
+    }
+    return;
+  }
   for (int64_t j = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; j < c; j += (int64_t)gridDim.x * blockDim.x) {
     float prob = expf(Io<T>::ld(p, j) - l);
     Io<T>::st(q, j, (prob - (j == t ? 1.0f : 0.0f)) * scale);
@@ -335,14 +458,25 @@ int32_t ah_layernorm_bwd(ah_ptr x, ah_ptr w, ah_ptr grad_out, int32_t grad_dtype
   float *part = (float *)scratch(sizeof(float) * 2 * (size_t)nblk * (size_t)dim);
   if (!part) return fail(AH_ERR_OOM, "ah_layernorm_bwd: no scratch");
   float *part_dw = part, *part_db = part + (size_t)nblk * dim;
-  if (grad_dtype == AH_F32)
+  bool vec = dim % 4 == 0 && dim <= 2048 && aligned16(x) && aligned16(w) && aligned16(dx) && (grad_out % 8 == 0) && (residual_grad % 16 == 0) &&
+             (dx_bf16 % 8 == 0) && (grad_dtype == AH_BF16 || aligned16(grad_out));
+  if (vec) {
+    int nvl = (int)cdiv(dim / 4, 64);
+#define LNB_CASE(NV, GT) hipLaunchKernelGGL((k_layernorm_bwd_vec<NV, GT>), dim3(nblk), dim3(TPB), lds, stream(), dp<const float>(x), dp<const float>(w), \
+      dp<const GT>(grad_out), dp<const float>(residual_grad), dp<float>(dx), dp<uint16_t>(dx_bf16), part_dw, part_db, rows, (int)dim, eps)
+#define LNB_SWITCH(GT) switch (nvl) { case 1: LNB_CASE(1, GT); break; case 2: LNB_CASE(2, GT); break; case 3: LNB_CASE(3, GT); break; \
+      case 4: LNB_CASE(4, GT); break; case 5: case 6: LNB_CASE(6, GT); break; default: LNB_CASE(8, GT); break; }
+    if (grad_dtype == AH_F32) { LNB_SWITCH(float) } else { LNB_SWITCH(uint16_t) }
+#undef LNB_SWITCH
+#undef LNB_CASE
+  } else if (grad_dtype == AH_F32)
     hipLaunchKernelGGL(k_layernorm_bwd<float>, dim3(nblk), dim3(TPB), lds, stream(), dp<const float>(x), dp<const float>(w),
                        dp<const float>(grad_out), dp<const float>(residual_grad), dp<float>(dx), dp<uint16_t>(dx_bf16), part_dw, part_db, rows, (int)dim, eps);
   else
     hipLaunchKernelGGL(k_layernorm_bwd<uint16_t>, dim3(nblk), dim3(TPB), lds, stream(), dp<const float>(x), dp<const float>(w),
                        dp<const uint16_t>(grad_out), dp<const float>(residual_grad), dp<float>(dx), dp<uint16_t>(dx_bf16), part_dw, part_db, rows, (int)dim, eps);
   AH_LAUNCH_CHECK();
-  hipLaunchKernelGGL(k_colsum_partials, dim3((unsigned)cdiv(dim, TPB)), dim3(TPB), 0, stream(), part_dw, part_db, nblk, (int)dim,
+  hipLaunchKernelGGL(k_colsum_partials, dim3((unsigned)cdiv(dim, 32)), dim3(TPB), 0, stream(), part_dw, part_db, nblk, (int)dim,
                      dp<float>(dw), dp<float>(db), accumulate);
   AH_LAUNCH_CHECK();
   return AH_OK;

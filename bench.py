@@ -95,7 +95,11 @@ def main():
     B.syncGpu()
     dt = time.perf_counter() - t0
     ms = dt / args.steps * 1e3
-    loss_last = losses[-1].loss if hasattr(losses[-1], "loss") else float(losses[-1])
+    if hasattr(runner, "history"):
+        hist = runner.history(0, args.warmup + args.steps)
+        loss_first, loss_last = hist[0].loss, hist[-1].loss
+    else:
+        loss_first, loss_last = losses[0].loss, losses[-1].loss
 
     # one instrumented step: every GEMM launch bracketed by HIP events on the library stream
     recs = runner.timed_step() if hasattr(runner, "timed_step") else _timed(B, one_step)
@@ -109,7 +113,7 @@ def main():
         "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic (Zipf s=1.1 token ids, seed 4; random-init N(0,0.02) weights, seed 0)",
         "config": {"workload": "GPT-2-small-shape train step: vocab 50304, d_model 768, 12 layers, 12 heads, ctx 1024, batch 16, "
                                "untied lmHead (163.0M params), AdamW lr 3e-4 betas (0.9,0.95) wd 0.1, grad-clip 1.0",
-                   "tokens_per_step": tokens, "mode": args.mode, "loss_after": loss_last},
+                   "tokens_per_step": tokens, "mode": args.mode, "loss_first_step": loss_first, "loss_last_step": loss_last},
         "step_tflops": flops / (ms * 1e-3) / 1e12, "mfu_vs_bf16_dense_peak": flops / (ms * 1e-3) / 1e12 / PEAK["bf16"],
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK[dtype], "unit": "TFLOP/s", "frac": achieved / PEAK[dtype],
                      "traffic": None, "kernel": "k_gemm_bf16_nt" if dtype == "bf16" else "k_gemm_f32",
