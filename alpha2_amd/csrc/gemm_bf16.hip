@@ -1,11 +1,11 @@
 // bf16 GEMM on v_mfma_f32_32x32x16_bf16 for all three operand layouts of the training step.
 //
-// Block tile BM x BN x 64, 4 waves (2 x 2), fp32 accumulators (AGPRs), LDS double-buffered.  Global loads run
-// PF k-tiles ahead in registers so HBM / L2 latency is covered by PF tiles of MFMA work.
+// Block tile BM x BN x 64 on WGM x WGN waves, fp32 accumulators, LDS double-buffered.  Global loads run one k-tile
+// ahead in registers so HBM / L2 latency is covered by a tile of MFMA work.
 //   k-contiguous operand ([row][K] in memory): LDS tile [rows][64 + 8]; a fragment is one 16-byte read; the
 //     144-byte pitch puts 8 consecutive rows on 8 distinct bank groups.
 //   k-major operand ([K][row] in memory: W for dX = G W, G and X for dW = G^T X): the tile is copied as it lies,
-//     LDS [64][rows + 16], and fragments come from ds_read_b64_tr_b16, the gfx950 LDS transpose read: within 16
+//     LDS [64][rows + 32], and fragments come from ds_read_b64_tr_b16, the gfx950 LDS transpose read: within 16
 //     lanes, lane j receives for q = 0..3 element [j % 4] of the 8 bytes addressed by lane 4q + j/4, so 16 lanes
 //     pointing at a 4(k) x 16(row) block each get 4 consecutive k of "their" row.
 // Addressing: one uniform 64-bit base per operand and k-tile (SGPRs) plus a 32-bit per-thread offset per chunk, so
@@ -18,21 +18,22 @@ using namespace ah;
 namespace {
 
 constexpr int G_BK = 64, G_PK = 72;      // k tile; k-contiguous LDS pitch (bf16 elements)
+constexpr int G_KPAD = 32;               // k-major LDS pitch = rows + 32: consecutive k rows 64 bytes apart modulo 256
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));   // a native vector (not the HIP struct) so staging arrays stay in VGPRs
 
-template <int ROWS, bool KMAJOR> struct TileGeom {
-  static constexpr int PITCH = KMAJOR ? ROWS + 16 : G_PK;
-  static constexpr int ELEMS = KMAJOR ? G_BK * (ROWS + 16) : ROWS * G_PK;
-  static constexpr int CHUNKS = ROWS * G_BK / 8 / 256;      // 16-byte chunks per thread and k-tile
+template <int ROWS, bool KMAJOR, int NT> struct TileGeom {
+  static constexpr int PITCH = KMAJOR ? ROWS + G_KPAD : G_PK;
+  static constexpr int ELEMS = KMAJOR ? G_BK * (ROWS + G_KPAD) : ROWS * G_PK;
+  static constexpr int CHUNKS = ROWS * G_BK / 8 / NT;       // 16-byte chunks per thread and k-tile
 };
 
 // per-thread byte offsets of this thread's chunks relative to (operand base + k-tile start)
-template <int ROWS, bool KMAJOR>
-__device__ __forceinline__ void g_offsets(int64_t ld, int row0, int rows, uint32_t (&off)[TileGeom<ROWS, KMAJOR>::CHUNKS]) {
+template <int ROWS, bool KMAJOR, int NT>
+__device__ __forceinline__ void g_offsets(int64_t ld, int row0, int rows, uint32_t (&off)[TileGeom<ROWS, KMAJOR, NT>::CHUNKS]) {
   int t = threadIdx.x;
 #pragma unroll
-  for (int i = 0; i < TileGeom<ROWS, KMAJOR>::CHUNKS; i++) {
-    int c = t + 256 * i;
+  for (int i = 0; i < TileGeom<ROWS, KMAJOR, NT>::CHUNKS; i++) {
+    int c = t + NT * i;
     if (!KMAJOR) {
       int r = min(row0 + (c >> 3), rows - 1);
       off[i] = (uint32_t)(((int64_t)r * ld + (c & 7) * 8) * 2);
@@ -47,14 +48,14 @@ __device__ __forceinline__ void g_load(const char *__restrict__ base, const uint
 #pragma unroll
   for (int i = 0; i < N; i++) v[i] = *reinterpret_cast<const u32x4 *>(base + off[i]);
 }
-template <int ROWS, bool KMAJOR>
-__device__ __forceinline__ void g_store(uint16_t *s, const u32x4 (&v)[TileGeom<ROWS, KMAJOR>::CHUNKS]) {
+template <int ROWS, bool KMAJOR, int NT>
+__device__ __forceinline__ void g_store(uint16_t *s, const u32x4 (&v)[TileGeom<ROWS, KMAJOR, NT>::CHUNKS]) {
   int t = threadIdx.x;
 #pragma unroll
-  for (int i = 0; i < TileGeom<ROWS, KMAJOR>::CHUNKS; i++) {
-    int c = t + 256 * i;
+  for (int i = 0; i < TileGeom<ROWS, KMAJOR, NT>::CHUNKS; i++) {
+    int c = t + NT * i;
     if (!KMAJOR) *reinterpret_cast<u32x4 *>(s + (c >> 3) * G_PK + (c & 7) * 8) = v[i];
-    else *reinterpret_cast<u32x4 *>(s + (c / (ROWS / 8)) * (ROWS + 16) + (c % (ROWS / 8)) * 8) = v[i];
+    else *reinterpret_cast<u32x4 *>(s + (c / (ROWS / 8)) * (ROWS + G_KPAD) + (c % (ROWS / 8)) * 8) = v[i];
   }
 }
 // LDS element offset of this lane's fragment for tile rows [r0, r0+32), k-slice 0 (add kk * KSTEP per slice)
@@ -62,7 +63,7 @@ template <int ROWS, bool KMAJOR>
 __device__ __forceinline__ int g_frag_base(int r0, int lane) {
   if (!KMAJOR) return (r0 + (lane & 31)) * G_PK + (lane >> 5) * 8;
   int j = lane & 15, g = lane >> 4;                  // 16-lane group g: rows r0 + 16*(g&1).., k half g>>1
-  return ((g >> 1) * 8 + (j >> 2)) * (ROWS + 16) + r0 + (g & 1) * 16 + (j & 3) * 4;
+  return ((g >> 1) * 8 + (j >> 2)) * (ROWS + G_KPAD) + r0 + (g & 1) * 16 + (j & 3) * 4;
 }
 template <int ROWS, bool KMAJOR>
 __device__ __forceinline__ bf16x8 g_frag(const uint16_t *s, int base, int kk) {
@@ -70,9 +71,9 @@ __device__ __forceinline__ bf16x8 g_frag(const uint16_t *s, int base, int kk) {
     return *reinterpret_cast<const bf16x8 *>(s + base + kk * 16);
   } else {
     typedef __attribute__((address_space(3))) bf16x4 lds_v4;
-    const uint16_t *p = s + base + kk * 16 * (ROWS + 16);
+    const uint16_t *p = s + base + kk * 16 * (ROWS + G_KPAD);
     bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_v4 *)p);
-    bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_v4 *)(p + 4 * (ROWS + 16)));
+    bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_v4 *)(p + 4 * (ROWS + G_KPAD)));
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
   }
 }
@@ -109,13 +110,11 @@ __global__ void k_splitk_reduce(const float *__restrict__ ws, float *__restrict_
   }
 }
 
-// PF = register sets of prefetched k-tiles (1: loads of tile t+1 fly during the MFMAs of tile t; 2: two tiles ahead).
-// The shipped configuration is 128x128, PF = 1, three blocks per CU hiding each other's latency.
-template <int BM, int BN, bool AKM, bool BKM, int PF>
-__global__ __launch_bounds__(256) void k_gemm_bf16(GemmArgs g, int out_f32) {
-  constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
-  typedef TileGeom<BM, AKM> GA;
-  typedef TileGeom<BN, BKM> GB;
+template <int BM, int BN, int WGM, int WGN, bool AKM, bool BKM>
+__global__ __launch_bounds__(64 * WGM * WGN) void k_gemm_bf16(GemmArgs g, int out_f32) {
+  constexpr int NT = 64 * WGM * WGN, WM = BM / WGM, WN = BN / WGN, TM = WM / 32, TN = WN / 32;
+  typedef TileGeom<BM, AKM, NT> GA;
+  typedef TileGeom<BN, BKM, NT> GB;
   extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
   uint16_t *As = smem;                       // [2][GA::ELEMS]
   uint16_t *Bs = smem + 2 * GA::ELEMS;       // [2][GB::ELEMS]
@@ -129,14 +128,14 @@ __global__ __launch_bounds__(256) void k_gemm_bf16(GemmArgs g, int out_f32) {
   int tiles_m = (g.M + BM - 1) / BM;
   int m0 = (blockIdx.x % tiles_m) * BM, n0 = (blockIdx.x / tiles_m) * BN;
   int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  int wm = (wave >> 1) * WM, wn = (wave & 1) * WN;
+  int wm = (wave / WGN) * WM, wn = (wave % WGN) * WN;
   // bytes to advance per k-tile: 64 elements along a k-contiguous row, 64 rows of a k-major operand
   const int64_t a_step = AKM ? (int64_t)G_BK * g.lda * 2 : (int64_t)G_BK * 2;
   const int64_t b_step = BKM ? (int64_t)G_BK * g.ldb * 2 : (int64_t)G_BK * 2;
 
   uint32_t offa[GA::CHUNKS], offb[GB::CHUNKS];
-  g_offsets<BM, AKM>(g.lda, m0, g.M, offa);
-  g_offsets<BN, BKM>(g.ldb, n0, g.N, offb);
+  g_offsets<BM, AKM, NT>(g.lda, m0, g.M, offa);
+  g_offsets<BN, BKM, NT>(g.ldb, n0, g.N, offb);
   int fa_base[TM], fb_base[TN];
 #pragma unroll
   for (int i = 0; i < TM; i++) fa_base[i] = g_frag_base<BM, AKM>(wm + 32 * i, lane);
@@ -151,60 +150,66 @@ __global__ __launch_bounds__(256) void k_gemm_bf16(GemmArgs g, int out_f32) {
 #pragma unroll
       for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
 
-  // register sets for the k-tiles in flight (named, never indexed dynamically, so they stay in VGPRs)
-  u32x4 ra0[GA::CHUNKS], rb0[GB::CHUNKS], ra1[GA::CHUNKS], rb1[GB::CHUNKS];
-  int nt = g.ksplit / G_BK;
+  // Staging registers for the one k-tile in flight between global memory and LDS.
+  u32x4 ra[GA::CHUNKS], rb[GB::CHUNKS];
+  const int nt = g.ksplit / G_BK, last = nt - 1;
+  bf16x8 fa[2][TM], fb[2][TN];       // fragments of the current and the next k-slice
 
-  auto compute = [&](int buf) {
+  auto read_frags = [&](int buf, int kk, int set) {
     const uint16_t *as = As + buf * GA::ELEMS, *bs = Bs + buf * GB::ELEMS;
 #pragma unroll
-    for (int kk = 0; kk < G_BK / 16; kk++) {
-      bf16x8 fa[TM], fb[TN];
+    for (int i = 0; i < TM; i++) fa[set][i] = g_frag<BM, AKM>(as, fa_base[i], kk);
 #pragma unroll
-      for (int i = 0; i < TM; i++) fa[i] = g_frag<BM, AKM>(as, fa_base[i], kk);
+    for (int j = 0; j < TN; j++) fb[set][j] = g_frag<BN, BKM>(bs, fb_base[j], kk);
+  };
+  auto mfma_slice = [&](int set) {
 #pragma unroll
-      for (int j = 0; j < TN; j++) fb[j] = g_frag<BN, BKM>(bs, fb_base[j], kk);
+    for (int i = 0; i < TM; i++)
 #pragma unroll
-      for (int i = 0; i < TM; i++)
-#pragma unroll
-        for (int j = 0; j < TN; j++)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[j], fa[i], acc[i][j], 0, 0, 0);   // operands swapped: C^T tile
-      if (BM * BN > 128 * 128) __builtin_amdgcn_sched_barrier(0);   // big tile: keep only one k-slice of fragments live
-    }
+      for (int j = 0; j < TN; j++)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[set][j], fa[set][i], acc[i][j], 0, 0, 0);   // operands swapped: C^T tile
+  };
+  // One k-tile (4 slices of 16).  Entering, LDS buffer `buf` holds tile t, fragment set 0 holds its slice 0, and the
+  // staging registers hold (or are receiving) tile t + 1.  The fragments of slice kk + 1 are read while the MFMAs of
+  // slice kk issue.  After slice 1 the staged tile goes to the other LDS buffer (free since the barrier that ended
+  // tile t - 1) and the loads of tile t + 2 start, so a load has a whole tile of MFMA work to land.  The barrier sits
+  // before the last slice: its MFMAs cover the LDS latency of the next tile's first fragments.  Tiles past the last
+  // are clamped onto it (loaded and stored, never consumed), which keeps the steady state branch-free.
+  auto tile = [&](int buf, int t) {
+    read_frags(buf, 1, 1);
+    mfma_slice(0);
+    __builtin_amdgcn_sched_barrier(0);
+    read_frags(buf, 2, 0);
+    mfma_slice(1);
+    __builtin_amdgcn_sched_barrier(0);
+    g_store<BM, AKM, NT>(As + (buf ^ 1) * GA::ELEMS, ra);
+    g_store<BN, BKM, NT>(Bs + (buf ^ 1) * GB::ELEMS, rb);
+    g_load(A + min(t + 2, last) * a_step, offa, ra);
+    g_load(B + min(t + 2, last) * b_step, offb, rb);
+    __builtin_amdgcn_sched_barrier(0);
+    read_frags(buf, 3, 1);
+    mfma_slice(0);
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();
+    read_frags(buf ^ 1, 0, 0);
+    mfma_slice(1);
+    __builtin_amdgcn_sched_barrier(0);
   };
 
-  // Steady state is branch-free: prefetches past the last k-tile are clamped onto it (loaded, never consumed).
-  const int last = nt - 1;
-  g_load(A, offa, ra0);
-  g_load(B, offb, rb0);
-  if (PF == 2) {
-    g_load(A + min(1, last) * a_step, offa, ra1);
-    g_load(B + min(1, last) * b_step, offb, rb1);
-  }
-  g_store<BM, AKM>(As, ra0);
-  g_store<BN, BKM>(Bs, rb0);
+  g_load(A, offa, ra);
+  g_load(B, offb, rb);
+  g_store<BM, AKM, NT>(As, ra);
+  g_store<BN, BKM, NT>(Bs, rb);
+  g_load(A + min(1, last) * a_step, offa, ra);
+  g_load(B + min(1, last) * b_step, offb, rb);
   __syncthreads();
-  // Tile t is computed from LDS buffer t%2.  While it is computed, the loads of tile t+PF are issued into the
-  // register set tile t just left, and tile t+1 moves from its registers into the other LDS buffer; with PF = 2 a
-  // load therefore has two full tiles of MFMA work to land before it is stored.
+  read_frags(0, 0, 0);
   int t = 0;
   for (; t + 2 <= nt; t += 2) {
-    // ---- even tile (LDS buffer 0)
-    g_load(A + min(t + PF, last) * a_step, offa, ra0);
-    g_load(B + min(t + PF, last) * b_step, offb, rb0);
-    compute(0);
-    if (PF == 2) { g_store<BM, AKM>(As + GA::ELEMS, ra1); g_store<BN, BKM>(Bs + GB::ELEMS, rb1); }
-    else { g_store<BM, AKM>(As + GA::ELEMS, ra0); g_store<BN, BKM>(Bs + GB::ELEMS, rb0); }
-    __syncthreads();
-    // ---- odd tile (LDS buffer 1)
-    if (PF == 2) { g_load(A + min(t + 3, last) * a_step, offa, ra1); g_load(B + min(t + 3, last) * b_step, offb, rb1); }
-    else { g_load(A + min(t + 2, last) * a_step, offa, ra0); g_load(B + min(t + 2, last) * b_step, offb, rb0); }
-    compute(1);
-    g_store<BM, AKM>(As, ra0);
-    g_store<BN, BKM>(Bs, rb0);
-    __syncthreads();
+    tile(0, t);
+    tile(1, t + 1);
   }
-  if (t < nt) compute(0);        // odd tile count: the last tile is waiting in buffer 0
+  if (t < nt) tile(0, t);
   int r0 = m0 + wm, c0 = n0 + wn;
   if (g.nsplit > 1) {     // g.c is the split-K workspace [nsplit][M][N] here
     store_tiles<AH_EPI_NONE, float, TM, TN>(g, (int64_t)blockIdx.y * g.M * g.N, r0, c0, lane, acc);
@@ -222,26 +227,30 @@ __global__ __launch_bounds__(256) void k_gemm_bf16(GemmArgs g, int out_f32) {
   }
 }
 
-template <int BM, int BN, bool AKM, bool BKM, int PF>
+template <int BM, int BN, int WGM, int WGN, bool AKM, bool BKM>
 int32_t launch(const GemmArgs &ga, int batch, int out_dtype) {
-  size_t lds = sizeof(uint16_t) * 2 * (size_t)(TileGeom<BM, AKM>::ELEMS + TileGeom<BN, BKM>::ELEMS);
+  constexpr int NT = 64 * WGM * WGN;
+  size_t lds = sizeof(uint16_t) * 2 * (size_t)(TileGeom<BM, AKM, NT>::ELEMS + TileGeom<BN, BKM, NT>::ELEMS);
   int64_t tiles = cdiv(ga.M, BM) * cdiv(ga.N, BN);
   dim3 grid((unsigned)tiles, (unsigned)ga.nsplit, (unsigned)batch);
-  auto kfn = k_gemm_bf16<BM, BN, AKM, BKM, PF>;
+  auto kfn = k_gemm_bf16<BM, BN, WGM, WGN, AKM, BKM>;
   if (lds > 64 * 1024) {
     static bool raised = false;      // per instantiation: the attribute only needs setting once
     if (!raised) { AH_HIP(hipFuncSetAttribute((const void *)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); raised = true; }
   }
-  hipLaunchKernelGGL(kfn, grid, dim3(256), lds, stream(), ga, out_dtype == AH_F32 ? 1 : 0);
+  hipLaunchKernelGGL(kfn, grid, dim3(NT), lds, stream(), ga, out_dtype == AH_F32 ? 1 : 0);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
 
 template <bool AKM, bool BKM>
 int32_t run(const GemmArgs &ga, int batch, int out_dtype) {
-  // 128x128 tiles at 3 blocks per CU: measured faster on MI355X than a 256x256 tile at one wave per SIMD, whose
-  // 256 accumulator + ~250 working registers the compiler cannot allocate without spilling into the k-loop.
-  return launch<128, 128, AKM, BKM, 1>(ga, batch, out_dtype);
+  // 256x256 tile on 8 waves (2 x 4, each 128 x 64): half the L2 traffic per flop of the 128x128 tile, two waves per
+  // SIMD to overlap each other's loads.  Used when it still fills the chip; otherwise 128x128 at 3 blocks per CU.
+  int64_t big_blocks = cdiv(ga.M, 256) * cdiv(ga.N, 256) * batch * ga.nsplit;
+  bool big = ga.M >= 256 && ga.N >= 256 && big_blocks >= num_cus();
+  if (big) return launch<256, 256, 2, 4, AKM, BKM>(ga, batch, out_dtype);
+  return launch<128, 128, 2, 2, AKM, BKM>(ga, batch, out_dtype);
 }
 
 }  // namespace
