@@ -88,12 +88,14 @@ SIGNATURES = {
     "ah_embedding": [u64, u64, u64, i64, i64, i64, i32],
     "ah_embedding_tok_pos": [u64, u64, u64, u64, i64, i64, i64, i64],
     "ah_embedding_bwd": [u64, u64, u64, i64, i64, i64, i32],
+    "ah_token_windows": [u64, i64, u64, i64, i64, u64, u64],
     "ah_pos_embedding_bwd": [u64, u64, i64, i64, i64, i32],
     "ah_layernorm": [u64, u64, u64, u64, i64, i64, f32, i32],
     "ah_layernorm_bwd": [u64, u64, u64, i32, u64, u64, u64, u64, u64, i64, i64, f32, i32],
     "ah_cross_entropy": [u64, i32, u64, u64, u64, i64, i64],
     "ah_cross_entropy_bwd": [u64, i32, u64, u64, u64, f32, u64, i64, i64],
     "ah_gemm": [C.POINTER(AhGemm)],
+    "ah_gemm_last_kernel": [C.c_char_p, C.c_int32, C.POINTER(C.c_int32)],
     "ah_flash_fwd": [C.POINTER(AhFlash)], "ah_flash_bwd": [C.POINTER(AhFlash)],
     "ah_adamw": [u64, u64, u64, u64, u64, C.POINTER(AhAdamW), u64, u64, u64],
     "ah_clip_coef": [u64, f32, f32, u64],

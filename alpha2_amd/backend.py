@@ -280,8 +280,15 @@ class HipBackend:
         check(self.lib.ah_event_record(e0))
         check(self.lib.ah_gemm(C.byref(g)))
         check(self.lib.ah_event_record(e1))
-        timed.append({"kind": "gemm", "layout": layout, "dtype": in_dtype, "m": m, "n": n, "k": k, "batch": batch,
-                      "flops": 2.0 * m * n * k * batch, "e0": e0, "e1": e1})
+        kernel, nsplit = self.lastGemmKernel()
+        timed.append({"kind": "gemm", "kernel": kernel, "nsplit": nsplit, "layout": layout, "dtype": in_dtype, "m": m, "n": n, "k": k,
+                      "batch": batch, "flops": 2.0 * m * n * k * batch, "e0": e0, "e1": e1})
+
+    def lastGemmKernel(self):
+        """(name, split-K slices) of the kernel the last ah_gemm call launched, named as a profiler prints it."""
+        buf, ns = C.create_string_buffer(128), C.c_int32(1)
+        check(self.lib.ah_gemm_last_kernel(buf, 128, C.byref(ns)))
+        return buf.value.decode(), ns.value
 
     def _event(self) -> int:
         ev = C.c_uint64()

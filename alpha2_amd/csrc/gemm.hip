@@ -5,7 +5,8 @@
 // TN: dW = G^T X).  Epilogues fuse GELU (+ saved pre-activation), the residual add, gradient
 // accumulation and the GELU derivative.
 #include "gemm_common.h"
-#include <cstdlib>
+#include <cstdarg>
+#include <cstdio>
 
 using namespace ah;
 
@@ -249,6 +250,8 @@ int32_t launch_bf16_nt_t(const GemmArgs &ga, int batch, int vec_c) {
     static bool raised = false;      // per instantiation: the attribute only needs setting once
     if (!raised) { AH_HIP(hipFuncSetAttribute((const void *)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); raised = true; }
   }
+  note_gemm_kernel("k_gemm_bf16_nt<%d, %d, %d, %d, %d, %s>", BM, BN, WGM, WGN, EPI, sizeof(OUT) == 4 ? "float" : "unsigned short");
+  note_gemm_split(1);
   hipLaunchKernelGGL(kfn, grid, dim3(256), lds, stream(), ga, vec_c);
   AH_LAUNCH_CHECK();
   return AH_OK;
@@ -269,6 +272,8 @@ int32_t run_bf16_nt(const GemmArgs &ga, int batch, int out_dtype, int vec_c) {
 template <int LAYOUT, int EPI, class OUT>
 int32_t launch_f32_t(const GemmArgs &ga, int batch, int vec_a, int vec_b, int vec_c) {
   dim3 grid((unsigned)cdiv(ga.N, F_BN), (unsigned)cdiv(ga.M, F_BM), (unsigned)batch);
+  note_gemm_kernel("k_gemm_f32<%d, %d, %s>", LAYOUT, EPI, sizeof(OUT) == 4 ? "float" : "unsigned short");
+  note_gemm_split(1);
   hipLaunchKernelGGL((k_gemm_f32<LAYOUT, EPI, OUT>), grid, dim3(256), 0, stream(), ga, vec_a, vec_b, vec_c);
   AH_LAUNCH_CHECK();
   return AH_OK;
@@ -287,7 +292,26 @@ int32_t launch_f32(const GemmArgs &ga, int batch, int out_dtype, int vec_a, int 
 
 }  // namespace
 
+namespace ah {
+static char g_last_kernel[96] = "";
+static int g_last_split = 1;
+void note_gemm_kernel(const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_last_kernel, sizeof(g_last_kernel), fmt, ap);
+  va_end(ap);
+}
+void note_gemm_split(int nsplit) { g_last_split = nsplit; }
+}  // namespace ah
+
 extern "C" {
+
+int32_t ah_gemm_last_kernel(char *name, int32_t capacity, int32_t *nsplit) {
+  AH_ARG(name != nullptr && capacity > 0, "ah_gemm_last_kernel: no output buffer");
+  snprintf(name, (size_t)capacity, "%s", g_last_kernel);
+  if (nsplit) *nsplit = g_last_split;
+  return AH_OK;
+}
 
 int32_t ah_gemm(const AhGemm *p) {
   AH_REQUIRE_READY();

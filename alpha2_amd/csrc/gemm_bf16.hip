@@ -238,6 +238,8 @@ int32_t launch(const GemmArgs &ga, int batch, int out_dtype) {
     static bool raised = false;      // per instantiation: the attribute only needs setting once
     if (!raised) { AH_HIP(hipFuncSetAttribute((const void *)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); raised = true; }
   }
+  note_gemm_kernel("k_gemm_bf16<%d, %d, %d, %d, %s, %s>", BM, BN, WGM, WGN, AKM ? "true" : "false", BKM ? "true" : "false");
+  note_gemm_split(ga.nsplit);
   hipLaunchKernelGGL(kfn, grid, dim3(NT), lds, stream(), ga, out_dtype == AH_F32 ? 1 : 0);
   AH_LAUNCH_CHECK();
   return AH_OK;

@@ -4,6 +4,10 @@
 
 namespace ah {
 
+// Records which kernel ah_gemm launched last (read back by ah_gemm_last_kernel).
+void note_gemm_kernel(const char *fmt, ...);
+void note_gemm_split(int nsplit);
+
 struct GemmArgs {
   const void *a, *b;
   void *c;

@@ -357,6 +357,18 @@ __global__ void k_ce_bwd(const T *__restrict__ logits, const int32_t *__restrict
   }
 }
 
+// Token windows of a device-resident corpus: one block row per batch item, modulo indexing reproduces the packed
+// loader's wrap-around (and is a no-op for random windows, which never reach the end of the corpus).
+__global__ void k_token_windows(const int32_t *__restrict__ corpus, int64_t n_tokens, const int64_t *__restrict__ starts, int64_t T,
+                                int32_t *__restrict__ inputs, int32_t *__restrict__ targets) {
+  int64_t b = blockIdx.y, start = starts[b];
+  for (int64_t t = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; t < T; t += (int64_t)gridDim.x * blockDim.x) {
+    int64_t p = (start + t) % n_tokens, q = p + 1 == n_tokens ? 0 : p + 1;
+    inputs[b * T + t] = corpus[p];
+    targets[b * T + t] = corpus[q];
+  }
+}
+
 }  // namespace
 
 template <class OUT>
@@ -402,6 +414,19 @@ int32_t ah_embedding_tok_pos(ah_ptr wte, ah_ptr wpe, ah_ptr tok, ah_ptr out, int
   AH_ARG(aligned16(wte) && aligned16(wpe) && aligned16(out), "ah_embedding_tok_pos: operands must be 16-byte aligned");
   hipLaunchKernelGGL(k_embedding_tok_pos, dim3((unsigned)cdiv(n_idx, WPB)), dim3(TPB), 0, stream(), dp<const float>(wte),
                      dp<const float>(wpe), dp<const int32_t>(tok), dp<float>(out), n_idx, T, dim, vocab);
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+
+int32_t ah_token_windows(ah_ptr corpus, int64_t n_tokens, ah_ptr starts, int64_t batch, int64_t T, ah_ptr inputs, ah_ptr targets) {
+  AH_REQUIRE_READY();
+  AH_ARG(batch >= 0 && T >= 0 && batch <= 65535, "ah_token_windows: bad batch %lld / block %lld", (long long)batch, (long long)T);
+  if (batch == 0 || T == 0) return AH_OK;
+  AH_ARG(n_tokens > 0, "ah_token_windows: empty corpus");
+  AH_ARG(corpus && starts && inputs && targets, "ah_token_windows: null operand");
+  unsigned bx = (unsigned)(cdiv(T, 256) < 64 ? cdiv(T, 256) : 64);
+  hipLaunchKernelGGL(k_token_windows, dim3(bx, (unsigned)batch), dim3(256), 0, stream(), dp<const int32_t>(corpus), n_tokens,
+                     dp<const int64_t>(starts), T, dp<int32_t>(inputs), dp<int32_t>(targets));
   AH_LAUNCH_CHECK();
   return AH_OK;
 }

@@ -135,7 +135,9 @@ class FusedTrainer:
         check(self.lib.ah_event_record(e0))
         check(self.lib.ah_gemm(C.byref(g)))
         check(self.lib.ah_event_record(e1))
-        self._timed.append({"kind": "gemm", "layout": layout, "m": m, "n": n, "k": k, "flops": 2.0 * m * n * k, "e0": e0, "e1": e1})
+        kernel, nsplit = self.B.lastGemmKernel()
+        self._timed.append({"kind": "gemm", "kernel": kernel, "nsplit": nsplit, "layout": layout, "m": m, "n": n, "k": k,
+                            "flops": 2.0 * m * n * k, "e0": e0, "e1": e1})
 
     def _flash(self, l: int, bwd: bool):
         Cc, T, D = self.C, self.T, self.D

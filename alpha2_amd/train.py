@@ -11,7 +11,8 @@ from typing import Dict, List, Optional, Sequence, Tuple
 import numpy as np
 
 from .autograd import DropoutRng, Tape, Variable
-from .backend import TensorData, shapeSize
+from ._ffi import check
+from .backend import HipBackend, TensorData, shapeSize
 from .model import ModelConfig, collectParamEntries, gptForward, initGPT
 
 
@@ -137,6 +138,49 @@ def zipfBatch(seed: int, Bt: int, T: int, vocab: int, s: float = 1.1) -> Tuple[T
     u = SeededRng(seed).fillUniform(Bt * (T + 1))
     ids = np.minimum(np.searchsorted(cdf, u, side="right"), vocab - 1).astype(np.int32).reshape(Bt, T + 1)
     return TensorData((Bt, T), "i32", ids[:, :T]), TensorData((Bt, T), "i32", ids[:, 1:])
+
+
+class DataLoader:
+    """DataLoader of packages/train/src/data.ts:19-175 with the corpus resident in HBM: the token array is uploaded
+    once, a batch is one `ah_token_windows` launch given B window starts.  Random mode draws
+    start = floor(rng.next() * (N - T)) per row (data.ts:104-114); packed mode keeps B cursors b*floor(N/B) that advance
+    T per batch and wrap at the end of the corpus (data.ts:131-167).  Batches come from a ring of two buffer pairs,
+    like the reference's, so a batch stays valid until the call after next."""
+
+    def __init__(self, B: HipBackend, tokens, rng, batchSize: int, blockSize: int, packed: bool = False):
+        self.B, self.rng, self.batchSize, self.blockSize, self.packed = B, rng, int(batchSize), int(blockSize), bool(packed)
+        tok = np.ascontiguousarray(tokens, dtype=np.int32).reshape(-1)
+        self.length = int(tok.size)
+        self._corpus = TensorData((max(1, self.length),), "i32", tok if self.length else np.zeros(1, np.int32))
+        B._ptr(self._corpus)
+        self.cursors = [b * (self.length // self.batchSize) for b in range(self.batchSize)] if packed else None
+        self._ring = [(B._new((self.batchSize, self.blockSize), "i32"), B._new((self.batchSize, self.blockSize), "i32")) for _ in range(2)]
+        self._ringIdx = 0
+
+    @property
+    def stepsPerEpoch(self) -> int:
+        return self.length // (self.batchSize * self.blockSize)
+
+    def nextBatch(self) -> Tuple[TensorData, TensorData]:
+        Bt, T, N = self.batchSize, self.blockSize, self.length
+        if self.packed:
+            if N == 0:
+                raise IndexError("packed DataLoader over an empty corpus")
+            starts = list(self.cursors)
+            self.cursors = [(c + T) % N for c in self.cursors]
+        else:
+            if N <= T:
+                raise IndexError(f"Token count ({N}) must exceed block size ({T}) — need at least {T + 1} tokens for input+target windows")
+            maxStart = N - T
+            starts = [int(math.floor(self.rng.next() * maxStart)) for _ in range(Bt)]
+        inputs, targets = self._ring[self._ringIdx]
+        self._ringIdx = (self._ringIdx + 1) % len(self._ring)
+        st = TensorData((Bt,), "f64", np.asarray(starts, dtype=np.int64).view(np.float64))     # 8-byte slots holding the int64 starts
+        B = self.B
+        check(B.lib.ah_token_windows(B._ptr(self._corpus), N, B._ptr(st), Bt, T, B._ptr(inputs), B._ptr(targets)))
+        B.releaseGpuTensor(st)
+        B._dirty(inputs), B._dirty(targets)
+        return inputs, targets
 
 
 @dataclass

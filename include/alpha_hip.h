@@ -175,6 +175,12 @@ int32_t ah_embedding_bwd(ah_ptr idx_i32, ah_ptr grad_out, ah_ptr grad_w, int64_t
 /* grad_wpe[T,dim] (+)= sum over the batch of grad_out[b,t,:]  (positions are 0..T-1 per row) */
 int32_t ah_pos_embedding_bwd(ah_ptr grad_out, ah_ptr grad_wpe, int64_t batch, int64_t T, int64_t dim,
                              int32_t accumulate);
+/* Batch assembly of DataLoader.nextBatch (packages/train/src/data.ts:94-167) from a corpus resident on the device:
+ *   inputs[b,t] = corpus[(start[b] + t) mod n_tokens],  targets[b,t] = corpus[(start[b] + t + 1) mod n_tokens].
+ * Random mode never wraps (start < n_tokens - T); packed mode wraps exactly as the reference's cursor loop does
+ * (the target of the corpus' last token is its first).  corpus, inputs, targets: i32; starts: i64[batch] on the device. */
+int32_t ah_token_windows(ah_ptr corpus_i32, int64_t n_tokens, ah_ptr starts_i64, int64_t batch, int64_t T,
+                         ah_ptr inputs_i32, ah_ptr targets_i32);
 int32_t ah_layernorm(ah_ptr x, ah_ptr w, ah_ptr b, ah_ptr out, int64_t rows, int64_t dim, float eps,
                      int32_t out_dtype);
 /* dx (+= residual_grad when that handle is non-zero), dw, db.  dw/db are deterministic column sums;
@@ -218,6 +224,10 @@ typedef struct {
   ah_ptr  a, b, c, aux;
 } AhGemm;
 int32_t ah_gemm(const AhGemm *g);
+/* Profiling aid (no counterpart in the reference): writes the name of the kernel the most recent ah_gemm call
+ * launched, spelled as a profiler demangles it (e.g. "k_gemm_bf16<256, 256, 2, 4, false, false>"), and the number
+ * of split-K slices it used (1 = none; > 1 means a k_splitk_reduce launch followed). */
+int32_t ah_gemm_last_kernel(char *name, int32_t capacity, int32_t *nsplit);
 
 /* ---- fused causal flash attention.  Backend.flashAttention / flashAttentionBackward
  *      (interfaces.ts:127-135; kernel semantics packages/helios/src/kernels/attention.ts:1-586):

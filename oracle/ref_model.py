@@ -604,3 +604,45 @@ def synthetic_batch(seed: int, Bt: int, T: int, vocab: int) -> Tuple[TD, TD]:
     ids = np.floor(u * vocab).astype(np.int32).reshape(Bt, T + 1)
     return (TD((Bt, T), "i32", np.ascontiguousarray(ids[:, :T]).reshape(-1)),
             TD((Bt, T), "i32", np.ascontiguousarray(ids[:, 1:]).reshape(-1)))
+
+
+class DataLoader:
+    """Batch sampler of packages/train/src/data.ts:30-167, slice by slice as written there.
+    Random mode (data.ts:94-120): per batch row, start = floor(rng.next() * (N - T)); inputs = tokens[start, start+T),
+    targets = tokens[start+1, start+T+1).  Packed mode (data.ts:131-167): cursor b starts at b*floor(N/B) and advances
+    T per batch; a window that reaches the end of the corpus continues at token 0, and the target of the corpus'
+    last token is its first."""
+
+    def __init__(self, tokens, rng: SeededRng, batchSize: int, blockSize: int, packed: bool = False):
+        self.tokens = np.ascontiguousarray(tokens, dtype=np.int32)
+        self.rng, self.batchSize, self.blockSize, self.packed = rng, batchSize, blockSize, packed
+        self.cursors = [b * (len(self.tokens) // batchSize) for b in range(batchSize)] if packed else None
+
+    def next_batch(self) -> Tuple[TD, TD]:
+        Bt, T, tok, N = self.batchSize, self.blockSize, self.tokens, len(self.tokens)
+        inputs, targets = np.zeros(Bt * T, np.int32), np.zeros(Bt * T, np.int32)
+        if not self.packed:
+            if N <= T:
+                raise IndexError(f"Token count ({N}) must exceed block size ({T})")
+            max_start = N - T
+            for b in range(Bt):
+                start = int(math.floor(self.rng.next() * max_start))
+                inputs[b * T:(b + 1) * T] = tok[start:start + T]
+                targets[b * T:(b + 1) * T] = tok[start + 1:start + T + 1]
+        else:
+            for b in range(Bt):
+                pos, remaining, dst = self.cursors[b], T, b * T
+                while remaining > 0:
+                    span = min(remaining, N - pos)
+                    inputs[dst:dst + span] = tok[pos:pos + span]
+                    if pos + span < N:
+                        targets[dst:dst + span] = tok[pos + 1:pos + span + 1]
+                    else:
+                        if span > 1:
+                            targets[dst:dst + span - 1] = tok[pos + 1:N]
+                        targets[dst + span - 1] = tok[0]
+                    dst, remaining, pos = dst + span, remaining - span, pos + span
+                    if pos == N:
+                        pos = 0
+                self.cursors[b] = pos
+        return TD((Bt, T), "i32", inputs), TD((Bt, T), "i32", targets)

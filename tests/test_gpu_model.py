@@ -157,3 +157,32 @@ def test_reference_flash_layout_is_exposed_and_differs(B):
         inp, tgt = syntheticBatch(8, 2, 16, 50)
         losses[mode] = float(gptForward(cfg, params, B, Tape(), inp, tgt, True)["loss"].data.data[0])
     assert math.isfinite(losses["reference-flash"]) and abs(losses["heads"] - losses["reference-flash"]) > 1e-6
+
+
+@pytest.mark.parametrize("N,Bt,T,packed", [(5000, 8, 128, False), (129, 2, 128, False), (1000, 4, 64, True), (10, 3, 7, True),
+                                            (5, 2, 12, True), (70000, 16, 1024, False)])
+def test_dataloader_batches_are_bit_exact(B, N, Bt, T, packed):
+    """Device-assembled batches equal the oracle's slice-by-slice loader, batch after batch (integer data: bit-exact)."""
+    from alpha2_amd.rng import SeededRng
+    from alpha2_amd.train import DataLoader
+    tok = (np.arange(N, dtype=np.int64) * 7919 % 50304).astype(np.int32)
+    dev = DataLoader(B, tok, SeededRng(5), Bt, T, packed)
+    orc = rm.DataLoader(tok, ref.SeededRng(5), Bt, T, packed)
+    held = []
+    for i in range(5):
+        x, y = dev.nextBatch()
+        xo, yo = orc.next_batch()
+        assert x.shape == (Bt, T) and x.dtype == "i32"
+        assert np.array_equal(x.data, xo.data) and np.array_equal(y.data, yo.data), i
+        held.append((x, xo.data.copy()))
+        if len(held) >= 2:        # the ring keeps the previous batch valid for one more call
+            px, pxo = held[-2]
+            assert np.array_equal(px.data, pxo)
+    assert dev.stepsPerEpoch == N // (Bt * T)
+
+
+def test_dataloader_rejects_a_corpus_not_longer_than_the_block(B):
+    from alpha2_amd.rng import SeededRng
+    from alpha2_amd.train import DataLoader
+    with pytest.raises(IndexError, match="must exceed block size"):
+        DataLoader(B, np.arange(16, dtype=np.int32), SeededRng(0), 2, 16).nextBatch()

@@ -4,6 +4,7 @@ autograd of the same network, and closed forms.  No GPU."""
 import math
 
 import numpy as np
+import pytest
 import torch
 import torch.nn.functional as F
 
@@ -190,3 +191,50 @@ def test_grad_accumulation_scales_by_one_over_k():
     assert abs(r.loss - (l1 + l2) / 2) < 1e-6              # gpu-perf.test.ts:303-321: sum(loss_i)/K
     sq = sum(ref.sum_sq(v.grad) for _, v in tr1.entries)
     assert abs(r.gradNorm - math.sqrt(sq) * 0.5) < 1e-9
+
+
+# ---------------------------------------------------------------------------------------------- DataLoader (data.ts:94-167)
+def _naive_windows(tok, starts, T):
+    """Element-by-element definition: inputs[b,t] = tok[(s+t) % N], targets[b,t] = tok[(s+t+1) % N]."""
+    N = len(tok)
+    inp = np.array([[tok[(s + t) % N] for t in range(T)] for s in starts], np.int32)
+    tgt = np.array([[tok[(s + t + 1) % N] for t in range(T)] for s in starts], np.int32)
+    return inp, tgt
+
+
+def test_dataloader_random_windows_follow_the_rng_stream():
+    tok = (np.arange(1000) * 7919 % 503).astype(np.int32)
+    dl = rm.DataLoader(tok, ref.SeededRng(11), 4, 16)
+    probe = ref.SeededRng(11)
+    for _ in range(3):
+        x, y = dl.next_batch()
+        starts = [int(np.floor(probe.next() * (1000 - 16))) for _ in range(4)]      # data.ts:105,111
+        assert all(0 <= s < 1000 - 16 for s in starts)
+        inp, tgt = _naive_windows(tok, starts, 16)
+        assert np.array_equal(x.data.reshape(4, 16), inp) and np.array_equal(y.data.reshape(4, 16), tgt)
+        assert np.array_equal(x.data.reshape(4, 16)[:, 1:], y.data.reshape(4, 16)[:, :-1])     # targets = inputs shifted by one
+
+
+def test_dataloader_needs_more_tokens_than_the_block():
+    with pytest.raises(IndexError):
+        rm.DataLoader(np.arange(16, dtype=np.int32), ref.SeededRng(0), 2, 16).next_batch()      # data.ts:97-101
+    rm.DataLoader(np.arange(17, dtype=np.int32), ref.SeededRng(0), 2, 16).next_batch()
+
+
+@pytest.mark.parametrize("N,Bt,T", [(103, 4, 8), (64, 4, 16), (10, 3, 7), (5, 2, 12), (9, 2, 1)])
+def test_dataloader_packed_cursors_cover_the_corpus_and_wrap(N, Bt, T):
+    tok = (np.arange(N) * 31 % 97).astype(np.int32)
+    dl = rm.DataLoader(tok, ref.SeededRng(0), Bt, T, packed=True)
+    cursors = [b * (N // Bt) for b in range(Bt)]                                    # data.ts:37-45
+    seen = np.zeros(N, np.int64)
+    for _ in range(2 * N):
+        x, y = dl.next_batch()
+        inp, tgt = _naive_windows(tok, cursors, T)
+        assert np.array_equal(x.data.reshape(Bt, T), inp) and np.array_equal(y.data.reshape(Bt, T), tgt)
+        for c in cursors:
+            for t in range(T):
+                seen[(c + t) % N] += 1
+        cursors = [(c + T) % N for c in cursors]
+        assert dl.cursors == cursors
+    # every cursor has advanced 2*N*T positions = 2*T whole passes: each token was served equally often
+    assert seen.min() == seen.max() == 2 * T * Bt
