@@ -10,6 +10,16 @@
 //
 // One block = 4 waves = 128 owned rows; the streamed operand moves in 64-row tiles, register-prefetched one tile
 // ahead and double-buffered in LDS (one barrier per 64 rows).
+//
+// The kernels are bound by the per-score VALU work (exp and rcp are quarter rate), not by the MFMAs, so the score
+// path is pared down to the instructions that cannot be avoided:
+//   * everything runs in base-2: constants carry log2(e), exp is the bare v_exp_f32;
+//   * with a soft cap c the capped score is c*tanh(u) = c - 2c*r, r = 1/(exp(2u) + 1), which is bounded by c.  For
+//     c <= 40 the running maximum of the online softmax is replaced by the constant c: p = exp(-2c*r) needs no max
+//     pass, no rescale of the output accumulators and no cross-lane traffic until the row sum is finished; the smallest
+//     possible p, exp(-80), is far inside fp32 / bf16 range.  tanh' = 4r(1 - r) reuses r in the backward kernels;
+//   * masking code runs only for tiles that touch the diagonal or the end of the sequence (a wave-uniform branch);
+//   * constant factors (scale, the 4 of tanh') are applied once to the accumulators, not per score.
 #include "attention_common.h"
 
 using namespace ah;
@@ -26,12 +36,11 @@ template <int D> struct Geo {
   static constexpr int CHUNKS = ST * D / 8 / 256;      // 16-byte chunks per thread per tile (D=32: 1, 64: 2, 128: 4)
 };
 
-__device__ __forceinline__ float softcap_f(float s, float cap, float inv_cap) {
-  // cap * tanh(s / cap) with tanh(x) = 1 - 2 / (exp(2x) + 1): one exp and one reciprocal
-  if (cap <= 0.f) return s;
-  float e = __expf(2.0f * s * inv_cap);
-  return cap * (1.0f - 2.0f * __frcp_rn(e + 1.0f));
-}
+constexpr float LOG2E = 1.4426950408889634f;
+constexpr float FIXED_MAX_CAP = 40.f;      // soft caps up to this use the constant-maximum softmax
+
+__device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float rcp_fast(float x) { return __builtin_amdgcn_rcpf(x); }
 
 // global -> registers: rows [row0, row0+64) of a [T][D] operand with row stride st (elements); rows >= T read as zero
 template <int D>
@@ -98,17 +107,20 @@ __device__ __forceinline__ void store_rows(uint16_t *__restrict__ dst, const f32
 }
 
 // ------------------------------------------------------------------------------------------ forward
-template <int D>
+template <int D, bool CAPPED>
 __global__ __launch_bounds__(256) void k_flash_fwd_bf16(FlashArgs a) {
   constexpr int DB = D / 32, KS = D / 16;
   __shared__ __attribute__((aligned(16))) uint16_t Ks[2][Geo<D>::ELEMS], Vs[2][Geo<D>::ELEMS];
   int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
   int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 31, lk = lane >> 5;
-  int q0 = blockIdx.x * 128 + wave * 32, qi = q0 + lr;
+  int qblk = gridDim.x - 1 - blockIdx.x;                           // longest (latest) query blocks are scheduled first
+  int q0 = qblk * 128 + wave * 32, qi = q0 + lr;
   const uint16_t *Q = (const uint16_t *)a.q + b * a.q_sb + h * a.q_sh;
   const uint16_t *K = (const uint16_t *)a.k + b * a.k_sb + h * a.k_sh;
   const uint16_t *V = (const uint16_t *)a.v + b * a.v_sb + h * a.v_sh;
-  float inv_cap = a.cap > 0.f ? 1.0f / a.cap : 0.f;
+  // CAPPED: u2 = s*c1 = 2*score/cap in base 2; p = 2^(c2*r).  Otherwise x = s*c1 = score in base 2.
+  const float c1 = CAPPED ? 2.0f * a.scale * LOG2E / a.cap : a.scale * LOG2E;
+  const float c2 = -2.0f * a.cap * LOG2E;
 
   bf16x8 qf[KS];
   row_frags<D>(Q, a.q_st, qi, qi < a.T, lane, qf);
@@ -117,9 +129,11 @@ __global__ __launch_bounds__(256) void k_flash_fwd_bf16(FlashArgs a) {
   for (int d = 0; d < DB; d++)
 #pragma unroll
     for (int e = 0; e < 16; e++) o[d][e] = 0.f;
-  float m = -INFINITY, l = 0.f;
+  // CAPPED: l and l_rnd are this half-wave's partial row sums of the probabilities as computed (for LSE, which the backward
+  // kernels use to rebuild them) and as rounded to bf16 for the MFMA (for normalising O); m is unused
+  float m = -INFINITY, l = 0.f, l_rnd = 0.f;
 
-  int kv_end = min(a.T, (int)(blockIdx.x + 1) * 128);            // causal: keys < kv_end
+  int kv_end = min(a.T, (qblk + 1) * 128);                         // causal: keys < kv_end
   int ntile = (kv_end + ST - 1) / ST;
   u32x4 rk[Geo<D>::CHUNKS], rv[Geo<D>::CHUNKS];
   tile_load<D>(K, a.k_st, 0, a.T, rk);
@@ -143,30 +157,58 @@ __global__ __launch_bounds__(256) void k_flash_fwd_bf16(FlashArgs a) {
 #pragma unroll
         for (int ks = 0; ks < KS; ks++)
           s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tile_frag<D>(Ks[cur], sub * 32, ks, lane), qf[ks], s, 0, 0, 0);   // S^T[kv, q]
-        float tmax = -INFINITY;
+        const bool edge = kv0 + 31 > q0 || kv0 + 32 > a.T;         // wave-uniform: some score of the tile is masked
+        if (CAPPED) {
 #pragma unroll
-        for (int e = 0; e < 16; e++) {
-          int kv = kv0 + 8 * (e >> 2) + 4 * lk + (e & 3);
-          float x = softcap_f(s[e] * a.scale, a.cap, inv_cap);
-          x = (kv > qi || kv >= a.T) ? -INFINITY : x;
-          s[e] = x;
-          tmax = fmaxf(tmax, x);
+          for (int e = 0; e < 16; e++) {
+            float r = rcp_fast(exp2_fast(s[e] * c1) + 1.0f);
+            s[e] = exp2_fast(c2 * r);
+          }
+          if (edge) {
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+              int kv = kv0 + 8 * (e >> 2) + 4 * lk + (e & 3);
+              s[e] = (kv > qi || kv >= a.T) ? 0.f : s[e];
+            }
+          }
+#pragma unroll
+          for (int e = 0; e < 16; e++) l += s[e];
+        } else {
+          float tmax = -INFINITY;
+#pragma unroll
+          for (int e = 0; e < 16; e++) {
+            float x = s[e] * c1;
+            if (edge) {
+              int kv = kv0 + 8 * (e >> 2) + 4 * lk + (e & 3);
+              x = (kv > qi || kv >= a.T) ? -INFINITY : x;
+            }
+            s[e] = x;
+            tmax = fmaxf(tmax, x);
+          }
+          tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+          float m_new = fmaxf(m, tmax);
+          float m_use = m_new == -INFINITY ? 0.f : m_new;
+          float alpha = exp2_fast(m - m_use);
+          float psum = 0.f;
+#pragma unroll
+          for (int e = 0; e < 16; e++) { float p = exp2_fast(s[e] - m_use); s[e] = p; psum += p; }
+          psum += __shfl_xor(psum, 32, 64);
+          l = l * alpha + psum;
+          m = m_new;
+#pragma unroll
+          for (int d = 0; d < DB; d++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) o[d][e] *= alpha;
         }
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-        float m_new = fmaxf(m, tmax);
-        float m_use = m_new == -INFINITY ? 0.f : m_new;
-        float alpha = __expf(m - m_use);
-        float psum = 0.f;
-#pragma unroll
-        for (int e = 0; e < 16; e++) { float p = __expf(s[e] - m_use); s[e] = p; psum += p; }
-        psum += __shfl_xor(psum, 32, 64);
-        l = l * alpha + psum;
-        m = m_new;
         bf16x8 pb0 = acc_to_b(s, 0), pb1 = acc_to_b(s, 1);
+        if (CAPPED) {
+          // O is normalised by the sum of the bf16-rounded probabilities the MFMA sees (a row with a single key
+          // returns that key's V exactly)
+#pragma unroll
+          for (int i = 0; i < 8; i++) l_rnd += (float)pb0[i] + (float)pb1[i];
+        }
 #pragma unroll
         for (int d = 0; d < DB; d++) {
-#pragma unroll
-          for (int e = 0; e < 16; e++) o[d][e] *= alpha;
           o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tile_frag_t<D>(Vs[cur], sub * 32, 0, d, lane), pb0, o[d], 0, 0, 0);   // O^T[d, q]
           o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tile_frag_t<D>(Vs[cur], sub * 32, 1, d, lane), pb1, o[d], 0, 0, 0);
         }
@@ -178,55 +220,73 @@ __global__ __launch_bounds__(256) void k_flash_fwd_bf16(FlashArgs a) {
     }
     __syncthreads();
   }
+  if (CAPPED) { l += __shfl_xor(l, 32, 64); l_rnd += __shfl_xor(l_rnd, 32, 64); } else l_rnd = l;
   if (qi < a.T) {
-    float inv_l = l > 0.f ? 1.0f / l : 0.f;
+    float inv_l = l_rnd > 0.f ? 1.0f / l_rnd : 0.f;
     store_rows<D>((uint16_t *)a.o + b * a.o_sb + h * a.o_sh + (int64_t)qi * a.o_st, o, inv_l, lane);
-    if (lk == 0) a.lse[((int64_t)b * a.H + h) * a.T + qi] = m + __logf(l);
+    // natural-log LSE: the constant maximum is the cap itself; the running maximum is held in base 2
+    if (lk == 0) a.lse[((int64_t)b * a.H + h) * a.T + qi] = (CAPPED ? a.cap : m * (1.0f / LOG2E)) + __logf(l);
   }
 }
 
-// delta[b,h,t] = sum_d dO[t,d] * O[t,d]   (one wave per row)
-template <int D>
-__global__ void k_flash_delta_bf16(FlashArgs a) {
-  int64_t row = blockIdx.x * (int64_t)(blockDim.x >> 6) + (threadIdx.x >> 6);
-  int64_t total = (int64_t)a.B * a.H * a.T;
-  if (row >= total) return;
-  int lane = threadIdx.x & 63;
-  int t = (int)(row % a.T), h = (int)((row / a.T) % a.H), b = (int)(row / ((int64_t)a.T * a.H));
-  const uint16_t *O = (const uint16_t *)a.o + b * a.o_sb + h * a.o_sh + (int64_t)t * a.o_st;
-  const uint16_t *dO = (const uint16_t *)a.d_o + b * a.o_sb + h * a.o_sh + (int64_t)t * a.o_st;
-  float s = 0.f;
-  for (int d = lane; d < D; d += 64) s += bf16_bits_to_f32(O[d]) * bf16_bits_to_f32(dO[d]);
-  s = wave_sum(s);
-  if (lane == 0) a.delta[row] = s;
+// Per-score backward arithmetic shared by the dQ and dK/dV kernels.  s = raw q.k, dp = dO.v, krow = (max - lse) in
+// base 2 (max = cap when CAPPED, else 0), delta = rowsum(dO*O).  Returns p and writes ds WITHOUT the constant factor
+// (scale, and 4 for tanh' when CAPPED), which the caller applies to its accumulators once.
+template <bool CAPPED>
+__device__ __forceinline__ float score_bwd(float s, float dp, float krow, float delta, float c1, float c2, float &ds) {
+  float p;
+  if (CAPPED) {
+    float r = rcp_fast(exp2_fast(s * c1) + 1.0f);
+    p = exp2_fast(fmaf(r, c2, krow));
+    ds = p * (dp - delta) * fmaf(-r, r, r);                        // tanh' / 4 = r (1 - r)
+  } else {
+    p = exp2_fast(fmaf(s, c1, krow));
+    ds = p * (dp - delta);
+  }
+  return p;
 }
 
-// ------------------------------------------------------------------------------------------ dQ
-template <int D>
+// ------------------------------------------------------------------------------------------ dQ (and delta)
+template <int D, bool CAPPED>
 __global__ __launch_bounds__(256) void k_flash_dq_bf16(FlashArgs a) {
   constexpr int DB = D / 32, KS = D / 16;
   __shared__ __attribute__((aligned(16))) uint16_t Ks[2][Geo<D>::ELEMS], Vs[2][Geo<D>::ELEMS];
   int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
   int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 31, lk = lane >> 5;
-  int q0 = blockIdx.x * 128 + wave * 32, qi = q0 + lr;
+  int qblk = gridDim.x - 1 - blockIdx.x;
+  int q0 = qblk * 128 + wave * 32, qi = q0 + lr;
   const uint16_t *Q = (const uint16_t *)a.q + b * a.q_sb + h * a.q_sh;
   const uint16_t *K = (const uint16_t *)a.k + b * a.k_sb + h * a.k_sh;
   const uint16_t *V = (const uint16_t *)a.v + b * a.v_sb + h * a.v_sh;
+  const uint16_t *O = (const uint16_t *)a.o + b * a.o_sb + h * a.o_sh;
   const uint16_t *dO = (const uint16_t *)a.d_o + b * a.o_sb + h * a.o_sh;
-  float inv_cap = a.cap > 0.f ? 1.0f / a.cap : 0.f;
+  const float c1 = CAPPED ? 2.0f * a.scale * LOG2E / a.cap : a.scale * LOG2E;
+  const float c2 = -2.0f * a.cap * LOG2E;
   bool live = qi < a.T;
   bf16x8 qf[KS], dof[KS];
   row_frags<D>(Q, a.q_st, qi, live, lane, qf);
   row_frags<D>(dO, a.o_st, qi, live, lane, dof);
   int64_t srow = ((int64_t)b * a.H + h) * a.T + qi;
-  float lse = live ? a.lse[srow] : 0.f, delta = live ? a.delta[srow] : 0.f;
+  // delta = rowsum(dO * O): each half-wave holds half of the row's features; also published for the dK/dV kernel
+  float delta = 0.f;
+  {
+    bf16x8 of[KS];
+    row_frags<D>(O, a.o_st, qi, live, lane, of);
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++)
+#pragma unroll
+      for (int i = 0; i < 8; i++) delta += (float)dof[ks][i] * (float)of[ks][i];
+    delta += __shfl_xor(delta, 32, 64);
+    if (live && lk == 0) a.delta[srow] = delta;
+  }
+  float krow = live ? ((CAPPED ? a.cap : 0.f) - a.lse[srow]) * LOG2E : 0.f;
   f32x16 dq[DB];
 #pragma unroll
   for (int d = 0; d < DB; d++)
 #pragma unroll
     for (int e = 0; e < 16; e++) dq[d][e] = 0.f;
 
-  int kv_end = min(a.T, (int)(blockIdx.x + 1) * 128);
+  int kv_end = min(a.T, (qblk + 1) * 128);
   int ntile = (kv_end + ST - 1) / ST;
   u32x4 rk[Geo<D>::CHUNKS], rv[Geo<D>::CHUNKS];
   tile_load<D>(K, a.k_st, 0, a.T, rk);
@@ -252,14 +312,19 @@ __global__ __launch_bounds__(256) void k_flash_dq_bf16(FlashArgs a) {
           s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tile_frag<D>(Ks[cur], sub * 32, ks, lane), qf[ks], s, 0, 0, 0);     // S^T[kv, q]
           dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tile_frag<D>(Vs[cur], sub * 32, ks, lane), dof[ks], dp, 0, 0, 0);  // dP^T[kv, q]
         }
+        const bool edge = kv0 + 31 > q0 || kv0 + 32 > a.T;
 #pragma unroll
         for (int e = 0; e < 16; e++) {
-          int kv = kv0 + 8 * (e >> 2) + 4 * lk + (e & 3);
-          float sc = softcap_f(s[e] * a.scale, a.cap, inv_cap);
-          float p = (kv > qi || kv >= a.T || !live) ? 0.f : __expf(sc - lse);
-          float ds = p * (dp[e] - delta);
-          if (a.cap > 0.f) { float t = sc * inv_cap; ds *= (1.0f - t * t); }
-          s[e] = ds * a.scale;
+          float ds;
+          score_bwd<CAPPED>(s[e], dp[e], krow, delta, c1, c2, ds);
+          s[e] = ds;
+        }
+        if (edge) {
+#pragma unroll
+          for (int e = 0; e < 16; e++) {
+            int kv = kv0 + 8 * (e >> 2) + 4 * lk + (e & 3);
+            s[e] = (kv > qi || kv >= a.T) ? 0.f : s[e];
+          }
         }
         bf16x8 b0 = acc_to_b(s, 0), b1 = acc_to_b(s, 1);
 #pragma unroll
@@ -275,15 +340,15 @@ __global__ __launch_bounds__(256) void k_flash_dq_bf16(FlashArgs a) {
     }
     __syncthreads();
   }
-  if (live) store_rows<D>((uint16_t *)a.dq + b * a.q_sb + h * a.q_sh + (int64_t)qi * a.q_st, dq, 1.0f, lane);
+  if (live) store_rows<D>((uint16_t *)a.dq + b * a.q_sb + h * a.q_sh + (int64_t)qi * a.q_st, dq, CAPPED ? 4.0f * a.scale : a.scale, lane);
 }
 
 // ------------------------------------------------------------------------------------------ dK, dV
-template <int D>
-__global__ __launch_bounds__(256) void k_flash_dkv_bf16(FlashArgs a) {
+template <int D, bool CAPPED>
+__global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void k_flash_dkv_bf16(FlashArgs a) {
   constexpr int DB = D / 32, KS = D / 16;
   __shared__ __attribute__((aligned(16))) uint16_t Qs[2][Geo<D>::ELEMS], dOs[2][Geo<D>::ELEMS];
-  __shared__ float Ls[2][ST], Ds[2][ST];
+  __shared__ __attribute__((aligned(16))) float Ls[2][ST], Ds[2][ST];      // per streamed query: (max - lse) in base 2; delta
   int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
   int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 31, lk = lane >> 5;
   int kv_blk0 = blockIdx.x * 128, kv0 = kv_blk0 + wave * 32, kvi = kv0 + lr;
@@ -291,7 +356,9 @@ __global__ __launch_bounds__(256) void k_flash_dkv_bf16(FlashArgs a) {
   const uint16_t *K = (const uint16_t *)a.k + b * a.k_sb + h * a.k_sh;
   const uint16_t *V = (const uint16_t *)a.v + b * a.v_sb + h * a.v_sh;
   const uint16_t *dO = (const uint16_t *)a.d_o + b * a.o_sb + h * a.o_sh;
-  float inv_cap = a.cap > 0.f ? 1.0f / a.cap : 0.f;
+  const float c1 = CAPPED ? 2.0f * a.scale * LOG2E / a.cap : a.scale * LOG2E;
+  const float c2 = -2.0f * a.cap * LOG2E;
+  const float lse_max = CAPPED ? a.cap : 0.f;
   bool live = kvi < a.T;
   bf16x8 kf[KS], vf[KS];
   row_frags<D>(K, a.k_st, kvi, live, lane, kf);
@@ -307,10 +374,11 @@ __global__ __launch_bounds__(256) void k_flash_dkv_bf16(FlashArgs a) {
   int ntile = (a.T - q_first + ST - 1) / ST;
   u32x4 rq[Geo<D>::CHUNKS], rdo[Geo<D>::CHUNKS];
   float rl = 0.f, rd = 0.f;
+  // rows past the end of the sequence carry zero Q / dO and finite statistics, so they contribute exact zeros
   auto load_stats = [&](int q_base) {
     if (threadIdx.x < ST) {
       int qi = q_base + threadIdx.x;
-      rl = qi < a.T ? a.lse[srow0 + qi] : 0.f;
+      rl = qi < a.T ? (lse_max - a.lse[srow0 + qi]) * LOG2E : 0.f;
       rd = qi < a.T ? a.delta[srow0 + qi] : 0.f;
     }
   };
@@ -340,18 +408,31 @@ __global__ __launch_bounds__(256) void k_flash_dkv_bf16(FlashArgs a) {
           s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tile_frag<D>(Qs[cur], sub * 32, ks, lane), kf[ks], s, 0, 0, 0);
           dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tile_frag<D>(dOs[cur], sub * 32, ks, lane), vf[ks], dp, 0, 0, 0);
         }
-        f32x16 pm;
+        const bool edge = qs < kv0 + 31;                           // wave-uniform: some query of the tile precedes some key
 #pragma unroll
-        for (int e = 0; e < 16; e++) {
-          int qr = sub * 32 + 8 * (e >> 2) + 4 * lk + (e & 3), qi = q_first + it * ST + qr;
-          float sc = softcap_f(s[e] * a.scale, a.cap, inv_cap);
-          float p = (kvi > qi || qi >= a.T || !live) ? 0.f : __expf(sc - Ls[cur][qr]);
-          float ds = p * (dp[e] - Ds[cur][qr]);
-          if (a.cap > 0.f) { float t = sc * inv_cap; ds *= (1.0f - t * t); }
-          pm[e] = p;
-          s[e] = ds * a.scale;
+        for (int j = 0; j < 4; j++) {
+          float4 kr = *reinterpret_cast<const float4 *>(&Ls[cur][sub * 32 + 8 * j + 4 * lk]);
+          float4 de = *reinterpret_cast<const float4 *>(&Ds[cur][sub * 32 + 8 * j + 4 * lk]);
+          float krv[4] = {kr.x, kr.y, kr.z, kr.w}, dev[4] = {de.x, de.y, de.z, de.w};
+#pragma unroll
+          for (int r = 0; r < 4; r++) {
+            int e = 4 * j + r;
+            float ds;
+            float p = score_bwd<CAPPED>(s[e], dp[e], krv[r], dev[r], c1, c2, ds);
+            dp[e] = p;
+            s[e] = ds;
+          }
         }
-        bf16x8 p0 = acc_to_b(pm, 0), p1 = acc_to_b(pm, 1), d0 = acc_to_b(s, 0), d1 = acc_to_b(s, 1);
+        if (edge) {
+#pragma unroll
+          for (int e = 0; e < 16; e++) {
+            int qi = qs + 8 * (e >> 2) + 4 * lk + (e & 3);
+            bool dead = kvi > qi;
+            dp[e] = dead ? 0.f : dp[e];
+            s[e] = dead ? 0.f : s[e];
+          }
+        }
+        bf16x8 p0 = acc_to_b(dp, 0), p1 = acc_to_b(dp, 1), d0 = acc_to_b(s, 0), d1 = acc_to_b(s, 1);
 #pragma unroll
         for (int d = 0; d < DB; d++) {
           dv[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tile_frag_t<D>(dOs[cur], sub * 32, 0, d, lane), p0, dv[d], 0, 0, 0);   // dV^T[d, kv]
@@ -369,33 +450,39 @@ __global__ __launch_bounds__(256) void k_flash_dkv_bf16(FlashArgs a) {
     __syncthreads();
   }
   if (live) {
-    store_rows<D>((uint16_t *)a.dk + b * a.k_sb + h * a.k_sh + (int64_t)kvi * a.k_st, dk, 1.0f, lane);
+    store_rows<D>((uint16_t *)a.dk + b * a.k_sb + h * a.k_sh + (int64_t)kvi * a.k_st, dk, CAPPED ? 4.0f * a.scale : a.scale, lane);
     store_rows<D>((uint16_t *)a.dv + b * a.v_sb + h * a.v_sh + (int64_t)kvi * a.v_st, dv, 1.0f, lane);
   }
 }
 
-template <int D>
+template <int D, bool CAPPED>
 int32_t run_fwd(const FlashArgs &a) {
   dim3 grid((unsigned)cdiv(a.T, 128), (unsigned)(a.B * a.H));
-  hipLaunchKernelGGL(k_flash_fwd_bf16<D>, grid, dim3(256), 0, stream(), a);
+  hipLaunchKernelGGL((k_flash_fwd_bf16<D, CAPPED>), grid, dim3(256), 0, stream(), a);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
-template <int D>
+template <int D, bool CAPPED>
 int32_t run_bwd(FlashArgs &a) {
   int64_t rows = (int64_t)a.B * a.H * a.T;
   ah_ptr delta = 0;
   int32_t rc = ah_alloc((uint64_t)rows * 4, &delta);
   if (rc) return rc;
   a.delta = dp<float>(delta);
-  hipLaunchKernelGGL(k_flash_delta_bf16<D>, dim3((unsigned)cdiv(rows, 4)), dim3(256), 0, stream(), a);
-  AH_LAUNCH_CHECK();
   dim3 grid((unsigned)cdiv(a.T, 128), (unsigned)(a.B * a.H));
-  hipLaunchKernelGGL(k_flash_dq_bf16<D>, grid, dim3(256), 0, stream(), a);
+  hipLaunchKernelGGL((k_flash_dq_bf16<D, CAPPED>), grid, dim3(256), 0, stream(), a);      // also writes delta
   AH_LAUNCH_CHECK();
-  hipLaunchKernelGGL(k_flash_dkv_bf16<D>, grid, dim3(256), 0, stream(), a);
+  hipLaunchKernelGGL((k_flash_dkv_bf16<D, CAPPED>), grid, dim3(256), 0, stream(), a);
   AH_LAUNCH_CHECK();
   return ah_free(delta);
+}
+template <int D>
+int32_t run_fwd_d(const FlashArgs &a) {
+  return a.cap > 0.f && a.cap <= FIXED_MAX_CAP ? run_fwd<D, true>(a) : run_fwd<D, false>(a);
+}
+template <int D>
+int32_t run_bwd_d(FlashArgs &a) {
+  return a.cap > 0.f && a.cap <= FIXED_MAX_CAP ? run_bwd<D, true>(a) : run_bwd<D, false>(a);
 }
 
 }  // namespace
@@ -404,16 +491,16 @@ namespace ah {
 
 int32_t flash_fwd_bf16(const FlashArgs &a, int head_dim) {
   switch (head_dim) {
-    case 32: return run_fwd<32>(a);
-    case 64: return run_fwd<64>(a);
-    default: return run_fwd<128>(a);
+    case 32: return run_fwd_d<32>(a);
+    case 64: return run_fwd_d<64>(a);
+    default: return run_fwd_d<128>(a);
   }
 }
 int32_t flash_bwd_bf16(FlashArgs &a, int head_dim) {
   switch (head_dim) {
-    case 32: return run_bwd<32>(a);
-    case 64: return run_bwd<64>(a);
-    default: return run_bwd<128>(a);
+    case 32: return run_bwd_d<32>(a);
+    case 64: return run_bwd_d<64>(a);
+    default: return run_bwd_d<128>(a);
   }
 }
 
