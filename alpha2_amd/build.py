@@ -14,7 +14,8 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(CSRC, "build")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIB_DIR, "libalpha_hip.so")
-SOURCES = ["runtime", "elementwise", "reduce", "nn", "optimizer", "gemm", "gemm_bf16", "attention", "attention_bf16"]
+SOURCES = ["runtime", "elementwise", "reduce", "nn", "optimizer", "gemm", "gemm_bf16", "gemm_bf16_dma_nt", "gemm_bf16_dma_nn",
+           "gemm_bf16_dma_tn", "attention", "attention_bf16"]
 # -packed-fp32-ops off: the compiler must not form v_pk_*_f32 from ordinary float code on this target.
 FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          "-Wno-unused-command-line-argument"]
@@ -30,7 +31,8 @@ def _hipcc() -> str:
 def _compile(name: str, force: bool) -> str:
     src = os.path.join(CSRC, name + ".hip")
     obj = os.path.join(OBJ, name + ".o")
-    deps = [src, os.path.join(CSRC, "common.h"), os.path.join(CSRC, "gemm_common.h"), os.path.join(CSRC, "attention_common.h"), os.path.join(HERE, "..", "include", "alpha_hip.h")]
+    deps = [src, os.path.join(CSRC, "common.h"), os.path.join(CSRC, "gemm_common.h"), os.path.join(CSRC, "gemm_bf16_dma.inc"),
+            os.path.join(CSRC, "attention_common.h"), os.path.join(HERE, "..", "include", "alpha_hip.h")]
     if not force and os.path.exists(obj) and all(os.path.getmtime(obj) >= os.path.getmtime(d) for d in deps):
         return obj
     cmd = [_hipcc()] + FLAGS + ["-c", src, "-o", obj]
@@ -40,7 +42,7 @@ def _compile(name: str, force: bool) -> str:
     return obj
 
 
-def build(force: bool = False, jobs: int = 6) -> str:
+def build(force: bool = False, jobs: int = 8) -> str:
     os.makedirs(OBJ, exist_ok=True)
     os.makedirs(LIB_DIR, exist_ok=True)
     with ThreadPoolExecutor(max_workers=jobs) as ex:

@@ -72,17 +72,21 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
-// tanh-approximation GELU and its derivative (cpu_ref.ts:422-427; ops.ts:405-417)
-__device__ __forceinline__ float gelu_f(float x) {
-  const float k = 0.7978845608028654f;
-  return 0.5f * x * (1.0f + tanhf(k * (x + 0.044715f * x * x * x)));
+// tanh-approximation GELU and its derivative (cpu_ref.ts:422-427; ops.ts:405-417), written on r = 1 / (exp(2u) + 1):
+// tanh(u) = 1 - 2r, so 0.5 (1 + tanh u) = 1 - r and sech^2 u = 4 r (1 - r).  Two hardware transcendentals, no
+// branches, absolute error at fp32 rounding level (the epilogues of the big GEMM tiles cannot afford libm's tanhf:
+// its register footprint on top of 256 live accumulators spills).
+__device__ __forceinline__ float gelu_gate_r(float x) {
+  const float k2 = 0.7978845608028654f * 2.0f * 1.4426950408889634f;      // 2 sqrt(2/pi) log2(e)
+  float u2 = k2 * (x + 0.044715f * x * x * x);
+  return __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(u2) + 1.0f);
 }
+__device__ __forceinline__ float gelu_f(float x) { return x * (1.0f - gelu_gate_r(x)); }
 __device__ __forceinline__ float gelu_grad_f(float x) {
   const float k = 0.7978845608028654f;
-  float t = tanhf(k * (x + 0.044715f * x * x * x));
-  float sech2 = 1.0f - t * t;
+  float r = gelu_gate_r(x);
   float dinner = k * (1.0f + 3.0f * 0.044715f * x * x);
-  return 0.5f * (1.0f + t) + 0.5f * x * sech2 * dinner;
+  return (1.0f - r) * (1.0f + 2.0f * x * r * dinner);
 }
 
 }  // namespace ah

@@ -78,21 +78,6 @@ __device__ __forceinline__ bf16x8 g_frag(const uint16_t *s, int base, int kk) {
   }
 }
 
-template <int EPI, class OUT, int TM, int TN>
-__device__ __forceinline__ void store_tiles(const GemmArgs &g, int64_t cbase, int row0, int col0, int lane, const f32x16 (&acc)[TM][TN]) {
-  int lr = lane & 31, lk = lane >> 5;
-#pragma unroll
-  for (int i = 0; i < TM; i++)
-#pragma unroll
-    for (int j = 0; j < TN; j++) {
-#pragma unroll
-      for (int q = 0; q < 4; q++)
-        epilogue4<EPI, OUT>(g, cbase, row0 + 32 * i + lr, col0 + 32 * j + 8 * q + 4 * lk, acc[i][j][4 * q], acc[i][j][4 * q + 1],
-                            acc[i][j][4 * q + 2], acc[i][j][4 * q + 3], true);
-      __builtin_amdgcn_sched_barrier(0);      // drain one 32x32 tile at a time: the accumulators leave AGPRs 16 at a time
-    }
-}
-
 // split-K: slice y writes its partial tile (plain f32 stores) to workspace[y][M][N]; this kernel then sums the slices
 // in fixed order into C (deterministic, unlike atomic accumulation).
 __global__ void k_splitk_reduce(const float *__restrict__ ws, float *__restrict__ c, int nsplit, int M, int N, int64_t ldc, int accumulate) {
@@ -247,11 +232,12 @@ int32_t launch(const GemmArgs &ga, int batch, int out_dtype) {
 
 template <bool AKM, bool BKM>
 int32_t run(const GemmArgs &ga, int batch, int out_dtype) {
-  // 256x256 tile on 8 waves (2 x 4, each 128 x 64): half the L2 traffic per flop of the 128x128 tile, two waves per
-  // SIMD to overlap each other's loads.  Used when it still fills the chip; otherwise 128x128 at 3 blocks per CU.
+  // Outputs with at least one 256x256 tile per CU go to the kernel fed by global->LDS loads (gemm_bf16_dma.inc): half
+  // the L2 traffic and a third of the LDS traffic per flop of the 128x128 tile.  Smaller outputs keep the 128x128 tile
+  // of this file, two blocks per CU.
   int64_t big_blocks = cdiv(ga.M, 256) * cdiv(ga.N, 256) * batch * ga.nsplit;
   bool big = ga.M >= 256 && ga.N >= 256 && big_blocks >= num_cus();
-  if (big) return launch<256, 256, 2, 4, AKM, BKM>(ga, batch, out_dtype);
+  if (big) return AKM ? gemm_bf16_dma_tn(ga, batch, out_dtype) : BKM ? gemm_bf16_dma_nn(ga, batch, out_dtype) : gemm_bf16_dma_nt(ga, batch, out_dtype);
   return launch<128, 128, 2, 2, AKM, BKM>(ga, batch, out_dtype);
 }
 

@@ -1,0 +1,5 @@
+// bf16 GEMM with direct global->LDS loads, TN layout (see gemm_bf16_dma.inc).
+#define DMA_AKM true
+#define DMA_BKM true
+#define DMA_ENTRY gemm_bf16_dma_tn
+#include "gemm_bf16_dma.inc"

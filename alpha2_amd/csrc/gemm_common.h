@@ -67,8 +67,28 @@ __device__ __forceinline__ void epilogue4(const GemmArgs &g, int64_t cbase, int 
   }
 }
 
+// Stores a wave's TM x TN grid of 32x32 accumulators (C^T orientation: 4 consecutive registers = 4 consecutive columns).
+template <int EPI, class OUT, int TM, int TN>
+__device__ __forceinline__ void store_tiles(const GemmArgs &g, int64_t cbase, int row0, int col0, int lane, const f32x16 (&acc)[TM][TN]) {
+  int lr = lane & 31, lk = lane >> 5;
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+#pragma unroll
+      for (int q = 0; q < 4; q++)
+        epilogue4<EPI, OUT>(g, cbase, row0 + 32 * i + lr, col0 + 32 * j + 8 * q + 4 * lk, acc[i][j][4 * q], acc[i][j][4 * q + 1],
+                            acc[i][j][4 * q + 2], acc[i][j][4 * q + 3], true);
+      __builtin_amdgcn_sched_barrier(0);      // drain one 32x32 tile at a time: the accumulators leave AGPRs 16 at a time
+    }
+}
+
 
 // gemm_bf16.hip
 int32_t gemm_bf16_direct(const GemmArgs &ga, int layout, int batch, int out_dtype);
+// gemm_bf16_dma_{nt,nn,tn}.hip: 256x256 tiles fed by direct global->LDS loads (same preconditions as the direct kernel)
+int32_t gemm_bf16_dma_nt(const GemmArgs &ga, int batch, int out_dtype);
+int32_t gemm_bf16_dma_nn(const GemmArgs &ga, int batch, int out_dtype);
+int32_t gemm_bf16_dma_tn(const GemmArgs &ga, int batch, int out_dtype);
 
 }  // namespace ah

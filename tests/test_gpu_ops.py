@@ -500,3 +500,36 @@ def test_flash_attention_bf16_vs_materialised(B, BH, T, D, cap):
         assert_close(g["dQ"].data, dq, rel=rel, what="flash16.dQ", **loose(dq))
         assert_close(g["dK"].data, dk, rel=rel, what="flash16.dK", **loose(dk))
     assert_close(g["dV"].data, dv, rel=rel, what="flash16.dV", **loose(dv))
+
+
+@pytest.mark.parametrize("K", [64, 192, 512])
+def test_gemm_bf16_large_tiles_direct_to_lds_kernel(B, K):
+    """Outputs with at least one 256x256 tile per CU take the kernel fed by global->LDS loads; edges in M and N, odd and
+    even k-tile counts, every layout and epilogue.  At this size the check is a float64 numpy product of the same
+    bf16-exact operands (the C oracle covers the small shapes above); fp32 accumulation of exact products."""
+    from alpha2_amd import _ffi as ffi
+    M, N = 4000, 4072          # 16 x 16 tiles of 256, ragged edges, N % 8 == 0 and M % 8 == 0 for the k-major layouts
+    a, b = _bf16_round(rs.randn(M, K).astype(np.float32))[0], _bf16_round(rs.randn(N, K).astype(np.float32))[0]
+    want = a.astype(np.float64) @ b.astype(np.float64).T
+    at, bt = np.ascontiguousarray(a.T), np.ascontiguousarray(b.T)
+
+    def used_dma():
+        name, _ = B.lastGemmKernel()
+        return name.startswith("k_gemm_bf16_dma")
+    got = _raw_gemm(B, ffi.GEMM_NT, a, b, M, N, K, ffi.BF16, ffi.F32)[0]
+    if B.getDeviceInfo()["computeUnits"] <= 256:
+        assert used_dma(), B.lastGemmKernel()
+    assert_close(got, want, rel=1e-4, what="NT f32")
+    assert_close(_raw_gemm(B, ffi.GEMM_NT, a, b, M, N, K, ffi.BF16, ffi.BF16)[0], want, rel=2.0 ** -7, what="NT bf16")
+    assert_close(_raw_gemm(B, ffi.GEMM_NN, a, bt, M, N, K, ffi.BF16, ffi.F32)[0], want, rel=1e-4, what="NN")
+    assert_close(_raw_gemm(B, ffi.GEMM_TN, at, bt, M, N, K, ffi.BF16, ffi.F32)[0], want, rel=1e-4, what="TN")
+    c0 = rs.randn(M, N).astype(np.float32)
+    assert_close(_raw_gemm(B, ffi.GEMM_TN, at, bt, M, N, K, ffi.BF16, ffi.F32, ffi.EPI_ACCUM, c_init=c0)[0], want + c0, rel=1e-4, what="TN ACCUM")
+    assert_close(_raw_gemm(B, ffi.GEMM_NT, a, b, M, N, K, ffi.BF16, ffi.F32, ffi.EPI_RESIDUAL, aux=c0)[0], want + c0, rel=1e-4, what="RESIDUAL")
+    got, pre = _raw_gemm(B, ffi.GEMM_NT, a, b, M, N, K, ffi.BF16, ffi.BF16, ffi.EPI_GELU)
+    assert_close(pre, want, rel=2.0 ** -7, what="GELU.pre")
+    w32 = want.astype(np.float32)
+    assert_close(got, O.gelu(orc(w32)).data.reshape(M, N), rel=2.0 ** -7, what="GELU")
+    pre_act = _bf16_round(rs.randn(M, N).astype(np.float32))[0]
+    gb = ref.gelu_backward(orc(pre_act), orc(w32), fused=True).data.reshape(M, N)
+    assert_close(_raw_gemm(B, ffi.GEMM_NN, a, bt, M, N, K, ffi.BF16, ffi.BF16, ffi.EPI_GELU_BWD, aux=pre_act)[0], gb, rel=2.0 ** -7, what="GELU_BWD")
