@@ -95,6 +95,9 @@ SIGNATURES = {
     "ah_cross_entropy": [u64, i32, u64, u64, u64, i64, i64],
     "ah_cross_entropy_bwd": [u64, i32, u64, u64, u64, f32, u64, i64, i64],
     "ah_gemm": [C.POINTER(AhGemm)],
+    "ah_gemm_grouped_plan": [C.POINTER(AhGemm), C.c_int32, C.POINTER(C.c_uint64)],
+    "ah_gemm_grouped_run": [u64, i32],
+    "ah_gemm_grouped_destroy": [u64],
     "ah_gemm_last_kernel": [C.c_char_p, C.c_int32, C.POINTER(C.c_int32)],
     "ah_flash_fwd": [C.POINTER(AhFlash)], "ah_flash_bwd": [C.POINTER(AhFlash)],
     "ah_adamw": [u64, u64, u64, u64, u64, C.POINTER(AhAdamW), u64, u64, u64],

@@ -6,6 +6,7 @@
 // accumulation and the GELU derivative.
 #include "gemm_common.h"
 #include <cstdarg>
+#include <vector>
 #include <cstdio>
 
 using namespace ah;
@@ -304,7 +305,76 @@ void note_gemm_kernel(const char *fmt, ...) {
 void note_gemm_split(int nsplit) { g_last_split = nsplit; }
 }  // namespace ah
 
+namespace {
+struct GroupPlan { ah_ptr table; int count, blocks, layout, out_dtype; bool live; };
+std::vector<GroupPlan> g_plans;      // plan id = index + 1
+}  // namespace
+
 extern "C" {
+
+int32_t ah_gemm_grouped_plan(const AhGemm *descs, int32_t count, uint64_t *plan_out) {
+  AH_REQUIRE_READY();
+  AH_ARG(descs != nullptr && plan_out != nullptr && count > 0 && count <= 4096, "ah_gemm_grouped_plan: bad descriptor list (count %d)", count);
+  std::vector<GemmGroupEntry> tab((size_t)count);
+  int64_t blocks = 0;
+  const int layout = descs[0].layout, out_dtype = descs[0].out_dtype;
+  AH_ARG(layout >= AH_GEMM_NN && layout <= AH_GEMM_TN, "ah_gemm_grouped_plan: bad layout %d", layout);
+  AH_ARG(out_dtype == AH_F32 || out_dtype == AH_BF16, "ah_gemm_grouped_plan: output must be f32 or bf16");
+  const bool akm = layout == AH_GEMM_TN, bkm = layout != AH_GEMM_NT;
+  const int osz = out_dtype == AH_F32 ? 4 : 2;
+  for (int i = 0; i < count; i++) {
+    const AhGemm &q = descs[i];
+    if (q.layout != layout || q.out_dtype != out_dtype || q.in_dtype != AH_BF16 || q.batch != 1 ||
+        (q.epilogue != AH_EPI_NONE && q.epilogue != AH_EPI_ACCUM))
+      return fail(AH_ERR_UNSUPPORTED, "ah_gemm_grouped_plan: problem %d: a group shares one layout and output type, takes bf16 operands, "
+                                      "batch 1 and the NONE / ACCUM epilogues", i);
+    AH_ARG(q.m > 0 && q.n > 0 && q.k >= 64 && q.k % 64 == 0 && q.m < (1ll << 31) && q.n < (1ll << 31) && q.k < (1ll << 31),
+           "ah_gemm_grouped_plan: problem %d: extents m=%lld n=%lld k=%lld (k must be a positive multiple of 64)", i, (long long)q.m,
+           (long long)q.n, (long long)q.k);
+    AH_ARG(q.a != 0 && q.b != 0 && q.c != 0, "ah_gemm_grouped_plan: problem %d: null operand", i);
+    int64_t a_cols = akm ? q.m : q.k, b_cols = bkm ? q.n : q.k;
+    AH_ARG(q.lda >= a_cols && q.ldb >= b_cols && q.ldc >= q.n, "matmul shape mismatch: problem %d: lda/ldb/ldc too small", i);
+    bool ok = aligned16(q.a) && aligned16(q.b) && q.lda % 8 == 0 && q.ldb % 8 == 0 && (!akm || q.m % 8 == 0) && (!bkm || q.n % 8 == 0) &&
+              (q.c % (4 * osz)) == 0 && q.ldc % 4 == 0;
+    AH_ARG(ok, "ah_gemm_grouped_plan: problem %d: operands need 16-byte aligned rows and a vector-aligned C", i);
+    int64_t a_span = (akm ? (int64_t)64 : q.m) * q.lda * 2, b_span = (bkm ? (int64_t)64 : q.n) * q.ldb * 2;
+    AH_ARG(a_span < (1ll << 32) && b_span < (1ll << 32), "ah_gemm_grouped_plan: problem %d: operand spans more than 4 GiB", i);
+    GemmGroupEntry &e = tab[(size_t)i];
+    e.a = dp<const void>(q.a); e.b = dp<const void>(q.b); e.c = dp<void>(q.c);
+    e.M = (int)q.m; e.N = (int)q.n; e.K = (int)q.k; e.tile_start = (int)blocks;
+    e.lda = q.lda; e.ldb = q.ldb; e.ldc = q.ldc;
+    blocks += cdiv(q.m, 256) * cdiv(q.n, 256);
+    AH_ARG(blocks < (1ll << 31), "ah_gemm_grouped_plan: too many tiles");
+  }
+  ah_ptr table = 0;
+  int32_t rc = ah_alloc(tab.size() * sizeof(GemmGroupEntry), &table);
+  if (rc) return rc;
+  rc = ah_upload(table, tab.data(), tab.size() * sizeof(GemmGroupEntry));
+  if (rc) { ah_free(table); return rc; }
+  g_plans.push_back(GroupPlan{table, count, (int)blocks, layout, out_dtype, true});
+  *plan_out = g_plans.size();
+  return AH_OK;
+}
+
+int32_t ah_gemm_grouped_run(uint64_t plan, int32_t epilogue) {
+  AH_REQUIRE_READY();
+  AH_ARG(plan >= 1 && plan <= g_plans.size() && g_plans[plan - 1].live, "ah_gemm_grouped_run: unknown plan %llu", (unsigned long long)plan);
+  const GroupPlan &p = g_plans[plan - 1];
+  AH_ARG(epilogue == AH_EPI_NONE || (epilogue == AH_EPI_ACCUM && p.out_dtype == AH_F32), "ah_gemm_grouped_run: epilogue %d is not provided for this plan", epilogue);
+  const GemmGroupEntry *tab = dp<const GemmGroupEntry>(p.table);
+  switch (p.layout) {
+    case AH_GEMM_NT: return gemm_bf16_dma_nt_grouped(tab, p.count, p.blocks, epilogue, p.out_dtype);
+    case AH_GEMM_NN: return gemm_bf16_dma_nn_grouped(tab, p.count, p.blocks, epilogue, p.out_dtype);
+    default: return gemm_bf16_dma_tn_grouped(tab, p.count, p.blocks, epilogue, p.out_dtype);
+  }
+}
+
+int32_t ah_gemm_grouped_destroy(uint64_t plan) {
+  AH_REQUIRE_READY();
+  AH_ARG(plan >= 1 && plan <= g_plans.size() && g_plans[plan - 1].live, "ah_gemm_grouped_destroy: unknown plan %llu", (unsigned long long)plan);
+  g_plans[plan - 1].live = false;
+  return ah_free(g_plans[plan - 1].table);
+}
 
 int32_t ah_gemm_last_kernel(char *name, int32_t capacity, int32_t *nsplit) {
   AH_ARG(name != nullptr && capacity > 0, "ah_gemm_last_kernel: no output buffer");

@@ -4,6 +4,14 @@
 
 namespace ah {
 
+// One problem of a grouped launch (device-resident table; see ah_gemm_grouped_plan).
+struct GemmGroupEntry {
+  const void *a, *b;
+  void *c;
+  int M, N, K, tile_start;      // tile_start: first block id of this problem
+  int64_t lda, ldb, ldc;
+};
+
 // Records which kernel ah_gemm launched last (read back by ah_gemm_last_kernel).
 void note_gemm_kernel(const char *fmt, ...);
 void note_gemm_split(int nsplit);
@@ -90,5 +98,8 @@ int32_t gemm_bf16_direct(const GemmArgs &ga, int layout, int batch, int out_dtyp
 int32_t gemm_bf16_dma_nt(const GemmArgs &ga, int batch, int out_dtype);
 int32_t gemm_bf16_dma_nn(const GemmArgs &ga, int batch, int out_dtype);
 int32_t gemm_bf16_dma_tn(const GemmArgs &ga, int batch, int out_dtype);
+int32_t gemm_bf16_dma_nt_grouped(const GemmGroupEntry *tab, int count, int blocks, int epi, int out_dtype);
+int32_t gemm_bf16_dma_nn_grouped(const GemmGroupEntry *tab, int count, int blocks, int epi, int out_dtype);
+int32_t gemm_bf16_dma_tn_grouped(const GemmGroupEntry *tab, int count, int blocks, int epi, int out_dtype);
 
 }  // namespace ah

@@ -105,13 +105,57 @@ class FusedTrainer:
         self.hact = [a(BT * Fd * 2) for _ in range(self.L)]
         self.lnf, self.logits, self.rowlse = a(BT * Cc * 2), a(BT * V * 2), a(BT * 4)
         self.dx = [a(BT * Cc * 4), a(BT * Cc * 4)]
-        self.dxb, self.dlnb, self.datt = a(BT * Cc * 2), a(BT * Cc * 2), a(BT * Cc * 2)
-        self.dh, self.dqkv = a(BT * Fd * 2), a(BT * 3 * Cc * 2)
+        self.dlnb, self.datt = a(BT * Cc * 2), a(BT * Cc * 2)
+        # Output gradients of the four linears are kept per layer (bf16): every weight gradient dW = dY^T X of the step is
+        # computed at the end of backward by ONE grouped GEMM launch over full K = tokens, instead of 4 small split-K
+        # GEMMs per layer.  dy_fc2[l] = grad of the layer's output, dy_wo[l] = grad after the MLP branch joins.
+        self.dy_fc2 = [a(BT * Cc * 2) for _ in range(self.L)]
+        self.dy_wo = [a(BT * Cc * 2) for _ in range(self.L)]
+        self.dh = [a(BT * Fd * 2) for _ in range(self.L)]
+        self.dqkv = [a(BT * 3 * Cc * 2) for _ in range(self.L)]
+        self.dxb0 = a(BT * Cc * 2)                # grad of the embedding output in bf16 (written by the last LayerNorm backward, unused)
         self.loss, self.sumsq, self.clip = a(4), a(4), a(8)
         self.hyper = a(ffi.C.sizeof(ffi.AhAdamW))
         self.loss_hist_cap = 4096
         self.loss_hist, self.norm_hist = a(self.loss_hist_cap * 4), a(self.loss_hist_cap * 8)
         self._batches: List[Tuple[int, int]] = []
+        self._plan_weight_grads()
+
+    def _plan_weight_grads(self):
+        """Descriptors of every dW = dY^T X of the step (TN layout: both operands token-major), lmHead first."""
+        BT, Cc, Fd, V, TN = self.BT, self.C, self.F, self.V, ffi.GEMM_TN
+
+        def desc(dy, x, gname, m, n):
+            return ffi.AhGemm(TN, BF16, F32, ffi.EPI_NONE, m, n, BT, m, n, n, 1, 0, 0, 0, dy, x, self.g(gname), 0)
+        descs = [desc(self.logits, self.lnf, "lmHead", V, Cc)]
+        for l in range(self.L):
+            pre = f"layer.{l}."
+            descs += [desc(self.dy_fc2[l], self.hact[l], pre + "mlp.fc2", Cc, Fd), desc(self.dh[l], self.ln2[l], pre + "mlp.fc1", Fd, Cc),
+                      desc(self.dy_wo[l], self.att[l], pre + "attn.wo", Cc, Cc), desc(self.dqkv[l], self.ln1[l], pre + "attn.wqkv", 3 * Cc, Cc)]
+        self._dw_descs = descs
+        self._dw_flops = sum(2.0 * d.m * d.n * d.k for d in descs)
+        self._dw_plan = None
+        if BT % 64 == 0:                          # the grouped kernel contracts in k-tiles of 64 tokens
+            arr = (ffi.AhGemm * len(descs))(*descs)
+            plan = C.c_uint64()
+            check(self.lib.ah_gemm_grouped_plan(arr, len(descs), C.byref(plan)))
+            self._dw_plan = plan.value
+
+    def _weight_grads(self, epilogue: int):
+        if self._dw_plan is None:                 # odd token counts: one general GEMM per weight
+            for d in self._dw_descs:
+                self._gemm(d.layout, d.a, d.b, d.c, d.m, d.n, d.k, d.lda, d.ldb, d.ldc, F32, epilogue)
+            return
+        if self._timed is None:
+            check(self.lib.ah_gemm_grouped_run(self._dw_plan, epilogue))
+            return
+        e0, e1 = self.B._event(), self.B._event()
+        check(self.lib.ah_event_record(e0))
+        check(self.lib.ah_gemm_grouped_run(self._dw_plan, epilogue))
+        check(self.lib.ah_event_record(e1))
+        kernel, nsplit = self.B.lastGemmKernel()
+        self._timed.append({"kind": "gemm", "kernel": kernel, "nsplit": nsplit, "layout": ffi.GEMM_TN, "m": 0, "n": 0, "k": self.BT,
+                            "flops": self._dw_flops, "e0": e0, "e1": e1})
 
     # ------------------------------------------------------------------ helpers
     def _alloc(self, nbytes: int) -> int:
@@ -150,7 +194,7 @@ class FusedTrainer:
         q = self.qkv[l]
         f.q, f.k, f.v, f.o, f.lse = q, q + Cc * 2, q + 2 * Cc * 2, self.att[l], self.lse[l]
         if bwd:
-            d = self.dqkv
+            d = self.dqkv[l]
             f.d_o, f.dq, f.dk, f.dv = self.datt, d, d + Cc * 2, d + 2 * Cc * 2
         t0 = None
         if self._timed is not None:
@@ -185,29 +229,25 @@ class FusedTrainer:
         check(lib.ah_cross_entropy_bwd(self.logits, BF16, self.tgt, self.rowlse, 0, 1.0, self.logits, BT, V))     # dlogits in place
 
         self._gemm(NN, self.logits, self.p("lmHead", True), self.dlnb, BT, Cc, V, V, Cc, Cc)
-        self._gemm(TN, self.logits, self.lnf, self.g("lmHead"), V, Cc, BT, V, Cc, Cc, F32, wepi)
         cur = 0
-        check(lib.ah_layernorm_bwd(self.x[L], self.p("lnF.weight"), self.dlnb, BF16, 0, self.dx[cur], self.dxb, self.g("lnF.weight"),
+        check(lib.ah_layernorm_bwd(self.x[L], self.p("lnF.weight"), self.dlnb, BF16, 0, self.dx[cur], self.dy_fc2[L - 1], self.g("lnF.weight"),
                                    self.g("lnF.bias"), BT, Cc, 1e-5, acc))
         for l in reversed(range(L)):
             pre = f"layer.{l}."
             # MLP: x_out = x_mid + fc2(gelu(fc1(ln2(x_mid))))
-            self._gemm(NN, self.dxb, self.p(pre + "mlp.fc2", True), self.dh, BT, Fd, Cc, Cc, Fd, Fd, BF16, ffi.EPI_GELU_BWD, self.hpre[l])
-            self._gemm(TN, self.dxb, self.hact[l], self.g(pre + "mlp.fc2"), Cc, Fd, BT, Cc, Fd, Fd, F32, wepi)
-            self._gemm(NN, self.dh, self.p(pre + "mlp.fc1", True), self.dlnb, BT, Cc, Fd, Fd, Cc, Cc)
-            self._gemm(TN, self.dh, self.ln2[l], self.g(pre + "mlp.fc1"), Fd, Cc, BT, Fd, Cc, Cc, F32, wepi)
-            check(lib.ah_layernorm_bwd(self.xmid[l], self.p(pre + "ln2.weight"), self.dlnb, BF16, self.dx[cur], self.dx[cur ^ 1], self.dxb,
+            self._gemm(NN, self.dy_fc2[l], self.p(pre + "mlp.fc2", True), self.dh[l], BT, Fd, Cc, Cc, Fd, Fd, BF16, ffi.EPI_GELU_BWD, self.hpre[l])
+            self._gemm(NN, self.dh[l], self.p(pre + "mlp.fc1", True), self.dlnb, BT, Cc, Fd, Fd, Cc, Cc)
+            check(lib.ah_layernorm_bwd(self.xmid[l], self.p(pre + "ln2.weight"), self.dlnb, BF16, self.dx[cur], self.dx[cur ^ 1], self.dy_wo[l],
                                        self.g(pre + "ln2.weight"), self.g(pre + "ln2.bias"), BT, Cc, 1e-5, acc))
             cur ^= 1
             # attention: x_mid = x_in + wo(attn(wqkv(ln1(x_in))))
-            self._gemm(NN, self.dxb, self.p(pre + "attn.wo", True), self.datt, BT, Cc, Cc, Cc, Cc, Cc)
-            self._gemm(TN, self.dxb, self.att[l], self.g(pre + "attn.wo"), Cc, Cc, BT, Cc, Cc, Cc, F32, wepi)
+            self._gemm(NN, self.dy_wo[l], self.p(pre + "attn.wo", True), self.datt, BT, Cc, Cc, Cc, Cc, Cc)
             self._flash(l, True)
-            self._gemm(NN, self.dqkv, self.p(pre + "attn.wqkv", True), self.dlnb, BT, Cc, 3 * Cc, 3 * Cc, Cc, Cc)
-            self._gemm(TN, self.dqkv, self.ln1[l], self.g(pre + "attn.wqkv"), 3 * Cc, Cc, BT, 3 * Cc, Cc, Cc, F32, wepi)
-            check(lib.ah_layernorm_bwd(self.x[l], self.p(pre + "ln1.weight"), self.dlnb, BF16, self.dx[cur], self.dx[cur ^ 1], self.dxb,
-                                       self.g(pre + "ln1.weight"), self.g(pre + "ln1.bias"), BT, Cc, 1e-5, acc))
+            self._gemm(NN, self.dqkv[l], self.p(pre + "attn.wqkv", True), self.dlnb, BT, Cc, 3 * Cc, 3 * Cc, Cc, Cc)
+            check(lib.ah_layernorm_bwd(self.x[l], self.p(pre + "ln1.weight"), self.dlnb, BF16, self.dx[cur], self.dx[cur ^ 1],
+                                       self.dy_fc2[l - 1] if l > 0 else self.dxb0, self.g(pre + "ln1.weight"), self.g(pre + "ln1.bias"), BT, Cc, 1e-5, acc))
             cur ^= 1
+        self._weight_grads(wepi)
         check(lib.ah_embedding_bwd(self.tok, self.dx[cur], self.g("wte"), BT, Cc, V, acc))
         check(lib.ah_pos_embedding_bwd(self.dx[cur], self.g("wpe"), self.batch, self.T, Cc, acc))
 
@@ -355,6 +395,9 @@ class FusedTrainer:
         if self._graph is not None:
             check(self.lib.ah_graph_destroy(self._graph))
             self._graph = None
+        if self._dw_plan is not None:
+            check(self.lib.ah_gemm_grouped_destroy(self._dw_plan))
+            self._dw_plan = None
         for b in self._bufs:
             self.lib.ah_free(b)
         self._bufs = []

@@ -224,6 +224,16 @@ typedef struct {
   ah_ptr  a, b, c, aux;
 } AhGemm;
 int32_t ah_gemm(const AhGemm *g);
+/* Grouped GEMM: several independent problems of ONE layout in one launch (256x256 tiles of all problems share the
+ * grid, so small outputs with a long contraction fill the chip without split-K).  Used for the weight gradients
+ * dW_i = G_i^T X_i of all layers at the end of backward; the reference computes them one matmul at a time
+ * (packages/autograd/src/ops.ts:197-234).  Requirements per problem: bf16 operands, batch 1, k a multiple of 64,
+ * 16-byte aligned rows, epilogue NONE or ACCUM; all problems share layout and output type.  The plan copies the
+ * descriptors to the device once; ah_gemm_grouped_run only launches (safe inside graph capture) and takes the
+ * epilogue (AH_EPI_NONE, or AH_EPI_ACCUM for f32 outputs) so one plan serves first and later micro-batches. */
+int32_t ah_gemm_grouped_plan(const AhGemm *descs, int32_t count, uint64_t *plan_out);
+int32_t ah_gemm_grouped_run(uint64_t plan, int32_t epilogue);
+int32_t ah_gemm_grouped_destroy(uint64_t plan);
 /* Profiling aid (no counterpart in the reference): writes the name of the kernel the most recent ah_gemm call
  * launched, spelled as a profiler demangles it (e.g. "k_gemm_bf16<256, 256, 2, 4, false, false>"), and the number
  * of split-K slices it used (1 = none; > 1 means a k_splitk_reduce launch followed). */

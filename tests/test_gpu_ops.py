@@ -533,3 +533,38 @@ def test_gemm_bf16_large_tiles_direct_to_lds_kernel(B, K):
     pre_act = _bf16_round(rs.randn(M, N).astype(np.float32))[0]
     gb = ref.gelu_backward(orc(pre_act), orc(w32), fused=True).data.reshape(M, N)
     assert_close(_raw_gemm(B, ffi.GEMM_NN, a, bt, M, N, K, ffi.BF16, ffi.BF16, ffi.EPI_GELU_BWD, aux=pre_act)[0], gb, rel=2.0 ** -7, what="GELU_BWD")
+
+
+def test_gemm_grouped_matches_separate_products(B):
+    """One grouped launch over problems of different sizes (ragged tile edges, NONE then ACCUM) against float64 numpy
+    products of the same bf16-exact operands; descriptor errors are reported, not launched."""
+    import ctypes as C
+    from alpha2_amd import TensorData, _ffi as ffi
+    K = 640
+    shapes = [(768, 768), (264, 520), (2304, 768), (8, 8), (1000, 256)]
+    keep, descs, wants, outs = [], [], [], []
+    for m, n in shapes:
+        gy, x = _bf16_round(rs.randn(K, m).astype(np.float32))[0], _bf16_round(rs.randn(K, n).astype(np.float32))[0]
+        tg, tx = TensorData(gy.shape, "f16", _bf16_round(gy)[1]), TensorData(x.shape, "f16", _bf16_round(x)[1])
+        out = B.zeros((m, n))
+        keep += [tg, tx]
+        outs.append(out)
+        wants.append(gy.astype(np.float64).T @ x.astype(np.float64))
+        descs.append(ffi.AhGemm(ffi.GEMM_TN, ffi.BF16, ffi.F32, ffi.EPI_NONE, m, n, K, m, n, n, 1, 0, 0, 0, B._ptr(tg), B._ptr(tx), B._ptr(out), 0))
+    arr = (ffi.AhGemm * len(descs))(*descs)
+    plan = C.c_uint64()
+    ffi.check(B.lib.ah_gemm_grouped_plan(arr, len(descs), C.byref(plan)))
+    ffi.check(B.lib.ah_gemm_grouped_run(plan.value, ffi.EPI_NONE))
+    assert B.lastGemmKernel()[0].startswith("k_gemm_bf16_dma_grouped<true, true")
+    for out, want, (m, n) in zip(outs, wants, shapes):
+        B._dirty(out)
+        assert_close(out.data.reshape(m, n), want, rel=1e-4, what=f"grouped NONE {m}x{n}")
+    ffi.check(B.lib.ah_gemm_grouped_run(plan.value, ffi.EPI_ACCUM))
+    for out, want, (m, n) in zip(outs, wants, shapes):
+        B._dirty(out)
+        assert_close(out.data.reshape(m, n), 2 * want, rel=1e-4, what=f"grouped ACCUM {m}x{n}")
+    assert B.lib.ah_gemm_grouped_run(plan.value, ffi.EPI_GELU) != 0 and b"not provided" in B.lib.ah_last_error()
+    ffi.check(B.lib.ah_gemm_grouped_destroy(plan.value))
+    assert B.lib.ah_gemm_grouped_run(plan.value, ffi.EPI_NONE) != 0 and b"unknown plan" in B.lib.ah_last_error()
+    bad = (ffi.AhGemm * 1)(ffi.AhGemm(ffi.GEMM_TN, ffi.BF16, ffi.F32, ffi.EPI_NONE, 64, 64, 100, 64, 64, 64, 1, 0, 0, 0, 1 << 20, 1 << 20, 1 << 20, 0))
+    assert B.lib.ah_gemm_grouped_plan(bad, 1, C.byref(plan)) != 0 and b"multiple of 64" in B.lib.ah_last_error()
