@@ -232,12 +232,22 @@ int32_t launch(const GemmArgs &ga, int batch, int out_dtype) {
 
 template <bool AKM, bool BKM>
 int32_t run(const GemmArgs &ga, int batch, int out_dtype) {
-  // Outputs with at least one 256x256 tile per CU go to the kernel fed by global->LDS loads (gemm_bf16_dma.inc): half
-  // the L2 traffic and a third of the LDS traffic per flop of the 128x128 tile.  Smaller outputs keep the 128x128 tile
-  // of this file, two blocks per CU.
-  int64_t big_blocks = cdiv(ga.M, 256) * cdiv(ga.N, 256) * batch * ga.nsplit;
-  bool big = ga.M >= 256 && ga.N >= 256 && big_blocks >= num_cus();
-  if (big) return AKM ? gemm_bf16_dma_tn(ga, batch, out_dtype) : BKM ? gemm_bf16_dma_nn(ga, batch, out_dtype) : gemm_bf16_dma_nt(ga, batch, out_dtype);
+  // Large outputs go to the kernel fed by global->LDS loads (gemm_bf16_dma.inc): half the L2 traffic and a third of the
+  // LDS traffic per flop of the 128x128 tile.  It holds one block per CU, so what matters is how evenly the tiles fill
+  // whole rounds of CUs: take 256 x 256 or 256 x 192 tiles, whichever wastes less of its last round, and keep the
+  // 128x128 tile of this file (two blocks per CU, finer grain) when neither fills 70 %.
+  if (ga.M >= 256 && ga.N >= 192) {
+    const int64_t cus = num_cus(), per = (int64_t)batch * ga.nsplit;
+    auto fill = [&](int bn) {
+      int64_t t = cdiv(ga.M, 256) * cdiv(ga.N, bn) * per;
+      double useful = (double)ga.N / (double)(cdiv(ga.N, bn) * bn);        // columns of edge tiles that exist
+      return useful * (double)t / (double)(cdiv(t, cus) * cus);
+    };
+    double f256 = ga.N >= 256 ? fill(256) : 0.0, f192 = 0.97 * fill(192);
+    int bn = f256 >= f192 ? 256 : 192;
+    if ((bn == 256 ? f256 : f192) >= 0.7)
+      return AKM ? gemm_bf16_dma_tn(ga, batch, out_dtype, bn) : BKM ? gemm_bf16_dma_nn(ga, batch, out_dtype, bn) : gemm_bf16_dma_nt(ga, batch, out_dtype, bn);
+  }
   return launch<128, 128, 2, 2, AKM, BKM>(ga, batch, out_dtype);
 }
 

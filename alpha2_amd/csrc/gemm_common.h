@@ -94,10 +94,11 @@ __device__ __forceinline__ void store_tiles(const GemmArgs &g, int64_t cbase, in
 
 // gemm_bf16.hip
 int32_t gemm_bf16_direct(const GemmArgs &ga, int layout, int batch, int out_dtype);
-// gemm_bf16_dma_{nt,nn,tn}.hip: 256x256 tiles fed by direct global->LDS loads (same preconditions as the direct kernel)
-int32_t gemm_bf16_dma_nt(const GemmArgs &ga, int batch, int out_dtype);
-int32_t gemm_bf16_dma_nn(const GemmArgs &ga, int batch, int out_dtype);
-int32_t gemm_bf16_dma_tn(const GemmArgs &ga, int batch, int out_dtype);
+// gemm_bf16_dma_{nt,nn,tn}.hip: 256 x bn tiles (bn = 256 or 192) fed by direct global->LDS loads (same preconditions as the
+// direct kernel)
+int32_t gemm_bf16_dma_nt(const GemmArgs &ga, int batch, int out_dtype, int bn);
+int32_t gemm_bf16_dma_nn(const GemmArgs &ga, int batch, int out_dtype, int bn);
+int32_t gemm_bf16_dma_tn(const GemmArgs &ga, int batch, int out_dtype, int bn);
 int32_t gemm_bf16_dma_nt_grouped(const GemmGroupEntry *tab, int count, int blocks, int epi, int out_dtype);
 int32_t gemm_bf16_dma_nn_grouped(const GemmGroupEntry *tab, int count, int blocks, int epi, int out_dtype);
 int32_t gemm_bf16_dma_tn_grouped(const GemmGroupEntry *tab, int count, int blocks, int epi, int out_dtype);

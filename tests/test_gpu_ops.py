@@ -502,23 +502,22 @@ def test_flash_attention_bf16_vs_materialised(B, BH, T, D, cap):
     assert_close(g["dV"].data, dv, rel=rel, what="flash16.dV", **loose(dv))
 
 
-@pytest.mark.parametrize("K", [64, 192, 512])
-def test_gemm_bf16_large_tiles_direct_to_lds_kernel(B, K):
+@pytest.mark.parametrize("M,N,K,tile", [(4000, 4072, 64, 4), (4000, 4072, 192, 4), (4000, 4072, 512, 4), (16376, 760, 128, 3), (8192, 1536, 320, 3)])
+def test_gemm_bf16_large_tiles_direct_to_lds_kernel(B, M, N, K, tile):
     """Outputs with at least one 256x256 tile per CU take the kernel fed by global->LDS loads; edges in M and N, odd and
     even k-tile counts, every layout and epilogue.  At this size the check is a float64 numpy product of the same
     bf16-exact operands (the C oracle covers the small shapes above); fp32 accumulation of exact products."""
     from alpha2_amd import _ffi as ffi
-    M, N = 4000, 4072          # 16 x 16 tiles of 256, ragged edges, N % 8 == 0 and M % 8 == 0 for the k-major layouts
+    # ragged edges with N % 8 == 0 and M % 8 == 0 (needed by the k-major layouts); `tile` = expected column tile / 64:
+    # 256 x 256 tiles, or 256 x 192 where those fill whole rounds of CUs better (N = 760, 1536)
     a, b = _bf16_round(rs.randn(M, K).astype(np.float32))[0], _bf16_round(rs.randn(N, K).astype(np.float32))[0]
     want = a.astype(np.float64) @ b.astype(np.float64).T
     at, bt = np.ascontiguousarray(a.T), np.ascontiguousarray(b.T)
 
-    def used_dma():
-        name, _ = B.lastGemmKernel()
-        return name.startswith("k_gemm_bf16_dma")
     got = _raw_gemm(B, ffi.GEMM_NT, a, b, M, N, K, ffi.BF16, ffi.F32)[0]
-    if B.getDeviceInfo()["computeUnits"] <= 256:
-        assert used_dma(), B.lastGemmKernel()
+    if B.getDeviceInfo()["computeUnits"] == 256:
+        name = B.lastGemmKernel()[0]
+        assert name.startswith("k_gemm_bf16_dma<") and name.endswith(f", {tile}>"), name
     assert_close(got, want, rel=1e-4, what="NT f32")
     assert_close(_raw_gemm(B, ffi.GEMM_NT, a, b, M, N, K, ffi.BF16, ffi.BF16)[0], want, rel=2.0 ** -7, what="NT bf16")
     assert_close(_raw_gemm(B, ffi.GEMM_NN, a, bt, M, N, K, ffi.BF16, ffi.F32)[0], want, rel=1e-4, what="NN")
