@@ -107,8 +107,11 @@ __device__ __forceinline__ void store_rows(uint16_t *__restrict__ dst, const f32
 }
 
 // ------------------------------------------------------------------------------------------ forward
+// Launch bounds ask for at least two (three) waves per SIMD at head sizes up to 64: besides the occupancy this keeps the
+// register budget at 256 (170), where the compiler uses the VGPR form of MFMA and no accumulator ever has to be copied
+// between AGPRs and VGPRs for the softmax arithmetic.
 template <int D, bool CAPPED>
-__global__ __launch_bounds__(256) void k_flash_fwd_bf16(FlashArgs a) {
+__global__ __launch_bounds__(256, D <= 64 ? 3 : 1) void k_flash_fwd_bf16(FlashArgs a) {
   constexpr int DB = D / 32, KS = D / 16;
   __shared__ __attribute__((aligned(16))) uint16_t Ks[2][Geo<D>::ELEMS], Vs[2][Geo<D>::ELEMS];
   int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
@@ -120,7 +123,7 @@ __global__ __launch_bounds__(256) void k_flash_fwd_bf16(FlashArgs a) {
   const uint16_t *V = (const uint16_t *)a.v + b * a.v_sb + h * a.v_sh;
   // CAPPED: u2 = s*c1 = 2*score/cap in base 2; p = 2^(c2*r).  Otherwise x = s*c1 = score in base 2.
   const float c1 = CAPPED ? 2.0f * a.scale * LOG2E / a.cap : a.scale * LOG2E;
-  const float c2 = -2.0f * a.cap * LOG2E;
+  const float ic2 = CAPPED ? -1.0f / (2.0f * a.cap * LOG2E) : 0.f;      // 1 / c2, c2 = -2 cap log2(e): p = 2^(c2 r)
 
   bf16x8 qf[KS];
   row_frags<D>(Q, a.q_st, qi, qi < a.T, lane, qf);
@@ -129,9 +132,15 @@ __global__ __launch_bounds__(256) void k_flash_fwd_bf16(FlashArgs a) {
   for (int d = 0; d < DB; d++)
 #pragma unroll
     for (int e = 0; e < 16; e++) o[d][e] = 0.f;
-  // CAPPED: l and l_rnd are this half-wave's partial row sums of the probabilities as computed (for LSE, which the backward
-  // kernels use to rebuild them) and as rounded to bf16 for the MFMA (for normalising O); m is unused
+  // CAPPED: l is this half-wave's partial row sum of the probabilities as computed (for LSE, from which the backward
+  // kernels rebuild them); lacc accumulates the row sum of the probabilities as rounded to bf16 (for normalising O); m is unused
   float m = -INFINITY, l = 0.f, l_rnd = 0.f;
+  f32x16 lacc;
+  bf16x8 ones;
+#pragma unroll
+  for (int e = 0; e < 16; e++) lacc[e] = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; i++) ones[i] = (__bf16)1.0f;
 
   int kv_end = min(a.T, (qblk + 1) * 128);                         // causal: keys < kv_end
   int ntile = (kv_end + ST - 1) / ST;
@@ -160,10 +169,8 @@ __global__ __launch_bounds__(256) void k_flash_fwd_bf16(FlashArgs a) {
         const bool edge = kv0 + 31 > q0 || kv0 + 32 > a.T;         // wave-uniform: some score of the tile is masked
         if (CAPPED) {
 #pragma unroll
-          for (int e = 0; e < 16; e++) {
-            float r = rcp_fast(exp2_fast(s[e] * c1) + 1.0f);
-            s[e] = exp2_fast(c2 * r);
-          }
+          for (int e = 0; e < 16; e++)        // c2 r = c2 / (e + 1) = 1 / (e / c2 + 1 / c2): one fma feeds the reciprocal
+            s[e] = exp2_fast(rcp_fast(fmaf(exp2_fast(s[e] * c1), ic2, ic2)));
           if (edge) {
 #pragma unroll
             for (int e = 0; e < 16; e++) {
@@ -203,9 +210,10 @@ __global__ __launch_bounds__(256) void k_flash_fwd_bf16(FlashArgs a) {
         bf16x8 pb0 = acc_to_b(s, 0), pb1 = acc_to_b(s, 1);
         if (CAPPED) {
           // O is normalised by the sum of the bf16-rounded probabilities the MFMA sees (a row with a single key
-          // returns that key's V exactly)
-#pragma unroll
-          for (int i = 0; i < 8; i++) l_rnd += (float)pb0[i] + (float)pb1[i];
+          // returns that key's V exactly).  That sum is taken by the idle matrix pipe: a ones operand in place of V
+          // leaves sum_kv p[kv][q] in every row of the accumulator.
+          lacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones, pb0, lacc, 0, 0, 0);
+          lacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones, pb1, lacc, 0, 0, 0);
         }
 #pragma unroll
         for (int d = 0; d < DB; d++) {
@@ -220,7 +228,7 @@ __global__ __launch_bounds__(256) void k_flash_fwd_bf16(FlashArgs a) {
     }
     __syncthreads();
   }
-  if (CAPPED) { l += __shfl_xor(l, 32, 64); l_rnd += __shfl_xor(l_rnd, 32, 64); } else l_rnd = l;
+  if (CAPPED) { l += __shfl_xor(l, 32, 64); l_rnd = lacc[0]; } else l_rnd = l;
   if (qi < a.T) {
     float inv_l = l_rnd > 0.f ? 1.0f / l_rnd : 0.f;
     store_rows<D>((uint16_t *)a.o + b * a.o_sb + h * a.o_sh + (int64_t)qi * a.o_st, o, inv_l, lane);
@@ -248,7 +256,7 @@ __device__ __forceinline__ float score_bwd(float s, float dp, float krow, float 
 
 // ------------------------------------------------------------------------------------------ dQ (and delta)
 template <int D, bool CAPPED>
-__global__ __launch_bounds__(256) void k_flash_dq_bf16(FlashArgs a) {
+__global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void k_flash_dq_bf16(FlashArgs a) {
   constexpr int DB = D / 32, KS = D / 16;
   __shared__ __attribute__((aligned(16))) uint16_t Ks[2][Geo<D>::ELEMS], Vs[2][Geo<D>::ELEMS];
   int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
