@@ -16,7 +16,7 @@ ADD, SUB, MUL, DIV = 0, 1, 2, 3
 NEG, EXP, LOG, SQRT, POW, SCALE, CLAMP, GELU, RELU, SILU, SOFTCAP = range(11)
 GELU_BWD, RELU_BWD, SILU_BWD, CLAMP_BWD, SOFTCAP_BWD = range(5)
 GEMM_NN, GEMM_NT, GEMM_TN = 0, 1, 2
-EPI_NONE, EPI_ACCUM, EPI_GELU, EPI_RESIDUAL, EPI_GELU_BWD = range(5)
+EPI_NONE, EPI_ACCUM, EPI_GELU, EPI_RESIDUAL, EPI_GELU_BWD, EPI_GELU_GRAD, EPI_MUL_AUX = range(7)
 
 u64, i64, i32, f32 = C.c_uint64, C.c_int64, C.c_int32, C.c_float
 p_i64 = C.POINTER(C.c_int64)

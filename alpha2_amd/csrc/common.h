@@ -82,6 +82,13 @@ __device__ __forceinline__ float gelu_gate_r(float x) {
   return __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(u2) + 1.0f);
 }
 __device__ __forceinline__ float gelu_f(float x) { return x * (1.0f - gelu_gate_r(x)); }
+// value and derivative from one gate evaluation
+__device__ __forceinline__ void gelu_both_f(float x, float &val, float &grad) {
+  const float k = 0.7978845608028654f;
+  float r = gelu_gate_r(x), one_minus_r = 1.0f - r;
+  val = x * one_minus_r;
+  grad = one_minus_r * (1.0f + 2.0f * x * r * (k * (1.0f + 3.0f * 0.044715f * x * x)));
+}
 __device__ __forceinline__ float gelu_grad_f(float x) {
   const float k = 0.7978845608028654f;
   float r = gelu_gate_r(x);

@@ -266,6 +266,8 @@ int32_t run_bf16_nt(const GemmArgs &ga, int batch, int out_dtype, int vec_c) {
     case AH_EPI_ACCUM: return launch_bf16_nt_t<128, 128, 2, 2, AH_EPI_ACCUM, float>(ga, batch, vec_c);
     case AH_EPI_RESIDUAL: return launch_bf16_nt_t<128, 128, 2, 2, AH_EPI_RESIDUAL, float>(ga, batch, vec_c);
     case AH_EPI_GELU: return launch_bf16_nt_t<128, 128, 2, 2, AH_EPI_GELU, uint16_t>(ga, batch, vec_c);
+    case AH_EPI_GELU_GRAD: return launch_bf16_nt_t<128, 128, 2, 2, AH_EPI_GELU_GRAD, uint16_t>(ga, batch, vec_c);
+    case AH_EPI_MUL_AUX: return launch_bf16_nt_t<128, 128, 2, 2, AH_EPI_MUL_AUX, uint16_t>(ga, batch, vec_c);
     default: return launch_bf16_nt_t<128, 128, 2, 2, AH_EPI_GELU_BWD, uint16_t>(ga, batch, vec_c);
   }
 }
@@ -287,6 +289,8 @@ int32_t launch_f32(const GemmArgs &ga, int batch, int out_dtype, int vec_a, int 
     case AH_EPI_ACCUM: return launch_f32_t<LAYOUT, AH_EPI_ACCUM, float>(ga, batch, vec_a, vec_b, vec_c);
     case AH_EPI_GELU: return launch_f32_t<LAYOUT, AH_EPI_GELU, float>(ga, batch, vec_a, vec_b, vec_c);
     case AH_EPI_RESIDUAL: return launch_f32_t<LAYOUT, AH_EPI_RESIDUAL, float>(ga, batch, vec_a, vec_b, vec_c);
+    case AH_EPI_GELU_GRAD: return launch_f32_t<LAYOUT, AH_EPI_GELU_GRAD, float>(ga, batch, vec_a, vec_b, vec_c);
+    case AH_EPI_MUL_AUX: return launch_f32_t<LAYOUT, AH_EPI_MUL_AUX, float>(ga, batch, vec_a, vec_b, vec_c);
     default: return launch_f32_t<LAYOUT, AH_EPI_GELU_BWD, float>(ga, batch, vec_a, vec_b, vec_c);
   }
 }
@@ -390,7 +394,7 @@ int32_t ah_gemm(const AhGemm *p) {
   AH_ARG(q.layout >= AH_GEMM_NN && q.layout <= AH_GEMM_TN, "ah_gemm: bad layout %d", q.layout);
   AH_ARG(q.in_dtype == AH_F32 || q.in_dtype == AH_BF16, "ah_gemm: operands must be f32 or bf16");
   AH_ARG(q.out_dtype == AH_F32 || q.out_dtype == AH_BF16, "ah_gemm: output must be f32 or bf16");
-  AH_ARG(q.epilogue >= AH_EPI_NONE && q.epilogue <= AH_EPI_GELU_BWD, "ah_gemm: bad epilogue %d", q.epilogue);
+  AH_ARG(q.epilogue >= AH_EPI_NONE && q.epilogue <= AH_EPI_MUL_AUX, "ah_gemm: bad epilogue %d", q.epilogue);
   AH_ARG(q.m >= 0 && q.n >= 0 && q.k >= 0 && q.batch >= 0, "ah_gemm: negative extent");
   AH_ARG(q.m < (1ll << 31) && q.n < (1ll << 31) && q.k < (1ll << 31) && q.batch <= 65535, "ah_gemm: extent too large");
   if (q.m == 0 || q.n == 0 || q.batch == 0) return AH_OK;
@@ -400,11 +404,12 @@ int32_t ah_gemm(const AhGemm *p) {
   int64_t a_cols = q.layout == AH_GEMM_TN ? q.m : q.k, b_cols = q.layout == AH_GEMM_NT ? q.k : q.n;
   AH_ARG(q.lda >= a_cols && q.ldb >= b_cols && q.ldc >= q.n, "matmul shape mismatch: lda/ldb/ldc (%lld,%lld,%lld) too small for m=%lld n=%lld k=%lld",
          (long long)q.lda, (long long)q.ldb, (long long)q.ldc, (long long)q.m, (long long)q.n, (long long)q.k);
-  if (q.epilogue == AH_EPI_GELU || q.epilogue == AH_EPI_RESIDUAL || q.epilogue == AH_EPI_GELU_BWD)
+  const bool gelu_like = q.epilogue == AH_EPI_GELU || q.epilogue == AH_EPI_GELU_BWD || q.epilogue == AH_EPI_GELU_GRAD || q.epilogue == AH_EPI_MUL_AUX;
+  if (gelu_like || q.epilogue == AH_EPI_RESIDUAL)
     AH_ARG(q.aux != 0, "ah_gemm: epilogue %d needs aux", q.epilogue);
   // epilogue / output-type combinations: NONE -> f32 or bf16; ACCUM, RESIDUAL -> f32; GELU, GELU_BWD -> the operand type
   bool combo = q.epilogue == AH_EPI_NONE || ((q.epilogue == AH_EPI_ACCUM || q.epilogue == AH_EPI_RESIDUAL) && q.out_dtype == AH_F32) ||
-               ((q.epilogue == AH_EPI_GELU || q.epilogue == AH_EPI_GELU_BWD) && q.out_dtype == q.in_dtype);
+               (gelu_like && q.out_dtype == q.in_dtype);
   if (!combo) return fail(AH_ERR_UNSUPPORTED, "ah_gemm: epilogue %d with operands of dtype %d and output dtype %d is not provided", q.epilogue, q.in_dtype, q.out_dtype);
 
   GemmArgs ga;
@@ -421,7 +426,7 @@ int32_t ah_gemm(const AhGemm *p) {
   int osz = q.out_dtype == AH_F32 ? 4 : 2;
   int vec_c = ((q.c % (4 * osz)) == 0) && (q.ldc % 4 == 0) && (q.stride_c % 4 == 0);
   if (q.epilogue == AH_EPI_RESIDUAL) vec_c = vec_c && (q.aux % 16 == 0);
-  if (q.epilogue == AH_EPI_GELU || q.epilogue == AH_EPI_GELU_BWD) vec_c = vec_c && (q.aux % (4 * osz) == 0);
+  if (gelu_like) vec_c = vec_c && (q.aux % (4 * osz) == 0);
   if (q.in_dtype == AH_F32) {
     int vec_a = aligned16(q.a) && (q.lda % 4 == 0) && (q.stride_a % 4 == 0);
     int vec_b = aligned16(q.b) && (q.ldb % 4 == 0) && (q.stride_b % 4 == 0);

@@ -52,6 +52,19 @@ __device__ __forceinline__ void epilogue4(const GemmArgs &g, int64_t cbase, int 
              x[0] = bf16_bits_to_f32(o.x & 0xffff); x[1] = bf16_bits_to_f32(o.x >> 16); x[2] = bf16_bits_to_f32(o.y & 0xffff); x[3] = bf16_bits_to_f32(o.y >> 16); }
 #pragma unroll
       for (int i = 0; i < 4; i++) v[i] *= gelu_grad_f(x[i]);
+    } else if (EPI == AH_EPI_MUL_AUX) {
+      float x[4];
+      if (sizeof(OUT) == 4) { float4 o = *reinterpret_cast<const float4 *>((const float *)g.aux + idx); x[0] = o.x; x[1] = o.y; x[2] = o.z; x[3] = o.w; }
+      else { uint2 o = *reinterpret_cast<const uint2 *>((const uint16_t *)g.aux + idx);
+             x[0] = bf16_bits_to_f32(o.x & 0xffff); x[1] = bf16_bits_to_f32(o.x >> 16); x[2] = bf16_bits_to_f32(o.y & 0xffff); x[3] = bf16_bits_to_f32(o.y >> 16); }
+#pragma unroll
+      for (int i = 0; i < 4; i++) v[i] *= x[i];
+    } else if (EPI == AH_EPI_GELU_GRAD) {
+      float d[4];
+#pragma unroll
+      for (int i = 0; i < 4; i++) gelu_both_f(v[i], v[i], d[i]);
+      if (sizeof(OUT) == 4) *reinterpret_cast<float4 *>((float *)g.aux_out + idx) = make_float4(d[0], d[1], d[2], d[3]);
+      else *reinterpret_cast<uint2 *>((uint16_t *)g.aux_out + idx) = make_uint2(pack_bf16x2(d[0], d[1]), pack_bf16x2(d[2], d[3]));
     } else if (EPI == AH_EPI_GELU) {
       if (sizeof(OUT) == 4) *reinterpret_cast<float4 *>((float *)g.aux_out + idx) = make_float4(v[0], v[1], v[2], v[3]);
       else *reinterpret_cast<uint2 *>((uint16_t *)g.aux_out + idx) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
@@ -70,6 +83,8 @@ __device__ __forceinline__ void epilogue4(const GemmArgs &g, int64_t cbase, int 
       else if (EPI == AH_EPI_RESIDUAL) a += ((const float *)g.aux)[idx + i];
       else if (EPI == AH_EPI_GELU_BWD) a *= gelu_grad_f(Io<OUT>::ld((const OUT *)g.aux, idx + i));
       else if (EPI == AH_EPI_GELU) { Io<OUT>::st((OUT *)g.aux_out, idx + i, a); a = gelu_f(a); }
+      else if (EPI == AH_EPI_MUL_AUX) a *= Io<OUT>::ld((const OUT *)g.aux, idx + i);
+      else if (EPI == AH_EPI_GELU_GRAD) { float d; gelu_both_f(a, a, d); Io<OUT>::st((OUT *)g.aux_out, idx + i, d); }
       Io<OUT>::st(c, idx + i, a);
     }
   }

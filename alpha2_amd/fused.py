@@ -101,7 +101,7 @@ class FusedTrainer:
         self.att = [a(BT * Cc * 2) for _ in range(self.L)]
         self.lse = [a(batch * self.H * self.T * 4) for _ in range(self.L)]
         self.ln2 = [a(BT * Cc * 2) for _ in range(self.L)]
-        self.hpre = [a(BT * Fd * 2) for _ in range(self.L)]
+        self.hgrad = [a(BT * Fd * 2) for _ in range(self.L)]          # gelu'(fc1 output), saved by the forward epilogue
         self.hact = [a(BT * Fd * 2) for _ in range(self.L)]
         self.lnf, self.logits, self.rowlse = a(BT * Cc * 2), a(BT * V * 2), a(BT * 4)
         self.dx = [a(BT * Cc * 4), a(BT * Cc * 4)]
@@ -221,7 +221,7 @@ class FusedTrainer:
             self._flash(l, False)
             self._gemm(NT, self.att[l], self.p(pre + "attn.wo", True), self.xmid[l], BT, Cc, Cc, Cc, Cc, Cc, F32, ffi.EPI_RESIDUAL, self.x[l])
             check(lib.ah_layernorm(self.xmid[l], self.p(pre + "ln2.weight"), self.p(pre + "ln2.bias"), self.ln2[l], BT, Cc, 1e-5, BF16))
-            self._gemm(NT, self.ln2[l], self.p(pre + "mlp.fc1", True), self.hact[l], BT, Fd, Cc, Cc, Cc, Fd, BF16, ffi.EPI_GELU, self.hpre[l])
+            self._gemm(NT, self.ln2[l], self.p(pre + "mlp.fc1", True), self.hact[l], BT, Fd, Cc, Cc, Cc, Fd, BF16, ffi.EPI_GELU_GRAD, self.hgrad[l])
             self._gemm(NT, self.hact[l], self.p(pre + "mlp.fc2", True), self.x[l + 1], BT, Cc, Fd, Fd, Fd, Cc, F32, ffi.EPI_RESIDUAL, self.xmid[l])
         check(lib.ah_layernorm(self.x[L], self.p("lnF.weight"), self.p("lnF.bias"), self.lnf, BT, Cc, 1e-5, BF16))
         self._gemm(NT, self.lnf, self.p("lmHead", True), self.logits, BT, V, Cc, Cc, Cc, V)
@@ -235,7 +235,7 @@ class FusedTrainer:
         for l in reversed(range(L)):
             pre = f"layer.{l}."
             # MLP: x_out = x_mid + fc2(gelu(fc1(ln2(x_mid))))
-            self._gemm(NN, self.dy_fc2[l], self.p(pre + "mlp.fc2", True), self.dh[l], BT, Fd, Cc, Cc, Fd, Fd, BF16, ffi.EPI_GELU_BWD, self.hpre[l])
+            self._gemm(NN, self.dy_fc2[l], self.p(pre + "mlp.fc2", True), self.dh[l], BT, Fd, Cc, Cc, Fd, Fd, BF16, ffi.EPI_MUL_AUX, self.hgrad[l])
             self._gemm(NN, self.dh[l], self.p(pre + "mlp.fc1", True), self.dlnb, BT, Cc, Fd, Fd, Cc, Cc)
             check(lib.ah_layernorm_bwd(self.xmid[l], self.p(pre + "ln2.weight"), self.dlnb, BF16, self.dx[cur], self.dx[cur ^ 1], self.dy_wo[l],
                                        self.g(pre + "ln2.weight"), self.g(pre + "ln2.bias"), BT, Cc, 1e-5, acc))

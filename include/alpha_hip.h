@@ -207,11 +207,14 @@ int32_t ah_cross_entropy_bwd(ah_ptr logits, int32_t dtype, ah_ptr targets_i32, a
  *      Epilogues: AH_EPI_NONE; AH_EPI_ACCUM  C += acc (gradient accumulation);
  *      AH_EPI_GELU  C = gelu(acc), aux (same dtype/ld as C) = acc  (matmulTransposedGelu, ops.ts:426-487);
  *      AH_EPI_RESIDUAL  C = acc + aux (aux f32 [M,N], ld = ldc) (residual add of gpt.ts:280-281);
- *      AH_EPI_GELU_BWD  C = acc * gelu'(aux) (aux = saved pre-activation, dtype of C).
- *      Provided combinations: NONE -> f32 or bf16 output; ACCUM and RESIDUAL -> f32 output; GELU and GELU_BWD ->
- *      output of the operand type.  Anything else returns AH_ERR_UNSUPPORTED. ---- */
+ *      AH_EPI_GELU_BWD  C = acc * gelu'(aux) (aux = saved pre-activation, dtype of C);
+ *      AH_EPI_GELU_GRAD C = gelu(acc), aux = gelu'(acc): the forward saves the derivative instead of the pre-activation,
+ *      so that the backward product needs only  AH_EPI_MUL_AUX  C = acc * aux  (one multiply per element instead of
+ *      re-evaluating the tanh; same mathematics as GELU / GELU_BWD with gelu' rounded to the storage type).
+ *      Provided combinations: NONE -> f32 or bf16 output; ACCUM and RESIDUAL -> f32 output; GELU, GELU_BWD,
+ *      GELU_GRAD and MUL_AUX -> output of the operand type.  Anything else returns AH_ERR_UNSUPPORTED. ---- */
 enum { AH_GEMM_NN = 0, AH_GEMM_NT = 1, AH_GEMM_TN = 2 };
-enum { AH_EPI_NONE = 0, AH_EPI_ACCUM = 1, AH_EPI_GELU = 2, AH_EPI_RESIDUAL = 3, AH_EPI_GELU_BWD = 4 };
+enum { AH_EPI_NONE = 0, AH_EPI_ACCUM = 1, AH_EPI_GELU = 2, AH_EPI_RESIDUAL = 3, AH_EPI_GELU_BWD = 4, AH_EPI_GELU_GRAD = 5, AH_EPI_MUL_AUX = 6 };
 typedef struct {
   int32_t layout;            /* AH_GEMM_* */
   int32_t in_dtype;          /* AH_F32 or AH_BF16 (both operands) */

@@ -409,7 +409,7 @@ def _raw_gemm(B, layout, a, b, m, n, k, in_dtype, out_dtype, epi=0, aux=None, c_
     paux = 0
     if aux is not None:
         taux, paux = up(aux, ffi.F32 if epi == ffi.EPI_RESIDUAL else out_dtype)
-    elif epi == ffi.EPI_GELU:
+    elif epi in (ffi.EPI_GELU, ffi.EPI_GELU_GRAD):
         taux, paux = up(np.zeros((m, n), np.float32), out_dtype)
     lda = a.shape[1]
     ldb = b.shape[1]
@@ -421,7 +421,7 @@ def _raw_gemm(B, layout, a, b, m, n, k, in_dtype, out_dtype, epi=0, aux=None, c_
         raw = t.data
         return (raw.astype(np.uint32) << 16).view(np.float32) if store == ffi.BF16 else raw
     out = down(tc, out_dtype).reshape(m, n)
-    aux_out = down(taux, out_dtype).reshape(m, n) if epi == ffi.EPI_GELU else None
+    aux_out = down(taux, out_dtype).reshape(m, n) if epi in (ffi.EPI_GELU, ffi.EPI_GELU_GRAD) else None
     return out, aux_out
 
 
@@ -458,6 +458,12 @@ def test_gemm_layouts_epilogues_dtypes(B, in_bf16, out_bf16, M, N, K):
             pre_act = _bf16_round(pre_act)[0]
         gb = ref.gelu_backward(orc(pre_act), orc(want), fused=True).data.reshape(M, N)
         cmp(_raw_gemm(B, ffi.GEMM_NN, a, np.ascontiguousarray(b.T), M, N, K, idt, odt, ffi.EPI_GELU_BWD, aux=pre_act)[0], gb, "GELU_BWD")
+        # the same pair with the derivative saved by the forward product: C = gelu(acc), aux = gelu'(acc); then C = acc * aux
+        got, dsaved = _raw_gemm(B, ffi.GEMM_NT, a, b, M, N, K, idt, odt, ffi.EPI_GELU_GRAD)
+        cmp(got, O.gelu(orc(want)).data.reshape(M, N), "GELU_GRAD.value")
+        ones = np.ones((M, N), np.float32)
+        cmp(dsaved, ref.gelu_backward(orc(want), orc(ones), fused=True).data.reshape(M, N), "GELU_GRAD.derivative")
+        cmp(_raw_gemm(B, ffi.GEMM_NN, a, np.ascontiguousarray(b.T), M, N, K, idt, odt, ffi.EPI_MUL_AUX, aux=pre_act)[0], want * pre_act, "MUL_AUX")
     else:
         import ctypes as C
         g = ffi.AhGemm(ffi.GEMM_NT, idt, odt, ffi.EPI_GELU, M, N, K, K, K, N, 1, 0, 0, 0, 1 << 20, 1 << 20, 1 << 20, 1 << 20)
@@ -533,6 +539,10 @@ def test_gemm_bf16_large_tiles_direct_to_lds_kernel(B, M, N, K, tile):
     pre_act = _bf16_round(rs.randn(M, N).astype(np.float32))[0]
     gb = ref.gelu_backward(orc(pre_act), orc(w32), fused=True).data.reshape(M, N)
     assert_close(_raw_gemm(B, ffi.GEMM_NN, a, bt, M, N, K, ffi.BF16, ffi.BF16, ffi.EPI_GELU_BWD, aux=pre_act)[0], gb, rel=2.0 ** -7, what="GELU_BWD")
+    got, dsaved = _raw_gemm(B, ffi.GEMM_NT, a, b, M, N, K, ffi.BF16, ffi.BF16, ffi.EPI_GELU_GRAD)
+    assert_close(got, O.gelu(orc(w32)).data.reshape(M, N), rel=2.0 ** -7, what="GELU_GRAD.value")
+    assert_close(dsaved, ref.gelu_backward(orc(w32), orc(np.ones((M, N), np.float32)), fused=True).data.reshape(M, N), rel=2.0 ** -7, what="GELU_GRAD.derivative")
+    assert_close(_raw_gemm(B, ffi.GEMM_NN, a, bt, M, N, K, ffi.BF16, ffi.BF16, ffi.EPI_MUL_AUX, aux=pre_act)[0], want * pre_act, rel=2.0 ** -7, what="MUL_AUX")
 
 
 def test_gemm_grouped_matches_separate_products(B):
