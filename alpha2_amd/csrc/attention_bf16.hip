@@ -237,19 +237,20 @@ __global__ __launch_bounds__(256, D <= 64 ? 3 : 1) void k_flash_fwd_bf16(FlashAr
   }
 }
 
-// Per-score backward arithmetic shared by the dQ and dK/dV kernels.  s = raw q.k, dp = dO.v, krow = (max - lse) in
-// base 2 (max = cap when CAPPED, else 0), delta = rowsum(dO*O).  Returns p and writes ds WITHOUT the constant factor
-// (scale, and 4 for tanh' when CAPPED), which the caller applies to its accumulators once.
+// Per-score backward arithmetic shared by the dQ and dK/dV kernels.  s = raw q.k, dpd = dO.v - delta (the dP accumulator
+// starts at -delta = -rowsum(dO*O), so the subtraction rides on the MFMA), krow = (max - lse) in base 2 (max = cap when
+// CAPPED, else 0).  Returns p and writes ds WITHOUT the constant factor (scale, and 4 for tanh' when CAPPED), which the
+// caller applies to its accumulators once.
 template <bool CAPPED>
-__device__ __forceinline__ float score_bwd(float s, float dp, float krow, float delta, float c1, float c2, float &ds) {
+__device__ __forceinline__ float score_bwd(float s, float dpd, float krow, float c1, float c2, float &ds) {
   float p;
   if (CAPPED) {
     float r = rcp_fast(exp2_fast(s * c1) + 1.0f);
     p = exp2_fast(fmaf(r, c2, krow));
-    ds = p * (dp - delta) * fmaf(-r, r, r);                        // tanh' / 4 = r (1 - r)
+    ds = p * dpd * fmaf(-r, r, r);                                 // tanh' / 4 = r (1 - r)
   } else {
     p = exp2_fast(fmaf(s, c1, krow));
-    ds = p * (dp - delta);
+    ds = p * dpd;
   }
   return p;
 }
@@ -314,7 +315,7 @@ __global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void k_flash_dq_bf16(FlashArg
       if (kv0 <= q0 + 31) {
         f32x16 s, dp;
 #pragma unroll
-        for (int e = 0; e < 16; e++) { s[e] = 0.f; dp[e] = 0.f; }
+        for (int e = 0; e < 16; e++) { s[e] = 0.f; dp[e] = -delta; }       // this lane's column is one query: dP - delta
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) {
           s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tile_frag<D>(Ks[cur], sub * 32, ks, lane), qf[ks], s, 0, 0, 0);     // S^T[kv, q]
@@ -324,7 +325,7 @@ __global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void k_flash_dq_bf16(FlashArg
 #pragma unroll
         for (int e = 0; e < 16; e++) {
           float ds;
-          score_bwd<CAPPED>(s[e], dp[e], krow, delta, c1, c2, ds);
+          score_bwd<CAPPED>(s[e], dp[e], krow, c1, c2, ds);
           s[e] = ds;
         }
         if (edge) {
@@ -356,7 +357,7 @@ template <int D, bool CAPPED>
 __global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void k_flash_dkv_bf16(FlashArgs a) {
   constexpr int DB = D / 32, KS = D / 16;
   __shared__ __attribute__((aligned(16))) uint16_t Qs[2][Geo<D>::ELEMS], dOs[2][Geo<D>::ELEMS];
-  __shared__ __attribute__((aligned(16))) float Ls[2][ST], Ds[2][ST];      // per streamed query: (max - lse) in base 2; delta
+  __shared__ __attribute__((aligned(16))) float Ls[2][ST], Ds[2][ST];      // per streamed query: (max - lse) in base 2; -delta
   int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
   int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 31, lk = lane >> 5;
   int kv_blk0 = blockIdx.x * 128, kv0 = kv_blk0 + wave * 32, kvi = kv0 + lr;
@@ -387,7 +388,7 @@ __global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void k_flash_dkv_bf16(FlashAr
     if (threadIdx.x < ST) {
       int qi = q_base + threadIdx.x;
       rl = qi < a.T ? (lse_max - a.lse[srow0 + qi]) * LOG2E : 0.f;
-      rd = qi < a.T ? a.delta[srow0 + qi] : 0.f;
+      rd = qi < a.T ? -a.delta[srow0 + qi] : 0.f;
     }
   };
   tile_load<D>(Q, a.q_st, q_first, a.T, rq);
@@ -410,7 +411,11 @@ __global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void k_flash_dkv_bf16(FlashAr
       if (qs + 31 >= kv0 && qs < a.T) {                            // otherwise every query of the sub-tile precedes this wave's keys
         f32x16 s, dp;
 #pragma unroll
-        for (int e = 0; e < 16; e++) { s[e] = 0.f; dp[e] = 0.f; }
+        for (int j = 0; j < 4; j++) {                              // accumulator rows are queries: dP starts at -delta[query]
+          float4 de = *reinterpret_cast<const float4 *>(&Ds[cur][sub * 32 + 8 * j + 4 * lk]);
+          s[4 * j] = 0.f; s[4 * j + 1] = 0.f; s[4 * j + 2] = 0.f; s[4 * j + 3] = 0.f;
+          dp[4 * j] = de.x; dp[4 * j + 1] = de.y; dp[4 * j + 2] = de.z; dp[4 * j + 3] = de.w;
+        }
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) {                          // rows = queries, columns = this wave's keys
           s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tile_frag<D>(Qs[cur], sub * 32, ks, lane), kf[ks], s, 0, 0, 0);
@@ -420,13 +425,12 @@ __global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void k_flash_dkv_bf16(FlashAr
 #pragma unroll
         for (int j = 0; j < 4; j++) {
           float4 kr = *reinterpret_cast<const float4 *>(&Ls[cur][sub * 32 + 8 * j + 4 * lk]);
-          float4 de = *reinterpret_cast<const float4 *>(&Ds[cur][sub * 32 + 8 * j + 4 * lk]);
-          float krv[4] = {kr.x, kr.y, kr.z, kr.w}, dev[4] = {de.x, de.y, de.z, de.w};
+          float krv[4] = {kr.x, kr.y, kr.z, kr.w};
 #pragma unroll
           for (int r = 0; r < 4; r++) {
             int e = 4 * j + r;
             float ds;
-            float p = score_bwd<CAPPED>(s[e], dp[e], krv[r], dev[r], c1, c2, ds);
+            float p = score_bwd<CAPPED>(s[e], dp[e], krv[r], c1, c2, ds);
             dp[e] = p;
             s[e] = ds;
           }

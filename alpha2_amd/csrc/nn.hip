@@ -163,18 +163,29 @@ __global__ void k_layernorm_bwd(const float *__restrict__ x, const float *__rest
     part_db[(size_t)blockIdx.x * dim + j] = c;
   }
 }
-// column sums of the per-block partials: 32 columns per block, 8 row slices per column, fixed summation order
-__global__ void k_colsum_partials(const float *__restrict__ part_dw, const float *__restrict__ part_db, int nparts, int dim,
-                                  float *__restrict__ dw, float *__restrict__ db, int accumulate) {
-  __shared__ double sa[8][33], sc[8][33];
+// column sums of the per-block partials: 32 columns per block, 32 row slices per column (1024 threads, so that the few
+// blocks of this launch keep many loads in flight), fixed summation order
+__global__ __launch_bounds__(1024) void k_colsum_partials(const float *__restrict__ part_dw, const float *__restrict__ part_db, int nparts, int dim,
+                                                          float *__restrict__ dw, float *__restrict__ db, int accumulate) {
+  __shared__ double sa[32][33], sc[32][33];
   int cx = threadIdx.x & 31, sl = threadIdx.x >> 5, j = blockIdx.x * 32 + cx;
   double a = 0, c = 0;
-  if (j < dim)
-    for (int p = sl; p < nparts; p += 8) { a += part_dw[(size_t)p * dim + j]; c += part_db[(size_t)p * dim + j]; }
+  if (j < dim) {
+    int p = sl;
+    for (; p + 96 < nparts; p += 128) {        // four independent loads per array in flight
+      float a0 = part_dw[(size_t)p * dim + j], a1 = part_dw[(size_t)(p + 32) * dim + j], a2 = part_dw[(size_t)(p + 64) * dim + j],
+            a3 = part_dw[(size_t)(p + 96) * dim + j];
+      float c0 = part_db[(size_t)p * dim + j], c1 = part_db[(size_t)(p + 32) * dim + j], c2 = part_db[(size_t)(p + 64) * dim + j],
+            c3 = part_db[(size_t)(p + 96) * dim + j];
+      a += a0; a += a1; a += a2; a += a3;
+      c += c0; c += c1; c += c2; c += c3;
+    }
+    for (; p < nparts; p += 32) { a += part_dw[(size_t)p * dim + j]; c += part_db[(size_t)p * dim + j]; }
+  }
   sa[sl][cx] = a; sc[sl][cx] = c;
   __syncthreads();
   if (sl == 0 && j < dim) {
-    for (int k = 1; k < 8; k++) { a += sa[k][cx]; c += sc[k][cx]; }
+    for (int k = 1; k < 32; k++) { a += sa[k][cx]; c += sc[k][cx]; }
     dw[j] = (accumulate ? dw[j] : 0.f) + (float)a;
     db[j] = (accumulate ? db[j] : 0.f) + (float)c;
   }
@@ -501,7 +512,7 @@ int32_t ah_layernorm_bwd(ah_ptr x, ah_ptr w, ah_ptr grad_out, int32_t grad_dtype
     hipLaunchKernelGGL(k_layernorm_bwd<uint16_t>, dim3(nblk), dim3(TPB), lds, stream(), dp<const float>(x), dp<const float>(w),
                        dp<const uint16_t>(grad_out), dp<const float>(residual_grad), dp<float>(dx), dp<uint16_t>(dx_bf16), part_dw, part_db, rows, (int)dim, eps);
   AH_LAUNCH_CHECK();
-  hipLaunchKernelGGL(k_colsum_partials, dim3((unsigned)cdiv(dim, 32)), dim3(TPB), 0, stream(), part_dw, part_db, nblk, (int)dim,
+  hipLaunchKernelGGL(k_colsum_partials, dim3((unsigned)cdiv(dim, 32)), dim3(1024), 0, stream(), part_dw, part_db, nblk, (int)dim,
                      dp<float>(dw), dp<float>(db), accumulate);
   AH_LAUNCH_CHECK();
   return AH_OK;
