@@ -93,7 +93,9 @@ class FusedTrainer:
         # ---- activations (all shapes are static, so every buffer is allocated once)
         BT, Cc, Fd, V = self.BT, self.C, self.F, self.V
         a = self._alloc
-        self.tok, self.tgt = a(BT * 4), a(BT * 4)
+        self.toks = [a(BT * 4) for _ in range(self.accum)]               # one resident token batch per micro-step
+        self.tgts = [a(BT * 4) for _ in range(self.accum)]
+        self.tok, self.tgt = self.toks[0], self.tgts[0]
         self.x = [a(BT * Cc * 4) for _ in range(self.L + 1)]            # residual stream entering layer l (f32)
         self.xmid = [a(BT * Cc * 4) for _ in range(self.L)]
         self.ln1 = [a(BT * Cc * 2) for _ in range(self.L)]
@@ -115,6 +117,7 @@ class FusedTrainer:
         self.dqkv = [a(BT * 3 * Cc * 2) for _ in range(self.L)]
         self.dxb0 = a(BT * Cc * 2)                # grad of the embedding output in bf16 (written by the last LayerNorm backward, unused)
         self.loss, self.sumsq, self.clip = a(4), a(4), a(8)
+        self.loss_micro = a(4)
         self.hyper = a(ffi.C.sizeof(ffi.AhAdamW))
         self.loss_hist_cap = 4096
         self.loss_hist, self.norm_hist = a(self.loss_hist_cap * 4), a(self.loss_hist_cap * 8)
@@ -208,7 +211,8 @@ class FusedTrainer:
             self._timed.append({"kind": "flash_bwd" if bwd else "flash_fwd", "flops": fl, "e0": t0, "e1": t1})
 
     # ------------------------------------------------------------------ the step
-    def _forward_backward(self, first_micro: bool):
+    def _forward_backward(self, first_micro: bool, micro: int = 0):
+        self.tok, self.tgt = self.toks[micro], self.tgts[micro]
         lib, BT, Cc, Fd, V, L = self.lib, self.BT, self.C, self.F, self.V, self.L
         NN, NT, TN = ffi.GEMM_NN, ffi.GEMM_NT, ffi.GEMM_TN
         acc = 0 if first_micro else 1
@@ -225,7 +229,13 @@ class FusedTrainer:
             self._gemm(NT, self.hact[l], self.p(pre + "mlp.fc2", True), self.x[l + 1], BT, Cc, Fd, Fd, Fd, Cc, F32, ffi.EPI_RESIDUAL, self.xmid[l])
         check(lib.ah_layernorm(self.x[L], self.p("lnF.weight"), self.p("lnF.bias"), self.lnf, BT, Cc, 1e-5, BF16))
         self._gemm(NT, self.lnf, self.p("lmHead", True), self.logits, BT, V, Cc, Cc, Cc, V)
-        check(lib.ah_cross_entropy(self.logits, BF16, self.tgt, self.loss, self.rowlse, BT, V))
+        if self.accum == 1:
+            check(lib.ah_cross_entropy(self.logits, BF16, self.tgt, self.loss, self.rowlse, BT, V))
+        else:                                     # reported loss = mean of the micro-step losses (trainer.ts:1270-1273)
+            check(lib.ah_cross_entropy(self.logits, BF16, self.tgt, self.loss_micro, self.rowlse, BT, V))
+            if first_micro:
+                check(lib.ah_fill_f32(self.loss, 0.0, 1))
+            check(lib.ah_axpy_inplace(self.loss, self.loss_micro, 1.0 / self.accum, 1))
         check(lib.ah_cross_entropy_bwd(self.logits, BF16, self.tgt, self.rowlse, 0, 1.0, self.logits, BT, V))     # dlogits in place
 
         self._gemm(NN, self.logits, self.p("lmHead", True), self.dlnb, BT, Cc, V, V, Cc, Cc)
@@ -266,7 +276,8 @@ class FusedTrainer:
                                self.clip, self.Pb + split * 2))
 
     def _whole_step(self):
-        self._forward_backward(True)
+        for m in range(self.accum):               # gradients of the micro-steps are summed in place; scaled once in the optimizer
+            self._forward_backward(m == 0, m)
         self._optimizer()
 
     def set_batch(self, inputs: TensorData, targets: TensorData):
@@ -285,10 +296,17 @@ class FusedTrainer:
         self._batches.append((ti, tt))
         return len(self._batches) - 1
 
-    def _use_batch(self, i: int):
+    def _use_batch(self, i, micro: int = 0):
+        """Copy stored batch i into the resident slot of micro-step `micro` (a sequence fills slots 0, 1, ...)."""
+        if isinstance(i, (list, tuple)):
+            if len(i) != self.accum:
+                raise ValueError(f"need {self.accum} batch indices, one per micro-step")
+            for m, bi in enumerate(i):
+                self._use_batch(bi, m)
+            return
         ti, tt = self._batches[i]
-        check(self.lib.ah_copy(self.tok, ti, self.BT * 4))
-        check(self.lib.ah_copy(self.tgt, tt, self.BT * 4))
+        check(self.lib.ah_copy(self.toks[micro], ti, self.BT * 4))
+        check(self.lib.ah_copy(self.tgts[micro], tt, self.BT * 4))
 
     def _write_hyper(self) -> float:
         tc = self.tc
@@ -299,16 +317,15 @@ class FusedTrainer:
         check(self.lib.ah_upload(self.hyper, C.byref(h), C.sizeof(h)))
         return lr
 
-    def step(self, batch_index: Optional[int] = None) -> int:
+    def step(self, batch_index=None) -> int:
         """Enqueue one optimizer step (no host synchronisation); returns the step index whose loss / grad-norm can be
-        read later with history()."""
+        read later with history().  `batch_index`: a stored batch, or with gradient accumulation a sequence of `accum`
+        stored batches (micro-steps run in that order); None keeps the resident ones."""
         if batch_index is not None:
             self._use_batch(batch_index)
         elif not self._batches:
             raise RuntimeError("no batch set")
         self._write_hyper()
-        if self.accum != 1:
-            raise NotImplementedError("micro-batch accumulation runs through step_accum()")
         if self.use_graph:
             if self._graph is None:
                 self.prepare()

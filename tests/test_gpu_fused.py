@@ -83,3 +83,30 @@ def test_fused_loss_parity_over_steps_graph_replay(B):
         assert abs(hg[s].gradNorm - he[s].gradNorm) <= 1e-3 * he[s].gradNorm
     assert all(math.isfinite(h.loss) for h in hg)
     ft.close(), eager.close()
+
+
+def test_fused_gradient_accumulation_matches_oracle(B):
+    """Two micro-batches per optimizer step: summed gradients scaled once, reported loss = mean of the micro losses
+    (trainer.ts:1164-1273); graph replay and eager execution agree."""
+    from alpha2_amd.fused import FusedTrainer
+    from alpha2_amd.model import ModelConfig
+    from alpha2_amd.train import TrainConfig, syntheticBatch
+    steps, K = 6, 2
+    tc = dict(iters=steps, gradAccumSteps=K)
+    mk = lambda graph: FusedTrainer(B, ModelConfig(**CFG), TrainConfig(**tc), 4, seed=5, use_graph=graph, accum=K)
+    ft, eager = mk(True), mk(False)
+    orc = rm.Trainer(rm.ModelConfig(**CFG), rm.TrainConfig(iters=steps, gradAccumSteps=K), seed=5)
+    for s in range(steps):
+        seeds = [300 + K * s + m for m in range(K)]
+        ids = [ft.add_batch(*syntheticBatch(sd, 4, 64, 256)) for sd in seeds]
+        ide = [eager.add_batch(*syntheticBatch(sd, 4, 64, 256)) for sd in seeds]
+        ft.step(ids)
+        eager.step(ide)
+        o = orc.step([rm.synthetic_batch(sd, 4, 64, 256) for sd in seeds])
+        hg, he = ft.history(s, 1)[0], eager.history(s, 1)[0]
+        assert abs(hg.loss - o.loss) <= 2e-2 * abs(o.loss), (s, hg.loss, o.loss)
+        assert abs(hg.gradNorm - o.gradNorm) <= 3e-2 * o.gradNorm, (s, hg.gradNorm, o.gradNorm)
+        assert abs(hg.loss - he.loss) <= 1e-4 * abs(he.loss) and abs(hg.gradNorm - he.gradNorm) <= 1e-3 * he.gradNorm
+    with pytest.raises(ValueError, match="one per micro-step"):
+        ft.step([0])
+    ft.close(), eager.close()
