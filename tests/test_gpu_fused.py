@@ -61,7 +61,7 @@ def test_fused_step_gradients_and_update_match_oracle(B):
 
 def test_fused_loss_parity_over_steps_graph_replay(B):
     from alpha2_amd.train import syntheticBatch
-    steps = 12
+    steps = 50
     tc = dict(iters=steps)
     ft = _make(B, tc, use_graph=True, seed=3)
     eager = _make(B, tc, use_graph=False, seed=3)

@@ -101,13 +101,13 @@ def test_tiny_char_gpt_one_step_matches_oracle(B):
 
 
 def test_loss_parity_over_steps_with_accumulation(B):
-    """Step loss within 1e-3 relative over a run (warm-up + cosine schedule, clip, 2 micro-batches)."""
+    """Step loss within 1e-3 relative over a 50-step run (10 warm-up steps, cosine decay, clip, 2 micro-batches)."""
     from alpha2_amd.train import syntheticBatch
     cfg = dict(vocabSize=96, blockSize=32, nLayer=2, nEmbd=64, nHead=2)
-    tc = dict(iters=12, gradAccumSteps=2)
+    tc = dict(iters=50, gradAccumSteps=2)
     dev, orc = _both(B, cfg, tc, seed=2)
     live = None
-    for s in range(12):
+    for s in range(50):
         db = [syntheticBatch(100 + 2 * s + i, 4, 32, 96) for i in range(2)]
         ob = [rm.synthetic_batch(100 + 2 * s + i, 4, 32, 96) for i in range(2)]
         r, o = dev.step(db), orc.step(ob)

@@ -578,3 +578,84 @@ def test_gemm_grouped_matches_separate_products(B):
     assert B.lib.ah_gemm_grouped_run(plan.value, ffi.EPI_NONE) != 0 and b"unknown plan" in B.lib.ah_last_error()
     bad = (ffi.AhGemm * 1)(ffi.AhGemm(ffi.GEMM_TN, ffi.BF16, ffi.F32, ffi.EPI_NONE, 64, 64, 100, 64, 64, 64, 1, 0, 0, 0, 1 << 20, 1 << 20, 1 << 20, 0))
     assert B.lib.ah_gemm_grouped_plan(bad, 1, C.byref(plan)) != 0 and b"multiple of 64" in B.lib.ah_last_error()
+
+
+# ---------------------------------------------------------------------------------------------- parity at the benchmark sizes
+def _gauss_bf16(shape, seed, std):
+    g = np.random.default_rng(seed)
+    x = g.standard_normal(shape, dtype=np.float32) * np.float32(std)
+    return _bf16_round(x)[0]
+
+
+@pytest.mark.parametrize("N", [768, 2304, 3072, 50304])
+def test_gemm_microbench_shapes_forward_and_both_backward(B, N):
+    """C = A B^T, dA = G B, dB = G^T A at M = 16384 (B*T), K = 768, N as in the GEMM microbenchmark; operands
+    N(0,1)*0.02 rounded to bf16, fp32 accumulate.  The full products are too large for the CPU oracle, so a sample of
+    output rows is read back and checked against float64 numpy products of the same operands."""
+    import ctypes as C
+    from alpha2_amd import _ffi as ffi
+    M, K = 16384, 768
+    lib = B.lib
+
+    def bits_of(shape, seed):           # bf16 bit patterns of N(0,1)*0.02, and nothing else kept on the host
+        x = np.random.default_rng(seed).standard_normal(shape, dtype=np.float32)
+        x *= np.float32(0.02)
+        u = x.view(np.uint32)
+        u += np.uint32(0x7FFF) + ((u >> np.uint32(16)) & np.uint32(1))          # round to nearest even
+        return (u >> np.uint32(16)).astype(np.uint16)
+
+    def f64(bits):
+        return (bits.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+
+    def up(bits):
+        p = C.c_uint64()
+        ffi.check(lib.ah_alloc(bits.nbytes, C.byref(p)))
+        ffi.check(lib.ah_upload(p.value, bits.ctypes.data_as(C.c_void_p), bits.nbytes))
+        return p.value
+
+    def rows_of(ptr, rows, ncols):
+        out = np.empty((len(rows), ncols), np.float32)
+        for i, r in enumerate(rows):
+            ffi.check(lib.ah_download(out[i].ctypes.data_as(C.c_void_p), ptr + int(r) * ncols * 4, ncols * 4))
+        return out
+    a, b, g_ = bits_of((M, K), 2), bits_of((N, K), 3), bits_of((M, N), 4)
+    pa, pb, pg = up(a), up(b), up(g_)
+    pick = np.random.default_rng(5)
+    rows_m, rows_n = np.sort(pick.choice(M, 24, replace=False)), np.sort(pick.choice(N, 24, replace=False))
+    out = C.c_uint64()
+    ffi.check(lib.ah_alloc(max(M * N, N * K, M * K) * 4, C.byref(out)))
+    run = lambda layout, pa_, pb_, m, n, k, lda, ldb: ffi.check(lib.ah_gemm(C.byref(
+        ffi.AhGemm(layout, ffi.BF16, ffi.F32, ffi.EPI_NONE, m, n, k, lda, ldb, n, 1, 0, 0, 0, pa_, pb_, out.value, 0))))
+    run(ffi.GEMM_NT, pa, pb, M, N, K, K, K)
+    assert_close(rows_of(out.value, rows_m, N), f64(a[rows_m]) @ f64(b).T, rel=1e-4, what=f"C rows N={N}")
+    run(ffi.GEMM_NN, pg, pb, M, K, N, N, K)                                   # dA = G [M,N] x B [N,K]
+    assert_close(rows_of(out.value, rows_m, K), f64(g_[rows_m]) @ f64(b), rel=1e-4, what=f"dA rows N={N}")
+    run(ffi.GEMM_TN, pg, pa, N, K, M, N, K)                                   # dB = G^T [N,M] x A [M,K]
+    assert_close(rows_of(out.value, rows_n, K), f64(np.ascontiguousarray(g_[:, rows_n])).T @ f64(a), rel=1e-4, what=f"dB rows N={N}")
+    for p in (pa, pb, pg, out.value):
+        lib.ah_free(p)
+
+
+@pytest.mark.parametrize("T", [256, 1024, 2048])
+@pytest.mark.parametrize("cap", [0.0, 30.0])
+def test_flash_attention_microbench_shapes(B, T, cap):
+    """B = 16, H = 12, head_dim 64, bf16 in / fp32 accumulate, scale 1/8, as in the attention microbenchmark.  The kernels
+    run on all 192 heads; three of them (first, a middle one, last) are checked against the oracle's materialised chain."""
+    BH, D, scale = 192, 64, 0.125
+    q, k, v, do = (_gauss_bf16((BH, T, D), 30 + i, 1.0) for i in range(4))
+    Q, K, V, dO = (B.castStore(dev(B, x), "bf16") for x in (q, k, v, do))
+    r = B.flashAttention(Q, K, V, T, scale, cap)
+    g = B.flashAttentionBackward(Q, K, V, r["output"], dO, r["lse"], T, scale, cap)
+    heads = [0, 77, 191]
+    want_o, want_lse, dq, dk, dv = _oracle_attention(q[heads], k[heads], v[heads], do[heads], scale, cap)
+    rel = 2.0 ** -6
+
+    def loose(x):
+        return dict(outlier_frac=2e-3, outlier_abs=0.1 * float(np.sqrt(np.mean(np.square(x)))) + 1e-6)
+    sel = lambda t: np.asarray(t.data).reshape(BH, T, -1)[heads]
+    # sums of bf16-rounded probabilities: a few entries in a hundred thousand sit a little outside the element-wise bound
+    assert_close(sel(r["output"]), want_o.reshape(3, T, D), rel=rel, what="O", **loose(want_o))
+    assert_close(np.asarray(r["lse"].data).reshape(BH, T)[heads], want_lse.reshape(3, T), rel=1e-4, what="LSE")
+    assert_close(sel(g["dQ"]), dq.reshape(3, T, D), rel=rel, what="dQ", **loose(dq))
+    assert_close(sel(g["dK"]), dk.reshape(3, T, D), rel=rel, what="dK", **loose(dk))
+    assert_close(sel(g["dV"]), dv.reshape(3, T, D), rel=rel, what="dV", **loose(dv))
