@@ -24,6 +24,10 @@ sys.path.insert(0, ROOT)
 GPT2 = dict(vocabSize=50304, blockSize=1024, nLayer=12, nEmbd=768, nHead=12)
 BATCH = 16
 PEAK = {"bf16": 2500.0, "f32": 157.3}          # MI355X dense MFMA, TFLOP/s
+# HBM-side bytes per launch of the kernels that can be the dominant one, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
+# runs of this benchmark (counter values scaled by what the same counters read for a plain copy of known size: x2.0
+# for FETCH_SIZE, x1.0 for WRITE_SIZE); the counter summary is kept under profiles/.
+TRAFFIC_BYTES = {"k_gemm_bf16_dma_grouped<true, true, 0, float>": 9.2336e9 + 0.4943e9}
 
 
 def step_flops(cfg, tokens):
@@ -117,15 +121,16 @@ def main():
     achieved = dom["flops"] / (dom["ms"] * 1e-3) / 1e12
     flops = step_flops(GPT2, tokens)
     out = {
-        "metric": "train tokens/sec (GPT-2-small-shape step, fwd+bwd+AdamW)", "value": tokens / (ms * 1e-3), "unit": "tokens/s",
+        "metric": "train tokens/sec + MFMA util % on GPT-124M step, 1xMI355X", "value": tokens / (ms * 1e-3), "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic (Zipf s=1.1 token ids, seed 4; random-init N(0,0.02) weights, seed 0)",
         "config": {"workload": "GPT-2-small-shape train step: vocab 50304, d_model 768, 12 layers, 12 heads, ctx 1024, batch 16, "
                                "untied lmHead (163.0M params), AdamW lr 3e-4 betas (0.9,0.95) wd 0.1, grad-clip 1.0",
                    "tokens_per_step": tokens, "mode": args.mode, "loss_first_step": loss_first, "loss_last_step": loss_last},
         "step_tflops": flops / (ms * 1e-3) / 1e12, "mfu_vs_bf16_dense_peak": flops / (ms * 1e-3) / 1e12 / PEAK["bf16"],
+        "mfma_util_pct": 100.0 * flops / (ms * 1e-3) / 1e12 / PEAK["bf16"],
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK[dtype], "unit": "TFLOP/s", "frac": achieved / PEAK[dtype],
-                     "traffic": None, "kernel": dom_name, "launches_per_step": dom["n"], "avg_launch_us": dom["ms"] / dom["n"] * 1e3,
+                     "traffic": TRAFFIC_BYTES.get(dom_name), "kernel": dom_name, "launches_per_step": dom["n"], "avg_launch_us": dom["ms"] / dom["n"] * 1e3,
                      "flops_per_launch": dom["flops"] / dom["n"], "ms_per_step": dom["ms"],
                      "all_gemm": {"launches_per_step": len(gemm), "ms_per_step": g_ms,
                                   "achieved": g_flops / (g_ms * 1e-3) / 1e12 if g_ms > 0 else 0.0}},
