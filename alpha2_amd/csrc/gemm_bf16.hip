@@ -247,6 +247,7 @@ int32_t run(const GemmArgs &ga, int batch, int out_dtype) {
     };
     double f256 = ga.N >= 256 ? fill(256) : 0.0, f192 = 0.97 * fill(192);
     int bn = f256 >= f192 ? 256 : 192;
+
     if ((bn == 256 ? f256 : f192) >= 0.7)
       return AKM ? gemm_bf16_dma_tn(ga, batch, out_dtype, bn) : BKM ? gemm_bf16_dma_nn(ga, batch, out_dtype, bn) : gemm_bf16_dma_nt(ga, batch, out_dtype, bn);
   }
