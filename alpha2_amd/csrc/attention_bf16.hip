@@ -156,6 +156,38 @@ __global__ __launch_bounds__(256, D <= 64 ? 3 : 1) void k_flash_fwd_bf16(FlashAr
       tile_load<D>(K, a.k_st, (it + 1) * ST, a.T, rk);
       tile_load<D>(V, a.v_st, (it + 1) * ST, a.T, rv);
     }
+    if (CAPPED && it * ST + ST - 1 <= q0) {
+      // Both 32-key halves of the tile lie entirely below this wave's diagonal (no masking, which is most tiles): run
+      // them as two independent MFMA chains so the softmax arithmetic of one overlaps the matrix work of the other.
+      f32x16 s0, s1;
+#pragma unroll
+      for (int e = 0; e < 16; e++) { s0[e] = 0.f; s1[e] = 0.f; }
+#pragma unroll
+      for (int ks = 0; ks < KS; ks++) {
+        s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tile_frag<D>(Ks[cur], 0, ks, lane), qf[ks], s0, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tile_frag<D>(Ks[cur], 32, ks, lane), qf[ks], s1, 0, 0, 0);
+      }
+#pragma unroll
+      for (int e = 0; e < 16; e++) { s0[e] = exp2_fast(rcp_fast(fmaf(exp2_fast(s0[e] * c1), ic2, ic2))); l += s0[e]; }
+      bf16x8 pa0 = acc_to_b(s0, 0), pa1 = acc_to_b(s0, 1);
+      lacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones, pa0, lacc, 0, 0, 0);
+      lacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones, pa1, lacc, 0, 0, 0);
+#pragma unroll
+      for (int d = 0; d < DB; d++) {
+        o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tile_frag_t<D>(Vs[cur], 0, 0, d, lane), pa0, o[d], 0, 0, 0);
+        o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tile_frag_t<D>(Vs[cur], 0, 1, d, lane), pa1, o[d], 0, 0, 0);
+      }
+#pragma unroll
+      for (int e = 0; e < 16; e++) { s1[e] = exp2_fast(rcp_fast(fmaf(exp2_fast(s1[e] * c1), ic2, ic2))); l += s1[e]; }
+      bf16x8 pc0 = acc_to_b(s1, 0), pc1 = acc_to_b(s1, 1);
+      lacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones, pc0, lacc, 0, 0, 0);
+      lacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones, pc1, lacc, 0, 0, 0);
+#pragma unroll
+      for (int d = 0; d < DB; d++) {
+        o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tile_frag_t<D>(Vs[cur], 32, 0, d, lane), pc0, o[d], 0, 0, 0);
+        o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tile_frag_t<D>(Vs[cur], 32, 1, d, lane), pc1, o[d], 0, 0, 0);
+      }
+    } else
 #pragma unroll
     for (int sub = 0; sub < ST / 32; sub++) {
       int kv0 = it * ST + sub * 32;
