@@ -407,6 +407,63 @@ class FusedTrainer:
         check(self.lib.ah_download(out.ctypes.data_as(C.c_void_p), self.g(name), n * 4))
         return out
 
+    # ------------------------------------------------------------------ checkpoints (reference file format)
+    def _arena_slice(self, arena: int, name: str) -> np.ndarray:
+        n = shapeSize(self.shapes[name])
+        out = np.empty(n, np.float32)
+        check(self.lib.ah_download(out.ctypes.data_as(C.c_void_p), arena + self.off[name] * 4, n * 4))
+        return out
+
+    def stateDict(self) -> dict:
+        """AdamW.stateDict (optimizers.ts:202-210) read from the moment arenas."""
+        self.B.syncGpu()
+        bufs = {}
+        for name, _ in self.entries:
+            n = shapeSize(self.shapes[name])
+            bufs[name + ".m"] = TensorData((n,), "f32", self._arena_slice(self.M, name))
+            bufs[name + ".v"] = TensorData((n,), "f32", self._arena_slice(self.Vm, name))
+        return {"step": self.stepIdx, "buffers": bufs}
+
+    def saveCheckpoint(self, path: str, configHash: str = "", tokenizerArtifacts=None):
+        from dataclasses import asdict
+        from .checkpoint import FileCheckpoint
+        self.B.syncGpu()
+        params = {name: {"shape": list(self.shapes[name]), "data": self.param(name)} for name, _ in self.entries}
+        FileCheckpoint().save(path, {"modelConfig": asdict(self.cfg), "params": params, "optimizerState": self.stateDict(),
+                                     "tokenizerArtifacts": tokenizerArtifacts, "rngState": 0, "configHash": configHash, "step": self.stepIdx})
+
+    def loadCheckpoint(self, path: str) -> dict:
+        """Parameters, moments and step counter from a checkpoint written by either trainer (or by the reference)."""
+        from .checkpoint import FileCheckpoint
+        st = FileCheckpoint().load(path)
+        self.B.syncGpu()
+
+        def put(arena, name, data):
+            a = np.ascontiguousarray(np.asarray(data, dtype=np.float32).reshape(-1))
+            n = shapeSize(self.shapes[name])
+            if a.size != n:
+                raise ValueError(f"checkpoint tensor {name} has {a.size} values, the model needs {n}")
+            check(self.lib.ah_upload(arena + self.off[name] * 4, a.ctypes.data_as(C.c_void_p), n * 4))
+        for name, _ in self.entries:
+            saved = st["params"].get(name)
+            if saved is None and name.endswith(".attn.wqkv"):       # pre-fusion checkpoints (checkpoint.ts:243-257)
+                pre = name[:-len(".attn.wqkv")]
+                parts = [st["params"].get(f"{pre}.attn.{w}") for w in ("wq", "wk", "wv")]
+                if all(p is not None for p in parts):
+                    saved = {"data": np.concatenate([np.asarray(p["data"], dtype=np.float32).reshape(-1) for p in parts])}
+            if saved is not None:
+                put(self.P, name, saved["data"])
+        bufs = st["optimizerState"]["buffers"]
+        check(self.lib.ah_fill_f32(self.M, 0.0, self.nparam))
+        check(self.lib.ah_fill_f32(self.Vm, 0.0, self.nparam))
+        for key, td in bufs.items():
+            if key[:-2] in self.off and key.endswith((".m", ".v")):
+                put(self.M if key.endswith(".m") else self.Vm, key[:-2], td.data)
+        check(self.lib.ah_cast(self.P, F32, self.Pb, BF16, self.nparam))
+        self.stepIdx = int(st["optimizerState"].get("step") or st.get("step") or 0)
+        self._b1p, self._b2p = self.tc.beta1 ** self.stepIdx, self.tc.beta2 ** self.stepIdx      # optimizers.ts:214-215
+        return st
+
     def close(self):
         self.B.syncGpu()
         if self._graph is not None:

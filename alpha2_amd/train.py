@@ -206,6 +206,24 @@ class Trainer:
         self.stepIdx = 0
         self.release = getattr(backend, "releaseGpuTensor", None)
 
+    def saveCheckpoint(self, path: str, configHash: str = "", tokenizerArtifacts=None):
+        """Full training state in the reference's file format (checkpoint.ts:197-221)."""
+        from dataclasses import asdict
+        from .checkpoint import FileCheckpoint, buildCheckpointState
+        self.backend.syncGpu()
+        rng_state = getattr(self.rng, "state", lambda: 0)()
+        FileCheckpoint().save(path, buildCheckpointState(self.entries, self.optimizer, rng_state, configHash, self.stepIdx,
+                                                         asdict(self.cfg), tokenizerArtifacts))
+
+    def loadCheckpoint(self, path: str) -> dict:
+        """Resume: parameters, Adam moments and the step counter (trainer.ts:905-960 restores the same three)."""
+        from .checkpoint import FileCheckpoint, restoreParams
+        st = FileCheckpoint().load(path)
+        restoreParams(self.entries, st["params"])
+        self.optimizer.loadStateDict(st["optimizerState"])
+        self.stepIdx = int(st.get("step") or 0)
+        return st
+
     def step(self, batches: Sequence[Tuple[TensorData, TensorData]]) -> StepResult:
         B, tc = self.backend, self.tc
         lr = lrAt(tc, self.stepIdx)

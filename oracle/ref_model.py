@@ -508,6 +508,25 @@ class AdamW:
             ref.adamw_step(var.data, var.grad, self.m[name], self.v[name], self.lr, self.beta1, self.beta2,
                            self.eps, wd, bc1, bc2, gradScale)
 
+    def state_dict(self) -> dict:
+        """optimizers.ts:202-210: "<name>.m" then "<name>.v" per parameter, in moment-map order."""
+        bufs = {}
+        for name, m in self.m.items():
+            bufs[name + ".m"] = TD((m.size,), "f32", m.copy())
+            bufs[name + ".v"] = TD((m.size,), "f32", self.v[name].copy())
+        return {"step": self._step, "buffers": bufs}
+
+    def load_state_dict(self, state: dict):
+        """optimizers.ts:212-229: the beta powers are rebuilt as pow(beta, step)."""
+        self._step = state["step"]
+        self._b1p, self._b2p = math.pow(self.beta1, self._step), math.pow(self.beta2, self._step)
+        self.m, self.v = {}, {}
+        for key, td in state["buffers"].items():
+            if key.endswith(".m"):
+                self.m[key[:-2]] = np.array(td.data, dtype=np.float32)
+            elif key.endswith(".v"):
+                self.v[key[:-2]] = np.array(td.data, dtype=np.float32)
+
 
 @dataclass
 class TrainConfig:
@@ -646,3 +665,78 @@ class DataLoader:
                         pos = 0
                 self.cursors[b] = pos
         return TD((Bt, T), "i32", inputs), TD((Bt, T), "i32", targets)
+
+
+# ------------------------------------------------------------------------------------------------ checkpoint files
+def checkpoint_save_bytes(state: dict) -> bytes:
+    """packages/train/src/checkpoint.ts:29-94 (saveBinary): "ALPH", uint32 LE header length, header JSON, then the
+    float32 payload: parameters ("p.<name>") in insertion order, then optimizer buffers ("o.<name>")."""
+    import json
+    import struct
+    tensors, chunks = [], []
+    for name, p in state["params"].items():
+        f32 = np.asarray(p["data"], dtype="<f4").reshape(-1)
+        tensors.append({"name": "p." + name, "shape": list(p["shape"]), "elements": int(f32.size)})
+        chunks.append(f32.tobytes())
+    opt = state.get("optimizerState")
+    if opt and opt.get("buffers"):
+        for name, td in opt["buffers"].items():
+            f32 = np.asarray(td.data, dtype="<f4").reshape(-1)
+            tensors.append({"name": "o." + name, "shape": list(td.shape), "elements": int(f32.size)})
+            chunks.append(f32.tobytes())
+    header = {"modelConfig": state.get("modelConfig"), "configHash": state.get("configHash"), "rngState": state.get("rngState"),
+              "step": state.get("step")}
+    if state.get("tokenizerArtifacts") is not None:
+        header["tokenizerArtifacts"] = state["tokenizerArtifacts"]
+    header["optimizerStep"] = opt["step"] if opt else 0
+    if state.get("symbioActivationGraph") is not None:
+        header["symbioActivationGraph"] = state["symbioActivationGraph"]
+    header["tensors"] = tensors
+    hb = json.dumps(header, separators=(",", ":"), ensure_ascii=False).encode("utf-8")
+    return b"ALPH" + struct.pack("<I", len(hb)) + hb + b"".join(chunks)
+
+
+def checkpoint_load_bytes(raw: bytes) -> dict:
+    """checkpoint.ts:98-136 (loadBinary) and :160-189 (format detection, legacy JSON)."""
+    import json
+    import struct
+    if raw[:4] != b"ALPH":
+        parsed = json.loads(raw.decode("utf-8"))
+        bufs = {k: TD(tuple(v["shape"]), "f32", np.asarray(v["data"], dtype=np.float32))
+                for k, v in ((parsed.get("optimizerState") or {}).get("buffers") or {}).items()}
+        return {"modelConfig": parsed.get("modelConfig"), "params": parsed.get("params"),
+                "optimizerState": {"step": (parsed.get("optimizerState") or {}).get("step") or 0, "buffers": bufs},
+                "tokenizerArtifacts": parsed.get("tokenizerArtifacts"), "rngState": parsed.get("rngState"),
+                "configHash": parsed.get("configHash"), "step": parsed.get("step")}
+    off = 4
+    (hlen,) = struct.unpack_from("<I", raw, off)
+    off += 4
+    header = json.loads(raw[off:off + hlen].decode("utf-8"))
+    off += hlen
+    params, bufs = {}, {}
+    for t in header["tensors"]:
+        n = t["elements"]
+        f32 = np.frombuffer(raw, dtype="<f4", count=n, offset=off).astype(np.float32)
+        off += 4 * n
+        if t["name"].startswith("p."):
+            params[t["name"][2:]] = {"shape": t["shape"], "data": f32}
+        elif t["name"].startswith("o."):
+            bufs[t["name"][2:]] = TD(tuple(t["shape"]), "f32", f32)
+    return {"modelConfig": header.get("modelConfig"), "params": params,
+            "optimizerState": {"step": header.get("optimizerStep") or 0, "buffers": bufs},
+            "tokenizerArtifacts": header.get("tokenizerArtifacts"), "rngState": header.get("rngState"),
+            "configHash": header.get("configHash"), "step": header.get("step")}
+
+
+def restore_params(entries, saved: dict):
+    """checkpoint.ts:224-259, including the wq / wk / wv -> wqkv concatenation for old checkpoints."""
+    for name, var in entries:
+        if name in saved:
+            src = np.asarray(saved[name]["data"], dtype=np.float32).reshape(-1)
+            var.data.data[:] = src[:var.data.data.size]
+            continue
+        if name.endswith(".attn.wqkv"):
+            prefix = name[:-len(".attn.wqkv")]
+            parts = [saved.get(f"{prefix}.attn.{w}") for w in ("wq", "wk", "wv")]
+            if all(p is not None for p in parts):
+                var.data.data[:] = np.concatenate([np.asarray(p["data"], dtype=np.float32).reshape(-1) for p in parts])

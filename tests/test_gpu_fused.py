@@ -110,3 +110,34 @@ def test_fused_gradient_accumulation_matches_oracle(B):
     with pytest.raises(ValueError, match="one per micro-step"):
         ft.step([0])
     ft.close(), eager.close()
+
+
+def test_fused_checkpoint_resume(B, tmp_path):
+    """The fast path writes and reads the same file format; a resumed run (graph captured after the load) follows the
+    uninterrupted one, and the generic trainer accepts the file too."""
+    from alpha2_amd.model import ModelConfig
+    from alpha2_amd.train import TrainConfig, Trainer, syntheticBatch
+    tc = dict(iters=8)
+    a = _make(B, tc, use_graph=True, seed=6)
+    ids = [a.add_batch(*syntheticBatch(700 + s, 4, 64, 256)) for s in range(8)]
+    for s in range(4):
+        a.step(ids[s])
+    path = str(tmp_path / "fused.alph")
+    a.saveCheckpoint(path)
+    at_save = a.param("layer.1.mlp.fc1")
+    b = _make(B, tc, use_graph=True, seed=11)
+    idb = [b.add_batch(*syntheticBatch(700 + s, 4, 64, 256)) for s in range(8)]
+    st = b.loadCheckpoint(path)
+    assert st["step"] == 4 and b.stepIdx == 4
+    for s in range(4, 8):
+        a.step(ids[s])
+        b.step(idb[s])
+    ha, hb = a.history(4, 4), b.history(4, 4)
+    for x, y in zip(ha, hb):
+        assert abs(x.loss - y.loss) <= 1e-4 * abs(x.loss) and abs(x.lr - y.lr) < 1e-15, (x, y)
+    g = Trainer(B, ModelConfig(**CFG), TrainConfig(**tc), seed=0)
+    g.loadCheckpoint(path)
+    assert g.stepIdx == 4 and g.optimizer._step == 4
+    assert np.array_equal(dict(g.entries)["layer.1.mlp.fc1"].data.data, at_save)       # bit-for-bit what was saved
+    assert not np.array_equal(a.param("layer.1.mlp.fc1"), at_save)                     # (training has moved on since)
+    a.close(), b.close()

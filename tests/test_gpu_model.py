@@ -186,3 +186,27 @@ def test_dataloader_rejects_a_corpus_not_longer_than_the_block(B):
     from alpha2_amd.train import DataLoader
     with pytest.raises(IndexError, match="must exceed block size"):
         DataLoader(B, np.arange(16, dtype=np.int32), SeededRng(0), 2, 16).nextBatch()
+
+
+def test_checkpoint_resume_matches_uninterrupted_run_and_loads_in_the_oracle(B, tmp_path):
+    """Save after 3 steps in the reference's file format, resume in a fresh trainer: the next steps follow the
+    uninterrupted run; the same file restores the CPU oracle, which then tracks the device trainer."""
+    from alpha2_amd.train import syntheticBatch
+    cfg = dict(vocabSize=96, blockSize=32, nLayer=2, nEmbd=64, nHead=2)
+    a, orc = _both(B, cfg, dict(iters=6), seed=4)
+    for s in range(3):
+        a.step([syntheticBatch(500 + s, 4, 32, 96)])
+    path = str(tmp_path / "ckpt.alph")
+    a.saveCheckpoint(path, configHash="cafe")
+    b, _ = _both(B, cfg, dict(iters=6), seed=9)               # different initial weights: everything must come from the file
+    st = b.loadCheckpoint(path)
+    assert st["configHash"] == "cafe" and st["step"] == 3 and st["modelConfig"]["nEmbd"] == 64
+    ost = rm.checkpoint_load_bytes(open(path, "rb").read())
+    rm.restore_params(orc.entries, ost["params"])
+    orc.opt.load_state_dict(ost["optimizerState"])
+    orc.step_idx = ost["step"]
+    for s in range(3, 6):
+        ra, rb = a.step([syntheticBatch(500 + s, 4, 32, 96)]), b.step([syntheticBatch(500 + s, 4, 32, 96)])
+        ro = orc.step([rm.synthetic_batch(500 + s, 4, 32, 96)])
+        assert abs(ra.loss - rb.loss) <= 1e-5 * abs(ra.loss) and ra.lr == rb.lr, (s, ra.loss, rb.loss)
+        assert abs(rb.loss - ro.loss) <= 1e-3 * abs(ro.loss), (s, rb.loss, ro.loss)
