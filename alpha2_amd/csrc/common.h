@@ -72,28 +72,31 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
-// tanh-approximation GELU and its derivative (cpu_ref.ts:422-427; ops.ts:405-417), written on r = 1 / (exp(2u) + 1):
-// tanh(u) = 1 - 2r, so 0.5 (1 + tanh u) = 1 - r and sech^2 u = 4 r (1 - r).  Two hardware transcendentals, no
-// branches, absolute error at fp32 rounding level (the epilogues of the big GEMM tiles cannot afford libm's tanhf:
-// its register footprint on top of 256 live accumulators spills).
-__device__ __forceinline__ float gelu_gate_r(float x) {
+// tanh-approximation GELU and its derivative (cpu_ref.ts:422-427; ops.ts:405-417) on the gate
+// s = sigmoid(2u) = (1 + tanh u) / 2 with u = sqrt(2/pi) (x + 0.044715 x^3):  gelu(x) = x s and
+// gelu'(x) = s + x s (1 - s) 2u'.  Two hardware transcendentals, no branches, absolute error at fp32 rounding level; a
+// value + derivative pair costs 9 simple operations (the epilogues of the big GEMM tiles run one wave per SIMD, where
+// every instruction costs 4 cycles, and cannot afford libm's tanhf: its register footprint on top of 256 live
+// accumulators spills).
+__device__ __forceinline__ float gelu_gate_s(float x, float x2) {
   const float k2 = 0.7978845608028654f * 2.0f * 1.4426950408889634f;      // 2 sqrt(2/pi) log2(e)
-  float u2 = k2 * (x + 0.044715f * x * x * x);
-  return __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(u2) + 1.0f);
+  float z = x * __builtin_fmaf(x2, -k2 * 0.044715f, -k2);
+  return __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(z) + 1.0f);
 }
-__device__ __forceinline__ float gelu_f(float x) { return x * (1.0f - gelu_gate_r(x)); }
+__device__ __forceinline__ float gelu_f(float x) { return x * gelu_gate_s(x, x * x); }
 // value and derivative from one gate evaluation
 __device__ __forceinline__ void gelu_both_f(float x, float &val, float &grad) {
   const float k = 0.7978845608028654f;
-  float r = gelu_gate_r(x), one_minus_r = 1.0f - r;
-  val = x * one_minus_r;
-  grad = one_minus_r * (1.0f + 2.0f * x * r * (k * (1.0f + 3.0f * 0.044715f * x * x)));
+  float x2 = x * x, s = gelu_gate_s(x, x2);
+  float h = x * s;
+  float d = __builtin_fmaf(x2, 6.0f * k * 0.044715f, 2.0f * k);           // 2 du/dx
+  val = h;
+  grad = __builtin_fmaf(h * d, 1.0f - s, s);
 }
 __device__ __forceinline__ float gelu_grad_f(float x) {
-  const float k = 0.7978845608028654f;
-  float r = gelu_gate_r(x);
-  float dinner = k * (1.0f + 3.0f * 0.044715f * x * x);
-  return (1.0f - r) * (1.0f + 2.0f * x * r * dinner);
+  float v, d;
+  gelu_both_f(x, v, d);
+  return d;
 }
 
 }  // namespace ah

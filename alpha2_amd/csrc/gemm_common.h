@@ -1,5 +1,6 @@
 // Shared between the GEMM translation units: argument block and the fused epilogues.
 #pragma once
+#include <type_traits>
 #include "common.h"
 
 namespace ah {
@@ -86,6 +87,133 @@ __device__ __forceinline__ void epilogue4(const GemmArgs &g, int64_t cbase, int 
       else if (EPI == AH_EPI_MUL_AUX) a *= Io<OUT>::ld((const OUT *)g.aux, idx + i);
       else if (EPI == AH_EPI_GELU_GRAD) { float d; gelu_both_f(a, a, d); Io<OUT>::st((OUT *)g.aux_out, idx + i, d); }
       Io<OUT>::st(c, idx + i, a);
+    }
+  }
+}
+
+// The values an epilogue reads beside the accumulators, 4 consecutive columns at a time.
+template <bool F32> struct AuxVec;
+template <> struct AuxVec<true> {
+  typedef float4 T;
+  static __device__ __forceinline__ void unpack(const float4 &o, float (&x)[4]) { x[0] = o.x; x[1] = o.y; x[2] = o.z; x[3] = o.w; }
+};
+template <> struct AuxVec<false> {
+  typedef uint2 T;
+  static __device__ __forceinline__ void unpack(const uint2 &o, float (&x)[4]) {
+    x[0] = bf16_bits_to_f32(o.x & 0xffff); x[1] = bf16_bits_to_f32(o.x >> 16); x[2] = bf16_bits_to_f32(o.y & 0xffff); x[3] = bf16_bits_to_f32(o.y >> 16);
+  }
+};
+
+// Four 4 KB pieces of LDS that belong to the calling wave alone (nobody else reads or writes them until the next
+// workgroup barrier).
+struct EpiStage { char *p[4]; };
+
+// Epilogue of a wave tile through LDS.  In the accumulator layout a lane owns 4 consecutive
+// columns of ONE row, so a store instruction written straight from the accumulators scatters 16-byte pieces over 32
+// rows: 32 partial cache lines per instruction (measured: the stores of a K = 768 product then take a third of its time).
+// Instead each 32 x 32 accumulator goes to LDS as f32 (row r at r * 128 bytes, 16-byte chunk c at position c ^ (r & 7):
+// conflict-free both ways) and comes back row-major: 8 (f32 output) or 16 (bf16 output, two tiles side by side) lanes
+// cover one row's 128 contiguous bytes, and everything an epilogue reads (residual, accumulate, saved gelu') is loaded in
+// that same coalesced layout.  Those loads are unconditional (lanes past an edge of C read a clamped, valid address and
+// only their stores are masked), so they can run ahead: vmcnt retires in issue order, stores included, so the reads of
+// pass p + DEPTH are issued before the stores of pass p.  Requires N % 4 == 0.
+template <int EPI, class OUT, int TM, int TN>
+__device__ __forceinline__ void store_tiles_lds(const GemmArgs &g, int64_t cbase, int row0, int col0, int lane, const f32x16 (&acc)[TM][TN],
+                                                const EpiStage &st) {
+  constexpr bool F32OUT = sizeof(OUT) == 4;
+  constexpr int JP = F32OUT ? 1 : 2;                  // 32 x 32 tiles per pass: a row of the pass is 128 bytes of output
+  constexpr int NJP = (TN + JP - 1) / JP, NPASS = TM * NJP;
+  constexpr bool READS = EPI == AH_EPI_ACCUM || EPI == AH_EPI_RESIDUAL || EPI == AH_EPI_GELU_BWD || EPI == AH_EPI_MUL_AUX;
+  constexpr bool AUX_F32 = EPI == AH_EPI_RESIDUAL || F32OUT;
+  constexpr int DEPTH = 4 < NPASS ? 4 : NPASS;        // passes of reads in flight: 4 x 16 registers
+  typedef AuxVec<AUX_F32> AV;
+  typedef typename AV::T AuxT;
+  typedef typename std::conditional<AUX_F32, float, uint16_t>::type AuxE;
+  const int lr = lane & 31, lk = lane >> 5;
+  OUT *c = (OUT *)g.c + cbase + (int64_t)row0 * g.ldc + col0;
+  const AuxE *aux = (const AuxE *)(EPI == AH_EPI_ACCUM ? (const void *)g.c : g.aux) + cbase + (int64_t)row0 * g.ldc + col0;
+  OUT *aux_out = (OUT *)g.aux_out + cbase + (int64_t)row0 * g.ldc + col0;
+  // a pass of NS tiles side by side comes back in 4 NS iterations of 8 / NS rows: lane -> (row in the group, chunk)
+  const int rr1 = lane >> 3, cc1 = lane & 7, rr2 = lane >> 4, cc2 = lane & 15;
+  const int rows_left = g.M - row0, cols_left = g.N - col0;        // lanes at or past these are outside C
+  int wofs[4];
+#pragma unroll
+  for (int q = 0; q < 4; q++) wofs[q] = lr * 128 + (((2 * q + lk) ^ (lr & 7)) << 4);
+
+  AuxT pre[DEPTH][8];
+  auto pass_row = [&](int p, int it) -> int {
+    const int i = p / NJP, j0 = (p % NJP) * JP, ns = TN - j0 < JP ? TN - j0 : JP;
+    return 32 * i + it * (8 / ns) + (ns == 2 ? rr2 : rr1);
+  };
+  auto pass_col = [&](int p) -> int {
+    const int j0 = (p % NJP) * JP, ns = TN - j0 < JP ? TN - j0 : JP;
+    return 32 * j0 + 4 * (ns == 2 ? cc2 : cc1);
+  };
+  auto pass_elem = [&](int p, int it) -> int64_t {      // element offset (from row0, col0) of this lane's 4 columns, clamped into C
+    return (int64_t)min(pass_row(p, it), rows_left - 1) * g.ldc + min(pass_col(p), cols_left - 4);
+  };
+  auto issue_reads = [&](int p) {
+    const int j0 = (p % NJP) * JP, ns = TN - j0 < JP ? TN - j0 : JP;
+#pragma unroll
+    for (int it = 0; it < 4 * ns; it++) pre[p % DEPTH][it] = *reinterpret_cast<const AuxT *>(aux + pass_elem(p, it));
+  };
+  if (READS) {
+#pragma unroll
+    for (int p = 0; p < DEPTH; p++) issue_reads(p);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+#pragma unroll
+  for (int p = 0; p < NPASS; p++) {
+    const int i = p / NJP, j0 = (p % NJP) * JP, ns = TN - j0 < JP ? TN - j0 : JP;
+    char *piece0 = st.p[JP == 2 ? 2 * (p & 1) : p & 3], *piece1 = st.p[JP == 2 ? 2 * (p & 1) + 1 : p & 3];
+#pragma unroll
+    for (int jj = 0; jj < ns; jj++)
+#pragma unroll
+      for (int q = 0; q < 4; q++)
+        *reinterpret_cast<float4 *>((jj ? piece1 : piece0) + wofs[q]) =
+            make_float4(acc[i][j0 + jj][4 * q], acc[i][j0 + jj][4 * q + 1], acc[i][j0 + jj][4 * q + 2], acc[i][j0 + jj][4 * q + 3]);
+#pragma unroll
+    for (int it = 0; it < 4 * ns; it++) {
+      const int r = it * (8 / ns) + (ns == 2 ? rr2 : rr1), ch = ns == 2 ? cc2 & 7 : cc1;
+      const char *src = (ns == 2 && cc2 >= 8 ? piece1 : piece0) + r * 128 + ((ch ^ (r & 7)) << 4);
+      const float4 t = *reinterpret_cast<const float4 *>(src);
+      float v[4] = {t.x, t.y, t.z, t.w};
+      const int64_t off = pass_elem(p, it);
+      const bool inside = pass_row(p, it) < rows_left && pass_col(p) < cols_left;
+      if (READS) {
+        float x[4];
+        AV::unpack(pre[p % DEPTH][it], x);
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          if (EPI == AH_EPI_ACCUM || EPI == AH_EPI_RESIDUAL) v[e] += x[e];
+          else if (EPI == AH_EPI_MUL_AUX) v[e] *= x[e];
+          else v[e] *= gelu_grad_f(x[e]);
+        }
+      } else if (EPI == AH_EPI_GELU_GRAD) {
+        float d[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) gelu_both_f(v[e], v[e], d[e]);
+        if (inside) {
+          if (F32OUT) *reinterpret_cast<float4 *>(aux_out + off) = make_float4(d[0], d[1], d[2], d[3]);
+          else *reinterpret_cast<uint2 *>(aux_out + off) = make_uint2(pack_bf16x2(d[0], d[1]), pack_bf16x2(d[2], d[3]));
+        }
+      } else if (EPI == AH_EPI_GELU) {
+        if (inside) {
+          if (F32OUT) *reinterpret_cast<float4 *>(aux_out + off) = make_float4(v[0], v[1], v[2], v[3]);
+          else *reinterpret_cast<uint2 *>(aux_out + off) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+        }
+#pragma unroll
+        for (int e = 0; e < 4; e++) v[e] = gelu_f(v[e]);
+      }
+      if (inside) {
+        if (F32OUT) *reinterpret_cast<float4 *>(c + off) = make_float4(v[0], v[1], v[2], v[3]);
+        else *reinterpret_cast<uint2 *>(c + off) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if (READS && p + DEPTH < NPASS) {
+      issue_reads(p + DEPTH);
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
 }
