@@ -5,7 +5,8 @@ ctx 1024, batch 16; forward + backward + AdamW with gradient clipping) on one MI
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--mode fast|parity] [--no-cpu]
 
 Prints ONE JSON line.  `value` is tokens/s with parameters, optimizer state and the token batch already resident in
-HBM.  `roofline` is for the dominant kernel, the MFMA GEMM instantiation with the largest summed duration in a step:
+HBM.  `roofline` is for the dominant kernel, the MFMA GEMM instantiation that does the most arithmetic in a step (which is
+also the one with the largest summed duration; going by arithmetic keeps the choice the same from run to run):
 2*M*N*K of its launches divided by their summed durations, each launch bracketed by HIP events on the library's
 stream (`all_gemm` gives the same over every GEMM launch of the step).  `cpu_baseline` times the CPU oracle
 (single-thread C restatement of the reference's cpu_ref loops) on a bounded sample of the same model.
@@ -27,7 +28,7 @@ PEAK = {"bf16": 2500.0, "f32": 157.3}          # MI355X dense MFMA, TFLOP/s
 # HBM-side bytes per launch of the kernels that can be the dominant one, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
 # runs of this benchmark (counter values scaled by what the same counters read for a plain copy of known size: x2.0
 # for FETCH_SIZE, x1.0 for WRITE_SIZE); the counter summary is kept under profiles/.
-TRAFFIC_BYTES = {"k_gemm_bf16_dma_grouped<true, true, 0, float>": 9.2336e9 + 0.4943e9}
+TRAFFIC_BYTES = {"k_gemm_bf16_dma_grouped<true, true, 0, float>": 9.2163e9 + 0.4943e9}
 
 
 def step_flops(cfg, tokens):
@@ -110,14 +111,14 @@ def main():
     recs = runner.timed_step() if hasattr(runner, "timed_step") else _timed(B, one_step)
     gemm = [r for r in recs if r["kind"] == "gemm"]
     g_flops, g_ms = sum(r["flops"] for r in gemm), sum(r["ms"] for r in gemm)
-    # the dominant kernel = the GEMM instantiation with the largest summed duration among launches that are one kernel
+    # the dominant kernel = the GEMM instantiation with the most arithmetic per step among launches that are one kernel
     # (a split-K launch is followed by its reduce kernel inside the same event bracket, so it is not a clean sample)
     groups = {}
     for r in gemm:
         if r["nsplit"] == 1:
             grp = groups.setdefault(r["kernel"], {"flops": 0.0, "ms": 0.0, "n": 0})
             grp["flops"] += r["flops"]; grp["ms"] += r["ms"]; grp["n"] += 1
-    dom_name, dom = max(groups.items(), key=lambda kv: kv[1]["ms"])
+    dom_name, dom = max(groups.items(), key=lambda kv: (kv[1]["flops"], kv[1]["ms"]))
     achieved = dom["flops"] / (dom["ms"] * 1e-3) / 1e12
     flops = step_flops(GPT2, tokens)
     out = {
