@@ -68,7 +68,8 @@ int32_t ah_adamw(ah_ptr p, ah_ptr g, ah_ptr m, ah_ptr v, uint64_t n, const AhAda
   AH_ARG(p && g && m && v, "ah_adamw: null operand");
   int vec = aligned16(p) && aligned16(g) && aligned16(m) && aligned16(v) && ((bf16_shadow & 7u) == 0);
   int64_t blocks = cdiv((int64_t)(vec ? n / 4 + 1 : n), TPB);
-  int64_t cap = (int64_t)num_cus() * 16;
+  // one float4 group per thread: measured 5.4 TB/s against 4.3 TB/s for a grid of 16 blocks per CU striding over the array
+  int64_t cap = (int64_t)1 << 22;
   if (blocks > cap) blocks = cap;
   hipLaunchKernelGGL(k_adamw, dim3((unsigned)blocks), dim3(TPB), 0, stream(), dp<float>(p), dp<const float>(g), dp<float>(m),
                      dp<float>(v), n, *h, dp<const AhAdamW>(dev_hyper), dp<const float>(dev_scale), dp<uint16_t>(bf16_shadow), vec);
