@@ -57,6 +57,15 @@ class AhAdamW(C.Structure):
                 ("bc1", f32), ("bc2", f32), ("grad_scale", f32)]
 
 
+class AhLion(C.Structure):
+    _fields_ = [("lr", C.c_double), ("beta1", C.c_double), ("beta2", C.c_double), ("weight_decay", C.c_double), ("grad_scale", C.c_double)]
+
+
+class AhAdafactor(C.Structure):
+    _fields_ = [("lr", C.c_double), ("beta2", C.c_double), ("eps", C.c_double), ("clip_threshold", C.c_double),
+                ("weight_decay", C.c_double), ("grad_scale", C.c_double)]
+
+
 # name -> argtypes (every function returns int32 except ah_last_error)
 SIGNATURES = {
     "ah_init": [i32], "ah_shutdown": [], "ah_device_info": [C.POINTER(AhDeviceInfo)], "ah_sync": [],
@@ -102,6 +111,9 @@ SIGNATURES = {
     "ah_flash_fwd": [C.POINTER(AhFlash)], "ah_flash_bwd": [C.POINTER(AhFlash)],
     "ah_adamw": [u64, u64, u64, u64, u64, C.POINTER(AhAdamW), u64, u64, u64],
     "ah_clip_coef": [u64, f32, f32, u64],
+    "ah_lion": [u64, u64, u64, u64, C.POINTER(AhLion)], "ah_sgd": [u64, u64, u64, C.c_double, C.c_double],
+    "ah_adafactor_2d": [u64, u64, u64, u64, i64, i64, C.POINTER(AhAdafactor)],
+    "ah_adafactor_flat": [u64, u64, u64, u64, C.POINTER(AhAdafactor)],
     "ah_rng_seed": [C.POINTER(AhRng), i32], "ah_rng_next": [C.POINTER(AhRng), C.POINTER(C.c_double)],
     "ah_rng_next_gauss": [C.POINTER(AhRng), C.POINTER(C.c_double)],
     "ah_rng_fill_gauss_f32": [C.POINTER(AhRng), C.c_void_p, u64, C.c_double],

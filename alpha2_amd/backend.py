@@ -786,6 +786,41 @@ class HipBackend:
         for t in (params, m, v):
             self._dirty(t)
 
+    # The reference runs its other optimizers as host loops inside the optimizer classes (optimizers.ts:236-593), not
+    # through the Backend interface; these device versions keep parameters and state resident.
+    def lionStep(self, params, grads, m, lr, beta1, beta2, weightDecay, gradScale=1.0):
+        self._f32(params, grads, m)
+        if not (params.size == grads.size == m.size):
+            raise ValueError("lionStep: params, grads, m must have the same size")
+        h = ffi.AhLion(lr, beta1, beta2, weightDecay, gradScale)
+        check(self.lib.ah_lion(self._ptr(params), self._ptr(grads), self._ptr(m), params.size, C.byref(h)))
+        self._dirty(params), self._dirty(m)
+
+    def sgdStep(self, params, grads, lr, gradScale=1.0):
+        self._f32(params, grads)
+        if params.size != grads.size:
+            raise ValueError("sgdStep: params and grads must have the same size")
+        check(self.lib.ah_sgd(self._ptr(params), self._ptr(grads), params.size, lr, gradScale))
+        self._dirty(params)
+
+    def adafactorStep2d(self, params, grads, vr, vc, lr, beta2, eps, clipThreshold, weightDecay, gradScale=1.0):
+        self._f32(params, grads, vr, vc)
+        rows, cols = params.shape
+        if grads.size != params.size or vr.size != rows or vc.size != cols:
+            raise ValueError("adafactorStep2d: grads / vr / vc do not match the parameter's shape")
+        h = ffi.AhAdafactor(lr, beta2, eps, clipThreshold, weightDecay, gradScale)
+        check(self.lib.ah_adafactor_2d(self._ptr(params), self._ptr(grads), self._ptr(vr), self._ptr(vc), rows, cols, C.byref(h)))
+        for t in (params, vr, vc):
+            self._dirty(t)
+
+    def adafactorStepFlat(self, params, grads, v, lr, beta2, eps, clipThreshold, weightDecay, gradScale=1.0):
+        self._f32(params, grads, v)
+        if not (params.size == grads.size == v.size):
+            raise ValueError("adafactorStepFlat: params, grads, v must have the same size")
+        h = ffi.AhAdafactor(lr, beta2, eps, clipThreshold, weightDecay, gradScale)
+        check(self.lib.ah_adafactor_flat(self._ptr(params), self._ptr(grads), self._ptr(v), params.size, C.byref(h)))
+        self._dirty(params), self._dirty(v)
+
 
 def _i32(x: int) -> int:
     x &= 0xFFFFFFFF

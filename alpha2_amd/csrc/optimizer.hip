@@ -56,9 +56,186 @@ __global__ void k_clip_coef(const float *__restrict__ sumsq, float grad_scale, f
   }
 }
 
+// ---- Lion, SGD, Adafactor: the reference's host loops (double arithmetic, one rounding per Float32Array store) ----
+// No contraction into fused multiply-adds from here on: JavaScript rounds every product.
+#pragma clang fp contract(off)
+__global__ void k_lion(float *__restrict__ p, const float *__restrict__ g, float *__restrict__ m, uint64_t n, AhLion h) {
+  const double decay = h.weight_decay > 0 ? 1.0 - h.lr * h.weight_decay : 1.0;
+  uint64_t i = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  double gi = (double)g[i] * h.grad_scale, mi = (double)m[i];
+  float pi = p[i];
+  if (h.weight_decay > 0) pi = (float)((double)pi * decay);
+  double update = h.beta1 * mi + (1.0 - h.beta1) * gi;
+  double sign = update > 0 ? 1.0 : update < 0 ? -1.0 : update;      // Math.sign keeps +-0 (and NaN)
+  p[i] = (float)((double)pi - h.lr * sign);
+  m[i] = (float)(h.beta2 * mi + (1.0 - h.beta2) * gi);
+}
+
+__global__ void k_sgd(float *__restrict__ p, const float *__restrict__ g, uint64_t n, double lr, double gs) {
+  uint64_t i = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x;
+  if (i < n) p[i] = (float)((double)p[i] - lr * ((double)g[i] * gs));
+}
+
+__device__ __forceinline__ double wave_sum_f64(double v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+// block-wide sum (256 threads) of doubles; the result is valid in thread 0
+__device__ __forceinline__ double block_sum_f64(double v, double *sh) {
+  v = wave_sum_f64(v);
+  if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = v;
+  __syncthreads();
+  double r = 0;
+  if (threadIdx.x == 0) for (int w = 0; w < (int)(blockDim.x >> 6); w++) r += sh[w];
+  __syncthreads();
+  return r;
+}
+
+// one block per row: vr[r] = beta2 vr[r] + (1 - beta2) mean_c (g gs)^2 + eps
+__global__ __launch_bounds__(256) void k_af_rows(const float *__restrict__ g, float *__restrict__ vr, int64_t cols, AhAdafactor h) {
+  __shared__ double sh[4];
+  const float *gr = g + blockIdx.x * cols;
+  double s = 0;
+  for (int64_t c = threadIdx.x; c < cols; c += blockDim.x) { double x = (double)gr[c] * h.grad_scale; s += x * x; }
+  s = block_sum_f64(s, sh);
+  if (threadIdx.x == 0) vr[blockIdx.x] = (float)(h.beta2 * (double)vr[blockIdx.x] + (1.0 - h.beta2) * (s * (1.0 / (double)cols)) + h.eps);
+}
+// one thread per column, rows in order (the reference's own summation order): vc[c] likewise
+__global__ void k_af_cols(const float *__restrict__ g, float *__restrict__ vc, int64_t rows, int64_t cols, AhAdafactor h) {
+  int64_t c = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+  if (c >= cols) return;
+  double s = 0;
+  for (int64_t r = 0; r < rows; r++) { double x = (double)g[r * cols + c] * h.grad_scale; s += x * x; }
+  vc[c] = (float)(h.beta2 * (double)vc[c] + (1.0 - h.beta2) * (s * (1.0 / (double)rows)) + h.eps);
+}
+// ws[0] = 1 / max(mean(vr), eps)
+__global__ __launch_bounds__(256) void k_af_vrmean(const float *__restrict__ vr, int64_t rows, double eps, double *__restrict__ ws) {
+  __shared__ double sh[4];
+  double s = 0;
+  for (int64_t r = threadIdx.x; r < rows; r += blockDim.x) s += (double)vr[r];
+  s = block_sum_f64(s, sh);
+  if (threadIdx.x == 0) { double mean = s * (1.0 / (double)rows); ws[0] = 1.0 / (mean > eps ? mean : eps); }
+}
+__device__ __forceinline__ double af_denom(const float *vr, const float *vc, int64_t r, int64_t c, double inv_vr_mean, double eps) {
+  double d = sqrt((double)vr[r] * inv_vr_mean) * sqrt((double)vc[c]);
+  return eps > d ? eps : d;
+}
+// part[b] = sum over the block's elements of (g gs / denom)^2; FLAT: denom = sqrt(v), after v's own update
+template <bool FLAT>
+__global__ __launch_bounds__(256) void k_af_update_sq(const float *__restrict__ g, const float *__restrict__ vr, const float *__restrict__ vc,
+                                                      float *__restrict__ v, uint64_t n, int64_t cols, AhAdafactor h, const double *__restrict__ ws,
+                                                      double *__restrict__ part) {
+  __shared__ double sh[4];
+  double s = 0;
+  for (uint64_t i = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x; i < n; i += (uint64_t)gridDim.x * blockDim.x) {
+    double x = (double)g[i] * h.grad_scale, d;
+    if (FLAT) {
+      float vi = (float)(h.beta2 * (double)v[i] + (1.0 - h.beta2) * (x * x) + h.eps);
+      v[i] = vi;
+      d = sqrt((double)vi);
+    } else {
+      d = af_denom(vr, vc, (int64_t)(i / (uint64_t)cols), (int64_t)(i % (uint64_t)cols), ws[0], h.eps);
+    }
+    double u = x / d;
+    s += u * u;
+  }
+  s = block_sum_f64(s, sh);
+  if (threadIdx.x == 0) part[blockIdx.x] = s;
+}
+// ws[1] = lr / max(1, rms / clip) with rms = sqrt(sum(part) / max(1, n))
+__global__ void k_af_step_scale(const double *__restrict__ part, int nblk, uint64_t n, AhAdafactor h, double *__restrict__ ws) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) {
+    double s = 0;
+    for (int b = 0; b < nblk; b++) s += part[b];
+    double rms = sqrt(s / (double)(n > 1 ? n : 1));
+    double den = h.clip_threshold > 0 ? (rms / h.clip_threshold > 1.0 ? rms / h.clip_threshold : 1.0) : 1.0;
+    ws[1] = h.lr / den;
+  }
+}
+template <bool FLAT>
+__global__ void k_af_apply(float *__restrict__ p, const float *__restrict__ g, const float *__restrict__ vr, const float *__restrict__ vc,
+                           const float *__restrict__ v, uint64_t n, int64_t cols, AhAdafactor h, const double *__restrict__ ws) {
+  uint64_t i = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const double decay = h.weight_decay > 0 ? 1.0 - h.lr * h.weight_decay : 1.0;
+  double x = (double)g[i] * h.grad_scale;
+  double d = FLAT ? sqrt((double)v[i]) : af_denom(vr, vc, (int64_t)(i / (uint64_t)cols), (int64_t)(i % (uint64_t)cols), ws[0], h.eps);
+  float pi = p[i];
+  if (h.weight_decay > 0) pi = (float)((double)pi * decay);
+  p[i] = (float)((double)pi - ws[1] * (x / d));
+}
+
+// the shared tail of the two Adafactor branches: RMS of the update -> step scale -> parameter update
+template <bool FLAT>
+int32_t adafactor_tail(ah_ptr p, ah_ptr g, ah_ptr vr, ah_ptr vc, ah_ptr v, uint64_t n, int64_t cols, const AhAdafactor &h, double *ws) {
+  int nblk = (int)(cdiv((int64_t)n, TPB) < 1024 ? cdiv((int64_t)n, TPB) : 1024);
+  double *part = ws + 2;
+  hipLaunchKernelGGL((k_af_update_sq<FLAT>), dim3(nblk), dim3(TPB), 0, stream(), dp<const float>(g), dp<const float>(vr), dp<const float>(vc),
+                     dp<float>(v), n, cols, h, ws, part);
+  AH_LAUNCH_CHECK();
+  hipLaunchKernelGGL(k_af_step_scale, dim3(1), dim3(64), 0, stream(), part, nblk, n, h, ws);
+  AH_LAUNCH_CHECK();
+  hipLaunchKernelGGL((k_af_apply<FLAT>), dim3((unsigned)cdiv((int64_t)n, TPB)), dim3(TPB), 0, stream(), dp<float>(p), dp<const float>(g),
+                     dp<const float>(vr), dp<const float>(vc), dp<const float>(v), n, cols, h, ws);
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+
 }  // namespace
 
 extern "C" {
+
+int32_t ah_lion(ah_ptr p, ah_ptr g, ah_ptr m, uint64_t n, const AhLion *h) {
+  AH_REQUIRE_READY();
+  AH_ARG(h != nullptr, "ah_lion: null hyper-parameters");
+  if (n == 0) return AH_OK;
+  AH_ARG(p && g && m, "ah_lion: null operand");
+  AH_ARG(n < ((uint64_t)1 << 39), "ah_lion: tensor too large");
+  hipLaunchKernelGGL(k_lion, dim3((unsigned)cdiv((int64_t)n, TPB)), dim3(TPB), 0, stream(), dp<float>(p), dp<const float>(g), dp<float>(m), n, *h);
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+
+int32_t ah_sgd(ah_ptr p, ah_ptr g, uint64_t n, double lr, double grad_scale) {
+  AH_REQUIRE_READY();
+  if (n == 0) return AH_OK;
+  AH_ARG(p && g, "ah_sgd: null operand");
+  AH_ARG(n < ((uint64_t)1 << 39), "ah_sgd: tensor too large");
+  hipLaunchKernelGGL(k_sgd, dim3((unsigned)cdiv((int64_t)n, TPB)), dim3(TPB), 0, stream(), dp<float>(p), dp<const float>(g), n, lr, grad_scale);
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+
+int32_t ah_adafactor_2d(ah_ptr p, ah_ptr g, ah_ptr vr, ah_ptr vc, int64_t rows, int64_t cols, const AhAdafactor *h) {
+  AH_REQUIRE_READY();
+  AH_ARG(h != nullptr, "ah_adafactor_2d: null hyper-parameters");
+  AH_ARG(rows >= 0 && cols >= 0, "ah_adafactor_2d: negative shape [%lld, %lld]", (long long)rows, (long long)cols);
+  if (rows == 0 || cols == 0) return AH_OK;
+  AH_ARG(p && g && vr && vc, "ah_adafactor_2d: null operand");
+  AH_ARG(rows < ((int64_t)1 << 31) && cols < ((int64_t)1 << 31), "ah_adafactor_2d: shape too large");
+  double *ws = (double *)scratch(sizeof(double) * (2 + 1024));
+  if (!ws) return fail(AH_ERR_OOM, "ah_adafactor_2d: no scratch");
+  hipLaunchKernelGGL(k_af_rows, dim3((unsigned)rows), dim3(TPB), 0, stream(), dp<const float>(g), dp<float>(vr), cols, *h);
+  AH_LAUNCH_CHECK();
+  hipLaunchKernelGGL(k_af_cols, dim3((unsigned)cdiv(cols, 64)), dim3(64), 0, stream(), dp<const float>(g), dp<float>(vc), rows, cols, *h);
+  AH_LAUNCH_CHECK();
+  hipLaunchKernelGGL(k_af_vrmean, dim3(1), dim3(TPB), 0, stream(), dp<const float>(vr), rows, h->eps, ws);
+  AH_LAUNCH_CHECK();
+  return adafactor_tail<false>(p, g, vr, vc, 0, (uint64_t)rows * (uint64_t)cols, cols, *h, ws);
+}
+
+int32_t ah_adafactor_flat(ah_ptr p, ah_ptr g, ah_ptr v, uint64_t n, const AhAdafactor *h) {
+  AH_REQUIRE_READY();
+  AH_ARG(h != nullptr, "ah_adafactor_flat: null hyper-parameters");
+  if (n == 0) return AH_OK;
+  AH_ARG(p && g && v, "ah_adafactor_flat: null operand");
+  AH_ARG(n < ((uint64_t)1 << 39), "ah_adafactor_flat: tensor too large");
+  double *ws = (double *)scratch(sizeof(double) * (2 + 1024));
+  if (!ws) return fail(AH_ERR_OOM, "ah_adafactor_flat: no scratch");
+  return adafactor_tail<true>(p, g, 0, 0, v, n, 1, *h, ws);
+}
 
 int32_t ah_adamw(ah_ptr p, ah_ptr g, ah_ptr m, ah_ptr v, uint64_t n, const AhAdamW *h, ah_ptr dev_hyper, ah_ptr dev_scale,
                  ah_ptr bf16_shadow) {

@@ -31,6 +31,7 @@ class TrainConfig:
     gradClip: float = 1.0
     seed: int = 42
     gradAccumSteps: int = 1
+    optimizer: str = "adamw"          # "adamw" | "lion" | "adafactor" | "sgd" (optimizers.ts:596-603)
 
 
 def noDecayNames(nLayer: int) -> set:
@@ -108,6 +109,23 @@ class AdamW:
         for key, td in state["buffers"].items():
             tgt = self._m if key.endswith(".m") else self._v
             tgt[key[:-2]] = TensorData(td.shape, "f32", np.array(td.data, dtype=np.float32))
+
+
+def makeOptimizer(backend, tc: TrainConfig, noDecay: set):
+    """apps/cli/src/commands/train.ts:333-340 with apps/cli/src/resolve.ts:25-36: the training configuration's lr / betas /
+    eps / weight decay / no-decay names go to AdamW, Lion and Adafactor (each takes the fields it knows: Adafactor's eps
+    becomes the training eps, its clip threshold stays 1); SGD comes from the registry with its own default lr, which
+    the trainer's setLr overrides before the first step."""
+    if tc.optimizer == "adamw":
+        return AdamW(backend, tc.lr, tc.beta1, tc.beta2, tc.eps, tc.weightDecay, noDecay)
+    from .optimizers import Adafactor, Lion, SGD
+    if tc.optimizer == "lion":
+        return Lion(backend, lr=tc.lr, beta1=tc.beta1, beta2=tc.beta2, weightDecay=tc.weightDecay, noDecayNames=noDecay)
+    if tc.optimizer == "adafactor":
+        return Adafactor(backend, lr=tc.lr, beta2=tc.beta2, eps=tc.eps, weightDecay=tc.weightDecay, noDecayNames=noDecay)
+    if tc.optimizer == "sgd":
+        return SGD(backend)
+    raise ValueError(f'Unknown optimizer: "{tc.optimizer}". Available: adamw, lion, adafactor, sgd')
 
 
 def lrAt(tc: TrainConfig, step: int) -> float:
@@ -200,7 +218,7 @@ class Trainer:
         self.rng = rng or SeededRng(seed)
         self.params = initGPT(cfg, backend, self.rng)
         self.entries = collectParamEntries(self.params)
-        self.optimizer = AdamW(backend, tc.lr, tc.beta1, tc.beta2, tc.eps, tc.weightDecay, noDecayNames(cfg.nLayer))
+        self.optimizer = makeOptimizer(backend, tc, noDecayNames(cfg.nLayer))
         self.tape = Tape()
         self.dropoutRng = DropoutRng(tc.seed)
         self.stepIdx = 0

@@ -278,6 +278,21 @@ int32_t ah_adamw(ah_ptr p, ah_ptr g, ah_ptr m, ah_ptr v, uint64_t n, const AhAda
  * out[1] = the norm itself. */
 int32_t ah_clip_coef(ah_ptr sumsq, float grad_scale, float clip, ah_ptr out2);
 
+/* ---- the other optimizers of the reference's registry (optimizers.ts:596-603).  The reference runs them as host loops
+ *      over Float32Arrays, i.e. in double precision with one rounding per store; the kernels compute in double the
+ *      same way, so Lion and SGD reproduce the loops bit for bit and Adafactor up to the order of its double sums. ---- */
+typedef struct { double lr, beta1, beta2, weight_decay, grad_scale; } AhLion;
+/* Lion.stepTensor (optimizers.ts:284-311): in place on p and the momentum m (f32). */
+int32_t ah_lion(ah_ptr p, ah_ptr g, ah_ptr m, uint64_t n, const AhLion *h);
+/* SGD (optimizers.ts:555-567): p -= lr * (g * grad_scale). */
+int32_t ah_sgd(ah_ptr p, ah_ptr g, uint64_t n, double lr, double grad_scale);
+typedef struct { double lr, beta2, eps, clip_threshold, weight_decay, grad_scale; } AhAdafactor;
+/* Adafactor.stepTensor, factored branch for a [rows, cols] parameter (optimizers.ts:412-475): vr f32[rows] and
+ * vc f32[cols] are the row / column second moments, updated in place. */
+int32_t ah_adafactor_2d(ah_ptr p, ah_ptr g, ah_ptr vr, ah_ptr vc, int64_t rows, int64_t cols, const AhAdafactor *h);
+/* Adafactor.stepTensor, unfactored branch for any other parameter (optimizers.ts:478-500): v f32[n]. */
+int32_t ah_adafactor_flat(ah_ptr p, ah_ptr g, ah_ptr v, uint64_t n, const AhAdafactor *h);
+
 /* ---- host-side SeededRng (packages/core/src/rng.ts:6-68): int32 xorshift pair, 20 warm-up draws,
  *      next() = ((s0+s1)>>>0)/2^32, polar Box-Muller with a cached spare.  Pure host code (no device work);
  *      here so that parameter initialisation (packages/model/src/gpt.ts:53-59,73-151) draws the reference's

@@ -6,6 +6,9 @@ Restatement of the reference's host-side training step as it runs on its CPU bac
   * initGPT / transformerBlock / gptForward (the NON-flash branch cpu_ref takes)
                                         packages/model/src/gpt.ts:73-151, 220-333, 344-427
   * AdamW.stepParamEntries              packages/train/src/optimizers.ts:54-115
+  * Lion, Adafactor, SGD                packages/train/src/optimizers.ts:246-593 (pinned in tests/test_optimizers.py by
+                                        closed forms: Lion's first step, Adafactor on a rank-one gradient, and the
+                                        reference's own gradScale / entry-vs-map properties, packages/tests/src/optimizer.test.ts)
   * LR schedule, grad-norm, clip        packages/train/src/trainer.ts:1088-1096,1150-1159,1297,
                                         1332-1349,1650-1656,1761-1784
   * no-decay set                        apps/cli/src/commands/train.ts:319-331
@@ -528,6 +531,130 @@ class AdamW:
                 self.v[key[:-2]] = np.array(td.data, dtype=np.float32)
 
 
+def _seq_sum(x: np.ndarray) -> float:
+    """Left-to-right double sum, the order of the reference's for loops (numpy's own sum is pairwise)."""
+    return float(np.cumsum(x.astype(np.float64))[-1]) if x.size else 0.0
+
+
+class Lion:
+    """optimizers.ts:246-336: host loop in double arithmetic, every Float32Array store rounds to f32."""
+
+    def __init__(self, lr=1e-4, beta1=0.9, beta2=0.99, weightDecay=0.01, noDecayNames=None):
+        self.lr, self.beta1, self.beta2, self.wd = lr, beta1, beta2, weightDecay
+        self.noDecay = noDecayNames or set()
+        self._step = 0
+        self.m: Dict[str, np.ndarray] = {}
+
+    def setLr(self, lr):
+        self.lr = lr
+
+    def _step_tensor(self, name, p: np.ndarray, g32: np.ndarray, gradScale):
+        """optimizers.ts:284-311; p (f32) is updated in place."""
+        if name not in self.m:
+            self.m[name] = np.zeros(p.size, dtype=np.float32)
+        m = self.m[name]
+        wd = 0.0 if name in self.noDecay else self.wd
+        g = g32.astype(np.float64) * gradScale
+        if wd > 0:
+            p[:] = (p.astype(np.float64) * (1 - self.lr * wd)).astype(np.float32)
+        update = self.beta1 * m.astype(np.float64) + (1 - self.beta1) * g
+        p[:] = (p.astype(np.float64) - self.lr * np.sign(update)).astype(np.float32)
+        m[:] = (self.beta2 * m.astype(np.float64) + (1 - self.beta2) * g).astype(np.float32)
+
+    def stepParamEntries(self, entries, gradScale=1.0):
+        self._step += 1
+        for name, var in entries:
+            if var.grad is not None:
+                self._step_tensor(name, var.data.data, var.grad.data, gradScale)
+
+    def state_dict(self) -> dict:
+        return {"step": self._step, "buffers": {name + ".m": TD((m.size,), "f32", m.copy()) for name, m in self.m.items()}}
+
+
+class Adafactor:
+    """optimizers.ts:349-543."""
+
+    def __init__(self, lr=1e-3, beta2=0.999, eps=1e-30, clipThreshold=1.0, weightDecay=0.0, noDecayNames=None):
+        self.lr, self.beta2, self.eps, self.clip, self.wd = lr, beta2, eps, clipThreshold, weightDecay
+        self.noDecay = noDecayNames or set()
+        self._step = 0
+        self.vr: Dict[str, np.ndarray] = {}
+        self.vc: Dict[str, np.ndarray] = {}
+        self.v: Dict[str, np.ndarray] = {}
+
+    def setLr(self, lr):
+        self.lr = lr
+
+    def _step_tensor(self, name, p: np.ndarray, shape, g32: np.ndarray, gradScale):
+        lr, beta2, eps = self.lr, self.beta2, self.eps
+        wd = 0.0 if name in self.noDecay else self.wd
+        decay = 1 - lr * wd if wd > 0 else 1.0
+        g = g32.astype(np.float64).reshape(-1) * gradScale
+        size = p.size
+        if len(shape) == 2:                                          # optimizers.ts:412-475
+            rows, cols = shape
+            if name not in self.vr or self.vr[name].size != rows:
+                self.vr[name] = np.zeros(rows, dtype=np.float32)
+            if name not in self.vc or self.vc[name].size != cols:
+                self.vc[name] = np.zeros(cols, dtype=np.float32)
+            vr, vc = self.vr[name], self.vc[name]
+            g2 = (g * g).reshape(rows, cols)
+            for r in range(rows):
+                vr[r] = np.float32(beta2 * float(vr[r]) + (1 - beta2) * (_seq_sum(g2[r]) * (1 / cols)) + eps)
+            for c in range(cols):
+                vc[c] = np.float32(beta2 * float(vc[c]) + (1 - beta2) * (_seq_sum(g2[:, c]) * (1 / rows)) + eps)
+            vr_mean = max(_seq_sum(vr) * (1 / rows), eps)
+            r_scale = np.sqrt(vr.astype(np.float64) * (1 / vr_mean))
+            denom = np.maximum(eps, r_scale[:, None] * np.sqrt(vc.astype(np.float64))[None, :]).reshape(-1)
+        else:                                                        # optimizers.ts:478-500
+            if name not in self.v or self.v[name].size != size:
+                self.v[name] = np.zeros(size, dtype=np.float32)
+            v = self.v[name]
+            v[:] = (beta2 * v.astype(np.float64) + (1 - beta2) * (g * g) + eps).astype(np.float32)
+            denom = np.sqrt(v.astype(np.float64))
+        upd = g / denom
+        rms = math.sqrt(_seq_sum(upd * upd) / max(1, size))
+        clip_den = max(1.0, rms / self.clip) if self.clip > 0 else 1.0
+        step_scale = lr / clip_den
+        flat = p.reshape(-1)
+        if wd > 0:
+            flat[:] = (flat.astype(np.float64) * decay).astype(np.float32)
+        flat[:] = (flat.astype(np.float64) - step_scale * upd).astype(np.float32)
+
+    def stepParamEntries(self, entries, gradScale=1.0):
+        self._step += 1
+        for name, var in entries:
+            if var.grad is not None:
+                self._step_tensor(name, var.data.data, tuple(var.data.shape), var.grad.data, gradScale)
+
+    def state_dict(self) -> dict:
+        bufs = {}
+        for suffix, table in ((".vr", self.vr), (".vc", self.vc), (".v", self.v)):
+            for name, t in table.items():
+                bufs[name + suffix] = TD((t.size,), "f32", t.copy())
+        return {"step": self._step, "buffers": bufs}
+
+
+class SGD:
+    """optimizers.ts:546-593."""
+
+    def __init__(self, lr=0.01):
+        self.lr, self._step = lr, 0
+
+    def setLr(self, lr):
+        self.lr = lr
+
+    def stepParamEntries(self, entries, gradScale=1.0):
+        self._step += 1
+        for _, var in entries:
+            if var.grad is not None:
+                p = var.data.data
+                p[:] = (p.astype(np.float64) - self.lr * (var.grad.data.astype(np.float64) * gradScale)).astype(np.float32)
+
+    def state_dict(self) -> dict:
+        return {"step": self._step, "buffers": {}}
+
+
 @dataclass
 class TrainConfig:
     iters: int = 1
@@ -540,6 +667,7 @@ class TrainConfig:
     weightDecay: float = 0.1
     gradClip: float = 1.0
     gradAccumSteps: int = 1
+    optimizer: str = "adamw"
 
 
 def lr_at(tc: TrainConfig, step: int) -> float:
@@ -572,7 +700,18 @@ class Trainer:
         self.rng = SeededRng(seed)
         self.params = initGPT(cfg, self.B, self.rng)
         self.entries = collectParamEntries(self.params)
-        self.opt = AdamW(tc.lr, tc.beta1, tc.beta2, tc.eps, tc.weightDecay, no_decay_names(cfg.nLayer))
+        nd = no_decay_names(cfg.nLayer)
+        kind = getattr(tc, "optimizer", "adamw")                     # apps/cli/src/resolve.ts:25-36
+        if kind == "adamw":
+            self.opt = AdamW(tc.lr, tc.beta1, tc.beta2, tc.eps, tc.weightDecay, nd)
+        elif kind == "lion":
+            self.opt = Lion(tc.lr, tc.beta1, tc.beta2, tc.weightDecay, nd)
+        elif kind == "adafactor":
+            self.opt = Adafactor(lr=tc.lr, beta2=tc.beta2, eps=tc.eps, weightDecay=tc.weightDecay, noDecayNames=nd)
+        elif kind == "sgd":
+            self.opt = SGD()
+        else:
+            raise ValueError(f'Unknown optimizer: "{kind}"')
         self.tape = Tape()
         self.step_idx = 0
 

@@ -121,6 +121,23 @@ def test_loss_parity_over_steps_with_accumulation(B):
     assert math.isfinite(r.loss)          # random batches at warm-up learning rates: the loss stays near log(vocab)
 
 
+@pytest.mark.parametrize("optimizer,lr", [("lion", 1e-4), ("adafactor", 1e-3), ("sgd", 1e-2)])
+def test_training_steps_with_the_other_optimizers_match_oracle(B, optimizer, lr):
+    """Ten trainer steps (warm-up, clip folded into gradScale) with each optimizer of the reference's registry besides AdamW
+    (apps/cli/src/resolve.ts:25-36): loss within 1e-3 relative, final parameters close."""
+    from alpha2_amd.train import syntheticBatch
+    cfg = dict(vocabSize=96, blockSize=32, nLayer=2, nEmbd=64, nHead=2)
+    dev, orc = _both(B, cfg, dict(iters=10, lr=lr, optimizer=optimizer), seed=5)
+    assert dev.optimizer.name == optimizer
+    for s in range(10):
+        r, o = dev.step([syntheticBatch(300 + s, 4, 32, 96)]), orc.step([rm.synthetic_batch(300 + s, 4, 32, 96)])
+        assert abs(r.loss - o.loss) <= 1e-3 * abs(o.loss), (s, r.loss, o.loss)
+    for (n1, v1), (_, v2) in zip(dev.entries, orc.entries):
+        # Lion moves every weight by +-lr per step: a gradient entry whose sign differs within fp32 noise shifts it by 2 lr
+        tol = 2.5 * lr * 10 if optimizer == "lion" else 0.0
+        assert_close(v1.data.data, v2.data.data, rel=2e-3, what=n1, outlier_frac=0.02 if optimizer == "lion" else 0.0, outlier_abs=tol)
+
+
 def test_activation_checkpointing_matches_plain(B):
     from alpha2_amd.autograd import Tape
     from alpha2_amd.model import ModelConfig, collectParamEntries, gptForward, initGPT
