@@ -6,6 +6,8 @@ Restatement of the reference's host-side training step as it runs on its CPU bac
   * initGPT / transformerBlock / gptForward (the NON-flash branch cpu_ref takes)
                                         packages/model/src/gpt.ts:73-151, 220-333, 344-427
   * AdamW.stepParamEntries              packages/train/src/optimizers.ts:54-115
+  * sample(): token selection + loop     packages/train/src/sample.ts:36-198 (pinned in tests/test_sample.py by hand-worked
+                                        distributions with scripted rng draws)
   * Lion, Adafactor, SGD                packages/train/src/optimizers.ts:246-593 (pinned in tests/test_optimizers.py by
                                         closed forms: Lion's first step, Adafactor on a rank-one gradient, and the
                                         reference's own gradScale / entry-vs-map properties, packages/tests/src/optimizer.test.ts)
@@ -469,6 +471,105 @@ def gptForward(cfg: ModelConfig, params: dict, B: CpuRef, tape: Tape, tokens: TD
         tf = TD((Bt * T,), "i32", targets.data)
         loss = crossEntropy(ctx, reshape(ctx, logits, [Bt * T, cfg.vocabSize]), tf)
     return logits, loss
+
+
+# ---- sample.ts ----------------------------------------------------------------------------------
+
+def select_token(last: np.ndarray, rng, temperature: float, topk: int, topP: float) -> int:
+    """sample.ts:85-193, element by element as written there (plain loops: vocabularies in the tests are small).
+    `last` is the Float32Array of logits already divided by the temperature."""
+    V = last.size
+    f32 = np.float32
+    if temperature <= 0:
+        best, bestVal = 0, last[0]
+        for v in range(1, V):
+            if last[v] > bestVal:
+                bestVal, best = last[v], v
+        return best
+    if 0 < topk < V:
+        order = sorted(range(V), key=lambda i: -float(last[i]))            # stable, descending
+        threshold = last[order[topk - 1]]
+        for v in range(V):
+            if last[v] < threshold:
+                last[v] = -np.inf
+    if 0 < topP < 1:
+        maxVal = -math.inf
+        for v in range(V):
+            if last[v] > maxVal:
+                maxVal = float(last[v])
+        if math.isfinite(maxVal):
+            probs = np.zeros(V, dtype=f32)
+            active, sumExp = [], 0.0
+            for v in range(V):
+                if math.isfinite(float(last[v])):
+                    p = math.exp(float(last[v]) - maxVal)
+                    probs[v] = p
+                    active.append(v)
+                    sumExp += p
+            if sumExp > 0 and active:
+                active.sort(key=lambda i: -float(probs[i]))
+                target = sumExp * topP
+                keptMass, keepCount = 0.0, 0
+                while keepCount < len(active):
+                    keptMass += float(probs[active[keepCount]])
+                    if keptMass >= target:
+                        keepCount += 1
+                        break
+                    keepCount += 1
+                if keepCount <= 0:
+                    keepCount = 1
+                if keptMass <= 0:
+                    keptMass = float(probs[active[0]])
+                r = rng.next() * keptMass
+                cum, sampled = 0.0, active[keepCount - 1]
+                for i in range(keepCount):
+                    cum += float(probs[active[i]])
+                    if r < cum:
+                        sampled = active[i]
+                        break
+                return sampled
+    maxVal = -math.inf
+    for v in range(V):
+        if last[v] > maxVal:
+            maxVal = float(last[v])
+    probs = np.zeros(V, dtype=f32)
+    sumExp = 0.0
+    for v in range(V):
+        probs[v] = math.exp(float(last[v]) - maxVal) if last[v] != -np.inf else 0.0
+        sumExp += float(probs[v])
+    for v in range(V):
+        probs[v] = float(probs[v]) / sumExp
+    r = rng.next()
+    cum = 0.0
+    for v in range(V):
+        cum += float(probs[v])
+        if r < cum:
+            return v
+    return 0
+
+
+def sample_tokens(cfg: ModelConfig, params: dict, B: CpuRef, rng, prompt, steps: int, temperature: float, topk: int, topp=1.0) -> np.ndarray:
+    """sample.ts:36-198 without the tokenizer."""
+    topP = min(1.0, max(0.0, topp)) if (topp is not None and math.isfinite(topp)) else 1.0
+    prompt = np.asarray(prompt, dtype=np.int32)
+    maxLen = min(prompt.size + steps, cfg.blockSize)
+    tokens = np.zeros(maxLen, dtype=np.int32)
+    tokens[:prompt.size] = prompt
+    cur = int(prompt.size)
+    for _ in range(steps):
+        if cur >= cfg.blockSize:
+            break
+        start = max(0, cur - cfg.blockSize)
+        ctx = tokens[start:cur].copy()
+        logits, _ = gptForward(cfg, params, B, Tape(), TD((1, ctx.size), "i32", ctx))
+        last = np.array(logits.data.data.reshape(-1)[(ctx.size - 1) * cfg.vocabSize:], dtype=np.float32)
+        if temperature > 0:
+            last = (last.astype(np.float64) / temperature).astype(np.float32)
+        nxt = select_token(last, rng, temperature, topk, topP)
+        if cur < maxLen:
+            tokens[cur] = nxt
+            cur += 1
+    return tokens[:cur]
 
 
 # ---- optimizers.ts / trainer.ts -----------------------------------------------------------------
