@@ -368,6 +368,70 @@ __global__ void k_ce_bwd(const T *__restrict__ logits, const int32_t *__restrict
   }
 }
 
+// Forward and backward of the loss in ONE pass over bf16 logits: the block keeps its whole row in registers (up to
+// CE_CHUNKS 16-byte chunks per thread), so the logits are read once instead of twice.  Same per-thread order of the online
+// (max, sum) updates and the same expressions as k_ce_fwd / k_ce_bwd: results are bit-identical to that pair.
+constexpr int CE_CHUNKS = 25;            // 25 x 256 threads x 8 classes = 51200 classes per row
+__global__ __launch_bounds__(256) void k_ce_fwd_bwd(const uint16_t *__restrict__ logits, const int32_t *__restrict__ targets,
+                                                    float *__restrict__ row_loss, float *__restrict__ lse_out, const float *__restrict__ g,
+                                                    float g_mul, uint16_t *__restrict__ out, int64_t n, int64_t c) {
+  __shared__ float shm[WPB], shs[WPB], sh_lse;
+  const int64_t row = blockIdx.x;
+  const uint16_t *p = logits + row * c;
+  const int nvec = (int)(c >> 3);
+  uint4 r[CE_CHUNKS];
+  float m = -INFINITY, s = 0.f;
+#pragma unroll
+  for (int k = 0; k < CE_CHUNKS; k++) {
+    const int j = threadIdx.x + k * 256;
+    if (j < nvec) {
+      const uint4 u = reinterpret_cast<const uint4 *>(p)[j];
+      r[k] = u;
+      float v[8] = {bf16_bits_to_f32(u.x & 0xffff), bf16_bits_to_f32(u.x >> 16), bf16_bits_to_f32(u.y & 0xffff), bf16_bits_to_f32(u.y >> 16),
+                    bf16_bits_to_f32(u.z & 0xffff), bf16_bits_to_f32(u.z >> 16), bf16_bits_to_f32(u.w & 0xffff), bf16_bits_to_f32(u.w >> 16)};
+      float vm = v[0];
+#pragma unroll
+      for (int i = 1; i < 8; i++) vm = fmaxf(vm, v[i]);
+      if (vm > m) { s *= __expf(m - vm); m = vm; }
+#pragma unroll
+      for (int i = 0; i < 8; i++) s += __expf(v[i] - m);
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) online_merge(m, s, __shfl_xor(m, off, 64), __shfl_xor(s, off, 64));
+  const int wv = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  if (lane == 0) { shm[wv] = m; shs[wv] = s; }
+  __syncthreads();
+  const int32_t t = targets[row];
+  if (threadIdx.x == 0) {
+    for (int k = 1; k < WPB; k++) online_merge(m, s, shm[k], shs[k]);
+    const float lse = m + logf(s);
+    const float picked = (t >= 0 && t < c) ? bf16_bits_to_f32(p[t]) : lse;     // an out-of-range target contributes 0 loss
+    row_loss[row] = lse - picked;
+    if (lse_out) lse_out[row] = lse;
+    sh_lse = lse;
+  }
+  __syncthreads();
+  const float l = sh_lse, scale = (g ? g[0] : 1.0f) * g_mul / (float)n;
+  uint16_t *q = out + row * c;
+#pragma unroll
+  for (int k = 0; k < CE_CHUNKS; k++) {
+    const int j8 = threadIdx.x + k * 256;
+    if (j8 < nvec) {
+      const uint32_t in[4] = {r[k].x, r[k].y, r[k].z, r[k].w};
+      uint32_t o[4];
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const int64_t j = (int64_t)j8 * 8 + 2 * i;
+        const float a = (__expf(bf16_bits_to_f32(in[i] & 0xffff) - l) - (j == t ? 1.0f : 0.0f)) * scale;
+        const float b = (__expf(bf16_bits_to_f32(in[i] >> 16) - l) - (j + 1 == t ? 1.0f : 0.0f)) * scale;
+        o[i] = pack_bf16x2(a, b);
+      }
+      reinterpret_cast<uint4 *>(q)[j8] = make_uint4(o[0], o[1], o[2], o[3]);
+    }
+  }
+}
+
 // Token windows of a device-resident corpus: one block row per batch item, modulo indexing reproduces the packed
 // loader's wrap-around (and is a no-op for random windows, which never reach the end of the corpus).
 __global__ void k_token_windows(const int32_t *__restrict__ corpus, int64_t n_tokens, const int64_t *__restrict__ starts, int64_t T,
@@ -559,6 +623,29 @@ int32_t ah_cross_entropy_bwd(ah_ptr logits, int32_t dtype, ah_ptr targets, ah_pt
                          dp<const int32_t>(targets) + r0, dp<const float>(lse) + r0, dp<const float>(g_scalar), g_mul, dp<uint16_t>(dl), n, c);
     AH_LAUNCH_CHECK();
   }
+  return AH_OK;
+}
+
+int32_t ah_cross_entropy_fwd_bwd(ah_ptr logits, int32_t dtype, ah_ptr targets, ah_ptr loss_out, ah_ptr lse_out, ah_ptr g_scalar, float g_mul,
+                                 ah_ptr dlogits, int64_t n, int64_t c) {
+  AH_REQUIRE_READY();
+  AH_ARG(dtype == AH_F32 || dtype == AH_BF16, "ah_cross_entropy_fwd_bwd: logits dtype must be f32 or bf16");
+  AH_ARG(loss_out != 0, "ah_cross_entropy_fwd_bwd: null loss_out");
+  AH_ARG(n > 0 && c > 0, "ah_cross_entropy_fwd_bwd: empty logits [%lld, %lld]", (long long)n, (long long)c);
+  AH_ARG(logits && targets && lse_out && dlogits, "ah_cross_entropy_fwd_bwd: null operand");
+  AH_ARG(n < (int64_t(1) << 31), "ah_cross_entropy_fwd_bwd: too many rows");
+  const bool one_pass = dtype == AH_BF16 && (c & 7) == 0 && (c >> 3) <= (int64_t)CE_CHUNKS * 256 && ((logits | dlogits) & 15u) == 0;
+  if (!one_pass) {                // rows that do not fit the registers of a block, f32 logits, odd alignments: the two kernels
+    int32_t rc = ah_cross_entropy(logits, dtype, targets, loss_out, lse_out, n, c);
+    return rc ? rc : ah_cross_entropy_bwd(logits, dtype, targets, lse_out, g_scalar, g_mul, dlogits, n, c);
+  }
+  float *rows = (float *)scratch(sizeof(float) * (size_t)n);
+  if (!rows) return fail(AH_ERR_OOM, "ah_cross_entropy_fwd_bwd: no scratch");
+  hipLaunchKernelGGL(k_ce_fwd_bwd, dim3((unsigned)n), dim3(256), 0, stream(), dp<const uint16_t>(logits), dp<const int32_t>(targets), rows,
+                     dp<float>(lse_out), dp<const float>(g_scalar), g_mul, dp<uint16_t>(dlogits), n, c);
+  AH_LAUNCH_CHECK();
+  hipLaunchKernelGGL(k_mean_rows, dim3(1), dim3(TPB), 0, stream(), rows, n, dp<float>(loss_out));
+  AH_LAUNCH_CHECK();
   return AH_OK;
 }
 

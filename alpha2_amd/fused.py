@@ -229,14 +229,14 @@ class FusedTrainer:
             self._gemm(NT, self.hact[l], self.p(pre + "mlp.fc2", True), self.x[l + 1], BT, Cc, Fd, Fd, Fd, Cc, F32, ffi.EPI_RESIDUAL, self.xmid[l])
         check(lib.ah_layernorm(self.x[L], self.p("lnF.weight"), self.p("lnF.bias"), self.lnf, BT, Cc, 1e-5, BF16))
         self._gemm(NT, self.lnf, self.p("lmHead", True), self.logits, BT, V, Cc, Cc, Cc, V)
+        # loss and dlogits (in place) from one read of the logits
         if self.accum == 1:
-            check(lib.ah_cross_entropy(self.logits, BF16, self.tgt, self.loss, self.rowlse, BT, V))
+            check(lib.ah_cross_entropy_fwd_bwd(self.logits, BF16, self.tgt, self.loss, self.rowlse, 0, 1.0, self.logits, BT, V))
         else:                                     # reported loss = mean of the micro-step losses (trainer.ts:1270-1273)
-            check(lib.ah_cross_entropy(self.logits, BF16, self.tgt, self.loss_micro, self.rowlse, BT, V))
+            check(lib.ah_cross_entropy_fwd_bwd(self.logits, BF16, self.tgt, self.loss_micro, self.rowlse, 0, 1.0, self.logits, BT, V))
             if first_micro:
                 check(lib.ah_fill_f32(self.loss, 0.0, 1))
             check(lib.ah_axpy_inplace(self.loss, self.loss_micro, 1.0 / self.accum, 1))
-        check(lib.ah_cross_entropy_bwd(self.logits, BF16, self.tgt, self.rowlse, 0, 1.0, self.logits, BT, V))     # dlogits in place
 
         self._gemm(NN, self.logits, self.p("lmHead", True), self.dlnb, BT, Cc, V, V, Cc, Cc)
         cur = 0

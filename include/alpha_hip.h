@@ -195,6 +195,11 @@ int32_t ah_cross_entropy(ah_ptr logits, int32_t logits_dtype, ah_ptr targets_i32
 /* dlogits = (softmax - onehot) * g[0] * g_mul / N; g_scalar = device f32 (0 = use 1.0); may run in place */
 int32_t ah_cross_entropy_bwd(ah_ptr logits, int32_t dtype, ah_ptr targets_i32, ah_ptr lse, ah_ptr g_scalar,
                              float g_mul, ah_ptr dlogits, int64_t n, int64_t c);
+/* Both of the above in one launch (crossEntropy + crossEntropyBackward, interfaces.ts:74,104; the backward of the loss
+ * does not depend on its value): bf16 rows of up to 51200 classes are read ONCE, kept in registers between the two
+ * halves, and the results are bit-identical to the pair; anything else runs the pair.  May run in place. */
+int32_t ah_cross_entropy_fwd_bwd(ah_ptr logits, int32_t dtype, ah_ptr targets_i32, ah_ptr loss_out, ah_ptr lse_out,
+                                 ah_ptr g_scalar, float g_mul, ah_ptr dlogits, int64_t n, int64_t c);
 
 /* ---- GEMM on MFMA.  Backend.matmul / matmulTransposed / matmulTransposedA (cpu_ref.ts:166-258;
  *      interfaces.ts:111-112; autograd use ops.ts:197-234).  C[M,N] = op(A) * op(B):

@@ -262,6 +262,46 @@ def test_cross_entropy_fwd_bwd(B, n, c):
     assert_close(B.crossEntropyBackward(fresh, tgd, gs).data, ref.cross_entropy_backward(orc(lg), orc(tg), 0.7).data, what="ce.bwd2")
 
 
+@pytest.mark.parametrize("n,c,dtype", [(7, 8, "bf16"), (33, 2056, "bf16"), (12, 50304, "bf16"), (5, 51200, "bf16"), (3, 51208, "bf16"), (9, 100, "bf16"),
+                                       (11, 37, "f32")])
+def test_cross_entropy_one_pass_equals_forward_then_backward(B, n, c, dtype):
+    """ah_cross_entropy_fwd_bwd keeps a bf16 row in registers between the two halves (rows of up to 51200 classes, a multiple
+    of 8) and otherwise runs the two kernels: loss, lse and dlogits are bit-identical to the pair either way, also in
+    place and with an out-of-range target; the values are checked against the oracle on the logits as stored."""
+    from alpha2_amd import _ffi as ffi
+    code = ffi.DTYPE_CODE[dtype]
+    lg = (rs.randn(n, c) * 3).astype(np.float32)
+    logits = lambda: B.castStore(dev(B, lg), dtype)
+    seen = np.array(logits().data, dtype=np.float32).reshape(n, c)
+
+    def run(entry, tg, inplace=False):
+        src, tgd = logits(), dev(B, tg, "i32")
+        loss, lse = B._new(()), B._new((n,))
+        dl = src if inplace else B._new((n, c), "f32", dtype)
+        if entry == "pair":
+            ffi.check(B.lib.ah_cross_entropy(B._ptr(src), code, B._ptr(tgd), B._ptr(loss), B._ptr(lse), n, c))
+            ffi.check(B.lib.ah_cross_entropy_bwd(B._ptr(src), code, B._ptr(tgd), B._ptr(lse), 0, 0.7, B._ptr(dl), n, c))
+        else:
+            ffi.check(B.lib.ah_cross_entropy_fwd_bwd(B._ptr(src), code, B._ptr(tgd), B._ptr(loss), B._ptr(lse), 0, 0.7, B._ptr(dl), n, c))
+        B._dirty(dl)
+        return [np.array(t.data).copy() for t in (loss, lse, dl)]
+
+    tg = rs.randint(0, c, n).astype(np.int32)
+    tg[-1] = c - 1
+    bad = tg.copy()
+    bad[0] = -1
+    for targets in (tg, bad):
+        want = run("pair", targets)
+        for inplace in (False, True):
+            for got, exp, what in zip(run("one", targets, inplace), want, ("loss", "lse", "dlogits")):
+                assert np.array_equal(got, exp), (what, inplace)
+    loss, _, dl = run("one", tg)
+    half = 2.0 ** -8 if dtype == "bf16" else 0.0               # rounding of the stored gradient
+    assert_close(loss, O.crossEntropy(orc(seen), orc(tg)).data, what="ce")
+    wantg = ref.cross_entropy_backward(orc(seen), orc(tg), 0.7).data
+    assert np.all(np.abs(dl - wantg) <= np.abs(wantg) * (half + 1e-4) + 1e-9), "ce.dlogits"
+
+
 @pytest.mark.parametrize("M,K,N", [(2, 2, 2), (33, 19, 47), (64, 64, 64), (128, 128, 128), (256, 256, 256), (1024, 128, 384), (130, 515, 257)])
 def test_gemm_f32_all_layouts(B, M, K, N):
     a, b = rs.randn(M, K).astype(np.float32), rs.randn(K, N).astype(np.float32)
@@ -393,8 +433,6 @@ def _bf16_round(x):
 
 def _raw_gemm(B, layout, a, b, m, n, k, in_dtype, out_dtype, epi=0, aux=None, c_init=None):
     """ah_gemm through the C ABI on raw buffers; returns C (f32 values) and aux-out if the epilogue writes one."""
-    import ctypes as C
-    from alpha2_amd import TensorData, _ffi as ffi
 
     def up(arr, store):
         if store == ffi.BF16:
@@ -548,8 +586,6 @@ def test_gemm_bf16_large_tiles_direct_to_lds_kernel(B, M, N, K, tile):
 def test_gemm_grouped_matches_separate_products(B):
     """One grouped launch over problems of different sizes (ragged tile edges, NONE then ACCUM) against float64 numpy
     products of the same bf16-exact operands; descriptor errors are reported, not launched."""
-    import ctypes as C
-    from alpha2_amd import TensorData, _ffi as ffi
     K = 640
     shapes = [(768, 768), (264, 520), (2304, 768), (8, 8), (1000, 256)]
     keep, descs, wants, outs = [], [], [], []
