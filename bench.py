@@ -2,7 +2,10 @@
 """Headline benchmark: training tokens/s of the GPT-2-small-shape step (vocab 50304, d 768, 12 layers, 12 heads,
 ctx 1024, batch 16; forward + backward + AdamW with gradient clipping) on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--mode fast|parity] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--mode fast|parity] [--no-cpu] [--workload gpt2-small|gpt-350m]
+
+The default workload is the one the metric is quoted on; `--workload gpt-350m` runs the 350M-shape step (d 1024, 24 layers,
+16 heads, batch 8 with 4 accumulated micro-steps, whole step in one hipGraph) and reports it the same way.
 
 Prints ONE JSON line.  `value` is tokens/s with parameters, optimizer state and the token batch already resident in
 HBM.  `roofline` is for the dominant kernel, the MFMA GEMM instantiation that does the most arithmetic in a step (which is
@@ -24,6 +27,13 @@ sys.path.insert(0, ROOT)
 
 GPT2 = dict(vocabSize=50304, blockSize=1024, nLayer=12, nEmbd=768, nHead=12)
 BATCH = 16
+WORKLOADS = {        # name -> (model, micro-batch, accumulated micro-steps, token seed, description)
+    "gpt2-small": (GPT2, BATCH, 1, 4, "GPT-2-small-shape train step: vocab 50304, d_model 768, 12 layers, 12 heads, ctx 1024, batch 16, "
+                                      "untied lmHead (163.0M params), AdamW lr 3e-4 betas (0.9,0.95) wd 0.1, grad-clip 1.0"),
+    "gpt-350m": (dict(vocabSize=50304, blockSize=1024, nLayer=24, nEmbd=1024, nHead=16), 8, 4, 5,
+                 "350M-shape train step: vocab 50304, d_model 1024, 24 layers, 16 heads, ctx 1024, batch 8 x 4 accumulated micro-steps, "
+                 "untied lmHead (406.2M params), AdamW lr 3e-4 betas (0.9,0.95) wd 0.1, grad-clip 1.0"),
+}
 PEAK = {"bf16": 2500.0, "f32": 157.3}          # MI355X dense MFMA, TFLOP/s
 # HBM-side bytes per launch of the kernels that can be the dominant one, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
 # runs of this benchmark (counter values scaled by what the same counters read for a plain copy of known size: x2.0
@@ -39,17 +49,17 @@ def step_flops(cfg, tokens):
     return (6 * p_mm + 12 * L * T * C_) * tokens
 
 
-def cpu_baseline(seq_tokens: int):
+def cpu_baseline(model: dict, seq_tokens: int):
     """Oracle (port of the reference CPU path), one thread, on the SAME model with 1 sequence of `seq_tokens` tokens."""
     from oracle import ref_model as rm
-    cfg = rm.ModelConfig(**GPT2)
+    cfg = rm.ModelConfig(**model)
     tr = rm.Trainer(cfg, rm.TrainConfig(iters=50), seed=0)
     batch = rm.synthetic_batch(4, 1, seq_tokens, cfg.vocabSize)
     t0 = time.perf_counter()
     r = tr.step([batch])
     dt = time.perf_counter() - t0
     return {"value": seq_tokens / dt, "unit": "tokens/s", "cores": 1, "kind": "port",
-            "sample": f"same model (163.0M params), 1 sequence x {seq_tokens} tokens, one full step "
+            "sample": f"same model ({sum(v.data.data.size for _, v in tr.entries) / 1e6:.1f}M params), 1 sequence x {seq_tokens} tokens, one full step "
                       f"(forward+backward+clip+AdamW) in {dt:.1f} s; loss {r.loss:.4f}"}
 
 
@@ -61,6 +71,7 @@ def main():
     ap.add_argument("--mode", choices=["fast", "parity"], default="fast")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--cpu-tokens", type=int, default=32)
+    ap.add_argument("--workload", choices=sorted(WORKLOADS), default="gpt2-small")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs the step on ONE GPU; --gpus must be 1 (no multi-GPU path exists in this run)", file=sys.stderr)
@@ -71,24 +82,26 @@ def main():
     from alpha2_amd.train import TrainConfig, zipfBatch
 
     B = HipBackend(0)
-    cfg = ModelConfig(**GPT2)
-    tc = TrainConfig(iters=50, batchSize=BATCH)
-    tokens = BATCH * cfg.blockSize
+    model, BATCH, accum, tok_seed, describe = WORKLOADS[args.workload]
+    cfg = ModelConfig(**model)
+    tc = TrainConfig(iters=50, batchSize=BATCH, gradAccumSteps=accum)
+    tokens = BATCH * cfg.blockSize * accum
+    micro = [zipfBatch(tok_seed + 100 * m, BATCH, cfg.blockSize, cfg.vocabSize) for m in range(accum)]
     if args.mode == "parity":
         from alpha2_amd.train import Trainer
         runner = Trainer(B, cfg, tc, seed=0)
         dtype = "f32"
-        batch = zipfBatch(4, BATCH, cfg.blockSize, cfg.vocabSize)
-        B._ptr(batch[0]), B._ptr(batch[1])
+        for x, y in micro:
+            B._ptr(x), B._ptr(y)
 
         def one_step():
             # the generic trainer releases its batch after use; keep ours resident by handing it views
-            return runner.step([(B.reshape(batch[0], batch[0].shape), B.reshape(batch[1], batch[1].shape))])
+            return runner.step([(B.reshape(x, x.shape), B.reshape(y, y.shape)) for x, y in micro])
     else:
         from alpha2_amd.fused import FusedTrainer
-        runner = FusedTrainer(B, cfg, tc, BATCH, seed=0)
+        runner = FusedTrainer(B, cfg, tc, BATCH, seed=0, accum=accum)
         dtype = "bf16"
-        runner.set_batch(*zipfBatch(4, BATCH, cfg.blockSize, cfg.vocabSize))
+        runner._use_batch([runner.add_batch(x, y) for x, y in micro])      # resident: step() keeps training on them
         one_step = runner.step
 
     losses = []
@@ -120,24 +133,23 @@ def main():
             grp["flops"] += r["flops"]; grp["ms"] += r["ms"]; grp["n"] += 1
     dom_name, dom = max(groups.items(), key=lambda kv: (kv[1]["flops"], kv[1]["ms"]))
     achieved = dom["flops"] / (dom["ms"] * 1e-3) / 1e12
-    flops = step_flops(GPT2, tokens)
+    flops = step_flops(model, tokens)
     out = {
         "metric": "train tokens/sec + MFMA util % on GPT-124M step, 1xMI355X", "value": tokens / (ms * 1e-3), "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic (Zipf s=1.1 token ids, seed 4; random-init N(0,0.02) weights, seed 0)",
-        "config": {"workload": "GPT-2-small-shape train step: vocab 50304, d_model 768, 12 layers, 12 heads, ctx 1024, batch 16, "
-                               "untied lmHead (163.0M params), AdamW lr 3e-4 betas (0.9,0.95) wd 0.1, grad-clip 1.0",
+        "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": f"synthetic (Zipf s=1.1 token ids, seed {tok_seed}; random-init N(0,0.02) weights, seed 0)",
+        "config": {"workload": describe,
                    "tokens_per_step": tokens, "mode": args.mode, "loss_first_step": loss_first, "loss_last_step": loss_last},
         "step_tflops": flops / (ms * 1e-3) / 1e12, "mfu_vs_bf16_dense_peak": flops / (ms * 1e-3) / 1e12 / PEAK["bf16"],
         "mfma_util_pct": 100.0 * flops / (ms * 1e-3) / 1e12 / PEAK["bf16"],
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK[dtype], "unit": "TFLOP/s", "frac": achieved / PEAK[dtype],
-                     "traffic": TRAFFIC_BYTES.get(dom_name), "kernel": dom_name, "launches_per_step": dom["n"], "avg_launch_us": dom["ms"] / dom["n"] * 1e3,
+                     "traffic": TRAFFIC_BYTES.get(dom_name) if args.workload == "gpt2-small" else None, "kernel": dom_name, "launches_per_step": dom["n"], "avg_launch_us": dom["ms"] / dom["n"] * 1e3,
                      "flops_per_launch": dom["flops"] / dom["n"], "ms_per_step": dom["ms"],
                      "all_gemm": {"launches_per_step": len(gemm), "ms_per_step": g_ms,
                                   "achieved": g_flops / (g_ms * 1e-3) / 1e12 if g_ms > 0 else 0.0}},
     }
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(args.cpu_tokens)
+        out["cpu_baseline"] = cpu_baseline(model, args.cpu_tokens)
     print(json.dumps(out))
 
 

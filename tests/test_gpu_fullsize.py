@@ -1,0 +1,81 @@
+"""The two full-size training workloads (GPT-2-small shape at batch 16; 350M shape at batch 8 with 4 micro-steps) through
+properties that do not need the CPU oracle, which would take hours at these sizes:
+
+* the loss of a freshly initialised model has a closed form: the logits of a pre-LayerNorm model with N(0, 0.02) weights
+  are ~N(0, s2) with s2 = 0.02^2 * nEmbd per class (the final LayerNorm output has unit variance), so the expected loss is
+  ln V + s2 / 2 (the mean of a log-sum-exp of V Gaussians, V >> e^s2);
+* hipGraph replay of the step and eager execution of the same kernels agree;
+* gradient accumulation is linear: K micro-steps on the SAME batch give the gradient norm, loss and update of one
+  (micro-batch gradients are summed and scaled by 1/K once: trainer.ts:1164-1273);
+* clipping: after a step whose gradient norm exceeded the clip, clipCoef * gradNorm == clip (trainer.ts:1650-1656).
+"""
+import math
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+SMALL = dict(vocabSize=50304, blockSize=1024, nLayer=12, nEmbd=768, nHead=12)
+M350 = dict(vocabSize=50304, blockSize=1024, nLayer=24, nEmbd=1024, nHead=16)
+
+
+@pytest.fixture(scope="module")
+def B():
+    from alpha2_amd import HipBackend
+    return HipBackend(0)
+
+
+def _trainer(B, cfg, batch, accum, graph):
+    from alpha2_amd.fused import FusedTrainer
+    from alpha2_amd.model import ModelConfig
+    from alpha2_amd.train import TrainConfig
+    return FusedTrainer(B, ModelConfig(**cfg), TrainConfig(iters=50, batchSize=batch, gradAccumSteps=accum), batch, seed=0,
+                        use_graph=graph, accum=accum)
+
+
+def _expected_initial_loss(cfg):
+    return math.log(cfg["vocabSize"]) + 0.5 * 0.02 ** 2 * cfg["nEmbd"]
+
+
+@pytest.mark.parametrize("name,cfg,batch,accum,seed", [("gpt2-small", SMALL, 16, 1, 4), ("350m", M350, 8, 4, 5)])
+def test_full_size_step_properties(B, name, cfg, batch, accum, seed):
+    from alpha2_amd.train import zipfBatch
+    steps = 6                                             # past the spike that the first warm-up steps make
+    graph, eager = _trainer(B, cfg, batch, accum, True), _trainer(B, cfg, batch, accum, False)
+    batches = [zipfBatch(seed + 100 * m, batch, cfg["blockSize"], cfg["vocabSize"]) for m in range(accum)]
+    ig = [graph.add_batch(*b) for b in batches]
+    ie = [eager.add_batch(*b) for b in batches]
+    for _ in range(steps):
+        graph.step(ig if accum > 1 else ig[0])
+        eager.step(ie if accum > 1 else ie[0])
+    hg, he = graph.history(0, steps), eager.history(0, steps)
+    assert abs(hg[0].loss - _expected_initial_loss(cfg)) < 0.08, (hg[0].loss, _expected_initial_loss(cfg))
+    for s in range(steps):
+        assert math.isfinite(hg[s].loss) and math.isfinite(hg[s].gradNorm)
+        assert abs(hg[s].loss - he[s].loss) <= 1e-4 * abs(he[s].loss), (s, hg[s].loss, he[s].loss)
+        assert abs(hg[s].gradNorm - he[s].gradNorm) <= 2e-3 * he[s].gradNorm, (s, hg[s].gradNorm, he[s].gradNorm)
+        if hg[s].gradNorm > 1.0:
+            assert abs(hg[s].clipCoef * hg[s].gradNorm - 1.0) < 1e-5, s
+        else:
+            assert hg[s].clipCoef == 1.0
+    assert hg[-1].loss < hg[0].loss                       # the same batches every step: the loss must fall
+    graph.close(), eager.close()
+
+
+def test_accumulating_one_batch_four_times_equals_one_micro_step(B):
+    """350M shape: 4 micro-steps on the same batch vs one micro-step on it."""
+    from alpha2_amd.train import zipfBatch
+    one, four = _trainer(B, M350, 8, 1, False), _trainer(B, M350, 8, 4, False)
+    b = zipfBatch(5, 8, 1024, 50304)
+    i1 = one.add_batch(*b)
+    i4 = [four.add_batch(*b)] * 4
+    one.step(i1)
+    four.step(i4)
+    h1, h4 = one.history(0, 1)[0], four.history(0, 1)[0]
+    assert abs(h1.loss - h4.loss) <= 1e-6 * abs(h1.loss), (h1.loss, h4.loss)
+    assert abs(h1.gradNorm - h4.gradNorm) <= 1e-4 * h1.gradNorm, (h1.gradNorm, h4.gradNorm)
+    for pname in ("wte", "layer.23.attn.wqkv", "layer.0.mlp.fc2", "lmHead", "lnF.weight"):
+        a, c = one.param(pname), four.param(pname)
+        assert np.max(np.abs(a - c)) <= 2e-6 + 1e-3 * 3e-4, pname          # AdamW's first step moves every entry by ~lr
+    one.close(), four.close()
