@@ -193,12 +193,25 @@ __global__ __launch_bounds__(1024) void k_colsum_partials(const float *__restric
 
 // Register-resident LayerNorm backward for rows of up to 256*NV floats (dim % 4 == 0): x, g and the residual gradient
 // are each read once; dw / db accumulate in per-lane registers over all rows a wave walks.
-template <class G> __device__ __forceinline__ float4 ld4(const G *p, int j);
-template <> __device__ __forceinline__ float4 ld4<float>(const float *p, int j) { return reinterpret_cast<const float4 *>(p)[j]; }
-template <> __device__ __forceinline__ float4 ld4<uint16_t>(const uint16_t *p, int j) {
-  uint2 u = reinterpret_cast<const uint2 *>(p)[j];
-  return make_float4(bf16_bits_to_f32(u.x & 0xffff), bf16_bits_to_f32(u.x >> 16), bf16_bits_to_f32(u.y & 0xffff), bf16_bits_to_f32(u.y >> 16));
-}
+// four gradient values as loaded (f32: 16 bytes, bf16: 8 bytes) and widened to float4 at the point of use
+template <class G> struct Raw4;
+template <> struct Raw4<float> {
+  float4 v;
+  __device__ __forceinline__ void load(const float *p, int j) { v = reinterpret_cast<const float4 *>(p)[j]; }
+  __device__ __forceinline__ void zero() { v = make_float4(0, 0, 0, 0); }
+  __device__ __forceinline__ float4 get() const { return v; }
+};
+template <> struct Raw4<uint16_t> {
+  uint2 v;
+  __device__ __forceinline__ void load(const uint16_t *p, int j) { v = reinterpret_cast<const uint2 *>(p)[j]; }
+  __device__ __forceinline__ void zero() { v = make_uint2(0, 0); }
+  __device__ __forceinline__ float4 get() const {
+    return make_float4(bf16_bits_to_f32(v.x & 0xffff), bf16_bits_to_f32(v.x >> 16), bf16_bits_to_f32(v.y & 0xffff), bf16_bits_to_f32(v.y >> 16));
+  }
+};
+// A wave walks its rows with the NEXT row's x, g and residual gradient already in flight while it reduces the current
+// one: a row is three dependent wave reductions long, and with the few waves per SIMD that the register-resident
+// column sums allow, nothing else would cover the load latency.
 template <int NV, class G>
 __global__ __launch_bounds__(256) void k_layernorm_bwd_vec(const float *__restrict__ x, const float *__restrict__ w, const G *__restrict__ g,
                                                            const float *__restrict__ res, float *__restrict__ dx, uint16_t *__restrict__ dx16,
@@ -213,18 +226,32 @@ __global__ __launch_bounds__(256) void k_layernorm_bwd_vec(const float *__restri
     wv[i] = j < nv ? reinterpret_cast<const float4 *>(w)[j] : make_float4(0, 0, 0, 0);
     adw[i] = make_float4(0, 0, 0, 0); adb[i] = make_float4(0, 0, 0, 0);
   }
-  int64_t stride = (int64_t)gridDim.x * WPB;
-  for (int64_t row = blockIdx.x * (int64_t)WPB + wave; row < rows; row += stride) {
+  float4 xv[NV], rv[NV], nx[NV], nr[NV];
+  Raw4<G> gr[NV], ng[NV];
+  auto load_row = [&](int64_t row, float4 (&xo)[NV], Raw4<G> (&go)[NV], float4 (&ro)[NV]) {
     const float *xr = x + row * (int64_t)dim;
-    const G *gr = g + row * (int64_t)dim;
-    float4 xv[NV], gv[NV];
-    float s = 0.f;
+    const G *grow = g + row * (int64_t)dim;
 #pragma unroll
     for (int i = 0; i < NV; i++) {
       int j = lane + 64 * i;
-      bool ok = j < nv;
-      xv[i] = ok ? reinterpret_cast<const float4 *>(xr)[j] : make_float4(0, 0, 0, 0);
-      gv[i] = ok ? ld4<G>(gr, j) : make_float4(0, 0, 0, 0);
+      if (j < nv) {
+        xo[i] = reinterpret_cast<const float4 *>(xr)[j];
+        go[i].load(grow, j);
+        ro[i] = res ? reinterpret_cast<const float4 *>(res + row * (int64_t)dim)[j] : make_float4(0, 0, 0, 0);
+      } else {
+        xo[i] = make_float4(0, 0, 0, 0); go[i].zero(); ro[i] = make_float4(0, 0, 0, 0);
+      }
+    }
+  };
+  int64_t stride = (int64_t)gridDim.x * WPB, row = blockIdx.x * (int64_t)WPB + wave;
+  if (row < rows) load_row(row, xv, gr, rv);
+  for (; row < rows; row += stride) {
+    if (row + stride < rows) load_row(row + stride, nx, ng, nr);
+    float4 gv[NV];
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+      gv[i] = gr[i].get();
       s += (xv[i].x + xv[i].y) + (xv[i].z + xv[i].w);
     }
     float mean = wave_sum(s) * inv_dim, q = 0.f;
@@ -252,11 +279,13 @@ __global__ __launch_bounds__(256) void k_layernorm_bwd_vec(const float *__restri
         float4 d;
         d.x = rstd * (gv[i].x * wv[i].x - (s1 + xv[i].x * s2)); d.y = rstd * (gv[i].y * wv[i].y - (s1 + xv[i].y * s2));
         d.z = rstd * (gv[i].z * wv[i].z - (s1 + xv[i].z * s2)); d.w = rstd * (gv[i].w * wv[i].w - (s1 + xv[i].w * s2));
-        if (res) { float4 r = reinterpret_cast<const float4 *>(res + row * (int64_t)dim)[j]; d.x += r.x; d.y += r.y; d.z += r.z; d.w += r.w; }
+        if (res) { d.x += rv[i].x; d.y += rv[i].y; d.z += rv[i].z; d.w += rv[i].w; }
         reinterpret_cast<float4 *>(dx + row * (int64_t)dim)[j] = d;
         if (dx16) reinterpret_cast<uint2 *>(dx16 + row * (int64_t)dim)[j] = make_uint2(pack_bf16x2(d.x, d.y), pack_bf16x2(d.z, d.w));
       }
     }
+#pragma unroll
+    for (int i = 0; i < NV; i++) { xv[i] = nx[i]; gr[i] = ng[i]; rv[i] = nr[i]; }
   }
 #pragma unroll
   for (int i = 0; i < NV; i++) {
@@ -551,8 +580,14 @@ int32_t ah_layernorm_bwd(ah_ptr x, ah_ptr w, ah_ptr grad_out, int32_t grad_dtype
   AH_ARG(x && w && grad_out && dx, "ah_layernorm_bwd: null operand");
   size_t lds = sizeof(float) * 2 * WPB * (size_t)dim;
   AH_ARG(lds <= 160 * 1024, "ah_layernorm_bwd: dim %lld too large for the LDS column accumulators", (long long)dim);
-  int nblk = (int)cdiv(rows, WPB * 8);            // >= 8 rows per wave amortises the partial write
-  int cap = num_cus() * 2;
+#ifndef LNB_ROWS
+#define LNB_ROWS 8
+#endif
+#ifndef LNB_CAP
+#define LNB_CAP 2
+#endif
+  int nblk = (int)cdiv(rows, WPB * LNB_ROWS);     // >= 8 rows per wave amortises the partial write
+  int cap = num_cus() * LNB_CAP;
   if (nblk > cap) nblk = cap;
   if (nblk < 1) nblk = 1;
   float *part = (float *)scratch(sizeof(float) * 2 * (size_t)nblk * (size_t)dim);

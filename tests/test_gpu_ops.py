@@ -433,6 +433,8 @@ def _bf16_round(x):
 
 def _raw_gemm(B, layout, a, b, m, n, k, in_dtype, out_dtype, epi=0, aux=None, c_init=None):
     """ah_gemm through the C ABI on raw buffers; returns C (f32 values) and aux-out if the epilogue writes one."""
+    import ctypes as C
+    from alpha2_amd import TensorData, _ffi as ffi
 
     def up(arr, store):
         if store == ffi.BF16:
@@ -586,6 +588,8 @@ def test_gemm_bf16_large_tiles_direct_to_lds_kernel(B, M, N, K, tile):
 def test_gemm_grouped_matches_separate_products(B):
     """One grouped launch over problems of different sizes (ragged tile edges, NONE then ACCUM) against float64 numpy
     products of the same bf16-exact operands; descriptor errors are reported, not launched."""
+    import ctypes as C
+    from alpha2_amd import TensorData, _ffi as ffi
     K = 640
     shapes = [(768, 768), (264, 520), (2304, 768), (8, 8), (1000, 256)]
     keep, descs, wants, outs = [], [], [], []
