@@ -343,6 +343,7 @@ int32_t ah_gemm_grouped_plan(const AhGemm *descs, int32_t count, uint64_t *plan_
     AH_ARG(ok, "ah_gemm_grouped_plan: problem %d: operands need 16-byte aligned rows and a vector-aligned C", i);
     int64_t a_span = (akm ? (int64_t)64 : q.m) * q.lda * 2, b_span = (bkm ? (int64_t)64 : q.n) * q.ldb * 2;
     AH_ARG(a_span < (1ll << 32) && b_span < (1ll << 32), "ah_gemm_grouped_plan: problem %d: operand spans more than 4 GiB", i);
+    AH_ARG(q.ldc < (1 << 22), "ah_gemm_grouped_plan: problem %d: ldc %lld too large (128 rows of C must span less than 2 GiB)", i, (long long)q.ldc);
     GemmGroupEntry &e = tab[(size_t)i];
     e.a = dp<const void>(q.a); e.b = dp<const void>(q.b); e.c = dp<void>(q.c);
     e.M = (int)q.m; e.N = (int)q.n; e.K = (int)q.k; e.tile_start = (int)blocks;

@@ -238,7 +238,7 @@ int32_t run(const GemmArgs &ga, int batch, int out_dtype) {
   // LDS traffic per flop of the 128x128 tile.  It holds one block per CU, so what matters is how evenly the tiles fill
   // whole rounds of CUs: take 256 x 256 or 256 x 192 tiles, whichever wastes less of its last round, and keep the
   // 128x128 tile of this file (two blocks per CU, finer grain) when neither fills 70 %.
-  if (ga.M >= 256 && ga.N >= 192) {
+  if (ga.M >= 256 && ga.N >= 192 && ga.ldc < (1 << 22)) {      // (its epilogue addresses 128 rows of C with 31-bit byte offsets)
     const int64_t cus = num_cus(), per = (int64_t)batch * ga.nsplit;
     auto fill = [&](int bn) {
       int64_t t = cdiv(ga.M, 256) * cdiv(ga.N, bn) * per;

@@ -91,18 +91,38 @@ __device__ __forceinline__ void epilogue4(const GemmArgs &g, int64_t cbase, int 
   }
 }
 
-// The values an epilogue reads beside the accumulators, 4 consecutive columns at a time.
+// The values an epilogue reads beside the accumulators, 4 consecutive columns at a time, as the buffer load delivers them.
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 template <bool F32> struct AuxVec;
 template <> struct AuxVec<true> {
-  typedef float4 T;
-  static __device__ __forceinline__ void unpack(const float4 &o, float (&x)[4]) { x[0] = o.x; x[1] = o.y; x[2] = o.z; x[3] = o.w; }
+  typedef u32x4 T;
+  static __device__ __forceinline__ T load(__amdgpu_buffer_rsrc_t r, uint32_t off) { return __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0); }
+  static __device__ __forceinline__ void unpack(const T &o, float (&x)[4]) {
+    x[0] = __uint_as_float(o.x); x[1] = __uint_as_float(o.y); x[2] = __uint_as_float(o.z); x[3] = __uint_as_float(o.w);
+  }
 };
 template <> struct AuxVec<false> {
-  typedef uint2 T;
-  static __device__ __forceinline__ void unpack(const uint2 &o, float (&x)[4]) {
+  typedef u32x2 T;
+  static __device__ __forceinline__ T load(__amdgpu_buffer_rsrc_t r, uint32_t off) { return __builtin_amdgcn_raw_buffer_load_b64(r, off, 0, 0); }
+  static __device__ __forceinline__ void unpack(const T &o, float (&x)[4]) {
     x[0] = bf16_bits_to_f32(o.x & 0xffff); x[1] = bf16_bits_to_f32(o.x >> 16); x[2] = bf16_bits_to_f32(o.y & 0xffff); x[3] = bf16_bits_to_f32(o.y >> 16);
   }
 };
+// Descriptor of the `bytes` bytes at p (none if bytes <= 0): a lane whose byte offset reaches past them has its store
+// dropped and its load answered with zeros by the address unit, so edge tiles need neither clamped addresses nor a
+// masked-off branch around every access.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t buffer_window(const void *p, int bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, max(bytes, 0), 0x00020000);
+}
+__device__ __forceinline__ void buffer_store4(float v0, float v1, float v2, float v3, float *, __amdgpu_buffer_rsrc_t r, uint32_t off) {
+  u32x4 d = {__float_as_uint(v0), __float_as_uint(v1), __float_as_uint(v2), __float_as_uint(v3)};
+  __builtin_amdgcn_raw_buffer_store_b128(d, r, off, 0, 0);
+}
+__device__ __forceinline__ void buffer_store4(float v0, float v1, float v2, float v3, uint16_t *, __amdgpu_buffer_rsrc_t r, uint32_t off) {
+  u32x2 d = {pack_bf16x2(v0, v1), pack_bf16x2(v2, v3)};
+  __builtin_amdgcn_raw_buffer_store_b64(d, r, off, 0, 0);
+}
 
 // Four 4 KB pieces of LDS that belong to the calling wave alone (nobody else reads or writes them until the next
 // workgroup barrier).
@@ -114,9 +134,13 @@ struct EpiStage { char *p[4]; };
 // Instead each 32 x 32 accumulator goes to LDS as f32 (row r at r * 128 bytes, 16-byte chunk c at position c ^ (r & 7):
 // conflict-free both ways) and comes back row-major: 8 (f32 output) or 16 (bf16 output, two tiles side by side) lanes
 // cover one row's 128 contiguous bytes, and everything an epilogue reads (residual, accumulate, saved gelu') is loaded in
-// that same coalesced layout.  Those loads are unconditional (lanes past an edge of C read a clamped, valid address and
-// only their stores are masked), so they can run ahead: vmcnt retires in issue order, stores included, so the reads of
-// pass p + DEPTH are issued before the stores of pass p.  Requires N % 4 == 0.
+// that same coalesced layout.
+// Addressing: every access goes through a buffer descriptor whose base is moved, with scalar arithmetic, to the first
+// row and column of the group of rows being written, and whose size is what is left of the wave tile's rows inside C
+// from there; the per-lane part of the address is one of two constants (row in the group x ldc + column).  A lane in a
+// row past the end of C is then out of the descriptor's range, a lane in a column past the end is given an offset that
+// always is.  The loads run ahead: vmcnt retires in issue order, stores included, so the reads of pass p + DEPTH are issued
+// before the stores of pass p.  Requires N % 4 == 0 and 128 rows of C to span less than 2 GiB.
 template <int EPI, class OUT, int TM, int TN>
 __device__ __forceinline__ void store_tiles_lds(const GemmArgs &g, int64_t cbase, int row0, int col0, int lane, const f32x16 (&acc)[TM][TN],
                                                 const EpiStage &st) {
@@ -126,36 +150,43 @@ __device__ __forceinline__ void store_tiles_lds(const GemmArgs &g, int64_t cbase
   constexpr bool READS = EPI == AH_EPI_ACCUM || EPI == AH_EPI_RESIDUAL || EPI == AH_EPI_GELU_BWD || EPI == AH_EPI_MUL_AUX;
   constexpr bool AUX_F32 = EPI == AH_EPI_RESIDUAL || F32OUT;
   constexpr int DEPTH = 4 < NPASS ? 4 : NPASS;        // passes of reads in flight: 4 x 16 registers
+  constexpr int ES = sizeof(OUT), AES = AUX_F32 ? 4 : 2;
+  constexpr uint32_t OUTSIDE = 0x80000000u;           // a byte offset no descriptor here reaches (they are shorter than 2 GiB)
   typedef AuxVec<AUX_F32> AV;
   typedef typename AV::T AuxT;
-  typedef typename std::conditional<AUX_F32, float, uint16_t>::type AuxE;
   const int lr = lane & 31, lk = lane >> 5;
-  OUT *c = (OUT *)g.c + cbase + (int64_t)row0 * g.ldc + col0;
-  const AuxE *aux = (const AuxE *)(EPI == AH_EPI_ACCUM ? (const void *)g.c : g.aux) + cbase + (int64_t)row0 * g.ldc + col0;
-  OUT *aux_out = (OUT *)g.aux_out + cbase + (int64_t)row0 * g.ldc + col0;
+  const int64_t origin = cbase + (int64_t)row0 * g.ldc + col0;
+  const char *c = (const char *)g.c + origin * ES;
+  const char *aux = (const char *)(EPI == AH_EPI_ACCUM ? (const void *)g.c : g.aux) + origin * AES;
+  const char *aux_out = (const char *)g.aux_out + origin * ES;
   // a pass of NS tiles side by side comes back in 4 NS iterations of 8 / NS rows: lane -> (row in the group, chunk)
   const int rr1 = lane >> 3, cc1 = lane & 7, rr2 = lane >> 4, cc2 = lane & 15;
-  const int rows_left = g.M - row0, cols_left = g.N - col0;        // lanes at or past these are outside C
+  const int rows_here = min(g.M - row0, 32 * TM), cols_left = g.N - col0;       // rows / columns of the wave tile inside C
+  const int ldc = (int)g.ldc, span = rows_here * ldc;       // span: elements from the origin to the end of the last row inside C (< 2^29)
+  const uint32_t lane_el1 = (uint32_t)(rr1 * ldc + 4 * cc1), lane_el2 = (uint32_t)(rr2 * ldc + 4 * cc2);
   int wofs[4];
 #pragma unroll
   for (int q = 0; q < 4; q++) wofs[q] = lr * 128 + (((2 * q + lk) ^ (lr & 7)) << 4);
 
   AuxT pre[DEPTH][8];
-  auto pass_row = [&](int p, int it) -> int {
+  // element offset (uniform) of the first row and column of iteration `it` of pass p, and this lane's part for the pass
+  auto group_el = [&](int p, int it) -> int {
     const int i = p / NJP, j0 = (p % NJP) * JP, ns = TN - j0 < JP ? TN - j0 : JP;
-    return 32 * i + it * (8 / ns) + (ns == 2 ? rr2 : rr1);
+    return (32 * i + it * (8 / ns)) * ldc + 32 * j0;
   };
-  auto pass_col = [&](int p) -> int {
+  auto lane_bytes = [&](int p, int esize) -> uint32_t {
     const int j0 = (p % NJP) * JP, ns = TN - j0 < JP ? TN - j0 : JP;
-    return 32 * j0 + 4 * (ns == 2 ? cc2 : cc1);
-  };
-  auto pass_elem = [&](int p, int it) -> int64_t {      // element offset (from row0, col0) of this lane's 4 columns, clamped into C
-    return (int64_t)min(pass_row(p, it), rows_left - 1) * g.ldc + min(pass_col(p), cols_left - 4);
+    const bool col_inside = 32 * j0 + 4 * (ns == 2 ? cc2 : cc1) < cols_left;
+    return col_inside ? (ns == 2 ? lane_el2 : lane_el1) * (uint32_t)esize : OUTSIDE;
   };
   auto issue_reads = [&](int p) {
     const int j0 = (p % NJP) * JP, ns = TN - j0 < JP ? TN - j0 : JP;
+    const uint32_t le = lane_bytes(p, AES);
 #pragma unroll
-    for (int it = 0; it < 4 * ns; it++) pre[p % DEPTH][it] = *reinterpret_cast<const AuxT *>(aux + pass_elem(p, it));
+    for (int it = 0; it < 4 * ns; it++) {
+      const int ge = group_el(p, it);
+      pre[p % DEPTH][it] = AV::load(buffer_window(aux + ge * AES, (span - ge) * AES), le);
+    }
   };
   if (READS) {
 #pragma unroll
@@ -172,14 +203,14 @@ __device__ __forceinline__ void store_tiles_lds(const GemmArgs &g, int64_t cbase
       for (int q = 0; q < 4; q++)
         *reinterpret_cast<float4 *>((jj ? piece1 : piece0) + wofs[q]) =
             make_float4(acc[i][j0 + jj][4 * q], acc[i][j0 + jj][4 * q + 1], acc[i][j0 + jj][4 * q + 2], acc[i][j0 + jj][4 * q + 3]);
+    const uint32_t le = lane_bytes(p, ES);
 #pragma unroll
     for (int it = 0; it < 4 * ns; it++) {
       const int r = it * (8 / ns) + (ns == 2 ? rr2 : rr1), ch = ns == 2 ? cc2 & 7 : cc1;
       const char *src = (ns == 2 && cc2 >= 8 ? piece1 : piece0) + r * 128 + ((ch ^ (r & 7)) << 4);
       const float4 t = *reinterpret_cast<const float4 *>(src);
       float v[4] = {t.x, t.y, t.z, t.w};
-      const int64_t off = pass_elem(p, it);
-      const bool inside = pass_row(p, it) < rows_left && pass_col(p) < cols_left;
+      const int ge = group_el(p, it);
       if (READS) {
         float x[4];
         AV::unpack(pre[p % DEPTH][it], x);
@@ -193,22 +224,13 @@ __device__ __forceinline__ void store_tiles_lds(const GemmArgs &g, int64_t cbase
         float d[4];
 #pragma unroll
         for (int e = 0; e < 4; e++) gelu_both_f(v[e], v[e], d[e]);
-        if (inside) {
-          if (F32OUT) *reinterpret_cast<float4 *>(aux_out + off) = make_float4(d[0], d[1], d[2], d[3]);
-          else *reinterpret_cast<uint2 *>(aux_out + off) = make_uint2(pack_bf16x2(d[0], d[1]), pack_bf16x2(d[2], d[3]));
-        }
+        buffer_store4(d[0], d[1], d[2], d[3], (OUT *)nullptr, buffer_window(aux_out + ge * ES, (span - ge) * ES), le);
       } else if (EPI == AH_EPI_GELU) {
-        if (inside) {
-          if (F32OUT) *reinterpret_cast<float4 *>(aux_out + off) = make_float4(v[0], v[1], v[2], v[3]);
-          else *reinterpret_cast<uint2 *>(aux_out + off) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
-        }
+        buffer_store4(v[0], v[1], v[2], v[3], (OUT *)nullptr, buffer_window(aux_out + ge * ES, (span - ge) * ES), le);
 #pragma unroll
         for (int e = 0; e < 4; e++) v[e] = gelu_f(v[e]);
       }
-      if (inside) {
-        if (F32OUT) *reinterpret_cast<float4 *>(c + off) = make_float4(v[0], v[1], v[2], v[3]);
-        else *reinterpret_cast<uint2 *>(c + off) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
-      }
+      buffer_store4(v[0], v[1], v[2], v[3], (OUT *)nullptr, buffer_window(c + ge * ES, (span - ge) * ES), le);
     }
     __builtin_amdgcn_sched_barrier(0);
     if (READS && p + DEPTH < NPASS) {
