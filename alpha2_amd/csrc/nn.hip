@@ -305,6 +305,10 @@ __global__ __launch_bounds__(256) void k_layernorm_bwd_vec(const float *__restri
 }
 
 // ---------------------------------------------------------------- softmax cross-entropy
+// exp(v - m) as one fused multiply-add into the bare base-2 exponential, with neg_m_l2 = -m log2(e) (the vector paths of
+// the three kernels below use the same form, so their results agree bit for bit)
+constexpr float CE_LOG2E = 1.4426950408889634f;
+__device__ __forceinline__ float exp_minus(float v, float neg_m_l2) { return __builtin_amdgcn_exp2f(fmaf(v, CE_LOG2E, neg_m_l2)); }
 __device__ __forceinline__ void online_merge(float &m, float &s, float m2, float s2) {
   float nm = fmaxf(m, m2);
   if (nm == -INFINITY) { m = nm; s = 0.f; return; }
@@ -333,8 +337,9 @@ __global__ void k_ce_fwd(const T *__restrict__ logits, const int32_t *__restrict
 #pragma unroll
     for (int i = 1; i < VW; i++) vm = fmaxf(vm, v[i]);
     if (vm > m) { s *= __expf(m - vm); m = vm; }
+    const float nm = -m * CE_LOG2E;
 #pragma unroll
-    for (int i = 0; i < VW; i++) s += __expf(v[i] - m);
+    for (int i = 0; i < VW; i++) s += exp_minus(v[i], nm);
   }
   for (int64_t j = nvec * VW + threadIdx.x; j < c; j += blockDim.x) {
     float v = Io<T>::ld(p, j);
@@ -357,7 +362,15 @@ __global__ void k_ce_fwd(const T *__restrict__ logits, const int32_t *__restrict
 __global__ void k_mean_rows(const float *__restrict__ v, int64_t n, float *__restrict__ out) {
   __shared__ double sh[WPB];
   double s = 0;
-  for (int64_t i = threadIdx.x; i < n; i += blockDim.x) s += (double)v[i];
+  int64_t i = threadIdx.x;
+  for (; i + 7 * (int64_t)blockDim.x < n; i += 8 * (int64_t)blockDim.x) {        // eight independent loads in flight (one block runs this)
+    float x[8];
+#pragma unroll
+    for (int k = 0; k < 8; k++) x[k] = v[i + k * (int64_t)blockDim.x];
+#pragma unroll
+    for (int k = 0; k < 8; k++) s += (double)x[k];
+  }
+  for (; i < n; i += blockDim.x) s += (double)v[i];
   s = wave_sum_d(s);
   if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = s;
   __syncthreads();
@@ -366,6 +379,24 @@ __global__ void k_mean_rows(const float *__restrict__ v, int64_t n, float *__res
     for (int k = 0; k < WPB; k++) t += sh[k];
     out[0] = (float)(t / (double)n);
   }
+}
+// (softmax - onehot) * scale for 8 bf16 logits: the subtraction of the one-hot is only spelled out in the one chunk of
+// a row that holds the target (`hot` = its position there, else -1); everywhere else (e - 0) * scale == e * scale bit for bit.
+__device__ __forceinline__ void ce_grad8(const uint4 &u, float lse, float scale, int hot, uint32_t (&o)[4]) {
+  const uint32_t in[4] = {u.x, u.y, u.z, u.w};
+  float e[8];
+  const float nl = -lse * CE_LOG2E;
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    e[2 * i] = exp_minus(bf16_bits_to_f32(in[i] & 0xffff), nl);
+    e[2 * i + 1] = exp_minus(bf16_bits_to_f32(in[i] >> 16), nl);
+  }
+  if (hot >= 0) {
+#pragma unroll
+    for (int i = 0; i < 8; i++) e[i] -= (i == hot ? 1.0f : 0.0f);
+  }
+#pragma unroll
+  for (int i = 0; i < 4; i++) o[i] = pack_bf16x2(e[2 * i] * scale, e[2 * i + 1] * scale);
 }
 template <class T>
 __global__ void k_ce_bwd(const T *__restrict__ logits, const int32_t *__restrict__ targets, const float *__restrict__ lse,
@@ -379,14 +410,8 @@ __global__ void k_ce_bwd(const T *__restrict__ logits, const int32_t *__restrict
   if (sizeof(T) == 2 && (c & 7) == 0 && (((uintptr_t)logits | (uintptr_t)out) & 15u) == 0) {      // bf16: 8 classes per 16-byte access
     for (int64_t j8 = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; j8 < (c >> 3); j8 += (int64_t)gridDim.x * blockDim.x) {
       uint4 u = reinterpret_cast<const uint4 *>(p)[j8];
-      uint32_t in[4] = {u.x, u.y, u.z, u.w}, o[4];
-#pragma unroll
-      for (int i = 0; i < 4; i++) {
-        int64_t j = j8 * 8 + 2 * i;
-        float a = (__expf(bf16_bits_to_f32(in[i] & 0xffff) - l) - (j == t ? 1.0f : 0.0f)) * scale;
-        float b = (__expf(bf16_bits_to_f32(in[i] >> 16) - l) - (j + 1 == t ? 1.0f : 0.0f)) * scale;
-        o[i] = pack_bf16x2(a, b);
-      }
+      uint32_t o[4];
+      ce_grad8(u, l, scale, j8 == (t >> 3) ? (int)(t & 7) : -1, o);
       reinterpret_cast<uint4 *>(q)[j8] = make_uint4(o[0], o[1], o[2], o[3]);
     }
     return;
@@ -422,8 +447,9 @@ __global__ __launch_bounds__(256) void k_ce_fwd_bwd(const uint16_t *__restrict__
 #pragma unroll
       for (int i = 1; i < 8; i++) vm = fmaxf(vm, v[i]);
       if (vm > m) { s *= __expf(m - vm); m = vm; }
+      const float nm = -m * CE_LOG2E;
 #pragma unroll
-      for (int i = 0; i < 8; i++) s += __expf(v[i] - m);
+      for (int i = 0; i < 8; i++) s += exp_minus(v[i], nm);
     }
   }
 #pragma unroll
@@ -447,15 +473,8 @@ __global__ __launch_bounds__(256) void k_ce_fwd_bwd(const uint16_t *__restrict__
   for (int k = 0; k < CE_CHUNKS; k++) {
     const int j8 = threadIdx.x + k * 256;
     if (j8 < nvec) {
-      const uint32_t in[4] = {r[k].x, r[k].y, r[k].z, r[k].w};
       uint32_t o[4];
-#pragma unroll
-      for (int i = 0; i < 4; i++) {
-        const int64_t j = (int64_t)j8 * 8 + 2 * i;
-        const float a = (__expf(bf16_bits_to_f32(in[i] & 0xffff) - l) - (j == t ? 1.0f : 0.0f)) * scale;
-        const float b = (__expf(bf16_bits_to_f32(in[i] >> 16) - l) - (j + 1 == t ? 1.0f : 0.0f)) * scale;
-        o[i] = pack_bf16x2(a, b);
-      }
+      ce_grad8(r[k], l, scale, j8 == (t >> 3) ? (int)(t & 7) : -1, o);
       reinterpret_cast<uint4 *>(q)[j8] = make_uint4(o[0], o[1], o[2], o[3]);
     }
   }
