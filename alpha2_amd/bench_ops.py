@@ -1,0 +1,201 @@
+"""Per-op microbenchmarks on the shapes of the training step, in the manner of the reference's scripts/bench-ops.ts
+(3 warm-up calls, then the mean of `iters` calls; TFLOP/s = flops / time, GB/s = algorithmic bytes / time):
+
+    python -m alpha2_amd.bench_ops [--iters 10] [--only gemm|flash|bandwidth] [--json]
+
+* GEMM: C = A B^T and both backward products, M = 16384 (batch x context), K = 768, N in {768, 2304, 3072, 50304},
+  bf16 operands with fp32 accumulation and fp32 throughout; flops 2 M N K (scripts/bench-ops.ts:302,328).
+* Causal flash attention forward and backward: B = 16, H = 12, head size 64, T in {256, 1024, 2048}, bf16, with and
+  without the soft cap of 30; flops counted non-causal like the reference: 4 B H T^2 D forward, 8 B H T^2 D backward
+  (scripts/bench-ops.ts:652,673).
+* Bandwidth-bound ops at the GPT-2-small step's sizes: LayerNorm forward / backward, GELU forward / backward, fused
+  cross-entropy forward + backward, embedding gather / scatter-add, sum of squares, AdamW; bytes = the algorithmic minimum.
+
+Every call goes through the C ABI; timing is by HIP events on the library's stream.  Peaks used for the last column:
+2.5 PFLOP/s (bf16 MFMA), 157.3 TFLOP/s (fp32 MFMA), 8 TB/s (HBM).
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import math
+import sys
+
+import numpy as np
+
+from . import HipBackend, _ffi as ffi
+
+PEAK_TFLOPS = {"bf16": 2500.0, "f32": 157.3}
+PEAK_GBS = 8000.0
+
+
+class Bench:
+    def __init__(self, iters: int):
+        self.B = HipBackend(0)
+        self.lib = self.B.lib
+        self.iters = iters
+        self.rows = []
+        self._live = []
+
+    def alloc(self, nbytes: int) -> int:
+        p = C.c_uint64()
+        ffi.check(self.lib.ah_alloc(max(nbytes, 16), C.byref(p)))
+        self._live.append(p.value)
+        return p.value
+
+    def release(self):
+        for p in self._live:
+            self.lib.ah_free(p)
+        self._live = []
+
+    def randn(self, n: int, dtype: int, std: float = 1.0, seed: int = 2) -> int:
+        """n values N(0, std) on the device in `dtype` (generated in blocks of 16 M on the host)."""
+        es = ffi.DTYPE_BYTES["bf16" if dtype == ffi.BF16 else "f32"]
+        dst = self.alloc(n * es)
+        blk = 1 << 24
+        tmp = self.alloc(min(n, blk) * 4)
+        host = (np.random.RandomState(seed).standard_normal(min(n, blk)) * std).astype(np.float32)
+        ffi.check(self.lib.ah_upload(tmp, host.ctypes.data_as(C.c_void_p), host.nbytes))
+        for o in range(0, n, blk):
+            m = min(blk, n - o)
+            if dtype == ffi.F32:
+                ffi.check(self.lib.ah_copy(dst + o * 4, tmp, m * 4))
+            else:
+                ffi.check(self.lib.ah_cast(tmp, ffi.F32, dst + o * es, dtype, m))
+        return dst
+
+    def time(self, fn) -> float:
+        """Mean milliseconds per call."""
+        for _ in range(3):
+            fn()
+        e0, e1 = self.B._event(), self.B._event()
+        ffi.check(self.lib.ah_event_record(e0))
+        for _ in range(self.iters):
+            fn()
+        ffi.check(self.lib.ah_event_record(e1))
+        ms = C.c_float()
+        ffi.check(self.lib.ah_event_elapsed_ms(e0, e1, C.byref(ms)))
+        for e in (e0, e1):
+            ffi.check(self.lib.ah_event_destroy(e))
+        return ms.value / self.iters
+
+    def record(self, name: str, ms: float, flops: float = 0.0, nbytes: float = 0.0, dtype: str = "bf16", note: str = ""):
+        tf = flops / (ms * 1e-3) / 1e12 if flops else None
+        gbs = nbytes / (ms * 1e-3) / 1e9 if nbytes else None
+        frac = tf / PEAK_TFLOPS[dtype] if flops else gbs / PEAK_GBS
+        self.rows.append({"op": name, "us": ms * 1e3, "tflops": tf, "gbs": gbs, "bound": "mfma" if flops else "hbm", "frac_of_peak": frac, "note": note})
+        perf = f"{tf:9.1f} TFLOP/s" if flops else f"{gbs:9.0f} GB/s   "
+        print(f"{name:34s} {ms * 1e3:10.1f} us {perf} {100 * frac:5.1f} %  {note}", flush=True)
+
+
+def bench_gemm(b: Bench):
+    M, K = 16384, 768
+    for dt, dname in ((ffi.BF16, "bf16"), (ffi.F32, "f32")):
+        es = 2 if dt == ffi.BF16 else 4
+        for N in (768, 2304, 3072, 50304):
+            a, w, g = b.randn(M * K, dt, 0.02), b.randn(N * K, dt, 0.02), b.randn(M * N, dt, 0.02)
+            c_fwd, c_da = b.alloc(M * N * es), b.alloc(M * K * es)
+            c_db = b.alloc(N * K * 4)                                     # weight gradients are kept in f32
+            flops = 2.0 * M * N * K
+            cases = (("fwd  C=A.B^T", ffi.GEMM_NT, (M, N, K, K, K, N), (a, w, c_fwd), dt),
+                     ("dA   G.B", ffi.GEMM_NN, (M, K, N, N, K, K), (g, w, c_da), dt),
+                     ("dB   G^T.A", ffi.GEMM_TN, (N, K, M, N, K, K), (g, a, c_db), ffi.F32))
+            for label, layout, (m, n, k, lda, ldb, ldc), (pa, pb, pc), out in cases:
+                d = ffi.AhGemm(layout, dt, out, ffi.EPI_NONE, m, n, k, lda, ldb, ldc, 1, 0, 0, 0, pa, pb, pc, 0)
+                ms = b.time(lambda: ffi.check(b.lib.ah_gemm(C.byref(d))))
+                kern, nsplit = b.B.lastGemmKernel()
+                b.record(f"gemm {dname} N={N} {label}", ms, flops=flops, dtype=dname, note=f"{kern}" + (f" split-K x{nsplit}" if nsplit > 1 else ""))
+            b.release()
+
+
+def bench_flash(b: Bench):
+    Bt, H, D = 16, 12, 64
+    Cc = H * D
+    for T in (256, 1024, 2048):
+        qkv, do = b.randn(Bt * T * 3 * Cc, ffi.BF16, 1.0, 3), b.randn(Bt * T * Cc, ffi.BF16, 1.0, 4)
+        o, dqkv, lse = b.alloc(Bt * T * Cc * 2), b.alloc(Bt * T * 3 * Cc * 2), b.alloc(Bt * H * T * 4)
+        for cap in (0.0, 30.0):
+            f = ffi.AhFlash()
+            f.dtype, f.batch, f.heads, f.seq, f.head_dim = ffi.BF16, Bt, H, T, D
+            for p in ("q", "k", "v"):
+                setattr(f, p + "_sb", T * 3 * Cc), setattr(f, p + "_sh", D), setattr(f, p + "_st", 3 * Cc)
+            f.o_sb, f.o_sh, f.o_st = T * Cc, D, Cc
+            f.scale, f.soft_cap = 1 / math.sqrt(D), cap
+            f.q, f.k, f.v, f.o, f.lse = qkv, qkv + Cc * 2, qkv + 2 * Cc * 2, o, lse
+            f.d_o, f.dq, f.dk, f.dv = do, dqkv, dqkv + Cc * 2, dqkv + 2 * Cc * 2
+            ms = b.time(lambda: ffi.check(b.lib.ah_flash_fwd(C.byref(f))))
+            b.record(f"flash fwd T={T} cap={cap:g}", ms, flops=4.0 * Bt * H * T * T * D, note="non-causal flop count; causal work is half")
+            ms = b.time(lambda: ffi.check(b.lib.ah_flash_bwd(C.byref(f))))
+            b.record(f"flash bwd T={T} cap={cap:g}", ms, flops=8.0 * Bt * H * T * T * D, note="dQ + dK/dV kernels")
+        b.release()
+
+
+def bench_bandwidth(b: Bench):
+    lib = b.lib
+    rows, dim, F, V, P = 16384, 768, 3072, 50304, 163_037_184
+    x, res = b.randn(rows * dim, ffi.F32), b.randn(rows * dim, ffi.F32)
+    g16 = b.randn(rows * dim, ffi.BF16)
+    w, bias = b.randn(dim, ffi.F32), b.randn(dim, ffi.F32)
+    out16, dx, dx16, dw, db = b.alloc(rows * dim * 2), b.alloc(rows * dim * 4), b.alloc(rows * dim * 2), b.alloc(dim * 4), b.alloc(dim * 4)
+    ms = b.time(lambda: ffi.check(lib.ah_layernorm(x, w, bias, out16, rows, dim, 1e-5, ffi.BF16)))
+    b.record("layernorm fwd 16384x768", ms, nbytes=rows * dim * 6, note="f32 in, bf16 out")
+    ms = b.time(lambda: ffi.check(lib.ah_layernorm_bwd(x, w, g16, ffi.BF16, res, dx, dx16, dw, db, rows, dim, 1e-5, 0)))
+    b.record("layernorm bwd 16384x768", ms, nbytes=rows * dim * 16, note="x f32, g bf16, + residual grad f32 -> dx f32 + bf16; dw, db")
+    b.release()
+
+    h = b.randn(rows * F, ffi.F32)
+    gh, oh = b.randn(rows * F, ffi.F32), b.alloc(rows * F * 4)
+    ms = b.time(lambda: ffi.check(lib.ah_unary(ffi.GELU, h, oh, rows * F, 0.0, 0.0)))
+    b.record("gelu fwd 16384x3072 f32", ms, nbytes=rows * F * 8, note="parity-mode op (the fast path fuses GELU into the GEMM epilogue)")
+    ms = b.time(lambda: ffi.check(lib.ah_unary_bwd(ffi.GELU_BWD, h, gh, oh, rows * F, 0.0, 0.0)))
+    b.record("gelu bwd 16384x3072 f32", ms, nbytes=rows * F * 12)
+    b.release()
+
+    lg = b.randn(rows * V, ffi.BF16, 2.0)
+    tg = b.alloc(rows * 4)
+    th = np.random.RandomState(5).randint(0, V, rows).astype(np.int32)
+    ffi.check(lib.ah_upload(tg, th.ctypes.data_as(C.c_void_p), th.nbytes))
+    loss, lse = b.alloc(4), b.alloc(rows * 4)
+    ms = b.time(lambda: ffi.check(lib.ah_cross_entropy_fwd_bwd(lg, ffi.BF16, tg, loss, lse, 0, 1.0, lg, rows, V)))
+    b.record("cross-entropy fwd+bwd 16384x50304", ms, nbytes=rows * V * 4, note="bf16 logits read once, gradient written in place")
+    b.release()
+
+    wte, tok = b.randn(V * dim, ffi.F32, 0.02), b.alloc(rows * 4)
+    ffi.check(lib.ah_upload(tok, th.ctypes.data_as(C.c_void_p), th.nbytes))
+    eo, gw = b.alloc(rows * dim * 4), b.alloc(V * dim * 4)
+    ms = b.time(lambda: ffi.check(lib.ah_embedding(wte, tok, eo, rows, dim, V, ffi.F32)))
+    b.record("embedding gather 16384x768", ms, nbytes=rows * dim * 8, note="uniform token ids")
+    ms = b.time(lambda: ffi.check(lib.ah_embedding_bwd(tok, eo, gw, rows, dim, V, 0)))
+    b.record("embedding scatter-add 16384x768", ms, nbytes=rows * dim * 8 + V * dim * 4, note="includes zero-filling the [50304, 768] gradient")
+    b.release()
+
+    p, g, m, v, sh = (b.randn(P, ffi.F32, 0.02, s) for s in (6, 7, 8, 9, 10))
+    ffi.check(lib.ah_binary(ffi.MUL, v, v, v, P))                       # second moment must be non-negative
+    acc = b.alloc(8)
+    ms = b.time(lambda: ffi.check(lib.ah_sum_sq(g, P, acc)))
+    b.record("sum of squares 163.0M", ms, nbytes=P * 4)
+    hyp = ffi.AhAdamW(3e-4, 0.9, 0.95, 1e-8, 0.1, 0.1, 0.05, 1.0)
+    ms = b.time(lambda: ffi.check(lib.ah_adamw(p, g, m, v, P, C.byref(hyp), 0, 0, sh)))
+    b.record("adamw 163.0M (+bf16 shadow)", ms, nbytes=P * 30, note="reads p g m v, writes p m v + bf16 copy of p")
+    b.release()
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser(description=__doc__.split("\n")[0])
+    ap.add_argument("--iters", type=int, default=10)
+    ap.add_argument("--only", choices=["gemm", "flash", "bandwidth"])
+    ap.add_argument("--json", action="store_true", help="also print one JSON line with every row")
+    args = ap.parse_args(argv)
+    b = Bench(args.iters)
+    print(f"{'op':34s} {'time':>13s} {'rate':>16s} {'peak':>7s}")
+    for name, fn in (("gemm", bench_gemm), ("flash", bench_flash), ("bandwidth", bench_bandwidth)):
+        if args.only in (None, name):
+            fn(b)
+    if args.json:
+        print(json.dumps(b.rows))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -431,11 +431,40 @@ int32_t ah_gemm(const AhGemm *p) {
   if (q.in_dtype == AH_F32) {
     int vec_a = aligned16(q.a) && (q.lda % 4 == 0) && (q.stride_a % 4 == 0);
     int vec_b = aligned16(q.b) && (q.ldb % 4 == 0) && (q.stride_b % 4 == 0);
-    switch (q.layout) {
-      case AH_GEMM_NN: return launch_f32<AH_GEMM_NN>(ga, batch, q.out_dtype, vec_a, vec_b, vec_c);
-      case AH_GEMM_NT: return launch_f32<AH_GEMM_NT>(ga, batch, q.out_dtype, vec_a, vec_b, vec_c);
-      default: return launch_f32<AH_GEMM_TN>(ga, batch, q.out_dtype, vec_a, vec_b, vec_c);
+    auto run_f32 = [&](const GemmArgs &g, int nb, int vc) -> int32_t {
+      switch (q.layout) {
+        case AH_GEMM_NN: return launch_f32<AH_GEMM_NN>(g, nb, q.out_dtype, vec_a, vec_b, vc);
+        case AH_GEMM_NT: return launch_f32<AH_GEMM_NT>(g, nb, q.out_dtype, vec_a, vec_b, vc);
+        default: return launch_f32<AH_GEMM_TN>(g, nb, q.out_dtype, vec_a, vec_b, vc);
+      }
+    };
+    // Split-K for a long contraction with too few output tiles to fill the chip (weight gradients: K = tokens): the
+    // slices run as batch entries of the same kernel (batch strides step along K) into a workspace [slices][M][N], which
+    // is then summed in fixed order.
+    int64_t tiles = cdiv(q.m, F_BM) * cdiv(q.n, F_BN);
+    if (batch == 1 && q.out_dtype == AH_F32 && (q.epilogue == AH_EPI_NONE || q.epilogue == AH_EPI_ACCUM) && tiles < num_cus() && q.k >= 2048 &&
+        (q.m * q.n) % 4 == 0 && q.n % 4 == 0 && vec_c) {
+      int s = (int)cdiv(2ll * num_cus(), tiles);
+      if (s > 32) s = 32;
+      while (s > 1 && (q.k % (s * 4) != 0 || q.k / s < 512)) s--;
+      if (s > 1) {
+        ah_ptr ws = 0;
+        int32_t rc = ah_alloc((uint64_t)s * q.m * q.n * 4, &ws);
+        if (rc) return rc;
+        GemmArgs gs = ga;
+        int64_t ks = q.k / s;
+        gs.K = (int)ks; gs.ksplit = (int)ks;
+        gs.sa = q.layout == AH_GEMM_TN ? ks * q.lda : ks;
+        gs.sb = q.layout == AH_GEMM_NT ? ks : ks * q.ldb;
+        gs.c = dp<void>(ws); gs.ldc = q.n; gs.sc = q.m * q.n; gs.epi = AH_EPI_NONE;
+        rc = run_f32(gs, s, 1);
+        if (rc == AH_OK) rc = ah::splitk_reduce(dp<const float>(ws), (float *)ga.c, s, ga.M, ga.N, ga.ldc, q.epilogue == AH_EPI_ACCUM);
+        note_gemm_split(s);
+        int32_t rf = ah_free(ws);
+        return rc ? rc : rf;
+      }
     }
+    return run_f32(ga, batch, vec_c);
   }
 
   AH_ARG(q.k % 8 == 0, "ah_gemm: bf16 contraction length %lld must be a multiple of 8", (long long)q.k);

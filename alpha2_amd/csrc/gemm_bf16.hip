@@ -260,6 +260,14 @@ namespace ah {
 
 // Preconditions (checked by the caller): K % 64 == 0; operands 16-byte aligned with lda/ldb/strides % 8 == 0;
 // M % 8 == 0 (N % 8 == 0) when A (B) is k-major; C/aux rows vector-aligned; a provided epilogue/output combination.
+int32_t splitk_reduce(const float *ws, float *c, int nsplit, int M, int N, int64_t ldc, bool accumulate) {
+  int64_t n4 = (int64_t)M * N / 4;
+  int blocks = (int)(cdiv(n4, 256) < 4096 ? cdiv(n4, 256) : 4096);
+  hipLaunchKernelGGL(k_splitk_reduce, dim3(blocks), dim3(256), 0, stream(), ws, c, nsplit, M, N, ldc, accumulate ? 1 : 0);
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+
 int32_t gemm_bf16_direct(const GemmArgs &ga, int layout, int batch, int out_dtype) {
   // per-thread offsets are 32-bit byte offsets from the operand base
   int64_t a_span = (layout == AH_GEMM_TN ? (int64_t)64 : (int64_t)ga.M) * ga.lda * 2;
@@ -283,14 +291,7 @@ int32_t gemm_bf16_direct(const GemmArgs &ga, int layout, int batch, int out_dtyp
   int32_t rc = layout == AH_GEMM_NT ? run<false, false>(gs, batch, out_dtype)
              : layout == AH_GEMM_NN ? run<false, true>(gs, batch, out_dtype) : run<true, true>(gs, batch, out_dtype);
   if (ws) {
-    if (rc == AH_OK) {
-      int64_t n4 = (int64_t)ga.M * ga.N / 4;
-      int blocks = (int)(cdiv(n4, 256) < 4096 ? cdiv(n4, 256) : 4096);
-      hipLaunchKernelGGL(k_splitk_reduce, dim3(blocks), dim3(256), 0, stream(), dp<const float>(ws), (float *)ga.c, gs.nsplit, ga.M, ga.N,
-                         ga.ldc, ga.epi == AH_EPI_ACCUM ? 1 : 0);
-      hipError_t e = hipGetLastError();
-      if (e != hipSuccess) rc = hip_fail(e, "k_splitk_reduce"); else count_op();
-    }
+    if (rc == AH_OK) rc = splitk_reduce(dp<const float>(ws), (float *)ga.c, gs.nsplit, ga.M, ga.N, ga.ldc, ga.epi == AH_EPI_ACCUM);
     int32_t rf = ah_free(ws);      // stream-ordered: reusable only by later work
     if (rc == AH_OK) rc = rf;
   }

@@ -259,6 +259,8 @@ __device__ __forceinline__ void store_tiles(const GemmArgs &g, int64_t cbase, in
 
 // gemm_bf16.hip
 int32_t gemm_bf16_direct(const GemmArgs &ga, int layout, int batch, int out_dtype);
+// c[M][N] (leading dimension ldc) = (accumulate ? c : 0) + sum over the nsplit slices of ws[nsplit][M][N], in fixed order; M N % 4 == 0
+int32_t splitk_reduce(const float *ws, float *c, int nsplit, int M, int N, int64_t ldc, bool accumulate);
 // gemm_bf16_dma_{nt,nn,tn}.hip: 256 x bn tiles (bn = 256 or 192) fed by direct global->LDS loads (same preconditions as the
 // direct kernel)
 int32_t gemm_bf16_dma_nt(const GemmArgs &ga, int batch, int out_dtype, int bn);

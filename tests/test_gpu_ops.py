@@ -315,6 +315,31 @@ def test_gemm_f32_all_layouts(B, M, K, N):
         B.matmul(dev(B, a), dev(B, rs.randn(K + 1, N).astype(np.float32)))
 
 
+@pytest.mark.parametrize("M,K,N", [(256, 4096, 128), (132, 2052, 260), (64, 8192, 64)])
+def test_gemm_f32_long_contraction_split_k(B, M, K, N):
+    """Few output tiles and a long contraction: the fp32 kernel runs K in slices (as batch entries) and sums the slices
+    in fixed order; all three layouts and the accumulating epilogue against a float64 product."""
+    from alpha2_amd import _ffi as ffi
+    a, b = rs.randn(M, K).astype(np.float32), rs.randn(K, N).astype(np.float32)
+    want = a.astype(np.float64) @ b.astype(np.float64)
+    scale = float(np.sqrt(K))                                   # size of a result entry
+    got = {"nn": B.matmul(dev(B, a), dev(B, b)), "nt": B.matmulTransposed(dev(B, a), dev(B, np.ascontiguousarray(b.T))),
+           "tn": B.matmulTransposedA(dev(B, np.ascontiguousarray(a.T)), dev(B, b))}
+    for name, t in got.items():
+        assert B.lastGemmKernel()[0].startswith("k_gemm_f32")
+        assert np.max(np.abs(t.data.reshape(M, N) - want)) <= 2e-6 * K ** 0.5 * scale, name
+    assert B.lastGemmKernel()[1] > 1                            # the product above did run in slices
+    # accumulate into an existing C through the raw entry point
+    import ctypes
+    c0 = rs.randn(M, N).astype(np.float32)
+    c, at, bb = dev(B, c0), dev(B, np.ascontiguousarray(a.T)), dev(B, b)
+    g = ffi.AhGemm(ffi.GEMM_TN, ffi.F32, ffi.F32, ffi.EPI_ACCUM, M, N, K, M, N, N, 1, 0, 0, 0, B._ptr(at), B._ptr(bb), B._ptr(c), 0)
+    ffi.check(B.lib.ah_gemm(ctypes.byref(g)))
+    B._dirty(c)
+    assert B.lastGemmKernel()[1] > 1
+    assert np.max(np.abs(c.data.reshape(M, N) - (want + c0))) <= 2e-6 * K ** 0.5 * scale
+
+
 def test_gemm_f32_batched_and_broadcast(B):
     a, b = rs.randn(2, 3, 40, 16).astype(np.float32), rs.randn(2, 3, 16, 24).astype(np.float32)
     assert_close(B.matmul(dev(B, a), dev(B, b)).data, O.matmul(orc(a), orc(b)).data)
