@@ -69,3 +69,15 @@ def test_host_rng_matches_reference_integer_stream():
     r = SeededRng(7)
     g = r.fillGauss(4001, 0.02)
     assert g.dtype == np.float32 and abs(float(g.mean())) < 2e-3 and abs(float(g.std()) - 0.02) < 2e-3
+
+
+def test_backend_class_has_every_member_of_the_reference_interface():
+    """Member names of the reference's `interface Backend` (the 40 required and 27 optional ones, fixture transcribed
+    from packages/core/src/interfaces.ts:38-151) and the duck-typed extras its trainer calls (trainer.ts:1003-1032)."""
+    import json
+    from alpha2_amd.backend import HipBackend
+    spec = json.load(open(os.path.join(ROOT, "tests", "golden", "backend_interface.json")))
+    assert len(spec["required"]) == 40 and len(spec["optional"]) == 27
+    missing = [n for n in spec["required"] + spec["optional"] + spec["duck_typed"] if not hasattr(HipBackend, n)]
+    assert not missing, missing
+    assert HipBackend.name == "hip"
