@@ -389,6 +389,20 @@ def siluMul(ctx, a, b):
     return _record(ctx, ctx.backend.siluMul(ad, bd), [a, b], lambda g, B, rel, n: B.siluMulBackward(ad, bd, g))
 
 
+def channelAct(ctx, a, coefs: dict):
+    """sum_k coef_k[channel] * basis_k(a) in one backend pass (bases: silu, relu, gelu, identity, square); gradients flow to
+    `a` and to every coefficient.  Same function as the chain of silu / relu / gelu / mul / add the reference records for its
+    universal and kan_spline activations (gpt.ts:295-321)."""
+    ad = a.data
+    names = list(coefs)
+    cds = {n: coefs[n].data for n in names}
+
+    def backward(g, B, rel, needs):
+        dx, dco = B.channelActBackward(ad, cds, g)
+        return [dx] + [dco[n] for n in names]
+    return _record(ctx, ctx.backend.channelAct(ad, cds), [a] + [coefs[n] for n in names], backward)
+
+
 def gelu(ctx, a):
     ad = a.data
     return _record(ctx, ctx.backend.gelu(ad), [a], lambda g, B, rel, n: [B.geluBackward(ad, g)])

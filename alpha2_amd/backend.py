@@ -446,6 +446,42 @@ class HipBackend:
         check(self.lib.ah_silu_mul_bwd(self._ptr(a), self._ptr(b), self._ptr(g), da._buf.ptr, db._buf.ptr, a.size))
         return [da, db]
 
+    # ---- per-channel mixtures of activation bases: not part of the reference interface (it composes them from separate
+    # ops, gpt.ts:295-321); the model uses these when the backend offers them, the way the reference probes its optionals
+    CHANNEL_BASES = ("silu", "relu", "gelu", "identity", "square")
+
+    def _channel_args(self, x, coefs):
+        """coefs: {basis name: [1, cols] tensor}.  Returns (mask, handle array, cols, rows)."""
+        self._f32(x, *coefs.values())
+        cols = x.shape[-1]
+        mask, arr = 0, (C.c_uint64 * 5)()
+        for name, t in coefs.items():
+            k = self.CHANNEL_BASES.index(name)
+            if t.size != cols:
+                raise ValueError(f"channelAct: coefficient '{name}' has {t.size} entries for {cols} channels")
+            mask |= 1 << k
+            arr[k] = self._ptr(t)
+        return mask, arr, cols, x.size // cols if cols else 0
+
+    def channelAct(self, x: TensorData, coefs: dict) -> TensorData:
+        """out = sum over the given bases of coef[channel] * basis(x): the universal / kan_spline MLP activations in one pass."""
+        mask, arr, cols, rows = self._channel_args(x, coefs)
+        out = self._new(x.shape)
+        check(self.lib.ah_channel_act(self._ptr(x), arr, mask, out._buf.ptr, rows, cols))
+        return out
+
+    def channelActBackward(self, x: TensorData, coefs: dict, g: TensorData):
+        """Returns (dx, {basis name: d coef [1, cols]})."""
+        self._f32(g)
+        mask, arr, cols, rows = self._channel_args(x, coefs)
+        dx = self._new(x.shape)
+        dco = {name: self._new(t.shape) for name, t in coefs.items()}
+        darr = (C.c_uint64 * 5)()
+        for name, t in dco.items():
+            darr[self.CHANNEL_BASES.index(name)] = t._buf.ptr
+        check(self.lib.ah_channel_act_bwd(self._ptr(x), arr, mask, self._ptr(g), dx._buf.ptr, darr, rows, cols))
+        return dx, dco
+
     def residualDropoutAdd(self, residual, projected, mask) -> TensorData:
         self._f32(residual, projected)
         out = self._new(residual.shape)

@@ -53,6 +53,90 @@ struct UnBwd {
   }
 };
 
+// ---------------------------------------------------------------- per-channel mixtures of activation bases
+// out[r][c] = sum over the selected bases k of coef_k[c] * basis_k(x[r][c]); bases: 0 silu, 1 relu, 2 gelu (tanh form),
+// 3 identity, 4 square.  The "universal" MLP activation is bases {0, 3}, "kan_spline" all five.
+struct ChannelAct {
+  const float *coef[5];
+  float *dcoef[5];          // backward only
+  int mask;
+};
+// value and derivative of basis k at x (silu and gelu share nothing with the others, so each costs what it costs alone)
+__device__ __forceinline__ void basis_eval(int k, float x, float &v, float &d) {
+  switch (k) {
+    case 0: { float s = 1.0f / (1.0f + expf(-x)); v = x * s; d = s * (1.0f + x * (1.0f - s)); break; }
+    case 1: v = x > 0.f ? x : 0.f; d = x > 0.f ? 1.0f : 0.f; break;
+    case 2: gelu_both_f(x, v, d); break;
+    case 3: v = x; d = 1.0f; break;
+    default: v = x * x; d = 2.0f * x; break;
+  }
+}
+__global__ void k_channel_act(const float *__restrict__ x, ChannelAct p, float *__restrict__ out, int64_t rows, int cols4) {
+  int64_t n4 = rows * (int64_t)cols4;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n4; i += (int64_t)gridDim.x * blockDim.x) {
+    int c4 = (int)(i % cols4);
+    float4 xv = reinterpret_cast<const float4 *>(x)[i];
+    float xs[4] = {xv.x, xv.y, xv.z, xv.w}, acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int k = 0; k < 5; k++)
+      if (p.mask >> k & 1) {
+        float4 cv = reinterpret_cast<const float4 *>(p.coef[k])[c4];
+        float cs[4] = {cv.x, cv.y, cv.z, cv.w};
+#pragma unroll
+        for (int e = 0; e < 4; e++) { float v, d; basis_eval(k, xs[e], v, d); acc[e] += cs[e] * v; }
+      }
+    reinterpret_cast<float4 *>(out)[i] = make_float4(acc[0], acc[1], acc[2], acc[3]);
+  }
+}
+// Backward: dx = g * sum_k coef_k basis_k'(x); partial[rb][k][c] = sum over the rows of row block rb of g * basis_k(x).
+// A block is 64 column quads x 4 row lanes; a wave reads 1 KB of one row.
+constexpr int CA_ROWLANES = 4;
+__global__ __launch_bounds__(256) void k_channel_act_bwd(const float *__restrict__ x, const float *__restrict__ g, ChannelAct p, float *__restrict__ dx,
+                                                         float *__restrict__ partial, int64_t rows, int cols4, int rows_per_block) {
+  __shared__ float4 red[5][CA_ROWLANES][64];
+  const int cq = threadIdx.x & 63, rl = threadIdx.x >> 6, c4 = blockIdx.x * 64 + cq;
+  const int64_t r0 = blockIdx.y * (int64_t)rows_per_block, r1 = min(rows, r0 + rows_per_block);
+  float sums[5][4] = {};
+  if (c4 < cols4) {
+    float cs[5][4] = {};
+#pragma unroll
+    for (int k = 0; k < 5; k++)
+      if (p.mask >> k & 1) { float4 cv = reinterpret_cast<const float4 *>(p.coef[k])[c4]; cs[k][0] = cv.x; cs[k][1] = cv.y; cs[k][2] = cv.z; cs[k][3] = cv.w; }
+    for (int64_t r = r0 + rl; r < r1; r += CA_ROWLANES) {
+      int64_t i = r * cols4 + c4;
+      float4 xv = reinterpret_cast<const float4 *>(x)[i], gv = reinterpret_cast<const float4 *>(g)[i];
+      float xs[4] = {xv.x, xv.y, xv.z, xv.w}, gs[4] = {gv.x, gv.y, gv.z, gv.w}, acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int k = 0; k < 5; k++)
+        if (p.mask >> k & 1) {
+#pragma unroll
+          for (int e = 0; e < 4; e++) { float v, d; basis_eval(k, xs[e], v, d); acc[e] += cs[k][e] * d; sums[k][e] += gs[e] * v; }
+        }
+      reinterpret_cast<float4 *>(dx)[i] = make_float4(gs[0] * acc[0], gs[1] * acc[1], gs[2] * acc[2], gs[3] * acc[3]);
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < 5; k++) red[k][rl][cq] = make_float4(sums[k][0], sums[k][1], sums[k][2], sums[k][3]);
+  __syncthreads();
+  if (rl == 0 && c4 < cols4) {
+#pragma unroll
+    for (int k = 0; k < 5; k++)
+      if (p.mask >> k & 1) {
+        float4 a = red[k][0][cq];
+        for (int j = 1; j < CA_ROWLANES; j++) { float4 b = red[k][j][cq]; a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w; }
+        reinterpret_cast<float4 *>(partial + ((int64_t)blockIdx.y * 5 + k) * cols4 * 4)[c4] = a;
+      }
+  }
+}
+// dcoef_k[c] = sum over row blocks of partial[rb][k][c], in double, fixed order
+__global__ void k_channel_act_colsum(const float *__restrict__ partial, ChannelAct p, int nrb, int cols) {
+  int c = blockIdx.x * blockDim.x + threadIdx.x, k = blockIdx.y;
+  if (c >= cols || !(p.mask >> k & 1)) return;
+  double s = 0;
+  for (int rb = 0; rb < nrb; rb++) s += (double)partial[((int64_t)rb * 5 + k) * cols + c];
+  p.dcoef[k][c] = (float)s;
+}
+
 template <class F>
 __global__ void k_unary(const float *__restrict__ x, float *__restrict__ out, uint64_t n, F f, int vec) {
   uint64_t tid = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x, stride = (uint64_t)gridDim.x * blockDim.x;
@@ -333,6 +417,59 @@ int32_t ah_silu_mul_bwd(ah_ptr a, ah_ptr b, ah_ptr g, ah_ptr da, ah_ptr db, uint
   AH_ARG(a && b && g && da && db, "ah_silu_mul_bwd: null operand");
   hipLaunchKernelGGL(k_silu_mul_bwd, dim3(grid_for(n)), dim3(TPB), 0, stream(), dp<const float>(a), dp<const float>(b),
                      dp<const float>(g), dp<float>(da), dp<float>(db), n);
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+// mask: bit k selects basis k (0 silu, 1 relu, 2 gelu, 3 identity, 4 square); coefs[k] = f32[cols] for the selected ones
+static int32_t channel_act_args(const char *who, const ah_ptr *coefs, int32_t mask, int64_t rows, int64_t cols, ChannelAct &p, const ah_ptr *dcoefs) {
+  AH_ARG(mask > 0 && mask < 32, "%s: basis mask %d selects nothing or an unknown basis", who, mask);
+  AH_ARG(rows >= 0 && cols > 0 && cols % 4 == 0 && cols < (1ll << 31), "%s: cols %lld must be a positive multiple of 4", who, (long long)cols);
+  AH_ARG(coefs != nullptr, "%s: null coefficient list", who);
+  p.mask = mask;
+  for (int k = 0; k < 5; k++) {
+    bool on = mask >> k & 1;
+    AH_ARG(!on || (coefs[k] != 0 && coefs[k] % 16 == 0), "%s: coefficient vector %d missing or not 16-byte aligned", who, k);
+    AH_ARG(!on || !dcoefs || dcoefs[k] != 0, "%s: gradient vector %d missing", who, k);
+    p.coef[k] = on ? dp<const float>(coefs[k]) : nullptr;
+    p.dcoef[k] = on && dcoefs ? dp<float>(dcoefs[k]) : nullptr;
+  }
+  return AH_OK;
+}
+int32_t ah_channel_act(ah_ptr x, const ah_ptr *coefs, int32_t mask, ah_ptr out, int64_t rows, int64_t cols) {
+  AH_REQUIRE_READY();
+  ChannelAct p;
+  int32_t rc = channel_act_args("ah_channel_act", coefs, mask, rows, cols, p, nullptr);
+  if (rc) return rc;
+  if (rows == 0) return AH_OK;
+  AH_ARG(x && out && aligned16(x) && aligned16(out), "ah_channel_act: operands must be non-null and 16-byte aligned");
+  hipLaunchKernelGGL(k_channel_act, dim3(grid_for((uint64_t)(rows * cols / 4))), dim3(TPB), 0, stream(), dp<const float>(x), p, dp<float>(out), rows, (int)(cols / 4));
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+int32_t ah_channel_act_bwd(ah_ptr x, const ah_ptr *coefs, int32_t mask, ah_ptr grad_out, ah_ptr dx, const ah_ptr *dcoefs, int64_t rows, int64_t cols) {
+  AH_REQUIRE_READY();
+  AH_ARG(dcoefs != nullptr, "ah_channel_act_bwd: null gradient list");
+  ChannelAct p;
+  int32_t rc = channel_act_args("ah_channel_act_bwd", coefs, mask, rows, cols, p, dcoefs);
+  if (rc) return rc;
+  if (rows == 0) {
+    for (int k = 0; k < 5; k++)
+      if (mask >> k & 1) { rc = ah_fill_f32(dcoefs[k], 0.f, (uint64_t)cols); if (rc) return rc; }
+    return AH_OK;
+  }
+  AH_ARG(x && grad_out && dx && aligned16(x) && aligned16(grad_out) && aligned16(dx), "ah_channel_act_bwd: operands must be non-null and 16-byte aligned");
+  const int cols4 = (int)(cols / 4), gx = (int)cdiv(cols4, 64);
+  int nrb = (int)cdiv(rows, 64);                                  // >= 64 rows per block amortise the partial write
+  int cap = (4 * num_cus() + gx - 1) / gx;
+  if (nrb > cap) nrb = cap;
+  const int rpb = (int)cdiv(rows, nrb);
+  nrb = (int)cdiv(rows, rpb);
+  float *partial = (float *)scratch(sizeof(float) * 5 * (size_t)nrb * (size_t)cols);
+  if (!partial) return fail(AH_ERR_OOM, "ah_channel_act_bwd: no scratch");
+  hipLaunchKernelGGL(k_channel_act_bwd, dim3(gx, nrb), dim3(256), 0, stream(), dp<const float>(x), dp<const float>(grad_out), p, dp<float>(dx), partial,
+                     rows, cols4, rpb);
+  AH_LAUNCH_CHECK();
+  hipLaunchKernelGGL(k_channel_act_colsum, dim3((unsigned)cdiv(cols, 256), 5), dim3(256), 0, stream(), partial, p, nrb, (int)cols);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }

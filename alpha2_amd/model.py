@@ -169,6 +169,13 @@ def transformerBlock(ctx: Ctx, x: Variable, layer: dict, cfg: ModelConfig, Bt: i
         mlpH = mt(ctx, _eval_activation_graph(ctx, h, cfg.activationGraph), m["fc2"])
     elif act == "swiglu":
         mlpH = mt(ctx, ag.siluMul(ctx, mt(ctx, flat, m["fc_gate"]), mt(ctx, flat, m["fc_up"])), m["fc_proj"])
+    elif act == "universal" and ag._has(Bk, "channelAct"):
+        h = mt(ctx, flat, m["fc1"])
+        mlpH = mt(ctx, ag.channelAct(ctx, h, {"silu": m["act_gate"], "identity": m["act_skip"]}), m["fc2"])
+    elif act == "kan_spline" and ag._has(Bk, "channelAct"):
+        h = mt(ctx, flat, m["fc1"])
+        coefs = {"silu": m["kan_c0"], "relu": m["kan_c1"], "gelu": m["kan_c2"], "identity": m["kan_c3"], "square": m["kan_c4"]}
+        mlpH = mt(ctx, ag.channelAct(ctx, h, coefs), m["fc2"])
     elif act == "universal":
         h = mt(ctx, flat, m["fc1"])
         mlpH = mt(ctx, ag.add(ctx, ag.mul(ctx, ag.silu(ctx, h), m["act_gate"]), ag.mul(ctx, h, m["act_skip"])), m["fc2"])

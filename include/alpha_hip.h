@@ -121,6 +121,15 @@ enum { AH_GELU_BWD = 0, AH_RELU_BWD = 1, AH_SILU_BWD = 2, AH_CLAMP_BWD = 3, AH_S
 int32_t ah_unary_bwd(int32_t op, ah_ptr x, ah_ptr grad_out, ah_ptr out, uint64_t n, float p0, float p1);
 int32_t ah_silu_mul(ah_ptr a, ah_ptr b, ah_ptr out, uint64_t n);
 int32_t ah_silu_mul_bwd(ah_ptr a, ah_ptr b, ah_ptr grad_out, ah_ptr da, ah_ptr db, uint64_t n);
+/* Per-channel mixture of activation bases, the MLP activations "universal" (silu(h)*gate + h*skip) and "kan_spline"
+ * (c0 silu + c1 relu + c2 gelu + c3 h + c4 h^2) that the reference composes from separate ops (packages/model/src/gpt.ts:295-321),
+ * in one pass:  out[r,c] = sum_k coefs[k][c] * basis_k(x[r,c])  over the bases whose bit is set in `mask`
+ * (bit 0 silu, 1 relu, 2 tanh-gelu, 3 identity, 4 square).  coefs: 5 handles of f32[cols] (unused ones 0); cols % 4 == 0.
+ * Backward: dx = grad_out * sum_k coefs[k] * basis_k'(x);  dcoefs[k][c] = sum_r grad_out[r,c] * basis_k(x[r,c])
+ * (column sums in fixed order; dcoefs are overwritten). */
+int32_t ah_channel_act(ah_ptr x, const ah_ptr *coefs, int32_t mask, ah_ptr out, int64_t rows, int64_t cols);
+int32_t ah_channel_act_bwd(ah_ptr x, const ah_ptr *coefs, int32_t mask, ah_ptr grad_out, ah_ptr dx, const ah_ptr *dcoefs,
+                           int64_t rows, int64_t cols);
 /* Backend.residualDropoutAdd: out = residual + projected*mask (interfaces.ts:110; mask may be 0 = no dropout) */
 int32_t ah_residual_dropout_add(ah_ptr residual, ah_ptr projected, ah_ptr mask, ah_ptr out, uint64_t n);
 /* Backend.dropoutMask: u32-wrapping splitmix hash of (seed, counter, i) > p ? 1/(1-p) : 0

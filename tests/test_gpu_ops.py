@@ -125,6 +125,36 @@ def test_elementwise_vs_oracle(B, n):
     assert_close(B.residualDropoutAdd(dev(B, x), dev(B, y), dev(B, g)).data, O.add(orc(x), O.mul(orc(y), orc(g))).data, what="rda")
 
 
+@pytest.mark.parametrize("rows,cols", [(1, 4), (37, 24), (130, 260), (1000, 512)])
+def test_channel_activation_mixtures_match_the_composed_ops(B, rows, cols):
+    """channelAct / channelActBackward (one pass) against the oracle running the chain of ops the reference records for its
+    universal and kan_spline activations (gpt.ts:295-321): values, dx and every coefficient gradient."""
+    x = (rs.randn(rows, cols) * 2).astype(np.float32)
+    g = rs.randn(rows, cols).astype(np.float32)
+    cases = {"universal": ("silu", "identity"), "kan_spline": ("silu", "relu", "gelu", "identity", "square"), "one basis": ("gelu",)}
+    for label, names in cases.items():
+        co = {n: (rs.randn(1, cols) * 0.7).astype(np.float32) for n in names}
+        tape = rm.Tape(); ctx = rm.Ctx(tape, O)
+        xv = rm.Variable(orc(x), True)
+        cv = {n: rm.Variable(orc(c), True) for n, c in co.items()}
+        basis = {"silu": lambda: rm.silu(ctx, xv), "relu": lambda: rm.relu(ctx, xv), "gelu": lambda: rm.gelu(ctx, xv), "identity": lambda: xv,
+                 "square": lambda: rm.mul(ctx, xv, xv)}
+        out = None
+        for n in names:
+            term = rm.mul(ctx, basis[n](), cv[n])
+            out = term if out is None else rm.add(ctx, out, term)
+        tape.backward(out, O, orc(g))
+        cod = {n: dev(B, c) for n, c in co.items()}
+        assert_close(B.channelAct(dev(B, x), cod).data, out.data.data, what=label)
+        dx, dco = B.channelActBackward(dev(B, x), cod, dev(B, g))
+        assert_close(dx.data, xv.grad.data, what=label + ".dx")
+        for n in names:
+            assert dco[n].shape == (1, cols)
+            assert_close(dco[n].data, cv[n].grad.data, what=f"{label}.d{n}", scale=float(np.sqrt(rows)))
+    with pytest.raises(ValueError):
+        B.channelAct(dev(B, x), {"silu": dev(B, np.ones((1, cols + 4), np.float32))})
+
+
 def test_empty_tensors(B):
     e = dev(B, np.zeros((0, 4), np.float32))
     assert B.add(e, e).data.size == 0 and B.gelu(e).data.size == 0
