@@ -604,14 +604,15 @@ def test_flash_attention_bf16_vs_materialised(B, BH, T, D, cap):
 
 
 @pytest.mark.parametrize("M,N,K,tile", [(4000, 4072, 64, 4), (4000, 4072, 192, 4), (4000, 4072, 512, 4), (16376, 760, 128, 3), (8192, 1536, 320, 3),
-                                           (4000, 4072, 2048, 4), (16384, 768, 2112, 3)])
+                                           (4000, 4072, 2048, 4), (16384, 768, 2112, 3), (8192, 1024, 320, 2), (8184, 1016, 128, 2),
+                                           (8192, 1024, 2112, 2)])
 def test_gemm_bf16_large_tiles_direct_to_lds_kernel(B, M, N, K, tile):
     """Outputs with at least one 256x256 tile per CU take the kernel fed by global->LDS loads; edges in M and N, odd and
     even k-tile counts, every layout and epilogue.  At this size the check is a float64 numpy product of the same
     bf16-exact operands (the C oracle covers the small shapes above); fp32 accumulation of exact products."""
     from alpha2_amd import _ffi as ffi
     # ragged edges with N % 8 == 0 and M % 8 == 0 (needed by the k-major layouts); `tile` = expected column tile / 64:
-    # 256 x 256 tiles, or 256 x 192 where those fill whole rounds of CUs better (N = 760, 1536)
+    # 256 x 256 tiles, or 256 x 192 / 256 x 128 where those fill whole rounds of CUs better (N = 760, 1536 / N = 1024)
     a, b = _bf16_round(rs.randn(M, K).astype(np.float32))[0], _bf16_round(rs.randn(N, K).astype(np.float32))[0]
     want = a.astype(np.float64) @ b.astype(np.float64).T
     at, bt = np.ascontiguousarray(a.T), np.ascontiguousarray(b.T)
