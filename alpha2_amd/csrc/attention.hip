@@ -42,9 +42,11 @@ template <int D>
 __global__ __launch_bounds__(256) void k_flash_fwd_f32(FlashArgs a) {
   constexpr int P = D + 1, DB = D / 32;
   __shared__ float Ks[BC * P], Vs[BC * P];
-  int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
+  int bh, xblk;
+  flash_block(bh, xblk);
+  int b = bh / a.H, h = bh % a.H;
   int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 31, lk = lane >> 5;
-  int q0 = blockIdx.x * (WAVES * 32) + wave * 32, qi = q0 + lr;
+  int q0 = xblk * (WAVES * 32) + wave * 32, qi = q0 + lr;
   const float *Q = (const float *)a.q + b * a.q_sb + h * a.q_sh;
   const float *K = (const float *)a.k + b * a.k_sb + h * a.k_sh;
   const float *V = (const float *)a.v + b * a.v_sb + h * a.v_sh;
@@ -61,7 +63,7 @@ __global__ __launch_bounds__(256) void k_flash_fwd_f32(FlashArgs a) {
     for (int e = 0; e < 16; e++) o[d][e] = 0.f;
   float m = -INFINITY, l = 0.f;
 
-  int q_block_end = min(a.T, (int)(blockIdx.x + 1) * (WAVES * 32));   // causal: keys < q_block_end
+  int q_block_end = min(a.T, (xblk + 1) * (WAVES * 32));   // causal: keys < q_block_end
   for (int kv0 = 0; kv0 < q_block_end; kv0 += BC) {
     __syncthreads();
     load_tile_f32<D>(Ks, K, a.k_st, kv0, a.T, 1.0f);
@@ -139,9 +141,11 @@ template <int D>
 __global__ __launch_bounds__(256) void k_flash_dq_f32(FlashArgs a) {
   constexpr int P = D + 1, DB = D / 32;
   __shared__ float Ks[BC * P], Vs[BC * P];
-  int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
+  int bh, xblk;
+  flash_block(bh, xblk);
+  int b = bh / a.H, h = bh % a.H;
   int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 31, lk = lane >> 5;
-  int q0 = blockIdx.x * (WAVES * 32) + wave * 32, qi = q0 + lr;
+  int q0 = xblk * (WAVES * 32) + wave * 32, qi = q0 + lr;
   const float *Q = (const float *)a.q + b * a.q_sb + h * a.q_sh;
   const float *K = (const float *)a.k + b * a.k_sb + h * a.k_sh;
   const float *V = (const float *)a.v + b * a.v_sb + h * a.v_sh;
@@ -163,7 +167,7 @@ __global__ __launch_bounds__(256) void k_flash_dq_f32(FlashArgs a) {
 #pragma unroll
     for (int e = 0; e < 16; e++) dq[d][e] = 0.f;
 
-  int q_block_end = min(a.T, (int)(blockIdx.x + 1) * (WAVES * 32));
+  int q_block_end = min(a.T, (xblk + 1) * (WAVES * 32));
   for (int kv0 = 0; kv0 < q_block_end; kv0 += BC) {
     __syncthreads();
     load_tile_f32<D>(Ks, K, a.k_st, kv0, a.T, 1.0f);
@@ -210,9 +214,11 @@ template <int D>
 __global__ __launch_bounds__(256) void k_flash_dkv_f32(FlashArgs a) {
   constexpr int P = D + 1, DB = D / 32;
   __shared__ float Qs[BC * P], dOs[BC * P], Ls[BC], Ds[BC];
-  int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
+  int bh, xblk;
+  flash_block(bh, xblk);
+  int b = bh / a.H, h = bh % a.H;
   int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 31, lk = lane >> 5;
-  int kv_blk0 = blockIdx.x * (WAVES * 32), kv0 = kv_blk0 + wave * 32, kvi = kv0 + lr;
+  int kv_blk0 = xblk * (WAVES * 32), kv0 = kv_blk0 + wave * 32, kvi = kv0 + lr;
   const float *Q = (const float *)a.q + b * a.q_sb + h * a.q_sh;
   const float *K = (const float *)a.k + b * a.k_sb + h * a.k_sh;
   const float *V = (const float *)a.v + b * a.v_sb + h * a.v_sh;

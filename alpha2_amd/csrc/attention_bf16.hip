@@ -114,9 +114,11 @@ template <int D, bool CAPPED>
 __global__ __launch_bounds__(256, D <= 64 ? 3 : 1) void k_flash_fwd_bf16(FlashArgs a) {
   constexpr int DB = D / 32, KS = D / 16;
   __shared__ __attribute__((aligned(16))) uint16_t Ks[2][Geo<D>::ELEMS], Vs[2][Geo<D>::ELEMS];
-  int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
+  int bh, xblk;
+  flash_block(bh, xblk);
+  int b = bh / a.H, h = bh % a.H;
   int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 31, lk = lane >> 5;
-  int qblk = gridDim.x - 1 - blockIdx.x;                           // longest (latest) query blocks are scheduled first
+  int qblk = gridDim.x - 1 - xblk;                                 // longest (latest) query blocks are scheduled first
   int q0 = qblk * 128 + wave * 32, qi = q0 + lr;
   const uint16_t *Q = (const uint16_t *)a.q + b * a.q_sb + h * a.q_sh;
   const uint16_t *K = (const uint16_t *)a.k + b * a.k_sb + h * a.k_sh;
@@ -292,9 +294,11 @@ template <int D, bool CAPPED>
 __global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void k_flash_dq_bf16(FlashArgs a) {
   constexpr int DB = D / 32, KS = D / 16;
   __shared__ __attribute__((aligned(16))) uint16_t Ks[2][Geo<D>::ELEMS], Vs[2][Geo<D>::ELEMS];
-  int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
+  int bh, xblk;
+  flash_block(bh, xblk);
+  int b = bh / a.H, h = bh % a.H;
   int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 31, lk = lane >> 5;
-  int qblk = gridDim.x - 1 - blockIdx.x;
+  int qblk = gridDim.x - 1 - xblk;
   int q0 = qblk * 128 + wave * 32, qi = q0 + lr;
   const uint16_t *Q = (const uint16_t *)a.q + b * a.q_sb + h * a.q_sh;
   const uint16_t *K = (const uint16_t *)a.k + b * a.k_sb + h * a.k_sh;
@@ -390,9 +394,11 @@ __global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void k_flash_dkv_bf16(FlashAr
   constexpr int DB = D / 32, KS = D / 16;
   __shared__ __attribute__((aligned(16))) uint16_t Qs[2][Geo<D>::ELEMS], dOs[2][Geo<D>::ELEMS];
   __shared__ __attribute__((aligned(16))) float Ls[2][ST], Ds[2][ST];      // per streamed query: (max - lse) in base 2; -delta
-  int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
+  int bh, xblk;
+  flash_block(bh, xblk);
+  int b = bh / a.H, h = bh % a.H;
   int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 31, lk = lane >> 5;
-  int kv_blk0 = blockIdx.x * 128, kv0 = kv_blk0 + wave * 32, kvi = kv0 + lr;
+  int kv_blk0 = xblk * 128, kv0 = kv_blk0 + wave * 32, kvi = kv0 + lr;
   const uint16_t *Q = (const uint16_t *)a.q + b * a.q_sb + h * a.q_sh;
   const uint16_t *K = (const uint16_t *)a.k + b * a.k_sb + h * a.k_sh;
   const uint16_t *V = (const uint16_t *)a.v + b * a.v_sb + h * a.v_sh;
