@@ -115,13 +115,18 @@ template <> struct AuxVec<false> {
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t buffer_window(const void *p, int bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, max(bytes, 0), 0x00020000);
 }
+// A plain epilogue whose stores carry the non-temporal hint: for an output far larger than the caches (the logits), whose
+// lines would otherwise push the operand panels the same XCD needs again out of its L2.  Internal to the dispatcher.
+constexpr int EPI_PLAIN_STREAMED = 7;
+template <int POLICY>
 __device__ __forceinline__ void buffer_store4(float v0, float v1, float v2, float v3, float *, __amdgpu_buffer_rsrc_t r, uint32_t off) {
   u32x4 d = {__float_as_uint(v0), __float_as_uint(v1), __float_as_uint(v2), __float_as_uint(v3)};
-  __builtin_amdgcn_raw_buffer_store_b128(d, r, off, 0, 0);
+  __builtin_amdgcn_raw_buffer_store_b128(d, r, off, 0, POLICY);
 }
+template <int POLICY>
 __device__ __forceinline__ void buffer_store4(float v0, float v1, float v2, float v3, uint16_t *, __amdgpu_buffer_rsrc_t r, uint32_t off) {
   u32x2 d = {pack_bf16x2(v0, v1), pack_bf16x2(v2, v3)};
-  __builtin_amdgcn_raw_buffer_store_b64(d, r, off, 0, 0);
+  __builtin_amdgcn_raw_buffer_store_b64(d, r, off, 0, POLICY);
 }
 
 // Four 4 KB pieces of LDS that belong to the calling wave alone (nobody else reads or writes them until the next
@@ -224,13 +229,13 @@ __device__ __forceinline__ void store_tiles_lds(const GemmArgs &g, int64_t cbase
         float d[4];
 #pragma unroll
         for (int e = 0; e < 4; e++) gelu_both_f(v[e], v[e], d[e]);
-        buffer_store4(d[0], d[1], d[2], d[3], (OUT *)nullptr, buffer_window(aux_out + ge * ES, (span - ge) * ES), le);
+        buffer_store4<0>(d[0], d[1], d[2], d[3], (OUT *)nullptr, buffer_window(aux_out + ge * ES, (span - ge) * ES), le);
       } else if (EPI == AH_EPI_GELU) {
-        buffer_store4(v[0], v[1], v[2], v[3], (OUT *)nullptr, buffer_window(aux_out + ge * ES, (span - ge) * ES), le);
+        buffer_store4<0>(v[0], v[1], v[2], v[3], (OUT *)nullptr, buffer_window(aux_out + ge * ES, (span - ge) * ES), le);
 #pragma unroll
         for (int e = 0; e < 4; e++) v[e] = gelu_f(v[e]);
       }
-      buffer_store4(v[0], v[1], v[2], v[3], (OUT *)nullptr, buffer_window(c + ge * ES, (span - ge) * ES), le);
+      buffer_store4<EPI == EPI_PLAIN_STREAMED ? 2 : 0>(v[0], v[1], v[2], v[3], (OUT *)nullptr, buffer_window(c + ge * ES, (span - ge) * ES), le);
     }
     __builtin_amdgcn_sched_barrier(0);
     if (READS && p + DEPTH < NPASS) {
