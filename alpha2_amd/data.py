@@ -18,6 +18,28 @@ MAX_STRING_BYTES = 30 * 1024 * 1024          # data.ts:180
 CHUNK_BYTES = 10 * 1024 * 1024               # data.ts:238
 
 
+def loadText(path: str) -> str:
+    """data.ts:182-193: the whole file as one string; files above 30 MB are refused (tokenise those with loadAndTokenize)."""
+    size = os.stat(path).st_size
+    if size > MAX_STRING_BYTES:
+        raise ValueError(f"File is {size / 1024 / 1024:.0f}MB — too large for a single string. "
+                         "Use loadAndTokenize() for data loading.")
+    with open(path, "r", encoding="utf-8", errors="replace") as f:
+        return f.read()
+
+
+FROM_TEXT_CHUNK_CHARS = 5_000_000            # data.ts:64
+
+
+def encodeText(text: str, tokenizer) -> np.ndarray:
+    """The tokenisation step of DataLoader.fromText (data.ts:61-87): at once up to 5 M characters, else in 5 M-character
+    pieces whose token arrays are concatenated."""
+    if len(text) <= FROM_TEXT_CHUNK_CHARS:
+        return np.asarray(tokenizer.encode(text), dtype=np.int32)
+    parts = [np.asarray(tokenizer.encode(text[i:i + FROM_TEXT_CHUNK_CHARS]), dtype=np.int32) for i in range(0, len(text), FROM_TEXT_CHUNK_CHARS)]
+    return np.concatenate(parts)
+
+
 def loadAndTokenize(path: str, tokenizer, range_: Optional[Tuple[int, int]] = None) -> np.ndarray:
     """data.ts:228-290: whole range at once up to 30 MB, else 10 MB chunks cut at the last newline."""
     size = os.stat(path).st_size

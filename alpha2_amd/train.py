@@ -175,6 +175,12 @@ class DataLoader:
         self._ring = [(B._new((self.batchSize, self.blockSize), "i32"), B._new((self.batchSize, self.blockSize), "i32")) for _ in range(2)]
         self._ringIdx = 0
 
+    @classmethod
+    def fromText(cls, B: HipBackend, text: str, tokenizer, rng, batchSize: int, blockSize: int, packed: bool = False) -> "DataLoader":
+        """data.ts:61-87."""
+        from .data import encodeText
+        return cls(B, encodeText(text, tokenizer), rng, batchSize, blockSize, packed)
+
     @property
     def stepsPerEpoch(self) -> int:
         return self.length // (self.batchSize * self.blockSize)

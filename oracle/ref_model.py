@@ -11,6 +11,8 @@ Restatement of the reference's host-side training step as it runs on its CPU bac
   * Lion, Adafactor, SGD                packages/train/src/optimizers.ts:246-593 (pinned in tests/test_optimizers.py by
                                         closed forms: Lion's first step, Adafactor on a rank-one gradient, and the
                                         reference's own gradScale / entry-vs-map properties, packages/tests/src/optimizer.test.ts)
+  * evaluate()                          packages/train/src/eval.ts:25-60 (pinned in tests/test_eval.py: loss = ln V and
+                                        perplexity = V for a model whose logits are all equal; mean over the rng's batches)
   * LR schedule, grad-norm, clip        packages/train/src/trainer.ts:1088-1096,1150-1159,1297,
                                         1332-1349,1650-1656,1761-1784
   * no-decay set                        apps/cli/src/commands/train.ts:319-331
@@ -546,6 +548,21 @@ def select_token(last: np.ndarray, rng, temperature: float, topk: int, topP: flo
         if r < cum:
             return v
     return 0
+
+
+def evaluate(cfg: ModelConfig, params: dict, B: CpuRef, tokens, rng, batchSize: int, nBatches: int = 50):
+    """packages/train/src/eval.ts:25-60 after tokenisation: nBatches random batches (one DataLoader over the whole token
+    array, the caller's rng), forward pass with targets, mean of the batch losses; returns (loss, perplexity = exp(loss))."""
+    loader = DataLoader(tokens, rng, batchSize, cfg.blockSize)
+    total = 0.0
+    for _ in range(nBatches):
+        inputs, targets = loader.next_batch()
+        tape = Tape()
+        _, loss = gptForward(cfg, params, B, tape, inputs, targets)
+        total += float(loss.data.data[0])
+        tape.clear()
+    avg = total / nBatches
+    return avg, math.exp(avg)
 
 
 def sample_tokens(cfg: ModelConfig, params: dict, B: CpuRef, rng, prompt, steps: int, temperature: float, topk: int, topp=1.0) -> np.ndarray:
