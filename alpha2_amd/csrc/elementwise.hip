@@ -228,10 +228,19 @@ __global__ void k_transpose_last2(const uint32_t *__restrict__ in, uint32_t *__r
   }
 }
 
+// 4-byte elements; 16-byte stores over the aligned middle of the range, single elements at its ragged ends
 template <class T>
 __global__ void k_fill(T *__restrict__ p, T v, uint64_t n) {
+  static_assert(sizeof(T) == 4, "k_fill writes 4-byte elements");
   uint64_t tid = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x, stride = (uint64_t)gridDim.x * blockDim.x;
-  for (uint64_t i = tid; i < n; i += stride) p[i] = v;
+  uint64_t head = (4 - (((uintptr_t)p >> 2) & 3)) & 3;            // elements before the first 16-byte boundary
+  if (head > n) head = n;
+  uint64_t n4 = (n - head) >> 2;
+  uint32_t bits = __builtin_bit_cast(uint32_t, v);
+  uint4 *q = reinterpret_cast<uint4 *>(p + head);
+  for (uint64_t i = tid; i < n4; i += stride) q[i] = make_uint4(bits, bits, bits, bits);
+  for (uint64_t i = tid; i < head; i += stride) p[i] = v;
+  for (uint64_t i = head + (n4 << 2) + tid; i < n; i += stride) p[i] = v;
 }
 
 __global__ void k_axpy(float *__restrict__ a, const float *__restrict__ b, float s, uint64_t n) {
@@ -327,7 +336,7 @@ int32_t ah_fill_f32(ah_ptr dst, float value, uint64_t n) {
   AH_REQUIRE_READY();
   if (n == 0) return AH_OK;
   AH_ARG(dst != 0, "ah_fill_f32: null dst");
-  hipLaunchKernelGGL(k_fill<float>, dim3(grid_for(n)), dim3(TPB), 0, stream(), dp<float>(dst), value, n);
+  hipLaunchKernelGGL(k_fill<float>, dim3(grid_for(n / 4 + 1)), dim3(TPB), 0, stream(), dp<float>(dst), value, n);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
@@ -335,7 +344,7 @@ int32_t ah_fill_i32(ah_ptr dst, int32_t value, uint64_t n) {
   AH_REQUIRE_READY();
   if (n == 0) return AH_OK;
   AH_ARG(dst != 0, "ah_fill_i32: null dst");
-  hipLaunchKernelGGL(k_fill<int32_t>, dim3(grid_for(n)), dim3(TPB), 0, stream(), dp<int32_t>(dst), value, n);
+  hipLaunchKernelGGL(k_fill<int32_t>, dim3(grid_for(n / 4 + 1)), dim3(TPB), 0, stream(), dp<int32_t>(dst), value, n);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }

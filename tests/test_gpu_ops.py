@@ -155,6 +155,30 @@ def test_channel_activation_mixtures_match_the_composed_ops(B, rows, cols):
         B.channelAct(dev(B, x), {"silu": dev(B, np.ones((1, cols + 4), np.float32))})
 
 
+def test_fill_at_every_alignment_touches_exactly_its_range(B):
+    """ah_fill_f32 / ah_fill_i32 write 16 bytes at a time over the aligned middle of the range: every start offset modulo 16
+    bytes and ragged lengths, with sentinels either side."""
+    import ctypes
+    from alpha2_amd import _ffi as ffi
+    total = 4096
+    for off in range(0, 5):
+        for n in (0, 1, 2, 3, 4, 5, 7, 8, 63, 64, 65, 1000, 4000):
+            host = np.full(total, -7.0, np.float32)
+            buf = dev(B, host)
+            ffi.check(B.lib.ah_fill_f32(B._ptr(buf) + 4 * off, 2.5, n))
+            B._dirty(buf)
+            got = buf.data
+            want = host.copy(); want[off:off + n] = 2.5
+            assert np.array_equal(got, want), (off, n)
+    ib = dev(B, np.full(100, 9, np.int32), "i32")
+    ffi.check(B.lib.ah_fill_i32(B._ptr(ib) + 4, -3, 50))
+    B._dirty(ib)
+    want = np.full(100, 9, np.int32); want[1:51] = -3
+    assert np.array_equal(ib.data, want)
+    big = B.full([1 << 20], 1.25)
+    assert np.all(big.data == 1.25)
+
+
 def test_empty_tensors(B):
     e = dev(B, np.zeros((0, 4), np.float32))
     assert B.add(e, e).data.size == 0 and B.gelu(e).data.size == 0
