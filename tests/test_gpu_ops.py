@@ -756,6 +756,26 @@ def test_gemm_microbench_shapes_forward_and_both_backward(B, N):
         lib.ah_free(p)
 
 
+@pytest.mark.parametrize("store", ["bf16", "f32"])
+def test_flash_attention_heads_are_independent_of_how_blocks_are_dealt_out(B, store):
+    """The kernels decode (head, sequence block) from the linear workgroup id so that a head's blocks share one XCD; heads
+    past the last multiple of 8 keep the natural order.  20 heads x 3 sequence blocks in one call must equal, bit for bit,
+    20 calls of one head each (where the mapping is the identity)."""
+    BH, T, D, scale, cap = 20, 384, 64, 0.125, 30.0
+    q, k, v, do = (_gauss_bf16((BH, T, D), 60 + i, 1.0) for i in range(4))
+    put = (lambda x: B.castStore(dev(B, x), "bf16")) if store == "bf16" else (lambda x: dev(B, x))
+    r = B.flashAttention(put(q), put(k), put(v), T, scale, cap)
+    g = B.flashAttentionBackward(put(q), put(k), put(v), r["output"], put(do), r["lse"], T, scale, cap)
+    whole = [np.asarray(t.data).reshape(BH, T, -1).copy() for t in (r["output"], g["dQ"], g["dK"], g["dV"])] + [np.asarray(r["lse"].data).reshape(BH, T).copy()]
+    for h in range(BH):
+        one = lambda x: put(x[h:h + 1])
+        r1 = B.flashAttention(one(q), one(k), one(v), T, scale, cap)
+        g1 = B.flashAttentionBackward(one(q), one(k), one(v), r1["output"], one(do), r1["lse"], T, scale, cap)
+        single = [np.asarray(t.data).reshape(T, -1) for t in (r1["output"], g1["dQ"], g1["dK"], g1["dV"])] + [np.asarray(r1["lse"].data).reshape(T)]
+        for a, b_, what in zip(whole, single, ("O", "dQ", "dK", "dV", "LSE")):
+            assert np.array_equal(a[h], b_), (h, what)
+
+
 @pytest.mark.parametrize("T", [256, 1024, 2048])
 @pytest.mark.parametrize("cap", [0.0, 30.0])
 def test_flash_attention_microbench_shapes(B, T, cap):
