@@ -76,14 +76,22 @@ __global__ void k_layernorm(const float *__restrict__ x, const float *__restrict
   float inv_dim = 1.0f / (float)dim;
   if constexpr (NV > 0) {
     int nv = dim >> 2;
-    float4 v[NV > 0 ? NV : 1];
+    float4 v[NV > 0 ? NV : 1], wv[NV > 0 ? NV : 1], bv[NV > 0 ? NV : 1];
+    const bool out_vec = (((uintptr_t)out | ((uintptr_t)dim * sizeof(OUT))) & 7u) == 0;      // 8-byte aligned rows of a 2-byte output
     float s = 0.f;
 #pragma unroll
     for (int i = 0; i < NV; i++) {
       int j = lane + 64 * i;
       v[i] = j < nv ? reinterpret_cast<const float4 *>(xr)[j] : make_float4(0, 0, 0, 0);
-      s += (v[i].x + v[i].y) + (v[i].z + v[i].w);
     }
+#pragma unroll
+    for (int i = 0; i < NV; i++) {       // weight and bias travel with the row instead of behind the two reductions
+      int j = lane + 64 * i;
+      wv[i] = j < nv ? reinterpret_cast<const float4 *>(w)[j] : make_float4(0, 0, 0, 0);
+      bv[i] = j < nv ? reinterpret_cast<const float4 *>(b)[j] : make_float4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < NV; i++) s += (v[i].x + v[i].y) + (v[i].z + v[i].w);
     float mean = wave_sum(s) * inv_dim;
     float q = 0.f;
 #pragma unroll
@@ -99,11 +107,15 @@ __global__ void k_layernorm(const float *__restrict__ x, const float *__restrict
     for (int i = 0; i < NV; i++) {
       int j = lane + 64 * i;
       if (j < nv) {
-        float4 ww = reinterpret_cast<const float4 *>(w)[j], bb = reinterpret_cast<const float4 *>(b)[j];
+        float4 ww = wv[i], bb = bv[i];
         float o0 = (v[i].x - mean) * rstd * ww.x + bb.x, o1 = (v[i].y - mean) * rstd * ww.y + bb.y;
         float o2 = (v[i].z - mean) * rstd * ww.z + bb.z, o3 = (v[i].w - mean) * rstd * ww.w + bb.w;
-        Io<OUT>::st(orow, 4 * j + 0, o0); Io<OUT>::st(orow, 4 * j + 1, o1);
-        Io<OUT>::st(orow, 4 * j + 2, o2); Io<OUT>::st(orow, 4 * j + 3, o3);
+        if constexpr (sizeof(OUT) == 4) reinterpret_cast<float4 *>(orow)[j] = make_float4(o0, o1, o2, o3);
+        else if (out_vec) reinterpret_cast<uint2 *>(orow)[j] = make_uint2(pack_bf16x2(o0, o1), pack_bf16x2(o2, o3));
+        else {
+          Io<OUT>::st(orow, 4 * j + 0, o0); Io<OUT>::st(orow, 4 * j + 1, o1);
+          Io<OUT>::st(orow, 4 * j + 2, o2); Io<OUT>::st(orow, 4 * j + 3, o3);
+        }
       }
     }
   } else {
@@ -497,7 +509,7 @@ __global__ void k_token_windows(const int32_t *__restrict__ corpus, int64_t n_to
 template <class OUT>
 static int32_t launch_ln(ah_ptr x, ah_ptr w, ah_ptr b, ah_ptr out, int64_t rows, int64_t dim, float eps) {
   dim3 grid((unsigned)cdiv(rows, WPB)), blk(TPB);
-  bool vec = (dim % 4 == 0) && dim <= 2048 && aligned16(x) && aligned16(w) && aligned16(b);
+  bool vec = (dim % 4 == 0) && dim <= 2048 && aligned16(x) && aligned16(w) && aligned16(b) && (sizeof(OUT) == 2 || aligned16(out));
   int nvl = vec ? (int)cdiv(dim / 4, 64) : 0;
 #define LN_CASE(NV) hipLaunchKernelGGL((k_layernorm<NV, OUT>), grid, blk, 0, stream(), dp<const float>(x), dp<const float>(w), dp<const float>(b), dp<OUT>(out), rows, (int)dim, eps)
   switch (nvl) {
