@@ -245,8 +245,9 @@ int32_t run(const GemmArgs &ga, int batch, int out_dtype) {
       double useful = (double)ga.N / (double)(cdiv(ga.N, bn) * bn);        // columns of edge tiles that exist
       return useful * (double)t / (double)(cdiv(t, cus) * cus);
     };
-    // (narrower tiles read more from LDS per flop: measured ~3 % and ~8 % slower per flop than the 256-wide one)
-    double f256 = ga.N >= 256 ? fill(256) : 0.0, f192 = 0.97 * fill(192), f128 = 0.92 * fill(128);
+    // (narrower tiles read more from LDS per flop: measured ~3 % and ~8 % slower per flop than the 256-wide one; with two
+    // k-major operands, whose transposing LDS reads run at half rate, the 128-wide tile is ~35 % slower per flop)
+    double f256 = ga.N >= 256 ? fill(256) : 0.0, f192 = 0.97 * fill(192), f128 = (AKM && BKM ? 0.65 : 0.92) * fill(128);
     int bn = f256 >= f192 && f256 >= f128 ? 256 : f192 >= f128 ? 192 : 128;
 
     if ((bn == 256 ? f256 : bn == 192 ? f192 : f128) >= 0.7)
