@@ -310,8 +310,57 @@ void note_gemm_split(int nsplit) { g_last_split = nsplit; }
 }  // namespace ah
 
 namespace {
-struct GroupPlan { ah_ptr table; int count, blocks, layout, out_dtype; bool live; };
+// A plan holds the device table of its problems.  Where it pays (see split_tail), the problems at the end of the launch
+// are each two entries, one per half of k: the first writes (or accumulates into) C, the second the plan's workspace, which
+// k_grouped_join then adds to C.
+struct JoinPart { float *c; float *ws; int M, N; int64_t ldc; };
+struct GroupPlan {
+  ah_ptr table; int count, blocks, layout, out_dtype; bool live;
+  ah_ptr parts, ws; int nparts;
+};
 std::vector<GroupPlan> g_plans;      // plan id = index + 1
+
+// C += ws, ws = 0 for every k-split problem of a grouped launch: block (x, y) walks the float4s of part y.  The workspace
+// is left all zero, so the second halves of an ACCUMULATING run (whose epilogue adds to what it finds) store into it just
+// as those of a plain run do.
+__global__ __launch_bounds__(256) void k_grouped_join(const JoinPart *__restrict__ parts) {
+  const JoinPart p = parts[blockIdx.y];
+  const int nq = p.N >> 2;
+  const int64_t total = (int64_t)p.M * nq;
+  for (int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x; q < total; q += (int64_t)gridDim.x * 256) {
+    const int64_t row = q / nq;
+    const int col = (int)(q - row * nq) * 4;
+    float4 *dst = (float4 *)(p.c + row * p.ldc + col), *src = (float4 *)(p.ws + row * p.N + col);
+    const float4 w = *src;
+    float4 v = *dst;
+    v.x += w.x; v.y += w.y; v.z += w.z; v.w += w.w;
+    *dst = v;
+    *src = make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+}
+
+constexpr int GROUP_ROUND = 256;     // tiles that run at a time: one per CU
+
+// The launch runs its 256 x 256 tiles one per CU, in rounds of 256; all tiles of a weight-gradient group take the same
+// time, so a last round of t < 256 tiles costs a whole round.  Cutting the problems that make up that round in two along
+// k turns it into 2 t half-length tiles, which still run at once when t <= 128: the round then costs half.  Chooses whole
+// problems from the end of the list whose tiles add up to between t and 128 and returns their indices (ascending), or
+// nothing when no such choice exists.
+std::vector<int> split_tail(const AhGemm *descs, int count, int64_t blocks) {
+  std::vector<int> chosen;
+  const int64_t tail = blocks % GROUP_ROUND;
+  if (descs[0].out_dtype != AH_F32 || tail == 0 || tail > GROUP_ROUND / 2) return chosen;
+  int64_t sum = 0;
+  for (int i = count - 1; i >= 0 && sum < tail; i--) {
+    const AhGemm &q = descs[i];
+    const int64_t t = cdiv(q.m, 256) * cdiv(q.n, 256);
+    if (q.k % 128 != 0 || q.n % 4 != 0 || sum + t > GROUP_ROUND / 2) continue;
+    chosen.insert(chosen.begin(), i);
+    sum += t;
+  }
+  if (sum < tail) chosen.clear();
+  return chosen;
+}
 }  // namespace
 
 extern "C" {
@@ -351,12 +400,58 @@ int32_t ah_gemm_grouped_plan(const AhGemm *descs, int32_t count, uint64_t *plan_
     blocks += cdiv(q.m, 256) * cdiv(q.n, 256);
     AH_ARG(blocks < (1ll << 31), "ah_gemm_grouped_plan: too many tiles");
   }
-  ah_ptr table = 0;
-  int32_t rc = ah_alloc(tab.size() * sizeof(GemmGroupEntry), &table);
-  if (rc) return rc;
-  rc = ah_upload(table, tab.data(), tab.size() * sizeof(GemmGroupEntry));
-  if (rc) { ah_free(table); return rc; }
-  g_plans.push_back(GroupPlan{table, count, (int)blocks, layout, out_dtype, true});
+  // the problems that make up a short last round are cut in two along k: they move to the end of the table as pairs of
+  // entries, the second of which writes the workspace
+  GroupPlan plan{0, count, (int)blocks, layout, out_dtype, true, 0, 0, 0};
+  const std::vector<int> chosen = split_tail(descs, count, blocks);
+  std::vector<JoinPart> parts;
+  int32_t rc = AH_OK;
+  if (!chosen.empty()) {
+    int64_t ws_bytes = 0;
+    for (int i : chosen) ws_bytes += descs[i].m * descs[i].n * 4;
+    rc = ah_alloc((size_t)ws_bytes, &plan.ws);
+    if (rc) return rc;
+    rc = ah_fill_f32(plan.ws, 0.f, (uint64_t)(ws_bytes / 4));         // the workspace is all zero between runs (see k_grouped_join)
+    std::vector<GemmGroupEntry> cut_tab;
+    std::vector<bool> cut((size_t)count, false);
+    for (int i : chosen) cut[(size_t)i] = true;
+    int64_t nblocks = 0;
+    auto push = [&](GemmGroupEntry e) {
+      e.tile_start = (int)nblocks;
+      nblocks += cdiv(e.M, 256) * cdiv(e.N, 256);
+      cut_tab.push_back(e);
+    };
+    for (int i = 0; i < count; i++)
+      if (!cut[(size_t)i]) push(tab[(size_t)i]);
+    char *ws = dp<char>(plan.ws);
+    for (int i : chosen) {
+      GemmGroupEntry lo = tab[(size_t)i], hi = lo;
+      lo.K = hi.K = lo.K / 2;
+      hi.a = (const char *)lo.a + (akm ? (int64_t)lo.K * lo.lda : (int64_t)lo.K) * 2;
+      hi.b = (const char *)lo.b + (bkm ? (int64_t)lo.K * lo.ldb : (int64_t)lo.K) * 2;
+      hi.c = ws;
+      hi.ldc = lo.N;
+      parts.push_back(JoinPart{(float *)lo.c, (float *)ws, lo.M, lo.N, lo.ldc});
+      ws += (int64_t)lo.M * lo.N * 4;
+      push(lo);
+      push(hi);
+    }
+    tab.swap(cut_tab);
+    plan.count = (int)tab.size();
+    plan.blocks = (int)nblocks;
+    plan.nparts = (int)parts.size();
+    if (rc == AH_OK) rc = ah_alloc(parts.size() * sizeof(JoinPart), &plan.parts);
+    if (rc == AH_OK) rc = ah_upload(plan.parts, parts.data(), parts.size() * sizeof(JoinPart));
+  }
+  if (rc == AH_OK) rc = ah_alloc(tab.size() * sizeof(GemmGroupEntry), &plan.table);
+  if (rc == AH_OK) rc = ah_upload(plan.table, tab.data(), tab.size() * sizeof(GemmGroupEntry));
+  if (rc) {
+    if (plan.ws) ah_free(plan.ws);
+    if (plan.parts) ah_free(plan.parts);
+    if (plan.table) ah_free(plan.table);
+    return rc;
+  }
+  g_plans.push_back(plan);
   *plan_out = g_plans.size();
   return AH_OK;
 }
@@ -367,18 +462,30 @@ int32_t ah_gemm_grouped_run(uint64_t plan, int32_t epilogue) {
   const GroupPlan &p = g_plans[plan - 1];
   AH_ARG(epilogue == AH_EPI_NONE || (epilogue == AH_EPI_ACCUM && p.out_dtype == AH_F32), "ah_gemm_grouped_run: epilogue %d is not provided for this plan", epilogue);
   const GemmGroupEntry *tab = dp<const GemmGroupEntry>(p.table);
+  int32_t rc;
   switch (p.layout) {
-    case AH_GEMM_NT: return gemm_bf16_dma_nt_grouped(tab, p.count, p.blocks, epilogue, p.out_dtype);
-    case AH_GEMM_NN: return gemm_bf16_dma_nn_grouped(tab, p.count, p.blocks, epilogue, p.out_dtype);
-    default: return gemm_bf16_dma_tn_grouped(tab, p.count, p.blocks, epilogue, p.out_dtype);
+    case AH_GEMM_NT: rc = gemm_bf16_dma_nt_grouped(tab, p.count, p.blocks, epilogue, p.out_dtype); break;
+    case AH_GEMM_NN: rc = gemm_bf16_dma_nn_grouped(tab, p.count, p.blocks, epilogue, p.out_dtype); break;
+    default: rc = gemm_bf16_dma_tn_grouped(tab, p.count, p.blocks, epilogue, p.out_dtype);
   }
+  if (rc != AH_OK || p.nparts == 0) return rc;
+  hipLaunchKernelGGL(k_grouped_join, dim3(128, (unsigned)p.nparts), dim3(256), 0, stream(), dp<const JoinPart>(p.parts));
+  AH_LAUNCH_CHECK();
+  ah::note_gemm_split(2);
+  return AH_OK;
 }
 
 int32_t ah_gemm_grouped_destroy(uint64_t plan) {
   AH_REQUIRE_READY();
   AH_ARG(plan >= 1 && plan <= g_plans.size() && g_plans[plan - 1].live, "ah_gemm_grouped_destroy: unknown plan %llu", (unsigned long long)plan);
-  g_plans[plan - 1].live = false;
-  return ah_free(g_plans[plan - 1].table);
+  GroupPlan &p = g_plans[plan - 1];
+  p.live = false;
+  if (p.nparts > 0) {
+    ah_free(p.parts);
+    ah_free(p.ws);
+    p.nparts = 0;
+  }
+  return ah_free(p.table);
 }
 
 int32_t ah_gemm_last_kernel(char *name, int32_t capacity, int32_t *nsplit) {

@@ -247,7 +247,10 @@ int32_t ah_gemm(const AhGemm *g);
  * (packages/autograd/src/ops.ts:197-234).  Requirements per problem: bf16 operands, batch 1, k a multiple of 64,
  * 16-byte aligned rows, epilogue NONE or ACCUM; all problems share layout and output type.  The plan copies the
  * descriptors to the device once; ah_gemm_grouped_run only launches (safe inside graph capture) and takes the
- * epilogue (AH_EPI_NONE, or AH_EPI_ACCUM for f32 outputs) so one plan serves first and later micro-batches. */
+ * epilogue (AH_EPI_NONE, or AH_EPI_ACCUM for f32 outputs) so one plan serves first and later micro-batches.
+ * Tiles run one per CU in rounds of 256; when the last round of an f32 plan is at most half full, the plan cuts the
+ * problems that make up that round in two along k (second halves into a workspace the plan owns, added to C by a short
+ * second kernel in a fixed order), which halves the cost of that round; ah_gemm_last_kernel then reports 2 slices. */
 int32_t ah_gemm_grouped_plan(const AhGemm *descs, int32_t count, uint64_t *plan_out);
 int32_t ah_gemm_grouped_run(uint64_t plan, int32_t epilogue);
 int32_t ah_gemm_grouped_destroy(uint64_t plan);

@@ -686,10 +686,12 @@ def test_gemm_grouped_matches_separate_products(B):
     ffi.check(B.lib.ah_gemm_grouped_plan(arr, len(descs), C.byref(plan)))
     ffi.check(B.lib.ah_gemm_grouped_run(plan.value, ffi.EPI_NONE))
     assert B.lastGemmKernel()[0].startswith("k_gemm_bf16_dma_grouped<true, true")
+    assert B.lastGemmKernel()[1] == 2                     # 47 tiles: less than half a round, so every problem is cut in two along k
     for out, want, (m, n) in zip(outs, wants, shapes):
         B._dirty(out)
         assert_close(out.data.reshape(m, n), want, rel=1e-4, what=f"grouped NONE {m}x{n}")
     ffi.check(B.lib.ah_gemm_grouped_run(plan.value, ffi.EPI_ACCUM))
+    assert B.lastGemmKernel()[1] == 2
     for out, want, (m, n) in zip(outs, wants, shapes):
         B._dirty(out)
         assert_close(out.data.reshape(m, n), 2 * want, rel=1e-4, what=f"grouped ACCUM {m}x{n}")
@@ -698,6 +700,49 @@ def test_gemm_grouped_matches_separate_products(B):
     assert B.lib.ah_gemm_grouped_run(plan.value, ffi.EPI_NONE) != 0 and b"unknown plan" in B.lib.ah_last_error()
     bad = (ffi.AhGemm * 1)(ffi.AhGemm(ffi.GEMM_TN, ffi.BF16, ffi.F32, ffi.EPI_NONE, 64, 64, 100, 64, 64, 64, 1, 0, 0, 0, 1 << 20, 1 << 20, 1 << 20, 0))
     assert B.lib.ah_gemm_grouped_plan(bad, 1, C.byref(plan)) != 0 and b"multiple of 64" in B.lib.ah_last_error()
+
+
+@pytest.mark.parametrize("shapes,K,cut", [
+    ([(4096, 4096), (768, 768), (1280, 1792)], 256, True),       # 256 + 9 + 35 tiles: the last round (44) is cut, the first problem is not
+    ([(2048, 2048), (1280, 1792)], 320, False),                  # 64 + 35 tiles, k not a multiple of 128: nothing to cut
+    ([(3072, 3072), (768, 768)], 128, False),                    # 144 + 9 tiles: more than half a round, cutting would not pay
+])
+def test_gemm_grouped_last_round_cut_in_two_along_k(B, shapes, K, cut):
+    """The problems that make up a short last round of the launch are computed as two k-halves and joined; the others
+    are not touched, and neither are plans where the cut does not apply.  Checked against float64 products; a second run
+    of the same plan must give bit-identical results (the join adds the halves in a fixed order)."""
+    import ctypes as C
+    from alpha2_amd import TensorData, _ffi as ffi
+    keep, descs, wants, outs = [], [], [], []
+    for m, n in shapes:
+        gy, x = _bf16_round(rs.randn(K, m).astype(np.float32))[0], _bf16_round(rs.randn(K, n).astype(np.float32))[0]
+        tg, tx = TensorData(gy.shape, "f16", _bf16_round(gy)[1]), TensorData(x.shape, "f16", _bf16_round(x)[1])
+        out = B.zeros((m, n))
+        keep += [tg, tx]
+        outs.append(out)
+        wants.append(gy.astype(np.float64).T @ x.astype(np.float64))
+        descs.append(ffi.AhGemm(ffi.GEMM_TN, ffi.BF16, ffi.F32, ffi.EPI_NONE, m, n, K, m, n, n, 1, 0, 0, 0, B._ptr(tg), B._ptr(tx), B._ptr(out), 0))
+    arr = (ffi.AhGemm * len(descs))(*descs)
+    plan = C.c_uint64()
+    ffi.check(B.lib.ah_gemm_grouped_plan(arr, len(descs), C.byref(plan)))
+    first = []
+    for run in range(2):
+        ffi.check(B.lib.ah_gemm_grouped_run(plan.value, ffi.EPI_NONE))
+        assert B.lastGemmKernel()[1] == (2 if cut else 1)
+        for i, (out, want, (m, n)) in enumerate(zip(outs, wants, shapes)):
+            B._dirty(out)
+            got = out.data.reshape(m, n).copy()
+            assert_close(got, want, rel=1e-4, what=f"run {run} {m}x{n}")
+            if run == 0:
+                first.append(got)
+            else:
+                assert np.array_equal(got, first[i]), f"{m}x{n}: the second run differs from the first"
+    for run in (2, 3):                                    # accumulating runs: their second halves rely on the join leaving the workspace zero
+        ffi.check(B.lib.ah_gemm_grouped_run(plan.value, ffi.EPI_ACCUM))
+        for out, want, (m, n) in zip(outs, wants, shapes):
+            B._dirty(out)
+            assert_close(out.data.reshape(m, n), run * want, rel=1e-4, what=f"ACCUM {m}x{n}")
+    ffi.check(B.lib.ah_gemm_grouped_destroy(plan.value))
 
 
 # ---------------------------------------------------------------------------------------------- parity at the benchmark sizes
