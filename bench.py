@@ -126,7 +126,7 @@ def main():
     g_flops, g_ms = sum(r["flops"] for r in gemm), sum(r["ms"] for r in gemm)
     # the dominant kernel = the GEMM instantiation with the most arithmetic per step among launches that are one kernel
     # (a split-K launch is followed by its reduce kernel inside the same event bracket, so it is not a clean sample; the
-    # grouped launch is kept: when the tiles of its last round are cut in two along k, the bracket also holds the ~15 us
+    # grouped launch is kept: when the tiles of its last round are cut in two along k, the bracket also holds the ~25 us
     # kernel that joins the halves, which is counted against it)
     groups = {}
     for r in gemm:
