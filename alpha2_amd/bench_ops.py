@@ -167,7 +167,12 @@ def bench_bandwidth(b: Bench):
     ms = b.time(lambda: ffi.check(lib.ah_embedding(wte, tok, eo, rows, dim, V, ffi.F32)))
     b.record("embedding gather 16384x768", ms, nbytes=rows * dim * 8, note="uniform token ids")
     ms = b.time(lambda: ffi.check(lib.ah_embedding_bwd(tok, eo, gw, rows, dim, V, 0)))
-    b.record("embedding scatter-add 16384x768", ms, nbytes=rows * dim * 8 + V * dim * 4, note="includes zero-filling the [50304, 768] gradient")
+    b.record("embedding scatter-add 16384x768", ms, nbytes=rows * dim * 8 + V * dim * 4, note="uniform ids; includes zero-filling the [50304, 768] gradient")
+    from .train import zipfBatch
+    zh = np.ascontiguousarray(zipfBatch(4, 16, rows // 16, V)[0].data, dtype=np.int32).reshape(-1)
+    ffi.check(lib.ah_upload(tok, zh.ctypes.data_as(C.c_void_p), zh.nbytes))
+    ms = b.time(lambda: ffi.check(lib.ah_embedding_bwd(tok, eo, gw, rows, dim, V, 0)))
+    b.record("embedding scatter-add, power-law ids", ms, nbytes=rows * dim * 8 + V * dim * 4, note="Zipf(1.1) ids as in the step benchmark; same bytes")
     b.release()
 
     p, g, m, v, sh = (b.randn(P, ffi.F32, 0.02, s) for s in (6, 7, 8, 9, 10))

@@ -55,6 +55,41 @@ __global__ void k_embedding_bwd(const int32_t *__restrict__ idx, const float *__
   float *dst = gw + r * dim;
   for (int64_t j = lane; j < dim; j += 64) unsafeAtomicAdd(dst + j, src[j]);
 }
+// The same with the repeats inside a block of 64 consecutive positions summed first: a block's first occurrence of an id
+// adds up the rows of all its occurrences in the block (in position order) and issues ONE atomic per element.  Token ids
+// follow a power law; the most frequent one takes a twelfth of all positions, and atomics to one address are served one
+// after the other, which made that row the whole cost of the plain kernel.  One wave per position, 16 at a time; lane l
+// holds columns l, l + 64, ... of the 1024 that group y covers.
+constexpr int EB_POS = 64;
+__global__ __launch_bounds__(1024) void k_embedding_bwd_blocks(const int32_t *__restrict__ idx, const float *__restrict__ g, float *__restrict__ gw,
+                                                               int64_t n_idx, int64_t dim, int64_t vocab) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int64_t p0 = blockIdx.x * (int64_t)EB_POS;
+  int32_t mine = p0 + lane < n_idx ? idx[p0 + lane] : -1;
+  if (mine < 0 || mine >= vocab) mine = -1;                 // ids out of range are skipped
+  const int64_t c0 = blockIdx.y * (int64_t)1024 + lane;
+  for (int p = wave; p < EB_POS; p += 16) {
+    const int32_t t = __shfl(mine, p, 64);
+    if (t < 0) continue;
+    uint64_t m = __ballot(mine == t);
+    if (m & ((1ull << p) - 1)) continue;                    // a repeat: its row is added by the first occurrence
+    float acc[16];
+#pragma unroll
+    for (int k = 0; k < 16; k++) acc[k] = 0.f;
+    while (m) {
+      const int q = __builtin_ctzll(m);
+      m &= m - 1;
+      const float *src = g + (p0 + q) * dim;
+#pragma unroll
+      for (int k = 0; k < 16; k++)
+        if (c0 + 64 * k < dim) acc[k] += src[c0 + 64 * k];
+    }
+    float *dst = gw + (int64_t)t * dim;
+#pragma unroll
+    for (int k = 0; k < 16; k++)
+      if (c0 + 64 * k < dim) unsafeAtomicAdd(dst + c0 + 64 * k, acc[k]);
+  }
+}
 __global__ void k_pos_embedding_bwd(const float *__restrict__ g, float *__restrict__ gw, int64_t batch, int64_t td, int accumulate) {
   int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
   if (i >= td) return;
@@ -572,8 +607,12 @@ int32_t ah_embedding_bwd(ah_ptr idx, ah_ptr grad_out, ah_ptr grad_w, int64_t n_i
   if (!accumulate) { int32_t rc = ah_fill_f32(grad_w, 0.f, (uint64_t)(vocab * dim)); if (rc) return rc; }
   if (n_idx == 0 || dim == 0) return AH_OK;
   AH_ARG(idx && grad_out, "ah_embedding_bwd: null operand");
-  hipLaunchKernelGGL(k_embedding_bwd, dim3((unsigned)cdiv(n_idx, WPB)), dim3(TPB), 0, stream(), dp<const int32_t>(idx),
-                     dp<const float>(grad_out), dp<float>(grad_w), n_idx, dim, vocab);
+  if (cdiv(n_idx, EB_POS) < (1ll << 31) && cdiv(dim, 1024) <= 65535)
+    hipLaunchKernelGGL(k_embedding_bwd_blocks, dim3((unsigned)cdiv(n_idx, EB_POS), (unsigned)cdiv(dim, 1024)), dim3(1024), 0, stream(),
+                       dp<const int32_t>(idx), dp<const float>(grad_out), dp<float>(grad_w), n_idx, dim, vocab);
+  else
+    hipLaunchKernelGGL(k_embedding_bwd, dim3((unsigned)cdiv(n_idx, WPB)), dim3(TPB), 0, stream(), dp<const int32_t>(idx),
+                       dp<const float>(grad_out), dp<float>(grad_w), n_idx, dim, vocab);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }

@@ -289,6 +289,28 @@ def test_embedding_fwd_bwd(B):
     assert_close(gw.data, ref.embedding_backward(orc(idx), orc(g), V).data, what="embeddingBackward")
 
 
+@pytest.mark.parametrize("n,dim,V", [(1000, 768, 300), (16384, 768, 50304), (131, 1000, 7), (513, 2052, 40), (300, 50, 9)])
+def test_embedding_backward_with_heavily_repeated_ids(B, n, dim, V):
+    """Power-law ids (the most frequent one takes a large share of the positions, as token ids do), positions that do not
+    fill the last block, rows that do not fill the last column group, ids out of range (skipped), and accumulation onto an
+    existing gradient; against a float64 scatter-add."""
+    from alpha2_amd import _ffi as ffi
+    r = np.random.RandomState(n + dim)
+    idx = np.minimum((V * r.rand(n) ** 4).astype(np.int64), V - 1).astype(np.int32)
+    idx[::97] = -3
+    idx[5::89] = V + 2
+    g = r.randn(n, dim).astype(np.float32)
+    ok = (idx >= 0) & (idx < V)
+    want = np.zeros((V, dim), np.float64)
+    np.add.at(want, idx[ok], g[ok].astype(np.float64))
+    di, dg = dev(B, idx, "i32"), dev(B, g)
+    gw = B.zeros((V, dim))
+    for k in (1, 2):                                       # the second call accumulates
+        ffi.check(B.lib.ah_embedding_bwd(B._ptr(di), B._ptr(dg), B._ptr(gw), n, dim, V, 0 if k == 1 else 1))
+        B._dirty(gw)
+        assert_close(gw.data.reshape(V, dim), k * want, what=f"scatter-add x{k}")
+
+
 @pytest.mark.parametrize("rows,dim", [(1, 2), (7, 48), (1024, 128), (333, 768), (5, 1000), (3, 4096)])
 def test_layernorm_fwd_bwd(B, rows, dim):
     x = (rs.randn(rows, dim) * 2 + 0.5).astype(np.float32)
