@@ -52,6 +52,11 @@ class AhRng(C.Structure):
     _fields_ = [("s0", i32), ("s1", i32), ("has_spare", i32), ("_pad", i32), ("spare", C.c_double)]
 
 
+class AhColsumJob(C.Structure):
+    _fields_ = [("partials", C.c_uint64), ("dw", C.c_uint64), ("db", C.c_uint64), ("rows", C.c_int64), ("dim", C.c_int64),
+                ("accumulate", C.c_int32), ("reserved", C.c_int32)]
+
+
 class AhAdamW(C.Structure):
     _fields_ = [("lr", f32), ("beta1", f32), ("beta2", f32), ("eps", f32), ("weight_decay", f32),
                 ("bc1", f32), ("bc2", f32), ("grad_scale", f32)]
@@ -102,6 +107,9 @@ SIGNATURES = {
     "ah_pos_embedding_bwd": [u64, u64, i64, i64, i64, i32],
     "ah_layernorm": [u64, u64, u64, u64, i64, i64, f32, i32],
     "ah_layernorm_bwd": [u64, u64, u64, i32, u64, u64, u64, u64, u64, i64, i64, f32, i32],
+    "ah_layernorm_bwd_partials_bytes": [i64, i64],
+    "ah_layernorm_bwd_deferred": [u64, u64, u64, i32, u64, u64, u64, u64, i64, i64, f32],
+    "ah_layernorm_colsums": [C.POINTER(AhColsumJob), i32],
     "ah_cross_entropy": [u64, i32, u64, u64, u64, i64, i64],
     "ah_cross_entropy_bwd": [u64, i32, u64, u64, u64, f32, u64, i64, i64],
     "ah_cross_entropy_fwd_bwd": [u64, i32, u64, u64, u64, u64, f32, u64, i64, i64],
@@ -145,6 +153,7 @@ def load():
         fn = getattr(lib, name)
         fn.argtypes = args
         fn.restype = i32
+    lib.ah_layernorm_bwd_partials_bytes.restype = i64       # a size, not a status
     lib.ah_last_error.argtypes = []
     lib.ah_last_error.restype = C.c_char_p
     _lib = lib

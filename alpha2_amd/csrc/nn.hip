@@ -212,8 +212,8 @@ __global__ void k_layernorm_bwd(const float *__restrict__ x, const float *__rest
 }
 // column sums of the per-block partials: 32 columns per block, 32 row slices per column (1024 threads, so that the few
 // blocks of this launch keep many loads in flight), fixed summation order
-__global__ __launch_bounds__(1024) void k_colsum_partials(const float *__restrict__ part_dw, const float *__restrict__ part_db, int nparts, int dim,
-                                                          float *__restrict__ dw, float *__restrict__ db, int accumulate) {
+__device__ __forceinline__ void colsum_partials(const float *__restrict__ part_dw, const float *__restrict__ part_db, int nparts, int dim,
+                                                float *__restrict__ dw, float *__restrict__ db, int accumulate) {
   __shared__ double sa[32][33], sc[32][33];
   int cx = threadIdx.x & 31, sl = threadIdx.x >> 5, j = blockIdx.x * 32 + cx;
   double a = 0, c = 0;
@@ -236,6 +236,19 @@ __global__ __launch_bounds__(1024) void k_colsum_partials(const float *__restric
     dw[j] = (accumulate ? dw[j] : 0.f) + (float)a;
     db[j] = (accumulate ? db[j] : 0.f) + (float)c;
   }
+}
+__global__ __launch_bounds__(1024) void k_colsum_partials(const float *__restrict__ part_dw, const float *__restrict__ part_db, int nparts, int dim,
+                                                          float *__restrict__ dw, float *__restrict__ db, int accumulate) {
+  colsum_partials(part_dw, part_db, nparts, dim, dw, db, accumulate);
+}
+// the column sums of several LayerNorms in one launch (job y), the jobs passed by value
+struct ColsumJob { const float *part; float *dw, *db; int nparts, dim, accumulate, pad; };
+constexpr int COLSUM_JOBS = 64;
+struct ColsumJobs { ColsumJob j[COLSUM_JOBS]; };
+__global__ __launch_bounds__(1024) void k_colsum_partials_batched(ColsumJobs jobs) {
+  const ColsumJob &q = jobs.j[blockIdx.y];
+  if ((int)blockIdx.x * 32 >= q.dim) return;
+  colsum_partials(q.part, q.part + (size_t)q.nparts * q.dim, q.nparts, q.dim, q.dw, q.db, q.accumulate);
 }
 
 // Register-resident LayerNorm backward for rows of up to 256*NV floats (dim % 4 == 0): x, g and the residual gradient
@@ -637,31 +650,24 @@ int32_t ah_layernorm(ah_ptr x, ah_ptr w, ah_ptr b, ah_ptr out, int64_t rows, int
   return out_dtype == AH_F32 ? launch_ln<float>(x, w, b, out, rows, dim, eps) : launch_ln<uint16_t>(x, w, b, out, rows, dim, eps);
 }
 
-int32_t ah_layernorm_bwd(ah_ptr x, ah_ptr w, ah_ptr grad_out, int32_t grad_dtype, ah_ptr residual_grad, ah_ptr dx, ah_ptr dx_bf16,
-                         ah_ptr dw, ah_ptr db, int64_t rows, int64_t dim, float eps, int32_t accumulate) {
-  AH_REQUIRE_READY();
-  AH_ARG(grad_dtype == AH_F32 || grad_dtype == AH_BF16, "ah_layernorm_bwd: grad dtype must be f32 or bf16");
-  if (dim == 0) return AH_OK;
-  AH_ARG(dw && db, "ah_layernorm_bwd: null dw/db");
-  if (rows == 0) {
-    if (!accumulate) { int32_t rc = ah_fill_f32(dw, 0.f, (uint64_t)dim); if (rc) return rc; return ah_fill_f32(db, 0.f, (uint64_t)dim); }
-    return AH_OK;
-  }
-  AH_ARG(x && w && grad_out && dx, "ah_layernorm_bwd: null operand");
-  size_t lds = sizeof(float) * 2 * WPB * (size_t)dim;
-  AH_ARG(lds <= 160 * 1024, "ah_layernorm_bwd: dim %lld too large for the LDS column accumulators", (long long)dim);
 #ifndef LNB_ROWS
 #define LNB_ROWS 8
 #endif
 #ifndef LNB_CAP
 #define LNB_CAP 2
 #endif
-  int nblk = (int)cdiv(rows, WPB * LNB_ROWS);     // >= 8 rows per wave amortises the partial write
-  int cap = num_cus() * LNB_CAP;
+// blocks of a LayerNorm-backward launch = rows of its partial column sums
+static int ln_bwd_blocks(int64_t rows) {
+  int64_t nblk = cdiv(rows, WPB * LNB_ROWS);      // >= 8 rows per wave amortises the partial write
+  int64_t cap = (int64_t)num_cus() * LNB_CAP;
   if (nblk > cap) nblk = cap;
-  if (nblk < 1) nblk = 1;
-  float *part = (float *)scratch(sizeof(float) * 2 * (size_t)nblk * (size_t)dim);
-  if (!part) return fail(AH_ERR_OOM, "ah_layernorm_bwd: no scratch");
+  return nblk < 1 ? 1 : (int)nblk;
+}
+
+// dx and the per-block partial column sums part[2][nblk][dim] (dw partials, then db partials)
+static int32_t ln_bwd_launch(ah_ptr x, ah_ptr w, ah_ptr grad_out, int32_t grad_dtype, ah_ptr residual_grad, ah_ptr dx, ah_ptr dx_bf16,
+                             float *part, int nblk, int64_t rows, int64_t dim, float eps) {
+  size_t lds = sizeof(float) * 2 * WPB * (size_t)dim;
   float *part_dw = part, *part_db = part + (size_t)nblk * dim;
   bool vec = dim % 4 == 0 && dim <= 2048 && aligned16(x) && aligned16(w) && aligned16(dx) && (grad_out % 8 == 0) && (residual_grad % 16 == 0) &&
              (dx_bf16 % 8 == 0) && (grad_dtype == AH_BF16 || aligned16(grad_out));
@@ -681,9 +687,65 @@ int32_t ah_layernorm_bwd(ah_ptr x, ah_ptr w, ah_ptr grad_out, int32_t grad_dtype
     hipLaunchKernelGGL(k_layernorm_bwd<uint16_t>, dim3(nblk), dim3(TPB), lds, stream(), dp<const float>(x), dp<const float>(w),
                        dp<const uint16_t>(grad_out), dp<const float>(residual_grad), dp<float>(dx), dp<uint16_t>(dx_bf16), part_dw, part_db, rows, (int)dim, eps);
   AH_LAUNCH_CHECK();
-  hipLaunchKernelGGL(k_colsum_partials, dim3((unsigned)cdiv(dim, 32)), dim3(1024), 0, stream(), part_dw, part_db, nblk, (int)dim,
+  return AH_OK;
+}
+
+int32_t ah_layernorm_bwd(ah_ptr x, ah_ptr w, ah_ptr grad_out, int32_t grad_dtype, ah_ptr residual_grad, ah_ptr dx, ah_ptr dx_bf16,
+                         ah_ptr dw, ah_ptr db, int64_t rows, int64_t dim, float eps, int32_t accumulate) {
+  AH_REQUIRE_READY();
+  AH_ARG(grad_dtype == AH_F32 || grad_dtype == AH_BF16, "ah_layernorm_bwd: grad dtype must be f32 or bf16");
+  if (dim == 0) return AH_OK;
+  AH_ARG(dw && db, "ah_layernorm_bwd: null dw/db");
+  if (rows == 0) {
+    if (!accumulate) { int32_t rc = ah_fill_f32(dw, 0.f, (uint64_t)dim); if (rc) return rc; return ah_fill_f32(db, 0.f, (uint64_t)dim); }
+    return AH_OK;
+  }
+  AH_ARG(x && w && grad_out && dx, "ah_layernorm_bwd: null operand");
+  AH_ARG(sizeof(float) * 2 * WPB * (size_t)dim <= 160 * 1024, "ah_layernorm_bwd: dim %lld too large for the LDS column accumulators", (long long)dim);
+  const int nblk = ln_bwd_blocks(rows);
+  float *part = (float *)scratch(sizeof(float) * 2 * (size_t)nblk * (size_t)dim);
+  if (!part) return fail(AH_ERR_OOM, "ah_layernorm_bwd: no scratch");
+  int32_t rc = ln_bwd_launch(x, w, grad_out, grad_dtype, residual_grad, dx, dx_bf16, part, nblk, rows, dim, eps);
+  if (rc) return rc;
+  hipLaunchKernelGGL(k_colsum_partials, dim3((unsigned)cdiv(dim, 32)), dim3(1024), 0, stream(), part, part + (size_t)nblk * dim, nblk, (int)dim,
                      dp<float>(dw), dp<float>(db), accumulate);
   AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+
+int64_t ah_layernorm_bwd_partials_bytes(int64_t rows, int64_t dim) {
+  if (rows <= 0 || dim <= 0 || !ready()) return 0;
+  return (int64_t)sizeof(float) * 2 * ln_bwd_blocks(rows) * dim;
+}
+
+int32_t ah_layernorm_bwd_deferred(ah_ptr x, ah_ptr w, ah_ptr grad_out, int32_t grad_dtype, ah_ptr residual_grad, ah_ptr dx, ah_ptr dx_bf16,
+                                  ah_ptr partials, int64_t rows, int64_t dim, float eps) {
+  AH_REQUIRE_READY();
+  AH_ARG(grad_dtype == AH_F32 || grad_dtype == AH_BF16, "ah_layernorm_bwd_deferred: grad dtype must be f32 or bf16");
+  AH_ARG(rows > 0 && dim > 0, "ah_layernorm_bwd_deferred: empty input [%lld, %lld]", (long long)rows, (long long)dim);
+  AH_ARG(x && w && grad_out && dx && partials, "ah_layernorm_bwd_deferred: null operand");
+  AH_ARG(partials % 4 == 0, "ah_layernorm_bwd_deferred: partials must be aligned to 4 bytes");
+  AH_ARG(sizeof(float) * 2 * WPB * (size_t)dim <= 160 * 1024, "ah_layernorm_bwd_deferred: dim %lld too large for the LDS column accumulators", (long long)dim);
+  return ln_bwd_launch(x, w, grad_out, grad_dtype, residual_grad, dx, dx_bf16, dp<float>(partials), ln_bwd_blocks(rows), rows, dim, eps);
+}
+
+int32_t ah_layernorm_colsums(const AhColsumJob *jobs, int32_t count) {
+  AH_REQUIRE_READY();
+  AH_ARG(count >= 0 && (count == 0 || jobs != nullptr), "ah_layernorm_colsums: bad job list (count %d)", count);
+  for (int32_t first = 0; first < count; first += COLSUM_JOBS) {
+    ColsumJobs tab;
+    const int n = count - first < COLSUM_JOBS ? count - first : COLSUM_JOBS;
+    int64_t max_dim = 0;
+    for (int i = 0; i < n; i++) {
+      const AhColsumJob &q = jobs[first + i];
+      AH_ARG(q.rows > 0 && q.dim > 0 && q.dim < (1ll << 31), "ah_layernorm_colsums: job %d: empty input [%lld, %lld]", first + i, (long long)q.rows, (long long)q.dim);
+      AH_ARG(q.partials && q.dw && q.db, "ah_layernorm_colsums: job %d: null operand", first + i);
+      tab.j[i] = ColsumJob{dp<const float>(q.partials), dp<float>(q.dw), dp<float>(q.db), ln_bwd_blocks(q.rows), (int)q.dim, q.accumulate, 0};
+      if (q.dim > max_dim) max_dim = q.dim;
+    }
+    hipLaunchKernelGGL(k_colsum_partials_batched, dim3((unsigned)cdiv(max_dim, 32), (unsigned)n), dim3(1024), 0, stream(), tab);
+    AH_LAUNCH_CHECK();
+  }
   return AH_OK;
 }
 

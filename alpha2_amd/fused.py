@@ -122,6 +122,13 @@ class FusedTrainer:
         self.loss_hist_cap = 4096
         self.loss_hist, self.norm_hist = a(self.loss_hist_cap * 4), a(self.loss_hist_cap * 8)
         self._batches: List[Tuple[int, int]] = []
+        # partial column sums of every LayerNorm backward (dw, db), reduced by ONE launch at the end of backward
+        part_bytes = int(self.lib.ah_layernorm_bwd_partials_bytes(BT, Cc))
+        assert part_bytes > 0
+        self._ln_jobs: List[Tuple[str, int]] = [("lnF", a(part_bytes))]
+        for l in range(self.L):
+            self._ln_jobs += [(f"layer.{l}.ln2", a(part_bytes)), (f"layer.{l}.ln1", a(part_bytes))]
+        self._ln_part = dict(self._ln_jobs)
         self._plan_weight_grads()
 
     def _plan_weight_grads(self):
@@ -240,23 +247,26 @@ class FusedTrainer:
 
         self._gemm(NN, self.logits, self.p("lmHead", True), self.dlnb, BT, Cc, V, V, Cc, Cc)
         cur = 0
-        check(lib.ah_layernorm_bwd(self.x[L], self.p("lnF.weight"), self.dlnb, BF16, 0, self.dx[cur], self.dy_fc2[L - 1], self.g("lnF.weight"),
-                                   self.g("lnF.bias"), BT, Cc, 1e-5, acc))
+        check(lib.ah_layernorm_bwd_deferred(self.x[L], self.p("lnF.weight"), self.dlnb, BF16, 0, self.dx[cur], self.dy_fc2[L - 1],
+                                            self._ln_part["lnF"], BT, Cc, 1e-5))
         for l in reversed(range(L)):
             pre = f"layer.{l}."
             # MLP: x_out = x_mid + fc2(gelu(fc1(ln2(x_mid))))
             self._gemm(NN, self.dy_fc2[l], self.p(pre + "mlp.fc2", True), self.dh[l], BT, Fd, Cc, Cc, Fd, Fd, BF16, ffi.EPI_MUL_AUX, self.hgrad[l])
             self._gemm(NN, self.dh[l], self.p(pre + "mlp.fc1", True), self.dlnb, BT, Cc, Fd, Fd, Cc, Cc)
-            check(lib.ah_layernorm_bwd(self.xmid[l], self.p(pre + "ln2.weight"), self.dlnb, BF16, self.dx[cur], self.dx[cur ^ 1], self.dy_wo[l],
-                                       self.g(pre + "ln2.weight"), self.g(pre + "ln2.bias"), BT, Cc, 1e-5, acc))
+            check(lib.ah_layernorm_bwd_deferred(self.xmid[l], self.p(pre + "ln2.weight"), self.dlnb, BF16, self.dx[cur], self.dx[cur ^ 1], self.dy_wo[l],
+                                                self._ln_part[pre + "ln2"], BT, Cc, 1e-5))
             cur ^= 1
             # attention: x_mid = x_in + wo(attn(wqkv(ln1(x_in))))
             self._gemm(NN, self.dy_wo[l], self.p(pre + "attn.wo", True), self.datt, BT, Cc, Cc, Cc, Cc, Cc)
             self._flash(l, True)
             self._gemm(NN, self.dqkv[l], self.p(pre + "attn.wqkv", True), self.dlnb, BT, Cc, 3 * Cc, 3 * Cc, Cc, Cc)
-            check(lib.ah_layernorm_bwd(self.x[l], self.p(pre + "ln1.weight"), self.dlnb, BF16, self.dx[cur], self.dx[cur ^ 1],
-                                       self.dy_fc2[l - 1] if l > 0 else self.dxb0, self.g(pre + "ln1.weight"), self.g(pre + "ln1.bias"), BT, Cc, 1e-5, acc))
+            check(lib.ah_layernorm_bwd_deferred(self.x[l], self.p(pre + "ln1.weight"), self.dlnb, BF16, self.dx[cur], self.dx[cur ^ 1],
+                                                self.dy_fc2[l - 1] if l > 0 else self.dxb0, self._ln_part[pre + "ln1"], BT, Cc, 1e-5))
             cur ^= 1
+        jobs = (ffi.AhColsumJob * len(self._ln_jobs))(*[
+            ffi.AhColsumJob(part, self.g(name + ".weight"), self.g(name + ".bias"), BT, Cc, acc, 0) for name, part in self._ln_jobs])
+        check(lib.ah_layernorm_colsums(jobs, len(self._ln_jobs)))
         self._weight_grads(wepi)
         check(lib.ah_embedding_bwd(self.tok, self.dx[cur], self.g("wte"), BT, Cc, V, acc))
         check(lib.ah_pos_embedding_bwd(self.dx[cur], self.g("wpe"), self.batch, self.T, Cc, acc))

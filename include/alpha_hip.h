@@ -198,6 +198,20 @@ int32_t ah_layernorm(ah_ptr x, ah_ptr w, ah_ptr b, ah_ptr out, int64_t rows, int
 int32_t ah_layernorm_bwd(ah_ptr x, ah_ptr w, ah_ptr grad_out, int32_t grad_dtype, ah_ptr residual_grad,
                          ah_ptr dx, ah_ptr dx_bf16, ah_ptr dw, ah_ptr db, int64_t rows, int64_t dim, float eps,
                          int32_t accumulate);
+/* The same with the column sums put off: the per-block partial sums of dw and db go to `partials` (caller-owned, at
+ * least ah_layernorm_bwd_partials_bytes(rows, dim) bytes, which is 0 before ah_init), and ONE later call of
+ * ah_layernorm_colsums reduces those of many LayerNorms (the 2 L + 1 of a model's backward pass) in one launch instead of
+ * one small launch each; per job the result is bit-identical to ah_layernorm_bwd's.  The reference computes dw / db inside
+ * layerNormBackward (packages/tensor/src/cpu_ref.ts, layerNormBackward); nothing of this split shows at the Backend level. */
+typedef struct {
+  ah_ptr  partials, dw, db;
+  int64_t rows, dim;          /* as passed to ah_layernorm_bwd_deferred */
+  int32_t accumulate, reserved;
+} AhColsumJob;
+int64_t ah_layernorm_bwd_partials_bytes(int64_t rows, int64_t dim);
+int32_t ah_layernorm_bwd_deferred(ah_ptr x, ah_ptr w, ah_ptr grad_out, int32_t grad_dtype, ah_ptr residual_grad,
+                                  ah_ptr dx, ah_ptr dx_bf16, ah_ptr partials, int64_t rows, int64_t dim, float eps);
+int32_t ah_layernorm_colsums(const AhColsumJob *jobs, int32_t count);
 /* loss[0] = mean_i (logsumexp(logits[i,:]) - logits[i,target[i]]); lse[N] kept for backward (0 = skip) */
 int32_t ah_cross_entropy(ah_ptr logits, int32_t logits_dtype, ah_ptr targets_i32, ah_ptr loss_out, ah_ptr lse_out,
                          int64_t n, int64_t c);

@@ -324,6 +324,42 @@ def test_layernorm_fwd_bwd(B, rows, dim):
     assert_close(r["db"].data, db.data, what="ln.db")
 
 
+def test_layernorm_backward_with_column_sums_put_off(B):
+    """ah_layernorm_bwd_deferred + one ah_layernorm_colsums over several LayerNorms of different sizes gives exactly the dx,
+    dw and db of ah_layernorm_bwd, also when accumulating onto existing dw / db; bad jobs are reported."""
+    import ctypes as C
+    from alpha2_amd import _ffi as ffi
+    lib = B.lib
+    cases = [(16384, 768), (333, 768), (7, 48), (5, 1000), (1, 2), (4096, 1024)]
+    keep, jobs, wants = [], [], []
+    for rows, dim in cases:
+        x, w, g = (rs.randn(rows, dim) * 2 + 0.5).astype(np.float32), rs.randn(dim).astype(np.float32), rs.randn(rows, dim).astype(np.float32)
+        dx_, dw_, db_ = B.zeros((rows, dim)), dev(B, np.full(dim, 3.0, np.float32)), dev(B, np.full(dim, -2.0, np.float32))
+        dx2, dw2, db2 = B.zeros((rows, dim)), dev(B, np.full(dim, 3.0, np.float32)), dev(B, np.full(dim, -2.0, np.float32))
+        xd, wd, gd = dev(B, x), dev(B, w), dev(B, g)
+        nbytes = lib.ah_layernorm_bwd_partials_bytes(rows, dim)
+        assert nbytes >= 8 * dim
+        part = B.zeros((nbytes // 4,))
+        keep += [xd, wd, gd, dx_, dw_, db_, dx2, dw2, db2, part]
+        ffi.check(lib.ah_layernorm_bwd(B._ptr(xd), B._ptr(wd), B._ptr(gd), ffi.F32, 0, B._ptr(dx_), 0, B._ptr(dw_), B._ptr(db_), rows, dim, 1e-5, 1))
+        ffi.check(lib.ah_layernorm_bwd_deferred(B._ptr(xd), B._ptr(wd), B._ptr(gd), ffi.F32, 0, B._ptr(dx2), 0, B._ptr(part), rows, dim, 1e-5))
+        jobs.append(ffi.AhColsumJob(B._ptr(part), B._ptr(dw2), B._ptr(db2), rows, dim, 1, 0))
+        wants.append((dx_, dw_, db_, dx2, dw2, db2))
+    arr = (ffi.AhColsumJob * len(jobs))(*jobs)
+    ffi.check(lib.ah_layernorm_colsums(arr, len(jobs)))
+    for (rows, dim), ts in zip(cases, wants):
+        for t in ts:
+            B._dirty(t)
+        assert np.array_equal(ts[0].data, ts[3].data), (rows, dim, "dx")
+        assert np.array_equal(ts[1].data, ts[4].data), (rows, dim, "dw")
+        assert np.array_equal(ts[2].data, ts[5].data), (rows, dim, "db")
+        assert not np.array_equal(ts[1].data, np.full(dim, 3.0, np.float32))
+    assert lib.ah_layernorm_colsums(arr, 0) == 0
+    bad = (ffi.AhColsumJob * 1)(ffi.AhColsumJob(0, 1 << 20, 1 << 20, 4, 4, 0, 0))
+    assert lib.ah_layernorm_colsums(bad, 1) != 0 and b"null operand" in lib.ah_last_error()
+    assert lib.ah_layernorm_bwd_deferred(1 << 20, 1 << 20, 1 << 20, ffi.F32, 0, 1 << 20, 0, 0, 4, 4, 1e-5) != 0 and b"null operand" in lib.ah_last_error()
+
+
 @pytest.mark.parametrize("n,c", [(2, 3), (11, 37), (128, 256), (16, 50304)])
 def test_cross_entropy_fwd_bwd(B, n, c):
     lg = (rs.randn(n, c) * 3).astype(np.float32)
