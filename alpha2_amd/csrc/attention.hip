@@ -43,7 +43,8 @@ __global__ __launch_bounds__(256) void k_flash_fwd_f32(FlashArgs a) {
   constexpr int P = D + 1, DB = D / 32;
   __shared__ float Ks[BC * P], Vs[BC * P];
   int bh, xblk;
-  flash_block(bh, xblk);
+  flash_block(bh, xblk, flash_head_group(a.T, D, 4));
+  xblk = gridDim.x - 1 - xblk;                                     // longest (latest) query blocks are scheduled first
   int b = bh / a.H, h = bh % a.H;
   int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 31, lk = lane >> 5;
   int q0 = xblk * (WAVES * 32) + wave * 32, qi = q0 + lr;
@@ -142,7 +143,8 @@ __global__ __launch_bounds__(256) void k_flash_dq_f32(FlashArgs a) {
   constexpr int P = D + 1, DB = D / 32;
   __shared__ float Ks[BC * P], Vs[BC * P];
   int bh, xblk;
-  flash_block(bh, xblk);
+  flash_block(bh, xblk, flash_head_group(a.T, D, 4));
+  xblk = gridDim.x - 1 - xblk;                                     // longest (latest) query blocks are scheduled first
   int b = bh / a.H, h = bh % a.H;
   int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 31, lk = lane >> 5;
   int q0 = xblk * (WAVES * 32) + wave * 32, qi = q0 + lr;
@@ -215,7 +217,7 @@ __global__ __launch_bounds__(256) void k_flash_dkv_f32(FlashArgs a) {
   constexpr int P = D + 1, DB = D / 32;
   __shared__ float Qs[BC * P], dOs[BC * P], Ls[BC], Ds[BC];
   int bh, xblk;
-  flash_block(bh, xblk);
+  flash_block(bh, xblk, flash_head_group(a.T, D, 4));
   int b = bh / a.H, h = bh % a.H;
   int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 31, lk = lane >> 5;
   int kv_blk0 = xblk * (WAVES * 32), kv0 = kv_blk0 + wave * 32, kvi = kv0 + lr;

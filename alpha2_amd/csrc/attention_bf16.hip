@@ -115,7 +115,7 @@ __global__ __launch_bounds__(256, D <= 64 ? 3 : 1) void k_flash_fwd_bf16(FlashAr
   constexpr int DB = D / 32, KS = D / 16;
   __shared__ __attribute__((aligned(16))) uint16_t Ks[2][Geo<D>::ELEMS], Vs[2][Geo<D>::ELEMS];
   int bh, xblk;
-  flash_block(bh, xblk);
+  flash_block(bh, xblk, flash_head_group(a.T, D, 2));
   int b = bh / a.H, h = bh % a.H;
   int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 31, lk = lane >> 5;
   int qblk = gridDim.x - 1 - xblk;                                 // longest (latest) query blocks are scheduled first
@@ -295,7 +295,7 @@ __global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void k_flash_dq_bf16(FlashArg
   constexpr int DB = D / 32, KS = D / 16;
   __shared__ __attribute__((aligned(16))) uint16_t Ks[2][Geo<D>::ELEMS], Vs[2][Geo<D>::ELEMS];
   int bh, xblk;
-  flash_block(bh, xblk);
+  flash_block(bh, xblk, flash_head_group(a.T, D, 2));
   int b = bh / a.H, h = bh % a.H;
   int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 31, lk = lane >> 5;
   int qblk = gridDim.x - 1 - xblk;
@@ -395,7 +395,7 @@ __global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void k_flash_dkv_bf16(FlashAr
   __shared__ __attribute__((aligned(16))) uint16_t Qs[2][Geo<D>::ELEMS], dOs[2][Geo<D>::ELEMS];
   __shared__ __attribute__((aligned(16))) float Ls[2][ST], Ds[2][ST];      // per streamed query: (max - lse) in base 2; -delta
   int bh, xblk;
-  flash_block(bh, xblk);
+  flash_block(bh, xblk, flash_head_group(a.T, D, 2));
   int b = bh / a.H, h = bh % a.H;
   int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, lr = lane & 31, lk = lane >> 5;
   int kv_blk0 = xblk * 128, kv0 = kv_blk0 + wave * 32, kvi = kv0 + lr;
