@@ -859,12 +859,15 @@ def test_gemm_microbench_shapes_forward_and_both_backward(B, N):
         lib.ah_free(p)
 
 
+@pytest.mark.parametrize("BH,T,D", [(20, 384, 64), (60, 2048, 128)])
 @pytest.mark.parametrize("store", ["bf16", "f32"])
-def test_flash_attention_heads_are_independent_of_how_blocks_are_dealt_out(B, store):
-    """The kernels decode (head, sequence block) from the linear workgroup id so that a head's blocks share one XCD; heads
-    past the last multiple of 8 keep the natural order.  20 heads x 3 sequence blocks in one call must equal, bit for bit,
-    20 calls of one head each (where the mapping is the identity)."""
-    BH, T, D, scale, cap = 20, 384, 64, 0.125, 30.0
+def test_flash_attention_heads_are_independent_of_how_blocks_are_dealt_out(B, store, BH, T, D):
+    """The kernels decode (head, sequence block) from the linear workgroup id so that a head's blocks share one XCD and an
+    XCD runs the longest blocks of a group of its heads first; heads past the last multiple of 8 keep the natural order.
+    One call over all heads must equal, bit for bit, one call per head (where the mapping is the identity).  20 heads x 3
+    blocks: one group of 2 heads per XCD and 4 heads left over; 60 heads x 16 blocks at head size 128: 7 heads per XCD in
+    groups of 6 + 1 (bf16) or 3 + 3 + 1 (f32), 4 left over."""
+    scale, cap = float(1.0 / np.sqrt(D)), 30.0
     q, k, v, do = (_gauss_bf16((BH, T, D), 60 + i, 1.0) for i in range(4))
     put = (lambda x: B.castStore(dev(B, x), "bf16")) if store == "bf16" else (lambda x: dev(B, x))
     r = B.flashAttention(put(q), put(k), put(v), T, scale, cap)
