@@ -499,7 +499,9 @@ __global__ __launch_bounds__(256) void k_ce_fwd_bwd(const uint16_t *__restrict__
   for (int k = 0; k < CE_CHUNKS; k++) {
     const int j = threadIdx.x + k * 256;
     if (j < nvec) {
-      const uint4 u = reinterpret_cast<const uint4 *>(p)[j];
+      typedef unsigned u4v __attribute__((ext_vector_type(4)));     // 1.65 GB read once and written once: non-temporal (-6 %)
+      const u4v un = __builtin_nontemporal_load(reinterpret_cast<const u4v *>(p) + j);
+      const uint4 u = make_uint4(un.x, un.y, un.z, un.w);
       r[k] = u;
       float v[8] = {bf16_bits_to_f32(u.x & 0xffff), bf16_bits_to_f32(u.x >> 16), bf16_bits_to_f32(u.y & 0xffff), bf16_bits_to_f32(u.y >> 16),
                     bf16_bits_to_f32(u.z & 0xffff), bf16_bits_to_f32(u.z >> 16), bf16_bits_to_f32(u.w & 0xffff), bf16_bits_to_f32(u.w >> 16)};
@@ -535,7 +537,8 @@ __global__ __launch_bounds__(256) void k_ce_fwd_bwd(const uint16_t *__restrict__
     if (j8 < nvec) {
       uint32_t o[4];
       ce_grad8(r[k], l, scale, j8 == (t >> 3) ? (int)(t & 7) : -1, o);
-      reinterpret_cast<uint4 *>(q)[j8] = make_uint4(o[0], o[1], o[2], o[3]);
+      typedef unsigned u4v __attribute__((ext_vector_type(4)));
+      __builtin_nontemporal_store(u4v{o[0], o[1], o[2], o[3]}, reinterpret_cast<u4v *>(q) + j8);
     }
   }
 }
