@@ -229,7 +229,7 @@ __device__ __forceinline__ void store_tiles_lds(const GemmArgs &g, int64_t cbase
         float d[4];
 #pragma unroll
         for (int e = 0; e < 4; e++) gelu_both_f(v[e], v[e], d[e]);
-        buffer_store4<0>(d[0], d[1], d[2], d[3], (OUT *)nullptr, buffer_window(aux_out + ge * ES, (span - ge) * ES), le);
+        buffer_store4<2>(d[0], d[1], d[2], d[3], (OUT *)nullptr, buffer_window(aux_out + ge * ES, (span - ge) * ES), le);   // kept for backward: streamed past the caches
       } else if (EPI == AH_EPI_GELU) {
         buffer_store4<0>(v[0], v[1], v[2], v[3], (OUT *)nullptr, buffer_window(aux_out + ge * ES, (span - ge) * ES), le);
 #pragma unroll
