@@ -295,9 +295,13 @@ __global__ __launch_bounds__(256) void k_layernorm_bwd_vec(const float *__restri
     for (int i = 0; i < NV; i++) {
       int j = lane + 64 * i;
       if (j < nv) {
-        xo[i] = reinterpret_cast<const float4 *>(xr)[j];
+        // x and the residual gradient were written long ago and are used here for the last time; dx (f32) is next read two
+        // GEMMs and an attention later: all three go past the caches (the bf16 copy of dx, the next GEMM's operand, does not)
+        typedef float f4v __attribute__((ext_vector_type(4)));
+        { const f4v t_ = __builtin_nontemporal_load(reinterpret_cast<const f4v *>(xr) + j); xo[i] = make_float4(t_.x, t_.y, t_.z, t_.w); }
         go[i].load(grow, j);
-        ro[i] = res ? reinterpret_cast<const float4 *>(res + row * (int64_t)dim)[j] : make_float4(0, 0, 0, 0);
+        if (res) { const f4v t_ = __builtin_nontemporal_load(reinterpret_cast<const f4v *>(res + row * (int64_t)dim) + j); ro[i] = make_float4(t_.x, t_.y, t_.z, t_.w); }
+        else ro[i] = make_float4(0, 0, 0, 0);
       } else {
         xo[i] = make_float4(0, 0, 0, 0); go[i].zero(); ro[i] = make_float4(0, 0, 0, 0);
       }
@@ -340,7 +344,7 @@ __global__ __launch_bounds__(256) void k_layernorm_bwd_vec(const float *__restri
         d.x = rstd * (gv[i].x * wv[i].x - (s1 + xv[i].x * s2)); d.y = rstd * (gv[i].y * wv[i].y - (s1 + xv[i].y * s2));
         d.z = rstd * (gv[i].z * wv[i].z - (s1 + xv[i].z * s2)); d.w = rstd * (gv[i].w * wv[i].w - (s1 + xv[i].w * s2));
         if (res) { d.x += rv[i].x; d.y += rv[i].y; d.z += rv[i].z; d.w += rv[i].w; }
-        reinterpret_cast<float4 *>(dx + row * (int64_t)dim)[j] = d;
+        { typedef float f4v __attribute__((ext_vector_type(4))); __builtin_nontemporal_store(f4v{d.x, d.y, d.z, d.w}, reinterpret_cast<f4v *>(dx + row * (int64_t)dim) + j); }
         if (dx16) reinterpret_cast<uint2 *>(dx16 + row * (int64_t)dim)[j] = make_uint2(pack_bf16x2(d.x, d.y), pack_bf16x2(d.z, d.w));
       }
     }
