@@ -38,7 +38,7 @@ PEAK = {"bf16": 2500.0, "f32": 157.3}          # MI355X dense MFMA, TFLOP/s
 # HBM-side bytes per launch of the kernels that can be the dominant one, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
 # runs of this benchmark (counter values scaled by what the same counters read for a plain copy of known size: x2.0
 # for FETCH_SIZE, x1.0 for WRITE_SIZE); the counter summary is kept under profiles/.
-TRAFFIC_BYTES = {"k_gemm_bf16_dma_grouped<true, true, 0, float>": 9.2737e9 + 0.5226e9}
+TRAFFIC_BYTES = {"k_gemm_bf16_dma_grouped<true, true, 0, float>": 9.2452e9 + 0.5226e9}
 
 
 def step_flops(cfg, tokens):
