@@ -88,7 +88,7 @@ SIGNATURES = {
     "ah_channel_act": [u64, C.c_void_p, i32, u64, i64, i64], "ah_channel_act_bwd": [u64, C.c_void_p, i32, u64, u64, C.c_void_p, i64, i64],
     "ah_silu_mul": [u64, u64, u64, u64], "ah_silu_mul_bwd": [u64, u64, u64, u64, u64, u64],
     "ah_residual_dropout_add": [u64, u64, u64, u64, u64],
-    "ah_dropout_mask": [u64, u64, i32, i32, f32],
+    "ah_dropout_mask": [u64, u64, i32, i32, C.c_double],
     "ah_masked_fill": [u64, u64, u64, u64, u64, f32], "ah_causal_mask": [u64, i64],
     "ah_cast": [u64, i32, u64, i32, u64], "ah_check_finite": [u64, u64, u64],
     "ah_transpose": [u64, u64, i32, p_i64, i32, i32],
@@ -121,6 +121,7 @@ SIGNATURES = {
     "ah_flash_fwd": [C.POINTER(AhFlash)], "ah_flash_bwd": [C.POINTER(AhFlash)],
     "ah_adamw": [u64, u64, u64, u64, u64, C.POINTER(AhAdamW), u64, u64, u64],
     "ah_clip_coef": [u64, f32, f32, u64],
+    "ah_step_guard": [u64, u64, f32, f32, C.c_double, C.c_double, u64, u64, u64],
     "ah_lion": [u64, u64, u64, u64, C.POINTER(AhLion)], "ah_sgd": [u64, u64, u64, C.c_double, C.c_double],
     "ah_adafactor_2d": [u64, u64, u64, u64, i64, i64, C.POINTER(AhAdafactor)],
     "ah_adafactor_flat": [u64, u64, u64, u64, C.POINTER(AhAdafactor)],

@@ -114,14 +114,19 @@ class Tape:
         self.entries = []
 
 
+def _to_i32(x: int) -> int:
+    x = int(x) & 0xFFFFFFFF
+    return x - (1 << 32) if x >> 31 else x
+
+
 class DropoutRng:
     """Counter-based mask parameters (ops.ts:25-82); the mask itself is generated on the device."""
 
     def __init__(self, seed: int):
-        self.seed, self.counter = seed, 0
+        self.seed, self.counter = _to_i32(seed), 0                    # `seed | 0`
 
     def reset(self, seed: int, counter: int = 0):
-        self.seed, self.counter = seed, counter
+        self.seed, self.counter = _to_i32(seed), _to_i32(counter)
 
     def nextMaskParams(self):
         r = {"seed": self.seed, "counter": self.counter}

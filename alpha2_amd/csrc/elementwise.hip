@@ -266,16 +266,22 @@ __global__ void k_residual_dropout_add(const float *__restrict__ r, const float 
   uint64_t tid = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x, stride = (uint64_t)gridDim.x * blockDim.x;
   for (uint64_t i = tid; i < n; i += stride) out[i] = r[i] + (m ? p[i] * m[i] : p[i]);
 }
-// u32-wrapping variant of the reference's splitmix-style hash (packages/helios/src/kernels/nn.ts:5600-5748)
-__global__ void k_dropout_mask(float *__restrict__ out, uint64_t n, uint32_t seed, uint32_t counter, float p, float keep) {
+// DropoutRng.hash of the reference's CPU path (packages/autograd/src/ops.ts:74-81), bit for bit: the first line is evaluated in
+// doubles, one rounding per operation (no fused multiply-add), and only then cut to 32 bits, so products past 2^53 have already
+// lost low bits exactly as a JS number does.  (The reference's own GPU kernel wraps in u32 instead,
+// packages/helios/src/kernels/nn.ts:5600-5748, and so differs from its CPU path for element indices above ~4.0 M.)
+// The sum is an integer-valued double below 2^63: the int64 conversion is exact and its low 32 bits are ToInt32.
+__global__ void k_dropout_mask(float *__restrict__ out, uint64_t n, int32_t seed, int32_t counter, double p, float keep) {
+#pragma clang fp contract(off)
   uint64_t tid = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x, stride = (uint64_t)gridDim.x * blockDim.x;
+  const double base = (double)seed + (double)counter * 2654435761.0;
   for (uint64_t i = tid; i < n; i += stride) {
-    uint32_t h = seed + counter * 2654435761u + (uint32_t)i * 2246822519u;
+    double sum = base + (double)i * 2246822519.0;
+    uint32_t h = (uint32_t)(int64_t)sum;
     h = (h ^ (h >> 16)) * 0x85ebca6bu;
     h = (h ^ (h >> 13)) * 0xc2b2ae35u;
     h = h ^ (h >> 16);
-    float x = (float)((double)h / 4294967296.0);
-    out[i] = x > p ? keep : 0.f;
+    out[i] = ((double)h * (1.0 / 4294967296.0) > p) ? keep : 0.f;
   }
 }
 __global__ void k_masked_fill(const float *__restrict__ a, const float *__restrict__ mask, float *__restrict__ out,
@@ -491,13 +497,14 @@ int32_t ah_residual_dropout_add(ah_ptr residual, ah_ptr projected, ah_ptr mask, 
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
-int32_t ah_dropout_mask(ah_ptr out, uint64_t n, int32_t seed, int32_t counter, float p) {
+int32_t ah_dropout_mask(ah_ptr out, uint64_t n, int32_t seed, int32_t counter, double p) {
   AH_REQUIRE_READY();
   if (n == 0) return AH_OK;
   AH_ARG(out != 0, "ah_dropout_mask: null out");
-  AH_ARG(p >= 0.f && p < 1.f, "ah_dropout_mask: p must be in [0,1)");
-  hipLaunchKernelGGL(k_dropout_mask, dim3(grid_for(n)), dim3(TPB), 0, stream(), dp<float>(out), n, (uint32_t)seed,
-                     (uint32_t)counter, p, 1.0f / (1.0f - p));
+  AH_ARG(p >= 0.0 && p < 1.0, "ah_dropout_mask: p must be in [0,1)");
+  AH_ARG(n <= (1ull << 32), "ah_dropout_mask: at most 2^32 elements (the hash sum must stay below 2^63)");
+  hipLaunchKernelGGL(k_dropout_mask, dim3(grid_for(n)), dim3(TPB), 0, stream(), dp<float>(out), n, seed, counter, p,
+                     (float)(1.0 / (1.0 - p)));
   AH_LAUNCH_CHECK();
   return AH_OK;
 }

@@ -23,6 +23,9 @@ __global__ void k_adamw(float *__restrict__ p, const float *__restrict__ g, floa
                         uint16_t *__restrict__ shadow, int vec) {
   if (dev_h) { float wd = h.weight_decay; h = *dev_h; h.weight_decay = wd; }   // weight decay stays per tensor
   float gs = h.grad_scale * (dev_scale ? dev_scale[0] : 1.0f);
+  // A gradient scale that is not finite means "skip this step" (ah_step_guard writes NaN for a non-finite loss or gradient
+  // norm, as the reference trainer skips the optimizer call, trainer.ts:1248-1262,1495-1522): p, m, v and the shadow stay.
+  if (!(fabsf(gs) <= 3.4028234e38f)) return;
   uint64_t tid = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x, stride = (uint64_t)gridDim.x * blockDim.x;
   uint64_t start = 0;
   if (vec) {
@@ -60,6 +63,29 @@ __global__ void k_clip_coef(const float *__restrict__ sumsq, float grad_scale, f
     out[0] = (clip > 0.f && norm > clip) ? clip / norm : 1.0f;
     out[1] = norm;
   }
+}
+
+// One thread: the clip coefficient of ah_clip_coef plus the decisions the reference trainer takes on the host between backward
+// and the optimizer call.  state (doubles): [0] beta1^t, [1] beta2^t, [2] steps skipped so far.
+__global__ void k_step_guard(const float *__restrict__ sumsq, const float *__restrict__ loss, float grad_scale, float clip,
+                             double beta1, double beta2, double *__restrict__ state, AhAdamW *__restrict__ hyper,
+                             float *__restrict__ out) {
+  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+  float norm = sqrtf(sumsq[0]) * fabsf(grad_scale);
+  bool ok = (fabsf(norm) <= 3.4028234e38f) && (!loss || fabsf(loss[0]) <= 3.4028234e38f);
+  out[1] = norm;
+  if (!ok) {
+    out[0] = __int_as_float(0x7fc00000);
+    out[2] = 1.0f;
+    state[2] += 1.0;
+    return;
+  }
+  out[0] = (clip > 0.f && norm > clip) ? clip / norm : 1.0f;
+  out[2] = 0.0f;
+  state[0] *= beta1;                       // running products of the betas advance with applied steps only (optimizers.ts:107-115)
+  state[1] *= beta2;
+  hyper->bc1 = (float)(1.0 - state[0]);
+  hyper->bc2 = (float)(1.0 - state[1]);
 }
 
 // ---- Lion, SGD, Adafactor: the reference's host loops (double arithmetic, one rounding per Float32Array store) ----
@@ -264,6 +290,17 @@ int32_t ah_clip_coef(ah_ptr sumsq, float grad_scale, float clip, ah_ptr out2) {
   AH_REQUIRE_READY();
   AH_ARG(sumsq && out2, "ah_clip_coef: null operand");
   hipLaunchKernelGGL(k_clip_coef, dim3(1), dim3(64), 0, stream(), dp<const float>(sumsq), grad_scale, clip, dp<float>(out2));
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+
+int32_t ah_step_guard(ah_ptr sumsq, ah_ptr loss, float grad_scale, float clip, double beta1, double beta2, ah_ptr state_f64x3,
+                      ah_ptr dev_hyper, ah_ptr out3) {
+  AH_REQUIRE_READY();
+  AH_ARG(sumsq && state_f64x3 && dev_hyper && out3, "ah_step_guard: null operand");
+  AH_ARG((state_f64x3 & 7u) == 0, "ah_step_guard: state must be 8-byte aligned");
+  hipLaunchKernelGGL(k_step_guard, dim3(1), dim3(64), 0, stream(), dp<const float>(sumsq), dp<const float>(loss), grad_scale, clip,
+                     beta1, beta2, dp<double>(state_f64x3), dp<AhAdamW>(dev_hyper), dp<float>(out3));
   AH_LAUNCH_CHECK();
   return AH_OK;
 }

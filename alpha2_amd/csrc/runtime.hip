@@ -76,9 +76,9 @@ int32_t hip_fail(hipError_t e, const char *what) {
 }
 void *scratch(size_t bytes) {
   if (bytes <= g.scratch_bytes) return g.scratch;
-  // Growing scratch is only legal outside capture (addresses inside a graph must stay put); ah_init
-  // sizes it for every reduction this library launches, so this branch is a safety net.
-  if (g.capturing) return nullptr;
+  // Growing scratch is only legal while no graph exists or is being captured (a graph replays into the addresses it
+  // was captured with); ah_init sizes it for every reduction this library launches, so this branch is a safety net.
+  if (g.capturing || !g.graphs.empty()) return nullptr;
   (void)hipStreamSynchronize(g.stream);
   if (g.scratch) (void)hipFree(g.scratch);
   g.scratch = nullptr; g.scratch_bytes = 0;

@@ -41,6 +41,7 @@ class StepStats:
     gradNorm: float
     clipCoef: float
     lr: float
+    skipped: bool = False         # loss or gradient norm was not finite: parameters and moments left as they were
 
 
 class FusedTrainer:
@@ -61,7 +62,6 @@ class FusedTrainer:
         self._timed = None
         self._snap = None
         self.stepIdx = 0
-        self._b1p = self._b2p = 1.0
 
         # ---- parameters: reference initialisation order (gpt.ts:73-151), then packed [decayed | not decayed]
         if params is None:
@@ -116,12 +116,15 @@ class FusedTrainer:
         self.dh = [a(BT * Fd * 2) for _ in range(self.L)]
         self.dqkv = [a(BT * 3 * Cc * 2) for _ in range(self.L)]
         self.dxb0 = a(BT * Cc * 2)                # grad of the embedding output in bf16 (written by the last LayerNorm backward, unused)
-        self.loss, self.sumsq, self.clip = a(4), a(4), a(8)
+        self.loss, self.sumsq, self.clip = a(4), a(4), a(16)         # clip: coefficient (NaN = skip), norm, skipped flag
         self.loss_micro = a(4)
         self.hyper = a(ffi.C.sizeof(ffi.AhAdamW))
+        self.guard = a(24)                                           # device doubles: beta1^t, beta2^t, steps skipped
+        self._write_guard_state()
         self.loss_hist_cap = 4096
-        self.loss_hist, self.norm_hist = a(self.loss_hist_cap * 4), a(self.loss_hist_cap * 8)
+        self.loss_hist, self.norm_hist = a(self.loss_hist_cap * 4), a(self.loss_hist_cap * 16)
         self._batches: List[Tuple[int, int]] = []
+        self._have_batch = False
         # partial column sums of every LayerNorm backward (dw, db), reduced by ONE launch at the end of backward
         part_bytes = int(self.lib.ah_layernorm_bwd_partials_bytes(BT, Cc))
         assert part_bytes > 0
@@ -275,7 +278,8 @@ class FusedTrainer:
         lib, tc = self.lib, self.tc
         split = self.off["_split"]
         check(lib.ah_sum_sq(self.G, self.nparam, self.sumsq))               # arena padding is zero and stays zero
-        check(lib.ah_clip_coef(self.sumsq, 1.0 / self.accum, tc.gradClip, self.clip))
+        # clip coefficient, non-finite guard and the bias corrections, all on the device (trainer.ts:1248-1262,1495-1522,1650-1656)
+        check(lib.ah_step_guard(self.sumsq, self.loss, 1.0 / self.accum, tc.gradClip, tc.beta1, tc.beta2, self.guard, self.hyper, self.clip))
         h = ffi.AhAdamW(tc.lr, tc.beta1, tc.beta2, tc.eps, tc.weightDecay, 1.0, 1.0, 1.0 / self.accum)
         if split > 0:
             check(lib.ah_adamw(self.P, self.G, self.M, self.Vm, split, C.byref(h), self.hyper, self.clip, self.Pb))
@@ -290,21 +294,34 @@ class FusedTrainer:
             self._forward_backward(m == 0, m)
         self._optimizer()
 
-    def set_batch(self, inputs: TensorData, targets: TensorData):
-        """Make one [B, T] token batch resident; step() then trains on it until another is set."""
-        self.add_batch(inputs, targets)
-        self._use_batch(len(self._batches) - 1)
-
-    def add_batch(self, inputs: TensorData, targets: TensorData) -> int:
+    def _upload_batch(self, inputs: TensorData, targets: TensorData, ti: int, tt: int):
         n = self.BT * 4
-        ti, tt = self._alloc(n), self._alloc(n)
         a, b = np.ascontiguousarray(inputs.data, dtype=np.int32), np.ascontiguousarray(targets.data, dtype=np.int32)
         if a.size != self.BT or b.size != self.BT:
             raise ValueError(f"batch must be [{self.batch}, {self.T}]")
         check(self.lib.ah_upload(ti, a.ctypes.data_as(C.c_void_p), n))
         check(self.lib.ah_upload(tt, b.ctypes.data_as(C.c_void_p), n))
+
+    def set_batch(self, inputs: TensorData, targets: TensorData, micro: int = 0):
+        """Upload one [B, T] token batch straight into the resident slot of micro-step `micro` (nothing is retained: a loop
+        that feeds a fresh batch every step allocates nothing); step() trains on the resident slots until they change."""
+        self._upload_batch(inputs, targets, self.toks[micro], self.tgts[micro])
+        self._have_batch = True
+
+    def add_batch(self, inputs: TensorData, targets: TensorData) -> int:
+        """Store a batch on the device for later steps (step(batch_index)); stored batches live until drop_batches()."""
+        n = self.BT * 4
+        ti, tt = self._alloc(n), self._alloc(n)
+        self._upload_batch(inputs, targets, ti, tt)
         self._batches.append((ti, tt))
         return len(self._batches) - 1
+
+    def drop_batches(self):
+        for pair in self._batches:
+            for b in pair:
+                check(self.lib.ah_free(b))
+                self._bufs.remove(b)
+        self._batches = []
 
     def _use_batch(self, i, micro: int = 0):
         """Copy stored batch i into the resident slot of micro-step `micro` (a sequence fills slots 0, 1, ...)."""
@@ -317,14 +334,21 @@ class FusedTrainer:
         ti, tt = self._batches[i]
         check(self.lib.ah_copy(self.toks[micro], ti, self.BT * 4))
         check(self.lib.ah_copy(self.tgts[micro], tt, self.BT * 4))
+        self._have_batch = True
+
+    def _write_guard_state(self, b1p: float = 1.0, b2p: float = 1.0, skipped: float = 0.0):
+        st = (C.c_double * 3)(b1p, b2p, skipped)
+        check(self.lib.ah_upload(self.guard, st, 24))
+        tc = self.tc
+        h = ffi.AhAdamW(tc.lr, tc.beta1, tc.beta2, tc.eps, tc.weightDecay, 1 - b1p, 1 - b2p, 1.0 / self.accum)
+        check(self.lib.ah_upload(self.hyper, C.byref(h), C.sizeof(h)))
 
     def _write_hyper(self) -> float:
-        tc = self.tc
-        lr = lrAt(tc, self.stepIdx)
-        self._b1p *= tc.beta1
-        self._b2p *= tc.beta2
-        h = ffi.AhAdamW(lr, tc.beta1, tc.beta2, tc.eps, tc.weightDecay, 1 - self._b1p, 1 - self._b2p, 1.0 / self.accum)
-        check(self.lib.ah_upload(self.hyper, C.byref(h), C.sizeof(h)))
+        """The learning rate of this step: the first field of the device AhAdamW.  Its bias corrections are kept by
+        ah_step_guard on the device, which advances them on applied steps only."""
+        lr = lrAt(self.tc, self.stepIdx)
+        v = C.c_float(lr)
+        check(self.lib.ah_upload(self.hyper, C.byref(v), 4))
         return lr
 
     def step(self, batch_index=None) -> int:
@@ -333,7 +357,7 @@ class FusedTrainer:
         stored batches (micro-steps run in that order); None keeps the resident ones."""
         if batch_index is not None:
             self._use_batch(batch_index)
-        elif not self._batches:
+        elif not self._have_batch:
             raise RuntimeError("no batch set")
         self._write_hyper()
         if self.use_graph:
@@ -354,7 +378,7 @@ class FusedTrainer:
             self._whole_step()
         i = self.stepIdx % self.loss_hist_cap
         check(self.lib.ah_copy(self.loss_hist + i * 4, self.loss, 4))
-        check(self.lib.ah_copy(self.norm_hist + i * 8, self.clip, 8))
+        check(self.lib.ah_copy(self.norm_hist + i * 16, self.clip, 16))
         self.stepIdx += 1
         return self.stepIdx - 1
 
@@ -363,6 +387,8 @@ class FusedTrainer:
         check(self.lib.ah_copy(self.P, self._snap[0], self.nparam * 4))
         check(self.lib.ah_copy(self.M, self._snap[1], self.nparam * 4))
         check(self.lib.ah_copy(self.Vm, self._snap[2], self.nparam * 4))
+        check(self.lib.ah_copy(self.guard, self._snap[3], 24))
+        check(self.lib.ah_copy(self.hyper, self._snap[3] + 32, C.sizeof(ffi.AhAdamW)))
         check(self.lib.ah_cast(self.P, F32, self.Pb, BF16, self.nparam))
         for s in self._snap:
             check(self.lib.ah_free(s))
@@ -371,20 +397,22 @@ class FusedTrainer:
 
     def prepare(self):
         """Snapshot state ahead of the warm-up run inside the first step()."""
-        self._snap = [self._alloc(self.nparam * 4) for _ in range(3)]
+        self._snap = [self._alloc(self.nparam * 4) for _ in range(3)] + [self._alloc(32 + C.sizeof(ffi.AhAdamW))]
         for dst, src in zip(self._snap, (self.P, self.M, self.Vm)):
             check(self.lib.ah_copy(dst, src, self.nparam * 4))
+        check(self.lib.ah_copy(self._snap[3], self.guard, 24))                     # running beta powers, skip count
+        check(self.lib.ah_copy(self._snap[3] + 32, self.hyper, C.sizeof(ffi.AhAdamW)))
 
     def history(self, first: int, count: int) -> List[StepStats]:
         """Blocks; loss, gradient norm and clip coefficient of steps [first, first+count)."""
         self.B.syncGpu()
         out = []
-        lo, nm = np.empty(self.loss_hist_cap, np.float32), np.empty(self.loss_hist_cap * 2, np.float32)
+        lo, nm = np.empty(self.loss_hist_cap, np.float32), np.empty(self.loss_hist_cap * 4, np.float32)
         check(self.lib.ah_download(lo.ctypes.data_as(C.c_void_p), self.loss_hist, lo.nbytes))
         check(self.lib.ah_download(nm.ctypes.data_as(C.c_void_p), self.norm_hist, nm.nbytes))
         for s in range(first, first + count):
             i = s % self.loss_hist_cap
-            out.append(StepStats(float(lo[i]), float(nm[2 * i + 1]), float(nm[2 * i]), lrAt(self.tc, s)))
+            out.append(StepStats(float(lo[i]), float(nm[4 * i + 1]), float(nm[4 * i]), lrAt(self.tc, s), bool(nm[4 * i + 2] != 0)))
         return out
 
     def timed_step(self) -> list:
@@ -471,7 +499,7 @@ class FusedTrainer:
                 put(self.M if key.endswith(".m") else self.Vm, key[:-2], td.data)
         check(self.lib.ah_cast(self.P, F32, self.Pb, BF16, self.nparam))
         self.stepIdx = int(st["optimizerState"].get("step") or st.get("step") or 0)
-        self._b1p, self._b2p = self.tc.beta1 ** self.stepIdx, self.tc.beta2 ** self.stepIdx      # optimizers.ts:214-215
+        self._write_guard_state(self.tc.beta1 ** self.stepIdx, self.tc.beta2 ** self.stepIdx)   # optimizers.ts:214-215
         return st
 
     def close(self):

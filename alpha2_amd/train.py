@@ -199,6 +199,15 @@ class DataLoader:
             starts = [int(math.floor(self.rng.next() * maxStart)) for _ in range(Bt)]
         inputs, targets = self._ring[self._ringIdx]
         self._ringIdx = (self._ringIdx + 1) % len(self._ring)
+        for t in (inputs, targets):
+            # The trainer releases the device copy of every batch it has consumed (trainer.ts:1267-1272); the reference's
+            # ring holds host arrays, so only that copy goes.  Here the ring IS the device copy: a released slot gets a
+            # fresh buffer before it is written again.
+            B_ = self.B
+            if t._buf is None:
+                fresh = B_._new(t.shape, "i32")
+                t._buf, t._off, t._dev_valid, t._backend = fresh._buf, 0, True, B_
+                fresh._buf = None
         st = TensorData((Bt,), "f64", np.asarray(starts, dtype=np.int64).view(np.float64))     # 8-byte slots holding the int64 starts
         B = self.B
         check(B.lib.ah_token_windows(B._ptr(self._corpus), N, B._ptr(st), Bt, T, B._ptr(inputs), B._ptr(targets)))

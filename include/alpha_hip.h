@@ -132,9 +132,10 @@ int32_t ah_channel_act_bwd(ah_ptr x, const ah_ptr *coefs, int32_t mask, ah_ptr g
                            int64_t rows, int64_t cols);
 /* Backend.residualDropoutAdd: out = residual + projected*mask (interfaces.ts:110; mask may be 0 = no dropout) */
 int32_t ah_residual_dropout_add(ah_ptr residual, ah_ptr projected, ah_ptr mask, ah_ptr out, uint64_t n);
-/* Backend.dropoutMask: u32-wrapping splitmix hash of (seed, counter, i) > p ? 1/(1-p) : 0
- * (interfaces.ts:125; packages/helios/src/kernels/nn.ts:5600-5748) */
-int32_t ah_dropout_mask(ah_ptr out, uint64_t n, int32_t seed, int32_t counter, float p);
+/* Backend.dropoutMask (interfaces.ts:125): out[i] = hash(seed, counter, i) / 2^32 > p ? (float)(1/(1-p)) : 0 with the hash of the
+ * reference's CPU path, DropoutRng.hash (packages/autograd/src/ops.ts:74-81), reproduced bit for bit for every index: its
+ * first line is evaluated in doubles before the cut to 32 bits.  n <= 2^32. */
+int32_t ah_dropout_mask(ah_ptr out, uint64_t n, int32_t seed, int32_t counter, double p);
 /* Backend.maskedFill with the mask tiled by i % mask_n (cpu_ref.ts:891-911) */
 int32_t ah_masked_fill(ah_ptr a, ah_ptr mask, ah_ptr out, uint64_t n, uint64_t mask_n, float value);
 /* Backend.causalMask (cpu_ref.ts:880-889) */
@@ -302,12 +303,22 @@ typedef struct {
  * clip coefficient computed by ah_clip_coef never visits the host.  `dev_hyper` (0 or a device AhAdamW)
  * overrides `h` with values read on the device: a captured graph then follows per-step lr / bias
  * corrections written by ah_upload between launches.  `bf16_shadow` (0 or bf16[n]) receives the updated
- * parameters rounded to bf16 for the next step's MFMA operands. */
+ * parameters rounded to bf16 for the next step's MFMA operands.  When the effective gradient scale
+ * (grad_scale x dev_scale[0]) is not finite the call changes nothing (see ah_step_guard). */
 int32_t ah_adamw(ah_ptr p, ah_ptr g, ah_ptr m, ah_ptr v, uint64_t n, const AhAdamW *h, ah_ptr dev_hyper,
                  ah_ptr dev_scale, ah_ptr bf16_shadow);
 /* out[0] = clip / (sqrt(sumsq[0]) * |grad_scale|) if that norm exceeds clip, else 1  (trainer.ts:1650-1656);
  * out[1] = the norm itself. */
 int32_t ah_clip_coef(ah_ptr sumsq, float grad_scale, float clip, ah_ptr out2);
+/* The same for a step that never visits the host, together with what the reference trainer decides there between backward and
+ * the optimizer call: a loss (0 = not checked) or gradient norm that is not finite skips the step (trainer.ts:1248-1262,
+ * 1495-1522).  out[0] = clip coefficient, or NaN to skip -- ah_adamw leaves p, m, v and the shadow untouched when its effective
+ * gradient scale is not finite; out[1] = the norm; out[2] = 1 if skipped else 0.  state = 3 doubles on the device
+ * {beta1^t, beta2^t, steps skipped}: on an applied step the powers advance and bc1 = 1 - beta1^t, bc2 = 1 - beta2^t are written
+ * into the device AhAdamW `dev_hyper` (optimizers.ts:107-115 advances them only when the optimizer runs); on a skipped step
+ * nothing but the skip count changes. */
+int32_t ah_step_guard(ah_ptr sumsq, ah_ptr loss, float grad_scale, float clip, double beta1, double beta2, ah_ptr state_f64x3,
+                      ah_ptr dev_hyper, ah_ptr out3);
 
 /* ---- the other optimizers of the reference's registry (optimizers.ts:596-603).  The reference runs them as host loops
  *      over Float32Arrays, i.e. in double precision with one rounding per store; the kernels compute in double the

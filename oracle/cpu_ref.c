@@ -15,8 +15,9 @@
  *   - orc_rng_*: integer stream pinned by an independent Python big-int restatement
  *     (bit-exact); the reference holds no golden stream -> "parity unpinned" against a
  *     reference run for the exact values of nextGauss (libm last-ulp).
- *   - orc_dropout_mask: restates the f64-multiply-then-|0 hash; unused at dropout 0
- *     -> "parity unpinned".
+ *   - orc_dropout_mask: restates the f64-multiply-then-|0 hash; pinned by an independent
+ *     Python restatement (doubles + big ints, every index range incl. products past 2^53)
+ *     and by the published MurmurHash3 fmix32 known answers for its mixing rounds.
  */
 #include <math.h>
 #include <stdint.h>
@@ -508,9 +509,11 @@ static int32_t js_to_int32(double d) {
   return (int32_t)(uint32_t)m;
 }
 static uint32_t js_imul(uint32_t a, uint32_t b) { return a * b; }
-void orc_dropout_mask(int32_t seed, int32_t counter, double p, float *mask, int64_t n) {
+/* mask[i - lo] for element indices lo <= i < hi */
+void orc_dropout_mask(int32_t seed, int32_t counter, double p, float *mask, int64_t lo, int64_t hi) {
   double scale = 1 / (1 - p);
-  for (int64_t i = 0; i < n; i++) {
+  mask -= lo;
+  for (int64_t i = lo; i < hi; i++) {
     double sum = (double)seed + (double)counter * 2654435761.0 + (double)i * 2246822519.0;
     uint32_t h = (uint32_t)js_to_int32(sum);
     h = js_imul(h ^ (h >> 16), 0x85ebca6bu);

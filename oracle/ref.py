@@ -446,5 +446,12 @@ def adamw_step(p: TD, g: TD, m: np.ndarray, v: np.ndarray, lr, beta1, beta2, eps
 def dropout_mask(seed: int, counter: int, p: float, n: int) -> np.ndarray:
     """packages/autograd/src/ops.ts:41-51,74-81."""
     out = np.empty(n, dtype=np.float32)
-    lib().orc_dropout_mask(C.c_int32(_to_i32(seed)), C.c_int32(_to_i32(counter)), _d(p), _fp(out), _n(n))
+    lib().orc_dropout_mask(C.c_int32(_to_i32(seed)), C.c_int32(_to_i32(counter)), _d(p), _fp(out), _n(0), _n(n))
+    return out
+
+
+def dropout_mask_range(seed: int, counter: int, p: float, lo: int, hi: int) -> np.ndarray:
+    """Elements [lo, hi) of the mask (the hash depends on the element index only, so a window needs no prefix)."""
+    out = np.empty(hi - lo, dtype=np.float32)
+    lib().orc_dropout_mask(C.c_int32(_to_i32(seed)), C.c_int32(_to_i32(counter)), _d(p), _fp(out), _n(lo), _n(hi))
     return out

@@ -77,10 +77,32 @@ class Tape:
         self.entries = []
 
 
+class DropoutRng:
+    """ops.ts:25-82: masks from a counter hash of (seed, counter, index); the counter advances once per mask."""
+
+    def __init__(self, seed: int):
+        self.seed, self.counter = ref._to_i32(seed), 0
+
+    def reset(self, seed: int, counter: int = 0):
+        self.seed, self.counter = ref._to_i32(seed), ref._to_i32(counter)
+
+    def nextMask(self, size: int, p: float) -> np.ndarray:
+        m = ref.dropout_mask(self.seed, self.counter, p, size)
+        self.counter += 1
+        return m
+
+    def saveCounter(self) -> int:
+        return self.counter
+
+    def restoreCounter(self, n: int):
+        self.counter = n
+
+
 @dataclass
 class Ctx:
     tape: Tape
     backend: CpuRef
+    dropoutRng: Optional[DropoutRng] = None
 
 
 def _record(ctx: Ctx, data: TD, inputs, backward) -> Variable:
@@ -322,10 +344,30 @@ def transpose(ctx, a, d0, d1):
     return _record(ctx, ctx.backend.transpose(a.data, d0, d1), [a], lambda g, B, n: [B.transpose(g, d0, d1)])
 
 
+def _cpu_mask(ctx, shape, p) -> TD:
+    """ops.ts:583-596, 635-647: cpu_ref has no dropoutMask, so the mask comes from DropoutRng.nextMask on the host.  (Without
+    a DropoutRng the reference draws Math.random(): not reproducible, not restated.)"""
+    if ctx.dropoutRng is None:
+        raise ValueError("dropout > 0 needs a DropoutRng")
+    return TD(tuple(shape), "f32", ctx.dropoutRng.nextMask(shape_size(shape), p))
+
+
+def dropout(ctx, a, p, training):
+    """ops.ts:574-613."""
+    if not training or p == 0:
+        return a
+    mask = _cpu_mask(ctx, a.data.shape, p)
+    return _record(ctx, ctx.backend.mul(a.data, mask), [a], lambda g, B, n: [B.mul(g, mask)])
+
+
 def residualDropoutAdd(ctx, residual, projected, p, training):
+    """ops.ts:615-685, the separate-ops branch (cpu_ref has no fused residualDropoutAdd)."""
     if not training or p == 0:
         return add(ctx, residual, projected)        # ops.ts:624
-    raise NotImplementedError("dropout > 0 is outside the measured configurations")
+    mask = _cpu_mask(ctx, projected.data.shape, p)
+    rs = residual.data.shape
+    out = ctx.backend.add(residual.data, ctx.backend.mul(projected.data, mask))
+    return _record(ctx, out, [residual, projected], lambda g, B, n: [_reduce_broadcast(B, g, rs), B.mul(g, mask)])
 
 
 # ---- gpt.ts -------------------------------------------------------------------------------------
@@ -341,6 +383,7 @@ class ModelConfig:
     ffnActivation: str = "gelu"
     ffnDim: Optional[int] = None
     softCap: Optional[float] = None
+    activationGraph: Optional[dict] = None
 
 
 def _init_weight(rng: SeededRng, shape, std) -> Variable:
@@ -399,6 +442,32 @@ def collectParamEntries(params: dict) -> List[Tuple[str, Variable]]:
     return e
 
 
+def _eval_activation_graph(ctx, x, node):
+    """gpt.ts:170-192: an expression tree whose leaves are the bases silu / relu / gelu / identity / square of the SAME
+    input (an unknown basis name evaluates as gelu) and whose inner nodes are scale-by-constant, add and mul."""
+    kind = node["type"]
+    if kind == "basis":
+        op = node["op"]
+        if op == "silu":
+            return silu(ctx, x)
+        if op == "relu":
+            return relu(ctx, x)
+        if op == "identity":
+            return x
+        if op == "square":
+            return mul(ctx, x, x)
+        return gelu(ctx, x)
+    if kind == "scale":
+        return scale(ctx, _eval_activation_graph(ctx, x, node["child"]), node["factor"])
+    lhs = _eval_activation_graph(ctx, x, node["left"])
+    rhs = _eval_activation_graph(ctx, x, node["right"])
+    if kind == "add":
+        return add(ctx, lhs, rhs)
+    if kind == "mul":
+        return mul(ctx, lhs, rhs)
+    raise ValueError(f"activation graph node {kind!r}")
+
+
 def _transformer_block(ctx, x, layer, cfg: ModelConfig, Bt, T, mask: TD, training):
     """gpt.ts:220-333, the branch taken when backend.flashAttention is absent (cpu_ref)."""
     H, Cc = cfg.nHead, cfg.nEmbd
@@ -419,7 +488,7 @@ def _transformer_block(ctx, x, layer, cfg: ModelConfig, Bt, T, mask: TD, trainin
     masked = Variable(ctx.backend.maskedFill(scores.data, mask, -1e9), True)
     ctx.tape.record(masked, [scores], lambda g, B, n: [B.maskedFill(g, mask, 0)])
     att = softmax(ctx, masked, -1)
-    out = matmul(ctx, att, vH)           # dropout p=0 is the identity (ops.ts:574)
+    out = matmul(ctx, dropout(ctx, att, cfg.dropout, training), vH)
     concat = reshape(ctx, transpose(ctx, out, 1, 2), [Bt * T, Cc])
     proj = reshape(ctx, matmulTransposed(ctx, concat, layer["attn"]["wo"]), [Bt, T, Cc])
     x = residualDropoutAdd(ctx, x, proj, cfg.dropout, training)
@@ -428,7 +497,10 @@ def _transformer_block(ctx, x, layer, cfg: ModelConfig, Bt, T, mask: TD, trainin
     flat = reshape(ctx, ln2, [Bt * T, Cc])
     act = cfg.ffnActivation or "gelu"
     m = layer["mlp"]
-    if act == "swiglu":
+    if act == "composed" and cfg.activationGraph:            # gpt.ts:290-294
+        h = matmulTransposed(ctx, flat, m["fc1"])
+        mlpH = matmulTransposed(ctx, _eval_activation_graph(ctx, h, cfg.activationGraph), m["fc2"])
+    elif act == "swiglu":
         gate = matmulTransposed(ctx, flat, m["fc_gate"])
         up = matmulTransposed(ctx, flat, m["fc_up"])
         mlpH = matmulTransposed(ctx, siluMul(ctx, gate, up), m["fc_proj"])
@@ -455,9 +527,9 @@ def _transformer_block(ctx, x, layer, cfg: ModelConfig, Bt, T, mask: TD, trainin
 
 
 def gptForward(cfg: ModelConfig, params: dict, B: CpuRef, tape: Tape, tokens: TD, targets: Optional[TD] = None,
-               training: bool = False):
+               training: bool = False, dropoutRng: Optional[DropoutRng] = None):
     """gpt.ts:344-427."""
-    ctx = Ctx(tape, B)
+    ctx = Ctx(tape, B, dropoutRng)
     Bt, T = tokens.shape
     tok = embedding(ctx, params["wte"], tokens)
     pos = TD((Bt, T), "i32", np.tile(np.arange(T, dtype=np.int32), Bt))
@@ -786,6 +858,7 @@ class TrainConfig:
     gradClip: float = 1.0
     gradAccumSteps: int = 1
     optimizer: str = "adamw"
+    seed: int = 42                    # packages/core/src/types.ts:126
 
 
 def lr_at(tc: TrainConfig, step: int) -> float:
@@ -832,9 +905,11 @@ class Trainer:
             raise ValueError(f'Unknown optimizer: "{kind}"')
         self.tape = Tape()
         self.step_idx = 0
+        self.dropoutRng = DropoutRng(tc.seed)                        # trainer.ts:1106
 
-    def forward_backward(self, inputs: TD, targets: TD) -> float:
-        _, loss = gptForward(self.cfg, self.params, self.B, self.tape, inputs, targets, True)
+    def forward_backward(self, inputs: TD, targets: TD, micro: int = 0) -> float:
+        self.dropoutRng.reset(self.tc.seed + self.step_idx * 1000 + micro, 0)       # trainer.ts:1169,1202
+        _, loss = gptForward(self.cfg, self.params, self.B, self.tape, inputs, targets, True, self.dropoutRng)
         self.tape.backward(loss, self.B)
         val = float(loss.data.data[0])
         self.tape.clear()
@@ -850,8 +925,8 @@ class Trainer:
             loss_val = self.forward_backward(*batches[0])
         else:  # trainer.ts:1208-1223: f32 scale by 1/accum then f32 add
             acc = None
-            for inp, tgt in batches:
-                lv = TD((), "f32", np.array([self.forward_backward(inp, tgt)], dtype=np.float32))
+            for micro, (inp, tgt) in enumerate(batches):
+                lv = TD((), "f32", np.array([self.forward_backward(inp, tgt, micro)], dtype=np.float32))
                 s = self.B.scale(lv, 1 / accum)
                 acc = s if acc is None else self.B.add(acc, s)
             loss_val = float(acc.data[0])

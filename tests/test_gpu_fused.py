@@ -141,3 +141,58 @@ def test_fused_checkpoint_resume(B, tmp_path):
     assert np.array_equal(dict(g.entries)["layer.1.mlp.fc1"].data.data, at_save)       # bit-for-bit what was saved
     assert not np.array_equal(a.param("layer.1.mlp.fc1"), at_save)                     # (training has moved on since)
     a.close(), b.close()
+
+
+def test_fused_step_with_a_non_finite_gradient_is_skipped_on_the_device(B):
+    """The reference trainer skips the optimizer call when the loss or the gradient norm is not finite
+    (trainer.ts:1248-1262,1495-1522).  The fast path takes that decision on the device: parameters, moments, the bf16
+    shadow and the running bias corrections stay as they were, the skip shows in history(), and the next clean step equals
+    the step a run without the incident takes."""
+    import ctypes as C
+    from alpha2_amd.train import syntheticBatch
+    tc = dict(iters=6)
+    a, b = _make(B, tc, use_graph=False, seed=8), _make(B, tc, use_graph=False, seed=8)
+    for t in (a, b):
+        t.set_batch(*syntheticBatch(900, 4, 64, 256))
+        t.step()
+    before = {n: a.param(n) for n in ("wte", "layer.0.mlp.fc1", "lnF.weight")}
+    m_before = a.stateDict()["buffers"]["layer.0.mlp.fc1.m"].data.copy()
+    # poison: run forward/backward, then put an Inf into the gradient arena before the optimizer part
+    a._write_hyper()
+    a._forward_backward(True, 0)
+    inf = np.array([np.inf], np.float32)
+    ffi_check = __import__("alpha2_amd._ffi", fromlist=["check"]).check
+    ffi_check(B.lib.ah_upload(a.g("layer.0.mlp.fc1") + 40, inf.ctypes.data_as(C.c_void_p), 4))
+    a._optimizer()
+    i = a.stepIdx % a.loss_hist_cap
+    ffi_check(B.lib.ah_copy(a.loss_hist + i * 4, a.loss, 4))
+    ffi_check(B.lib.ah_copy(a.norm_hist + i * 16, a.clip, 16))
+    a.stepIdx += 1
+    h = a.history(1, 1)[0]
+    assert h.skipped and not math.isfinite(h.gradNorm) and math.isnan(h.clipCoef)
+    for n, v in before.items():
+        assert np.array_equal(a.param(n), v), n
+    assert np.array_equal(a.stateDict()["buffers"]["layer.0.mlp.fc1.m"].data, m_before)
+    # the next clean step of `a` (schedule index 2) against `b` stepping the same batch at the same schedule index
+    b.stepIdx = 2
+    a.step(), b.step()
+    ha, hb = a.history(2, 1)[0], b.history(2, 1)[0]
+    assert not ha.skipped and abs(ha.loss - hb.loss) <= 1e-6 * abs(hb.loss)
+    for n in before:
+        assert np.allclose(a.param(n), b.param(n), rtol=0, atol=1e-7), n          # same bias corrections: beta powers did not advance
+    a.close(), b.close()
+
+
+def test_set_batch_reuses_the_resident_slot(B):
+    from alpha2_amd.train import syntheticBatch
+    ft = _make(B, dict(iters=4), use_graph=False, seed=1)
+    ft.set_batch(*syntheticBatch(1, 4, 64, 256))
+    live = B.gpuMemStats()["liveAllocs"]
+    for s in range(5):
+        ft.set_batch(*syntheticBatch(2 + s, 4, 64, 256))
+    assert B.gpuMemStats()["liveAllocs"] == live
+    i = ft.add_batch(*syntheticBatch(9, 4, 64, 256))
+    assert B.gpuMemStats()["liveAllocs"] == live + 2
+    ft.drop_batches()
+    assert B.gpuMemStats()["liveAllocs"] == live and i == 0
+    ft.close()

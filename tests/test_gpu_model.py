@@ -52,12 +52,15 @@ def test_forward_backward_grads_match_oracle(B, attention):
         assert_close(v.grad.data, ov.grad.data, what=f"grad {n}")
 
 
-@pytest.mark.parametrize("act", ["swiglu", "universal", "kan_spline", "silu", "relu"])
+@pytest.mark.parametrize("act", ["swiglu", "universal", "kan_spline", "silu", "relu", "composed"])
 def test_custom_activation_models_match_oracle(B, act):
     from alpha2_amd.autograd import Tape
     from alpha2_amd.model import gptForward
     from alpha2_amd.train import syntheticBatch
     cfg = dict(vocabSize=40, blockSize=16, nLayer=1, nEmbd=64, nHead=2, ffnActivation=act)
+    if act == "composed":           # the expression tree of the oracle's own pin (every node type and basis, an unknown basis name)
+        from tests.test_oracle_model import COMPOSED_GRAPH
+        cfg["activationGraph"] = COMPOSED_GRAPH
     dev, orc = _both(B, cfg, dict(iters=1), seed=5)
     rs = np.random.RandomState(1)
     for (n, v), (_, ov) in zip(dev.entries, orc.entries):           # generic gates / coefficients
@@ -196,6 +199,45 @@ def test_dataloader_batches_are_bit_exact(B, N, Bt, T, packed):
             px, pxo = held[-2]
             assert np.array_equal(px.data, pxo)
     assert dev.stepsPerEpoch == N // (Bt * T)
+
+
+@pytest.mark.parametrize("accum", [1, 2])
+def test_trainer_driven_by_the_dataloader_matches_oracle(B, accum):
+    """The training loop as the reference runs it: every micro-step takes loader.nextBatch(), and the trainer releases
+    the batch tensors it consumed (trainer.ts:1190,1267-1272), so each ring slot is written again after a release."""
+    from alpha2_amd.rng import SeededRng
+    from alpha2_amd.train import DataLoader
+    cfg = dict(vocabSize=96, blockSize=32, nLayer=2, nEmbd=64, nHead=2)
+    dev, orc = _both(B, cfg, dict(iters=6, gradAccumSteps=accum), seed=3)
+    tok = (np.arange(5000, dtype=np.int64) * 7919 % 96).astype(np.int32)
+    dl, odl = DataLoader(B, tok, SeededRng(8), 4, 32), rm.DataLoader(tok, ref.SeededRng(8), 4, 32)
+    for s in range(6):
+        r = dev.step([dl.nextBatch() for _ in range(accum)])
+        o = orc.step([odl.next_batch() for _ in range(accum)])
+        assert abs(r.loss - o.loss) <= 1e-3 * abs(o.loss), (s, r.loss, o.loss)
+        assert abs(r.gradNorm - o.gradNorm) <= 1e-3 * o.gradNorm, (s, r.gradNorm, o.gradNorm)
+
+
+def test_training_steps_with_dropout_match_oracle(B):
+    """dropout = 0.1: masks at the three sites of every layer (attention weights, both residual branches) come from the
+    reference's counter hash, re-seeded with seed + step * 1000 + microStep before every forward (trainer.ts:1169,1202;
+    ops.ts:25-82); the device masks are bit-equal to the CPU path's, so losses agree as tightly as without dropout."""
+    from alpha2_amd.train import syntheticBatch
+    cfg = dict(vocabSize=96, blockSize=32, nLayer=2, nEmbd=64, nHead=2, dropout=0.1)
+    dev, orc = _both(B, cfg, dict(iters=4, gradAccumSteps=2, seed=7), seed=2)
+    nodrop, _ = _both(B, dict(cfg, dropout=0.0), dict(iters=4, gradAccumSteps=2, seed=7), seed=2)
+    for s in range(4):
+        bs = [syntheticBatch(300 + 2 * s + m, 4, 32, 96) for m in range(2)]
+        obs = [rm.synthetic_batch(300 + 2 * s + m, 4, 32, 96) for m in range(2)]
+        r, o = dev.step(bs), orc.step(obs)
+        assert abs(r.loss - o.loss) <= 1e-3 * abs(o.loss), (s, r.loss, o.loss)
+        assert abs(r.gradNorm - o.gradNorm) <= 1e-3 * o.gradNorm, (s, r.gradNorm, o.gradNorm)
+        if s == 0:
+            r0 = nodrop.step([syntheticBatch(300 + m, 4, 32, 96) for m in range(2)])
+            assert abs(r0.loss - r.loss) > 1e-4 * abs(r.loss)                  # dropout really is on
+    for (n, v), (_, ov) in zip(dev.entries, orc.entries):
+        assert_close(v.data.data, ov.data.data, rel=1e-3, what=f"param {n} after 4 steps", outlier_frac=max(2e-3, 2.5 / v.data.size),
+                     outlier_abs=4 * 0.1 * 3e-4)
 
 
 def test_dataloader_rejects_a_corpus_not_longer_than_the_block(B):

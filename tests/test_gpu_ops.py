@@ -125,6 +125,23 @@ def test_elementwise_vs_oracle(B, n):
     assert_close(B.residualDropoutAdd(dev(B, x), dev(B, y), dev(B, g)).data, O.add(orc(x), O.mul(orc(y), orc(g))).data, what="rda")
 
 
+def test_dropout_mask_equals_the_cpu_path_for_every_index(B):
+    """Backend.dropoutMask against DropoutRng.nextMask of the reference's CPU path (packages/autograd/src/ops.ts:41-51,74-81),
+    bit for bit, over 6 M elements: past index 4 008 862 the product index * 2246822519 exceeds 2^53 and the double has lost
+    low bits before the cut to 32 bits, which the kernel reproduces (the reference's own GPU kernel does not)."""
+    n = 6_000_000
+    for seed, counter, p in ((42, 0, 0.1), (-7, 11, 0.5), (2 ** 31 - 1, 2 ** 21, 0.25), (42 + 3 * 1000 + 1, 2, 0.1)):
+        got = B.dropoutMask([n], seed, counter, p).data
+        want = ref.dropout_mask(seed, counter, p, n)
+        assert np.array_equal(got, want), (seed, counter, p, int((got != want).sum()))
+    from tests.util import py_dropout_mask
+    idx = list(range(0, 50)) + list(range(4_008_800, 4_008_900)) + list(range(n - 50, n))
+    assert np.array_equal(B.dropoutMask([n], 42, 0, 0.1).data[idx], py_dropout_mask(42, 0, 0.1, idx))
+    assert B.dropoutMask([0], 1, 0, 0.1).data.size == 0
+    with pytest.raises(Exception):
+        B.dropoutMask([4], 1, 0, 1.0)
+
+
 @pytest.mark.parametrize("rows,cols", [(1, 4), (37, 24), (130, 260), (1000, 512)])
 def test_channel_activation_mixtures_match_the_composed_ops(B, rows, cols):
     """channelAct / channelActBackward (one pass) against the oracle running the chain of ops the reference records for its
@@ -648,7 +665,8 @@ def test_gemm_layouts_epilogues_dtypes(B, in_bf16, out_bf16, M, N, K):
 
 
 def test_gemm_bf16_split_k_weight_gradient(B):
-    """dW = G^T X with a long token axis and few output tiles takes the split-K path (atomic f32 partial sums)."""
+    """dW = G^T X with a long token axis and few output tiles takes the split-K path (slices of the token axis into a
+    workspace, summed in a fixed order by a second kernel)."""
     from alpha2_amd import _ffi as ffi
     Kc, M, N = 4096, 256, 128
     g_, x = _bf16_round(rs.randn(Kc, M).astype(np.float32) * 0.1)[0], _bf16_round(rs.randn(Kc, N).astype(np.float32))[0]
@@ -811,23 +829,29 @@ def _gauss_bf16(shape, seed, std):
 
 
 @pytest.mark.parametrize("N", [768, 2304, 3072, 50304])
-def test_gemm_microbench_shapes_forward_and_both_backward(B, N):
+@pytest.mark.parametrize("in_dtype", ["bf16", "f32"])
+def test_gemm_microbench_shapes_forward_and_both_backward(B, N, in_dtype):
     """C = A B^T, dA = G B, dB = G^T A at M = 16384 (B*T), K = 768, N as in the GEMM microbenchmark; operands
-    N(0,1)*0.02 rounded to bf16, fp32 accumulate.  The full products are too large for the CPU oracle, so a sample of
-    output rows is read back and checked against float64 numpy products of the same operands."""
+    N(0,1)*0.02, as f32 (fp32 MFMA) and rounded to bf16 (bf16 MFMA, fp32 accumulate).  The full products are too large for
+    the CPU oracle, so a sample of output rows is read back and checked against float64 numpy products of the same operands."""
     import ctypes as C
     from alpha2_amd import _ffi as ffi
     M, K = 16384, 768
     lib = B.lib
+    idt = ffi.BF16 if in_dtype == "bf16" else ffi.F32
 
-    def bits_of(shape, seed):           # bf16 bit patterns of N(0,1)*0.02, and nothing else kept on the host
+    def bits_of(shape, seed):           # the operand as the device stores it, and nothing else kept on the host
         x = np.random.default_rng(seed).standard_normal(shape, dtype=np.float32)
         x *= np.float32(0.02)
+        if in_dtype == "f32":
+            return x
         u = x.view(np.uint32)
         u += np.uint32(0x7FFF) + ((u >> np.uint32(16)) & np.uint32(1))          # round to nearest even
         return (u >> np.uint32(16)).astype(np.uint16)
 
     def f64(bits):
+        if bits.dtype == np.float32:
+            return bits.astype(np.float64)
         return (bits.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
 
     def up(bits):
@@ -848,7 +872,7 @@ def test_gemm_microbench_shapes_forward_and_both_backward(B, N):
     out = C.c_uint64()
     ffi.check(lib.ah_alloc(max(M * N, N * K, M * K) * 4, C.byref(out)))
     run = lambda layout, pa_, pb_, m, n, k, lda, ldb: ffi.check(lib.ah_gemm(C.byref(
-        ffi.AhGemm(layout, ffi.BF16, ffi.F32, ffi.EPI_NONE, m, n, k, lda, ldb, n, 1, 0, 0, 0, pa_, pb_, out.value, 0))))
+        ffi.AhGemm(layout, idt, ffi.F32, ffi.EPI_NONE, m, n, k, lda, ldb, n, 1, 0, 0, 0, pa_, pb_, out.value, 0))))
     run(ffi.GEMM_NT, pa, pb, M, N, K, K, K)
     assert_close(rows_of(out.value, rows_m, N), f64(a[rows_m]) @ f64(b).T, rel=1e-4, what=f"C rows N={N}")
     run(ffi.GEMM_NN, pg, pb, M, K, N, N, K)                                   # dA = G [M,N] x B [N,K]

@@ -85,8 +85,26 @@ def test_init_order_and_std():
     assert "lmHead" not in rm.no_decay_names(2) and "wte" in rm.no_decay_names(2)
 
 
-def _torch_forward(cfg, P, tokens, targets, cap=30.0):
-    """The same network in PyTorch float64 (library ops; independent of the oracle's loops)."""
+# A composed activation (packages/model/src/gpt.ts:170-192) that uses every node type, every basis, a repeated sub-tree
+# and an unknown basis name (which the reference evaluates as gelu) ...
+COMPOSED_GRAPH = {"type": "add",
+                  "left": {"type": "scale", "factor": 0.5, "child": {"type": "mul", "left": {"type": "basis", "op": "silu"},
+                                                                     "right": {"type": "basis", "op": "square"}}},
+                  "right": {"type": "add",
+                            "left": {"type": "mul", "left": {"type": "basis", "op": "relu"}, "right": {"type": "basis", "op": "gelu"}},
+                            "right": {"type": "add", "left": {"type": "scale", "factor": -0.3, "child": {"type": "basis", "op": "identity"}},
+                                      "right": {"type": "scale", "factor": 0.25, "child": {"type": "basis", "op": "softsign"}}}}}
+
+
+def _composed_closed_form(h):
+    """... and the function it denotes, written out by hand."""
+    g = lambda t: F.gelu(t, approximate="tanh")
+    return 0.5 * (F.silu(h) * (h * h)) + (F.relu(h) * g(h) + (-0.3 * h + 0.25 * g(h)))
+
+
+def _torch_forward(cfg, P, tokens, targets, cap=30.0, masks=None):
+    """The same network in PyTorch float64 (library ops; independent of the oracle's loops).  `masks`: per layer the
+    dropout masks of the attention weights and of the two residual branches, in the order the model draws them."""
     Bt, T = tokens.shape
     H, Cc = cfg.nHead, cfg.nEmbd
     D = Cc // H
@@ -100,8 +118,12 @@ def _torch_forward(cfg, P, tokens, targets, cap=30.0):
         s = (q @ k.transpose(2, 3)) / math.sqrt(D)
         s = cap * torch.tanh(s / cap)
         s = s.masked_fill(mask, -1e9)
-        a = torch.softmax(s, -1) @ v
-        x = x + (a.transpose(1, 2).reshape(Bt * T, Cc) @ g("attn.wo").T).reshape(Bt, T, Cc)
+        w = torch.softmax(s, -1)
+        if masks is not None:
+            w = w * masks[i][0].reshape(w.shape)
+        a = w @ v
+        proj = (a.transpose(1, 2).reshape(Bt * T, Cc) @ g("attn.wo").T).reshape(Bt, T, Cc)
+        x = x + (proj * masks[i][1].reshape(proj.shape) if masks is not None else proj)
         h = F.layer_norm(x, (Cc,), g("ln2.weight"), g("ln2.bias"), 1e-5).reshape(Bt * T, Cc)
         act = cfg.ffnActivation
         if act == "swiglu":
@@ -117,18 +139,22 @@ def _torch_forward(cfg, P, tokens, targets, cap=30.0):
                 hh = F.relu(pre)
             elif act == "universal":
                 hh = F.silu(pre) * g("mlp.act_gate") + pre * g("mlp.act_skip")
+            elif act == "composed":
+                hh = _composed_closed_form(pre)
             else:
                 hh = (F.silu(pre) * g("mlp.kan_c0") + F.relu(pre) * g("mlp.kan_c1") + F.gelu(pre, approximate="tanh") * g("mlp.kan_c2")
                       + pre * g("mlp.kan_c3") + pre * pre * g("mlp.kan_c4"))
             m = hh @ g("mlp.fc2").T
-        x = x + m.reshape(Bt, T, Cc)
+        m = m.reshape(Bt, T, Cc)
+        x = x + (m * masks[i][2].reshape(m.shape) if masks is not None else m)
     x = F.layer_norm(x, (Cc,), P["lnF.weight"], P["lnF.bias"], 1e-5)
     logits = x.reshape(Bt * T, Cc) @ P["lmHead"].T
     return logits, F.cross_entropy(logits, targets.reshape(-1))
 
 
-def _check_model(act, seed):
-    cfg = rm.ModelConfig(vocabSize=29, blockSize=12, nLayer=2, nEmbd=16, nHead=4, ffnActivation=act)
+def _check_model(act, seed, dropout=0.0):
+    cfg = rm.ModelConfig(vocabSize=29, blockSize=12, nLayer=2, nEmbd=16, nHead=4, ffnActivation=act, dropout=dropout,
+                         activationGraph=COMPOSED_GRAPH if act == "composed" else None)
     Bm = ref.CpuRef()
     params = rm.initGPT(cfg, Bm, ref.SeededRng(seed))
     entries = rm.collectParamEntries(params)
@@ -137,11 +163,21 @@ def _check_model(act, seed):
         v.data.data += (rs.randn(v.data.data.size) * 0.05).astype(np.float32)
     inp, tgt = rm.synthetic_batch(seed + 1, 3, 12, 29)
     tape = rm.Tape()
-    logits, loss = rm.gptForward(cfg, params, Bm, tape, inp, tgt, True)
+    masks = None
+    drng = None
+    if dropout:
+        # DropoutRng (ops.ts:25-82): one mask per dropout site, the counter advancing by one each; per layer the sites are
+        # the attention weights [B, H, T, T], the attention branch [B, T, C], the MLP branch [B, T, C] (gpt.ts:276,281,332)
+        from tests.util import py_dropout_mask
+        drng = rm.DropoutRng(77)
+        sizes = [3 * 4 * 12 * 12, 3 * 12 * 16, 3 * 12 * 16]
+        masks = [[torch.tensor(py_dropout_mask(77, 3 * l + j, dropout, range(n)).astype(np.float64)) for j, n in enumerate(sizes)]
+                 for l in range(cfg.nLayer)]
+    logits, loss = rm.gptForward(cfg, params, Bm, tape, inp, tgt, True, drng)
     tape.backward(loss, Bm)
     P = {n: torch.tensor(v.data.data.astype(np.float64)).reshape(v.data.shape).requires_grad_() for n, v in entries}
     tl, tloss = _torch_forward(cfg, P, torch.tensor(inp.data.astype(np.int64)).reshape(3, 12),
-                               torch.tensor(tgt.data.astype(np.int64)).reshape(3, 12))
+                               torch.tensor(tgt.data.astype(np.int64)).reshape(3, 12), masks=masks)
     tloss.backward()
     assert abs(float(loss.data.data[0]) - tloss.item()) < 2e-6
     assert np.max(np.abs(logits.data.data - tl.detach().numpy().reshape(-1))) < 2e-6
@@ -158,6 +194,32 @@ def test_full_model_forward_backward_vs_torch_f64_gelu():
 def test_full_model_forward_backward_vs_torch_f64_custom_activations():
     for act in ("swiglu", "universal", "kan_spline", "silu", "relu"):
         _check_model(act, 3)
+
+
+def test_full_model_forward_backward_vs_torch_f64_composed_activation():
+    _check_model("composed", 4)
+
+
+def test_full_model_forward_backward_vs_torch_f64_with_dropout():
+    """Dropout 0.2 at the three sites of every layer, masks from the independently restated hash."""
+    _check_model("gelu", 6, dropout=0.2)
+
+
+def test_dropout_is_off_when_not_training_and_masks_follow_the_step_seed():
+    cfg = rm.ModelConfig(vocabSize=29, blockSize=12, nLayer=1, nEmbd=16, nHead=4, dropout=0.3)
+    Bm = ref.CpuRef()
+    params = rm.initGPT(cfg, Bm, ref.SeededRng(0))
+    inp, tgt = rm.synthetic_batch(1, 2, 12, 29)
+    ev = [rm.gptForward(cfg, params, Bm, rm.Tape(), inp, tgt, False, rm.DropoutRng(s))[1].data.data[0] for s in (1, 2)]
+    assert ev[0] == ev[1]                                                      # ops.ts:575,624: identity unless training
+    tr = [rm.gptForward(cfg, params, Bm, rm.Tape(), inp, tgt, True, rm.DropoutRng(s))[1].data.data[0] for s in (1, 1, 2)]
+    assert tr[0] == tr[1] and tr[0] != tr[2] and tr[0] != ev[0]
+    # trainer.ts:1169,1202: the stream is re-seeded with seed + step * 1000 + microStep before every forward
+    t = rm.Trainer(cfg, rm.TrainConfig(iters=3, seed=5), seed=0)
+    t.step([(inp, tgt), (inp, tgt)])
+    assert (t.dropoutRng.seed, t.dropoutRng.counter) == (5 + 0 * 1000 + 1, 3)
+    t.step([(inp, tgt), (inp, tgt)])
+    assert (t.dropoutRng.seed, t.dropoutRng.counter) == (5 + 1 * 1000 + 1, 3)
 
 
 def test_lr_schedule_closed_form():

@@ -305,3 +305,51 @@ def test_adamw_vs_torch_and_closed_form():
 def test_sum_sq_and_clip_identity():
     a = ref.f32(rs.randn(1000))
     assert abs(ref.sum_sq(a) - float(np.sum(a.data.astype(np.float64) ** 2))) < 1e-9
+
+
+# ---- DropoutRng.nextMask (packages/autograd/src/ops.ts:41-51,74-81) --------------------------------------------------------
+def test_dropout_hash_mixing_rounds_are_murmur3_fmix32():
+    """With counter = index = 0 the hash is the published MurmurHash3 32-bit finaliser of the seed; fmix32(0) = 0,
+    fmix32(1) = 0x514E28B7 and fmix32(2) = 0x30F4C306 are its known answers.  A mask value is hash / 2^32 > p."""
+    from tests.util import py_dropout_hash
+    assert [py_dropout_hash(s, 0, 0) for s in (0, 1, 2)] == [0, 0x514E28B7, 0x30F4C306]
+    for seed, want in ((0, 0), (1, 0x514E28B7), (2, 0x30F4C306)):
+        for p in (0.1, 0.3, 0.9):
+            m = ref.dropout_mask(seed, 0, p, 1)
+            assert m[0] == (np.float32(1 / (1 - p)) if want / 2 ** 32 > p else 0)
+
+
+def test_dropout_mask_equals_the_independent_restatement():
+    """Every branch of the first line: small sums (exact), negative seeds (ToInt32 of a negative number), sums past 2^32
+    (wrap) and index * 2246822519 past 2^53, where the double has already dropped low bits before the |0 (indices above
+    ~4.0 M: there the reference's own GPU kernel, which wraps in u32, gives different masks)."""
+    from tests.util import py_dropout_mask
+    idx = np.concatenate([np.arange(0, 3000), np.arange(4_000_000, 4_003_000), np.arange(4_009_000_000 // 1000, 4_009_000_000 // 1000 + 10),
+                          np.arange(2 ** 31 - 2000, 2 ** 31 - 1)])
+    for seed, counter, p in ((0, 0, 0.1), (42, 3, 0.1), (-7, 11, 0.5), (2 ** 31 - 1, 2 ** 21, 0.25), (42 + 17 * 1000 + 1, 5, 0.1)):
+        n = int(idx.max()) + 1
+        got = np.empty(len(idx), np.float32)
+        # the C oracle fills [0, n); evaluate it in windows around the probed indices instead of 2^31 elements
+        for lo, hi in ((0, 3000), (4_000_000, 4_003_000), (4_009_000, 4_009_010), (2 ** 31 - 2000, 2 ** 31 - 1)):
+            sel = (idx >= lo) & (idx < hi)
+            got[sel] = ref.dropout_mask_range(seed, counter, p, lo, hi)
+        assert np.array_equal(got, py_dropout_mask(seed, counter, p, idx)), (seed, counter, p)
+    m = ref.dropout_mask(42, 0, 0.1, 200_000)
+    assert set(np.unique(m)) == {np.float32(0), np.float32(1 / 0.9)}
+    assert abs((m == 0).mean() - 0.1) < 0.005                    # drop rate p
+    assert not np.array_equal(m, ref.dropout_mask(42, 1, 0.1, 200_000))       # the counter changes the mask
+
+
+def test_dropout_hash_differs_from_u32_wrapping_beyond_2_to_53():
+    """Documents the reference's CPU/GPU divergence: the u32-wrapping kernel (packages/helios/src/kernels/nn.ts:5600-5748)
+    equals the CPU hash while index * 2246822519 < 2^53 and not beyond."""
+    from tests.util import py_dropout_hash
+
+    def wrap(seed, counter, i):
+        h = (seed + counter * 2654435761 + i * 2246822519) & 0xFFFFFFFF
+        h = ((h ^ (h >> 16)) * 0x85EBCA6B) & 0xFFFFFFFF
+        h = ((h ^ (h >> 13)) * 0xC2B2AE35) & 0xFFFFFFFF
+        return h ^ (h >> 16)
+    limit = 2 ** 53 // 2246822519
+    assert all(py_dropout_hash(42, 3, i) == wrap(42, 3, i) for i in list(range(2000)) + list(range(limit - 2000, limit - 8)))
+    assert sum(py_dropout_hash(42, 3, i) != wrap(42, 3, i) for i in range(limit + 10, limit + 2010)) > 500
