@@ -99,7 +99,7 @@ SIGNATURES = {
     "ah_broadcast": [u64, u64, i32, p_i64, p_i64],
     "ah_sum_axis": [u64, u64, i64, i64, i64, i32], "ah_sum_all": [u64, u64, u64, i32],
     "ah_softmax": [u64, u64, i64, i64, i64, i32], "ah_argmax": [u64, u64, i64, i64, i64],
-    "ah_sum_sq": [u64, u64, u64], "ah_softmax_bwd": [u64, u64, u64, i64, i64],
+    "ah_sum_sq": [u64, u64, u64], "ah_sum_sq_static": [u64, u64, u64], "ah_softmax_bwd": [u64, u64, u64, i64, i64],
     "ah_embedding": [u64, u64, u64, i64, i64, i64, i32],
     "ah_embedding_tok_pos": [u64, u64, u64, u64, i64, i64, i64, i64],
     "ah_embedding_bwd": [u64, u64, u64, i64, i64, i64, i32],

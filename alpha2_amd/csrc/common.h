@@ -18,6 +18,8 @@ int         num_cus();
 // Scratch for two-stage reductions: a library-owned device buffer of at least `bytes` bytes that stays
 // valid until the next call that asks for scratch on the same stream (calls are stream-ordered).
 void       *scratch(size_t bytes);
+int         current_device();                     // the device ah_init was called with
+int32_t     static_partials_init(int device);     // reduce.hip: device address of its static scratch array (called by ah_init)
 
 #define AH_REQUIRE_READY() do { if (!ah::ready()) return ah::fail(AH_ERR_STATE, "%s: ah_init has not been called", __func__); } while (0)
 #define AH_HIP(expr) do { hipError_t _e = (expr); if (_e != hipSuccess) return ah::hip_fail(_e, #expr); } while (0)

@@ -143,6 +143,14 @@ __global__ void k_argmax(const float *__restrict__ a, int32_t *__restrict__ out,
   }
 }
 
+// Partial sums of ah_sum_sq_static: device memory that exists from load time to process exit, so that entry point never
+// allocates.  In host code this name is only a stand-in for the symbol; the device address comes from hipGetSymbolAddress
+// (static_partials_init) and is what every launch is given.
+constexpr int STATIC_PARTIALS = 4096;
+static __device__ __align__(256) double g_static_partials[STATIC_PARTIALS];
+constexpr int MAX_DEVICES = 16;
+double *g_static_partials_ptr[MAX_DEVICES] = {};
+
 int partial_blocks(uint64_t n) {
   int64_t b = cdiv((int64_t)cdiv((int64_t)n, 4), TPB);
   int64_t cap = (int64_t)num_cus() * 8;
@@ -150,6 +158,18 @@ int partial_blocks(uint64_t n) {
 }
 
 }  // namespace
+
+namespace ah {
+// Called by ah_init with the device current: each device holds its own copy of the array at its own address.
+int32_t static_partials_init(int device) {
+  if (device < 0 || device >= MAX_DEVICES) return fail(AH_ERR_ARG, "ah_init: device %d beyond the %d this library keeps static scratch for", device, MAX_DEVICES);
+  void *ptr = nullptr;
+  hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_static_partials));
+  if (e != hipSuccess) return hip_fail(e, "hipGetSymbolAddress(g_static_partials)");
+  g_static_partials_ptr[device] = static_cast<double *>(ptr);
+  return AH_OK;
+}
+}  // namespace ah
 
 extern "C" {
 
@@ -190,6 +210,24 @@ int32_t ah_sum_all(ah_ptr a, ah_ptr out, uint64_t n, int32_t mean) {
   return full_reduce(a, n, out, mean ? (double)n : 1.0, 0, "ah_sum_all");
 }
 int32_t ah_sum_sq(ah_ptr x, uint64_t n, ah_ptr out) { return full_reduce(x, n, out, 1.0, 1, "ah_sum_sq"); }
+
+int32_t ah_sum_sq_static(ah_ptr x, uint64_t n, ah_ptr out) {
+  AH_REQUIRE_READY();
+  AH_ARG(out != 0, "ah_sum_sq_static: null out");
+  AH_ARG(n >= 1, "ah_sum_sq_static: n must be at least 1");
+  AH_ARG(n <= (uint64_t(1) << 32), "ah_sum_sq_static: n = %llu exceeds the maximum of 2^32 elements", (unsigned long long)n);
+  AH_ARG(x != 0, "ah_sum_sq_static: null input");
+  int nb = partial_blocks(n);                       // the same partition as ah_sum_sq: results are bit-identical
+  if (nb > STATIC_PARTIALS) return fail(AH_ERR_UNSUPPORTED, "ah_sum_sq_static: %d partial sums exceed the static %d", nb, STATIC_PARTIALS);
+  double *partial = g_static_partials_ptr[current_device()];
+  if (!partial) return fail(AH_ERR_STATE, "ah_sum_sq_static: static scratch of device %d was not set up", current_device());
+  // partial[0, nb) is written in full by the first kernel before the second reads exactly that range: nothing to clear.
+  hipLaunchKernelGGL(k_partial_sum<1>, dim3(nb), dim3(TPB), 0, stream(), dp<const float>(x), n, partial);
+  AH_LAUNCH_CHECK();
+  hipLaunchKernelGGL(k_final_sum, dim3(1), dim3(TPB), 0, stream(), partial, nb, dp<float>(out), 1.0);
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
 
 int32_t ah_softmax(ah_ptr a, ah_ptr out, int64_t outer, int64_t dim, int64_t inner, int32_t log_softmax) {
   AH_REQUIRE_READY();

@@ -62,6 +62,7 @@ namespace ah {
 hipStream_t stream() { return g.stream; }
 bool ready() { return g.inited; }
 int num_cus() { return g.prop.multiProcessorCount; }
+int current_device() { return g.device; }
 void count_op() { g.ops++; }
 int32_t fail(int32_t code, const char *fmt, ...) {
   va_list ap;
@@ -112,6 +113,7 @@ int32_t ah_init(int32_t device) {
   AH_HIP(hipEventCreateWithFlags(&g.ring_ev[0], hipEventDisableTiming));
   AH_HIP(hipEventCreateWithFlags(&g.ring_ev[1], hipEventDisableTiming));
   g.device = device;
+  { int32_t rc = static_partials_init(device); if (rc != AH_OK) return rc; }
   g.inited = true;
   g.err[0] = 0;
   return AH_OK;

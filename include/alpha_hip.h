@@ -168,6 +168,13 @@ int32_t ah_softmax(ah_ptr a, ah_ptr out, int64_t outer, int64_t dim, int64_t inn
 int32_t ah_argmax(ah_ptr a, ah_ptr out_i32, int64_t outer, int64_t dim, int64_t inner);
 /* out[0] (f32) = sum of x^2 over n elements; deterministic two-stage f64 reduction */
 int32_t ah_sum_sq(ah_ptr x, uint64_t n, ah_ptr out);
+/* ah_sum_sq for callers that cannot allocate (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc): it has no counterpart in the reference.  Same kernels, same partition and so bit-identical results, but the
+ * partial sums live in a 32 KiB array that is part of the library image on each device (held until the process ends) instead
+ * of pool scratch; the call makes no hipMalloc / hipFree and no allocating library call.  1 <= n <= 2^32 elements, anything
+ * larger is refused with AH_ERR_ARG.  All calls on one GPU share that array: calls that overlap on one GPU (other streams,
+ * other threads) race; calls on this library's single stream are ordered and safe. */
+int32_t ah_sum_sq_static(ah_ptr x, uint64_t n, ah_ptr out);
 /* softmax backward: s*(g - sum(g*s)) over the last dim (ops.ts:688-700), rows x dim */
 int32_t ah_softmax_bwd(ah_ptr s, ah_ptr g, ah_ptr out, int64_t rows, int64_t dim);
 
