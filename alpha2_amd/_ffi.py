@@ -29,7 +29,8 @@ class AhDeviceInfo(C.Structure):
 
 class AhStats(C.Structure):
     _fields_ = [("live_allocs", u64), ("live_bytes", u64), ("pool_blocks", u64), ("pool_bytes", u64),
-                ("device_mallocs", u64), ("ops_launched", u64), ("graphs_live", u64)]
+                ("device_mallocs", u64), ("ops_launched", u64), ("graphs_live", u64),
+                ("steps_recorded", u64), ("steps_replayed", u64), ("steps_fallback", u64), ("step_node_updates", u64)]
 
 
 class AhGemm(C.Structure):
@@ -121,6 +122,7 @@ SIGNATURES = {
     "ah_flash_fwd": [C.POINTER(AhFlash)], "ah_flash_bwd": [C.POINTER(AhFlash)],
     "ah_adamw": [u64, u64, u64, u64, u64, C.POINTER(AhAdamW), u64, u64, u64],
     "ah_clip_coef": [u64, f32, f32, u64],
+    "ah_step_begin": [u64], "ah_step_end": [C.POINTER(C.c_int32)], "ah_step_reset": [u64],
     "ah_step_guard": [u64, u64, f32, f32, C.c_double, C.c_double, u64, u64, u64],
     "ah_lion": [u64, u64, u64, u64, C.POINTER(AhLion)], "ah_sgd": [u64, u64, u64, C.c_double, C.c_double],
     "ah_adafactor_2d": [u64, u64, u64, u64, i64, i64, C.POINTER(AhAdafactor)],
@@ -157,6 +159,8 @@ def load():
     lib.ah_layernorm_bwd_partials_bytes.restype = i64       # a size, not a status
     lib.ah_last_error.argtypes = []
     lib.ah_last_error.restype = C.c_char_p
+    lib.ah_step_note.argtypes = []
+    lib.ah_step_note.restype = C.c_char_p
     _lib = lib
     return lib
 

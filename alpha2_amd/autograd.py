@@ -50,12 +50,12 @@ class Tape:
         """tape.ts:60-157: reverse walk; first gradient is cloned, later ones accumulate in place; each consumed
         gradient and each entry's forward activation is released as soon as nothing later can read it."""
         loss.grad = initialGrad if initialGrad is not None else backend.ones(loss.data.shape, loss.data.dtype)
-        released = set()
+        released = {}        # id -> the tensor itself: keeping it alive keeps its id from being handed to a new object
 
         def release_once(td):
             if releaseTensor is None or td is None or id(td) in released:
                 return
-            released.add(id(td))
+            released[id(td)] = td
             releaseTensor(td)
 
         for entry in reversed(self.entries):

@@ -104,6 +104,10 @@ class HipBackend:
         self.lib = ffi.load()
         check(self.lib.ah_init(device))
         self._min_gpu_size = 0
+        self._step_graphs, self._step_open, self._step_key = False, False, 0
+        self.lastStepHow, self.lastStepNote = "eager", ""
+        self.stepFallbackNotes: List[str] = []
+        self._hyper_dev, self._hyper_key = None, None
 
     # ------------------------------------------------------------------ residency helpers
     def _new(self, shape, dtype="f32", store: Optional[str] = None) -> TensorData:
@@ -161,7 +165,45 @@ class HipBackend:
         t._buf, t._dev_valid = None, False
 
     def flush(self):
-        """Work is already on the stream in call order; nothing is batched on the host."""
+        """The trainer's end-of-step call (trainer.ts:1776-1784).  Work is already on the stream in call order, so there
+        is nothing to submit; with step graphs enabled it is the seam between two steps: the open step plan is closed
+        (recorded, replayed or fallen back) and the next one is opened, so everything the unchanged trainer issues from one
+        flush() to the next runs as recorded hipGraph segments from the third step on."""
+        if self._step_graphs:
+            if self._step_open:
+                self.stepEnd()
+            self.stepBegin()
+
+    # ------------------------------------------------------------------ step plans (record -> verify -> replay)
+    STEP_HOW = ("eager", "recorded", "replayed", "fell-back")
+
+    def enableStepGraphs(self, on: bool = True, key: int = 0):
+        """Bracket every flush()-to-flush() interval with ah_step_begin / ah_step_end."""
+        if not on and self._step_open:
+            self.stepEnd()
+        self._step_graphs, self._step_key = bool(on), int(key)
+
+    def stepBegin(self, key: Optional[int] = None):
+        check(self.lib.ah_step_begin(self._step_key if key is None else int(key)))
+        self._step_open = True
+
+    def stepEnd(self) -> str:
+        how = C.c_int32(0)
+        self._step_open = False
+        check(self.lib.ah_step_end(C.byref(how)))
+        self.lastStepHow = self.STEP_HOW[how.value]
+        self.lastStepNote = self.lib.ah_step_note().decode("utf-8", "replace")
+        if how.value == 3:
+            self.stepFallbackNotes.append(self.lastStepNote)
+        return self.lastStepHow
+
+    def resetStepPlan(self, key: Optional[int] = None):
+        """Forget the recorded plan (the next bracketed step records again)."""
+        check(self.lib.ah_step_reset(self._step_key if key is None else int(key)))
+
+    def stepStats(self) -> dict:
+        s = self._stats()
+        return {"recorded": s.steps_recorded, "replayed": s.steps_replayed, "fellBack": s.steps_fallback, "nodeUpdates": s.step_node_updates}
 
     def syncGpu(self):
         check(self.lib.ah_sync())
@@ -263,6 +305,12 @@ class HipBackend:
         for t in ts:
             if t.dtype != "f32" or t.store != "f32":
                 raise TypeError(f"op expects f32 tensors, got {t.dtype}/{t.store}")
+
+    def _words(self, *ts):
+        """The data-movement kernels copy 4-byte elements: a tensor stored in 2 bytes must not reach them as it is."""
+        for t in ts:
+            if ffi.DTYPE_BYTES[t.store] != 4:
+                raise TypeError(f"data-movement op expects 4-byte storage, got {t.dtype}/{t.store}")
 
     def add(self, a, b): return self._binary(ffi.ADD, a, b)
     def sub(self, a, b): return self._binary(ffi.SUB, a, b)
@@ -598,16 +646,19 @@ class HipBackend:
         d0, d1 = self._axis(dim0, nd), self._axis(dim1, nd)
         ns = list(a.shape)
         ns[d0], ns[d1] = a.shape[d1], a.shape[d0]
+        self._words(a)
         out = self._new(ns, a.dtype)
         check(self.lib.ah_transpose(self._ptr(a), out._buf.ptr, nd, ffi.shape_arr(a.shape), d0, d1))
         return out
 
     def slice(self, a: TensorData, starts, ends) -> TensorData:
+        self._words(a)
         out = self._new([e - s for s, e in zip(starts, ends)], a.dtype)
         check(self.lib.ah_slice(self._ptr(a), out._buf.ptr, len(a.shape), ffi.shape_arr(a.shape), ffi.shape_arr(starts), ffi.shape_arr(ends)))
         return out
 
     def scatterSlice(self, grad: TensorData, origShape, starts, ends) -> TensorData:
+        self._words(grad)
         out = self._new(origShape, grad.dtype)
         check(self.lib.ah_scatter_slice(self._ptr(grad), out._buf.ptr, len(origShape), ffi.shape_arr(grad.shape), ffi.shape_arr(origShape),
                                         ffi.shape_arr(starts)))
@@ -616,6 +667,7 @@ class HipBackend:
     def sliceQkv(self, a: TensorData):
         rows, c3 = a.shape
         d = c3 // 3
+        self._words(a)
         q, k, v = self._new((rows, d)), self._new((rows, d)), self._new((rows, d))
         check(self.lib.ah_slice_qkv(self._ptr(a), q._buf.ptr, k._buf.ptr, v._buf.ptr, rows, d))
         return [q, k, v]
@@ -632,6 +684,7 @@ class HipBackend:
                     oshape[d] += t.shape[d]
                 elif t.shape[d] != oshape[d]:
                     raise ValueError(f"cat: shape mismatch at dim {d}")
+        self._words(*tensors)
         out = self._new(oshape, tensors[0].dtype)
         off = 0
         for t in tensors:
@@ -642,6 +695,7 @@ class HipBackend:
     def broadcast(self, a: TensorData, targetShape) -> TensorData:
         nd = len(targetShape)
         src = (1,) * (nd - len(a.shape)) + tuple(a.shape)
+        self._words(a)
         out = self._new(targetShape, a.dtype)
         check(self.lib.ah_broadcast(self._ptr(a), out._buf.ptr, nd, ffi.shape_arr(targetShape), ffi.shape_arr(self._bstrides(src, targetShape))))
         return out
@@ -817,10 +871,23 @@ class HipBackend:
         self._f32(params, grads, m, v)
         if not (params.size == grads.size == m.size == v.size):
             raise ValueError("adamwStep: params, grads, m, v must have the same size")
-        h = ffi.AhAdamW(lr, beta1, beta2, eps, weightDecay, bc1, bc2, gradScale)
-        check(self.lib.ah_adamw(self._ptr(params), self._ptr(grads), self._ptr(m), self._ptr(v), params.size, C.byref(h), 0, 0, 0))
+        h, dev = self._adam_hyper(lr, beta1, beta2, eps, weightDecay, bc1, bc2, gradScale)
+        check(self.lib.ah_adamw(self._ptr(params), self._ptr(grads), self._ptr(m), self._ptr(v), params.size, C.byref(h), dev, 0, 0))
         for t in (params, m, v):
             self._dirty(t)
+
+    def _adam_hyper(self, lr, beta1, beta2, eps, weightDecay, bc1, bc2, gradScale):
+        """The optimizer's scalars are the same for every tensor of a step except the weight decay (optimizers.ts:54-94): they
+        are written to a small device struct once per step, which the kernel reads, and the by-value argument carries only
+        the weight decay.  A recorded step plan then needs no node rewritten when the learning rate moves."""
+        key = (lr, beta1, beta2, eps, bc1, bc2, gradScale)
+        if self._hyper_dev is None:
+            self._hyper_dev = _Buf(self.lib, C.sizeof(ffi.AhAdamW))
+        if key != self._hyper_key:
+            full = ffi.AhAdamW(lr, beta1, beta2, eps, 0.0, bc1, bc2, gradScale)
+            check(self.lib.ah_upload(self._hyper_dev.ptr, C.byref(full), C.sizeof(full)))
+            self._hyper_key = key
+        return ffi.AhAdamW(0.0, 0.0, 0.0, 0.0, weightDecay, 0.0, 0.0, 0.0), self._hyper_dev.ptr
 
     # The reference runs its other optimizers as host loops inside the optimizer classes (optimizers.ts:236-593), not
     # through the Backend interface; these device versions keep parameters and state resident.

@@ -1,0 +1,433 @@
+"""`FastHipBackend`: the same `Backend` interface as `HipBackend` (packages/core/src/interfaces.ts:38-151), with the fast mode
+kept entirely behind it -- callers still see "f32" TensorData (the reference's Dtype has no bf16, packages/core/src/types.ts:6)
+and still issue one call per op, as the reference's tape-driven trainer does (packages/autograd/src/ops.ts:197-234,426-487;
+packages/train/src/trainer.ts:1188-1273,1761-1784).  Behind the interface:
+
+  * activations that only feed matrix products are STORED as bf16 (LayerNorm outputs, linear-layer outputs, attention
+    outputs, their gradients); the residual stream, parameters, gradients of parameters and optimizer state stay f32;
+  * every 2-D parameter has a bf16 shadow that `adamwStep` refreshes in the same pass (the MFMA operand of the next step);
+  * a linear layer's product is held back by ONE call, so that the op the reference issues next can become its epilogue:
+        gelu(matmulTransposed(x, W))                   -> AH_EPI_GELU      (ops.ts:426-487 issues exactly these two calls)
+        geluBackward(pre, matmul(g, W))                -> AH_EPI_GELU_BWD
+        add(x, reshape(matmulTransposed(h, W)))        -> AH_EPI_RESIDUAL  (gpt.ts:280-281,331-332 via residualDropoutAdd)
+    anything else that touches the held-back product simply launches it as it is;
+  * weight gradients dW = G^T X (matmulTransposedA) are held back until something reads one of them (in the trainer: the
+    gradient norm), then computed by ONE grouped launch over all of them, accumulating straight into an existing gradient
+    when the tape's addInplace asked for that;
+  * clone() is copy-on-write (the tape clones every first gradient, tape.ts:126).
+
+Everything not named here runs the inherited f32 kernels after an on-the-fly cast, so the whole interface keeps working.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import List, Optional, Sequence
+
+import numpy as np
+
+from . import _ffi as ffi
+from ._ffi import check
+from .backend import HipBackend, TensorData, _Buf, shapeSize
+
+BF16, F32 = ffi.BF16, ffi.F32
+
+
+class _HeldGemm:
+    """A product whose launch is held back by one call.  It holds a reference on its operands' buffers and on its output
+    buffer until it is launched (or dropped, when nobody but this record still refers to the output)."""
+    __slots__ = ("layout", "a_ptr", "b_ptr", "out_buf", "out_off", "m", "n", "k", "lda", "ldb", "holds")
+
+    def __init__(self, layout, a_ptr, b_ptr, out, m, n, k, lda, ldb, holds):
+        self.layout, self.a_ptr, self.b_ptr, self.out_buf, self.out_off = layout, a_ptr, b_ptr, out._buf, out._off
+        self.m, self.n, self.k, self.lda, self.ldb, self.holds = m, n, k, lda, ldb, holds
+
+    @property
+    def out_ptr(self) -> int:
+        return self.out_buf.ptr + self.out_off
+
+
+class _HeldWeightGrad:
+    __slots__ = ("g_ptr", "x_ptr", "out_buf", "out_off", "m", "n", "k", "holds", "into")
+
+    def __init__(self, g_ptr, x_ptr, out, m, n, k, holds):
+        self.g_ptr, self.x_ptr, self.out_buf, self.out_off, self.m, self.n, self.k, self.holds = g_ptr, x_ptr, out._buf, out._off, m, n, k, holds
+        self.into = None                  # (buffer, offset) of an existing gradient to accumulate into instead
+
+
+class FastHipBackend(HipBackend):
+    name = "hip"
+
+    def __init__(self, device: int = 0, group_weight_grads: bool = True):
+        super().__init__(device)
+        self._held: Optional[_HeldGemm] = None
+        self._wgrads: List[_HeldWeightGrad] = []
+        self._group = group_weight_grads
+        self._plans = {}                 # descriptor tuple -> grouped plan id
+        # products that became another op's epilogue and were never written themselves: computed only if somebody reads them
+        self._orphans = {}               # id(_Buf) -> _HeldGemm
+
+    # ------------------------------------------------------------------ storage helpers
+    def _hold(self, *bufs):
+        for b in bufs:
+            b.refs += 1
+        return list(bufs)
+
+    def _unhold(self, holds):
+        for b in holds:
+            b.release()
+
+    def _is_held(self, t: TensorData) -> bool:
+        h = self._held
+        return h is not None and t._buf is h.out_buf
+
+    def _is_queued(self, buf) -> bool:
+        return any(buf is w.out_buf for w in self._wgrads)
+
+    def _ptr(self, t: TensorData) -> int:
+        if not t._dev_valid and t._buf is not None:
+            t._shadow = None                                    # the host wrote new contents: the bf16 shadow is stale
+        if t._buf is not None:
+            if self._held is not None and t._buf is self._held.out_buf:
+                self._launch_held()
+            elif self._wgrads and (self._is_queued(t._buf) or any(w.into is not None and w.into[0] is t._buf for w in self._wgrads)):
+                self._launch_weight_grads()
+            elif self._orphans and id(t._buf) in self._orphans:
+                h = self._orphans.pop(id(t._buf))
+                self._gemm(h.layout, h.a_ptr, h.b_ptr, h.out_ptr, h.m, h.n, h.k, h.lda, h.ldb, h.n, in_dtype=BF16, out_dtype=BF16)
+                self._unhold(h.holds)
+        return super()._ptr(t)
+
+    def _download(self, t: TensorData):
+        self._ptr(t)
+        return super()._download(t)
+
+    def _f32(self, *ts):
+        """Ops inherited from HipBackend take f32 storage: a bf16-stored operand gets an f32 copy of its own."""
+        for t in ts:
+            if t.dtype != "f32":
+                raise TypeError(f"op expects f32 tensors, got {t.dtype}")
+            if t.store == "bf16":
+                src = self._ptr(t)
+                buf = _Buf(self.lib, t.size * 4)
+                check(self.lib.ah_cast(src, BF16, buf.ptr, F32, t.size))
+                t._buf.release()
+                t._buf, t._off, t.store = buf, 0, "f32"
+
+    def _words(self, *ts):
+        """Inherited data-movement kernels copy 4-byte elements: a bf16-stored tensor gets f32 storage first."""
+        self._f32(*[t for t in ts if t.store == "bf16"])
+
+    def _dirty(self, t: TensorData):
+        super()._dirty(t)
+        t._shadow = None
+
+    def _operand(self, t: TensorData):
+        """Device address of `t` as a bf16 matrix operand, and the buffer that must outlive the launch."""
+        if t.store == "bf16":
+            return self._ptr(t), t._buf
+        p = self._ptr(t)
+        sh = getattr(t, "_shadow", None)
+        if sh is None or sh.ptr == 0:
+            sh = _Buf(self.lib, t.size * 2)
+            check(self.lib.ah_cast(p, F32, sh.ptr, BF16, t.size))
+            t._shadow = sh
+        return sh.ptr, sh
+
+    def releaseGpuTensor(self, t: TensorData):
+        if t is None or t._buf is None:
+            return
+        sh = getattr(t, "_shadow", None)
+        if sh is not None:
+            sh.release()
+            t._shadow = None
+        buf = t._buf
+        super().releaseGpuTensor(t)
+        if buf.refs == 1:                                       # only a held-back record still refers to it: nobody will read it
+            if self._held is not None and buf is self._held.out_buf:
+                h, self._held = self._held, None
+                self._unhold(h.holds)
+            elif self._orphans and id(buf) in self._orphans:
+                self._unhold(self._orphans.pop(id(buf)).holds)
+            elif self._wgrads:
+                for i, w in enumerate(self._wgrads):
+                    if buf is w.out_buf and w.into is None:
+                        del self._wgrads[i]
+                        self._unhold(w.holds)
+                        break
+
+    def _view(self, t: TensorData, shape, byte_off: int = 0) -> TensorData:
+        if t._buf is not None and t._dev_valid and (self._is_held(t) or id(t._buf) in self._orphans or self._is_queued(t._buf)):
+            v = TensorData(shape, t.dtype)                      # a view of a held-back product stays held back
+            v.store, v._buf, v._off = t.store, t._buf, t._off + byte_off
+            t._buf.refs += 1
+            v._dev_valid, v._backend = True, self
+            return v
+        return super()._view(t, shape, byte_off)
+
+    # ------------------------------------------------------------------ held-back linear-layer products
+    def _launch_held(self, epilogue=ffi.EPI_NONE, aux: int = 0, out: Optional[TensorData] = None, out_dtype=BF16):
+        h, self._held = self._held, None
+        if h is None:
+            return
+        if out is None and h.out_buf.refs == 1:                 # every tensor that named this product has been released
+            self._unhold(h.holds)
+            return
+        dst = h.out_ptr if out is None else out._buf.ptr + out._off
+        self._gemm(h.layout, h.a_ptr, h.b_ptr, dst, h.m, h.n, h.k, h.lda, h.ldb, h.n, in_dtype=BF16, out_dtype=out_dtype,
+                   epilogue=epilogue, aux=aux)
+        if out is not None and epilogue != ffi.EPI_GELU and h.out_buf.refs > 1:
+            self._orphans[id(h.out_buf)] = h                    # the plain product was not written: keep the recipe
+        else:
+            self._unhold(h.holds)
+
+    def _hold_gemm(self, layout, a: TensorData, b: TensorData, oshape, m, n, k, lda, ldb) -> TensorData:
+        self._launch_held()
+        ap, ah = self._operand(a)
+        bp, bh = self._operand(b)
+        out = self._new(oshape, "f32", "bf16")
+        self._held = _HeldGemm(layout, ap, bp, out, m, n, k, lda, ldb, self._hold(ah, bh, out._buf))
+        return out
+
+    def matmulTransposed(self, a: TensorData, b: TensorData) -> TensorData:
+        if len(a.shape) != 2 or len(b.shape) != 2:
+            return super().matmulTransposed(a, b)
+        M, K, N = a.shape[0], a.shape[1], b.shape[0]
+        if b.shape[1] != K:
+            raise ValueError(f"matmul shape mismatch: [{a.shape}] x [{b.shape}]^T")
+        return self._hold_gemm(ffi.GEMM_NT, a, b, (M, N), M, N, K, K, K)
+
+    def matmul(self, a: TensorData, b: TensorData) -> TensorData:
+        if len(a.shape) != 2 or len(b.shape) != 2:
+            return super().matmul(a, b)
+        M, K, N = a.shape[0], a.shape[1], b.shape[1]
+        if b.shape[0] != K:
+            raise ValueError(f"matmul shape mismatch: [{a.shape}] x [{b.shape}]")
+        return self._hold_gemm(ffi.GEMM_NN, a, b, (M, N), M, N, K, K, N)
+
+    def gelu(self, a: TensorData) -> TensorData:
+        if self._is_held(a) and self._held.layout == ffi.GEMM_NT:
+            out = self._new(a.shape, "f32", "bf16")             # `a` receives the pre-activation, as the caller expects
+            self._launch_held(ffi.EPI_GELU, aux=a._buf.ptr + a._off, out=out)
+            return out
+        return super().gelu(a)
+
+    def geluBackward(self, x: TensorData, g: TensorData) -> TensorData:
+        if self._is_held(g) and x.store == "bf16" and x.shape == g.shape and not self._is_held(x):
+            pre = self._ptr(x)
+            out = self._new(g.shape, "f32", "bf16")
+            self._launch_held(ffi.EPI_GELU_BWD, aux=pre, out=out)
+            return out
+        return super().geluBackward(x, g)
+
+    def add(self, a: TensorData, b: TensorData) -> TensorData:
+        for res, prod in ((a, b), (b, a)):
+            if self._is_held(prod) and res.store == "f32" and tuple(res.shape) == tuple(prod.shape) and res.dtype == "f32" and not self._is_held(res):
+                out = self._new(res.shape)
+                rp = self._ptr(res)
+                self._launch_held(ffi.EPI_RESIDUAL, aux=rp, out=out, out_dtype=F32)
+                return out
+        return super().add(a, b)
+
+    def residualDropoutAdd(self, residual, projected, mask) -> TensorData:
+        if mask is None:
+            return self.add(residual, projected)
+        return super().residualDropoutAdd(residual, projected, mask)
+
+    # ------------------------------------------------------------------ weight gradients, grouped
+    def matmulTransposedA(self, a: TensorData, b: TensorData) -> TensorData:
+        """A[M,K]^T @ B[M,N] -> [K,N]: in the trainer, dW = G^T X over M = tokens."""
+        if len(a.shape) != 2 or len(b.shape) != 2:
+            return super().matmulTransposedA(a, b)
+        M, K, N = a.shape[0], a.shape[1], b.shape[1]
+        if b.shape[0] != M:
+            raise ValueError(f"matmul shape mismatch: [{a.shape}]^T x [{b.shape}]")
+        ap, ah = self._operand(a)
+        bp, bh = self._operand(b)
+        out = self._new((K, N))
+        self._wgrads.append(_HeldWeightGrad(ap, bp, out, K, N, M, self._hold(ah, bh, out._buf)))
+        if not self._group:
+            self._launch_weight_grads()
+        return out
+
+    def _launch_weight_grads(self):
+        ws, self._wgrads = self._wgrads, []
+        descs = []
+        for w in ws:
+            if w.into is None and w.out_buf.refs == 1:          # released unread
+                continue
+            dst, epi = (w.out_buf.ptr + w.out_off, ffi.EPI_NONE) if w.into is None else (w.into[0].ptr + w.into[1], ffi.EPI_ACCUM)
+            descs.append(ffi.AhGemm(ffi.GEMM_TN, BF16, F32, epi, w.m, w.n, w.k, w.m, w.n, w.n, 1, 0, 0, 0, w.g_ptr, w.x_ptr, dst, 0))
+        groupable = all(d.k % 64 == 0 and d.m % 8 == 0 and d.n % 8 == 0 for d in descs)
+        for epi in (ffi.EPI_NONE, ffi.EPI_ACCUM):
+            part = [d for d in descs if d.epilogue == epi]
+            if groupable and len(part) > 1:
+                key = tuple((d.a, d.b, d.c, d.m, d.n, d.k) for d in part)
+                plan = self._plans.get(key)
+                if plan is None:
+                    if len(self._plans) >= 8:                   # buffers moved: old plans will not be asked for again
+                        for p in self._plans.values():
+                            check(self.lib.ah_gemm_grouped_destroy(p))
+                        self._plans = {}
+                    arr = (ffi.AhGemm * len(part))(*part)
+                    pid = C.c_uint64()
+                    check(self.lib.ah_gemm_grouped_plan(arr, len(part), C.byref(pid)))
+                    plan = self._plans[key] = pid.value
+                timed = getattr(self, "_timed", None)
+                if timed is None:
+                    check(self.lib.ah_gemm_grouped_run(plan, epi))
+                else:
+                    e0, e1 = self._event(), self._event()
+                    check(self.lib.ah_event_record(e0))
+                    check(self.lib.ah_gemm_grouped_run(plan, epi))
+                    check(self.lib.ah_event_record(e1))
+                    kernel, nsplit = self.lastGemmKernel()
+                    timed.append({"kind": "gemm", "kernel": kernel, "nsplit": nsplit, "layout": ffi.GEMM_TN, "dtype": BF16, "m": 0, "n": 0,
+                                  "k": part[0].k, "batch": 1, "flops": sum(2.0 * d.m * d.n * d.k for d in part), "e0": e0, "e1": e1})
+            else:
+                for d in part:
+                    check(self.lib.ah_gemm(C.byref(d)))
+        for w in ws:
+            self._unhold(w.holds)
+
+    def addInplace(self, a: TensorData, b: TensorData):
+        for w in self._wgrads:
+            if b._buf is w.out_buf and w.into is None and a.store == "f32" and a.size == b.size and a._buf is not None and a._dev_valid \
+                    and a._buf.refs == 1 and not self._is_queued(a._buf) and not any(o.into is not None and o.into[0] is a._buf for o in self._wgrads):
+                w.into = (a._buf, a._off)                        # the grouped launch adds into `a`; `b` itself is never computed
+                a._buf.refs += 1
+                w.holds.append(a._buf)
+                self._dirty(a)
+                return
+        self._launch_held()
+        self._ptr(a), self._ptr(b)                               # launches whatever still has to produce (or add into) them
+        if a._buf is not None and a._buf.refs > 1 and a._dev_valid and a.store == "f32" and b.store == "f32":
+            # copy-on-write: `a` shares its buffer (clone): the sum goes to a buffer of its own in one pass
+            pa, pb = self._ptr(a), self._ptr(b)
+            buf = _Buf(self.lib, a.size * 4)
+            check(self.lib.ah_binary(ffi.ADD, pa, pb, buf.ptr, a.size))
+            a._buf.release()
+            a._buf, a._off = buf, 0
+            self._dirty(a)
+            return
+        self._f32(a, b)
+        self._own(a)
+        super().addInplace(a, b)
+
+    def _own(self, t: TensorData):
+        """Before an in-place write: give `t` a buffer nobody else shares."""
+        if t._buf is not None and t._buf.refs > 1 and t._dev_valid:
+            n = t.size * ffi.DTYPE_BYTES[t.store]
+            buf = _Buf(self.lib, n)
+            check(self.lib.ah_copy(buf.ptr, self._ptr(t), n))
+            t._buf.release()
+            t._buf, t._off = buf, 0
+
+    def scaleInplace(self, a: TensorData, s: float):
+        self._f32(a)
+        self._own(a)
+        super().scaleInplace(a, s)
+
+    def clone(self, a: TensorData) -> TensorData:
+        """Copy-on-write: the copy shares the buffer until one side is written in place (addInplace / scaleInplace /
+        adamwStep copy first).  A host-created tensor is uploaded by _view, as the eager clone would."""
+        return self._view(a, a.shape)
+
+    # ------------------------------------------------------------------ nn with bf16 storage
+    def layerNorm(self, x, weight, bias, eps) -> TensorData:
+        if x.store != "f32":
+            return super().layerNorm(x, weight, bias, eps)
+        dim = x.shape[-1]
+        if weight.size != dim or bias.size != dim:
+            raise ValueError("layerNorm: weight/bias length must equal the last dimension")
+        out = self._new(x.shape, "f32", "bf16")
+        check(self.lib.ah_layernorm(self._ptr(x), self._ptr(weight), self._ptr(bias), out._buf.ptr, x.size // max(1, dim), dim, eps, BF16))
+        return out
+
+    def layerNormBackward(self, x, weight, gradOutput, eps) -> dict:
+        if x.store != "f32":
+            return super().layerNormBackward(x, weight, gradOutput, eps)
+        dim = x.shape[-1]
+        gp = self._ptr(gradOutput)
+        dx, dw, db = self._new(x.shape), self._new(weight.shape), self._new(weight.shape)
+        check(self.lib.ah_layernorm_bwd(self._ptr(x), self._ptr(weight), gp, ffi.DTYPE_CODE[gradOutput.store], 0, dx._buf.ptr, 0, dw._buf.ptr,
+                                        db._buf.ptr, x.size // max(1, dim), dim, eps, 0))
+        return {"dx": dx, "dw": dw, "db": db}
+
+    def crossEntropy(self, logits: TensorData, targets: TensorData) -> TensorData:
+        N, Cc = logits.shape
+        out, lse = self._new(()), self._new((N,))
+        check(self.lib.ah_cross_entropy(self._ptr(logits), ffi.DTYPE_CODE[logits.store], self._ptr(targets), out._buf.ptr, lse._buf.ptr, N, Cc))
+        logits._ce_lse = lse
+        return out
+
+    def crossEntropyBackward(self, logits, targets, gradOutput) -> TensorData:
+        lse = getattr(logits, "_ce_lse", None)
+        if lse is None or lse._buf is None or logits.store != "bf16":
+            self._f32(logits)
+            return super().crossEntropyBackward(logits, targets, gradOutput)
+        N, Cc = logits.shape
+        out = self._new((N, Cc), "f32", "bf16")
+        check(self.lib.ah_cross_entropy_bwd(self._ptr(logits), BF16, self._ptr(targets), lse._buf.ptr, self._ptr(gradOutput), 1.0,
+                                            out._buf.ptr, N, Cc))
+        return out
+
+    def flashAttention(self, Q, K, V, T, scale, softCap) -> dict:
+        if not (Q.store == K.store == V.store):
+            self._words(Q, K, V)
+        return super().flashAttention(Q, K, V, T, scale, softCap)
+
+    def flashAttentionBackward(self, Q, K, V, O, dO, lse, T, scale, softCap) -> dict:
+        if not (Q.store == K.store == V.store == O.store == dO.store):
+            self._words(Q, K, V, O, dO)
+        return super().flashAttentionBackward(Q, K, V, O, dO, lse, T, scale, softCap)
+
+    def attentionQkvBackward(self, qkv, out, dOut, lse, Bt, T, nHead, scale, softCap) -> TensorData:
+        if not (qkv.store == out.store == dOut.store):
+            self._words(qkv, out, dOut)
+        return super().attentionQkvBackward(qkv, out, dOut, lse, Bt, T, nHead, scale, softCap)
+
+    # ------------------------------------------------------------------ optimizer
+    def totalSumOfSquares(self, tensors: Sequence[TensorData]) -> TensorData:
+        self._launch_held()
+        self._launch_weight_grads()
+        return super().totalSumOfSquares(tensors)
+
+    def adamwStep(self, params, grads, m, v, lr, beta1, beta2, eps, weightDecay, bc1, bc2, gradScale=1.0):
+        self._launch_held()
+        self._f32(params, grads, m, v)
+        if not (params.size == grads.size == m.size == v.size):
+            raise ValueError("adamwStep: params, grads, m, v must have the same size")
+        for t in (params, m, v):
+            self._own(t)
+        pp = self._ptr(params)
+        sh = getattr(params, "_shadow", None)
+        h, dev = self._adam_hyper(lr, beta1, beta2, eps, weightDecay, bc1, bc2, gradScale)
+        check(self.lib.ah_adamw(pp, self._ptr(grads), self._ptr(m), self._ptr(v), params.size, C.byref(h), dev, 0, sh.ptr if sh is not None else 0))
+        for t in (params, m, v):
+            HipBackend._dirty(self, t)                          # host copies are stale; the shadow was refreshed by the kernel
+
+    def lionStep(self, params, grads, m, *a, **kw):
+        self._own(params), self._own(m)
+        super().lionStep(params, grads, m, *a, **kw)
+
+    def sgdStep(self, params, grads, *a, **kw):
+        self._own(params)
+        super().sgdStep(params, grads, *a, **kw)
+
+    def adafactorStep2d(self, params, grads, vr, vc, *a, **kw):
+        self._own(params), self._own(vr), self._own(vc)
+        super().adafactorStep2d(params, grads, vr, vc, *a, **kw)
+
+    def adafactorStepFlat(self, params, grads, v, *a, **kw):
+        self._own(params), self._own(v)
+        super().adafactorStepFlat(params, grads, v, *a, **kw)
+
+    def flush(self):
+        self._launch_held()
+        self._launch_weight_grads()
+        super().flush()
+
+    def syncGpu(self):
+        self._launch_held()
+        self._launch_weight_grads()
+        super().syncGpu()

@@ -325,7 +325,7 @@ int32_t check(const AhFlash *f, bool bwd, FlashArgs &a) {
 template <int D>
 int32_t run_fwd(const FlashArgs &a) {
   dim3 grid((unsigned)cdiv(a.T, WAVES * 32), (unsigned)(a.B * a.H));
-  hipLaunchKernelGGL(k_flash_fwd_f32<D>, grid, dim3(256), 0, stream(), a);
+  ah::launch_kernel(k_flash_fwd_f32<D>, grid, dim3(256), 0, a);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
@@ -336,12 +336,12 @@ int32_t run_bwd(FlashArgs &a) {
   int32_t rc = ah_alloc((uint64_t)rows * 4, &delta);
   if (rc) return rc;
   a.delta = dp<float>(delta);
-  hipLaunchKernelGGL(k_flash_delta_f32<D>, dim3((unsigned)cdiv(rows, 4)), dim3(256), 0, stream(), a);
+  ah::launch_kernel(k_flash_delta_f32<D>, dim3((unsigned)cdiv(rows, 4)), dim3(256), 0, a);
   AH_LAUNCH_CHECK();
   dim3 grid((unsigned)cdiv(a.T, WAVES * 32), (unsigned)(a.B * a.H));
-  hipLaunchKernelGGL(k_flash_dq_f32<D>, grid, dim3(256), 0, stream(), a);
+  ah::launch_kernel(k_flash_dq_f32<D>, grid, dim3(256), 0, a);
   AH_LAUNCH_CHECK();
-  hipLaunchKernelGGL(k_flash_dkv_f32<D>, grid, dim3(256), 0, stream(), a);
+  ah::launch_kernel(k_flash_dkv_f32<D>, grid, dim3(256), 0, a);
   AH_LAUNCH_CHECK();
   return ah_free(delta);
 }

@@ -508,7 +508,7 @@ __global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void k_flash_dkv_bf16(FlashAr
 template <int D, bool CAPPED>
 int32_t run_fwd(const FlashArgs &a) {
   dim3 grid((unsigned)cdiv(a.T, 128), (unsigned)(a.B * a.H));
-  hipLaunchKernelGGL((k_flash_fwd_bf16<D, CAPPED>), grid, dim3(256), 0, stream(), a);
+  ah::launch_kernel((k_flash_fwd_bf16<D, CAPPED>), grid, dim3(256), 0, a);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
@@ -520,9 +520,9 @@ int32_t run_bwd(FlashArgs &a) {
   if (rc) return rc;
   a.delta = dp<float>(delta);
   dim3 grid((unsigned)cdiv(a.T, 128), (unsigned)(a.B * a.H));
-  hipLaunchKernelGGL((k_flash_dq_bf16<D, CAPPED>), grid, dim3(256), 0, stream(), a);      // also writes delta
+  ah::launch_kernel((k_flash_dq_bf16<D, CAPPED>), grid, dim3(256), 0, a);      // also writes delta
   AH_LAUNCH_CHECK();
-  hipLaunchKernelGGL((k_flash_dkv_bf16<D, CAPPED>), grid, dim3(256), 0, stream(), a);
+  ah::launch_kernel((k_flash_dkv_bf16<D, CAPPED>), grid, dim3(256), 0, a);
   AH_LAUNCH_CHECK();
   return ah_free(delta);
 }

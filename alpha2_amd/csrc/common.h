@@ -4,6 +4,8 @@
 #include <hip/hip_bf16.h>
 #include <stdint.h>
 #include <stddef.h>
+#include <tuple>
+#include <utility>
 #include "../../include/alpha_hip.h"
 
 namespace ah {
@@ -20,6 +22,29 @@ int         num_cus();
 void       *scratch(size_t bytes);
 int         current_device();                     // the device ah_init was called with
 int32_t     static_partials_init(int device);     // reduce.hip: device address of its static scratch array (called by ah_init)
+
+// Every kernel of the library is launched through launch_kernel(): the arguments are converted to the kernel's parameter
+// types and handed, as an array of pointers to them, to launch_raw (runtime.hip).  Outside a step plan that is
+// hipLaunchKernel on the library stream.  Inside one (ah_step_begin .. ah_step_end) the launch is recorded into the
+// stream capture, or -- when a plan exists -- compared with the plan's next kernel node: same kernel, same grid means
+// "skip, the graph will run it", with the node's parameters rewritten if any argument differs.
+void launch_raw(const void *func, dim3 grid, dim3 block, unsigned shmem, void **args, const uint32_t *sizes, int nargs);
+template <class... KArgs, class... Args, size_t... I>
+inline void launch_impl(void (*kernel)(KArgs...), dim3 grid, dim3 block, unsigned shmem, std::index_sequence<I...>, Args &&...args) {
+  std::tuple<KArgs...> vals{static_cast<KArgs>(std::forward<Args>(args))...};
+  void *ptrs[sizeof...(KArgs) + 1] = {(void *)&std::get<I>(vals)..., nullptr};
+  const uint32_t sizes[sizeof...(KArgs) + 1] = {(uint32_t)sizeof(KArgs)..., 0u};
+  launch_raw(reinterpret_cast<const void *>(kernel), grid, block, shmem, ptrs, sizes, (int)sizeof...(KArgs));
+}
+template <class... KArgs, class... Args>
+inline void launch_kernel(void (*kernel)(KArgs...), dim3 grid, dim3 block, unsigned shmem, Args &&...args) {
+  static_assert(sizeof...(KArgs) == sizeof...(Args), "kernel argument count");
+  launch_impl(kernel, grid, block, shmem, std::index_sequence_for<KArgs...>{}, std::forward<Args>(args)...);
+}
+// A point where the host needs the stream's results or touches it outside a kernel launch (download, sync, events):
+// inside a step plan the work recorded so far is launched first.  Returns AH_OK or an error code.
+int32_t step_boundary(const char *what);
+bool    step_active();
 
 #define AH_REQUIRE_READY() do { if (!ah::ready()) return ah::fail(AH_ERR_STATE, "%s: ah_init has not been called", __func__); } while (0)
 #define AH_HIP(expr) do { hipError_t _e = (expr); if (_e != hipSuccess) return ah::hip_fail(_e, #expr); } while (0)

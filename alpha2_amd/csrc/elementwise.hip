@@ -342,7 +342,7 @@ int32_t ah_fill_f32(ah_ptr dst, float value, uint64_t n) {
   AH_REQUIRE_READY();
   if (n == 0) return AH_OK;
   AH_ARG(dst != 0, "ah_fill_f32: null dst");
-  hipLaunchKernelGGL(k_fill<float>, dim3(grid_for(n / 4 + 1)), dim3(TPB), 0, stream(), dp<float>(dst), value, n);
+  ah::launch_kernel(k_fill<float>, dim3(grid_for(n / 4 + 1)), dim3(TPB), 0, dp<float>(dst), value, n);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
@@ -350,7 +350,7 @@ int32_t ah_fill_i32(ah_ptr dst, int32_t value, uint64_t n) {
   AH_REQUIRE_READY();
   if (n == 0) return AH_OK;
   AH_ARG(dst != 0, "ah_fill_i32: null dst");
-  hipLaunchKernelGGL(k_fill<int32_t>, dim3(grid_for(n / 4 + 1)), dim3(TPB), 0, stream(), dp<int32_t>(dst), value, n);
+  ah::launch_kernel(k_fill<int32_t>, dim3(grid_for(n / 4 + 1)), dim3(TPB), 0, dp<int32_t>(dst), value, n);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
@@ -361,7 +361,7 @@ int32_t ah_binary(int32_t op, ah_ptr a, ah_ptr b, ah_ptr out, uint64_t n) {
   if (n == 0) return AH_OK;
   AH_ARG(a && b && out, "ah_binary: null operand");
   int vec = vec_ok(n, a, b, out);
-  hipLaunchKernelGGL(k_binary<BinOp>, dim3(grid_for(vec ? n / 4 + 1 : n)), dim3(TPB), 0, stream(),
+  ah::launch_kernel(k_binary<BinOp>, dim3(grid_for(vec ? n / 4 + 1 : n)), dim3(TPB), 0, 
                      dp<const float>(a), dp<const float>(b), dp<float>(out), n, BinOp{op}, vec);
   AH_LAUNCH_CHECK();
   return AH_OK;
@@ -377,7 +377,7 @@ int32_t ah_binary_broadcast(int32_t op, ah_ptr a, ah_ptr b, ah_ptr out, int32_t 
   uint64_t n = (uint64_t)prod(nd, shape);
   if (n == 0) return AH_OK;
   AH_ARG(a && b && out, "ah_binary_broadcast: null operand");
-  hipLaunchKernelGGL(k_binary_bcast, dim3(grid_for(n)), dim3(TPB), 0, stream(), dp<const float>(a), dp<const float>(b),
+  ah::launch_kernel(k_binary_bcast, dim3(grid_for(n)), dim3(TPB), 0, dp<const float>(a), dp<const float>(b),
                      dp<float>(out), n, d, BinOp{op});
   AH_LAUNCH_CHECK();
   return AH_OK;
@@ -389,7 +389,7 @@ int32_t ah_unary(int32_t op, ah_ptr x, ah_ptr out, uint64_t n, float p0, float p
   if (n == 0) return AH_OK;
   AH_ARG(x && out, "ah_unary: null operand");
   int vec = vec_ok(n, x, x, out);
-  hipLaunchKernelGGL(k_unary<UnOp>, dim3(grid_for(vec ? n / 4 + 1 : n)), dim3(TPB), 0, stream(), dp<const float>(x),
+  ah::launch_kernel(k_unary<UnOp>, dim3(grid_for(vec ? n / 4 + 1 : n)), dim3(TPB), 0, dp<const float>(x),
                      dp<float>(out), n, UnOp{op, p0, p1}, vec);
   AH_LAUNCH_CHECK();
   return AH_OK;
@@ -401,7 +401,7 @@ int32_t ah_axpy_inplace(ah_ptr a, ah_ptr b, float s, uint64_t n) {
   AH_REQUIRE_READY();
   if (n == 0) return AH_OK;
   AH_ARG(a && b, "ah_axpy_inplace: null operand");
-  hipLaunchKernelGGL(k_axpy, dim3(grid_for(n)), dim3(TPB), 0, stream(), dp<float>(a), dp<const float>(b), s, n);
+  ah::launch_kernel(k_axpy, dim3(grid_for(n)), dim3(TPB), 0, dp<float>(a), dp<const float>(b), s, n);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
@@ -412,7 +412,7 @@ int32_t ah_unary_bwd(int32_t op, ah_ptr x, ah_ptr grad_out, ah_ptr out, uint64_t
   if (n == 0) return AH_OK;
   AH_ARG(x && grad_out && out, "ah_unary_bwd: null operand");
   int vec = vec_ok(n, x, grad_out, out);
-  hipLaunchKernelGGL(k_binary<UnBwd>, dim3(grid_for(vec ? n / 4 + 1 : n)), dim3(TPB), 0, stream(), dp<const float>(x),
+  ah::launch_kernel(k_binary<UnBwd>, dim3(grid_for(vec ? n / 4 + 1 : n)), dim3(TPB), 0, dp<const float>(x),
                      dp<const float>(grad_out), dp<float>(out), n, UnBwd{op, p0, p1}, vec);
   AH_LAUNCH_CHECK();
   return AH_OK;
@@ -422,7 +422,7 @@ int32_t ah_silu_mul(ah_ptr a, ah_ptr b, ah_ptr out, uint64_t n) {
   AH_REQUIRE_READY();
   if (n == 0) return AH_OK;
   AH_ARG(a && b && out, "ah_silu_mul: null operand");
-  hipLaunchKernelGGL(k_silu_mul, dim3(grid_for(n)), dim3(TPB), 0, stream(), dp<const float>(a), dp<const float>(b), dp<float>(out), n);
+  ah::launch_kernel(k_silu_mul, dim3(grid_for(n)), dim3(TPB), 0, dp<const float>(a), dp<const float>(b), dp<float>(out), n);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
@@ -430,7 +430,7 @@ int32_t ah_silu_mul_bwd(ah_ptr a, ah_ptr b, ah_ptr g, ah_ptr da, ah_ptr db, uint
   AH_REQUIRE_READY();
   if (n == 0) return AH_OK;
   AH_ARG(a && b && g && da && db, "ah_silu_mul_bwd: null operand");
-  hipLaunchKernelGGL(k_silu_mul_bwd, dim3(grid_for(n)), dim3(TPB), 0, stream(), dp<const float>(a), dp<const float>(b),
+  ah::launch_kernel(k_silu_mul_bwd, dim3(grid_for(n)), dim3(TPB), 0, dp<const float>(a), dp<const float>(b),
                      dp<const float>(g), dp<float>(da), dp<float>(db), n);
   AH_LAUNCH_CHECK();
   return AH_OK;
@@ -457,7 +457,7 @@ int32_t ah_channel_act(ah_ptr x, const ah_ptr *coefs, int32_t mask, ah_ptr out, 
   if (rc) return rc;
   if (rows == 0) return AH_OK;
   AH_ARG(x && out && aligned16(x) && aligned16(out), "ah_channel_act: operands must be non-null and 16-byte aligned");
-  hipLaunchKernelGGL(k_channel_act, dim3(grid_for((uint64_t)(rows * cols / 4))), dim3(TPB), 0, stream(), dp<const float>(x), p, dp<float>(out), rows, (int)(cols / 4));
+  ah::launch_kernel(k_channel_act, dim3(grid_for((uint64_t)(rows * cols / 4))), dim3(TPB), 0, dp<const float>(x), p, dp<float>(out), rows, (int)(cols / 4));
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
@@ -481,10 +481,10 @@ int32_t ah_channel_act_bwd(ah_ptr x, const ah_ptr *coefs, int32_t mask, ah_ptr g
   nrb = (int)cdiv(rows, rpb);
   float *partial = (float *)scratch(sizeof(float) * 5 * (size_t)nrb * (size_t)cols);
   if (!partial) return fail(AH_ERR_OOM, "ah_channel_act_bwd: no scratch");
-  hipLaunchKernelGGL(k_channel_act_bwd, dim3(gx, nrb), dim3(256), 0, stream(), dp<const float>(x), dp<const float>(grad_out), p, dp<float>(dx), partial,
+  ah::launch_kernel(k_channel_act_bwd, dim3(gx, nrb), dim3(256), 0, dp<const float>(x), dp<const float>(grad_out), p, dp<float>(dx), partial,
                      rows, cols4, rpb);
   AH_LAUNCH_CHECK();
-  hipLaunchKernelGGL(k_channel_act_colsum, dim3((unsigned)cdiv(cols, 256), 5), dim3(256), 0, stream(), partial, p, nrb, (int)cols);
+  ah::launch_kernel(k_channel_act_colsum, dim3((unsigned)cdiv(cols, 256), 5), dim3(256), 0, partial, p, nrb, (int)cols);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
@@ -492,7 +492,7 @@ int32_t ah_residual_dropout_add(ah_ptr residual, ah_ptr projected, ah_ptr mask, 
   AH_REQUIRE_READY();
   if (n == 0) return AH_OK;
   AH_ARG(residual && projected && out, "ah_residual_dropout_add: null operand");
-  hipLaunchKernelGGL(k_residual_dropout_add, dim3(grid_for(n)), dim3(TPB), 0, stream(), dp<const float>(residual),
+  ah::launch_kernel(k_residual_dropout_add, dim3(grid_for(n)), dim3(TPB), 0, dp<const float>(residual),
                      dp<const float>(projected), dp<const float>(mask), dp<float>(out), n);
   AH_LAUNCH_CHECK();
   return AH_OK;
@@ -503,7 +503,7 @@ int32_t ah_dropout_mask(ah_ptr out, uint64_t n, int32_t seed, int32_t counter, d
   AH_ARG(out != 0, "ah_dropout_mask: null out");
   AH_ARG(p >= 0.0 && p < 1.0, "ah_dropout_mask: p must be in [0,1)");
   AH_ARG(n <= (1ull << 32), "ah_dropout_mask: at most 2^32 elements (the hash sum must stay below 2^63)");
-  hipLaunchKernelGGL(k_dropout_mask, dim3(grid_for(n)), dim3(TPB), 0, stream(), dp<float>(out), n, seed, counter, p,
+  ah::launch_kernel(k_dropout_mask, dim3(grid_for(n)), dim3(TPB), 0, dp<float>(out), n, seed, counter, p,
                      (float)(1.0 / (1.0 - p)));
   AH_LAUNCH_CHECK();
   return AH_OK;
@@ -512,7 +512,7 @@ int32_t ah_masked_fill(ah_ptr a, ah_ptr mask, ah_ptr out, uint64_t n, uint64_t m
   AH_REQUIRE_READY();
   if (n == 0) return AH_OK;
   AH_ARG(a && mask && out && mask_n > 0, "ah_masked_fill: null operand or empty mask");
-  hipLaunchKernelGGL(k_masked_fill, dim3(grid_for(n)), dim3(TPB), 0, stream(), dp<const float>(a), dp<const float>(mask),
+  ah::launch_kernel(k_masked_fill, dim3(grid_for(n)), dim3(TPB), 0, dp<const float>(a), dp<const float>(mask),
                      dp<float>(out), n, mask_n, value);
   AH_LAUNCH_CHECK();
   return AH_OK;
@@ -521,7 +521,7 @@ int32_t ah_causal_mask(ah_ptr out, int64_t size) {
   AH_REQUIRE_READY();
   if (size <= 0) return AH_OK;
   AH_ARG(out != 0, "ah_causal_mask: null out");
-  hipLaunchKernelGGL(k_causal_mask, dim3(grid_for((uint64_t)size * size)), dim3(TPB), 0, stream(), dp<float>(out), size);
+  ah::launch_kernel(k_causal_mask, dim3(grid_for((uint64_t)size * size)), dim3(TPB), 0, dp<float>(out), size);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
@@ -530,7 +530,7 @@ int32_t ah_cast(ah_ptr src, int32_t sd, ah_ptr dst, int32_t dd, uint64_t n) {
   AH_ARG(sd >= AH_F32 && sd <= AH_F16 && dd >= AH_F32 && dd <= AH_F16, "ah_cast: bad dtype");
   if (n == 0) return AH_OK;
   AH_ARG(src && dst, "ah_cast: null operand");
-  hipLaunchKernelGGL(k_cast, dim3(grid_for(n)), dim3(TPB), 0, stream(), dp<const void>(src), sd, dp<void>(dst), dd, n);
+  ah::launch_kernel(k_cast, dim3(grid_for(n)), dim3(TPB), 0, dp<const void>(src), sd, dp<void>(dst), dd, n);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
@@ -541,7 +541,7 @@ int32_t ah_check_finite(ah_ptr x, uint64_t n, ah_ptr out_flag) {
   if (rc) return rc;
   if (n == 0) return AH_OK;
   AH_ARG(x != 0, "ah_check_finite: null x");
-  hipLaunchKernelGGL(k_check_finite, dim3(grid_for(n)), dim3(TPB), 0, stream(), dp<const float>(x), n, dp<float>(out_flag));
+  ah::launch_kernel(k_check_finite, dim3(grid_for(n)), dim3(TPB), 0, dp<const float>(x), n, dp<float>(out_flag));
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
@@ -561,7 +561,7 @@ int32_t ah_transpose(ah_ptr a, ah_ptr out, int32_t nd, const int64_t *shape, int
     int64_t R = shape[nd - 2], C = shape[nd - 1], batch = (int64_t)(n / (uint64_t)(R * C));
     if (batch <= 65535) {
       dim3 grid((unsigned)cdiv(C, 32), (unsigned)cdiv(R, 32), (unsigned)batch);
-      hipLaunchKernelGGL(k_transpose_last2, grid, dim3(32, 8), 0, stream(), dp<const uint32_t>(a), dp<uint32_t>(out), R, C);
+      ah::launch_kernel(k_transpose_last2, grid, dim3(32, 8), 0, dp<const uint32_t>(a), dp<uint32_t>(out), R, C);
       AH_LAUNCH_CHECK();
       return AH_OK;
     }
@@ -571,7 +571,7 @@ int32_t ah_transpose(ah_ptr a, ah_ptr out, int32_t nd, const int64_t *shape, int
   Gather6 g; g.nd = nd; g.offset = 0;
   for (int i = 0; i < nd; i++) { g.shape[i] = shape[i]; g.stride[i] = st[i]; }
   { int64_t t = g.shape[d0]; g.shape[d0] = g.shape[d1]; g.shape[d1] = t; t = g.stride[d0]; g.stride[d0] = g.stride[d1]; g.stride[d1] = t; }
-  hipLaunchKernelGGL(k_gather, dim3(grid_for(n)), dim3(TPB), 0, stream(), dp<const uint32_t>(a), dp<uint32_t>(out), n, g);
+  ah::launch_kernel(k_gather, dim3(grid_for(n)), dim3(TPB), 0, dp<const uint32_t>(a), dp<uint32_t>(out), n, g);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
@@ -589,7 +589,7 @@ int32_t ah_slice(ah_ptr a, ah_ptr out, int32_t nd, const int64_t *shape, const i
   uint64_t n = (uint64_t)prod(nd, g.shape);
   if (n == 0) return AH_OK;
   AH_ARG(a && out, "ah_slice: null operand");
-  hipLaunchKernelGGL(k_gather, dim3(grid_for(n)), dim3(TPB), 0, stream(), dp<const uint32_t>(a), dp<uint32_t>(out), n, g);
+  ah::launch_kernel(k_gather, dim3(grid_for(n)), dim3(TPB), 0, dp<const uint32_t>(a), dp<uint32_t>(out), n, g);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
@@ -610,7 +610,7 @@ int32_t ah_scatter_slice(ah_ptr grad, ah_ptr out, int32_t nd, const int64_t *gsh
   if (rc) return rc;
   if (n == 0) return AH_OK;
   AH_ARG(grad != 0, "ah_scatter_slice: null grad");
-  hipLaunchKernelGGL(k_scatter, dim3(grid_for(n)), dim3(TPB), 0, stream(), dp<const uint32_t>(grad), dp<uint32_t>(out), n, g);
+  ah::launch_kernel(k_scatter, dim3(grid_for(n)), dim3(TPB), 0, dp<const uint32_t>(grad), dp<uint32_t>(out), n, g);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
@@ -631,7 +631,7 @@ int32_t ah_cat_part(ah_ptr src, ah_ptr dst, int32_t nd, const int64_t *src_shape
   uint64_t n = (uint64_t)prod(nd, src_shape);
   if (n == 0) return AH_OK;
   AH_ARG(src && dst, "ah_cat_part: null operand");
-  hipLaunchKernelGGL(k_scatter, dim3(grid_for(n)), dim3(TPB), 0, stream(), dp<const uint32_t>(src), dp<uint32_t>(dst), n, g);
+  ah::launch_kernel(k_scatter, dim3(grid_for(n)), dim3(TPB), 0, dp<const uint32_t>(src), dp<uint32_t>(dst), n, g);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
@@ -655,7 +655,7 @@ int32_t ah_broadcast(ah_ptr a, ah_ptr out, int32_t nd, const int64_t *out_shape,
   uint64_t n = (uint64_t)prod(nd, out_shape);
   if (n == 0) return AH_OK;
   AH_ARG(a && out, "ah_broadcast: null operand");
-  hipLaunchKernelGGL(k_gather, dim3(grid_for(n)), dim3(TPB), 0, stream(), dp<const uint32_t>(a), dp<uint32_t>(out), n, g);
+  ah::launch_kernel(k_gather, dim3(grid_for(n)), dim3(TPB), 0, dp<const uint32_t>(a), dp<uint32_t>(out), n, g);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }

@@ -253,7 +253,7 @@ int32_t launch_bf16_nt_t(const GemmArgs &ga, int batch, int vec_c) {
   }
   note_gemm_kernel("k_gemm_bf16_nt<%d, %d, %d, %d, %d, %s>", BM, BN, WGM, WGN, EPI, sizeof(OUT) == 4 ? "float" : "unsigned short");
   note_gemm_split(1);
-  hipLaunchKernelGGL(kfn, grid, dim3(256), lds, stream(), ga, vec_c);
+  ah::launch_kernel(kfn, grid, dim3(256), lds, ga, vec_c);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
@@ -277,7 +277,7 @@ int32_t launch_f32_t(const GemmArgs &ga, int batch, int vec_a, int vec_b, int ve
   dim3 grid((unsigned)cdiv(ga.N, F_BN), (unsigned)cdiv(ga.M, F_BM), (unsigned)batch);
   note_gemm_kernel("k_gemm_f32<%d, %d, %s>", LAYOUT, EPI, sizeof(OUT) == 4 ? "float" : "unsigned short");
   note_gemm_split(1);
-  hipLaunchKernelGGL((k_gemm_f32<LAYOUT, EPI, OUT>), grid, dim3(256), 0, stream(), ga, vec_a, vec_b, vec_c);
+  ah::launch_kernel((k_gemm_f32<LAYOUT, EPI, OUT>), grid, dim3(256), 0, ga, vec_a, vec_b, vec_c);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
@@ -469,7 +469,7 @@ int32_t ah_gemm_grouped_run(uint64_t plan, int32_t epilogue) {
     default: rc = gemm_bf16_dma_tn_grouped(tab, p.count, p.blocks, epilogue, p.out_dtype);
   }
   if (rc != AH_OK || p.nparts == 0) return rc;
-  hipLaunchKernelGGL(k_grouped_join, dim3(128, (unsigned)p.nparts), dim3(256), 0, stream(), dp<const JoinPart>(p.parts));
+  ah::launch_kernel(k_grouped_join, dim3(128, (unsigned)p.nparts), dim3(256), 0, dp<const JoinPart>(p.parts));
   AH_LAUNCH_CHECK();
   ah::note_gemm_split(2);
   return AH_OK;
@@ -591,7 +591,7 @@ int32_t ah_gemm(const AhGemm *p) {
     int64_t ldt = (q.k + 7) & ~7ll;
     rc = ah_alloc((uint64_t)q.m * ldt * 2, &ta);
     if (rc) return rc;
-    hipLaunchKernelGGL(k_transpose_u16, dim3((unsigned)cdiv(q.m, 64), (unsigned)cdiv(q.k, 64)), dim3(64, 4), 0, stream(),
+    ah::launch_kernel(k_transpose_u16, dim3((unsigned)cdiv(q.m, 64), (unsigned)cdiv(q.k, 64)), dim3(64, 4), 0, 
                        (const uint16_t *)ga.a, q.lda, dp<uint16_t>(ta), ldt, (int)q.k, (int)q.m);
     AH_LAUNCH_CHECK();
     ga.a = dp<const void>(ta); ga.lda = ldt;
@@ -600,7 +600,7 @@ int32_t ah_gemm(const AhGemm *p) {
     int64_t ldt = (q.k + 7) & ~7ll;
     rc = ah_alloc((uint64_t)q.n * ldt * 2, &tb);
     if (rc) { if (ta) ah_free(ta); return rc; }
-    hipLaunchKernelGGL(k_transpose_u16, dim3((unsigned)cdiv(q.n, 64), (unsigned)cdiv(q.k, 64)), dim3(64, 4), 0, stream(),
+    ah::launch_kernel(k_transpose_u16, dim3((unsigned)cdiv(q.n, 64), (unsigned)cdiv(q.k, 64)), dim3(64, 4), 0, 
                        (const uint16_t *)ga.b, q.ldb, dp<uint16_t>(tb), ldt, (int)q.k, (int)q.n);
     AH_LAUNCH_CHECK();
     ga.b = dp<const void>(tb); ga.ldb = ldt;

@@ -227,7 +227,7 @@ int32_t launch(const GemmArgs &ga, int batch, int out_dtype) {
   }
   note_gemm_kernel("k_gemm_bf16<%d, %d, %d, %d, %s, %s>", BM, BN, WGM, WGN, AKM ? "true" : "false", BKM ? "true" : "false");
   note_gemm_split(ga.nsplit);
-  hipLaunchKernelGGL(kfn, grid, dim3(NT), lds, stream(), ga, out_dtype == AH_F32 ? 1 : 0);
+  ah::launch_kernel(kfn, grid, dim3(NT), lds, ga, out_dtype == AH_F32 ? 1 : 0);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
@@ -265,7 +265,7 @@ namespace ah {
 int32_t splitk_reduce(const float *ws, float *c, int nsplit, int M, int N, int64_t ldc, bool accumulate) {
   int64_t n4 = (int64_t)M * N / 4;
   int blocks = (int)(cdiv(n4, 256) < 4096 ? cdiv(n4, 256) : 4096);
-  hipLaunchKernelGGL(k_splitk_reduce, dim3(blocks), dim3(256), 0, stream(), ws, c, nsplit, M, N, ldc, accumulate ? 1 : 0);
+  ah::launch_kernel(k_splitk_reduce, dim3(blocks), dim3(256), 0, ws, c, nsplit, M, N, ldc, accumulate ? 1 : 0);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }

@@ -566,7 +566,7 @@ static int32_t launch_ln(ah_ptr x, ah_ptr w, ah_ptr b, ah_ptr out, int64_t rows,
   dim3 grid((unsigned)cdiv(rows, WPB)), blk(TPB);
   bool vec = (dim % 4 == 0) && dim <= 2048 && aligned16(x) && aligned16(w) && aligned16(b) && (sizeof(OUT) == 2 || aligned16(out));
   int nvl = vec ? (int)cdiv(dim / 4, 64) : 0;
-#define LN_CASE(NV) hipLaunchKernelGGL((k_layernorm<NV, OUT>), grid, blk, 0, stream(), dp<const float>(x), dp<const float>(w), dp<const float>(b), dp<OUT>(out), rows, (int)dim, eps)
+#define LN_CASE(NV) ah::launch_kernel((k_layernorm<NV, OUT>), grid, blk, 0, dp<const float>(x), dp<const float>(w), dp<const float>(b), dp<OUT>(out), rows, (int)dim, eps)
   switch (nvl) {
     case 1: LN_CASE(1); break;
     case 2: LN_CASE(2); break;
@@ -590,9 +590,9 @@ int32_t ah_embedding(ah_ptr weight, ah_ptr idx, ah_ptr out, int64_t n_idx, int64
   AH_ARG(weight && idx && out, "ah_embedding: null operand");
   dim3 grid((unsigned)cdiv(n_idx, WPB));
   if (out_dtype == AH_F32)
-    hipLaunchKernelGGL(k_embedding<float>, grid, dim3(TPB), 0, stream(), dp<const float>(weight), dp<const int32_t>(idx), dp<float>(out), n_idx, dim, vocab);
+    ah::launch_kernel(k_embedding<float>, grid, dim3(TPB), 0, dp<const float>(weight), dp<const int32_t>(idx), dp<float>(out), n_idx, dim, vocab);
   else
-    hipLaunchKernelGGL(k_embedding<uint16_t>, grid, dim3(TPB), 0, stream(), dp<const float>(weight), dp<const int32_t>(idx), dp<uint16_t>(out), n_idx, dim, vocab);
+    ah::launch_kernel(k_embedding<uint16_t>, grid, dim3(TPB), 0, dp<const float>(weight), dp<const int32_t>(idx), dp<uint16_t>(out), n_idx, dim, vocab);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
@@ -602,7 +602,7 @@ int32_t ah_embedding_tok_pos(ah_ptr wte, ah_ptr wpe, ah_ptr tok, ah_ptr out, int
   if (n_idx == 0 || dim == 0) return AH_OK;
   AH_ARG(wte && wpe && tok && out && T > 0, "ah_embedding_tok_pos: null operand");
   AH_ARG(aligned16(wte) && aligned16(wpe) && aligned16(out), "ah_embedding_tok_pos: operands must be 16-byte aligned");
-  hipLaunchKernelGGL(k_embedding_tok_pos, dim3((unsigned)cdiv(n_idx, WPB)), dim3(TPB), 0, stream(), dp<const float>(wte),
+  ah::launch_kernel(k_embedding_tok_pos, dim3((unsigned)cdiv(n_idx, WPB)), dim3(TPB), 0, dp<const float>(wte),
                      dp<const float>(wpe), dp<const int32_t>(tok), dp<float>(out), n_idx, T, dim, vocab);
   AH_LAUNCH_CHECK();
   return AH_OK;
@@ -615,7 +615,7 @@ int32_t ah_token_windows(ah_ptr corpus, int64_t n_tokens, ah_ptr starts, int64_t
   AH_ARG(n_tokens > 0, "ah_token_windows: empty corpus");
   AH_ARG(corpus && starts && inputs && targets, "ah_token_windows: null operand");
   unsigned bx = (unsigned)(cdiv(T, 256) < 64 ? cdiv(T, 256) : 64);
-  hipLaunchKernelGGL(k_token_windows, dim3(bx, (unsigned)batch), dim3(256), 0, stream(), dp<const int32_t>(corpus), n_tokens,
+  ah::launch_kernel(k_token_windows, dim3(bx, (unsigned)batch), dim3(256), 0, dp<const int32_t>(corpus), n_tokens,
                      dp<const int64_t>(starts), T, dp<int32_t>(inputs), dp<int32_t>(targets));
   AH_LAUNCH_CHECK();
   return AH_OK;
@@ -628,10 +628,10 @@ int32_t ah_embedding_bwd(ah_ptr idx, ah_ptr grad_out, ah_ptr grad_w, int64_t n_i
   if (n_idx == 0 || dim == 0) return AH_OK;
   AH_ARG(idx && grad_out, "ah_embedding_bwd: null operand");
   if (cdiv(n_idx, EB_POS) < (1ll << 31) && cdiv(dim, 1024) <= 65535)
-    hipLaunchKernelGGL(k_embedding_bwd_blocks, dim3((unsigned)cdiv(n_idx, EB_POS), (unsigned)cdiv(dim, 1024)), dim3(1024), 0, stream(),
+    ah::launch_kernel(k_embedding_bwd_blocks, dim3((unsigned)cdiv(n_idx, EB_POS), (unsigned)cdiv(dim, 1024)), dim3(1024), 0, 
                        dp<const int32_t>(idx), dp<const float>(grad_out), dp<float>(grad_w), n_idx, dim, vocab);
   else
-    hipLaunchKernelGGL(k_embedding_bwd, dim3((unsigned)cdiv(n_idx, WPB)), dim3(TPB), 0, stream(), dp<const int32_t>(idx),
+    ah::launch_kernel(k_embedding_bwd, dim3((unsigned)cdiv(n_idx, WPB)), dim3(TPB), 0, dp<const int32_t>(idx),
                        dp<const float>(grad_out), dp<float>(grad_w), n_idx, dim, vocab);
   AH_LAUNCH_CHECK();
   return AH_OK;
@@ -642,7 +642,7 @@ int32_t ah_pos_embedding_bwd(ah_ptr grad_out, ah_ptr grad_wpe, int64_t batch, in
   int64_t td = T * dim;
   if (td == 0) return AH_OK;
   AH_ARG(grad_out && grad_wpe, "ah_pos_embedding_bwd: null operand");
-  hipLaunchKernelGGL(k_pos_embedding_bwd, dim3((unsigned)cdiv(td, TPB)), dim3(TPB), 0, stream(), dp<const float>(grad_out),
+  ah::launch_kernel(k_pos_embedding_bwd, dim3((unsigned)cdiv(td, TPB)), dim3(TPB), 0, dp<const float>(grad_out),
                      dp<float>(grad_wpe), batch, td, accumulate);
   AH_LAUNCH_CHECK();
   return AH_OK;
@@ -680,7 +680,7 @@ static int32_t ln_bwd_launch(ah_ptr x, ah_ptr w, ah_ptr grad_out, int32_t grad_d
              (dx_bf16 % 8 == 0) && (grad_dtype == AH_BF16 || aligned16(grad_out));
   if (vec) {
     int nvl = (int)cdiv(dim / 4, 64);
-#define LNB_CASE(NV, GT) hipLaunchKernelGGL((k_layernorm_bwd_vec<NV, GT>), dim3(nblk), dim3(TPB), lds, stream(), dp<const float>(x), dp<const float>(w), \
+#define LNB_CASE(NV, GT) ah::launch_kernel((k_layernorm_bwd_vec<NV, GT>), dim3(nblk), dim3(TPB), lds, dp<const float>(x), dp<const float>(w), \
       dp<const GT>(grad_out), dp<const float>(residual_grad), dp<float>(dx), dp<uint16_t>(dx_bf16), part_dw, part_db, rows, (int)dim, eps)
 #define LNB_SWITCH(GT) switch (nvl) { case 1: LNB_CASE(1, GT); break; case 2: LNB_CASE(2, GT); break; case 3: LNB_CASE(3, GT); break; \
       case 4: LNB_CASE(4, GT); break; case 5: case 6: LNB_CASE(6, GT); break; default: LNB_CASE(8, GT); break; }
@@ -688,10 +688,10 @@ static int32_t ln_bwd_launch(ah_ptr x, ah_ptr w, ah_ptr grad_out, int32_t grad_d
 #undef LNB_SWITCH
 #undef LNB_CASE
   } else if (grad_dtype == AH_F32)
-    hipLaunchKernelGGL(k_layernorm_bwd<float>, dim3(nblk), dim3(TPB), lds, stream(), dp<const float>(x), dp<const float>(w),
+    ah::launch_kernel(k_layernorm_bwd<float>, dim3(nblk), dim3(TPB), lds, dp<const float>(x), dp<const float>(w),
                        dp<const float>(grad_out), dp<const float>(residual_grad), dp<float>(dx), dp<uint16_t>(dx_bf16), part_dw, part_db, rows, (int)dim, eps);
   else
-    hipLaunchKernelGGL(k_layernorm_bwd<uint16_t>, dim3(nblk), dim3(TPB), lds, stream(), dp<const float>(x), dp<const float>(w),
+    ah::launch_kernel(k_layernorm_bwd<uint16_t>, dim3(nblk), dim3(TPB), lds, dp<const float>(x), dp<const float>(w),
                        dp<const uint16_t>(grad_out), dp<const float>(residual_grad), dp<float>(dx), dp<uint16_t>(dx_bf16), part_dw, part_db, rows, (int)dim, eps);
   AH_LAUNCH_CHECK();
   return AH_OK;
@@ -714,7 +714,7 @@ int32_t ah_layernorm_bwd(ah_ptr x, ah_ptr w, ah_ptr grad_out, int32_t grad_dtype
   if (!part) return fail(AH_ERR_OOM, "ah_layernorm_bwd: no scratch");
   int32_t rc = ln_bwd_launch(x, w, grad_out, grad_dtype, residual_grad, dx, dx_bf16, part, nblk, rows, dim, eps);
   if (rc) return rc;
-  hipLaunchKernelGGL(k_colsum_partials, dim3((unsigned)cdiv(dim, 32)), dim3(1024), 0, stream(), part, part + (size_t)nblk * dim, nblk, (int)dim,
+  ah::launch_kernel(k_colsum_partials, dim3((unsigned)cdiv(dim, 32)), dim3(1024), 0, part, part + (size_t)nblk * dim, nblk, (int)dim,
                      dp<float>(dw), dp<float>(db), accumulate);
   AH_LAUNCH_CHECK();
   return AH_OK;
@@ -750,7 +750,7 @@ int32_t ah_layernorm_colsums(const AhColsumJob *jobs, int32_t count) {
       tab.j[i] = ColsumJob{dp<const float>(q.partials), dp<float>(q.dw), dp<float>(q.db), ln_bwd_blocks(q.rows), (int)q.dim, q.accumulate, 0};
       if (q.dim > max_dim) max_dim = q.dim;
     }
-    hipLaunchKernelGGL(k_colsum_partials_batched, dim3((unsigned)cdiv(max_dim, 32), (unsigned)n), dim3(1024), 0, stream(), tab);
+    ah::launch_kernel(k_colsum_partials_batched, dim3((unsigned)cdiv(max_dim, 32), (unsigned)n), dim3(1024), 0, tab);
     AH_LAUNCH_CHECK();
   }
   return AH_OK;
@@ -766,11 +766,11 @@ int32_t ah_cross_entropy(ah_ptr logits, int32_t dtype, ah_ptr targets, ah_ptr lo
   float *rows = (float *)scratch(sizeof(float) * (size_t)n);
   if (!rows) return fail(AH_ERR_OOM, "ah_cross_entropy: no scratch");
   if (dtype == AH_F32)
-    hipLaunchKernelGGL(k_ce_fwd<float>, dim3((unsigned)n), dim3(TPB), 0, stream(), dp<const float>(logits), dp<const int32_t>(targets), rows, dp<float>(lse_out), c);
+    ah::launch_kernel(k_ce_fwd<float>, dim3((unsigned)n), dim3(TPB), 0, dp<const float>(logits), dp<const int32_t>(targets), rows, dp<float>(lse_out), c);
   else
-    hipLaunchKernelGGL(k_ce_fwd<uint16_t>, dim3((unsigned)n), dim3(TPB), 0, stream(), dp<const uint16_t>(logits), dp<const int32_t>(targets), rows, dp<float>(lse_out), c);
+    ah::launch_kernel(k_ce_fwd<uint16_t>, dim3((unsigned)n), dim3(TPB), 0, dp<const uint16_t>(logits), dp<const int32_t>(targets), rows, dp<float>(lse_out), c);
   AH_LAUNCH_CHECK();
-  hipLaunchKernelGGL(k_mean_rows, dim3(1), dim3(TPB), 0, stream(), rows, n, dp<float>(loss_out));
+  ah::launch_kernel(k_mean_rows, dim3(1), dim3(TPB), 0, rows, n, dp<float>(loss_out));
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
@@ -790,10 +790,10 @@ int32_t ah_cross_entropy_bwd(ah_ptr logits, int32_t dtype, ah_ptr targets, ah_pt
     size_t esz = dtype == AH_F32 ? 4 : 2;
     ah_ptr lg = logits + (uint64_t)(r0 * c) * esz, dl = dlogits + (uint64_t)(r0 * c) * esz;
     if (dtype == AH_F32)
-      hipLaunchKernelGGL(k_ce_bwd<float>, dim3(gx, (unsigned)nr), dim3(TPB), 0, stream(), dp<const float>(lg),
+      ah::launch_kernel(k_ce_bwd<float>, dim3(gx, (unsigned)nr), dim3(TPB), 0, dp<const float>(lg),
                          dp<const int32_t>(targets) + r0, dp<const float>(lse) + r0, dp<const float>(g_scalar), g_mul, dp<float>(dl), n, c);
     else
-      hipLaunchKernelGGL(k_ce_bwd<uint16_t>, dim3(gx, (unsigned)nr), dim3(TPB), 0, stream(), dp<const uint16_t>(lg),
+      ah::launch_kernel(k_ce_bwd<uint16_t>, dim3(gx, (unsigned)nr), dim3(TPB), 0, dp<const uint16_t>(lg),
                          dp<const int32_t>(targets) + r0, dp<const float>(lse) + r0, dp<const float>(g_scalar), g_mul, dp<uint16_t>(dl), n, c);
     AH_LAUNCH_CHECK();
   }
@@ -815,10 +815,10 @@ int32_t ah_cross_entropy_fwd_bwd(ah_ptr logits, int32_t dtype, ah_ptr targets, a
   }
   float *rows = (float *)scratch(sizeof(float) * (size_t)n);
   if (!rows) return fail(AH_ERR_OOM, "ah_cross_entropy_fwd_bwd: no scratch");
-  hipLaunchKernelGGL(k_ce_fwd_bwd, dim3((unsigned)n), dim3(256), 0, stream(), dp<const uint16_t>(logits), dp<const int32_t>(targets), rows,
+  ah::launch_kernel(k_ce_fwd_bwd, dim3((unsigned)n), dim3(256), 0, dp<const uint16_t>(logits), dp<const int32_t>(targets), rows,
                      dp<float>(lse_out), dp<const float>(g_scalar), g_mul, dp<uint16_t>(dlogits), n, c);
   AH_LAUNCH_CHECK();
-  hipLaunchKernelGGL(k_mean_rows, dim3(1), dim3(TPB), 0, stream(), rows, n, dp<float>(loss_out));
+  ah::launch_kernel(k_mean_rows, dim3(1), dim3(TPB), 0, rows, n, dp<float>(loss_out));
   AH_LAUNCH_CHECK();
   return AH_OK;
 }

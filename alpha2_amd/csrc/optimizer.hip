@@ -204,12 +204,12 @@ template <bool FLAT>
 int32_t adafactor_tail(ah_ptr p, ah_ptr g, ah_ptr vr, ah_ptr vc, ah_ptr v, uint64_t n, int64_t cols, const AhAdafactor &h, double *ws) {
   int nblk = (int)(cdiv((int64_t)n, TPB) < 1024 ? cdiv((int64_t)n, TPB) : 1024);
   double *part = ws + 2;
-  hipLaunchKernelGGL((k_af_update_sq<FLAT>), dim3(nblk), dim3(TPB), 0, stream(), dp<const float>(g), dp<const float>(vr), dp<const float>(vc),
+  ah::launch_kernel((k_af_update_sq<FLAT>), dim3(nblk), dim3(TPB), 0, dp<const float>(g), dp<const float>(vr), dp<const float>(vc),
                      dp<float>(v), n, cols, h, ws, part);
   AH_LAUNCH_CHECK();
-  hipLaunchKernelGGL(k_af_step_scale, dim3(1), dim3(64), 0, stream(), part, nblk, n, h, ws);
+  ah::launch_kernel(k_af_step_scale, dim3(1), dim3(64), 0, part, nblk, n, h, ws);
   AH_LAUNCH_CHECK();
-  hipLaunchKernelGGL((k_af_apply<FLAT>), dim3((unsigned)cdiv((int64_t)n, TPB)), dim3(TPB), 0, stream(), dp<float>(p), dp<const float>(g),
+  ah::launch_kernel((k_af_apply<FLAT>), dim3((unsigned)cdiv((int64_t)n, TPB)), dim3(TPB), 0, dp<float>(p), dp<const float>(g),
                      dp<const float>(vr), dp<const float>(vc), dp<const float>(v), n, cols, h, ws);
   AH_LAUNCH_CHECK();
   return AH_OK;
@@ -225,7 +225,7 @@ int32_t ah_lion(ah_ptr p, ah_ptr g, ah_ptr m, uint64_t n, const AhLion *h) {
   if (n == 0) return AH_OK;
   AH_ARG(p && g && m, "ah_lion: null operand");
   AH_ARG(n < ((uint64_t)1 << 39), "ah_lion: tensor too large");
-  hipLaunchKernelGGL(k_lion, dim3((unsigned)cdiv((int64_t)n, TPB)), dim3(TPB), 0, stream(), dp<float>(p), dp<const float>(g), dp<float>(m), n, *h);
+  ah::launch_kernel(k_lion, dim3((unsigned)cdiv((int64_t)n, TPB)), dim3(TPB), 0, dp<float>(p), dp<const float>(g), dp<float>(m), n, *h);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
@@ -235,7 +235,7 @@ int32_t ah_sgd(ah_ptr p, ah_ptr g, uint64_t n, double lr, double grad_scale) {
   if (n == 0) return AH_OK;
   AH_ARG(p && g, "ah_sgd: null operand");
   AH_ARG(n < ((uint64_t)1 << 39), "ah_sgd: tensor too large");
-  hipLaunchKernelGGL(k_sgd, dim3((unsigned)cdiv((int64_t)n, TPB)), dim3(TPB), 0, stream(), dp<float>(p), dp<const float>(g), n, lr, grad_scale);
+  ah::launch_kernel(k_sgd, dim3((unsigned)cdiv((int64_t)n, TPB)), dim3(TPB), 0, dp<float>(p), dp<const float>(g), n, lr, grad_scale);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
@@ -249,11 +249,11 @@ int32_t ah_adafactor_2d(ah_ptr p, ah_ptr g, ah_ptr vr, ah_ptr vc, int64_t rows, 
   AH_ARG(rows < ((int64_t)1 << 31) && cols < ((int64_t)1 << 31), "ah_adafactor_2d: shape too large");
   double *ws = (double *)scratch(sizeof(double) * (2 + 1024));
   if (!ws) return fail(AH_ERR_OOM, "ah_adafactor_2d: no scratch");
-  hipLaunchKernelGGL(k_af_rows, dim3((unsigned)rows), dim3(TPB), 0, stream(), dp<const float>(g), dp<float>(vr), cols, *h);
+  ah::launch_kernel(k_af_rows, dim3((unsigned)rows), dim3(TPB), 0, dp<const float>(g), dp<float>(vr), cols, *h);
   AH_LAUNCH_CHECK();
-  hipLaunchKernelGGL(k_af_cols, dim3((unsigned)cdiv(cols, 64)), dim3(64), 0, stream(), dp<const float>(g), dp<float>(vc), rows, cols, *h);
+  ah::launch_kernel(k_af_cols, dim3((unsigned)cdiv(cols, 64)), dim3(64), 0, dp<const float>(g), dp<float>(vc), rows, cols, *h);
   AH_LAUNCH_CHECK();
-  hipLaunchKernelGGL(k_af_vrmean, dim3(1), dim3(TPB), 0, stream(), dp<const float>(vr), rows, h->eps, ws);
+  ah::launch_kernel(k_af_vrmean, dim3(1), dim3(TPB), 0, dp<const float>(vr), rows, h->eps, ws);
   AH_LAUNCH_CHECK();
   return adafactor_tail<false>(p, g, vr, vc, 0, (uint64_t)rows * (uint64_t)cols, cols, *h, ws);
 }
@@ -280,7 +280,7 @@ int32_t ah_adamw(ah_ptr p, ah_ptr g, ah_ptr m, ah_ptr v, uint64_t n, const AhAda
   // one float4 group per thread: measured 5.4 TB/s against 4.3 TB/s for a grid of 16 blocks per CU striding over the array
   int64_t cap = (int64_t)1 << 22;
   if (blocks > cap) blocks = cap;
-  hipLaunchKernelGGL(k_adamw, dim3((unsigned)blocks), dim3(TPB), 0, stream(), dp<float>(p), dp<const float>(g), dp<float>(m),
+  ah::launch_kernel(k_adamw, dim3((unsigned)blocks), dim3(TPB), 0, dp<float>(p), dp<const float>(g), dp<float>(m),
                      dp<float>(v), n, *h, dp<const AhAdamW>(dev_hyper), dp<const float>(dev_scale), dp<uint16_t>(bf16_shadow), vec);
   AH_LAUNCH_CHECK();
   return AH_OK;
@@ -289,7 +289,7 @@ int32_t ah_adamw(ah_ptr p, ah_ptr g, ah_ptr m, ah_ptr v, uint64_t n, const AhAda
 int32_t ah_clip_coef(ah_ptr sumsq, float grad_scale, float clip, ah_ptr out2) {
   AH_REQUIRE_READY();
   AH_ARG(sumsq && out2, "ah_clip_coef: null operand");
-  hipLaunchKernelGGL(k_clip_coef, dim3(1), dim3(64), 0, stream(), dp<const float>(sumsq), grad_scale, clip, dp<float>(out2));
+  ah::launch_kernel(k_clip_coef, dim3(1), dim3(64), 0, dp<const float>(sumsq), grad_scale, clip, dp<float>(out2));
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
@@ -299,7 +299,7 @@ int32_t ah_step_guard(ah_ptr sumsq, ah_ptr loss, float grad_scale, float clip, d
   AH_REQUIRE_READY();
   AH_ARG(sumsq && state_f64x3 && dev_hyper && out3, "ah_step_guard: null operand");
   AH_ARG((state_f64x3 & 7u) == 0, "ah_step_guard: state must be 8-byte aligned");
-  hipLaunchKernelGGL(k_step_guard, dim3(1), dim3(64), 0, stream(), dp<const float>(sumsq), dp<const float>(loss), grad_scale, clip,
+  ah::launch_kernel(k_step_guard, dim3(1), dim3(64), 0, dp<const float>(sumsq), dp<const float>(loss), grad_scale, clip,
                      beta1, beta2, dp<double>(state_f64x3), dp<AhAdamW>(dev_hyper), dp<float>(out3));
   AH_LAUNCH_CHECK();
   return AH_OK;

@@ -181,11 +181,11 @@ int32_t ah_sum_axis(ah_ptr a, ah_ptr out, int64_t outer, int64_t dim, int64_t in
   AH_ARG(a && out, "ah_sum_axis: null operand");
   if (dim == 0) return ah_fill_f32(out, 0.f, (uint64_t)lines);
   if (inner > 1 && lines >= 4096) {
-    hipLaunchKernelGGL(k_sum_strided, dim3((unsigned)cdiv(lines, TPB)), dim3(TPB), 0, stream(), dp<const float>(a),
+    ah::launch_kernel(k_sum_strided, dim3((unsigned)cdiv(lines, TPB)), dim3(TPB), 0, dp<const float>(a),
                        dp<float>(out), outer, dim, inner, mean);
   } else {
     AH_ARG(lines < (int64_t(1) << 31), "ah_sum_axis: too many lines");
-    hipLaunchKernelGGL(k_sum_lines, dim3((unsigned)lines), dim3(TPB), 0, stream(), dp<const float>(a), dp<float>(out), dim, inner, mean);
+    ah::launch_kernel(k_sum_lines, dim3((unsigned)lines), dim3(TPB), 0, dp<const float>(a), dp<float>(out), dim, inner, mean);
   }
   AH_LAUNCH_CHECK();
   return AH_OK;
@@ -199,10 +199,10 @@ static int32_t full_reduce(ah_ptr a, uint64_t n, ah_ptr out, double div, int sq,
   int nb = partial_blocks(n);
   double *partial = (double *)scratch(sizeof(double) * (size_t)nb);
   if (!partial) return fail(AH_ERR_OOM, "%s: no scratch", who);
-  if (sq) hipLaunchKernelGGL(k_partial_sum<1>, dim3(nb), dim3(TPB), 0, stream(), dp<const float>(a), n, partial);
-  else hipLaunchKernelGGL(k_partial_sum<0>, dim3(nb), dim3(TPB), 0, stream(), dp<const float>(a), n, partial);
+  if (sq) ah::launch_kernel(k_partial_sum<1>, dim3(nb), dim3(TPB), 0, dp<const float>(a), n, partial);
+  else ah::launch_kernel(k_partial_sum<0>, dim3(nb), dim3(TPB), 0, dp<const float>(a), n, partial);
   AH_LAUNCH_CHECK();
-  hipLaunchKernelGGL(k_final_sum, dim3(1), dim3(TPB), 0, stream(), partial, nb, dp<float>(out), div);
+  ah::launch_kernel(k_final_sum, dim3(1), dim3(TPB), 0, partial, nb, dp<float>(out), div);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
@@ -222,9 +222,9 @@ int32_t ah_sum_sq_static(ah_ptr x, uint64_t n, ah_ptr out) {
   double *partial = g_static_partials_ptr[current_device()];
   if (!partial) return fail(AH_ERR_STATE, "ah_sum_sq_static: static scratch of device %d was not set up", current_device());
   // partial[0, nb) is written in full by the first kernel before the second reads exactly that range: nothing to clear.
-  hipLaunchKernelGGL(k_partial_sum<1>, dim3(nb), dim3(TPB), 0, stream(), dp<const float>(x), n, partial);
+  ah::launch_kernel(k_partial_sum<1>, dim3(nb), dim3(TPB), 0, dp<const float>(x), n, partial);
   AH_LAUNCH_CHECK();
-  hipLaunchKernelGGL(k_final_sum, dim3(1), dim3(TPB), 0, stream(), partial, nb, dp<float>(out), 1.0);
+  ah::launch_kernel(k_final_sum, dim3(1), dim3(TPB), 0, partial, nb, dp<float>(out), 1.0);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
@@ -235,7 +235,7 @@ int32_t ah_softmax(ah_ptr a, ah_ptr out, int64_t outer, int64_t dim, int64_t inn
   if (lines == 0 || dim == 0) return AH_OK;
   AH_ARG(a && out, "ah_softmax: null operand");
   AH_ARG(lines < (int64_t(1) << 31), "ah_softmax: too many lines");
-  hipLaunchKernelGGL(k_softmax, dim3((unsigned)lines), dim3(TPB), 0, stream(), dp<const float>(a), dp<float>(out), dim, inner, log_softmax);
+  ah::launch_kernel(k_softmax, dim3((unsigned)lines), dim3(TPB), 0, dp<const float>(a), dp<float>(out), dim, inner, log_softmax);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
@@ -244,7 +244,7 @@ int32_t ah_softmax_bwd(ah_ptr s, ah_ptr g, ah_ptr out, int64_t rows, int64_t dim
   if (rows == 0 || dim == 0) return AH_OK;
   AH_ARG(s && g && out, "ah_softmax_bwd: null operand");
   AH_ARG(rows < (int64_t(1) << 31), "ah_softmax_bwd: too many rows");
-  hipLaunchKernelGGL(k_softmax_bwd, dim3((unsigned)rows), dim3(TPB), 0, stream(), dp<const float>(s), dp<const float>(g), dp<float>(out), dim);
+  ah::launch_kernel(k_softmax_bwd, dim3((unsigned)rows), dim3(TPB), 0, dp<const float>(s), dp<const float>(g), dp<float>(out), dim);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
@@ -255,7 +255,7 @@ int32_t ah_argmax(ah_ptr a, ah_ptr out, int64_t outer, int64_t dim, int64_t inne
   AH_ARG(a && out, "ah_argmax: null operand");
   AH_ARG(dim < (int64_t(1) << 31), "ah_argmax: axis longer than an i32 index");
   AH_ARG(lines < (int64_t(1) << 31), "ah_argmax: too many lines");
-  hipLaunchKernelGGL(k_argmax, dim3((unsigned)lines), dim3(TPB), 0, stream(), dp<const float>(a), dp<int32_t>(out), dim, inner);
+  ah::launch_kernel(k_argmax, dim3((unsigned)lines), dim3(TPB), 0, dp<const float>(a), dp<int32_t>(out), dim, inner);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }

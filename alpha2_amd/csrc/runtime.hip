@@ -3,11 +3,14 @@
 // addon (packages/helios/native/helios_vk.c:818-934 slab allocator + slot tables, :1068-1125 timeline
 // submit/wait, :3192-3419 batch execute) with the HIP-native equivalents.
 #include "common.h"
+#include <algorithm>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <cmath>
 #include <map>
+#include <string>
 #include <unordered_map>
 #include <vector>
 
@@ -20,6 +23,35 @@ struct Graph {
   hipGraphExec_t exec = nullptr;
   std::vector<Block> reserved;      // blocks whose addresses are baked into the graph
 };
+
+// ---- step plans: the kernel launches of one training step, recorded once as hipGraph segments and replayed ----
+struct StepOp {
+  const void *func = nullptr;
+  dim3 grid, block;
+  unsigned shmem = 0;
+  std::vector<uint32_t> off, size;     // per kernel argument: offset into blob, byte size
+  std::vector<char> blob;              // the argument values of the most recent step
+  hipGraphNode_t node = nullptr;
+  void fill_ptrs(std::vector<void *> &ptrs) {
+    ptrs.resize(off.size() + 1);
+    for (size_t i = 0; i < off.size(); i++) ptrs[i] = blob.data() + off[i];
+    ptrs[off.size()] = nullptr;
+  }
+};
+struct StepSeg {                       // the launches between two points where the host needs the stream
+  std::vector<StepOp> ops;
+  std::string boundary;                // what ended the segment: "ah_download", "ah_sync", ..., "ah_step_end"
+  hipGraph_t graph = nullptr;
+  hipGraphExec_t exec = nullptr;
+  hipEvent_t done = nullptr;           // recorded after every launch of exec
+};
+struct PinnedSlot { char *host = nullptr; void *dev = nullptr; size_t bytes = 0; size_t seg = 0; };
+struct StepPlan {
+  std::vector<StepSeg> segs;
+  std::vector<PinnedSlot> slots;       // one per ah_upload of the step, in call order
+  bool complete = false, broken = false;
+};
+enum { STEP_OFF = 0, STEP_RECORD = 1, STEP_VERIFY = 2, STEP_EAGER = 3 };
 
 struct Context {
   bool inited = false;
@@ -46,6 +78,16 @@ struct Context {
   char *ring = nullptr;
   unsigned ring_next = 0;
   hipEvent_t ring_ev[2] = {nullptr, nullptr};
+  // step plans
+  int step_mode = STEP_OFF;
+  bool step_capture_open = false, step_fellback = false;
+  uint64_t step_key = 0;
+  StepPlan *plan = nullptr;
+  size_t seg = 0, op = 0, slot = 0;
+  std::vector<char> seg_waited;          // per segment: its previous launch is known to have finished (this step)
+  std::map<uint64_t, StepPlan> plans;
+  uint64_t steps_recorded = 0, steps_replayed = 0, steps_fallback = 0, step_node_updates = 0;
+  char step_why[256] = "";
 };
 Context g;
 
@@ -87,6 +129,209 @@ void *scratch(size_t bytes) {
   g.scratch_bytes = bytes;
   return g.scratch;
 }
+
+// ------------------------------------------------------------------------------------------ step plans
+namespace {
+constexpr size_t STEP_UPLOAD_MAX = size_t(16) << 20;     // larger uploads inside a step are a boundary, not a node
+// A segment is closed after this many launches even when the host does not need the stream: on replay the graph of a
+// chunk is launched as soon as its last launch has been verified, so the device works on chunk k while the host is still
+// issuing (verifying) chunk k+1 -- the overlap eager execution has, at graph-launch cost.
+size_t step_chunk() {
+  static const size_t n = [] { const char *e = getenv("AH_STEP_CHUNK"); long v = e ? atol(e) : 0; return v > 0 ? (size_t)v : (size_t)32; }();
+  return n;
+}
+
+__global__ void k_step_copy(char *__restrict__ dst, const char *__restrict__ src, uint64_t bytes) {
+  uint64_t tid = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x, stride = (uint64_t)gridDim.x * blockDim.x;
+  if ((((uintptr_t)dst | (uintptr_t)src) & 15u) == 0) {
+    uint64_t n16 = bytes >> 4;
+    for (uint64_t i = tid; i < n16; i += stride) reinterpret_cast<uint4 *>(dst)[i] = reinterpret_cast<const uint4 *>(src)[i];
+    for (uint64_t i = (n16 << 4) + tid; i < bytes; i += stride) dst[i] = src[i];
+  } else {
+    for (uint64_t i = tid; i < bytes; i += stride) dst[i] = src[i];
+  }
+}
+void step_copy(void *dst, const void *src, uint64_t bytes) {
+  uint64_t blocks = (bytes / 16 + 255) / 256;
+  if (blocks < 1) blocks = 1;
+  if (blocks > 4096) blocks = 4096;
+  ah::launch_kernel(k_step_copy, dim3((unsigned)blocks), dim3(256), 0, (char *)dst, (const char *)src, bytes);
+}
+
+void plan_destroy(StepPlan &p) {
+  for (auto &sg : p.segs) {
+    if (sg.done) { (void)hipEventSynchronize(sg.done); (void)hipEventDestroy(sg.done); }
+    if (sg.exec) (void)hipGraphExecDestroy(sg.exec);
+    if (sg.graph) (void)hipGraphDestroy(sg.graph);
+  }
+  for (auto &sl : p.slots) if (sl.host) (void)hipHostFree(sl.host);
+  p = StepPlan();
+}
+void step_note(const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g.step_why, sizeof(g.step_why), fmt, ap);
+  va_end(ap);
+}
+// The previous launch of this segment's graph must have finished before its parameters or its pinned slots change.
+void seg_wait(size_t si) {
+  if (si < g.seg_waited.size() && !g.seg_waited[si]) {
+    StepSeg &sg = g.plan->segs[si];
+    if (sg.done) (void)hipEventSynchronize(sg.done);
+    g.seg_waited[si] = 1;
+  }
+}
+// VERIFY -> EAGER: this step does not follow the plan.  The launches of the current segment that were skipped so far
+// are issued now, from the recorded arguments (which are this step's: every difference was copied in); earlier segments
+// have already run as graphs.  The plan is dropped at ah_step_end and recorded again by the next step.
+void step_fallback(const char *why) {
+  if (g.step_mode != STEP_VERIFY) return;
+  StepSeg &sg = g.plan->segs[g.seg];
+  std::vector<void *> ptrs;
+  for (size_t i = 0; i < g.op && i < sg.ops.size(); i++) {
+    StepOp &o = sg.ops[i];
+    o.fill_ptrs(ptrs);
+    (void)hipLaunchKernel(o.func, o.grid, o.block, ptrs.data(), o.shmem, g.stream);
+  }
+  g.step_mode = STEP_EAGER;
+  g.step_fellback = true;
+  step_note("%s (segment %zu, launch %zu)", why, g.seg, g.op);
+}
+bool same_launch(const StepOp &o, const void *func, dim3 grid, dim3 block, unsigned shmem, const uint32_t *sizes, int n) {
+  if (o.func != func || o.shmem != shmem || (int)o.size.size() != n) return false;
+  if (o.grid.x != grid.x || o.grid.y != grid.y || o.grid.z != grid.z) return false;
+  if (o.block.x != block.x || o.block.y != block.y || o.block.z != block.z) return false;
+  for (int i = 0; i < n; i++) if (o.size[i] != sizes[i]) return false;
+  return true;
+}
+int32_t step_begin_capture() {
+  AH_HIP(hipStreamBeginCapture(g.stream, hipStreamCaptureModeRelaxed));
+  g.step_capture_open = true;
+  return AH_OK;
+}
+// RECORD: close the capture of the current segment, instantiate and launch it.
+int32_t step_close_segment(const char *what) {
+  StepSeg &sg = g.plan->segs.back();
+  sg.boundary = what;
+  if (g.step_capture_open) {
+    g.step_capture_open = false;
+    AH_HIP(hipStreamEndCapture(g.stream, &sg.graph));
+  }
+  if (!sg.ops.empty()) {
+    AH_HIP(hipGraphInstantiate(&sg.exec, sg.graph, nullptr, nullptr, 0));
+    AH_HIP(hipEventCreateWithFlags(&sg.done, hipEventDisableTiming));
+    AH_HIP(hipGraphLaunch(sg.exec, g.stream));
+    AH_HIP(hipEventRecord(sg.done, g.stream));
+  }
+  return AH_OK;
+}
+}  // namespace
+
+void launch_raw(const void *func, dim3 grid, dim3 block, unsigned shmem, void **args, const uint32_t *sizes, int nargs) {
+  if (g.step_mode == STEP_OFF || g.step_mode == STEP_EAGER) {
+    (void)hipLaunchKernel(func, grid, block, args, shmem, g.stream);       // an error is picked up by hipGetLastError
+    return;
+  }
+  if (g.step_mode == STEP_RECORD) {
+    if (hipLaunchKernel(func, grid, block, args, shmem, g.stream) != hipSuccess) { g.plan->broken = true; return; }
+    StepSeg &sg = g.plan->segs.back();
+    sg.ops.emplace_back();
+    StepOp &o = sg.ops.back();
+    o.func = func; o.grid = grid; o.block = block; o.shmem = shmem;
+    uint32_t at = 0;
+    for (int i = 0; i < nargs; i++) { o.off.push_back(at); o.size.push_back(sizes[i]); at += (sizes[i] + 15u) & ~15u; }
+    o.blob.assign(at ? at : 16, 0);
+    for (int i = 0; i < nargs; i++) memcpy(o.blob.data() + o.off[i], args[i], sizes[i]);
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    const hipGraphNode_t *deps = nullptr;
+    size_t ndeps = 0;
+    if (hipStreamGetCaptureInfo_v2(g.stream, &st, nullptr, nullptr, &deps, &ndeps) == hipSuccess &&
+        st == hipStreamCaptureStatusActive && ndeps == 1) o.node = deps[0];
+    else g.plan->broken = true;            // cannot name the node: this plan will not be replayed
+    if (sg.ops.size() >= step_chunk() && step_boundary("chunk") == AH_OK) (void)step_begin_capture();
+    return;
+  }
+  // STEP_VERIFY
+  StepSeg &sg = g.plan->segs[g.seg];
+  if (g.op < sg.ops.size() && same_launch(sg.ops[g.op], func, grid, block, shmem, sizes, nargs)) {
+    StepOp &o = sg.ops[g.op];
+    bool differ = false;
+    static const bool debug = getenv("AH_STEP_DEBUG") != nullptr;
+    for (int i = 0; i < nargs; i++)
+      if (memcmp(o.blob.data() + o.off[i], args[i], sizes[i]) != 0) {
+        if (debug) fprintf(stderr, "[ah step] seg %zu launch %zu %s: argument %d (%u bytes) differs\n", g.seg, g.op,
+                           hipKernelNameRefByPtr(func, g.stream), i, sizes[i]);
+        memcpy(o.blob.data() + o.off[i], args[i], sizes[i]);
+        differ = true;
+      }
+    g.op++;
+    if (differ) {
+      g.step_node_updates++;
+      seg_wait(g.seg);
+      std::vector<void *> ptrs;
+      o.fill_ptrs(ptrs);
+      hipKernelNodeParams kp;
+      memset(&kp, 0, sizeof(kp));
+      kp.func = const_cast<void *>(o.func); kp.gridDim = o.grid; kp.blockDim = o.block; kp.sharedMemBytes = o.shmem;
+      kp.kernelParams = ptrs.data(); kp.extra = nullptr;
+      if (hipGraphExecKernelNodeSetParams(sg.exec, o.node, &kp) != hipSuccess) {
+        (void)hipGetLastError();
+        step_fallback("a kernel node refused new parameters");    // launches [0, g.op) incl. this one, from the blobs
+        return;
+      }
+    }
+    if (g.op == sg.ops.size() && sg.boundary == "chunk") (void)step_boundary("chunk");
+    return;
+  }
+  step_fallback("a different kernel launch than the plan's");
+  (void)hipLaunchKernel(func, grid, block, args, shmem, g.stream);
+}
+
+bool step_active() { return g.step_mode != STEP_OFF; }
+
+int32_t step_boundary(const char *what) {
+  if (g.step_mode == STEP_OFF || g.step_mode == STEP_EAGER) return AH_OK;
+  if (g.step_mode == STEP_RECORD) {
+    if (g.plan->segs.back().ops.empty() && strcmp(what, "ah_step_end") != 0) {
+      // nothing recorded since the last boundary: the host may touch the stream without a segment of its own
+      if (g.step_capture_open) {
+        g.step_capture_open = false;
+        hipGraph_t junk = nullptr;
+        AH_HIP(hipStreamEndCapture(g.stream, &junk));
+        if (junk) (void)hipGraphDestroy(junk);
+      }
+      return AH_OK;
+    }
+    int32_t rc = step_close_segment(what);
+    if (rc != AH_OK) { g.plan->broken = true; return rc; }
+    g.plan->segs.emplace_back();
+    return AH_OK;
+  }
+  StepSeg &sg = g.plan->segs[g.seg];
+  if (g.op == 0 && !(sg.ops.empty() && sg.boundary == what) && strcmp(what, "ah_step_end") != 0) return AH_OK;   // likewise on replay
+  if (g.op == sg.ops.size() && sg.boundary == what) {
+    if (sg.exec) {
+      AH_HIP(hipGraphLaunch(sg.exec, g.stream));
+      AH_HIP(hipEventRecord(sg.done, g.stream));
+      if (g.seg < g.seg_waited.size()) g.seg_waited[g.seg] = 0;
+    }
+    g.seg++; g.op = 0;
+    if (g.seg >= g.plan->segs.size() && strcmp(what, "ah_step_end") != 0) {   // the plan ended here, the step goes on
+      g.seg = g.plan->segs.size() - 1;
+      g.op = g.plan->segs[g.seg].ops.size();
+      g.step_mode = STEP_EAGER; g.step_fellback = true;
+      step_note("the step continues past the end of the plan (%s)", what);
+    }
+    return AH_OK;
+  }
+  step_fallback(what);
+  return AH_OK;
+}
+// After the blocking part of a boundary: RECORD resumes capturing into the next segment.
+static int32_t step_resume() {
+  if (g.step_mode == STEP_RECORD && !g.step_capture_open) return step_begin_capture();
+  return AH_OK;
+}
 }  // namespace ah
 
 using namespace ah;
@@ -121,7 +366,10 @@ int32_t ah_init(int32_t device) {
 
 int32_t ah_shutdown(void) {
   if (!g.inited) return AH_OK;
+  if (g.step_capture_open) { hipGraph_t junk = nullptr; (void)hipStreamEndCapture(g.stream, &junk); if (junk) (void)hipGraphDestroy(junk); }
   (void)hipStreamSynchronize(g.stream);
+  for (auto &kv : g.plans) plan_destroy(kv.second);
+  g.plans.clear();
   for (auto &kv : g.graphs) {
     if (kv.second.exec) (void)hipGraphExecDestroy(kv.second.exec);
     if (kv.second.graph) (void)hipGraphDestroy(kv.second.graph);
@@ -161,8 +409,9 @@ int32_t ah_device_info(AhDeviceInfo *out) {
 int32_t ah_sync(void) {
   AH_REQUIRE_READY();
   if (g.capturing) return fail(AH_ERR_STATE, "ah_sync: illegal while a graph is being captured");
+  { int32_t rc = step_boundary("ah_sync"); if (rc != AH_OK) return rc; }
   AH_HIP(hipStreamSynchronize(g.stream));
-  return AH_OK;
+  return step_resume();
 }
 
 int32_t ah_alloc(uint64_t bytes, ah_ptr *out) {
@@ -219,6 +468,40 @@ int32_t ah_upload(ah_ptr dst, const void *host, uint64_t bytes) {
   if (g.capturing) return fail(AH_ERR_STATE, "ah_upload: illegal while a graph is being captured");
   if (bytes == 0) return AH_OK;
   AH_ARG(dst != 0 && host != nullptr, "ah_upload: null pointer");
+  if (g.step_mode == STEP_RECORD || g.step_mode == STEP_VERIFY) {
+    // Inside a step plan an upload is a pinned slot owned by the plan plus a copy kernel: the graph node reads the slot,
+    // and every later step only rewrites the slot's contents.
+    if (bytes <= STEP_UPLOAD_MAX) {
+      size_t k = g.slot++;
+      StepPlan &pl = *g.plan;
+      if (g.step_mode == STEP_RECORD) {
+        PinnedSlot sl;
+        sl.bytes = (size_t)((bytes + 255) & ~uint64_t(255));
+        sl.seg = pl.segs.size() - 1;
+        if (hipHostMalloc((void **)&sl.host, sl.bytes, hipHostMallocDefault) != hipSuccess ||
+            hipHostGetDevicePointer(&sl.dev, sl.host, 0) != hipSuccess) {
+          (void)hipGetLastError();
+          pl.broken = true;
+          return fail(AH_ERR_OOM, "ah_upload: no pinned slot of %zu bytes for the step plan", sl.bytes);
+        }
+        pl.slots.push_back(sl);
+      } else if (k >= pl.slots.size() || pl.slots[k].bytes < bytes || pl.slots[k].seg != g.seg) {
+        step_fallback("an upload the plan does not have");
+      }
+      if (g.step_mode != STEP_EAGER) {
+        PinnedSlot &sl = pl.slots[k];
+        if (g.step_mode == STEP_VERIFY) seg_wait(g.seg);
+        memcpy(sl.host, host, bytes);
+        step_copy(dp<void>(dst), sl.dev, bytes);
+        AH_LAUNCH_CHECK();
+        return AH_OK;
+      }
+    } else {
+      int32_t rc = step_boundary("ah_upload(large)");
+      if (rc != AH_OK) return rc;
+    }
+  }
+  struct Resume { ~Resume() { (void)step_resume(); } } resume_capture_on_return;
   if (bytes <= RING_SLOT_BYTES) {
     // Small upload: copy into the next pinned ring slot and enqueue; no wait.  An event per half of the ring
     // guarantees a slot's previous copy has completed before the slot is overwritten.
@@ -250,6 +533,8 @@ int32_t ah_download(void *host, ah_ptr src, uint64_t bytes) {
   if (g.capturing) return fail(AH_ERR_STATE, "ah_download: illegal while a graph is being captured");
   if (bytes == 0) return AH_OK;
   AH_ARG(src != 0 && host != nullptr, "ah_download: null pointer");
+  { int32_t rc = step_boundary("ah_download"); if (rc != AH_OK) return rc; }
+  struct Resume { ~Resume() { (void)step_resume(); } } resume_capture_on_return;
   char *dst = (char *)host;
   uint64_t off = 0;
   while (off < bytes) {
@@ -266,6 +551,11 @@ int32_t ah_copy(ah_ptr dst, ah_ptr src, uint64_t bytes) {
   AH_REQUIRE_READY();
   if (bytes == 0) return AH_OK;
   AH_ARG(dst != 0 && src != 0, "ah_copy: null pointer");
+  if (g.step_mode != STEP_OFF) {                 // a kernel node like every other launch of the step
+    step_copy(dp<void>(dst), dp<void>(src), bytes);
+    AH_LAUNCH_CHECK();
+    return AH_OK;
+  }
   AH_HIP(hipMemcpyAsync(dp<void>(dst), dp<void>(src), bytes, hipMemcpyDeviceToDevice, g.stream));
   g.ops++;
   return AH_OK;
@@ -283,6 +573,10 @@ int32_t ah_stats(AhStats *out) {
   out->device_mallocs = g.device_mallocs;
   out->ops_launched = g.ops;
   out->graphs_live = g.graphs.size();
+  out->steps_recorded = g.steps_recorded;
+  out->steps_replayed = g.steps_replayed;
+  out->steps_fallback = g.steps_fallback;
+  out->step_node_updates = g.step_node_updates;
   return AH_OK;
 }
 
@@ -291,6 +585,8 @@ int32_t ah_reset_op_count(void) { g.ops = 0; return AH_OK; }
 int32_t ah_trim_pool(void) {
   AH_REQUIRE_READY();
   if (g.capturing) return fail(AH_ERR_STATE, "ah_trim_pool: illegal while a graph is being captured");
+  { int32_t rc = step_boundary("ah_trim_pool"); if (rc != AH_OK) return rc; }
+  struct Resume { ~Resume() { (void)step_resume(); } } resume_capture_on_return;
   AH_HIP(hipStreamSynchronize(g.stream));
   for (auto &kv : g.pool) for (void *p : kv.second) (void)hipFree(p);
   g.pool.clear();
@@ -301,6 +597,7 @@ int32_t ah_trim_pool(void) {
 int32_t ah_graph_begin(void) {
   AH_REQUIRE_READY();
   if (g.capturing) return fail(AH_ERR_STATE, "ah_graph_begin: a capture is already open");
+  if (g.step_mode != STEP_OFF) return fail(AH_ERR_STATE, "ah_graph_begin: illegal inside ah_step_begin .. ah_step_end");
   // Relaxed mode: allocator calls (hipMalloc) from this thread stay legal while capturing.
   AH_HIP(hipStreamBeginCapture(g.stream, hipStreamCaptureModeRelaxed));
   g.capturing = true;
@@ -333,6 +630,7 @@ int32_t ah_graph_launch(uint64_t graph) {
   auto it = g.graphs.find(graph);
   if (it == g.graphs.end() || !it->second.exec) return fail(AH_ERR_ARG, "ah_graph_launch: unknown graph %llu", (unsigned long long)graph);
   if (g.capturing) return fail(AH_ERR_STATE, "ah_graph_launch: illegal while a graph is being captured");
+  if (g.step_mode != STEP_OFF) return fail(AH_ERR_STATE, "ah_graph_launch: illegal inside ah_step_begin .. ah_step_end");
   AH_HIP(hipGraphLaunch(it->second.exec, g.stream));
   return AH_OK;
 }
@@ -349,6 +647,67 @@ int32_t ah_graph_destroy(uint64_t graph) {
   return AH_OK;
 }
 
+int32_t ah_step_begin(uint64_t key) {
+  AH_REQUIRE_READY();
+  if (g.capturing) return fail(AH_ERR_STATE, "ah_step_begin: illegal while a graph is being captured");
+  if (g.step_mode != STEP_OFF) return fail(AH_ERR_STATE, "ah_step_begin: a step is already open");
+  // Free lists hand out their most recently freed block, so the order in which one step frees its buffers permutes the
+  // addresses the next step gets, and a replay would have to rewrite most nodes.  Every step therefore starts from the
+  // same order of every free list: steps that allocate and free in the same sequence then get the same addresses.
+  for (auto &kv : g.pool) std::sort(kv.second.begin(), kv.second.end());
+  StepPlan &pl = g.plans[key];
+  g.plan = &pl; g.step_key = key; g.seg = 0; g.op = 0; g.slot = 0; g.step_fellback = false; g.step_why[0] = 0;
+  if (pl.complete) {
+    g.seg_waited.assign(pl.segs.size(), 0);
+    g.step_mode = STEP_VERIFY;
+    return AH_OK;
+  }
+  plan_destroy(pl);
+  pl.segs.emplace_back();
+  g.step_mode = STEP_RECORD;
+  int32_t rc = step_begin_capture();
+  if (rc != AH_OK) { g.step_mode = STEP_OFF; g.plans.erase(key); g.plan = nullptr; }
+  return rc;
+}
+
+int32_t ah_step_end(int32_t *out_how) {
+  AH_REQUIRE_READY();
+  if (g.step_mode == STEP_OFF) return fail(AH_ERR_STATE, "ah_step_end: no step is open");
+  int32_t how = AH_STEP_EAGER, rc = AH_OK;
+  if (g.step_mode == STEP_VERIFY && g.seg == 0 && g.op == 0 && g.slot == 0) {
+    // nothing was issued since ah_step_begin (a bracket opened after the last step of a run): the plan stays as it is
+  } else if (g.step_mode == STEP_RECORD && g.plan->segs.size() == 1 && g.plan->segs[0].ops.empty()) {
+    if (g.step_capture_open) { hipGraph_t junk = nullptr; (void)hipStreamEndCapture(g.stream, &junk); if (junk) (void)hipGraphDestroy(junk); }
+    plan_destroy(*g.plan);
+    g.plans.erase(g.step_key);
+  } else if (g.step_mode == STEP_RECORD) {
+    rc = step_close_segment("ah_step_end");
+    if (rc == AH_OK && !g.plan->broken) { g.plan->complete = true; how = AH_STEP_RECORDED; g.steps_recorded++; }
+    else { (void)hipStreamSynchronize(g.stream); plan_destroy(*g.plan); g.plans.erase(g.step_key); }
+  } else {
+    if (g.step_mode == STEP_VERIFY) rc = step_boundary("ah_step_end");     // launches the last segment, or falls back
+    if (g.step_fellback || rc != AH_OK) {
+      how = AH_STEP_FELL_BACK; g.steps_fallback++;
+      (void)hipStreamSynchronize(g.stream);
+      plan_destroy(*g.plan);
+      g.plans.erase(g.step_key);
+    } else { how = AH_STEP_REPLAYED; g.steps_replayed++; }
+  }
+  g.step_mode = STEP_OFF; g.plan = nullptr; g.step_capture_open = false;
+  if (out_how) *out_how = how;
+  return rc;
+}
+
+int32_t ah_step_reset(uint64_t key) {
+  AH_REQUIRE_READY();
+  if (g.step_mode != STEP_OFF) return fail(AH_ERR_STATE, "ah_step_reset: illegal while a step is open");
+  auto it = g.plans.find(key);
+  if (it != g.plans.end()) { (void)hipStreamSynchronize(g.stream); plan_destroy(it->second); g.plans.erase(it); }
+  return AH_OK;
+}
+
+const char *ah_step_note(void) { return g.step_why; }
+
 int32_t ah_event_create(uint64_t *out_event) {
   AH_REQUIRE_READY();
   AH_ARG(out_event != nullptr, "ah_event_create: null out");
@@ -359,8 +718,9 @@ int32_t ah_event_create(uint64_t *out_event) {
 }
 int32_t ah_event_record(uint64_t event) {
   AH_REQUIRE_READY();
+  { int32_t rc = step_boundary("ah_event_record"); if (rc != AH_OK) return rc; }
   AH_HIP(hipEventRecord((hipEvent_t)(uintptr_t)event, g.stream));
-  return AH_OK;
+  return step_resume();
 }
 int32_t ah_event_elapsed_ms(uint64_t start, uint64_t stop, float *out_ms) {
   AH_REQUIRE_READY();

@@ -2,7 +2,12 @@
 """Headline benchmark: training tokens/s of the GPT-2-small-shape step (vocab 50304, d 768, 12 layers, 12 heads,
 ctx 1024, batch 16; forward + backward + AdamW with gradient clipping) on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--mode fast|parity] [--no-cpu] [--workload gpt2-small|gpt-350m]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--mode fast|backend|parity] [--no-cpu] [--workload gpt2-small|gpt-350m]
+
+`--mode fast` (default) is the hand-scheduled step (FusedTrainer); `--mode backend` runs the generic tape-driven Trainer -- one
+`Backend` call per op, host-side loss / norm / clip, exactly the call structure of the reference trainer -- on FastHipBackend
+(bf16 storage, fused epilogues and grouped weight gradients behind the interface, steps replayed as recorded hipGraph
+segments); `--mode parity` runs the same Trainer on the fp32 kernels.
 
 The default workload is the one the metric is quoted on; `--workload gpt-350m` runs the 350M-shape step (d 1024, 24 layers,
 16 heads, batch 8 with 4 accumulated micro-steps, whole step in one hipGraph) and reports it the same way.
@@ -68,7 +73,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--mode", choices=["fast", "parity"], default="fast")
+    ap.add_argument("--mode", choices=["fast", "backend", "parity"], default="fast")
+    ap.add_argument("--no-step-graphs", action="store_true", help="backend mode: issue every launch eagerly")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--cpu-tokens", type=int, default=32)
     ap.add_argument("--workload", choices=sorted(WORKLOADS), default="gpt2-small")
@@ -77,22 +83,24 @@ def main():
         print("bench.py: this build runs the step on ONE GPU; --gpus must be 1 (no multi-GPU path exists in this run)", file=sys.stderr)
         sys.exit(2)
 
-    from alpha2_amd import HipBackend
+    from alpha2_amd import FastHipBackend, HipBackend
     from alpha2_amd.model import ModelConfig
     from alpha2_amd.train import TrainConfig, zipfBatch
 
-    B = HipBackend(0)
+    B = FastHipBackend(0) if args.mode == "backend" else HipBackend(0)
     model, BATCH, accum, tok_seed, describe = WORKLOADS[args.workload]
     cfg = ModelConfig(**model)
     tc = TrainConfig(iters=50, batchSize=BATCH, gradAccumSteps=accum)
     tokens = BATCH * cfg.blockSize * accum
     micro = [zipfBatch(tok_seed + 100 * m, BATCH, cfg.blockSize, cfg.vocabSize) for m in range(accum)]
-    if args.mode == "parity":
+    if args.mode in ("parity", "backend"):
         from alpha2_amd.train import Trainer
         runner = Trainer(B, cfg, tc, seed=0)
-        dtype = "f32"
+        dtype = "f32" if args.mode == "parity" else "bf16"
         for x, y in micro:
             B._ptr(x), B._ptr(y)
+        if args.mode == "backend" and not args.no_step_graphs:
+            B.enableStepGraphs(True)
 
         def one_step():
             # the generic trainer releases its batch after use; keep ours resident by handing it views
@@ -120,6 +128,10 @@ def main():
     else:
         loss_first, loss_last = losses[0].loss, losses[-1].loss
 
+    step_stats = None
+    if args.mode == "backend":
+        B.enableStepGraphs(False)
+        step_stats = dict(B.stepStats(), fallbackNotes=B.stepFallbackNotes[-4:])
     # one instrumented step: every GEMM launch bracketed by HIP events on the library stream
     recs = runner.timed_step() if hasattr(runner, "timed_step") else _timed(B, one_step)
     gemm = [r for r in recs if r["kind"] == "gemm"]
@@ -150,6 +162,8 @@ def main():
                      "all_gemm": {"launches_per_step": len(gemm), "ms_per_step": g_ms,
                                   "achieved": g_flops / (g_ms * 1e-3) / 1e12 if g_ms > 0 else 0.0}},
     }
+    if step_stats is not None:
+        out["config"]["step_plans"] = step_stats
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(model, args.cpu_tokens)
     print(json.dumps(out))

@@ -78,6 +78,10 @@ typedef struct {
   uint64_t device_mallocs;      /* hipMalloc calls so far */
   uint64_t ops_launched;        /* kernels enqueued since ah_reset_op_count */
   uint64_t graphs_live;
+  uint64_t steps_recorded;      /* ah_step_end results so far: plans recorded, steps replayed, steps that fell back */
+  uint64_t steps_replayed;
+  uint64_t steps_fallback;
+  uint64_t step_node_updates;   /* kernel nodes whose arguments were rewritten during replays */
 } AhStats;
 int32_t ah_stats(AhStats *out);
 int32_t ah_reset_op_count(void);
@@ -90,6 +94,28 @@ int32_t ah_graph_begin(void);
 int32_t ah_graph_end(uint64_t *out_graph);
 int32_t ah_graph_launch(uint64_t graph);
 int32_t ah_graph_destroy(uint64_t graph);
+
+/* ---- step plans: record -> verify -> replay.  The caller keeps issuing the SAME Backend-level calls every training step
+ *      (the reference's tape-driven trainer, packages/train/src/trainer.ts:1188-1273,1761-1784, cannot do otherwise); the library
+ *      turns them into graph launches.  Between ah_step_begin(key) and ah_step_end:
+ *        - with no plan for `key`, every kernel launch is captured instead of run; at each point where the host needs the
+ *          stream (ah_download, ah_sync, ...) the launches so far become one hipGraph segment, which is launched, and capture
+ *          resumes.  ah_step_end stores the segments as the plan (result AH_STEP_RECORDED).
+ *        - with a plan, every call is compared with the plan's next kernel node: same kernel and grid means the launch is
+ *          skipped (the graph holds it); arguments that differ (learning rate, bias corrections, seeds, a buffer that moved)
+ *          are written into the node.  Boundaries launch the segment's graph.  ah_upload copies into a pinned slot owned by
+ *          the plan, read by a copy node.  Result AH_STEP_REPLAYED.
+ *        - the first call that does not match (another kernel, another grid, a boundary elsewhere) ends the replay: the
+ *          skipped launches of the open segment are issued from the plan, the rest of the step runs eagerly, the plan is
+ *          dropped and the next step records again (AH_STEP_FELL_BACK; ah_step_note() says what differed).
+ *      Results are those of eager execution in every case.  Replaces the reference's per-step batching of dispatches
+ *      (batchBegin / batchDispatchMany / batchSubmit, helios_vk.c:4414-4419; packages/helios/src/backend.ts:880-1134). ---- */
+/*      A bracket in which nothing was issued changes nothing (AH_STEP_EAGER). */
+enum { AH_STEP_EAGER = 0, AH_STEP_RECORDED = 1, AH_STEP_REPLAYED = 2, AH_STEP_FELL_BACK = 3 };
+int32_t     ah_step_begin(uint64_t key);
+int32_t     ah_step_end(int32_t *out_how);
+int32_t     ah_step_reset(uint64_t key);          /* drop the plan of `key` */
+const char *ah_step_note(void);                    /* why the last step fell back ("" if it did not) */
 
 /* ---- timing on the library stream.  Replaces gpuTime (helios_vk.c:3448). ---- */
 int32_t ah_event_create(uint64_t *out_event);

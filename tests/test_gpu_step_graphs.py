@@ -1,0 +1,85 @@
+"""Step plans (ah_step_begin / ah_step_end): the generic tape-driven trainer issues the same Backend calls every step;
+the library records them once as hipGraph segments and replays them.  Replayed steps must give exactly what eager
+execution gives (the same kernels in the same order: bit-identical), and a step that deviates from the plan must fall back
+to eager execution with the right results."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+CFG = dict(vocabSize=96, blockSize=32, nLayer=2, nEmbd=64, nHead=2)
+
+
+@pytest.fixture()
+def B():
+    from alpha2_amd import HipBackend
+    b = HipBackend(0)
+    b.resetStepPlan()
+    yield b
+    b.enableStepGraphs(False)
+    b.resetStepPlan()
+
+
+def _trainer(B, accum=1, **kw):
+    from alpha2_amd.model import ModelConfig
+    from alpha2_amd.train import TrainConfig, Trainer
+    return Trainer(B, ModelConfig(**dict(CFG, **kw)), TrainConfig(iters=12, gradAccumSteps=accum), seed=3)
+
+
+def _run(B, graphs, steps=8, accum=1, batch_of=None, **kw):
+    from alpha2_amd.train import syntheticBatch
+    tr = _trainer(B, accum, **kw)
+    B.enableStepGraphs(graphs)
+    out, hows = [], []
+    for s in range(steps):
+        bs = batch_of(s) if batch_of else [syntheticBatch(40 + accum * s + m, 4, 32, 96) for m in range(accum)]
+        r = tr.step(bs)
+        out.append((r.loss, r.gradNorm, r.clipCoef, r.lr))
+        hows.append(B.lastStepHow if graphs else "eager")
+    B.enableStepGraphs(False)
+    params = {n: v.data.data.copy() for n, v in tr.entries}
+    return out, hows, params
+
+
+@pytest.mark.parametrize("accum", [1, 2])
+def test_replayed_steps_are_bit_identical_to_eager_steps(B, accum):
+    before = B.stepStats()
+    eager, _, pe = _run(B, False, accum=accum)
+    graph, hows, pg = _run(B, True, accum=accum)
+    after = B.stepStats()
+    assert graph == eager, (graph, eager)
+    for n in pe:
+        assert np.array_equal(pe[n], pg[n]), n
+    # flush() ends step s and opens the plan for step s+1: step 0 runs before the first flush (eager, parameters are
+    # uploaded and moments created), step 1 is recorded, every later step is replayed
+    assert after["recorded"] - before["recorded"] == 1, (before, after, hows, B.lastStepNote)
+    assert after["replayed"] - before["replayed"] >= 5 and after["fellBack"] == before["fellBack"], (before, after, B.lastStepNote)
+
+
+def test_a_step_that_deviates_falls_back_and_the_plan_is_recorded_again(B):
+    """Step 4 uses a batch of another size: other grids, so the replay stops at the first launch that differs, the step
+    finishes eagerly with the right numbers, and the following steps record and replay a new plan."""
+    from alpha2_amd.train import syntheticBatch
+
+    def batch_of(s):
+        return [syntheticBatch(70 + s, 2 if s == 4 else 4, 32, 96)]
+    before = B.stepStats()
+    eager, _, pe = _run(B, False, steps=9, batch_of=batch_of)
+    graph, hows, pg = _run(B, True, steps=9, batch_of=batch_of)
+    after = B.stepStats()
+    assert graph == eager
+    for n in pe:
+        assert np.array_equal(pe[n], pg[n]), n
+    assert after["fellBack"] - before["fellBack"] >= 1 and after["recorded"] - before["recorded"] >= 2
+    assert after["replayed"] - before["replayed"] >= 3
+
+
+def test_per_step_scalars_and_dropout_seeds_follow_the_caller(B):
+    """Learning rate, bias corrections, the clip coefficient and the dropout seed change every step: they are kernel
+    arguments, rewritten in the graph nodes, not frozen at recording time."""
+    eager, _, pe = _run(B, False, dropout=0.1)
+    graph, hows, pg = _run(B, True, dropout=0.1)
+    assert graph == eager
+    assert len({x[3] for x in graph}) > 3                       # the schedule moved
+    for n in pe:
+        assert np.array_equal(pe[n], pg[n]), n
