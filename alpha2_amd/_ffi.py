@@ -46,7 +46,7 @@ class AhFlash(C.Structure):
                 ("v_sb", i64), ("v_sh", i64), ("v_st", i64), ("o_sb", i64), ("o_sh", i64), ("o_st", i64),
                 ("scale", f32), ("soft_cap", f32),
                 ("q", u64), ("k", u64), ("v", u64), ("o", u64), ("lse", u64),
-                ("d_o", u64), ("dq", u64), ("dk", u64), ("dv", u64)]
+                ("d_o", u64), ("dq", u64), ("dk", u64), ("dv", u64), ("bwd_variant", i32), ("reserved", i32)]
 
 
 class AhRng(C.Structure):

@@ -108,6 +108,7 @@ class HipBackend:
         self.lastStepHow, self.lastStepNote = "eager", ""
         self.stepFallbackNotes: List[str] = []
         self._hyper_dev, self._hyper_key = None, None
+        self.flashBackwardVariant = 0          # AhFlash.bwd_variant for the bf16 backward kernels (1: one pass over the scores)
 
     # ------------------------------------------------------------------ residency helpers
     def _new(self, shape, dtype="f32", store: Optional[str] = None) -> TensorData:
@@ -785,6 +786,7 @@ class HipBackend:
         for p in ("q", "k", "v", "o"):
             setattr(f, p + "_sb", T * D), setattr(f, p + "_sh", 0), setattr(f, p + "_st", D)
         f.scale, f.soft_cap = scale, softCap
+        f.bwd_variant = self.flashBackwardVariant
         return f
 
     def flashAttention(self, Q, K, V, T, scale, softCap) -> dict:
@@ -816,6 +818,7 @@ class HipBackend:
             setattr(f, p + "_sb", T * c3), setattr(f, p + "_sh", D), setattr(f, p + "_st", c3)
         f.o_sb, f.o_sh, f.o_st = T * Cc, D, Cc
         f.scale, f.soft_cap = scale, softCap
+        f.bwd_variant = self.flashBackwardVariant
         return f
 
     def attentionQkv(self, qkv: TensorData, Bt: int, T: int, nHead: int, scale: float, softCap: float) -> dict:

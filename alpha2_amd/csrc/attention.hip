@@ -312,7 +312,7 @@ int32_t check(const AhFlash *f, bool bwd, FlashArgs &a) {
   a.q = dp<const void>(f->q); a.k = dp<const void>(f->k); a.v = dp<const void>(f->v);
   a.o = dp<void>(f->o); a.lse = dp<float>(f->lse);
   a.d_o = dp<const void>(f->d_o); a.dq = dp<void>(f->dq); a.dk = dp<void>(f->dk); a.dv = dp<void>(f->dv);
-  a.delta = nullptr;
+  a.delta = nullptr; a.variant = f->bwd_variant;
   a.B = f->batch; a.H = f->heads; a.T = f->seq;
   a.q_sb = f->q_sb; a.q_sh = f->q_sh; a.q_st = f->q_st;
   a.k_sb = f->k_sb; a.k_sh = f->k_sh; a.k_st = f->k_st;

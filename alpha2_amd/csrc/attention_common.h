@@ -14,6 +14,7 @@ struct FlashArgs {
   int B, H, T;
   int64_t q_sb, q_sh, q_st, k_sb, k_sh, k_st, v_sb, v_sh, v_st, o_sb, o_sh, o_st;
   float scale, cap;
+  int variant;             // AhFlash::bwd_variant
 };
 
 // Which (batch x head, block along the sequence) this workgroup works on.  Workgroups are dealt to the 8 XCDs round-robin

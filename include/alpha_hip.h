@@ -324,6 +324,10 @@ typedef struct {
   float   scale, soft_cap;
   ah_ptr  q, k, v, o, lse;
   ah_ptr  d_o, dq, dk, dv;   /* backward only; dq/dk/dv share the strides of q/k/v */
+  int32_t bwd_variant;       /* backward, bf16, head_dim <= 64: 0 = a dQ kernel and a dK/dV kernel (each evaluates every score);
+                                1 = one pass over the scores (a workgroup per 256 keys, dQ parts reduced in a fixed order).
+                                Same results to bf16 rounding, both deterministic; 0 is the faster one today. */
+  int32_t reserved;
 } AhFlash;
 int32_t ah_flash_fwd(const AhFlash *f);
 int32_t ah_flash_bwd(const AhFlash *f);

@@ -676,10 +676,20 @@ def test_gemm_bf16_split_k_weight_gradient(B):
     assert_close(_raw_gemm(B, ffi.GEMM_TN, g_, x, M, N, Kc, ffi.BF16, ffi.F32, ffi.EPI_ACCUM, c_init=c0)[0], want + c0, what="split-K ACCUM")
 
 
-@pytest.mark.parametrize("BH,T,D,cap", [(2, 64, 32, 30.0), (3, 100, 64, 0.0), (2, 129, 64, 30.0), (2, 320, 64, 30.0), (1, 256, 128, 30.0), (2, 1, 64, 0.0)])
-def test_flash_attention_bf16_vs_materialised(B, BH, T, D, cap):
+@pytest.fixture(params=[0, 1], ids=["pair", "onepass"])
+def bwd_variant(request, B):
+    """Both arrangements of the bf16 backward pass: a dQ and a dK/dV kernel, or one pass over the scores."""
+    B.flashBackwardVariant = request.param
+    yield request.param
+    B.flashBackwardVariant = 0
+
+
+@pytest.mark.parametrize("BH,T,D,cap", [(2, 64, 32, 30.0), (3, 100, 64, 0.0), (2, 129, 64, 30.0), (2, 320, 64, 30.0), (1, 256, 128, 30.0), (2, 1, 64, 0.0),
+                                        (3, 700, 64, 30.0), (2, 513, 32, 0.0)])
+def test_flash_attention_bf16_vs_materialised(B, bwd_variant, BH, T, D, cap):
     """bf16 operands, fp32 accumulation.  Inputs are bf16-exact so the oracle sees the same numbers; the kernel rounds P and
-    dS to bf16 before the second product and its outputs to bf16, so the bar is bf16 resolution (2^-7 of the tensor scale)."""
+    dS to bf16 before the second product and its outputs to bf16, so the bar is bf16 resolution (2^-7 of the tensor scale).
+    T = 700 and 513 give the one-pass kernel several 256-key blocks with a ragged last one."""
     q, k, v, do = (_bf16_round(rs.randn(BH, T, D).astype(np.float32))[0] for _ in range(4))
     scale = 1 / math.sqrt(D)
     want_o, want_lse, dq, dk, dv = _oracle_attention(q, k, v, do, scale, cap)
@@ -908,7 +918,7 @@ def test_flash_attention_heads_are_independent_of_how_blocks_are_dealt_out(B, st
 
 @pytest.mark.parametrize("T", [256, 1024, 2048])
 @pytest.mark.parametrize("cap", [0.0, 30.0])
-def test_flash_attention_microbench_shapes(B, T, cap):
+def test_flash_attention_microbench_shapes(B, bwd_variant, T, cap):
     """B = 16, H = 12, head_dim 64, bf16 in / fp32 accumulate, scale 1/8, as in the attention microbenchmark.  The kernels
     run on all 192 heads; three of them (first, a middle one, last) are checked against the oracle's materialised chain."""
     BH, D, scale = 192, 64, 0.125
