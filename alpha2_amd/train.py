@@ -158,6 +158,22 @@ def zipfBatch(seed: int, Bt: int, T: int, vocab: int, s: float = 1.1) -> Tuple[T
     return TensorData((Bt, T), "i32", ids[:, :T]), TensorData((Bt, T), "i32", ids[:, 1:])
 
 
+def zipfBatches(seed: int, count: int, Bt: int, T: int, vocab: int, s: float = 1.1) -> List[Tuple[TensorData, TensorData]]:
+    """`count` successive batches cut from ONE seeded uniform stream (batch k takes draws [k B (T+1), (k+1) B (T+1))).  Streams
+    of neighbouring seeds are no substitute for this: the reference's xorshift (packages/core/src/rng.ts:13-50) seeded with s
+    and s + 1 gives sequences that correlate at 0.5, i.e. near-copies of the same batch."""
+    from .rng import SeededRng
+    w = 1.0 / np.power(np.arange(1, vocab + 1, dtype=np.float64), s)
+    cdf = np.cumsum(w / w.sum())
+    n = Bt * (T + 1)
+    u = SeededRng(seed).fillUniform(count * n)
+    out = []
+    for k in range(count):
+        ids = np.minimum(np.searchsorted(cdf, u[k * n:(k + 1) * n], side="right"), vocab - 1).astype(np.int32).reshape(Bt, T + 1)
+        out.append((TensorData((Bt, T), "i32", ids[:, :T]), TensorData((Bt, T), "i32", ids[:, 1:])))
+    return out
+
+
 class DataLoader:
     """DataLoader of packages/train/src/data.ts:19-175 with the corpus resident in HBM: the token array is uploaded
     once, a batch is one `ah_token_windows` launch given B window starts.  Random mode draws

@@ -40,18 +40,35 @@ WORKLOADS = {        # name -> (model, micro-batch, accumulated micro-steps, tok
                  "untied lmHead (406.2M params), AdamW lr 3e-4 betas (0.9,0.95) wd 0.1, grad-clip 1.0"),
 }
 PEAK = {"bf16": 2500.0, "f32": 157.3}          # MI355X dense MFMA, TFLOP/s
-# HBM-side bytes per launch of the kernels that can be the dominant one, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
-# runs of this benchmark (counter values scaled by what the same counters read for a plain copy of known size: x2.0
-# for FETCH_SIZE, x1.0 for WRITE_SIZE); the counter summary is kept under profiles/.
-TRAFFIC_BYTES = {"k_gemm_bf16_dma_grouped<true, true, 0, float>": 9.2452e9 + 0.5226e9}
+# Counter summaries of this benchmark (rocprofv3 --pmc passes; the files say how they were made and calibrated).  What the
+# JSON line reports from counters -- HBM-side bytes per launch of the dominant kernel, time-weighted MFMA-busy fraction of the
+# step -- is read from the table in the file of the workload, never typed in here.
+COUNTER_TABLES = {"gpt2-small": "profiles/train_step_gpt2small_bf16_counters.md", "gpt-350m": "profiles/train_step_gpt350m_bf16_counters.md"}
 
 
-def step_flops(cfg, tokens):
-    """6*P_mm + 12*L*T*C per token (attention counted non-causal, the reference's convention:
-    scripts/bench-ops.ts:652,673)."""
+def counter_table(workload: str):
+    """Rows of the '| kernel | launches | us per step | clock GHz | MFMA busy | fetched MB | written MB | ...' table."""
+    path = os.path.join(ROOT, COUNTER_TABLES.get(workload, ""))
+    rows = {}
+    if not os.path.isfile(path):
+        return rows, None
+    for line in open(path):
+        cells = [c.strip() for c in line.strip().strip("|").split("|")]
+        if len(cells) >= 7 and cells[0].startswith("k_"):
+            try:
+                rows[cells[0]] = {"launches": float(cells[1]), "us": float(cells[2]), "busy": float(cells[4]),
+                                  "fetched_mb": float(cells[5]), "written_mb": float(cells[6])}
+            except ValueError:
+                pass
+    return rows, COUNTER_TABLES[workload]
+
+
+def step_flops(cfg, tokens, causal=False):
+    """6*P_mm + 12*L*T*C per token: attention counted non-causal, the reference's convention (scripts/bench-ops.ts:652,673);
+    `causal` counts the half of the score / value products a causal kernel has to do (6*L*T*C, the diagonal aside)."""
     C_, L, F, V, T = cfg["nEmbd"], cfg["nLayer"], 4 * cfg["nEmbd"], cfg["vocabSize"], cfg["blockSize"]
     p_mm = L * (3 * C_ * C_ + C_ * C_ + 2 * C_ * F) + V * C_
-    return (6 * p_mm + 12 * L * T * C_) * tokens
+    return (6 * p_mm + (6 if causal else 12) * L * T * C_) * tokens
 
 
 def cpu_baseline(model: dict, seq_tokens: int):
@@ -85,14 +102,17 @@ def main():
 
     from alpha2_amd import FastHipBackend, HipBackend
     from alpha2_amd.model import ModelConfig
-    from alpha2_amd.train import TrainConfig, zipfBatch
+    from alpha2_amd.train import TrainConfig, zipfBatches
 
     B = FastHipBackend(0) if args.mode == "backend" else HipBackend(0)
     model, BATCH, accum, tok_seed, describe = WORKLOADS[args.workload]
     cfg = ModelConfig(**model)
     tc = TrainConfig(iters=50, batchSize=BATCH, gradAccumSteps=accum)
     tokens = BATCH * cfg.blockSize * accum
-    micro = [zipfBatch(tok_seed + 100 * m, BATCH, cfg.blockSize, cfg.vocabSize) for m in range(accum)]
+    # a ring of distinct resident batches: every step trains on the next `accum` of them, so the reported losses are a
+    # training curve and not the memorisation of one batch
+    ring = max(8, accum * 4)
+    micro = zipfBatches(tok_seed, ring, BATCH, cfg.blockSize, cfg.vocabSize)        # one stream from the workload's seed
     if args.mode in ("parity", "backend"):
         from alpha2_amd.train import Trainer
         runner = Trainer(B, cfg, tc, seed=0)
@@ -102,15 +122,24 @@ def main():
         if args.mode == "backend" and not args.no_step_graphs:
             B.enableStepGraphs(True)
 
+        cursor = [0]
+
         def one_step():
             # the generic trainer releases its batch after use; keep ours resident by handing it views
-            return runner.step([(B.reshape(x, x.shape), B.reshape(y, y.shape)) for x, y in micro])
+            pick = [micro[(cursor[0] + m) % ring] for m in range(accum)]
+            cursor[0] += accum
+            return runner.step([(B.reshape(x, x.shape), B.reshape(y, y.shape)) for x, y in pick])
     else:
         from alpha2_amd.fused import FusedTrainer
         runner = FusedTrainer(B, cfg, tc, BATCH, seed=0, accum=accum)
         dtype = "bf16"
-        runner._use_batch([runner.add_batch(x, y) for x, y in micro])      # resident: step() keeps training on them
-        one_step = runner.step
+        ids = [runner.add_batch(x, y) for x, y in micro]                   # resident in HBM before the timed region
+        cursor = [0]
+
+        def one_step():
+            pick = [ids[(cursor[0] + m) % ring] for m in range(accum)]
+            cursor[0] += accum
+            return runner.step(pick if accum > 1 else pick[0])             # two 64 KB device-to-device copies, then the graph
 
     losses = []
     for _ in range(args.warmup):
@@ -147,17 +176,28 @@ def main():
             grp["flops"] += r["flops"]; grp["ms"] += r["ms"]; grp["n"] += 1
     dom_name, dom = max(groups.items(), key=lambda kv: (kv[1]["flops"], kv[1]["ms"]))
     achieved = dom["flops"] / (dom["ms"] * 1e-3) / 1e12
-    flops = step_flops(model, tokens)
+    flops, flops_causal = step_flops(model, tokens), step_flops(model, tokens, causal=True)
+    table, table_path = counter_table(args.workload) if args.mode == "fast" else ({}, None)
+    trow = table.get(dom_name)
+    traffic = (trow["fetched_mb"] + trow["written_mb"]) * 1e6 / trow["launches"] if trow else None
+    # MFMA-busy fraction of the step by the SQ_VALU_MFMA_BUSY_CYCLES counter: kernels weighted by their time in the step
+    busy = (sum(r["busy"] * r["us"] for r in table.values()) / sum(r["us"] for r in table.values())) if table else None
     out = {
         "metric": "train tokens/sec + MFMA util % on GPT-124M step, 1xMI355X", "value": tokens / (ms * 1e-3), "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": f"synthetic (Zipf s=1.1 token ids, seed {tok_seed}; random-init N(0,0.02) weights, seed 0)",
         "config": {"workload": describe,
                    "tokens_per_step": tokens, "mode": args.mode, "loss_first_step": loss_first, "loss_last_step": loss_last},
+        # model flops per second against the dense bf16 MFMA peak: by the reference's (non-causal) attention count, and with
+        # the causal half of the attention products only
         "step_tflops": flops / (ms * 1e-3) / 1e12, "mfu_vs_bf16_dense_peak": flops / (ms * 1e-3) / 1e12 / PEAK["bf16"],
+        "step_tflops_causal": flops_causal / (ms * 1e-3) / 1e12, "mfu_causal": flops_causal / (ms * 1e-3) / 1e12 / PEAK["bf16"],
+        # the "MFMA util %" of the metric: model flops / peak (= mfu_vs_bf16_dense_peak); beside it what the hardware counter
+        # says, from the committed counter summary of this workload (not measured in this run)
         "mfma_util_pct": 100.0 * flops / (ms * 1e-3) / 1e12 / PEAK["bf16"],
+        "mfma_busy_counter": {"frac_of_step_time": busy, "source": table_path},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK[dtype], "unit": "TFLOP/s", "frac": achieved / PEAK[dtype],
-                     "traffic": TRAFFIC_BYTES.get(dom_name) if args.workload == "gpt2-small" else None, "kernel": dom_name, "launches_per_step": dom["n"], "avg_launch_us": dom["ms"] / dom["n"] * 1e3,
+                     "traffic": traffic, "traffic_source": table_path if trow else None, "kernel": dom_name, "launches_per_step": dom["n"], "avg_launch_us": dom["ms"] / dom["n"] * 1e3,
                      "flops_per_launch": dom["flops"] / dom["n"], "ms_per_step": dom["ms"],
                      "all_gemm": {"launches_per_step": len(gemm), "ms_per_step": g_ms,
                                   "achieved": g_flops / (g_ms * 1e-3) / 1e12 if g_ms > 0 else 0.0}},
