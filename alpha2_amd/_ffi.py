@@ -104,6 +104,8 @@ SIGNATURES = {
     "ah_embedding": [u64, u64, u64, i64, i64, i64, i32],
     "ah_embedding_tok_pos": [u64, u64, u64, u64, i64, i64, i64, i64],
     "ah_embedding_bwd": [u64, u64, u64, i64, i64, i64, i32],
+    "ah_embedding_index_bytes": [i64, i64], "ah_embedding_index": [u64, i64, i64, u64],
+    "ah_embedding_bwd_indexed": [u64, u64, u64, i64, i64, i64, i32],
     "ah_token_windows": [u64, i64, u64, i64, i64, u64, u64],
     "ah_pos_embedding_bwd": [u64, u64, i64, i64, i64, i32],
     "ah_layernorm": [u64, u64, u64, u64, i64, i64, f32, i32],
@@ -157,6 +159,7 @@ def load():
         fn.argtypes = args
         fn.restype = i32
     lib.ah_layernorm_bwd_partials_bytes.restype = i64       # a size, not a status
+    lib.ah_embedding_index_bytes.restype = i64
     lib.ah_last_error.argtypes = []
     lib.ah_last_error.restype = C.c_char_p
     lib.ah_step_note.argtypes = []

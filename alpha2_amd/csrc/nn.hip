@@ -90,6 +90,115 @@ __global__ __launch_bounds__(1024) void k_embedding_bwd_blocks(const int32_t *__
       if (c0 + 64 * k < dim) unsafeAtomicAdd(dst + c0 + 64 * k, acc[k]);
   }
 }
+// ---- the same sum with a fixed order of additions (what ah_embedding_bwd runs when the sizes allow) ---------------------
+// The reference adds the rows of an id in position order (packages/autograd/src/ops.ts:491-507); atomics add them in whatever
+// order the launch happens to take, so the last bit of the gradient changed from run to run.  Here:
+//   1. one workgroup sorts the keys (id << 16 | position) of all positions in LDS (bitonic network; ids out of range sort last);
+//   2. a wave takes 32 consecutive sorted keys and a slice of 256 columns and adds the rows of each id in its chunk in
+//      position order.  An id whose run lies inside the chunk is finished: its row is stored (nobody else writes it).  A run
+//      that crosses a chunk border leaves its part in one of the chunk's two side slots;
+//   3. for every run that crosses borders, the wave of the chunk where it starts adds the parts chunk by chunk.
+// Every row of the result is written by exactly one lane, the order of every addition is a function of the token ids alone.
+constexpr int ES_MAX = 32768;           // positions per call (keys must fit the 64 KB ... 128 KB of LDS the sort uses)
+constexpr int ES_CHUNK = 32;
+__global__ __launch_bounds__(1024) void k_emb_sort(const int32_t *__restrict__ idx, uint32_t *__restrict__ sorted, int n, int npad, int vocab) {
+  __shared__ uint32_t keys[ES_MAX];
+  for (int i = threadIdx.x; i < npad; i += 1024) {
+    uint32_t key = 0xFFFFFFFFu;
+    if (i < n) { int32_t t = idx[i]; if (t >= 0 && t < vocab) key = ((uint32_t)t << 16) | (uint32_t)i; }
+    keys[i] = key;
+  }
+  for (int k = 2; k <= npad; k <<= 1)
+    for (int j = k >> 1; j > 0; j >>= 1) {
+      __syncthreads();
+      for (int t = threadIdx.x; t < (npad >> 1); t += 1024) {
+        int i = ((t & ~(j - 1)) << 1) | (t & (j - 1)), p = i | j;
+        uint32_t a = keys[i], b = keys[p];
+        bool up = (i & k) == 0;
+        if ((a > b) == up) { keys[i] = b; keys[p] = a; }
+      }
+    }
+  __syncthreads();
+  for (int i = threadIdx.x; i < npad; i += 1024) sorted[i] = keys[i];
+}
+struct EmbChunk { int32_t first_id, last_id, flags, pad; };        // flags: 1 one run only, 2 first run continues the previous chunk's, 4 last run goes on
+__device__ __forceinline__ int es_id(uint32_t key) { return key == 0xFFFFFFFFu ? -1 : (int)(key >> 16); }
+__global__ __launch_bounds__(256) void k_emb_runs(const uint32_t *__restrict__ sorted, const float *__restrict__ g, float *__restrict__ gw,
+                                                  float *__restrict__ part, EmbChunk *__restrict__ meta, int npad, int64_t dim, int accumulate) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int c = blockIdx.x * 4 + wave;
+  if (c * ES_CHUNK >= npad) return;
+  const int64_t col = blockIdx.y * (int64_t)256 + lane * 4;
+  const bool col_live = col < dim;
+  const uint32_t mykey = sorted[c * ES_CHUNK + (lane & 31)];
+  const int prev_id = c > 0 ? es_id(sorted[c * ES_CHUNK - 1]) : -1;
+  const int next_id = (c + 1) * ES_CHUNK < npad ? es_id(sorted[(c + 1) * ES_CHUNK]) : -1;
+  const int first_id = es_id(__shfl(mykey, 0, 64));
+  if (first_id < 0) {                                               // nothing but padding
+    if (blockIdx.y == 0 && lane == 0) meta[c] = EmbChunk{-1, -1, 0, 0};
+    return;
+  }
+  // all rows of the chunk are requested before the first addition: the additions then run in order at register speed
+  float4 rows[ES_CHUNK];
+#pragma unroll
+  for (int e = 0; e < ES_CHUNK; e++) {
+    const uint32_t key = __shfl(mykey, e, 64);
+    rows[e] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (key != 0xFFFFFFFFu && col_live) rows[e] = *reinterpret_cast<const float4 *>(g + (int64_t)(key & 0xFFFFu) * dim + col);
+  }
+  const bool head_cont = first_id == prev_id;
+  int cur = first_id, run = 0, last_id = first_id;
+  bool tail_cont = false;
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  auto emit = [&](int id, bool is_first, bool is_last_and_goes_on) {
+    if (!col_live) return;
+    if (is_first && head_cont) *reinterpret_cast<float4 *>(part + ((int64_t)c * 2 + 0) * dim + col) = acc;
+    else if (is_last_and_goes_on) *reinterpret_cast<float4 *>(part + ((int64_t)c * 2 + 1) * dim + col) = acc;
+    else {
+      float4 *dst = reinterpret_cast<float4 *>(gw + (int64_t)id * dim + col);
+      if (accumulate) { float4 o = *dst; acc.x += o.x; acc.y += o.y; acc.z += o.z; acc.w += o.w; }
+      *dst = acc;
+    }
+  };
+#pragma unroll
+  for (int e = 0; e < ES_CHUNK; e++) {
+    const int id = es_id(__shfl(mykey, e, 64));
+    if (id >= 0) {                                                  // wave-uniform
+      if (id != cur) {
+        emit(cur, run == 0, false);
+        cur = id; run++;
+        acc = make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+      acc.x += rows[e].x; acc.y += rows[e].y; acc.z += rows[e].z; acc.w += rows[e].w;
+      last_id = id;
+      if (e == ES_CHUNK - 1) tail_cont = id == next_id;
+    }
+  }
+  emit(cur, run == 0, tail_cont);
+  if (blockIdx.y == 0 && lane == 0) meta[c] = EmbChunk{first_id, last_id, (run == 0 ? 1 : 0) | (head_cont ? 2 : 0) | (tail_cont ? 4 : 0), 0};
+}
+__global__ __launch_bounds__(256) void k_emb_join(const float *__restrict__ part, const EmbChunk *__restrict__ meta, float *__restrict__ gw,
+                                                  int nchunks, int64_t dim, int accumulate) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int c = blockIdx.x * 4 + wave;
+  if (c >= nchunks) return;
+  const int64_t col = blockIdx.y * (int64_t)256 + lane * 4;
+  if (col >= dim) return;
+  const EmbChunk m = meta[c];
+  // the run that crosses this chunk's right border starts here unless the whole chunk is the middle of a longer run
+  if (!(m.flags & 4) || ((m.flags & 1) && (m.flags & 2))) return;
+  float4 acc = *reinterpret_cast<const float4 *>(part + ((int64_t)c * 2 + 1) * dim + col);
+  for (int cc = c + 1; cc < nchunks; cc++) {
+    const EmbChunk mm = meta[cc];
+    float4 x = *reinterpret_cast<const float4 *>(part + ((int64_t)cc * 2 + 0) * dim + col);
+    acc.x += x.x; acc.y += x.y; acc.z += x.z; acc.w += x.w;
+    if (!((mm.flags & 1) && (mm.flags & 4))) break;                // the run ends inside chunk cc
+  }
+  float4 *dst = reinterpret_cast<float4 *>(gw + (int64_t)m.last_id * dim + col);
+  if (accumulate) { float4 o = *dst; acc.x += o.x; acc.y += o.y; acc.z += o.z; acc.w += o.w; }
+  *dst = acc;
+}
+
 __global__ void k_pos_embedding_bwd(const float *__restrict__ g, float *__restrict__ gw, int64_t batch, int64_t td, int accumulate) {
   int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
   if (i >= td) return;
@@ -621,12 +730,67 @@ int32_t ah_token_windows(ah_ptr corpus, int64_t n_tokens, ah_ptr starts, int64_t
   return AH_OK;
 }
 
+static int es_npad(int64_t n_idx) {
+  int npad = 64;
+  while (npad < n_idx) npad <<= 1;
+  return npad;
+}
+int64_t ah_embedding_index_bytes(int64_t n_idx, int64_t vocab) {
+  return (n_idx >= 1 && n_idx <= ES_MAX && vocab >= 1 && vocab < 65535) ? (int64_t)es_npad(n_idx) * 4 : 0;
+}
+int32_t ah_embedding_index(ah_ptr idx, int64_t n_idx, int64_t vocab, ah_ptr index_out) {
+  AH_REQUIRE_READY();
+  AH_ARG(ah_embedding_index_bytes(n_idx, vocab) > 0, "ah_embedding_index: %lld positions over %lld ids is outside the indexed path (at most %d positions, ids below 65535)",
+         (long long)n_idx, (long long)vocab, ES_MAX);
+  AH_ARG(idx && index_out, "ah_embedding_index: null operand");
+  ah::launch_kernel(k_emb_sort, dim3(1), dim3(1024), 0, dp<const int32_t>(idx), dp<uint32_t>(index_out), (int)n_idx, es_npad(n_idx), (int)vocab);
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+// zero fill (unless accumulating) must already have happened
+static int32_t embedding_bwd_sorted(ah_ptr index, ah_ptr grad_out, ah_ptr grad_w, int64_t n_idx, int64_t dim, int32_t accumulate) {
+  const int npad = es_npad(n_idx), nchunks = npad / ES_CHUNK;
+  const size_t b_meta = ((size_t)nchunks * sizeof(EmbChunk) + 255) & ~size_t(255), b_part = (size_t)nchunks * 2 * dim * 4;
+  ah_ptr ws = 0;
+  int32_t rc = ah_alloc(b_meta + b_part, &ws);
+  if (rc) return rc;
+  EmbChunk *meta = dp<EmbChunk>(ws);
+  float *part = reinterpret_cast<float *>(dp<char>(ws) + b_meta);
+  dim3 grid((unsigned)cdiv(nchunks, 4), (unsigned)cdiv(dim, 256));
+  ah::launch_kernel(k_emb_runs, grid, dim3(256), 0, dp<const uint32_t>(index), dp<const float>(grad_out), dp<float>(grad_w), part, meta, npad, dim,
+                    (int)accumulate);
+  AH_LAUNCH_CHECK();
+  ah::launch_kernel(k_emb_join, grid, dim3(256), 0, (const float *)part, (const EmbChunk *)meta, dp<float>(grad_w), nchunks, dim, (int)accumulate);
+  AH_LAUNCH_CHECK();
+  return ah_free(ws);
+}
+int32_t ah_embedding_bwd_indexed(ah_ptr index, ah_ptr grad_out, ah_ptr grad_w, int64_t n_idx, int64_t dim, int64_t vocab, int32_t accumulate) {
+  AH_REQUIRE_READY();
+  AH_ARG(grad_w != 0 || vocab * dim == 0, "ah_embedding_bwd_indexed: null grad_w");
+  if (!accumulate) { int32_t rc = ah_fill_f32(grad_w, 0.f, (uint64_t)(vocab * dim)); if (rc) return rc; }
+  if (n_idx == 0 || dim == 0) return AH_OK;
+  AH_ARG(ah_embedding_index_bytes(n_idx, vocab) > 0, "ah_embedding_bwd_indexed: sizes outside the indexed path");
+  AH_ARG(index && grad_out, "ah_embedding_bwd_indexed: null operand");
+  AH_ARG(dim % 4 == 0 && cdiv(dim, 256) <= 65535 && aligned16(grad_out) && aligned16(grad_w), "ah_embedding_bwd_indexed: rows must be 16-byte aligned multiples of 4 floats");
+  return embedding_bwd_sorted(index, grad_out, grad_w, n_idx, dim, accumulate);
+}
+
 int32_t ah_embedding_bwd(ah_ptr idx, ah_ptr grad_out, ah_ptr grad_w, int64_t n_idx, int64_t dim, int64_t vocab, int32_t accumulate) {
   AH_REQUIRE_READY();
   AH_ARG(grad_w != 0 || vocab * dim == 0, "ah_embedding_bwd: null grad_w");
   if (!accumulate) { int32_t rc = ah_fill_f32(grad_w, 0.f, (uint64_t)(vocab * dim)); if (rc) return rc; }
   if (n_idx == 0 || dim == 0) return AH_OK;
   AH_ARG(idx && grad_out, "ah_embedding_bwd: null operand");
+  if (ah_embedding_index_bytes(n_idx, vocab) > 0 && dim % 4 == 0 && cdiv(dim, 256) <= 65535 && aligned16(grad_out) && aligned16(grad_w)) {
+    // fixed summation order: sort the positions by id, then ah_embedding_bwd_indexed
+    ah_ptr index = 0;
+    int32_t rc = ah_alloc((uint64_t)ah_embedding_index_bytes(n_idx, vocab), &index);
+    if (rc) return rc;
+    rc = ah_embedding_index(idx, n_idx, vocab, index);
+    if (rc == AH_OK) rc = embedding_bwd_sorted(index, grad_out, grad_w, n_idx, dim, accumulate);
+    int32_t rc2 = ah_free(index);
+    return rc ? rc : rc2;
+  }
   if (cdiv(n_idx, EB_POS) < (1ll << 31) && cdiv(dim, 1024) <= 65535)
     ah::launch_kernel(k_embedding_bwd_blocks, dim3((unsigned)cdiv(n_idx, EB_POS), (unsigned)cdiv(dim, 1024)), dim3(1024), 0, 
                        dp<const int32_t>(idx), dp<const float>(grad_out), dp<float>(grad_w), n_idx, dim, vocab);

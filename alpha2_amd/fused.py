@@ -96,6 +96,10 @@ class FusedTrainer:
         self.toks = [a(BT * 4) for _ in range(self.accum)]               # one resident token batch per micro-step
         self.tgts = [a(BT * 4) for _ in range(self.accum)]
         self.tok, self.tgt = self.toks[0], self.tgts[0]
+        # positions of every resident batch sorted by token id, built once when the batch arrives: the embedding scatter-add
+        # of every step then sums in a fixed order without sorting again (0 bytes = sizes outside that path)
+        self._index_bytes = int(self.lib.ah_embedding_index_bytes(BT, V))
+        self.tok_index = [a(self._index_bytes) if self._index_bytes else 0 for _ in range(self.accum)]
         self.x = [a(BT * Cc * 4) for _ in range(self.L + 1)]            # residual stream entering layer l (f32)
         self.xmid = [a(BT * Cc * 4) for _ in range(self.L)]
         self.ln1 = [a(BT * Cc * 2) for _ in range(self.L)]
@@ -123,7 +127,7 @@ class FusedTrainer:
         self._write_guard_state()
         self.loss_hist_cap = 4096
         self.loss_hist, self.norm_hist = a(self.loss_hist_cap * 4), a(self.loss_hist_cap * 16)
-        self._batches: List[Tuple[int, int]] = []
+        self._batches: List[Tuple[int, int, int]] = []
         self._have_batch = False
         # partial column sums of every LayerNorm backward (dw, db), reduced by ONE launch at the end of backward
         part_bytes = int(self.lib.ah_layernorm_bwd_partials_bytes(BT, Cc))
@@ -271,7 +275,10 @@ class FusedTrainer:
             ffi.AhColsumJob(part, self.g(name + ".weight"), self.g(name + ".bias"), BT, Cc, acc, 0) for name, part in self._ln_jobs])
         check(lib.ah_layernorm_colsums(jobs, len(self._ln_jobs)))
         self._weight_grads(wepi)
-        check(lib.ah_embedding_bwd(self.tok, self.dx[cur], self.g("wte"), BT, Cc, V, acc))
+        if self._index_bytes:
+            check(lib.ah_embedding_bwd_indexed(self.tok_index[micro], self.dx[cur], self.g("wte"), BT, Cc, V, acc))
+        else:
+            check(lib.ah_embedding_bwd(self.tok, self.dx[cur], self.g("wte"), BT, Cc, V, acc))
         check(lib.ah_pos_embedding_bwd(self.dx[cur], self.g("wpe"), self.batch, self.T, Cc, acc))
 
     def _optimizer(self):
@@ -306,6 +313,8 @@ class FusedTrainer:
         """Upload one [B, T] token batch straight into the resident slot of micro-step `micro` (nothing is retained: a loop
         that feeds a fresh batch every step allocates nothing); step() trains on the resident slots until they change."""
         self._upload_batch(inputs, targets, self.toks[micro], self.tgts[micro])
+        if self._index_bytes:
+            check(self.lib.ah_embedding_index(self.toks[micro], self.BT, self.V, self.tok_index[micro]))
         self._have_batch = True
 
     def add_batch(self, inputs: TensorData, targets: TensorData) -> int:
@@ -313,14 +322,19 @@ class FusedTrainer:
         n = self.BT * 4
         ti, tt = self._alloc(n), self._alloc(n)
         self._upload_batch(inputs, targets, ti, tt)
-        self._batches.append((ti, tt))
+        ix = 0
+        if self._index_bytes:
+            ix = self._alloc(self._index_bytes)
+            check(self.lib.ah_embedding_index(ti, self.BT, self.V, ix))
+        self._batches.append((ti, tt, ix))
         return len(self._batches) - 1
 
     def drop_batches(self):
         for pair in self._batches:
             for b in pair:
-                check(self.lib.ah_free(b))
-                self._bufs.remove(b)
+                if b:
+                    check(self.lib.ah_free(b))
+                    self._bufs.remove(b)
         self._batches = []
 
     def _use_batch(self, i, micro: int = 0):
@@ -331,9 +345,11 @@ class FusedTrainer:
             for m, bi in enumerate(i):
                 self._use_batch(bi, m)
             return
-        ti, tt = self._batches[i]
+        ti, tt, ix = self._batches[i]
         check(self.lib.ah_copy(self.toks[micro], ti, self.BT * 4))
         check(self.lib.ah_copy(self.tgts[micro], tt, self.BT * 4))
+        if ix:
+            check(self.lib.ah_copy(self.tok_index[micro], ix, self._index_bytes))
         self._have_batch = True
 
     def _write_guard_state(self, b1p: float = 1.0, b2p: float = 1.0, skipped: float = 0.0):

@@ -212,9 +212,20 @@ int32_t ah_embedding(ah_ptr weight, ah_ptr idx_i32, ah_ptr out, int64_t n_idx, i
 /* out[i] = wte[tok[i]] + wpe[i % T]  -- tok+pos embedding and the add of gpt.ts:362-379 in one pass */
 int32_t ah_embedding_tok_pos(ah_ptr wte, ah_ptr wpe, ah_ptr tok_i32, ah_ptr out, int64_t n_idx, int64_t T,
                              int64_t dim, int64_t vocab);
-/* grad_w[vocab,dim] = scatter-add of grad_out rows (zero-filled first unless accumulate != 0) */
+/* grad_w[vocab,dim] = scatter-add of grad_out rows (zero-filled first unless accumulate != 0); ids outside [0, vocab) are
+ * skipped.  Up to 32768 positions over fewer than 65535 ids (rows of 4 k floats) the order of the additions is fixed: the
+ * positions are sorted by (id, position), the rows of an id are added in position order inside chunks of 32 sorted positions
+ * (as the reference's loop adds them, packages/autograd/src/ops.ts:491-507) and the chunks of a longer run in chunk order, so
+ * the result is the same from run to run.  Beyond those sizes the rows are added with f32 atomics (order not fixed). */
 int32_t ah_embedding_bwd(ah_ptr idx_i32, ah_ptr grad_out, ah_ptr grad_w, int64_t n_idx, int64_t dim,
                          int64_t vocab, int32_t accumulate);
+/* The same in two steps for a token batch that stays on the device for several backward passes (a resident batch, the
+ * micro-batches of an accumulating step): ah_embedding_index sorts once into `index_out` (ah_embedding_index_bytes(n_idx, vocab)
+ * bytes; 0 = sizes outside the fixed-order path), ah_embedding_bwd_indexed is ah_embedding_bwd without the sort. */
+int64_t ah_embedding_index_bytes(int64_t n_idx, int64_t vocab);
+int32_t ah_embedding_index(ah_ptr idx_i32, int64_t n_idx, int64_t vocab, ah_ptr index_out);
+int32_t ah_embedding_bwd_indexed(ah_ptr index, ah_ptr grad_out, ah_ptr grad_w, int64_t n_idx, int64_t dim, int64_t vocab,
+                                 int32_t accumulate);
 /* grad_wpe[T,dim] (+)= sum over the batch of grad_out[b,t,:]  (positions are 0..T-1 per row) */
 int32_t ah_pos_embedding_bwd(ah_ptr grad_out, ah_ptr grad_wpe, int64_t batch, int64_t T, int64_t dim,
                              int32_t accumulate);

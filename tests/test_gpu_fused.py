@@ -192,7 +192,29 @@ def test_set_batch_reuses_the_resident_slot(B):
         ft.set_batch(*syntheticBatch(2 + s, 4, 64, 256))
     assert B.gpuMemStats()["liveAllocs"] == live
     i = ft.add_batch(*syntheticBatch(9, 4, 64, 256))
-    assert B.gpuMemStats()["liveAllocs"] == live + 2
+    assert B.gpuMemStats()["liveAllocs"] == live + 3                  # tokens, targets, sorted-position index
     ft.drop_batches()
     assert B.gpuMemStats()["liveAllocs"] == live and i == 0
     ft.close()
+
+
+def test_fused_step_is_bit_identical_from_run_to_run(B):
+    """Every sum of the step has a fixed order (split-K and grouped GEMM joins, LayerNorm column sums, the embedding
+    scatter-add over positions sorted by id, the gradient norm): two runs from the same seed give the same bits, and the
+    replayed graph gives the bits of eager execution."""
+    from alpha2_amd.train import syntheticBatch
+    runs = []
+    for graph in (False, False, True):
+        ft = _make(B, dict(iters=4), use_graph=graph, seed=9)
+        ids = [ft.add_batch(*syntheticBatch(400 + s, 4, 64, 256)) for s in range(4)]
+        for s in range(4):
+            ft.step(ids[s])
+        h = ft.history(0, 4)
+        runs.append(([(x.loss, x.gradNorm) for x in h], {n: ft.param(n) for n in ("wte", "wpe", "layer.0.attn.wqkv", "lnF.weight")},
+                     ft.grad("wte")))
+        ft.close()
+    for other in runs[1:]:
+        assert other[0] == runs[0][0]
+        assert np.array_equal(other[2], runs[0][2])
+        for n, v in runs[0][1].items():
+            assert np.array_equal(other[1][n], v), n

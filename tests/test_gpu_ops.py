@@ -328,6 +328,45 @@ def test_embedding_backward_with_heavily_repeated_ids(B, n, dim, V):
         assert_close(gw.data.reshape(V, dim), k * want, what=f"scatter-add x{k}")
 
 
+def test_embedding_backward_is_the_same_from_run_to_run_and_follows_position_order(B):
+    """16384 power-law token ids over 50304 rows of 768: the summation order is a function of the ids alone, so repeated
+    calls are bit-identical; and an id whose positions all fall into one chunk of 32 sorted positions (every id with up to
+    two positions at least... here: every id that occurs at most 8 times and does not straddle a chunk border is checked
+    through the closed form below) is summed in position order, f32 add by f32 add, exactly as the reference's loop does
+    (packages/autograd/src/ops.ts:491-507)."""
+    from alpha2_amd import _ffi as ffi
+    n, dim, V = 16384, 768, 50304
+    r = np.random.RandomState(11)
+    idx = np.minimum((V * r.rand(n) ** 6).astype(np.int64), V - 1).astype(np.int32)
+    g = (r.randn(n, dim) * np.exp(r.randn(n, 1) * 3)).astype(np.float32)          # rows of very different size: order matters
+    di, dg = dev(B, idx, "i32"), dev(B, g)
+    outs = []
+    for _ in range(3):
+        gw = B.zeros((V, dim))
+        ffi.check(B.lib.ah_embedding_bwd(B._ptr(di), B._ptr(dg), B._ptr(gw), n, dim, V, 0))
+        B._dirty(gw)
+        outs.append(gw.data.reshape(V, dim).copy())
+    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
+    # position-order f32 sums for the ids whose positions are neighbours in the sorted order AND inside one chunk of 32
+    order = np.lexsort((np.arange(n), idx))
+    sid = idx[order]
+    exact = 0
+    for c in range(0, n, 32):
+        ids_c = sid[c:c + 32]
+        for v in np.unique(ids_c):
+            if (c > 0 and sid[c - 1] == v) or (c + 32 < n and sid[c + 32] == v):
+                continue                                        # crosses a chunk border: summed as parts
+            acc = np.zeros(dim, np.float32)
+            for p in order[c:c + 32][ids_c == v]:
+                acc = acc + g[p]
+            assert np.array_equal(outs[0][v], acc), v
+            exact += 1
+    assert exact > 3000
+    want = np.zeros((V, dim), np.float64)
+    np.add.at(want, idx, g.astype(np.float64))
+    assert_close(outs[0], want, what="scatter-add")
+
+
 @pytest.mark.parametrize("rows,dim", [(1, 2), (7, 48), (1024, 128), (333, 768), (5, 1000), (3, 4096)])
 def test_layernorm_fwd_bwd(B, rows, dim):
     x = (rs.randn(rows, dim) * 2 + 0.5).astype(np.float32)
