@@ -57,6 +57,9 @@ struct Context {
   bool inited = false;
   int device = -1;
   hipStream_t stream = nullptr;
+  hipStream_t side = nullptr, cur = nullptr;      // side stream for ah_side_begin .. ah_side_end; cur = where launches go now
+  hipEvent_t side_ev[2] = {nullptr, nullptr};     // main -> side ("start after this"), side -> main ("wait for the side work")
+  bool side_used = false;
   hipDeviceProp_t prop;
   char err[512] = "";
   // allocator
@@ -101,7 +104,7 @@ size_t round_size(size_t b) {
 }  // namespace
 
 namespace ah {
-hipStream_t stream() { return g.stream; }
+hipStream_t stream() { return g.cur; }
 bool ready() { return g.inited; }
 int num_cus() { return g.prop.multiProcessorCount; }
 int current_device() { return g.device; }
@@ -229,7 +232,7 @@ int32_t step_close_segment(const char *what) {
 
 void launch_raw(const void *func, dim3 grid, dim3 block, unsigned shmem, void **args, const uint32_t *sizes, int nargs) {
   if (g.step_mode == STEP_OFF || g.step_mode == STEP_EAGER) {
-    (void)hipLaunchKernel(func, grid, block, args, shmem, g.stream);       // an error is picked up by hipGetLastError
+    (void)hipLaunchKernel(func, grid, block, args, shmem, g.cur);          // an error is picked up by hipGetLastError
     return;
   }
   if (g.step_mode == STEP_RECORD) {
@@ -350,6 +353,10 @@ int32_t ah_init(int32_t device) {
   if (strncmp(g.prop.gcnArchName, "gfx950", 6) != 0)
     return fail(AH_ERR_UNSUPPORTED, "ah_init: this library is built for gfx950 only, device is %s", g.prop.gcnArchName);
   AH_HIP(hipStreamCreateWithFlags(&g.stream, hipStreamNonBlocking));
+  AH_HIP(hipStreamCreateWithFlags(&g.side, hipStreamNonBlocking));       // same (default) priority as the main stream
+  AH_HIP(hipEventCreateWithFlags(&g.side_ev[0], hipEventDisableTiming));
+  AH_HIP(hipEventCreateWithFlags(&g.side_ev[1], hipEventDisableTiming));
+  g.cur = g.stream;
   g.scratch_bytes = size_t(64) << 20;
   AH_HIP(hipMalloc(&g.scratch, g.scratch_bytes));
   g.pinned_bytes = size_t(64) << 20;
@@ -387,6 +394,9 @@ int32_t ah_shutdown(void) {
   if (g.ring) (void)hipHostFree(g.ring);
   if (g.ring_ev[0]) (void)hipEventDestroy(g.ring_ev[0]);
   if (g.ring_ev[1]) (void)hipEventDestroy(g.ring_ev[1]);
+  if (g.side) { (void)hipStreamSynchronize(g.side); (void)hipStreamDestroy(g.side); }
+  if (g.side_ev[0]) (void)hipEventDestroy(g.side_ev[0]);
+  if (g.side_ev[1]) (void)hipEventDestroy(g.side_ev[1]);
   (void)hipStreamDestroy(g.stream);
   g = Context();
   return AH_OK;
@@ -410,6 +420,7 @@ int32_t ah_sync(void) {
   AH_REQUIRE_READY();
   if (g.capturing) return fail(AH_ERR_STATE, "ah_sync: illegal while a graph is being captured");
   { int32_t rc = step_boundary("ah_sync"); if (rc != AH_OK) return rc; }
+  if (g.side_used) AH_HIP(hipStreamSynchronize(g.side));
   AH_HIP(hipStreamSynchronize(g.stream));
   return step_resume();
 }
@@ -534,6 +545,7 @@ int32_t ah_download(void *host, ah_ptr src, uint64_t bytes) {
   if (bytes == 0) return AH_OK;
   AH_ARG(src != 0 && host != nullptr, "ah_download: null pointer");
   { int32_t rc = step_boundary("ah_download"); if (rc != AH_OK) return rc; }
+  if (g.side_used && !g.capturing) AH_HIP(hipStreamSynchronize(g.side));     // side work may be what wrote `src`
   struct Resume { ~Resume() { (void)step_resume(); } } resume_capture_on_return;
   char *dst = (char *)host;
   uint64_t off = 0;
@@ -609,6 +621,10 @@ int32_t ah_graph_begin(void) {
 int32_t ah_graph_end(uint64_t *out_graph) {
   AH_REQUIRE_READY();
   if (!g.capturing) return fail(AH_ERR_STATE, "ah_graph_end: no capture is open");
+  if (g.cur != g.stream || g.side_used) {                 // a capture cannot end with forked work outstanding
+    g.cur = g.stream;
+    if (g.side_used) { (void)hipEventRecord(g.side_ev[1], g.side); (void)hipStreamWaitEvent(g.stream, g.side_ev[1], 0); g.side_used = false; }
+  }
   Graph &gr = g.graphs[g.open_graph];
   hipError_t e = hipStreamEndCapture(g.stream, &gr.graph);
   g.capturing = false;
@@ -644,6 +660,31 @@ int32_t ah_graph_destroy(uint64_t graph) {
   if (it->second.graph) (void)hipGraphDestroy(it->second.graph);
   for (auto &b : it->second.reserved) { g.pool[b.bytes].push_back(b.ptr); g.pool_bytes += b.bytes; }
   g.graphs.erase(it);
+  return AH_OK;
+}
+
+int32_t ah_side_begin(void) {
+  AH_REQUIRE_READY();
+  if (g.cur != g.stream) return fail(AH_ERR_STATE, "ah_side_begin: the side stream is already open");
+  if (g.step_mode != STEP_OFF) return AH_OK;              // inside a step plan everything stays on the one recorded stream
+  AH_HIP(hipEventRecord(g.side_ev[0], g.stream));
+  AH_HIP(hipStreamWaitEvent(g.side, g.side_ev[0], 0));
+  g.cur = g.side;
+  g.side_used = true;
+  return AH_OK;
+}
+int32_t ah_side_end(void) {
+  AH_REQUIRE_READY();
+  g.cur = g.stream;
+  return AH_OK;
+}
+int32_t ah_side_join(void) {
+  AH_REQUIRE_READY();
+  if (g.cur != g.stream) return fail(AH_ERR_STATE, "ah_side_join: ah_side_end first");
+  if (!g.side_used) return AH_OK;
+  AH_HIP(hipEventRecord(g.side_ev[1], g.side));
+  AH_HIP(hipStreamWaitEvent(g.stream, g.side_ev[1], 0));
+  g.side_used = false;
   return AH_OK;
 }
 

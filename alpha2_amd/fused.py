@@ -46,7 +46,7 @@ class StepStats:
 
 class FusedTrainer:
     def __init__(self, backend: HipBackend, cfg: ModelConfig, tc: TrainConfig, batch: int, seed: int = 0, use_graph: bool = True,
-                 accum: int = 1, params: Optional[dict] = None):
+                 accum: int = 1, params: Optional[dict] = None, dw_groups: int = 1):
         if (cfg.ffnActivation or "gelu") != "gelu" or cfg.dropout != 0:
             raise ValueError("FusedTrainer schedules the default GELU block without dropout; use train.Trainer for the variants")
         self.B, self.lib, self.cfg, self.tc = backend, backend.lib, cfg, tc
@@ -56,6 +56,7 @@ class FusedTrainer:
         if self.D not in (32, 64, 128) or self.C % 8 or self.F % 64 or self.C % 64 or self.V % 8:
             raise ValueError("FusedTrainer needs head_dim in {32,64,128}, nEmbd and ffnDim multiples of 64, vocab multiple of 8")
         self.BT = batch * self.T
+        self.dw_groups = max(1, min(int(dw_groups), self.L))
         self.cap = cfg.softCap if cfg.softCap is not None else 30.0
         self._bufs: List[int] = []
         self._graph = None
@@ -139,40 +140,68 @@ class FusedTrainer:
         self._plan_weight_grads()
 
     def _plan_weight_grads(self):
-        """Descriptors of every dW = dY^T X of the step (TN layout: both operands token-major), lmHead first."""
+        """Descriptors of every dW = dY^T X of the step (TN layout: both operands token-major), lmHead first.  With
+        dw_groups = 1 they are ONE grouped launch at the end of backward.  With dw_groups = n the layers are cut into n
+        runs (the last layers, whose gradients exist first, and lmHead in run 0): run k is launched on the side stream as
+        soon as backward has passed its lowest layer, beside the backward kernels of the layers below."""
         BT, Cc, Fd, V, TN = self.BT, self.C, self.F, self.V, ffi.GEMM_TN
 
         def desc(dy, x, gname, m, n):
             return ffi.AhGemm(TN, BF16, F32, ffi.EPI_NONE, m, n, BT, m, n, n, 1, 0, 0, 0, dy, x, self.g(gname), 0)
-        descs = [desc(self.logits, self.lnf, "lmHead", V, Cc)]
-        for l in range(self.L):
-            pre = f"layer.{l}."
-            descs += [desc(self.dy_fc2[l], self.hact[l], pre + "mlp.fc2", Cc, Fd), desc(self.dh[l], self.ln2[l], pre + "mlp.fc1", Fd, Cc),
-                      desc(self.dy_wo[l], self.att[l], pre + "attn.wo", Cc, Cc), desc(self.dqkv[l], self.ln1[l], pre + "attn.wqkv", 3 * Cc, Cc)]
-        self._dw_descs = descs
-        self._dw_flops = sum(2.0 * d.m * d.n * d.k for d in descs)
-        self._dw_plan = None
-        if BT % 64 == 0:                          # the grouped kernel contracts in k-tiles of 64 tokens
-            arr = (ffi.AhGemm * len(descs))(*descs)
-            plan = C.c_uint64()
-            check(self.lib.ah_gemm_grouped_plan(arr, len(descs), C.byref(plan)))
-            self._dw_plan = plan.value
 
-    def _weight_grads(self, epilogue: int):
-        if self._dw_plan is None:                 # odd token counts: one general GEMM per weight
-            for d in self._dw_descs:
-                self._gemm(d.layout, d.a, d.b, d.c, d.m, d.n, d.k, d.lda, d.ldb, d.ldc, F32, epilogue)
-            return
-        if self._timed is None:
-            check(self.lib.ah_gemm_grouped_run(self._dw_plan, epilogue))
-            return
-        e0, e1 = self.B._event(), self.B._event()
-        check(self.lib.ah_event_record(e0))
-        check(self.lib.ah_gemm_grouped_run(self._dw_plan, epilogue))
-        check(self.lib.ah_event_record(e1))
-        kernel, nsplit = self.B.lastGemmKernel()
-        self._timed.append({"kind": "gemm", "kernel": kernel, "nsplit": nsplit, "layout": ffi.GEMM_TN, "m": 0, "n": 0, "k": self.BT,
-                            "flops": self._dw_flops, "e0": e0, "e1": e1})
+        def layer(l):
+            pre = f"layer.{l}."
+            return [desc(self.dy_fc2[l], self.hact[l], pre + "mlp.fc2", Cc, Fd), desc(self.dh[l], self.ln2[l], pre + "mlp.fc1", Fd, Cc),
+                    desc(self.dy_wo[l], self.att[l], pre + "attn.wo", Cc, Cc), desc(self.dqkv[l], self.ln1[l], pre + "attn.wqkv", 3 * Cc, Cc)]
+        n = self.dw_groups
+        bounds = [self.L - (self.L * (k + 1)) // n for k in range(n)]          # lowest layer of run k (run n-1 ends at layer 0)
+        self._dw_after_layer = {}                                                # layer whose backward completes run k -> k
+        groups, hi = [], self.L
+        for k, lo in enumerate(bounds):
+            d = [desc(self.logits, self.lnf, "lmHead", V, Cc)] if k == 0 else []
+            if n == 1:                                                           # the order the single launch has always had
+                for l in range(self.L):
+                    d += layer(l)
+            else:
+                for l in reversed(range(lo, hi)):
+                    d += layer(l)
+            groups.append(d)
+            self._dw_after_layer[lo] = k
+            hi = lo
+        self._dw_descs = [d for g_ in groups for d in g_]
+        self._dw_group_descs = groups
+        self._dw_flops = [sum(2.0 * d.m * d.n * d.k for d in g_) for g_ in groups]
+        self._dw_plans = None
+        if BT % 64 == 0:                          # the grouped kernel contracts in k-tiles of 64 tokens
+            self._dw_plans = []
+            for g_ in groups:
+                arr = (ffi.AhGemm * len(g_))(*g_)
+                plan = C.c_uint64()
+                check(self.lib.ah_gemm_grouped_plan(arr, len(g_), C.byref(plan)))
+                self._dw_plans.append(plan.value)
+
+    def _weight_grads(self, epilogue: int, k: int):
+        """Run k of the weight gradients (all of them when dw_groups = 1)."""
+        side = self.dw_groups > 1 and self._timed is None
+        if side:
+            check(self.lib.ah_side_begin())
+        try:
+            if self._dw_plans is None:            # odd token counts: one general GEMM per weight
+                for d in self._dw_group_descs[k]:
+                    self._gemm(d.layout, d.a, d.b, d.c, d.m, d.n, d.k, d.lda, d.ldb, d.ldc, F32, epilogue)
+            elif self._timed is None:
+                check(self.lib.ah_gemm_grouped_run(self._dw_plans[k], epilogue))
+            else:
+                e0, e1 = self.B._event(), self.B._event()
+                check(self.lib.ah_event_record(e0))
+                check(self.lib.ah_gemm_grouped_run(self._dw_plans[k], epilogue))
+                check(self.lib.ah_event_record(e1))
+                kernel, nsplit = self.B.lastGemmKernel()
+                self._timed.append({"kind": "gemm", "kernel": kernel, "nsplit": nsplit, "layout": ffi.GEMM_TN, "m": 0, "n": 0, "k": self.BT,
+                                    "flops": self._dw_flops[k], "e0": e0, "e1": e1})
+        finally:
+            if side:
+                check(self.lib.ah_side_end())
 
     # ------------------------------------------------------------------ helpers
     def _alloc(self, nbytes: int) -> int:
@@ -271,15 +300,20 @@ class FusedTrainer:
             check(lib.ah_layernorm_bwd_deferred(self.x[l], self.p(pre + "ln1.weight"), self.dlnb, BF16, self.dx[cur], self.dx[cur ^ 1],
                                                 self.dy_fc2[l - 1] if l > 0 else self.dxb0, self._ln_part[pre + "ln1"], BT, Cc, 1e-5))
             cur ^= 1
+            if self.dw_groups > 1 and l in self._dw_after_layer:
+                self._weight_grads(wepi, self._dw_after_layer[l])
         jobs = (ffi.AhColsumJob * len(self._ln_jobs))(*[
             ffi.AhColsumJob(part, self.g(name + ".weight"), self.g(name + ".bias"), BT, Cc, acc, 0) for name, part in self._ln_jobs])
         check(lib.ah_layernorm_colsums(jobs, len(self._ln_jobs)))
-        self._weight_grads(wepi)
+        if self.dw_groups == 1:
+            self._weight_grads(wepi, 0)
         if self._index_bytes:
             check(lib.ah_embedding_bwd_indexed(self.tok_index[micro], self.dx[cur], self.g("wte"), BT, Cc, V, acc))
         else:
             check(lib.ah_embedding_bwd(self.tok, self.dx[cur], self.g("wte"), BT, Cc, V, acc))
         check(lib.ah_pos_embedding_bwd(self.dx[cur], self.g("wpe"), self.batch, self.T, Cc, acc))
+        if self.dw_groups > 1:                    # the next micro-step overwrites the operands, the optimizer reads the results
+            check(lib.ah_side_join())
 
     def _optimizer(self):
         lib, tc = self.lib, self.tc
@@ -523,9 +557,9 @@ class FusedTrainer:
         if self._graph is not None:
             check(self.lib.ah_graph_destroy(self._graph))
             self._graph = None
-        if self._dw_plan is not None:
-            check(self.lib.ah_gemm_grouped_destroy(self._dw_plan))
-            self._dw_plan = None
+        for plan in self._dw_plans or []:
+            check(self.lib.ah_gemm_grouped_destroy(plan))
+        self._dw_plans = None
         for b in self._bufs:
             self.lib.ah_free(b)
         self._bufs = []

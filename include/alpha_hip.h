@@ -117,6 +117,17 @@ int32_t     ah_step_end(int32_t *out_how);
 int32_t     ah_step_reset(uint64_t key);          /* drop the plan of `key` */
 const char *ah_step_note(void);                    /* why the last step fell back ("" if it did not) */
 
+/* ---- a side stream (same priority) for work nothing depends on for a while, e.g. weight gradients, which only the
+ *      gradient norm reads: launches between ah_side_begin and ah_side_end go to the side stream, which first waits for
+ *      everything issued on the main stream so far; the main stream carries on at once.  ah_side_join makes the main stream
+ *      wait for all side work.  Legal inside ah_graph_begin .. ah_graph_end (the fork and join become graph edges; join
+ *      before ah_graph_end) and a no-op inside a step plan.  Allocation and frees stay ordered on the main stream: buffers
+ *      that side work reads or writes must not be freed before ah_side_join.  No counterpart in the reference, whose
+ *      dispatches are strictly serial (helios_vk.c:3291-3328 orders them with buffer barriers). ---- */
+int32_t ah_side_begin(void);
+int32_t ah_side_end(void);
+int32_t ah_side_join(void);
+
 /* ---- timing on the library stream.  Replaces gpuTime (helios_vk.c:3448). ---- */
 int32_t ah_event_create(uint64_t *out_event);
 int32_t ah_event_record(uint64_t event);

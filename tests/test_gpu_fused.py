@@ -218,3 +218,27 @@ def test_fused_step_is_bit_identical_from_run_to_run(B):
         assert np.array_equal(other[2], runs[0][2])
         for n, v in runs[0][1].items():
             assert np.array_equal(other[1][n], v), n
+
+
+@pytest.mark.parametrize("graph", [False, True])
+@pytest.mark.parametrize("accum", [1, 2])
+def test_weight_gradients_on_the_side_stream_give_the_same_step(B, graph, accum):
+    """dw_groups = 2 launches the weight-gradient GEMMs of the upper layer beside the backward kernels of the lower one on
+    a second stream; every product keeps its own kernel configuration, so the step must not change by a bit."""
+    from alpha2_amd.fused import FusedTrainer
+    from alpha2_amd.model import ModelConfig
+    from alpha2_amd.train import TrainConfig, syntheticBatch
+    mk = lambda groups: FusedTrainer(B, ModelConfig(**CFG), TrainConfig(iters=6, gradAccumSteps=accum), 4, seed=0, use_graph=graph,
+                                     accum=accum, dw_groups=groups)
+    one, two = mk(1), mk(2)
+    batches = [syntheticBatch(3 + m, 4, 64, 256) for m in range(accum)]
+    i1, i2 = [one.add_batch(*b) for b in batches], [two.add_batch(*b) for b in batches]
+    for _ in range(4):
+        one.step(i1 if accum > 1 else i1[0])
+        two.step(i2 if accum > 1 else i2[0])
+    h1, h2 = one.history(0, 4), two.history(0, 4)
+    for a, b in zip(h1, h2):
+        assert a.loss == b.loss and a.gradNorm == b.gradNorm, (a, b)
+    for name in ("wte", "lmHead", "layer.0.attn.wqkv", "layer.1.mlp.fc2", "layer.1.ln1.weight"):
+        assert np.array_equal(one.param(name), two.param(name)), name
+    one.close(), two.close()
