@@ -1,10 +1,13 @@
 """Per-op microbenchmarks on the shapes of the training step, in the manner of the reference's scripts/bench-ops.ts
 (3 warm-up calls, then the mean of `iters` calls; TFLOP/s = flops / time, GB/s = algorithmic bytes / time):
 
-    python -m alpha2_amd.bench_ops [--iters 10] [--only gemm|flash|bandwidth] [--json]
+    python -m alpha2_amd.bench_ops [--iters 10] [--only gemm|flash|bandwidth|epilogue] [--json]
 
 * GEMM: C = A B^T and both backward products, M = 16384 (batch x context), K = 768, N in {768, 2304, 3072, 50304},
   bf16 operands with fp32 accumulation and fp32 throughout; flops 2 M N K (scripts/bench-ops.ts:302,328).
+* `--only epilogue` (not part of the default run): the fc1-shaped product M = 16384, N = 3072, K = 768 (and fc2's dX, K and
+  N swapped) with every epilogue the library has, to separate what an epilogue's arithmetic costs from what its second
+  operand or second result costs: each epilogue is its own kernel instance, so a counter run sees them apart.
 * Causal flash attention forward and backward: B = 16, H = 12, head size 64, T in {256, 1024, 2048}, bf16, with and
   without the soft cap of 30; flops counted non-causal like the reference: 4 B H T^2 D forward, 8 B H T^2 D backward
   (scripts/bench-ops.ts:652,673).
@@ -109,6 +112,35 @@ def bench_gemm(b: Bench):
             b.release()
 
 
+def bench_epilogues(b: Bench):
+    """One product shape, every epilogue.  bytes beside the operands: plain 1 store; GELU 2 stores (7 operations per element:
+    C = gelu(acc), aux = acc); GELU_GRAD 2 stores (11 operations: C = gelu(acc), aux = gelu'(acc)); GELU_BWD 1 load + 1 store
+    (11 operations); MUL_AUX 1 load + 1 store (1 operation); RESIDUAL 1 f32 load + 1 f32 store (1 operation)."""
+    M, K, N = 16384, 768, 3072
+    a, w = b.randn(M * K, ffi.BF16, 1.0), b.randn(N * K, ffi.BF16, 0.02)
+    g, w2 = b.randn(M * K, ffi.BF16, 0.02, 5), b.randn(K * N, ffi.BF16, 0.02, 6)     # dY [M,768] . W2 [768,3072] (NN)
+    aux_bf, aux_f = b.randn(M * N, ffi.BF16, 1.0, 7), b.randn(M * N, ffi.F32, 1.0, 8)
+    c_bf, c_f = b.alloc(M * N * 2), b.alloc(M * N * 4)
+    flops = 2.0 * M * N * K
+    nt, nn = (ffi.GEMM_NT, (M, N, K, K, K, N), a, w), (ffi.GEMM_NN, (M, N, K, K, N, N), g, w2)
+    for label, (layout, (m, n, k, lda, ldb, ldc), pa, pb), out, epi, aux, pc in (
+            ("fc1 fwd plain", nt, ffi.BF16, ffi.EPI_NONE, 0, c_bf),
+            ("fc1 fwd gelu, saves acc", nt, ffi.BF16, ffi.EPI_GELU, aux_bf, c_bf),
+            ("fc1 fwd gelu, saves gelu'", nt, ffi.BF16, ffi.EPI_GELU_GRAD, aux_bf, c_bf),
+            ("fc1 fwd * aux", nt, ffi.BF16, ffi.EPI_MUL_AUX, aux_bf, c_bf),
+            ("fc1 fwd * gelu'(aux)", nt, ffi.BF16, ffi.EPI_GELU_BWD, aux_bf, c_bf),
+            ("fc1 fwd plain, f32 out", nt, ffi.F32, ffi.EPI_NONE, 0, c_f),
+            ("fc1 fwd + residual, f32 out", nt, ffi.F32, ffi.EPI_RESIDUAL, aux_f, c_f),
+            ("fc2 dX plain", nn, ffi.BF16, ffi.EPI_NONE, 0, c_bf),
+            ("fc2 dX * aux", nn, ffi.BF16, ffi.EPI_MUL_AUX, aux_bf, c_bf),
+            ("fc2 dX * gelu'(aux)", nn, ffi.BF16, ffi.EPI_GELU_BWD, aux_bf, c_bf)):
+        d = ffi.AhGemm(layout, ffi.BF16, out, epi, m, n, k, lda, ldb, ldc, 1, 0, 0, 0, pa, pb, pc, aux)
+        ms = b.time(lambda: ffi.check(b.lib.ah_gemm(C.byref(d))))
+        kern, nsplit = b.B.lastGemmKernel()
+        b.record(f"{label}", ms, flops=flops, note=kern)
+    b.release()
+
+
 def bench_flash(b: Bench):
     Bt, H, D = 16, 12, 64
     Cc = H * D
@@ -189,7 +221,7 @@ def bench_bandwidth(b: Bench):
 def main(argv=None):
     ap = argparse.ArgumentParser(description=__doc__.split("\n")[0])
     ap.add_argument("--iters", type=int, default=10)
-    ap.add_argument("--only", choices=["gemm", "flash", "bandwidth"])
+    ap.add_argument("--only", choices=["gemm", "flash", "bandwidth", "epilogue"])
     ap.add_argument("--json", action="store_true", help="also print one JSON line with every row")
     args = ap.parse_args(argv)
     b = Bench(args.iters)
@@ -197,6 +229,8 @@ def main(argv=None):
     for name, fn in (("gemm", bench_gemm), ("flash", bench_flash), ("bandwidth", bench_bandwidth)):
         if args.only in (None, name):
             fn(b)
+    if args.only == "epilogue":
+        bench_epilogues(b)
     if args.json:
         print(json.dumps(b.rows))
     return 0
