@@ -516,7 +516,7 @@ class HipBackend:
         """out = sum over the given bases of coef[channel] * basis(x): the universal / kan_spline MLP activations in one pass."""
         mask, arr, cols, rows = self._channel_args(x, coefs)
         out = self._new(x.shape)
-        check(self.lib.ah_channel_act(self._ptr(x), arr, mask, out._buf.ptr, rows, cols))
+        check(self.lib.ah_channel_act(ffi.F32, self._ptr(x), arr, mask, out._buf.ptr, rows, cols))
         return out
 
     def channelActBackward(self, x: TensorData, coefs: dict, g: TensorData):
@@ -528,7 +528,7 @@ class HipBackend:
         darr = (C.c_uint64 * 5)()
         for name, t in dco.items():
             darr[self.CHANNEL_BASES.index(name)] = t._buf.ptr
-        check(self.lib.ah_channel_act_bwd(self._ptr(x), arr, mask, self._ptr(g), dx._buf.ptr, darr, rows, cols))
+        check(self.lib.ah_channel_act_bwd(ffi.F32, self._ptr(x), arr, mask, self._ptr(g), dx._buf.ptr, darr, 0, rows, cols))
         return dx, dco
 
     def residualDropoutAdd(self, residual, projected, mask) -> TensorData:

@@ -71,27 +71,52 @@ __device__ __forceinline__ void basis_eval(int k, float x, float &v, float &d) {
     default: v = x * x; d = 2.0f * x; break;
   }
 }
-__global__ void k_channel_act(const float *__restrict__ x, ChannelAct p, float *__restrict__ out, int64_t rows, int cols4) {
+// four consecutive elements of an f32 or bf16 row (i counts quads)
+template <class T> __device__ __forceinline__ void ld4(const T *p, int64_t i, float v[4]);
+template <> __device__ __forceinline__ void ld4<float>(const float *p, int64_t i, float v[4]) {
+  float4 u = reinterpret_cast<const float4 *>(p)[i];
+  v[0] = u.x; v[1] = u.y; v[2] = u.z; v[3] = u.w;
+}
+template <> __device__ __forceinline__ void ld4<uint16_t>(const uint16_t *p, int64_t i, float v[4]) {
+  uint2 u = reinterpret_cast<const uint2 *>(p)[i];
+  v[0] = bf16_bits_to_f32(u.x & 0xffffu); v[1] = bf16_bits_to_f32(u.x >> 16);
+  v[2] = bf16_bits_to_f32(u.y & 0xffffu); v[3] = bf16_bits_to_f32(u.y >> 16);
+}
+template <class T> __device__ __forceinline__ void st4(T *p, int64_t i, const float v[4]);
+template <> __device__ __forceinline__ void st4<float>(float *p, int64_t i, const float v[4]) {
+  reinterpret_cast<float4 *>(p)[i] = make_float4(v[0], v[1], v[2], v[3]);
+}
+template <> __device__ __forceinline__ void st4<uint16_t>(uint16_t *p, int64_t i, const float v[4]) {
+  reinterpret_cast<uint2 *>(p)[i] = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+}
+// coefficient quad of basis k at column quad c4; a null vector is the constant 1 (a plain activation)
+__device__ __forceinline__ void coef4(const ChannelAct &p, int k, int c4, float cs[4]) {
+  if (p.coef[k]) ld4<float>(p.coef[k], c4, cs);
+  else cs[0] = cs[1] = cs[2] = cs[3] = 1.0f;
+}
+template <class T>
+__global__ void k_channel_act(const T *__restrict__ x, ChannelAct p, T *__restrict__ out, int64_t rows, int cols4) {
   int64_t n4 = rows * (int64_t)cols4;
   for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n4; i += (int64_t)gridDim.x * blockDim.x) {
     int c4 = (int)(i % cols4);
-    float4 xv = reinterpret_cast<const float4 *>(x)[i];
-    float xs[4] = {xv.x, xv.y, xv.z, xv.w}, acc[4] = {0.f, 0.f, 0.f, 0.f};
+    float xs[4], acc[4] = {0.f, 0.f, 0.f, 0.f};
+    ld4<T>(x, i, xs);
 #pragma unroll
     for (int k = 0; k < 5; k++)
       if (p.mask >> k & 1) {
-        float4 cv = reinterpret_cast<const float4 *>(p.coef[k])[c4];
-        float cs[4] = {cv.x, cv.y, cv.z, cv.w};
+        float cs[4];
+        coef4(p, k, c4, cs);
 #pragma unroll
         for (int e = 0; e < 4; e++) { float v, d; basis_eval(k, xs[e], v, d); acc[e] += cs[e] * v; }
       }
-    reinterpret_cast<float4 *>(out)[i] = make_float4(acc[0], acc[1], acc[2], acc[3]);
+    st4<T>(out, i, acc);
   }
 }
 // Backward: dx = g * sum_k coef_k basis_k'(x); partial[rb][k][c] = sum over the rows of row block rb of g * basis_k(x).
-// A block is 64 column quads x 4 row lanes; a wave reads 1 KB of one row.
+// A block is 64 column quads x 4 row lanes; a wave reads 1 KB (f32) of one row.
 constexpr int CA_ROWLANES = 4;
-__global__ __launch_bounds__(256) void k_channel_act_bwd(const float *__restrict__ x, const float *__restrict__ g, ChannelAct p, float *__restrict__ dx,
+template <class T>
+__global__ __launch_bounds__(256) void k_channel_act_bwd(const T *__restrict__ x, const T *__restrict__ g, ChannelAct p, T *__restrict__ dx,
                                                          float *__restrict__ partial, int64_t rows, int cols4, int rows_per_block) {
   __shared__ float4 red[5][CA_ROWLANES][64];
   const int cq = threadIdx.x & 63, rl = threadIdx.x >> 6, c4 = blockIdx.x * 64 + cq;
@@ -101,40 +126,79 @@ __global__ __launch_bounds__(256) void k_channel_act_bwd(const float *__restrict
     float cs[5][4] = {};
 #pragma unroll
     for (int k = 0; k < 5; k++)
-      if (p.mask >> k & 1) { float4 cv = reinterpret_cast<const float4 *>(p.coef[k])[c4]; cs[k][0] = cv.x; cs[k][1] = cv.y; cs[k][2] = cv.z; cs[k][3] = cv.w; }
+      if (p.mask >> k & 1) coef4(p, k, c4, cs[k]);
     for (int64_t r = r0 + rl; r < r1; r += CA_ROWLANES) {
       int64_t i = r * cols4 + c4;
-      float4 xv = reinterpret_cast<const float4 *>(x)[i], gv = reinterpret_cast<const float4 *>(g)[i];
-      float xs[4] = {xv.x, xv.y, xv.z, xv.w}, gs[4] = {gv.x, gv.y, gv.z, gv.w}, acc[4] = {0.f, 0.f, 0.f, 0.f};
+      float xs[4], gs[4], acc[4] = {0.f, 0.f, 0.f, 0.f};
+      ld4<T>(x, i, xs);
+      ld4<T>(g, i, gs);
 #pragma unroll
       for (int k = 0; k < 5; k++)
         if (p.mask >> k & 1) {
 #pragma unroll
           for (int e = 0; e < 4; e++) { float v, d; basis_eval(k, xs[e], v, d); acc[e] += cs[k][e] * d; sums[k][e] += gs[e] * v; }
         }
-      reinterpret_cast<float4 *>(dx)[i] = make_float4(gs[0] * acc[0], gs[1] * acc[1], gs[2] * acc[2], gs[3] * acc[3]);
+      const float o[4] = {gs[0] * acc[0], gs[1] * acc[1], gs[2] * acc[2], gs[3] * acc[3]};
+      st4<T>(dx, i, o);
     }
   }
+  if (!partial) return;                               // no coefficient has a gradient (block-uniform)
 #pragma unroll
   for (int k = 0; k < 5; k++) red[k][rl][cq] = make_float4(sums[k][0], sums[k][1], sums[k][2], sums[k][3]);
   __syncthreads();
   if (rl == 0 && c4 < cols4) {
 #pragma unroll
     for (int k = 0; k < 5; k++)
-      if (p.mask >> k & 1) {
+      if (p.dcoef[k]) {
         float4 a = red[k][0][cq];
         for (int j = 1; j < CA_ROWLANES; j++) { float4 b = red[k][j][cq]; a.x += b.x; a.y += b.y; a.z += b.z; a.w += b.w; }
         reinterpret_cast<float4 *>(partial + ((int64_t)blockIdx.y * 5 + k) * cols4 * 4)[c4] = a;
       }
   }
 }
-// dcoef_k[c] = sum over row blocks of partial[rb][k][c], in double, fixed order
-__global__ void k_channel_act_colsum(const float *__restrict__ partial, ChannelAct p, int nrb, int cols) {
+// dcoef_k[c] = (accumulate ? dcoef_k[c] : 0) + sum over row blocks of partial[rb][k][c], in double, fixed order
+__global__ void k_channel_act_colsum(const float *__restrict__ partial, ChannelAct p, int nrb, int cols, int accumulate) {
   int c = blockIdx.x * blockDim.x + threadIdx.x, k = blockIdx.y;
-  if (c >= cols || !(p.mask >> k & 1)) return;
+  if (c >= cols || !p.dcoef[k]) return;
   double s = 0;
   for (int rb = 0; rb < nrb; rb++) s += (double)partial[((int64_t)rb * 5 + k) * cols + c];
-  p.dcoef[k][c] = (float)s;
+  p.dcoef[k][c] = accumulate ? (float)((double)p.dcoef[k][c] + s) : (float)s;
+}
+
+// SwiGLU on the packed pre-activation gu = [gate | up], rows of 2 * cols (packages/model/src/gpt.ts:295-299; the element
+// arithmetic of Backend.siluMul / siluMulBackward, ops.ts:284-417):  out = silu(gate) * up;
+// dgate = g * up * s (1 + gate (1 - s)),  dup = g * gate * s,  s = sigmoid(gate).
+template <class T>
+__global__ void k_swiglu(const T *__restrict__ gu, T *__restrict__ out, int64_t rows, int cols4) {
+  int64_t n4 = rows * (int64_t)cols4;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n4; i += (int64_t)gridDim.x * blockDim.x) {
+    int64_t r = i / cols4, c4 = i - r * cols4;
+    float a[4], b[4], o[4];
+    ld4<T>(gu, r * 2 * cols4 + c4, a);
+    ld4<T>(gu, r * 2 * cols4 + cols4 + c4, b);
+#pragma unroll
+    for (int e = 0; e < 4; e++) o[e] = a[e] / (1.0f + expf(-a[e])) * b[e];
+    st4<T>(out, i, o);
+  }
+}
+template <class T>
+__global__ void k_swiglu_bwd(const T *__restrict__ gu, const T *__restrict__ g, T *__restrict__ dgu, int64_t rows, int cols4) {
+  int64_t n4 = rows * (int64_t)cols4;
+  for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n4; i += (int64_t)gridDim.x * blockDim.x) {
+    int64_t r = i / cols4, c4 = i - r * cols4;
+    float a[4], b[4], gs[4], da[4], db[4];
+    ld4<T>(gu, r * 2 * cols4 + c4, a);
+    ld4<T>(gu, r * 2 * cols4 + cols4 + c4, b);
+    ld4<T>(g, i, gs);
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      float s = 1.0f / (1.0f + expf(-a[e]));
+      da[e] = gs[e] * b[e] * s * (1.0f + a[e] * (1.0f - s));
+      db[e] = gs[e] * a[e] * s;
+    }
+    st4<T>(dgu, r * 2 * cols4 + c4, da);
+    st4<T>(dgu, r * 2 * cols4 + cols4 + c4, db);
+  }
 }
 
 template <class F>
@@ -435,41 +499,46 @@ int32_t ah_silu_mul_bwd(ah_ptr a, ah_ptr b, ah_ptr g, ah_ptr da, ah_ptr db, uint
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
-// mask: bit k selects basis k (0 silu, 1 relu, 2 gelu, 3 identity, 4 square); coefs[k] = f32[cols] for the selected ones
-static int32_t channel_act_args(const char *who, const ah_ptr *coefs, int32_t mask, int64_t rows, int64_t cols, ChannelAct &p, const ah_ptr *dcoefs) {
+// mask: bit k selects basis k (0 silu, 1 relu, 2 gelu, 3 identity, 4 square); coefs[k] = f32[cols] for the selected ones,
+// 0 for the constant 1 (then no gradient is produced for it)
+static int32_t channel_act_args(const char *who, int32_t dtype, const ah_ptr *coefs, int32_t mask, int64_t rows, int64_t cols, ChannelAct &p, const ah_ptr *dcoefs) {
+  AH_ARG(dtype == AH_F32 || dtype == AH_BF16, "%s: dtype must be AH_F32 or AH_BF16", who);
   AH_ARG(mask > 0 && mask < 32, "%s: basis mask %d selects nothing or an unknown basis", who, mask);
   AH_ARG(rows >= 0 && cols > 0 && cols % 4 == 0 && cols < (1ll << 31), "%s: cols %lld must be a positive multiple of 4", who, (long long)cols);
-  AH_ARG(coefs != nullptr, "%s: null coefficient list", who);
   p.mask = mask;
   for (int k = 0; k < 5; k++) {
-    bool on = mask >> k & 1;
-    AH_ARG(!on || (coefs[k] != 0 && coefs[k] % 16 == 0), "%s: coefficient vector %d missing or not 16-byte aligned", who, k);
+    bool on = (mask >> k & 1) && coefs && coefs[k] != 0;
+    AH_ARG(!on || coefs[k] % 16 == 0, "%s: coefficient vector %d is not 16-byte aligned", who, k);
     AH_ARG(!on || !dcoefs || dcoefs[k] != 0, "%s: gradient vector %d missing", who, k);
     p.coef[k] = on ? dp<const float>(coefs[k]) : nullptr;
     p.dcoef[k] = on && dcoefs ? dp<float>(dcoefs[k]) : nullptr;
   }
   return AH_OK;
 }
-int32_t ah_channel_act(ah_ptr x, const ah_ptr *coefs, int32_t mask, ah_ptr out, int64_t rows, int64_t cols) {
+int32_t ah_channel_act(int32_t dtype, ah_ptr x, const ah_ptr *coefs, int32_t mask, ah_ptr out, int64_t rows, int64_t cols) {
   AH_REQUIRE_READY();
   ChannelAct p;
-  int32_t rc = channel_act_args("ah_channel_act", coefs, mask, rows, cols, p, nullptr);
+  int32_t rc = channel_act_args("ah_channel_act", dtype, coefs, mask, rows, cols, p, nullptr);
   if (rc) return rc;
   if (rows == 0) return AH_OK;
   AH_ARG(x && out && aligned16(x) && aligned16(out), "ah_channel_act: operands must be non-null and 16-byte aligned");
-  ah::launch_kernel(k_channel_act, dim3(grid_for((uint64_t)(rows * cols / 4))), dim3(TPB), 0, dp<const float>(x), p, dp<float>(out), rows, (int)(cols / 4));
+  const dim3 grid(grid_for((uint64_t)(rows * cols / 4)));
+  if (dtype == AH_F32) ah::launch_kernel(k_channel_act<float>, grid, dim3(TPB), 0, dp<const float>(x), p, dp<float>(out), rows, (int)(cols / 4));
+  else ah::launch_kernel(k_channel_act<uint16_t>, grid, dim3(TPB), 0, dp<const uint16_t>(x), p, dp<uint16_t>(out), rows, (int)(cols / 4));
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
-int32_t ah_channel_act_bwd(ah_ptr x, const ah_ptr *coefs, int32_t mask, ah_ptr grad_out, ah_ptr dx, const ah_ptr *dcoefs, int64_t rows, int64_t cols) {
+int32_t ah_channel_act_bwd(int32_t dtype, ah_ptr x, const ah_ptr *coefs, int32_t mask, ah_ptr grad_out, ah_ptr dx, const ah_ptr *dcoefs,
+                           int32_t accumulate, int64_t rows, int64_t cols) {
   AH_REQUIRE_READY();
-  AH_ARG(dcoefs != nullptr, "ah_channel_act_bwd: null gradient list");
   ChannelAct p;
-  int32_t rc = channel_act_args("ah_channel_act_bwd", coefs, mask, rows, cols, p, dcoefs);
+  int32_t rc = channel_act_args("ah_channel_act_bwd", dtype, coefs, mask, rows, cols, p, dcoefs);
   if (rc) return rc;
+  bool any = false;
+  for (int k = 0; k < 5; k++) any = any || p.dcoef[k];
   if (rows == 0) {
     for (int k = 0; k < 5; k++)
-      if (mask >> k & 1) { rc = ah_fill_f32(dcoefs[k], 0.f, (uint64_t)cols); if (rc) return rc; }
+      if (p.dcoef[k] && !accumulate) { rc = ah_fill_f32(dcoefs[k], 0.f, (uint64_t)cols); if (rc) return rc; }
     return AH_OK;
   }
   AH_ARG(x && grad_out && dx && aligned16(x) && aligned16(grad_out) && aligned16(dx), "ah_channel_act_bwd: operands must be non-null and 16-byte aligned");
@@ -479,12 +548,54 @@ int32_t ah_channel_act_bwd(ah_ptr x, const ah_ptr *coefs, int32_t mask, ah_ptr g
   if (nrb > cap) nrb = cap;
   const int rpb = (int)cdiv(rows, nrb);
   nrb = (int)cdiv(rows, rpb);
-  float *partial = (float *)scratch(sizeof(float) * 5 * (size_t)nrb * (size_t)cols);
-  if (!partial) return fail(AH_ERR_OOM, "ah_channel_act_bwd: no scratch");
-  ah::launch_kernel(k_channel_act_bwd, dim3(gx, nrb), dim3(256), 0, dp<const float>(x), dp<const float>(grad_out), p, dp<float>(dx), partial,
-                     rows, cols4, rpb);
+  float *partial = nullptr;
+  if (any) {
+    partial = (float *)scratch(sizeof(float) * 5 * (size_t)nrb * (size_t)cols);
+    if (!partial) return fail(AH_ERR_OOM, "ah_channel_act_bwd: no scratch");
+  }
+  if (dtype == AH_F32)
+    ah::launch_kernel(k_channel_act_bwd<float>, dim3(gx, nrb), dim3(256), 0, dp<const float>(x), dp<const float>(grad_out), p, dp<float>(dx), partial,
+                       rows, cols4, rpb);
+  else
+    ah::launch_kernel(k_channel_act_bwd<uint16_t>, dim3(gx, nrb), dim3(256), 0, dp<const uint16_t>(x), dp<const uint16_t>(grad_out), p, dp<uint16_t>(dx),
+                       partial, rows, cols4, rpb);
   AH_LAUNCH_CHECK();
-  ah::launch_kernel(k_channel_act_colsum, dim3((unsigned)cdiv(cols, 256), 5), dim3(256), 0, partial, p, nrb, (int)cols);
+  if (any) {
+    ah::launch_kernel(k_channel_act_colsum, dim3((unsigned)cdiv(cols, 256), 5), dim3(256), 0, partial, p, nrb, (int)cols, accumulate);
+    AH_LAUNCH_CHECK();
+  }
+  return AH_OK;
+}
+static int32_t swiglu_args(const char *who, int32_t dtype, int64_t rows, int64_t cols) {
+  AH_ARG(dtype == AH_F32 || dtype == AH_BF16, "%s: dtype must be AH_F32 or AH_BF16", who);
+  AH_ARG(rows >= 0 && cols > 0 && cols % 4 == 0 && cols < (1ll << 30), "%s: cols %lld must be a positive multiple of 4", who, (long long)cols);
+  return AH_OK;
+}
+int32_t ah_swiglu(int32_t dtype, ah_ptr gate_up, ah_ptr out, int64_t rows, int64_t cols) {
+  AH_REQUIRE_READY();
+  int32_t rc = swiglu_args("ah_swiglu", dtype, rows, cols);
+  if (rc) return rc;
+  if (rows == 0) return AH_OK;
+  AH_ARG(gate_up && out && aligned16(gate_up) && aligned16(out), "ah_swiglu: operands must be non-null and 16-byte aligned");
+  const dim3 grid(grid_for((uint64_t)(rows * cols / 4)));
+  if (dtype == AH_F32) ah::launch_kernel(k_swiglu<float>, grid, dim3(TPB), 0, dp<const float>(gate_up), dp<float>(out), rows, (int)(cols / 4));
+  else ah::launch_kernel(k_swiglu<uint16_t>, grid, dim3(TPB), 0, dp<const uint16_t>(gate_up), dp<uint16_t>(out), rows, (int)(cols / 4));
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+int32_t ah_swiglu_bwd(int32_t dtype, ah_ptr gate_up, ah_ptr grad_out, ah_ptr d_gate_up, int64_t rows, int64_t cols) {
+  AH_REQUIRE_READY();
+  int32_t rc = swiglu_args("ah_swiglu_bwd", dtype, rows, cols);
+  if (rc) return rc;
+  if (rows == 0) return AH_OK;
+  AH_ARG(gate_up && grad_out && d_gate_up && aligned16(gate_up) && aligned16(grad_out) && aligned16(d_gate_up),
+         "ah_swiglu_bwd: operands must be non-null and 16-byte aligned");
+  const dim3 grid(grid_for((uint64_t)(rows * cols / 4)));
+  if (dtype == AH_F32)
+    ah::launch_kernel(k_swiglu_bwd<float>, grid, dim3(TPB), 0, dp<const float>(gate_up), dp<const float>(grad_out), dp<float>(d_gate_up), rows, (int)(cols / 4));
+  else
+    ah::launch_kernel(k_swiglu_bwd<uint16_t>, grid, dim3(TPB), 0, dp<const uint16_t>(gate_up), dp<const uint16_t>(grad_out), dp<uint16_t>(d_gate_up), rows,
+                       (int)(cols / 4));
   AH_LAUNCH_CHECK();
   return AH_OK;
 }

@@ -47,8 +47,10 @@ class StepStats:
 class FusedTrainer:
     def __init__(self, backend: HipBackend, cfg: ModelConfig, tc: TrainConfig, batch: int, seed: int = 0, use_graph: bool = True,
                  accum: int = 1, params: Optional[dict] = None, dw_groups: int = 1):
-        if (cfg.ffnActivation or "gelu") != "gelu" or cfg.dropout != 0:
-            raise ValueError("FusedTrainer schedules the default GELU block without dropout; use train.Trainer for the variants")
+        self.act = cfg.ffnActivation or "gelu"
+        if self.act not in ("gelu", "silu", "relu", "swiglu", "universal", "kan_spline") or cfg.dropout != 0:
+            raise ValueError("FusedTrainer schedules the gelu / silu / relu / swiglu / universal / kan_spline blocks without dropout; "
+                             "use train.Trainer for composed activations and dropout")
         self.B, self.lib, self.cfg, self.tc = backend, backend.lib, cfg, tc
         self.batch, self.T, self.accum, self.use_graph = batch, cfg.blockSize, accum, use_graph
         self.C, self.H, self.L, self.V, self.F = cfg.nEmbd, cfg.nHead, cfg.nLayer, cfg.vocabSize, ffn_dim(cfg)
@@ -108,7 +110,22 @@ class FusedTrainer:
         self.att = [a(BT * Cc * 2) for _ in range(self.L)]
         self.lse = [a(batch * self.H * self.T * 4) for _ in range(self.L)]
         self.ln2 = [a(BT * Cc * 2) for _ in range(self.L)]
-        self.hgrad = [a(BT * Fd * 2) for _ in range(self.L)]          # gelu'(fc1 output), saved by the forward epilogue
+        # MLP (gpt.ts:286-321).  gelu: activation and derivative are epilogues of the fc1 product, the derivative is what is
+        # saved.  The other activations save the pre-activation (Fin columns: 2 F for swiglu, whose gate and up weights are
+        # adjacent in the arena and therefore ONE [2F, C] operand) and run one element-wise pass each way.
+        self.Fin = 2 * Fd if self.act == "swiglu" else Fd
+        self.w1 = "mlp.fc_gate" if self.act == "swiglu" else "mlp.fc1"
+        self.w2 = "mlp.fc_proj" if self.act == "swiglu" else "mlp.fc2"
+        if self.act == "swiglu":
+            assert all(self.off[f"layer.{l}.mlp.fc_up"] == self.off[f"layer.{l}.mlp.fc_gate"] + Fd * Cc for l in range(self.L))
+        self._act_coefs = {"universal": (("act_gate", 0), ("act_skip", 3)),
+                           "kan_spline": (("kan_c0", 0), ("kan_c1", 1), ("kan_c2", 2), ("kan_c3", 3), ("kan_c4", 4))}.get(self.act, ())
+        self._act_mask = {"silu": 1, "relu": 2, "universal": 0b01001, "kan_spline": 0b11111}.get(self.act, 0)
+        if self.act == "gelu":
+            self.hgrad = [a(BT * Fd * 2) for _ in range(self.L)]      # gelu'(fc1 output), saved by the forward epilogue
+        else:
+            self.hpre = [a(BT * self.Fin * 2) for _ in range(self.L)]
+            self.dact = a(BT * Fd * 2)                                # gradient of the activation's output (one layer at a time)
         self.hact = [a(BT * Fd * 2) for _ in range(self.L)]
         self.lnf, self.logits, self.rowlse = a(BT * Cc * 2), a(BT * V * 2), a(BT * 4)
         self.dx = [a(BT * Cc * 4), a(BT * Cc * 4)]
@@ -118,7 +135,7 @@ class FusedTrainer:
         # GEMMs per layer.  dy_fc2[l] = grad of the layer's output, dy_wo[l] = grad after the MLP branch joins.
         self.dy_fc2 = [a(BT * Cc * 2) for _ in range(self.L)]
         self.dy_wo = [a(BT * Cc * 2) for _ in range(self.L)]
-        self.dh = [a(BT * Fd * 2) for _ in range(self.L)]
+        self.dh = [a(BT * self.Fin * 2) for _ in range(self.L)]
         self.dqkv = [a(BT * 3 * Cc * 2) for _ in range(self.L)]
         self.dxb0 = a(BT * Cc * 2)                # grad of the embedding output in bf16 (written by the last LayerNorm backward, unused)
         self.loss, self.sumsq, self.clip = a(4), a(4), a(16)         # clip: coefficient (NaN = skip), norm, skipped flag
@@ -144,14 +161,14 @@ class FusedTrainer:
         dw_groups = 1 they are ONE grouped launch at the end of backward.  With dw_groups = n the layers are cut into n
         runs (the last layers, whose gradients exist first, and lmHead in run 0): run k is launched on the side stream as
         soon as backward has passed its lowest layer, beside the backward kernels of the layers below."""
-        BT, Cc, Fd, V, TN = self.BT, self.C, self.F, self.V, ffi.GEMM_TN
+        BT, Cc, Fd, V, TN = self.BT, self.C, self.F, self.V, ffi.GEMM_TN     # (swiglu: d[gate; up] is one [2F, C] product)
 
         def desc(dy, x, gname, m, n):
             return ffi.AhGemm(TN, BF16, F32, ffi.EPI_NONE, m, n, BT, m, n, n, 1, 0, 0, 0, dy, x, self.g(gname), 0)
 
         def layer(l):
             pre = f"layer.{l}."
-            return [desc(self.dy_fc2[l], self.hact[l], pre + "mlp.fc2", Cc, Fd), desc(self.dh[l], self.ln2[l], pre + "mlp.fc1", Fd, Cc),
+            return [desc(self.dy_fc2[l], self.hact[l], pre + self.w2, Cc, Fd), desc(self.dh[l], self.ln2[l], pre + self.w1, self.Fin, Cc),
                     desc(self.dy_wo[l], self.att[l], pre + "attn.wo", Cc, Cc), desc(self.dqkv[l], self.ln1[l], pre + "attn.wqkv", 3 * Cc, Cc)]
         n = self.dw_groups
         bounds = [self.L - (self.L * (k + 1)) // n for k in range(n)]          # lowest layer of run k (run n-1 ends at layer 0)
@@ -209,6 +226,13 @@ class FusedTrainer:
         check(self.lib.ah_alloc(max(16, nbytes), C.byref(p)))
         self._bufs.append(p.value)
         return p.value
+
+    def _coef_handles(self, l: int, where):
+        """The five per-channel coefficient (or gradient) vectors of layer l's activation; 0 = none."""
+        arr = (C.c_uint64 * 5)()
+        for name, k in self._act_coefs:
+            arr[k] = where(f"layer.{l}.mlp.{name}")
+        return arr
 
     def p(self, name: str, bf16: bool = False) -> int:
         return (self.Pb + self.off[name] * 2) if bf16 else (self.P + self.off[name] * 4)
@@ -268,8 +292,16 @@ class FusedTrainer:
             self._flash(l, False)
             self._gemm(NT, self.att[l], self.p(pre + "attn.wo", True), self.xmid[l], BT, Cc, Cc, Cc, Cc, Cc, F32, ffi.EPI_RESIDUAL, self.x[l])
             check(lib.ah_layernorm(self.xmid[l], self.p(pre + "ln2.weight"), self.p(pre + "ln2.bias"), self.ln2[l], BT, Cc, 1e-5, BF16))
-            self._gemm(NT, self.ln2[l], self.p(pre + "mlp.fc1", True), self.hact[l], BT, Fd, Cc, Cc, Cc, Fd, BF16, ffi.EPI_GELU_GRAD, self.hgrad[l])
-            self._gemm(NT, self.hact[l], self.p(pre + "mlp.fc2", True), self.x[l + 1], BT, Cc, Fd, Fd, Fd, Cc, F32, ffi.EPI_RESIDUAL, self.xmid[l])
+            if self.act == "gelu":
+                self._gemm(NT, self.ln2[l], self.p(pre + "mlp.fc1", True), self.hact[l], BT, Fd, Cc, Cc, Cc, Fd, BF16, ffi.EPI_GELU_GRAD, self.hgrad[l])
+            else:
+                Fin = self.Fin
+                self._gemm(NT, self.ln2[l], self.p(pre + self.w1, True), self.hpre[l], BT, Fin, Cc, Cc, Cc, Fin)
+                if self.act == "swiglu":
+                    check(lib.ah_swiglu(BF16, self.hpre[l], self.hact[l], BT, Fd))
+                else:
+                    check(lib.ah_channel_act(BF16, self.hpre[l], self._coef_handles(l, self.p), self._act_mask, self.hact[l], BT, Fd))
+            self._gemm(NT, self.hact[l], self.p(pre + self.w2, True), self.x[l + 1], BT, Cc, Fd, Fd, Fd, Cc, F32, ffi.EPI_RESIDUAL, self.xmid[l])
         check(lib.ah_layernorm(self.x[L], self.p("lnF.weight"), self.p("lnF.bias"), self.lnf, BT, Cc, 1e-5, BF16))
         self._gemm(NT, self.lnf, self.p("lmHead", True), self.logits, BT, V, Cc, Cc, Cc, V)
         # loss and dlogits (in place) from one read of the logits
@@ -288,8 +320,16 @@ class FusedTrainer:
         for l in reversed(range(L)):
             pre = f"layer.{l}."
             # MLP: x_out = x_mid + fc2(gelu(fc1(ln2(x_mid))))
-            self._gemm(NN, self.dy_fc2[l], self.p(pre + "mlp.fc2", True), self.dh[l], BT, Fd, Cc, Cc, Fd, Fd, BF16, ffi.EPI_MUL_AUX, self.hgrad[l])
-            self._gemm(NN, self.dh[l], self.p(pre + "mlp.fc1", True), self.dlnb, BT, Cc, Fd, Fd, Cc, Cc)
+            if self.act == "gelu":
+                self._gemm(NN, self.dy_fc2[l], self.p(pre + "mlp.fc2", True), self.dh[l], BT, Fd, Cc, Cc, Fd, Fd, BF16, ffi.EPI_MUL_AUX, self.hgrad[l])
+            else:
+                self._gemm(NN, self.dy_fc2[l], self.p(pre + self.w2, True), self.dact, BT, Fd, Cc, Cc, Fd, Fd)
+                if self.act == "swiglu":
+                    check(lib.ah_swiglu_bwd(BF16, self.hpre[l], self.dact, self.dh[l], BT, Fd))
+                else:
+                    check(lib.ah_channel_act_bwd(BF16, self.hpre[l], self._coef_handles(l, self.p), self._act_mask, self.dact, self.dh[l],
+                                                 self._coef_handles(l, self.g), acc, BT, Fd))
+            self._gemm(NN, self.dh[l], self.p(pre + self.w1, True), self.dlnb, BT, Cc, self.Fin, self.Fin, Cc, Cc)
             check(lib.ah_layernorm_bwd_deferred(self.xmid[l], self.p(pre + "ln2.weight"), self.dlnb, BF16, self.dx[cur], self.dx[cur ^ 1], self.dy_wo[l],
                                                 self._ln_part[pre + "ln2"], BT, Cc, 1e-5))
             cur ^= 1

@@ -161,12 +161,21 @@ int32_t ah_silu_mul_bwd(ah_ptr a, ah_ptr b, ah_ptr grad_out, ah_ptr da, ah_ptr d
 /* Per-channel mixture of activation bases, the MLP activations "universal" (silu(h)*gate + h*skip) and "kan_spline"
  * (c0 silu + c1 relu + c2 gelu + c3 h + c4 h^2) that the reference composes from separate ops (packages/model/src/gpt.ts:295-321),
  * in one pass:  out[r,c] = sum_k coefs[k][c] * basis_k(x[r,c])  over the bases whose bit is set in `mask`
- * (bit 0 silu, 1 relu, 2 tanh-gelu, 3 identity, 4 square).  coefs: 5 handles of f32[cols] (unused ones 0); cols % 4 == 0.
- * Backward: dx = grad_out * sum_k coefs[k] * basis_k'(x);  dcoefs[k][c] = sum_r grad_out[r,c] * basis_k(x[r,c])
- * (column sums in fixed order; dcoefs are overwritten). */
-int32_t ah_channel_act(ah_ptr x, const ah_ptr *coefs, int32_t mask, ah_ptr out, int64_t rows, int64_t cols);
-int32_t ah_channel_act_bwd(ah_ptr x, const ah_ptr *coefs, int32_t mask, ah_ptr grad_out, ah_ptr dx, const ah_ptr *dcoefs,
-                           int64_t rows, int64_t cols);
+ * (bit 0 silu, 1 relu, 2 tanh-gelu, 3 identity, 4 square).  dtype (AH_F32 or AH_BF16) is the type of x, out, grad_out and dx;
+ * coefs: 5 handles of f32[cols]; a 0 handle (or coefs == NULL) for a selected basis is the constant 1, so one selected basis
+ * without coefficients is the plain silu / relu / gelu MLP activation.  cols % 4 == 0.
+ * Backward: dx = grad_out * sum_k coefs[k] * basis_k'(x);  dcoefs[k][c] = sum_r grad_out[r,c] * basis_k(x[r,c]) for the bases
+ * that have a coefficient vector (column sums in fixed order; overwritten, or added to when `accumulate` is non-zero:
+ * gradient accumulation over micro-steps, trainer.ts:1164-1273). */
+int32_t ah_channel_act(int32_t dtype, ah_ptr x, const ah_ptr *coefs, int32_t mask, ah_ptr out, int64_t rows, int64_t cols);
+int32_t ah_channel_act_bwd(int32_t dtype, ah_ptr x, const ah_ptr *coefs, int32_t mask, ah_ptr grad_out, ah_ptr dx, const ah_ptr *dcoefs,
+                           int32_t accumulate, int64_t rows, int64_t cols);
+/* SwiGLU on a packed pre-activation (packages/model/src/gpt.ts:295-299 computes silu(x Wgate^T) * (x Wup^T) with
+ * Backend.siluMul, interfaces.ts:105-106): gate_up = [rows, 2 cols], gate in the first `cols` columns of a row and up in
+ * the last -- what ONE product with the two weight matrices stacked gives.  out[r,c] = silu(gate[r,c]) * up[r,c];
+ * backward writes d_gate_up in the same packed layout.  dtype AH_F32 or AH_BF16 for every operand; cols % 4 == 0. */
+int32_t ah_swiglu(int32_t dtype, ah_ptr gate_up, ah_ptr out, int64_t rows, int64_t cols);
+int32_t ah_swiglu_bwd(int32_t dtype, ah_ptr gate_up, ah_ptr grad_out, ah_ptr d_gate_up, int64_t rows, int64_t cols);
 /* Backend.residualDropoutAdd: out = residual + projected*mask (interfaces.ts:110; mask may be 0 = no dropout) */
 int32_t ah_residual_dropout_add(ah_ptr residual, ah_ptr projected, ah_ptr mask, ah_ptr out, uint64_t n);
 /* Backend.dropoutMask (interfaces.ts:125): out[i] = hash(seed, counter, i) / 2^32 > p ? (float)(1/(1-p)) : 0 with the hash of the

@@ -242,3 +242,44 @@ def test_weight_gradients_on_the_side_stream_give_the_same_step(B, graph, accum)
     for name in ("wte", "lmHead", "layer.0.attn.wqkv", "layer.1.mlp.fc2", "layer.1.ln1.weight"):
         assert np.array_equal(one.param(name), two.param(name)), name
     one.close(), two.close()
+
+
+@pytest.mark.parametrize("act", ["silu", "relu", "swiglu", "universal", "kan_spline"])
+@pytest.mark.parametrize("accum", [1, 2])
+def test_fused_step_with_the_other_mlp_activations_matches_oracle(B, act, accum):
+    """gpt.ts:286-321: the MLP variants in the hand-scheduled bf16 step (pre-activation saved in bf16, one element-wise pass
+    each way; swiglu's gate and up weights as one stacked operand).  Loss, gradient norm, every gradient's direction and size,
+    and the parameters after the update against the fp32 oracle, with and without accumulation over two micro-batches."""
+    from alpha2_amd.fused import FusedTrainer
+    from alpha2_amd.model import ModelConfig
+    from alpha2_amd.train import TrainConfig, syntheticBatch
+    cfg = dict(CFG, ffnActivation=act)
+    ft = FusedTrainer(B, ModelConfig(**cfg), TrainConfig(iters=3, gradAccumSteps=accum), 4, seed=0, use_graph=True, accum=accum)
+    orc = rm.Trainer(rm.ModelConfig(**cfg), rm.TrainConfig(iters=3, gradAccumSteps=accum), seed=0)
+    for name, v in orc.entries:
+        assert np.array_equal(ft.param(name), v.data.data), name
+    idx = [ft.add_batch(*syntheticBatch(1 + m, 4, 64, 256)) for m in range(accum)]
+    obs = [rm.synthetic_batch(1 + m, 4, 64, 256) for m in range(accum)]
+    # oracle gradients (sum over micro-batches, as the gradient arena holds them before the 1 / accum scale) before its optimizer step
+    for ob in obs:
+        _, oloss = rm.gptForward(orc.cfg, orc.params, orc.B, orc.tape, ob[0], ob[1], True)
+        orc.tape.backward(oloss, orc.B)
+        orc.tape.clear()
+    ograds = {n: v.grad.data.copy() for n, v in orc.entries}
+    for _, v in orc.entries:
+        v.grad = None
+    for s in range(3):
+        o = orc.step(obs)
+        ft.step(idx if accum > 1 else idx[0])
+        st = ft.history(s, s + 1)[0]
+        assert abs(st.loss - o.loss) <= 2e-2 * abs(o.loss), (s, st.loss, o.loss)
+        assert abs(st.gradNorm - o.gradNorm) <= 3e-2 * o.gradNorm, (s, st.gradNorm, o.gradNorm)
+        if s == 0:
+            for name, g in ograds.items():
+                got, w = ft.grad(name).astype(np.float64), g.astype(np.float64)
+                cos = float(got @ w / (np.linalg.norm(got) * np.linalg.norm(w) + 1e-300))
+                assert cos > 0.995, (name, cos)
+                assert abs(np.linalg.norm(got) / np.linalg.norm(w) - 1) < 3e-2, name
+    for name, v in orc.entries:                                           # three AdamW steps: every entry within 3 lr of the oracle's
+        assert np.max(np.abs(ft.param(name) - v.data.data)) <= 3 * 2 * 3e-4 * 1.001 + 1e-6, name
+    ft.close()

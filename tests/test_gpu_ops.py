@@ -172,6 +172,92 @@ def test_channel_activation_mixtures_match_the_composed_ops(B, rows, cols):
         B.channelAct(dev(B, x), {"silu": dev(B, np.ones((1, cols + 4), np.float32))})
 
 
+def _raw_buf(B, arr, bf16):
+    """Device copy of `arr` as f32 or as raw bf16 bits; returns (TensorData that owns it, handle)."""
+    from alpha2_amd import TensorData
+    t = TensorData(arr.shape, "f16", _bf16_round(arr)[1]) if bf16 else TensorData(arr.shape, "f32", np.ascontiguousarray(arr, np.float32))
+    return t, B._ptr(t)
+
+
+def _raw_read(B, t, bf16):
+    B._dirty(t)
+    raw = t.data
+    return ((raw.astype(np.uint32) << 16).view(np.float32) if bf16 else raw).reshape(t.shape)
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("rows,cols", [(3, 8), (130, 260), (517, 384)])
+def test_plain_and_bf16_channel_activations_and_accumulated_coefficient_gradients(B, bf16, rows, cols):
+    """ah_channel_act / ah_channel_act_bwd through the C ABI: a selected basis without a coefficient vector is the plain
+    activation (silu, relu, gelu against the oracle's element-wise ops and their backward, cpu_ref.ts:422-435, ops.ts:284-417);
+    bf16 operands give the f32 result of the bf16-rounded inputs, rounded once; `accumulate` adds the coefficient gradients to
+    what the vectors hold."""
+    import ctypes as C
+    from alpha2_amd import _ffi as ffi
+    dt = ffi.BF16 if bf16 else ffi.F32
+    rnd = (lambda a: _bf16_round(a)[0]) if bf16 else (lambda a: a)
+    x, g = rnd((rs.randn(rows, cols) * 2).astype(np.float32)), rnd(rs.randn(rows, cols).astype(np.float32))
+    tol = 2.0 ** -8 if bf16 else 2e-5
+    tx, px = _raw_buf(B, x, bf16)
+    tg, pg = _raw_buf(B, g, bf16)
+    for k, name in ((0, "silu"), (1, "relu"), (2, "gelu")):
+        tape = rm.Tape(); ctx = rm.Ctx(tape, O)
+        xv = rm.Variable(orc(x), True)
+        out = getattr(rm, name)(ctx, xv)
+        tape.backward(out, O, orc(g))
+        to, po = _raw_buf(B, np.zeros((rows, cols), np.float32), bf16)
+        td, pd = _raw_buf(B, np.zeros((rows, cols), np.float32), bf16)
+        ffi.check(B.lib.ah_channel_act(dt, px, None, 1 << k, po, rows, cols))
+        ffi.check(B.lib.ah_channel_act_bwd(dt, px, None, 1 << k, pg, pd, None, 0, rows, cols))
+        got, gdx = _raw_read(B, to, bf16), _raw_read(B, td, bf16)
+        assert np.max(np.abs(got - out.data.data.reshape(rows, cols)) / (np.abs(out.data.data.reshape(rows, cols)) + 1e-2)) <= tol, name
+        assert np.max(np.abs(gdx - xv.grad.data.reshape(rows, cols)) / (np.abs(xv.grad.data.reshape(rows, cols)) + 1e-2)) <= tol, name
+    # a mixture with coefficients: the second call accumulates, so the coefficient gradients double while dx stays
+    co = {0: (rs.randn(cols) * 0.7).astype(np.float32), 3: (rs.randn(cols) * 0.7).astype(np.float32)}
+    arr, darr, keep = (C.c_uint64 * 5)(), (C.c_uint64 * 5)(), []
+    for k, v in co.items():
+        t, ptr = _raw_buf(B, v, False); keep.append(t); arr[k] = ptr
+        t, ptr = _raw_buf(B, np.zeros(cols, np.float32), False); keep.append(t); darr[k] = ptr
+    td, pd = _raw_buf(B, np.zeros((rows, cols), np.float32), bf16)
+    ffi.check(B.lib.ah_channel_act_bwd(dt, px, arr, 0b01001, pg, pd, darr, 0, rows, cols))
+    first = {k: _raw_read(B, keep[2 * i + 1], False).copy() for i, k in enumerate(co)}
+    dx1 = _raw_read(B, td, bf16).copy()
+    ffi.check(B.lib.ah_channel_act_bwd(dt, px, arr, 0b01001, pg, pd, darr, 1, rows, cols))
+    sig = 1.0 / (1.0 + np.exp(-x.astype(np.float64)))
+    want = {0: (g * x * sig).sum(0), 3: (g.astype(np.float64) * x).sum(0)}
+    for i, k in enumerate(co):
+        second = _raw_read(B, keep[2 * i + 1], False)
+        assert np.allclose(first[k], want[k], rtol=1e-4, atol=1e-4 * np.sqrt(rows)), k
+        assert np.allclose(second, 2 * first[k], rtol=1e-6, atol=1e-6), k
+    assert np.array_equal(dx1, _raw_read(B, td, bf16))
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+@pytest.mark.parametrize("rows,cols", [(1, 4), (37, 24), (513, 384)])
+def test_swiglu_on_the_packed_pre_activation(B, bf16, rows, cols):
+    """ah_swiglu / ah_swiglu_bwd on [gate | up] rows against the oracle's siluMul and its backward on the two halves
+    (gpt.ts:295-299)."""
+    from alpha2_amd import _ffi as ffi
+    dt = ffi.BF16 if bf16 else ffi.F32
+    rnd = (lambda a: _bf16_round(a)[0]) if bf16 else (lambda a: a)
+    gu, g = rnd((rs.randn(rows, 2 * cols) * 2).astype(np.float32)), rnd(rs.randn(rows, cols).astype(np.float32))
+    tol = 2.0 ** -8 if bf16 else 2e-5
+    tape = rm.Tape(); ctx = rm.Ctx(tape, O)
+    a, b = rm.Variable(orc(np.ascontiguousarray(gu[:, :cols])), True), rm.Variable(orc(np.ascontiguousarray(gu[:, cols:])), True)
+    out = rm.siluMul(ctx, a, b)
+    tape.backward(out, O, orc(g))
+    tgu, pgu = _raw_buf(B, gu, bf16)
+    tg, pg = _raw_buf(B, g, bf16)
+    to, po = _raw_buf(B, np.zeros((rows, cols), np.float32), bf16)
+    td, pd = _raw_buf(B, np.zeros((rows, 2 * cols), np.float32), bf16)
+    ffi.check(B.lib.ah_swiglu(dt, pgu, po, rows, cols))
+    ffi.check(B.lib.ah_swiglu_bwd(dt, pgu, pg, pd, rows, cols))
+    got, d = _raw_read(B, to, bf16), _raw_read(B, td, bf16)
+    close = lambda x, w: np.max(np.abs(x - w) / (np.abs(w) + 1e-2)) <= tol
+    assert close(got, out.data.data.reshape(rows, cols))
+    assert close(d[:, :cols], a.grad.data.reshape(rows, cols)) and close(d[:, cols:], b.grad.data.reshape(rows, cols))
+
+
 def test_fill_at_every_alignment_touches_exactly_its_range(B):
     """ah_fill_f32 / ah_fill_i32 write 16 bytes at a time over the aligned middle of the range: every start offset modulo 16
     bytes and ragged lengths, with sentinels either side."""
