@@ -822,7 +822,10 @@ def test_flash_attention_bf16_vs_materialised(B, bwd_variant, BH, T, D, cap):
     r = B.flashAttention(Q, K, V, T, scale, cap)
     assert r["output"].store == "bf16"
     rel = 2.0 ** -6
-    assert_close(r["output"].data, want_o, rel=rel, what="flash16.O")
+    # O = sum_j p_j v_j with every p_j rounded to bf16 (relative error <= 2^-9): the error of an entry is at most
+    # 2^-9 sum_j p_j |v_j| <= 2^-9 max|v| whatever the entry's own size, and over long rows the entries themselves average
+    # out towards 0, so that -- not the rms of O -- is the floor of the bound (rel x scale = 2^-9 max|v|)
+    assert_close(r["output"].data, want_o, rel=rel, what="flash16.O", scale=float(np.abs(v).max()) / 8)
     assert_close(r["lse"].data, want_lse, rel=1e-4, what="flash16.LSE")
     g = B.flashAttentionBackward(Q, K, V, r["output"], dO, r["lse"], T, scale, cap)
     term = float(np.abs(np.einsum("bqd,bkd->bqk", do, v)).max() * max(np.abs(k).max(), np.abs(q).max()) * scale)
