@@ -103,16 +103,16 @@ SIGNATURES = {
     "ah_softmax": [u64, u64, i64, i64, i64, i32], "ah_argmax": [u64, u64, i64, i64, i64],
     "ah_sum_sq": [u64, u64, u64], "ah_sum_sq_static": [u64, u64, u64], "ah_softmax_bwd": [u64, u64, u64, i64, i64],
     "ah_embedding": [u64, u64, u64, i64, i64, i64, i32],
-    "ah_embedding_tok_pos": [u64, u64, u64, u64, i64, i64, i64, i64],
+    "ah_embedding_tok_pos": [u64, u64, u64, u64, i64, i64, i64, i64, i32],
     "ah_embedding_bwd": [u64, u64, u64, i64, i64, i64, i32],
     "ah_embedding_index_bytes": [i64, i64], "ah_embedding_index": [u64, i64, i64, u64],
     "ah_embedding_bwd_indexed": [u64, u64, u64, i64, i64, i64, i32],
     "ah_token_windows": [u64, i64, u64, i64, i64, u64, u64],
     "ah_pos_embedding_bwd": [u64, u64, i64, i64, i64, i32],
-    "ah_layernorm": [u64, u64, u64, u64, i64, i64, f32, i32],
+    "ah_layernorm": [u64, u64, u64, u64, i64, i64, f32, i32, i32],
     "ah_layernorm_bwd": [u64, u64, u64, i32, u64, u64, u64, u64, u64, i64, i64, f32, i32],
     "ah_layernorm_bwd_partials_bytes": [i64, i64],
-    "ah_layernorm_bwd_deferred": [u64, u64, u64, i32, u64, u64, u64, u64, i64, i64, f32],
+    "ah_layernorm_bwd_deferred": [u64, u64, u64, i32, u64, u64, u64, u64, i64, i64, f32, i32],
     "ah_layernorm_colsums": [C.POINTER(AhColsumJob), i32],
     "ah_cross_entropy": [u64, i32, u64, u64, u64, i64, i64],
     "ah_cross_entropy_bwd": [u64, i32, u64, u64, u64, f32, u64, i64, i64],

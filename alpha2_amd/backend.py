@@ -576,7 +576,7 @@ class HipBackend:
         if weight.size != dim or bias.size != dim:
             raise ValueError("layerNorm: weight/bias length must equal the last dimension")
         out = self._new(x.shape)
-        check(self.lib.ah_layernorm(self._ptr(x), self._ptr(weight), self._ptr(bias), out._buf.ptr, x.size // max(1, dim), dim, eps, ffi.F32))
+        check(self.lib.ah_layernorm(self._ptr(x), self._ptr(weight), self._ptr(bias), out._buf.ptr, x.size // max(1, dim), dim, eps, ffi.F32, ffi.F32))
         return out
 
     def layerNormBackward(self, x, weight, gradOutput, eps) -> dict:

@@ -340,7 +340,7 @@ class FastHipBackend(HipBackend):
         if weight.size != dim or bias.size != dim:
             raise ValueError("layerNorm: weight/bias length must equal the last dimension")
         out = self._new(x.shape, "f32", "bf16")
-        check(self.lib.ah_layernorm(self._ptr(x), self._ptr(weight), self._ptr(bias), out._buf.ptr, x.size // max(1, dim), dim, eps, BF16))
+        check(self.lib.ah_layernorm(self._ptr(x), self._ptr(weight), self._ptr(bias), out._buf.ptr, x.size // max(1, dim), dim, eps, BF16, ffi.F32))
         return out
 
     def layerNormBackward(self, x, weight, gradOutput, eps) -> dict:

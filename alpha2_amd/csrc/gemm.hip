@@ -264,7 +264,8 @@ int32_t run_bf16_nt(const GemmArgs &ga, int batch, int out_dtype, int vec_c) {
     case AH_EPI_NONE: return f32 ? launch_bf16_nt_t<128, 128, 2, 2, AH_EPI_NONE, float>(ga, batch, vec_c)
                                  : launch_bf16_nt_t<128, 128, 2, 2, AH_EPI_NONE, uint16_t>(ga, batch, vec_c);
     case AH_EPI_ACCUM: return launch_bf16_nt_t<128, 128, 2, 2, AH_EPI_ACCUM, float>(ga, batch, vec_c);
-    case AH_EPI_RESIDUAL: return launch_bf16_nt_t<128, 128, 2, 2, AH_EPI_RESIDUAL, float>(ga, batch, vec_c);
+    case AH_EPI_RESIDUAL: return f32 ? launch_bf16_nt_t<128, 128, 2, 2, AH_EPI_RESIDUAL, float>(ga, batch, vec_c)
+                                     : launch_bf16_nt_t<128, 128, 2, 2, AH_EPI_RESIDUAL, uint16_t>(ga, batch, vec_c);
     case AH_EPI_GELU: return launch_bf16_nt_t<128, 128, 2, 2, AH_EPI_GELU, uint16_t>(ga, batch, vec_c);
     case AH_EPI_GELU_GRAD: return launch_bf16_nt_t<128, 128, 2, 2, AH_EPI_GELU_GRAD, uint16_t>(ga, batch, vec_c);
     case AH_EPI_MUL_AUX: return launch_bf16_nt_t<128, 128, 2, 2, AH_EPI_MUL_AUX, uint16_t>(ga, batch, vec_c);
@@ -515,9 +516,10 @@ int32_t ah_gemm(const AhGemm *p) {
   const bool gelu_like = q.epilogue == AH_EPI_GELU || q.epilogue == AH_EPI_GELU_BWD || q.epilogue == AH_EPI_GELU_GRAD || q.epilogue == AH_EPI_MUL_AUX;
   if (gelu_like || q.epilogue == AH_EPI_RESIDUAL)
     AH_ARG(q.aux != 0, "ah_gemm: epilogue %d needs aux", q.epilogue);
-  // epilogue / output-type combinations: NONE -> f32 or bf16; ACCUM, RESIDUAL -> f32; GELU, GELU_BWD -> the operand type
+  // epilogue / output-type combinations: NONE -> f32 or bf16; ACCUM -> f32; RESIDUAL -> f32, or bf16 from bf16 operands (aux
+  // then bf16 too); GELU, GELU_BWD -> the operand type
   bool combo = q.epilogue == AH_EPI_NONE || ((q.epilogue == AH_EPI_ACCUM || q.epilogue == AH_EPI_RESIDUAL) && q.out_dtype == AH_F32) ||
-               (gelu_like && q.out_dtype == q.in_dtype);
+               (q.epilogue == AH_EPI_RESIDUAL && q.in_dtype == AH_BF16 && q.out_dtype == AH_BF16) || (gelu_like && q.out_dtype == q.in_dtype);
   if (!combo) return fail(AH_ERR_UNSUPPORTED, "ah_gemm: epilogue %d with operands of dtype %d and output dtype %d is not provided", q.epilogue, q.in_dtype, q.out_dtype);
 
   GemmArgs ga;
@@ -533,7 +535,7 @@ int32_t ah_gemm(const AhGemm *p) {
   // 4-wide epilogue accesses need 16-byte (f32) / 8-byte (bf16) aligned rows of C and aux
   int osz = q.out_dtype == AH_F32 ? 4 : 2;
   int vec_c = ((q.c % (4 * osz)) == 0) && (q.ldc % 4 == 0) && (q.stride_c % 4 == 0);
-  if (q.epilogue == AH_EPI_RESIDUAL) vec_c = vec_c && (q.aux % 16 == 0);
+  if (q.epilogue == AH_EPI_RESIDUAL) vec_c = vec_c && (q.aux % (4 * osz) == 0);
   if (gelu_like) vec_c = vec_c && (q.aux % (4 * osz) == 0);
   if (q.in_dtype == AH_F32) {
     int vec_a = aligned16(q.a) && (q.lda % 4 == 0) && (q.stride_a % 4 == 0);

@@ -206,7 +206,10 @@ __global__ __launch_bounds__(64 * WGM * WGN) void k_gemm_bf16(GemmArgs g, int ou
       else store_tiles<AH_EPI_NONE, uint16_t, TM, TN>(g, cbase, r0, c0, lane, acc);
       break;
     case AH_EPI_ACCUM: store_tiles<AH_EPI_ACCUM, float, TM, TN>(g, cbase, r0, c0, lane, acc); break;
-    case AH_EPI_RESIDUAL: store_tiles<AH_EPI_RESIDUAL, float, TM, TN>(g, cbase, r0, c0, lane, acc); break;
+    case AH_EPI_RESIDUAL:
+      if (out_f32) store_tiles<AH_EPI_RESIDUAL, float, TM, TN>(g, cbase, r0, c0, lane, acc);
+      else store_tiles<AH_EPI_RESIDUAL, uint16_t, TM, TN>(g, cbase, r0, c0, lane, acc);
+      break;
     case AH_EPI_GELU: store_tiles<AH_EPI_GELU, uint16_t, TM, TN>(g, cbase, r0, c0, lane, acc); break;
     case AH_EPI_GELU_GRAD: store_tiles<AH_EPI_GELU_GRAD, uint16_t, TM, TN>(g, cbase, r0, c0, lane, acc); break;
     case AH_EPI_MUL_AUX: store_tiles<AH_EPI_MUL_AUX, uint16_t, TM, TN>(g, cbase, r0, c0, lane, acc); break;

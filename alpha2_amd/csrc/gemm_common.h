@@ -20,7 +20,7 @@ void note_gemm_split(int nsplit);
 struct GemmArgs {
   const void *a, *b;
   void *c;
-  const void *aux;     // EPI_RESIDUAL: f32 [M,N]; EPI_GELU_BWD: pre-activation (C dtype)
+  const void *aux;     // EPI_RESIDUAL: [M,N] of C's dtype; EPI_GELU_BWD: pre-activation (C dtype)
   void *aux_out;       // EPI_GELU: pre-activation out (C dtype)
   int M, N, K;
   int64_t lda, ldb, ldc;
@@ -44,8 +44,9 @@ __device__ __forceinline__ void epilogue4(const GemmArgs &g, int64_t cbase, int 
       else { uint2 o = *reinterpret_cast<const uint2 *>((const uint16_t *)g.c + idx);
              v[0] += bf16_bits_to_f32(o.x & 0xffff); v[1] += bf16_bits_to_f32(o.x >> 16); v[2] += bf16_bits_to_f32(o.y & 0xffff); v[3] += bf16_bits_to_f32(o.y >> 16); }
     } else if (EPI == AH_EPI_RESIDUAL) {
-      float4 o = *reinterpret_cast<const float4 *>((const float *)g.aux + idx);
-      v[0] += o.x; v[1] += o.y; v[2] += o.z; v[3] += o.w;
+      if (sizeof(OUT) == 4) { float4 o = *reinterpret_cast<const float4 *>((const float *)g.aux + idx); v[0] += o.x; v[1] += o.y; v[2] += o.z; v[3] += o.w; }
+      else { uint2 o = *reinterpret_cast<const uint2 *>((const uint16_t *)g.aux + idx);
+             v[0] += bf16_bits_to_f32(o.x & 0xffff); v[1] += bf16_bits_to_f32(o.x >> 16); v[2] += bf16_bits_to_f32(o.y & 0xffff); v[3] += bf16_bits_to_f32(o.y >> 16); }
     } else if (EPI == AH_EPI_GELU_BWD) {
       float x[4];
       if (sizeof(OUT) == 4) { float4 o = *reinterpret_cast<const float4 *>((const float *)g.aux + idx); x[0] = o.x; x[1] = o.y; x[2] = o.z; x[3] = o.w; }
@@ -81,7 +82,7 @@ __device__ __forceinline__ void epilogue4(const GemmArgs &g, int64_t cbase, int 
     if (col + i < g.N) {
       float a = v[i];
       if (EPI == AH_EPI_ACCUM) a += Io<OUT>::ld(c, idx + i);
-      else if (EPI == AH_EPI_RESIDUAL) a += ((const float *)g.aux)[idx + i];
+      else if (EPI == AH_EPI_RESIDUAL) a += Io<OUT>::ld((const OUT *)g.aux, idx + i);
       else if (EPI == AH_EPI_GELU_BWD) a *= gelu_grad_f(Io<OUT>::ld((const OUT *)g.aux, idx + i));
       else if (EPI == AH_EPI_GELU) { Io<OUT>::st((OUT *)g.aux_out, idx + i, a); a = gelu_f(a); }
       else if (EPI == AH_EPI_MUL_AUX) a *= Io<OUT>::ld((const OUT *)g.aux, idx + i);
@@ -153,7 +154,7 @@ __device__ __forceinline__ void store_tiles_lds(const GemmArgs &g, int64_t cbase
   constexpr int JP = F32OUT ? 1 : 2;                  // 32 x 32 tiles per pass: a row of the pass is 128 bytes of output
   constexpr int NJP = (TN + JP - 1) / JP, NPASS = TM * NJP;
   constexpr bool READS = EPI == AH_EPI_ACCUM || EPI == AH_EPI_RESIDUAL || EPI == AH_EPI_GELU_BWD || EPI == AH_EPI_MUL_AUX;
-  constexpr bool AUX_F32 = EPI == AH_EPI_RESIDUAL || F32OUT;
+  constexpr bool AUX_F32 = F32OUT;                    // what an epilogue reads has the type of C
   constexpr int DEPTH = 4 < NPASS ? 4 : NPASS;        // passes of reads in flight: 4 x 16 registers
   constexpr int ES = sizeof(OUT), AES = AUX_F32 ? 4 : 2;
   constexpr uint32_t OUTSIDE = 0x80000000u;           // a byte offset no descriptor here reaches (they are shorter than 2 GiB)

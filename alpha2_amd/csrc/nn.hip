@@ -23,23 +23,25 @@ __global__ void k_embedding(const float *__restrict__ w, const int32_t *__restri
   OUT *dst = out + row * dim;
   for (int64_t j = lane; j < dim; j += 64) Io<OUT>::st(dst, j, ok ? src[j] : 0.f);
 }
+template <class OUT>
 __global__ void k_embedding_tok_pos(const float *__restrict__ wte, const float *__restrict__ wpe, const int32_t *__restrict__ tok,
-                                    float *__restrict__ out, int64_t n_idx, int64_t T, int64_t dim, int64_t vocab) {
+                                    OUT *__restrict__ out, int64_t n_idx, int64_t T, int64_t dim, int64_t vocab) {
   int64_t row = blockIdx.x * (int64_t)WPB + (threadIdx.x >> 6);
   if (row >= n_idx) return;
   int lane = threadIdx.x & 63;
   int64_t r = tok[row];
   bool ok = r >= 0 && r < vocab;
   const float *a = wte + (ok ? r : 0) * dim, *b = wpe + (row % T) * dim;
-  float *dst = out + row * dim;
+  OUT *dst = out + row * dim;
   if ((dim & 3) == 0) {
     for (int64_t j = lane; j < (dim >> 2); j += 64) {
       float4 u = reinterpret_cast<const float4 *>(a)[j], v = reinterpret_cast<const float4 *>(b)[j];
       if (!ok) u = make_float4(0, 0, 0, 0);
-      reinterpret_cast<float4 *>(dst)[j] = make_float4(u.x + v.x, u.y + v.y, u.z + v.z, u.w + v.w);
+      if constexpr (sizeof(OUT) == 4) reinterpret_cast<float4 *>(dst)[j] = make_float4(u.x + v.x, u.y + v.y, u.z + v.z, u.w + v.w);
+      else reinterpret_cast<uint2 *>(dst)[j] = make_uint2(pack_bf16x2(u.x + v.x, u.y + v.y), pack_bf16x2(u.z + v.z, u.w + v.w));
     }
   } else {
-    for (int64_t j = lane; j < dim; j += 64) dst[j] = (ok ? a[j] : 0.f) + b[j];
+    for (int64_t j = lane; j < dim; j += 64) Io<OUT>::st(dst, j, (ok ? a[j] : 0.f) + b[j]);
   }
 }
 // scatter-add with hardware f32 atomics (the reference's GPU kernel uses CAS-loop atomics:
@@ -207,15 +209,43 @@ __global__ void k_pos_embedding_bwd(const float *__restrict__ g, float *__restri
   gw[i] = s;
 }
 
+// four values of a row as loaded (f32: 16 bytes, bf16: 8 bytes) and widened to float4 at the point of use;
+// load_nt: past the caches, for data that is read here for the last time
+template <class G> struct Raw4;
+template <> struct Raw4<float> {
+  float4 v;
+  __device__ __forceinline__ void load(const float *p, int j) { v = reinterpret_cast<const float4 *>(p)[j]; }
+  __device__ __forceinline__ void load_nt(const float *p, int j) {
+    typedef float f4v __attribute__((ext_vector_type(4)));
+    const f4v t = __builtin_nontemporal_load(reinterpret_cast<const f4v *>(p) + j);
+    v = make_float4(t.x, t.y, t.z, t.w);
+  }
+  __device__ __forceinline__ void zero() { v = make_float4(0, 0, 0, 0); }
+  __device__ __forceinline__ float4 get() const { return v; }
+};
+template <> struct Raw4<uint16_t> {
+  uint2 v;
+  __device__ __forceinline__ void load(const uint16_t *p, int j) { v = reinterpret_cast<const uint2 *>(p)[j]; }
+  __device__ __forceinline__ void load_nt(const uint16_t *p, int j) {
+    typedef unsigned u2v __attribute__((ext_vector_type(2)));
+    const u2v t = __builtin_nontemporal_load(reinterpret_cast<const u2v *>(p) + j);
+    v = make_uint2(t.x, t.y);
+  }
+  __device__ __forceinline__ void zero() { v = make_uint2(0, 0); }
+  __device__ __forceinline__ float4 get() const {
+    return make_float4(bf16_bits_to_f32(v.x & 0xffff), bf16_bits_to_f32(v.x >> 16), bf16_bits_to_f32(v.y & 0xffff), bf16_bits_to_f32(v.y >> 16));
+  }
+};
+
 // ---------------------------------------------------------------- LayerNorm
 // NV = float4 per lane held in registers (row length <= 256*NV); NV == 0: generic re-reading path.
-template <int NV, class OUT>
-__global__ void k_layernorm(const float *__restrict__ x, const float *__restrict__ w, const float *__restrict__ b,
+template <int NV, class OUT, class IN = float>
+__global__ void k_layernorm(const IN *__restrict__ x, const float *__restrict__ w, const float *__restrict__ b,
                             OUT *__restrict__ out, int64_t rows, int dim, float eps) {
   int64_t row = blockIdx.x * (int64_t)WPB + (threadIdx.x >> 6);
   if (row >= rows) return;
   int lane = threadIdx.x & 63;
-  const float *xr = x + row * (int64_t)dim;
+  const IN *xr = x + row * (int64_t)dim;
   OUT *orow = out + row * (int64_t)dim;
   float inv_dim = 1.0f / (float)dim;
   if constexpr (NV > 0) {
@@ -226,7 +256,9 @@ __global__ void k_layernorm(const float *__restrict__ x, const float *__restrict
 #pragma unroll
     for (int i = 0; i < NV; i++) {
       int j = lane + 64 * i;
-      v[i] = j < nv ? reinterpret_cast<const float4 *>(xr)[j] : make_float4(0, 0, 0, 0);
+      Raw4<IN> raw;
+      if (j < nv) raw.load(xr, j); else raw.zero();
+      v[i] = raw.get();
     }
 #pragma unroll
     for (int i = 0; i < NV; i++) {       // weight and bias travel with the row instead of behind the two reductions
@@ -264,12 +296,12 @@ __global__ void k_layernorm(const float *__restrict__ x, const float *__restrict
     }
   } else {
     float s = 0.f;
-    for (int j = lane; j < dim; j += 64) s += xr[j];
+    for (int j = lane; j < dim; j += 64) s += Io<IN>::ld(xr, j);
     float mean = wave_sum(s) * inv_dim;
     float q = 0.f;
-    for (int j = lane; j < dim; j += 64) { float d = xr[j] - mean; q += d * d; }
+    for (int j = lane; j < dim; j += 64) { float d = Io<IN>::ld(xr, j) - mean; q += d * d; }
     float rstd = 1.0f / sqrtf(wave_sum(q) * inv_dim + eps);
-    for (int j = lane; j < dim; j += 64) Io<OUT>::st(orow, j, (xr[j] - mean) * rstd * w[j] + b[j]);
+    for (int j = lane; j < dim; j += 64) Io<OUT>::st(orow, j, (Io<IN>::ld(xr, j) - mean) * rstd * w[j] + b[j]);
   }
 }
 
@@ -362,28 +394,14 @@ __global__ __launch_bounds__(1024) void k_colsum_partials_batched(ColsumJobs job
 
 // Register-resident LayerNorm backward for rows of up to 256*NV floats (dim % 4 == 0): x, g and the residual gradient
 // are each read once; dw / db accumulate in per-lane registers over all rows a wave walks.
-// four gradient values as loaded (f32: 16 bytes, bf16: 8 bytes) and widened to float4 at the point of use
-template <class G> struct Raw4;
-template <> struct Raw4<float> {
-  float4 v;
-  __device__ __forceinline__ void load(const float *p, int j) { v = reinterpret_cast<const float4 *>(p)[j]; }
-  __device__ __forceinline__ void zero() { v = make_float4(0, 0, 0, 0); }
-  __device__ __forceinline__ float4 get() const { return v; }
-};
-template <> struct Raw4<uint16_t> {
-  uint2 v;
-  __device__ __forceinline__ void load(const uint16_t *p, int j) { v = reinterpret_cast<const uint2 *>(p)[j]; }
-  __device__ __forceinline__ void zero() { v = make_uint2(0, 0); }
-  __device__ __forceinline__ float4 get() const {
-    return make_float4(bf16_bits_to_f32(v.x & 0xffff), bf16_bits_to_f32(v.x >> 16), bf16_bits_to_f32(v.y & 0xffff), bf16_bits_to_f32(v.y >> 16));
-  }
-};
 // A wave walks its rows with the NEXT row's x, g and residual gradient already in flight while it reduces the current
 // one: a row is three dependent wave reductions long, and with the few waves per SIMD that the register-resident
 // column sums allow, nothing else would cover the load latency.
-template <int NV, class G>
-__global__ __launch_bounds__(256) void k_layernorm_bwd_vec(const float *__restrict__ x, const float *__restrict__ w, const G *__restrict__ g,
-                                                           const float *__restrict__ res, float *__restrict__ dx, uint16_t *__restrict__ dx16,
+// X = type of x and of the residual gradient (the residual stream and its gradient stream: f32, or bf16 when the caller keeps
+// them in bf16; dx may then be null, dx16 being the stream)
+template <int NV, class G, class X = float>
+__global__ __launch_bounds__(256) void k_layernorm_bwd_vec(const X *__restrict__ x, const float *__restrict__ w, const G *__restrict__ g,
+                                                           const X *__restrict__ res, float *__restrict__ dx, uint16_t *__restrict__ dx16,
                                                            float *__restrict__ part_dw, float *__restrict__ part_db, int64_t rows, int dim, float eps) {
   extern __shared__ float sh[];      // [2][WPB][dim]
   int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nv = dim >> 2;
@@ -395,10 +413,11 @@ __global__ __launch_bounds__(256) void k_layernorm_bwd_vec(const float *__restri
     wv[i] = j < nv ? reinterpret_cast<const float4 *>(w)[j] : make_float4(0, 0, 0, 0);
     adw[i] = make_float4(0, 0, 0, 0); adb[i] = make_float4(0, 0, 0, 0);
   }
-  float4 xv[NV], rv[NV], nx[NV], nr[NV];
+  float4 xv[NV], rv[NV];
+  Raw4<X> nx[NV], nr[NV];
   Raw4<G> gr[NV], ng[NV];
-  auto load_row = [&](int64_t row, float4 (&xo)[NV], Raw4<G> (&go)[NV], float4 (&ro)[NV]) {
-    const float *xr = x + row * (int64_t)dim;
+  auto load_row = [&](int64_t row, Raw4<X> (&xo)[NV], Raw4<G> (&go)[NV], Raw4<X> (&ro)[NV]) {
+    const X *xr = x + row * (int64_t)dim;
     const G *grow = g + row * (int64_t)dim;
 #pragma unroll
     for (int i = 0; i < NV; i++) {
@@ -406,18 +425,21 @@ __global__ __launch_bounds__(256) void k_layernorm_bwd_vec(const float *__restri
       if (j < nv) {
         // x and the residual gradient were written long ago and are used here for the last time; dx (f32) is next read two
         // GEMMs and an attention later: all three go past the caches (the bf16 copy of dx, the next GEMM's operand, does not)
-        typedef float f4v __attribute__((ext_vector_type(4)));
-        { const f4v t_ = __builtin_nontemporal_load(reinterpret_cast<const f4v *>(xr) + j); xo[i] = make_float4(t_.x, t_.y, t_.z, t_.w); }
+        xo[i].load_nt(xr, j);
         go[i].load(grow, j);
-        if (res) { const f4v t_ = __builtin_nontemporal_load(reinterpret_cast<const f4v *>(res + row * (int64_t)dim) + j); ro[i] = make_float4(t_.x, t_.y, t_.z, t_.w); }
-        else ro[i] = make_float4(0, 0, 0, 0);
+        if (res) ro[i].load_nt(res + row * (int64_t)dim, j);
+        else ro[i].zero();
       } else {
-        xo[i] = make_float4(0, 0, 0, 0); go[i].zero(); ro[i] = make_float4(0, 0, 0, 0);
+        xo[i].zero(); go[i].zero(); ro[i].zero();
       }
     }
   };
   int64_t stride = (int64_t)gridDim.x * WPB, row = blockIdx.x * (int64_t)WPB + wave;
-  if (row < rows) load_row(row, xv, gr, rv);
+  if (row < rows) {
+    load_row(row, nx, gr, nr);
+#pragma unroll
+    for (int i = 0; i < NV; i++) { xv[i] = nx[i].get(); rv[i] = nr[i].get(); }
+  }
   for (; row < rows; row += stride) {
     if (row + stride < rows) load_row(row + stride, nx, ng, nr);
     float4 gv[NV];
@@ -453,12 +475,12 @@ __global__ __launch_bounds__(256) void k_layernorm_bwd_vec(const float *__restri
         d.x = rstd * (gv[i].x * wv[i].x - (s1 + xv[i].x * s2)); d.y = rstd * (gv[i].y * wv[i].y - (s1 + xv[i].y * s2));
         d.z = rstd * (gv[i].z * wv[i].z - (s1 + xv[i].z * s2)); d.w = rstd * (gv[i].w * wv[i].w - (s1 + xv[i].w * s2));
         if (res) { d.x += rv[i].x; d.y += rv[i].y; d.z += rv[i].z; d.w += rv[i].w; }
-        { typedef float f4v __attribute__((ext_vector_type(4))); __builtin_nontemporal_store(f4v{d.x, d.y, d.z, d.w}, reinterpret_cast<f4v *>(dx + row * (int64_t)dim) + j); }
+        if (dx) { typedef float f4v __attribute__((ext_vector_type(4))); __builtin_nontemporal_store(f4v{d.x, d.y, d.z, d.w}, reinterpret_cast<f4v *>(dx + row * (int64_t)dim) + j); }
         if (dx16) reinterpret_cast<uint2 *>(dx16 + row * (int64_t)dim)[j] = make_uint2(pack_bf16x2(d.x, d.y), pack_bf16x2(d.z, d.w));
       }
     }
 #pragma unroll
-    for (int i = 0; i < NV; i++) { xv[i] = nx[i]; gr[i] = ng[i]; rv[i] = nr[i]; }
+    for (int i = 0; i < NV; i++) { xv[i] = nx[i].get(); gr[i] = ng[i]; rv[i] = nr[i].get(); }
   }
 #pragma unroll
   for (int i = 0; i < NV; i++) {
@@ -670,12 +692,12 @@ __global__ void k_token_windows(const int32_t *__restrict__ corpus, int64_t n_to
 
 }  // namespace
 
-template <class OUT>
+template <class OUT, class IN>
 static int32_t launch_ln(ah_ptr x, ah_ptr w, ah_ptr b, ah_ptr out, int64_t rows, int64_t dim, float eps) {
   dim3 grid((unsigned)cdiv(rows, WPB)), blk(TPB);
-  bool vec = (dim % 4 == 0) && dim <= 2048 && aligned16(x) && aligned16(w) && aligned16(b) && (sizeof(OUT) == 2 || aligned16(out));
+  bool vec = (dim % 4 == 0) && dim <= 2048 && x % (4 * sizeof(IN)) == 0 && aligned16(w) && aligned16(b) && (sizeof(OUT) == 2 || aligned16(out));
   int nvl = vec ? (int)cdiv(dim / 4, 64) : 0;
-#define LN_CASE(NV) ah::launch_kernel((k_layernorm<NV, OUT>), grid, blk, 0, dp<const float>(x), dp<const float>(w), dp<const float>(b), dp<OUT>(out), rows, (int)dim, eps)
+#define LN_CASE(NV) ah::launch_kernel((k_layernorm<NV, OUT, IN>), grid, blk, 0, dp<const IN>(x), dp<const float>(w), dp<const float>(b), dp<OUT>(out), rows, (int)dim, eps)
   switch (nvl) {
     case 1: LN_CASE(1); break;
     case 2: LN_CASE(2); break;
@@ -706,13 +728,19 @@ int32_t ah_embedding(ah_ptr weight, ah_ptr idx, ah_ptr out, int64_t n_idx, int64
   return AH_OK;
 }
 
-int32_t ah_embedding_tok_pos(ah_ptr wte, ah_ptr wpe, ah_ptr tok, ah_ptr out, int64_t n_idx, int64_t T, int64_t dim, int64_t vocab) {
+int32_t ah_embedding_tok_pos(ah_ptr wte, ah_ptr wpe, ah_ptr tok, ah_ptr out, int64_t n_idx, int64_t T, int64_t dim, int64_t vocab,
+                             int32_t out_dtype) {
   AH_REQUIRE_READY();
+  AH_ARG(out_dtype == AH_F32 || out_dtype == AH_BF16, "ah_embedding_tok_pos: out dtype must be f32 or bf16");
   if (n_idx == 0 || dim == 0) return AH_OK;
   AH_ARG(wte && wpe && tok && out && T > 0, "ah_embedding_tok_pos: null operand");
   AH_ARG(aligned16(wte) && aligned16(wpe) && aligned16(out), "ah_embedding_tok_pos: operands must be 16-byte aligned");
-  ah::launch_kernel(k_embedding_tok_pos, dim3((unsigned)cdiv(n_idx, WPB)), dim3(TPB), 0, dp<const float>(wte),
-                     dp<const float>(wpe), dp<const int32_t>(tok), dp<float>(out), n_idx, T, dim, vocab);
+  if (out_dtype == AH_F32)
+    ah::launch_kernel(k_embedding_tok_pos<float>, dim3((unsigned)cdiv(n_idx, WPB)), dim3(TPB), 0, dp<const float>(wte),
+                       dp<const float>(wpe), dp<const int32_t>(tok), dp<float>(out), n_idx, T, dim, vocab);
+  else
+    ah::launch_kernel(k_embedding_tok_pos<uint16_t>, dim3((unsigned)cdiv(n_idx, WPB)), dim3(TPB), 0, dp<const float>(wte),
+                       dp<const float>(wpe), dp<const int32_t>(tok), dp<uint16_t>(out), n_idx, T, dim, vocab);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
@@ -812,13 +840,15 @@ int32_t ah_pos_embedding_bwd(ah_ptr grad_out, ah_ptr grad_wpe, int64_t batch, in
   return AH_OK;
 }
 
-int32_t ah_layernorm(ah_ptr x, ah_ptr w, ah_ptr b, ah_ptr out, int64_t rows, int64_t dim, float eps, int32_t out_dtype) {
+int32_t ah_layernorm(ah_ptr x, ah_ptr w, ah_ptr b, ah_ptr out, int64_t rows, int64_t dim, float eps, int32_t out_dtype, int32_t x_dtype) {
   AH_REQUIRE_READY();
   AH_ARG(out_dtype == AH_F32 || out_dtype == AH_BF16, "ah_layernorm: out dtype must be f32 or bf16");
+  AH_ARG(x_dtype == AH_F32 || (x_dtype == AH_BF16 && out_dtype == AH_BF16), "ah_layernorm: x is f32, or bf16 with a bf16 result");
   if (rows == 0 || dim == 0) return AH_OK;
   AH_ARG(x && w && b && out, "ah_layernorm: null operand");
   AH_ARG(dim < (int64_t(1) << 30), "ah_layernorm: row too long");
-  return out_dtype == AH_F32 ? launch_ln<float>(x, w, b, out, rows, dim, eps) : launch_ln<uint16_t>(x, w, b, out, rows, dim, eps);
+  if (x_dtype == AH_BF16) return launch_ln<uint16_t, uint16_t>(x, w, b, out, rows, dim, eps);
+  return out_dtype == AH_F32 ? launch_ln<float, float>(x, w, b, out, rows, dim, eps) : launch_ln<uint16_t, float>(x, w, b, out, rows, dim, eps);
 }
 
 #ifndef LNB_ROWS
@@ -837,18 +867,24 @@ static int ln_bwd_blocks(int64_t rows) {
 
 // dx and the per-block partial column sums part[2][nblk][dim] (dw partials, then db partials)
 static int32_t ln_bwd_launch(ah_ptr x, ah_ptr w, ah_ptr grad_out, int32_t grad_dtype, ah_ptr residual_grad, ah_ptr dx, ah_ptr dx_bf16,
-                             float *part, int nblk, int64_t rows, int64_t dim, float eps) {
+                             float *part, int nblk, int64_t rows, int64_t dim, float eps, int32_t stream_dtype = AH_F32) {
   size_t lds = sizeof(float) * 2 * WPB * (size_t)dim;
   float *part_dw = part, *part_db = part + (size_t)nblk * dim;
-  bool vec = dim % 4 == 0 && dim <= 2048 && aligned16(x) && aligned16(w) && aligned16(dx) && (grad_out % 8 == 0) && (residual_grad % 16 == 0) &&
+  const unsigned sa = stream_dtype == AH_BF16 ? 8 : 16;       // bytes of four stream elements
+  bool vec = dim % 4 == 0 && dim <= 2048 && x % sa == 0 && aligned16(w) && aligned16(dx) && (grad_out % 8 == 0) && (residual_grad % sa == 0) &&
              (dx_bf16 % 8 == 0) && (grad_dtype == AH_BF16 || aligned16(grad_out));
+  if (stream_dtype == AH_BF16)
+    AH_ARG(vec && grad_dtype == AH_BF16 && dx_bf16, "ah_layernorm_bwd_deferred: a bf16 stream needs bf16 gradients, a bf16 dx and rows of 4 k <= 2048 aligned elements");
+  else
+    AH_ARG(dx != 0, "ah_layernorm_bwd: null dx");
   if (vec) {
     int nvl = (int)cdiv(dim / 4, 64);
-#define LNB_CASE(NV, GT) ah::launch_kernel((k_layernorm_bwd_vec<NV, GT>), dim3(nblk), dim3(TPB), lds, dp<const float>(x), dp<const float>(w), \
-      dp<const GT>(grad_out), dp<const float>(residual_grad), dp<float>(dx), dp<uint16_t>(dx_bf16), part_dw, part_db, rows, (int)dim, eps)
-#define LNB_SWITCH(GT) switch (nvl) { case 1: LNB_CASE(1, GT); break; case 2: LNB_CASE(2, GT); break; case 3: LNB_CASE(3, GT); break; \
-      case 4: LNB_CASE(4, GT); break; case 5: case 6: LNB_CASE(6, GT); break; default: LNB_CASE(8, GT); break; }
-    if (grad_dtype == AH_F32) { LNB_SWITCH(float) } else { LNB_SWITCH(uint16_t) }
+#define LNB_CASE(NV, GT, XT) ah::launch_kernel((k_layernorm_bwd_vec<NV, GT, XT>), dim3(nblk), dim3(TPB), lds, dp<const XT>(x), dp<const float>(w), \
+      dp<const GT>(grad_out), dp<const XT>(residual_grad), dp<float>(dx), dp<uint16_t>(dx_bf16), part_dw, part_db, rows, (int)dim, eps)
+#define LNB_SWITCH(GT, XT) switch (nvl) { case 1: LNB_CASE(1, GT, XT); break; case 2: LNB_CASE(2, GT, XT); break; case 3: LNB_CASE(3, GT, XT); break; \
+      case 4: LNB_CASE(4, GT, XT); break; case 5: case 6: LNB_CASE(6, GT, XT); break; default: LNB_CASE(8, GT, XT); break; }
+    if (stream_dtype == AH_BF16) { LNB_SWITCH(uint16_t, uint16_t) }
+    else if (grad_dtype == AH_F32) { LNB_SWITCH(float, float) } else { LNB_SWITCH(uint16_t, float) }
 #undef LNB_SWITCH
 #undef LNB_CASE
   } else if (grad_dtype == AH_F32)
@@ -890,14 +926,15 @@ int64_t ah_layernorm_bwd_partials_bytes(int64_t rows, int64_t dim) {
 }
 
 int32_t ah_layernorm_bwd_deferred(ah_ptr x, ah_ptr w, ah_ptr grad_out, int32_t grad_dtype, ah_ptr residual_grad, ah_ptr dx, ah_ptr dx_bf16,
-                                  ah_ptr partials, int64_t rows, int64_t dim, float eps) {
+                                  ah_ptr partials, int64_t rows, int64_t dim, float eps, int32_t stream_dtype) {
   AH_REQUIRE_READY();
   AH_ARG(grad_dtype == AH_F32 || grad_dtype == AH_BF16, "ah_layernorm_bwd_deferred: grad dtype must be f32 or bf16");
+  AH_ARG(stream_dtype == AH_F32 || stream_dtype == AH_BF16, "ah_layernorm_bwd_deferred: stream dtype must be f32 or bf16");
   AH_ARG(rows > 0 && dim > 0, "ah_layernorm_bwd_deferred: empty input [%lld, %lld]", (long long)rows, (long long)dim);
-  AH_ARG(x && w && grad_out && dx && partials, "ah_layernorm_bwd_deferred: null operand");
+  AH_ARG(x && w && grad_out && (dx || stream_dtype == AH_BF16) && partials, "ah_layernorm_bwd_deferred: null operand");
   AH_ARG(partials % 4 == 0, "ah_layernorm_bwd_deferred: partials must be aligned to 4 bytes");
   AH_ARG(sizeof(float) * 2 * WPB * (size_t)dim <= 160 * 1024, "ah_layernorm_bwd_deferred: dim %lld too large for the LDS column accumulators", (long long)dim);
-  return ln_bwd_launch(x, w, grad_out, grad_dtype, residual_grad, dx, dx_bf16, dp<float>(partials), ln_bwd_blocks(rows), rows, dim, eps);
+  return ln_bwd_launch(x, w, grad_out, grad_dtype, residual_grad, dx, dx_bf16, dp<float>(partials), ln_bwd_blocks(rows), rows, dim, eps, stream_dtype);
 }
 
 int32_t ah_layernorm_colsums(const AhColsumJob *jobs, int32_t count) {

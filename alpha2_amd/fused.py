@@ -7,6 +7,8 @@ Differences from the op-by-op path are layout and fusion only; the arithmetic is
   * tok+pos embedding and their add are one kernel; the residual adds are GEMM epilogues; GELU (+ saved
     pre-activation) and its derivative are GEMM epilogues; attention reads Q, K, V in place out of the [BT, 3C]
     projection and writes merged heads;
+  * every activation is bf16, by default the residual stream and the gradient flowing back along it too (stream="f32"
+    keeps those two in f32: 3 % slower, losses equal to 1e-4 relative);
   * parameters, gradients and Adam moments each live in ONE arena ordered [decayed | not decayed], so the gradient
     norm is one reduction and AdamW is two launches; the clip coefficient never visits the host
     (trainer.ts:1650-1656 computes it on the host from a read-back norm);
@@ -46,7 +48,7 @@ class StepStats:
 
 class FusedTrainer:
     def __init__(self, backend: HipBackend, cfg: ModelConfig, tc: TrainConfig, batch: int, seed: int = 0, use_graph: bool = True,
-                 accum: int = 1, params: Optional[dict] = None, dw_groups: int = 1):
+                 accum: int = 1, params: Optional[dict] = None, dw_groups: int = 1, stream: str = "bf16"):
         self.act = cfg.ffnActivation or "gelu"
         if self.act not in ("gelu", "silu", "relu", "swiglu", "universal", "kan_spline") or cfg.dropout != 0:
             raise ValueError("FusedTrainer schedules the gelu / silu / relu / swiglu / universal / kan_spline blocks without dropout; "
@@ -59,6 +61,15 @@ class FusedTrainer:
             raise ValueError("FusedTrainer needs head_dim in {32,64,128}, nEmbd and ffnDim multiples of 64, vocab multiple of 8")
         self.BT = batch * self.T
         self.dw_groups = max(1, min(int(dw_groups), self.L))
+        # The residual stream x and the gradient that flows back along it: f32, or bf16 like every other activation
+        # ("bf16": the residual epilogues and the LayerNorm kernels move half the bytes; each add into the stream then rounds
+        # to 8 bits, as in any all-bf16-activation step)
+        if stream not in ("f32", "bf16"):
+            raise ValueError("stream must be 'f32' or 'bf16'")
+        self.stream = stream
+        self.SD = F32 if stream == "f32" else BF16
+        if stream == "bf16" and (self.C % 4 or self.C > 2048):
+            raise ValueError("a bf16 residual stream needs nEmbd % 4 == 0 and nEmbd <= 2048")
         self.cap = cfg.softCap if cfg.softCap is not None else 30.0
         self._bufs: List[int] = []
         self._graph = None
@@ -103,8 +114,9 @@ class FusedTrainer:
         # of every step then sums in a fixed order without sorting again (0 bytes = sizes outside that path)
         self._index_bytes = int(self.lib.ah_embedding_index_bytes(BT, V))
         self.tok_index = [a(self._index_bytes) if self._index_bytes else 0 for _ in range(self.accum)]
-        self.x = [a(BT * Cc * 4) for _ in range(self.L + 1)]            # residual stream entering layer l (f32)
-        self.xmid = [a(BT * Cc * 4) for _ in range(self.L)]
+        ss = 4 if self.SD == F32 else 2
+        self.x = [a(BT * Cc * ss) for _ in range(self.L + 1)]           # residual stream entering layer l
+        self.xmid = [a(BT * Cc * ss) for _ in range(self.L)]
         self.ln1 = [a(BT * Cc * 2) for _ in range(self.L)]
         self.qkv = [a(BT * 3 * Cc * 2) for _ in range(self.L)]
         self.att = [a(BT * Cc * 2) for _ in range(self.L)]
@@ -128,7 +140,7 @@ class FusedTrainer:
             self.dact = a(BT * Fd * 2)                                # gradient of the activation's output (one layer at a time)
         self.hact = [a(BT * Fd * 2) for _ in range(self.L)]
         self.lnf, self.logits, self.rowlse = a(BT * Cc * 2), a(BT * V * 2), a(BT * 4)
-        self.dx = [a(BT * Cc * 4), a(BT * Cc * 4)]
+        self.dx = [a(BT * Cc * 4), a(BT * Cc * 4) if self.SD == F32 else 0]      # f32 gradient stream (bf16 stream: only the embedding's)
         self.dlnb, self.datt = a(BT * Cc * 2), a(BT * Cc * 2)
         # Output gradients of the four linears are kept per layer (bf16): every weight gradient dW = dY^T X of the step is
         # computed at the end of backward by ONE grouped GEMM launch over full K = tokens, instead of 4 small split-K
@@ -284,14 +296,15 @@ class FusedTrainer:
         NN, NT, TN = ffi.GEMM_NN, ffi.GEMM_NT, ffi.GEMM_TN
         acc = 0 if first_micro else 1
         wepi = ffi.EPI_NONE if first_micro else ffi.EPI_ACCUM
-        check(lib.ah_embedding_tok_pos(self.p("wte"), self.p("wpe"), self.tok, self.x[0], BT, self.T, Cc, V))
+        SD = self.SD
+        check(lib.ah_embedding_tok_pos(self.p("wte"), self.p("wpe"), self.tok, self.x[0], BT, self.T, Cc, V, SD))
         for l in range(L):
             pre = f"layer.{l}."
-            check(lib.ah_layernorm(self.x[l], self.p(pre + "ln1.weight"), self.p(pre + "ln1.bias"), self.ln1[l], BT, Cc, 1e-5, BF16))
+            check(lib.ah_layernorm(self.x[l], self.p(pre + "ln1.weight"), self.p(pre + "ln1.bias"), self.ln1[l], BT, Cc, 1e-5, BF16, SD))
             self._gemm(NT, self.ln1[l], self.p(pre + "attn.wqkv", True), self.qkv[l], BT, 3 * Cc, Cc, Cc, Cc, 3 * Cc)
             self._flash(l, False)
-            self._gemm(NT, self.att[l], self.p(pre + "attn.wo", True), self.xmid[l], BT, Cc, Cc, Cc, Cc, Cc, F32, ffi.EPI_RESIDUAL, self.x[l])
-            check(lib.ah_layernorm(self.xmid[l], self.p(pre + "ln2.weight"), self.p(pre + "ln2.bias"), self.ln2[l], BT, Cc, 1e-5, BF16))
+            self._gemm(NT, self.att[l], self.p(pre + "attn.wo", True), self.xmid[l], BT, Cc, Cc, Cc, Cc, Cc, SD, ffi.EPI_RESIDUAL, self.x[l])
+            check(lib.ah_layernorm(self.xmid[l], self.p(pre + "ln2.weight"), self.p(pre + "ln2.bias"), self.ln2[l], BT, Cc, 1e-5, BF16, SD))
             if self.act == "gelu":
                 self._gemm(NT, self.ln2[l], self.p(pre + "mlp.fc1", True), self.hact[l], BT, Fd, Cc, Cc, Cc, Fd, BF16, ffi.EPI_GELU_GRAD, self.hgrad[l])
             else:
@@ -301,8 +314,8 @@ class FusedTrainer:
                     check(lib.ah_swiglu(BF16, self.hpre[l], self.hact[l], BT, Fd))
                 else:
                     check(lib.ah_channel_act(BF16, self.hpre[l], self._coef_handles(l, self.p), self._act_mask, self.hact[l], BT, Fd))
-            self._gemm(NT, self.hact[l], self.p(pre + self.w2, True), self.x[l + 1], BT, Cc, Fd, Fd, Fd, Cc, F32, ffi.EPI_RESIDUAL, self.xmid[l])
-        check(lib.ah_layernorm(self.x[L], self.p("lnF.weight"), self.p("lnF.bias"), self.lnf, BT, Cc, 1e-5, BF16))
+            self._gemm(NT, self.hact[l], self.p(pre + self.w2, True), self.x[l + 1], BT, Cc, Fd, Fd, Fd, Cc, SD, ffi.EPI_RESIDUAL, self.xmid[l])
+        check(lib.ah_layernorm(self.x[L], self.p("lnF.weight"), self.p("lnF.bias"), self.lnf, BT, Cc, 1e-5, BF16, SD))
         self._gemm(NT, self.lnf, self.p("lmHead", True), self.logits, BT, V, Cc, Cc, Cc, V)
         # loss and dlogits (in place) from one read of the logits
         if self.accum == 1:
@@ -315,8 +328,9 @@ class FusedTrainer:
 
         self._gemm(NN, self.logits, self.p("lmHead", True), self.dlnb, BT, Cc, V, V, Cc, Cc)
         cur = 0
-        check(lib.ah_layernorm_bwd_deferred(self.x[L], self.p("lnF.weight"), self.dlnb, BF16, 0, self.dx[cur], self.dy_fc2[L - 1],
-                                            self._ln_part["lnF"], BT, Cc, 1e-5))
+        f32s = SD == F32                           # f32 stream: gradient in dx[cur] with bf16 copies; bf16 stream: the copies are the stream
+        check(lib.ah_layernorm_bwd_deferred(self.x[L], self.p("lnF.weight"), self.dlnb, BF16, 0, self.dx[cur] if f32s else 0, self.dy_fc2[L - 1],
+                                            self._ln_part["lnF"], BT, Cc, 1e-5, SD))
         for l in reversed(range(L)):
             pre = f"layer.{l}."
             # MLP: x_out = x_mid + fc2(gelu(fc1(ln2(x_mid))))
@@ -330,16 +344,17 @@ class FusedTrainer:
                     check(lib.ah_channel_act_bwd(BF16, self.hpre[l], self._coef_handles(l, self.p), self._act_mask, self.dact, self.dh[l],
                                                  self._coef_handles(l, self.g), acc, BT, Fd))
             self._gemm(NN, self.dh[l], self.p(pre + self.w1, True), self.dlnb, BT, Cc, self.Fin, self.Fin, Cc, Cc)
-            check(lib.ah_layernorm_bwd_deferred(self.xmid[l], self.p(pre + "ln2.weight"), self.dlnb, BF16, self.dx[cur], self.dx[cur ^ 1], self.dy_wo[l],
-                                                self._ln_part[pre + "ln2"], BT, Cc, 1e-5))
-            cur ^= 1
+            check(lib.ah_layernorm_bwd_deferred(self.xmid[l], self.p(pre + "ln2.weight"), self.dlnb, BF16, self.dx[cur] if f32s else self.dy_fc2[l],
+                                                self.dx[cur ^ 1] if f32s else 0, self.dy_wo[l], self._ln_part[pre + "ln2"], BT, Cc, 1e-5, SD))
+            cur ^= f32s
             # attention: x_mid = x_in + wo(attn(wqkv(ln1(x_in))))
             self._gemm(NN, self.dy_wo[l], self.p(pre + "attn.wo", True), self.datt, BT, Cc, Cc, Cc, Cc, Cc)
             self._flash(l, True)
             self._gemm(NN, self.dqkv[l], self.p(pre + "attn.wqkv", True), self.dlnb, BT, Cc, 3 * Cc, 3 * Cc, Cc, Cc)
-            check(lib.ah_layernorm_bwd_deferred(self.x[l], self.p(pre + "ln1.weight"), self.dlnb, BF16, self.dx[cur], self.dx[cur ^ 1],
-                                                self.dy_fc2[l - 1] if l > 0 else self.dxb0, self._ln_part[pre + "ln1"], BT, Cc, 1e-5))
-            cur ^= 1
+            check(lib.ah_layernorm_bwd_deferred(self.x[l], self.p(pre + "ln1.weight"), self.dlnb, BF16, self.dx[cur] if f32s else self.dy_wo[l],
+                                                self.dx[cur ^ 1] if f32s else (self.dx[0] if l == 0 else 0),      # the embeddings take their gradient in f32
+                                                self.dy_fc2[l - 1] if l > 0 else self.dxb0, self._ln_part[pre + "ln1"], BT, Cc, 1e-5, SD))
+            cur ^= f32s
             if self.dw_groups > 1 and l in self._dw_after_layer:
                 self._weight_grads(wepi, self._dw_after_layer[l])
         jobs = (ffi.AhColsumJob * len(self._ln_jobs))(*[

@@ -93,6 +93,7 @@ def main():
     ap.add_argument("--mode", choices=["fast", "backend", "parity"], default="fast")
     ap.add_argument("--no-step-graphs", action="store_true", help="backend mode: issue every launch eagerly")
     ap.add_argument("--dw-groups", type=int, default=1, help="fast mode: weight-gradient GEMMs in this many runs on a second stream")
+    ap.add_argument("--stream", choices=["f32", "bf16"], default="bf16", help="fast mode: storage type of the residual stream and its gradient")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--cpu-tokens", type=int, default=32)
     ap.add_argument("--workload", choices=sorted(WORKLOADS), default="gpt2-small")
@@ -132,7 +133,7 @@ def main():
             return runner.step([(B.reshape(x, x.shape), B.reshape(y, y.shape)) for x, y in pick])
     else:
         from alpha2_amd.fused import FusedTrainer
-        runner = FusedTrainer(B, cfg, tc, BATCH, seed=0, accum=accum, dw_groups=args.dw_groups)
+        runner = FusedTrainer(B, cfg, tc, BATCH, seed=0, accum=accum, dw_groups=args.dw_groups, stream=args.stream)
         dtype = "bf16"
         ids = [runner.add_batch(x, y) for x, y in micro]                   # resident in HBM before the timed region
         cursor = [0]
@@ -207,6 +208,8 @@ def main():
         out["config"]["step_plans"] = step_stats
     if args.mode == "fast" and args.dw_groups > 1:
         out["config"]["dw_groups"] = args.dw_groups
+    if args.mode == "fast":
+        out["config"]["residual_stream"] = args.stream
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(model, args.cpu_tokens)
     print(json.dumps(out))

@@ -231,7 +231,7 @@ int32_t ah_embedding(ah_ptr weight, ah_ptr idx_i32, ah_ptr out, int64_t n_idx, i
                      int32_t out_dtype);
 /* out[i] = wte[tok[i]] + wpe[i % T]  -- tok+pos embedding and the add of gpt.ts:362-379 in one pass */
 int32_t ah_embedding_tok_pos(ah_ptr wte, ah_ptr wpe, ah_ptr tok_i32, ah_ptr out, int64_t n_idx, int64_t T,
-                             int64_t dim, int64_t vocab);
+                             int64_t dim, int64_t vocab, int32_t out_dtype);
 /* grad_w[vocab,dim] = scatter-add of grad_out rows (zero-filled first unless accumulate != 0); ids outside [0, vocab) are
  * skipped.  Up to 32768 positions over fewer than 65535 ids (rows of 4 k floats) the order of the additions is fixed: the
  * positions are sorted by (id, position), the rows of an id are added in position order inside chunks of 32 sorted positions
@@ -255,8 +255,9 @@ int32_t ah_pos_embedding_bwd(ah_ptr grad_out, ah_ptr grad_wpe, int64_t batch, in
  * (the target of the corpus' last token is its first).  corpus, inputs, targets: i32; starts: i64[batch] on the device. */
 int32_t ah_token_windows(ah_ptr corpus_i32, int64_t n_tokens, ah_ptr starts_i64, int64_t batch, int64_t T,
                          ah_ptr inputs_i32, ah_ptr targets_i32);
+/* x_dtype: AH_F32, or AH_BF16 (with a bf16 result) for a caller that keeps its residual stream in bf16 */
 int32_t ah_layernorm(ah_ptr x, ah_ptr w, ah_ptr b, ah_ptr out, int64_t rows, int64_t dim, float eps,
-                     int32_t out_dtype);
+                     int32_t out_dtype, int32_t x_dtype);
 /* dx (+= residual_grad when that handle is non-zero), dw, db.  dw/db are deterministic column sums;
  * accumulate != 0 adds them into existing dw/db (gradient accumulation). grad_out dtype f32 or bf16.
  * dx_bf16 (0 = none) also receives dx rounded to bf16, the operand of the next backward GEMMs. */
@@ -267,7 +268,9 @@ int32_t ah_layernorm_bwd(ah_ptr x, ah_ptr w, ah_ptr grad_out, int32_t grad_dtype
  * least ah_layernorm_bwd_partials_bytes(rows, dim) bytes, which is 0 before ah_init), and ONE later call of
  * ah_layernorm_colsums reduces those of many LayerNorms (the 2 L + 1 of a model's backward pass) in one launch instead of
  * one small launch each; per job the result is bit-identical to ah_layernorm_bwd's.  The reference computes dw / db inside
- * layerNormBackward (packages/tensor/src/cpu_ref.ts, layerNormBackward); nothing of this split shows at the Backend level. */
+ * layerNormBackward (packages/tensor/src/cpu_ref.ts, layerNormBackward); nothing of this split shows at the Backend level.
+ * stream_dtype = the type of x and residual_grad: AH_F32, or AH_BF16 for a residual stream and gradient stream kept in bf16
+ * (bf16 grad_out, dim % 4 == 0, dim <= 2048); dx (f32) may then be 0, dx_bf16 being the stream that the next call adds to. */
 typedef struct {
   ah_ptr  partials, dw, db;
   int64_t rows, dim;          /* as passed to ah_layernorm_bwd_deferred */
@@ -275,7 +278,8 @@ typedef struct {
 } AhColsumJob;
 int64_t ah_layernorm_bwd_partials_bytes(int64_t rows, int64_t dim);
 int32_t ah_layernorm_bwd_deferred(ah_ptr x, ah_ptr w, ah_ptr grad_out, int32_t grad_dtype, ah_ptr residual_grad,
-                                  ah_ptr dx, ah_ptr dx_bf16, ah_ptr partials, int64_t rows, int64_t dim, float eps);
+                                  ah_ptr dx, ah_ptr dx_bf16, ah_ptr partials, int64_t rows, int64_t dim, float eps,
+                                  int32_t stream_dtype);
 int32_t ah_layernorm_colsums(const AhColsumJob *jobs, int32_t count);
 /* loss[0] = mean_i (logsumexp(logits[i,:]) - logits[i,target[i]]); lse[N] kept for backward (0 = skip) */
 int32_t ah_cross_entropy(ah_ptr logits, int32_t logits_dtype, ah_ptr targets_i32, ah_ptr loss_out, ah_ptr lse_out,
@@ -299,7 +303,7 @@ int32_t ah_cross_entropy_fwd_bwd(ah_ptr logits, int32_t dtype, ah_ptr targets_i3
  *      (0 = operand shared across the batch).
  *      Epilogues: AH_EPI_NONE; AH_EPI_ACCUM  C += acc (gradient accumulation);
  *      AH_EPI_GELU  C = gelu(acc), aux (same dtype/ld as C) = acc  (matmulTransposedGelu, ops.ts:426-487);
- *      AH_EPI_RESIDUAL  C = acc + aux (aux f32 [M,N], ld = ldc) (residual add of gpt.ts:280-281);
+ *      AH_EPI_RESIDUAL  C = acc + aux (aux [M,N] of C's dtype, ld = ldc; f32, or bf16 from bf16 operands) (residual add of gpt.ts:280-281);
  *      AH_EPI_GELU_BWD  C = acc * gelu'(aux) (aux = saved pre-activation, dtype of C);
  *      AH_EPI_GELU_GRAD C = gelu(acc), aux = gelu'(acc): the forward saves the derivative instead of the pre-activation,
  *      so that the backward product needs only  AH_EPI_MUL_AUX  C = acc * aux  (one multiply per element instead of

@@ -283,3 +283,42 @@ def test_fused_step_with_the_other_mlp_activations_matches_oracle(B, act, accum)
     for name, v in orc.entries:                                           # three AdamW steps: every entry within 3 lr of the oracle's
         assert np.max(np.abs(ft.param(name) - v.data.data)) <= 3 * 2 * 3e-4 * 1.001 + 1e-6, name
     ft.close()
+
+
+def test_fused_step_with_a_bf16_residual_stream_tracks_the_oracle(B):
+    """stream = "bf16" (the default): the residual stream and its gradient in bf16 like every other activation; stream = "f32"
+    keeps them in f32.  Both against the fp32 oracle at the bf16 bars (loss 2e-2 relative over 50 steps, gradient direction and
+    size), and against each other."""
+    from alpha2_amd.fused import FusedTrainer
+    from alpha2_amd.model import ModelConfig
+    from alpha2_amd.train import TrainConfig, syntheticBatch
+    steps = 50
+    tc = dict(iters=steps, lr=1e-3)
+    f16 = FusedTrainer(B, ModelConfig(**CFG), TrainConfig(**tc), 4, seed=0, use_graph=True, stream="bf16")
+    f32 = FusedTrainer(B, ModelConfig(**CFG), TrainConfig(**tc), 4, seed=0, use_graph=True, stream="f32")
+    orc = rm.Trainer(rm.ModelConfig(**CFG), rm.TrainConfig(**tc), seed=0)
+    ob = rm.synthetic_batch(1, 4, 64, 256)
+    _, oloss = rm.gptForward(orc.cfg, orc.params, orc.B, orc.tape, ob[0], ob[1], True)
+    orc.tape.backward(oloss, orc.B)
+    ograds = {n: v.grad.data.copy() for n, v in orc.entries}
+    orc.tape.clear()
+    for _, v in orc.entries:
+        v.grad = None
+    i16, i32 = f16.add_batch(*syntheticBatch(1, 4, 64, 256)), f32.add_batch(*syntheticBatch(1, 4, 64, 256))
+    worst = worst_pair = 0.0
+    for s in range(steps):
+        o = orc.step([ob])
+        f16.step(i16), f32.step(i32)
+        a, b = f16.history(s, s + 1)[0], f32.history(s, s + 1)[0]
+        worst = max(worst, abs(a.loss - o.loss) / abs(o.loss), abs(b.loss - o.loss) / abs(o.loss))
+        worst_pair = max(worst_pair, abs(a.loss - b.loss) / abs(b.loss))
+        if s == 0:
+            for ft in (f16, f32):
+                for name, g in ograds.items():
+                    got, w = ft.grad(name).astype(np.float64), g.astype(np.float64)
+                    cos = float(got @ w / (np.linalg.norm(got) * np.linalg.norm(w) + 1e-300))
+                    assert cos > 0.995, (ft.stream, name, cos)
+                    assert abs(np.linalg.norm(got) / np.linalg.norm(w) - 1) < 3e-2, (ft.stream, name)
+    assert worst <= 2e-2, worst
+    assert worst_pair <= 1e-2, worst_pair
+    f16.close(), f32.close()

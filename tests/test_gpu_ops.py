@@ -466,6 +466,56 @@ def test_layernorm_fwd_bwd(B, rows, dim):
     assert_close(r["db"].data, db.data, what="ln.db")
 
 
+@pytest.mark.parametrize("rows,dim", [(3, 8), (130, 260), (333, 768), (64, 2048), (4096, 1024)])
+def test_layernorm_on_a_bf16_residual_stream(B, rows, dim):
+    """x, the residual gradient and dx in bf16 (ah_layernorm with x_dtype = bf16, ah_layernorm_bwd_deferred with stream_dtype = bf16;
+    cpu_ref.ts:387-420, ops.ts:509-571): the f32 arithmetic of the oracle on the bf16-rounded inputs, results rounded once.  The
+    f32 copy of dx is written only where asked for.  tok + pos embedding straight to bf16 as well."""
+    import ctypes as C
+    from alpha2_amd import _ffi as ffi
+    lib = B.lib
+    x = _bf16_round((rs.randn(rows, dim) * 2 + 0.5).astype(np.float32))[0]
+    g, res = _bf16_round(rs.randn(rows, dim).astype(np.float32))[0], _bf16_round(rs.randn(rows, dim).astype(np.float32))[0]
+    w, b_ = rs.randn(dim).astype(np.float32), rs.randn(dim).astype(np.float32)
+    tx, px = _raw_buf(B, x, True); tg, pg = _raw_buf(B, g, True); tr, pr = _raw_buf(B, res, True)
+    wd, bd = dev(B, w), dev(B, b_)
+    to, po = _raw_buf(B, np.zeros((rows, dim), np.float32), True)
+    ffi.check(lib.ah_layernorm(px, B._ptr(wd), B._ptr(bd), po, rows, dim, 1e-5, ffi.BF16, ffi.BF16))
+    want = O.layerNorm(orc(x), orc(w), orc(b_), 1e-5).data.reshape(rows, dim)
+    assert_close(_raw_read(B, to, True), want, rel=2.0 ** -8, what="ln16")
+    assert lib.ah_layernorm(px, B._ptr(wd), B._ptr(bd), po, rows, dim, 1e-5, ffi.F32, ffi.BF16) != 0          # bf16 in, f32 out: not provided
+    dx, dw, db = ref.layernorm_backward(orc(x), orc(w), orc(g), 1e-5)
+    want_dx = dx.data.reshape(rows, dim) + res
+    nbytes = lib.ah_layernorm_bwd_partials_bytes(rows, dim)
+    part = B.zeros((nbytes // 4,))
+    td, pd = _raw_buf(B, np.zeros((rows, dim), np.float32), True)
+    df = B.zeros((rows, dim))
+    dwd, dbd = B.zeros((dim,)), B.zeros((dim,))
+    for f32_copy in (0, B._ptr(df)):
+        ffi.check(lib.ah_layernorm_bwd_deferred(px, B._ptr(wd), pg, ffi.BF16, pr, f32_copy, pd, B._ptr(part), rows, dim, 1e-5, ffi.BF16))
+        term = float(np.max(np.abs(g * w)) / np.sqrt(np.min(x.var(-1)) + 1e-5))
+        assert_close(_raw_read(B, td, True), want_dx, rel=2.0 ** -8, what="ln16.dx", scale=term if dim < 16 else 0.0)
+    B._dirty(df)
+    assert_close(df.data, want_dx, what="ln16.dx f32 copy", scale=term if dim < 16 else 0.0)
+    jobs = (ffi.AhColsumJob * 1)(ffi.AhColsumJob(B._ptr(part), B._ptr(dwd), B._ptr(dbd), rows, dim, 0, 0))
+    ffi.check(lib.ah_layernorm_colsums(jobs, 1))
+    B._dirty(dwd); B._dirty(dbd)
+    assert_close(dwd.data, dw.data, what="ln16.dw")
+    assert_close(dbd.data, db.data, what="ln16.db")
+    # a bf16 stream with f32 gradients is refused
+    assert lib.ah_layernorm_bwd_deferred(px, B._ptr(wd), B._ptr(df), ffi.F32, pr, 0, pd, B._ptr(part), rows, dim, 1e-5, ffi.BF16) != 0
+    # tok + pos embedding written as bf16
+    V, T = 50, 7
+    n = (rows // T) * T
+    if n:
+        wte, wpe = rs.randn(V, dim).astype(np.float32), rs.randn(T, dim).astype(np.float32)
+        tok = rs.randint(0, V, size=n).astype(np.int32)
+        te, pe = _raw_buf(B, np.zeros((n, dim), np.float32), True)
+        wted, wped, tokd = dev(B, wte), dev(B, wpe), dev(B, tok, "i32")
+        ffi.check(lib.ah_embedding_tok_pos(B._ptr(wted), B._ptr(wped), B._ptr(tokd), pe, n, T, dim, V, ffi.BF16))
+        assert np.array_equal(_raw_read(B, te, True), _bf16_round(wte[tok] + wpe[np.arange(n) % T])[0])
+
+
 def test_layernorm_backward_with_column_sums_put_off(B):
     """ah_layernorm_bwd_deferred + one ah_layernorm_colsums over several LayerNorms of different sizes gives exactly the dx,
     dw and db of ah_layernorm_bwd, also when accumulating onto existing dw / db; bad jobs are reported."""
@@ -484,7 +534,7 @@ def test_layernorm_backward_with_column_sums_put_off(B):
         part = B.zeros((nbytes // 4,))
         keep += [xd, wd, gd, dx_, dw_, db_, dx2, dw2, db2, part]
         ffi.check(lib.ah_layernorm_bwd(B._ptr(xd), B._ptr(wd), B._ptr(gd), ffi.F32, 0, B._ptr(dx_), 0, B._ptr(dw_), B._ptr(db_), rows, dim, 1e-5, 1))
-        ffi.check(lib.ah_layernorm_bwd_deferred(B._ptr(xd), B._ptr(wd), B._ptr(gd), ffi.F32, 0, B._ptr(dx2), 0, B._ptr(part), rows, dim, 1e-5))
+        ffi.check(lib.ah_layernorm_bwd_deferred(B._ptr(xd), B._ptr(wd), B._ptr(gd), ffi.F32, 0, B._ptr(dx2), 0, B._ptr(part), rows, dim, 1e-5, ffi.F32))
         jobs.append(ffi.AhColsumJob(B._ptr(part), B._ptr(dw2), B._ptr(db2), rows, dim, 1, 0))
         wants.append((dx_, dw_, db_, dx2, dw2, db2))
     arr = (ffi.AhColsumJob * len(jobs))(*jobs)
@@ -499,7 +549,7 @@ def test_layernorm_backward_with_column_sums_put_off(B):
     assert lib.ah_layernorm_colsums(arr, 0) == 0
     bad = (ffi.AhColsumJob * 1)(ffi.AhColsumJob(0, 1 << 20, 1 << 20, 4, 4, 0, 0))
     assert lib.ah_layernorm_colsums(bad, 1) != 0 and b"null operand" in lib.ah_last_error()
-    assert lib.ah_layernorm_bwd_deferred(1 << 20, 1 << 20, 1 << 20, ffi.F32, 0, 1 << 20, 0, 0, 4, 4, 1e-5) != 0 and b"null operand" in lib.ah_last_error()
+    assert lib.ah_layernorm_bwd_deferred(1 << 20, 1 << 20, 1 << 20, ffi.F32, 0, 1 << 20, 0, 0, 4, 4, 1e-5, ffi.F32) != 0 and b"null operand" in lib.ah_last_error()
 
 
 @pytest.mark.parametrize("n,c", [(2, 3), (11, 37), (128, 256), (16, 50304)])
@@ -727,7 +777,7 @@ def _raw_gemm(B, layout, a, b, m, n, k, in_dtype, out_dtype, epi=0, aux=None, c_
     tc, pc = up(cinit, out_dtype)
     paux = 0
     if aux is not None:
-        taux, paux = up(aux, ffi.F32 if epi == ffi.EPI_RESIDUAL else out_dtype)
+        taux, paux = up(aux, out_dtype)                               # what an epilogue reads has the type of C
     elif epi in (ffi.EPI_GELU, ffi.EPI_GELU_GRAD):
         taux, paux = up(np.zeros((m, n), np.float32), out_dtype)
     lda = a.shape[1]
@@ -760,7 +810,7 @@ def test_gemm_layouts_epilogues_dtypes(B, in_bf16, out_bf16, M, N, K):
     cmp(_raw_gemm(B, ffi.GEMM_NT, a, b, M, N, K, idt, odt)[0], want, "NT")
     cmp(_raw_gemm(B, ffi.GEMM_NN, a, np.ascontiguousarray(b.T), M, N, K, idt, odt)[0], want, "NN")
     cmp(_raw_gemm(B, ffi.GEMM_TN, np.ascontiguousarray(a.T), np.ascontiguousarray(b.T), M, N, K, idt, odt)[0], want, "TN")
-    # provided combinations: ACCUM / RESIDUAL write f32; GELU / GELU_BWD write the operand type
+    # provided combinations: ACCUM / RESIDUAL write f32 (RESIDUAL also bf16 from bf16 operands); GELU / GELU_BWD write the operand type
     if not out_bf16:
         c0 = rs.randn(M, N).astype(np.float32)
         cmp(_raw_gemm(B, ffi.GEMM_NT, a, b, M, N, K, idt, odt, ffi.EPI_ACCUM, c_init=c0)[0], want + c0, "ACCUM")
@@ -768,6 +818,9 @@ def test_gemm_layouts_epilogues_dtypes(B, in_bf16, out_bf16, M, N, K):
             want + c0, "TN ACCUM")
         res = rs.randn(M, N).astype(np.float32)
         cmp(_raw_gemm(B, ffi.GEMM_NT, a, b, M, N, K, idt, odt, ffi.EPI_RESIDUAL, aux=res)[0], want + res, "RESIDUAL")
+    if in_bf16 and out_bf16:                                 # a residual stream kept in bf16: aux and C both bf16
+        res = _bf16_round(rs.randn(M, N).astype(np.float32))[0]
+        cmp(_raw_gemm(B, ffi.GEMM_NT, a, b, M, N, K, idt, odt, ffi.EPI_RESIDUAL, aux=res)[0], want + res, "RESIDUAL bf16")
     if in_bf16 == out_bf16:
         got, pre = _raw_gemm(B, ffi.GEMM_NT, a, b, M, N, K, idt, odt, ffi.EPI_GELU)
         cmp(pre, want, "GELU.pre")
@@ -865,6 +918,8 @@ def test_gemm_bf16_large_tiles_direct_to_lds_kernel(B, M, N, K, tile):
     assert_close(_raw_gemm(B, ffi.GEMM_TN, at, bt, M, N, K, ffi.BF16, ffi.F32)[0], want, rel=1e-4, what="TN")
     c0 = rs.randn(M, N).astype(np.float32)
     assert_close(_raw_gemm(B, ffi.GEMM_TN, at, bt, M, N, K, ffi.BF16, ffi.F32, ffi.EPI_ACCUM, c_init=c0)[0], want + c0, rel=1e-4, what="TN ACCUM")
+    r16 = _bf16_round(c0 * 8)[0]
+    assert_close(_raw_gemm(B, ffi.GEMM_NT, a, b, M, N, K, ffi.BF16, ffi.BF16, ffi.EPI_RESIDUAL, aux=r16)[0], want + r16, rel=2.0 ** -7, what="NT RESIDUAL bf16")
     assert_close(_raw_gemm(B, ffi.GEMM_NT, a, b, M, N, K, ffi.BF16, ffi.F32, ffi.EPI_RESIDUAL, aux=c0)[0], want + c0, rel=1e-4, what="RESIDUAL")
     got, pre = _raw_gemm(B, ffi.GEMM_NT, a, b, M, N, K, ffi.BF16, ffi.BF16, ffi.EPI_GELU)
     assert_close(pre, want, rel=2.0 ** -7, what="GELU.pre")
