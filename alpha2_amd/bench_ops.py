@@ -174,6 +174,12 @@ def bench_bandwidth(b: Bench):
     b.record("layernorm fwd 16384x768", ms, nbytes=rows * dim * 6, note="f32 in, bf16 out")
     ms = b.time(lambda: ffi.check(lib.ah_layernorm_bwd(x, w, g16, ffi.BF16, res, dx, dx16, dw, db, rows, dim, 1e-5, 0)))
     b.record("layernorm bwd 16384x768", ms, nbytes=rows * dim * 16, note="x f32, g bf16, + residual grad f32 -> dx f32 + bf16; dw, db")
+    x16, res16 = b.randn(rows * dim, ffi.BF16, 1.0, 11), b.randn(rows * dim, ffi.BF16, 1.0, 12)
+    part = b.alloc(int(lib.ah_layernorm_bwd_partials_bytes(rows, dim)))
+    ms = b.time(lambda: ffi.check(lib.ah_layernorm(x16, w, bias, out16, rows, dim, 1e-5, ffi.BF16, ffi.BF16)))
+    b.record("layernorm fwd 16384x768, bf16 stream", ms, nbytes=rows * dim * 4, note="bf16 in, bf16 out")
+    ms = b.time(lambda: ffi.check(lib.ah_layernorm_bwd_deferred(x16, w, g16, ffi.BF16, res16, 0, dx16, part, rows, dim, 1e-5, ffi.BF16)))
+    b.record("layernorm bwd 16384x768, bf16 stream", ms, nbytes=rows * dim * 8, note="x, g, residual grad bf16 -> dx bf16; partial dw, db (column sums put off)")
     b.release()
 
     h = b.randn(rows * F, ffi.F32)
@@ -204,7 +210,13 @@ def bench_bandwidth(b: Bench):
     zh = np.ascontiguousarray(zipfBatch(4, 16, rows // 16, V)[0].data, dtype=np.int32).reshape(-1)
     ffi.check(lib.ah_upload(tok, zh.ctypes.data_as(C.c_void_p), zh.nbytes))
     ms = b.time(lambda: ffi.check(lib.ah_embedding_bwd(tok, eo, gw, rows, dim, V, 0)))
-    b.record("embedding scatter-add, power-law ids", ms, nbytes=rows * dim * 8 + V * dim * 4, note="Zipf(1.1) ids as in the step benchmark; same bytes")
+    b.record("embedding scatter-add, power-law ids", ms, nbytes=rows * dim * 8 + V * dim * 4, note="Zipf(1.1) ids as in the step benchmark; same bytes; sorts the ids in every call")
+    ib = int(lib.ah_embedding_index_bytes(rows, V))
+    if ib:
+        index = b.alloc(ib)
+        ffi.check(lib.ah_embedding_index(tok, rows, V, index))
+        ms = b.time(lambda: ffi.check(lib.ah_embedding_bwd_indexed(index, eo, gw, rows, dim, V, 0)))
+        b.record("embedding scatter-add, ids sorted once", ms, nbytes=rows * dim * 8 + V * dim * 4, note="power-law ids, index of the resident batch built beforehand")
     b.release()
 
     p, g, m, v, sh = (b.randn(P, ffi.F32, 0.02, s) for s in (6, 7, 8, 9, 10))

@@ -453,6 +453,31 @@ def test_embedding_backward_is_the_same_from_run_to_run_and_follows_position_ord
     assert_close(outs[0], want, what="scatter-add")
 
 
+
+@pytest.mark.parametrize("n,vocab", [(1, 7), (700, 50304), (1024, 300), (5000, 50304), (16384, 50304), (16384, 3), (20000, 65534), (32768, 50304)])
+def test_embedding_index_is_the_stable_order_by_id(B, n, vocab):
+    """ah_embedding_index: keys (id << 16 | position) of the valid positions in ascending order -- positions of one id in position
+    order, the order ops.ts:491-507 adds them in -- then padding.  Both sort kernels (radix up to 16384 positions, bitonic beyond),
+    power-law ids, ids out of range."""
+    from alpha2_amd import _ffi as ffi
+    lib = B.lib
+    ids = (rs.zipf(1.3, size=n) % vocab).astype(np.int32)
+    ids[rs.rand(n) < 0.01] = -1
+    ids[rs.rand(n) < 0.01] = vocab
+    nbytes = lib.ah_embedding_index_bytes(n, vocab)
+    assert nbytes >= 4 * n
+    tok = dev(B, ids, "i32")
+    out = dev(B, np.zeros(nbytes // 4, np.int32), "i32")
+    ffi.check(lib.ah_embedding_index(B._ptr(tok), n, vocab, B._ptr(out)))
+    B._dirty(out)
+    got = out.data.view(np.uint32)
+    valid = np.nonzero((ids >= 0) & (ids < vocab))[0]
+    order = valid[np.argsort(ids[valid], kind="stable")]
+    want = np.full(nbytes // 4, 0xFFFFFFFF, np.uint32)
+    want[:len(order)] = (ids[order].astype(np.uint32) << 16) | order.astype(np.uint32)
+    assert np.array_equal(got, want)
+
+
 @pytest.mark.parametrize("rows,dim", [(1, 2), (7, 48), (1024, 128), (333, 768), (5, 1000), (3, 4096)])
 def test_layernorm_fwd_bwd(B, rows, dim):
     x = (rs.randn(rows, dim) * 2 + 0.5).astype(np.float32)
