@@ -322,3 +322,36 @@ def test_fused_step_with_a_bf16_residual_stream_tracks_the_oracle(B):
     assert worst <= 2e-2, worst
     assert worst_pair <= 1e-2, worst_pair
     f16.close(), f32.close()
+
+
+@pytest.mark.parametrize("stream", ["bf16", "f32"])
+def test_fused_step_on_a_ragged_shape(B, stream):
+    """72 tokens per batch (3 x 24: not a multiple of the 64-token k-tile, so every weight gradient is a general GEMM instead of
+    the grouped launch; a context shorter than an attention tile), head size 64, a vocabulary that is not a multiple of 64:
+    the edge paths of the same step against the oracle."""
+    from alpha2_amd.fused import FusedTrainer
+    from alpha2_amd.model import ModelConfig
+    from alpha2_amd.train import TrainConfig, syntheticBatch
+    cfg = dict(vocabSize=264, blockSize=24, nLayer=2, nEmbd=128, nHead=2)
+    ft = FusedTrainer(B, ModelConfig(**cfg), TrainConfig(iters=3), 3, seed=0, use_graph=True, stream=stream)
+    orc = rm.Trainer(rm.ModelConfig(**cfg), rm.TrainConfig(iters=3), seed=0)
+    ob = rm.synthetic_batch(2, 3, 24, 264)
+    _, oloss = rm.gptForward(orc.cfg, orc.params, orc.B, orc.tape, ob[0], ob[1], True)
+    orc.tape.backward(oloss, orc.B)
+    ograds = {n: v.grad.data.copy() for n, v in orc.entries}
+    orc.tape.clear()
+    for _, v in orc.entries:
+        v.grad = None
+    i = ft.add_batch(*syntheticBatch(2, 3, 24, 264))
+    for s in range(3):
+        o = orc.step([ob])
+        ft.step(i)
+        st = ft.history(s, s + 1)[0]
+        assert abs(st.loss - o.loss) <= 2e-2 * abs(o.loss), (s, st.loss, o.loss)
+        assert abs(st.gradNorm - o.gradNorm) <= 3e-2 * o.gradNorm, (s, st.gradNorm, o.gradNorm)
+        if s == 0:
+            for name, g in ograds.items():
+                got, w = ft.grad(name).astype(np.float64), g.astype(np.float64)
+                cos = float(got @ w / (np.linalg.norm(got) * np.linalg.norm(w) + 1e-300))
+                assert cos > 0.995, (name, cos)
+    ft.close()
