@@ -121,6 +121,50 @@ class FastHipBackend(HipBackend):
         super()._dirty(t)
         t._shadow = None
 
+    # ---- data movement on bf16 storage.  The kernels behind slice / transpose / scatter copy 4-byte words and never look
+    # inside them, so a bf16 tensor whose innermost dimension is even and is left whole (or cut at even columns) is moved as
+    # the tensor of half that width: q, k, v and the head transposes of the reference's attention branch (gpt.ts:232-253) stay
+    # in bf16 instead of being widened to f32 first.
+    def sliceQkv(self, a: TensorData):
+        rows, c3 = a.shape
+        d = c3 // 3
+        if a.store != "bf16" or d % 2 or c3 != 3 * d:
+            return super().sliceQkv(a)
+        q, k, v = (self._new((rows, d), "f32", "bf16") for _ in range(3))
+        check(self.lib.ah_slice_qkv(self._ptr(a), q._buf.ptr, k._buf.ptr, v._buf.ptr, rows, d // 2))
+        return [q, k, v]
+
+    def transpose(self, a: TensorData, dim0: int, dim1: int) -> TensorData:
+        nd = len(a.shape)
+        d0, d1 = self._axis(dim0, nd), self._axis(dim1, nd)
+        if a.store != "bf16" or nd < 3 or nd - 1 in (d0, d1) or a.shape[-1] % 2:
+            return super().transpose(a, dim0, dim1)
+        ns = list(a.shape)
+        ns[d0], ns[d1] = a.shape[d1], a.shape[d0]
+        half = list(a.shape)
+        half[-1] //= 2
+        out = self._new(ns, a.dtype, "bf16")
+        check(self.lib.ah_transpose(self._ptr(a), out._buf.ptr, nd, ffi.shape_arr(half), d0, d1))
+        return out
+
+    def slice(self, a: TensorData, starts, ends) -> TensorData:
+        if a.store != "bf16" or not a.shape or a.shape[-1] % 2 or starts[-1] % 2 or ends[-1] % 2:
+            return super().slice(a, starts, ends)
+        halve = lambda xs: list(xs[:-1]) + [xs[-1] // 2]
+        out = self._new([e - s for s, e in zip(starts, ends)], a.dtype, "bf16")
+        check(self.lib.ah_slice(self._ptr(a), out._buf.ptr, len(a.shape), ffi.shape_arr(halve(a.shape)), ffi.shape_arr(halve(starts)),
+                                ffi.shape_arr(halve(ends))))
+        return out
+
+    def scatterSlice(self, grad: TensorData, origShape, starts, ends) -> TensorData:
+        if grad.store != "bf16" or not grad.shape or grad.shape[-1] % 2 or origShape[-1] % 2 or starts[-1] % 2:
+            return super().scatterSlice(grad, origShape, starts, ends)
+        halve = lambda xs: list(xs[:-1]) + [xs[-1] // 2]
+        out = self._new(origShape, grad.dtype, "bf16")
+        check(self.lib.ah_scatter_slice(self._ptr(grad), out._buf.ptr, len(origShape), ffi.shape_arr(halve(grad.shape)),
+                                        ffi.shape_arr(halve(origShape)), ffi.shape_arr(halve(starts))))
+        return out
+
     def _operand(self, t: TensorData):
         """Device address of `t` as a bf16 matrix operand, and the buffer that must outlive the launch."""
         if t.store == "bf16":

@@ -94,6 +94,9 @@ def main():
     ap.add_argument("--no-step-graphs", action="store_true", help="backend mode: issue every launch eagerly")
     ap.add_argument("--dw-groups", type=int, default=1, help="fast mode: weight-gradient GEMMs in this many runs on a second stream")
     ap.add_argument("--stream", choices=["f32", "bf16"], default="bf16", help="fast mode: storage type of the residual stream and its gradient")
+    ap.add_argument("--attention", choices=["heads", "reference-flash", "unfused"], default="heads",
+                    help="backend / parity mode: which attention branch of the model runs (reference-flash = the op sequence of the "
+                         "reference's flash branch, gpt.ts:232-253; unfused = its CPU branch)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--cpu-tokens", type=int, default=32)
     ap.add_argument("--workload", choices=sorted(WORKLOADS), default="gpt2-small")
@@ -108,7 +111,7 @@ def main():
 
     B = FastHipBackend(0) if args.mode == "backend" else HipBackend(0)
     model, BATCH, accum, tok_seed, describe = WORKLOADS[args.workload]
-    cfg = ModelConfig(**model)
+    cfg = ModelConfig(**model, attention=args.attention)
     tc = TrainConfig(iters=50, batchSize=BATCH, gradAccumSteps=accum)
     tokens = BATCH * cfg.blockSize * accum
     # a ring of distinct resident batches: every step trains on the next `accum` of them, so the reported losses are a
@@ -189,7 +192,8 @@ def main():
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": f"synthetic (Zipf s=1.1 token ids, seed {tok_seed}; random-init N(0,0.02) weights, seed 0)",
         "config": {"workload": describe,
-                   "tokens_per_step": tokens, "mode": args.mode, "loss_first_step": loss_first, "loss_last_step": loss_last},
+                   "tokens_per_step": tokens, "mode": args.mode, "loss_first_step": loss_first, "loss_last_step": loss_last,
+                   **({"attention": args.attention} if args.mode != "fast" else {})},
         # model flops per second against the dense bf16 MFMA peak: by the reference's (non-causal) attention count, and with
         # the causal half of the attention products only
         "step_tflops": flops / (ms * 1e-3) / 1e12, "mfu_vs_bf16_dense_peak": flops / (ms * 1e-3) / 1e12 / PEAK["bf16"],

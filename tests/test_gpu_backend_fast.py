@@ -159,3 +159,43 @@ def test_accumulation_and_other_model_variants_still_run_on_the_fast_backend(FB)
             r = tr.step([syntheticBatch(90 + accum * s + m, 4, 64, 256) for m in range(accum)])
             o = orc.step([rm.synthetic_batch(90 + accum * s + m, 4, 64, 256) for m in range(accum)])
             assert abs(r.loss - o.loss) <= 2e-2 * abs(o.loss), (kw, s, r.loss, o.loss)
+
+
+def test_bf16_tensors_move_as_words_and_the_reference_flash_branch_stays_in_bf16(FB):
+    """slice / sliceQkv / transpose / scatterSlice on bf16-stored tensors with an even innermost dimension give exactly what the
+    f32 kernels give on the same values (the copies never look inside a word), and the model with the reference's own flash
+    branch (gpt.ts:232-253: sliceQkv, reshape to [B*H, T, D] without a head transpose, flashAttention, transpose back) trains on
+    the fast backend within the bf16 bar of the same model on the fp32 backend, replayed from a step plan."""
+    from alpha2_amd import HipBackend
+    from alpha2_amd.model import ModelConfig
+    from alpha2_amd.train import TrainConfig, Trainer, syntheticBatch
+    rs = np.random.RandomState(11)
+    x = _bf16(rs.randn(6, 5, 4, 8))
+    t = FB.castStore(_td(x), "bf16")
+    assert np.array_equal(FB.transpose(t, 1, 2).data.reshape(6, 4, 5, 8), x.transpose(0, 2, 1, 3)) and FB.transpose(t, 1, 2).store == "bf16"
+    assert np.array_equal(FB.transpose(t, 0, 2).data.reshape(4, 5, 6, 8), x.transpose(2, 1, 0, 3))
+    assert np.array_equal(FB.transpose(t, 2, 3).data.reshape(6, 5, 8, 4), x.transpose(0, 1, 3, 2))          # touches the last axis: f32 route
+    m = _bf16(rs.randn(10, 24))
+    tm = FB.castStore(_td(m), "bf16")
+    q, k, v = FB.sliceQkv(tm)
+    assert q.store == "bf16" and all(np.array_equal(p.data.reshape(10, 8), m[:, 8 * i:8 * i + 8]) for i, p in enumerate((q, k, v)))
+    sl = FB.slice(tm, [2, 4], [9, 20])
+    assert sl.store == "bf16" and np.array_equal(sl.data.reshape(7, 16), m[2:9, 4:20])
+    assert np.array_equal(FB.slice(tm, [2, 3], [9, 20]).data.reshape(7, 17), m[2:9, 3:20])                    # odd column: f32 route
+    sc = FB.scatterSlice(q, (10, 24), [0, 8], [10, 16])
+    want = np.zeros((10, 24), np.float32); want[:, 8:16] = m[:, :8]
+    assert sc.store == "bf16" and np.array_equal(sc.data.reshape(10, 24), want)
+
+    cfg = dict(CFG, attention="reference-flash")
+    ref_b = HipBackend(0)
+    slow = Trainer(ref_b, ModelConfig(**cfg), TrainConfig(iters=6), seed=4)
+    fast = Trainer(FB, ModelConfig(**cfg), TrainConfig(iters=6), seed=4)
+    want = [slow.step([syntheticBatch(70 + s, 4, 64, 256)]) for s in range(8)]
+    FB.enableStepGraphs(True)
+    before = FB.stepStats()
+    for s, a in enumerate(want):
+        b = fast.step([syntheticBatch(70 + s, 4, 64, 256)])
+        assert math.isfinite(b.loss) and abs(a.loss - b.loss) <= 2e-2 * abs(a.loss), (s, a.loss, b.loss)
+        assert abs(a.gradNorm - b.gradNorm) <= 5e-2 * a.gradNorm, (s, a.gradNorm, b.gradNorm)
+    FB.enableStepGraphs(False)
+    assert FB.stepStats()["replayed"] - before["replayed"] >= 4, (before, FB.stepStats(), FB.stepFallbackNotes)
