@@ -270,6 +270,12 @@ class FastHipBackend(HipBackend):
                 rp = self._ptr(res)
                 self._launch_held(ffi.EPI_RESIDUAL, aux=rp, out=out, out_dtype=F32)
                 return out
+        if a.store == b.store == "bf16" and tuple(a.shape) == tuple(b.shape):        # e.g. the three scattered parts of d(qkv)
+            pa, pb = self._ptr(a), self._ptr(b)
+            if (pa | pb) % 16 == 0:
+                out = self._new(a.shape, "f32", "bf16")
+                check(self.lib.ah_add_bf16(pa, pb, out._buf.ptr, a.size))
+                return out
         return super().add(a, b)
 
     def residualDropoutAdd(self, residual, projected, mask) -> TensorData:
@@ -344,6 +350,17 @@ class FastHipBackend(HipBackend):
                 return
         self._launch_held()
         self._ptr(a), self._ptr(b)                               # launches whatever still has to produce (or add into) them
+        if a.store == b.store == "bf16" and a.size == b.size and a._dev_valid and (self._ptr(a) | self._ptr(b)) % 16 == 0:
+            pa, pb = self._ptr(a), self._ptr(b)
+            if a._buf.refs > 1:                                  # copy-on-write, as below
+                buf = _Buf(self.lib, a.size * 2)
+                check(self.lib.ah_add_bf16(pa, pb, buf.ptr, a.size))
+                a._buf.release()
+                a._buf, a._off = buf, 0
+            else:
+                check(self.lib.ah_add_bf16(pa, pb, pa, a.size))
+            self._dirty(a)
+            return
         if a._buf is not None and a._buf.refs > 1 and a._dev_valid and a.store == "f32" and b.store == "f32":
             # copy-on-write: `a` shares its buffer (clone): the sum goes to a buffer of its own in one pass
             pa, pb = self._ptr(a), self._ptr(b)

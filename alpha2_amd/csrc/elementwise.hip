@@ -312,6 +312,21 @@ __global__ void k_axpy(float *__restrict__ a, const float *__restrict__ b, float
   for (uint64_t i = tid; i < n; i += stride) a[i] += b[i] * s;
 }
 
+// out = a + b on bf16 storage, 8 elements per thread (out may be a or b)
+__global__ void k_add_bf16(const uint16_t *a, const uint16_t *b, uint16_t *out, uint64_t n) {
+  const uint64_t tid = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x, stride = (uint64_t)gridDim.x * blockDim.x, n8 = n >> 3;
+  for (uint64_t i = tid; i < n8; i += stride) {
+    const uint4 x = reinterpret_cast<const uint4 *>(a)[i], y = reinterpret_cast<const uint4 *>(b)[i];
+    const uint32_t xs[4] = {x.x, x.y, x.z, x.w}, ys[4] = {y.x, y.y, y.z, y.w};
+    uint32_t o[4];
+#pragma unroll
+    for (int q = 0; q < 4; q++)
+      o[q] = pack_bf16x2(bf16_bits_to_f32(xs[q] & 0xffffu) + bf16_bits_to_f32(ys[q] & 0xffffu), bf16_bits_to_f32(xs[q] >> 16) + bf16_bits_to_f32(ys[q] >> 16));
+    reinterpret_cast<uint4 *>(out)[i] = make_uint4(o[0], o[1], o[2], o[3]);
+  }
+  for (uint64_t i = (n8 << 3) + tid; i < n; i += stride) out[i] = f32_to_bf16_bits(bf16_bits_to_f32(a[i]) + bf16_bits_to_f32(b[i]));
+}
+
 __global__ void k_silu_mul(const float *__restrict__ a, const float *__restrict__ b, float *__restrict__ out, uint64_t n) {
   uint64_t tid = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x, stride = (uint64_t)gridDim.x * blockDim.x;
   for (uint64_t i = tid; i < n; i += stride) { float x = a[i]; out[i] = x / (1.0f + expf(-x)) * b[i]; }
@@ -466,6 +481,16 @@ int32_t ah_axpy_inplace(ah_ptr a, ah_ptr b, float s, uint64_t n) {
   if (n == 0) return AH_OK;
   AH_ARG(a && b, "ah_axpy_inplace: null operand");
   ah::launch_kernel(k_axpy, dim3(grid_for(n)), dim3(TPB), 0, dp<float>(a), dp<const float>(b), s, n);
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+
+int32_t ah_add_bf16(ah_ptr a, ah_ptr b, ah_ptr out, uint64_t n) {
+  AH_REQUIRE_READY();
+  if (n == 0) return AH_OK;
+  AH_ARG(a && b && out, "ah_add_bf16: null operand");
+  AH_ARG(aligned16(a) && aligned16(b) && aligned16(out), "ah_add_bf16: operands must be 16-byte aligned");
+  ah::launch_kernel(k_add_bf16, dim3(grid_for(n / 8 + 1)), dim3(TPB), 0, dp<const uint16_t>(a), dp<const uint16_t>(b), dp<uint16_t>(out), n);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }

@@ -149,6 +149,9 @@ int32_t ah_unary(int32_t op, ah_ptr x, ah_ptr out, uint64_t n, float p0, float p
 /* in place: Backend.addInplace / scaleInplace (interfaces.ts:113-114) */
 int32_t ah_add_inplace(ah_ptr a, ah_ptr b, uint64_t n);
 int32_t ah_scale_inplace(ah_ptr a, float s, uint64_t n);
+/* out = a + b on bf16 storage, rounded once (Backend.add / addInplace, interfaces.ts:49,113, for tensors a bf16 backend keeps
+ * in bf16: the tape's gradient accumulation, tape.ts:116-127); out may be a or b; 16-byte aligned */
+int32_t ah_add_bf16(ah_ptr a, ah_ptr b, ah_ptr out, uint64_t n);
 /* a[i] += b[i] * s  -- loss accumulation over micro-steps (trainer.ts:1208-1223) without a temporary */
 int32_t ah_axpy_inplace(ah_ptr a, ah_ptr b, float s, uint64_t n);
 

@@ -186,6 +186,17 @@ def test_bf16_tensors_move_as_words_and_the_reference_flash_branch_stays_in_bf16
     want = np.zeros((10, 24), np.float32); want[:, 8:16] = m[:, :8]
     assert sc.store == "bf16" and np.array_equal(sc.data.reshape(10, 24), want)
 
+    # sums of bf16-stored tensors stay in bf16 (one rounding), in place as well, also when the target shares its buffer
+    y = _bf16(rs.randn(10, 24))
+    tm, ty = FB.castStore(_td(m), "bf16"), FB.castStore(_td(y), "bf16")      # (the odd-column slice above widened the old `tm` to f32)
+    s2 = FB.add(tm, ty)
+    assert s2.store == "bf16" and np.array_equal(s2.data.reshape(10, 24), _bf16(m + y))
+    acc = FB.clone(tm)
+    FB.addInplace(acc, ty)
+    assert acc.store == "bf16" and np.array_equal(acc.data.reshape(10, 24), _bf16(m + y)) and np.array_equal(tm.data.reshape(10, 24), m)
+    FB.addInplace(acc, ty)
+    assert np.array_equal(acc.data.reshape(10, 24), _bf16(_bf16(m + y) + y))
+
     cfg = dict(CFG, attention="reference-flash")
     ref_b = HipBackend(0)
     slow = Trainer(ref_b, ModelConfig(**cfg), TrainConfig(iters=6), seed=4)
