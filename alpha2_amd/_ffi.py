@@ -88,6 +88,7 @@ SIGNATURES = {
     "ah_unary_bwd": [i32, u64, u64, u64, u64, f32, f32],
     "ah_channel_act": [i32, u64, C.c_void_p, i32, u64, i64, i64], "ah_channel_act_bwd": [i32, u64, C.c_void_p, i32, u64, u64, C.c_void_p, i32, i64, i64],
     "ah_add_bf16": [u64, u64, u64, u64],
+    "ah_sum_sq_list": [C.c_void_p, C.c_void_p, i32, u64],
     "ah_swiglu": [i32, u64, u64, i64, i64], "ah_swiglu_bwd": [i32, u64, u64, u64, i64, i64],
     "ah_silu_mul": [u64, u64, u64, u64], "ah_silu_mul_bwd": [u64, u64, u64, u64, u64, u64],
     "ah_residual_dropout_add": [u64, u64, u64, u64, u64],

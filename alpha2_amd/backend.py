@@ -855,13 +855,12 @@ class HipBackend:
     def totalSumOfSquares(self, tensors: Sequence[TensorData]) -> TensorData:
         """One scalar for the whole gradient set (packages/train/src/trainer.ts:1345-1349)."""
         total = self._new((1,))
-        check(self.lib.ah_fill_f32(total._buf.ptr, 0.0, 1))
-        part = self._new((1,))
         for t in tensors:
             self._f32(t)
-            check(self.lib.ah_sum_sq(self._ptr(t), t.size, part._buf.ptr))
-            check(self.lib.ah_add_inplace(total._buf.ptr, part._buf.ptr, 1))
-        self.releaseGpuTensor(part)
+        n = len(tensors)
+        xs = (C.c_uint64 * max(n, 1))(*[self._ptr(t) for t in tensors])
+        ns = (C.c_uint64 * max(n, 1))(*[t.size for t in tensors])
+        check(self.lib.ah_sum_sq_list(xs, ns, n, total._buf.ptr))
         return total
 
     def checkFinite(self, data: TensorData) -> TensorData:

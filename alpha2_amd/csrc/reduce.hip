@@ -75,6 +75,40 @@ __global__ void k_partial_sum(const float *__restrict__ a, uint64_t n, double *_
   s = block_sum_d(s, sh);
   if (threadIdx.x == 0) partial[blockIdx.x] = s;
 }
+// stage 1 for a LIST of tensors in one launch: block b sums the squares of one 64 K-element chunk of one tensor (the table is
+// passed by value; a block finds its tensor by bisection of the chunk offsets).  The partition depends on the sizes only.
+constexpr int SL_MAX = 120;
+constexpr uint64_t SL_CHUNK = uint64_t(1) << 16;
+struct SumList {
+  const float *x[SL_MAX];
+  uint64_t n[SL_MAX];
+  uint32_t first[SL_MAX + 1];      // first block of tensor t; first[count] = number of blocks
+  int count;
+};
+__global__ void k_sum_sq_list(SumList L, double *__restrict__ partial) {
+  __shared__ double sh[TPB / 64];
+  const uint32_t b = blockIdx.x;
+  int lo = 0, hi = L.count - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (L.first[mid] <= b) lo = mid; else hi = mid - 1;
+  }
+  const float *a = L.x[lo];
+  const uint64_t n = L.n[lo], c0 = (uint64_t)(b - L.first[lo]) * SL_CHUNK, c1 = c0 + SL_CHUNK < n ? c0 + SL_CHUNK : n;
+  double s = 0;
+  if ((((uintptr_t)a) & 15u) == 0) {                 // chunk starts are multiples of 64 K elements: as aligned as the tensor
+    const uint64_t q0 = c0 >> 2, q1 = c1 >> 2;
+    for (uint64_t i = q0 + threadIdx.x; i < q1; i += blockDim.x) {
+      float4 v = reinterpret_cast<const float4 *>(a)[i];
+      s += (double)v.x * v.x + (double)v.y * v.y + (double)v.z * v.z + (double)v.w * v.w;
+    }
+    for (uint64_t i = (q1 << 2) + threadIdx.x; i < c1; i += blockDim.x) { double v = a[i]; s += v * v; }
+  } else {
+    for (uint64_t i = c0 + threadIdx.x; i < c1; i += blockDim.x) { double v = a[i]; s += v * v; }
+  }
+  s = block_sum_d(s, sh);
+  if (threadIdx.x == 0) partial[b] = s;
+}
 // stage 2: fixed-order sum of the partials by one block
 __global__ void k_final_sum(const double *__restrict__ partial, int nparts, float *__restrict__ out, double div) {
   __shared__ double sh[TPB / 64];
@@ -210,6 +244,45 @@ int32_t ah_sum_all(ah_ptr a, ah_ptr out, uint64_t n, int32_t mean) {
   return full_reduce(a, n, out, mean ? (double)n : 1.0, 0, "ah_sum_all");
 }
 int32_t ah_sum_sq(ah_ptr x, uint64_t n, ah_ptr out) { return full_reduce(x, n, out, 1.0, 1, "ah_sum_sq"); }
+
+int32_t ah_sum_sq_list(const ah_ptr *xs, const uint64_t *ns, int32_t count, ah_ptr out) {
+  AH_REQUIRE_READY();
+  AH_ARG(out != 0, "ah_sum_sq_list: null out");
+  AH_ARG(count >= 0 && (count == 0 || (xs && ns)), "ah_sum_sq_list: bad list");
+  uint64_t blocks = 0;
+  for (int i = 0; i < count; i++) {
+    AH_ARG(ns[i] == 0 || xs[i] != 0, "ah_sum_sq_list: null tensor %d", i);
+    blocks += (ns[i] + SL_CHUNK - 1) / SL_CHUNK;
+  }
+  if (blocks == 0) return ah_fill_f32(out, 0.f, 1);
+  AH_ARG(blocks < (uint64_t(1) << 24), "ah_sum_sq_list: too many elements");
+  double *partial = (double *)scratch(sizeof(double) * (size_t)blocks);
+  if (!partial) return fail(AH_ERR_OOM, "ah_sum_sq_list: no scratch");
+  uint32_t done = 0;
+  int i = 0;
+  while (i < count) {                                // launches of up to SL_MAX non-empty tensors, partial sums side by side
+    SumList L;
+    L.count = 0;
+    uint32_t nb = 0;
+    for (; i < count && L.count < SL_MAX; i++) {
+      if (ns[i] == 0) continue;
+      L.x[L.count] = dp<const float>(xs[i]);
+      L.n[L.count] = ns[i];
+      L.first[L.count] = nb;
+      nb += (uint32_t)((ns[i] + SL_CHUNK - 1) / SL_CHUNK);
+      L.count++;
+    }
+    if (L.count == 0) break;
+    L.first[L.count] = nb;
+    for (int k = L.count; k < SL_MAX; k++) { L.x[k] = nullptr; L.n[k] = 0; L.first[k + 1] = nb; }
+    ah::launch_kernel(k_sum_sq_list, dim3(nb), dim3(TPB), 0, L, partial + done);
+    AH_LAUNCH_CHECK();
+    done += nb;
+  }
+  ah::launch_kernel(k_final_sum, dim3(1), dim3(TPB), 0, (const double *)partial, (int)done, dp<float>(out), 1.0);
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
 
 int32_t ah_sum_sq_static(ah_ptr x, uint64_t n, ah_ptr out) {
   AH_REQUIRE_READY();

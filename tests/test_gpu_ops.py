@@ -320,6 +320,18 @@ def test_reductions_vs_oracle(B):
     assert_close(B.sumOfSquares(dev(B, big)).data, [ref.sum_sq(orc(big))], rel=1e-6)
     parts = [rs.randn(n).astype(np.float32) for n in (1, 7, 4096, 33333)]
     assert_close(B.totalSumOfSquares([dev(B, p) for p in parts]).data, [sum(ref.sum_sq(orc(p)) for p in parts)], rel=1e-6)
+    # one launch for a whole gradient set: more tensors than one launch's table holds, an empty one, tensors of several chunks,
+    # a view that is not 16-byte aligned; the same call twice gives the same bits (fixed partition, fixed order)
+    sizes = [0, 1, 7, 65536, 65537, 200001, 3] + [int(rs.randint(1, 3000)) for _ in range(260)] + [1 << 20]
+    parts = [rs.randn(n).astype(np.float32) for n in sizes]
+    devs = [dev(B, p) for p in parts]
+    odd = dev(B, rs.randn(1001).astype(np.float32))
+    devs.append(B.slice(odd, [1], [1000]))
+    want = sum(float(np.sum(p.astype(np.float64) ** 2)) for p in parts) + float(np.sum(odd.data[1:1000].astype(np.float64) ** 2))
+    got = B.totalSumOfSquares(devs).data
+    assert abs(float(got[0]) - want) <= 1e-6 * want
+    assert np.array_equal(got, B.totalSumOfSquares(devs).data)
+    assert float(B.totalSumOfSquares([]).data[0]) == 0.0
 
 
 def test_softmax_family_vs_oracle(B):
