@@ -63,6 +63,10 @@ class AhAdamW(C.Structure):
                 ("bc1", f32), ("bc2", f32), ("grad_scale", f32)]
 
 
+class AhAdamWItem(C.Structure):
+    _fields_ = [("p", u64), ("g", u64), ("m", u64), ("v", u64), ("shadow", u64), ("n", u64), ("weight_decay", f32), ("reserved", i32)]
+
+
 class AhLion(C.Structure):
     _fields_ = [("lr", C.c_double), ("beta1", C.c_double), ("beta2", C.c_double), ("weight_decay", C.c_double), ("grad_scale", C.c_double)]
 
@@ -89,6 +93,7 @@ SIGNATURES = {
     "ah_channel_act": [i32, u64, C.c_void_p, i32, u64, i64, i64], "ah_channel_act_bwd": [i32, u64, C.c_void_p, i32, u64, u64, C.c_void_p, i32, i64, i64],
     "ah_add_bf16": [u64, u64, u64, u64],
     "ah_sum_sq_list": [C.c_void_p, C.c_void_p, i32, u64],
+    "ah_adamw_list": [C.c_void_p, i32, C.c_void_p, u64, u64],
     "ah_swiglu": [i32, u64, u64, i64, i64], "ah_swiglu_bwd": [i32, u64, u64, u64, i64, i64],
     "ah_silu_mul": [u64, u64, u64, u64], "ah_silu_mul_bwd": [u64, u64, u64, u64, u64, u64],
     "ah_residual_dropout_add": [u64, u64, u64, u64, u64],
@@ -112,7 +117,7 @@ SIGNATURES = {
     "ah_token_windows": [u64, i64, u64, i64, i64, u64, u64],
     "ah_pos_embedding_bwd": [u64, u64, i64, i64, i64, i32],
     "ah_layernorm": [u64, u64, u64, u64, i64, i64, f32, i32, i32],
-    "ah_layernorm_bwd": [u64, u64, u64, i32, u64, u64, u64, u64, u64, i64, i64, f32, i32],
+    "ah_layernorm_bwd": [u64, u64, u64, i32, u64, u64, u64, u64, u64, i64, i64, f32, i32, i32],
     "ah_layernorm_bwd_partials_bytes": [i64, i64],
     "ah_layernorm_bwd_deferred": [u64, u64, u64, i32, u64, u64, u64, u64, i64, i64, f32, i32],
     "ah_layernorm_colsums": [C.POINTER(AhColsumJob), i32],

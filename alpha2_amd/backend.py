@@ -584,7 +584,7 @@ class HipBackend:
         dim = x.shape[-1]
         dx, dw, db = self._new(x.shape), self._new(weight.shape), self._new(weight.shape)
         check(self.lib.ah_layernorm_bwd(self._ptr(x), self._ptr(weight), self._ptr(gradOutput), ffi.F32, 0, dx._buf.ptr, 0, dw._buf.ptr,
-                                        db._buf.ptr, x.size // max(1, dim), dim, eps, 0))
+                                        db._buf.ptr, x.size // max(1, dim), dim, eps, 0, ffi.F32))
         return {"dx": dx, "dw": dw, "db": db}
 
     def softmax(self, a, axis=None) -> TensorData:

@@ -57,14 +57,22 @@ class _HeldWeightGrad:
 class FastHipBackend(HipBackend):
     name = "hip"
 
-    def __init__(self, device: int = 0, group_weight_grads: bool = True):
+    def __init__(self, device: int = 0, group_weight_grads: bool = True, stream_bf16: bool = True):
         super().__init__(device)
+        # the residual stream (the running sum the residual adds produce) and the gradient flowing back along it are stored in
+        # bf16 like every other activation; False keeps both in f32
+        self.streamBf16 = stream_bf16
         self._held: Optional[_HeldGemm] = None
         self._wgrads: List[_HeldWeightGrad] = []
         self._group = group_weight_grads
         self._plans = {}                 # descriptor tuple -> grouped plan id
         # products that became another op's epilogue and were never written themselves: computed only if somebody reads them
         self._orphans = {}               # id(_Buf) -> _HeldGemm
+        # adamwStep calls of one optimizer pass, launched together (one kernel per 48 tensors) when anything needs their result
+        self._adam_q: List[tuple] = []   # (p, g, m, v, shadow, n, weight decay) as device addresses
+        self._adam_key = None
+        self._adam_holds: List[_Buf] = []
+        self._adam_bufs = set()          # id(_Buf) of every buffer a queued update reads or writes
 
     # ------------------------------------------------------------------ storage helpers
     def _hold(self, *bufs):
@@ -86,6 +94,8 @@ class FastHipBackend(HipBackend):
     def _ptr(self, t: TensorData) -> int:
         if not t._dev_valid and t._buf is not None:
             t._shadow = None                                    # the host wrote new contents: the bf16 shadow is stale
+        if self._adam_q and t._buf is not None and id(t._buf) in self._adam_bufs:
+            self._flush_adam()
         if t._buf is not None:
             if self._held is not None and t._buf is self._held.out_buf:
                 self._launch_held()
@@ -99,6 +109,9 @@ class FastHipBackend(HipBackend):
 
     def _download(self, t: TensorData):
         self._ptr(t)
+        # the host is about to wait for the device: whatever is queued and will be needed anyway (the weight gradients once
+        # backward has been issued) goes out first, so the device has work while the host reads and carries on
+        self._launch_weight_grads()
         return super()._download(t)
 
     def _f32(self, *ts):
@@ -180,6 +193,8 @@ class FastHipBackend(HipBackend):
     def releaseGpuTensor(self, t: TensorData):
         if t is None or t._buf is None:
             return
+        if self._adam_q and id(t._buf) in self._adam_bufs:
+            self._flush_adam()
         sh = getattr(t, "_shadow", None)
         if sh is not None:
             sh.release()
@@ -265,11 +280,20 @@ class FastHipBackend(HipBackend):
 
     def add(self, a: TensorData, b: TensorData) -> TensorData:
         for res, prod in ((a, b), (b, a)):
-            if self._is_held(prod) and res.store == "f32" and tuple(res.shape) == tuple(prod.shape) and res.dtype == "f32" and not self._is_held(res):
-                out = self._new(res.shape)
-                rp = self._ptr(res)
-                self._launch_held(ffi.EPI_RESIDUAL, aux=rp, out=out, out_dtype=F32)
-                return out
+            if self._is_held(prod) and res.store in ("f32", "bf16") and tuple(res.shape) == tuple(prod.shape) and res.dtype == "f32" \
+                    and not self._is_held(res):
+                if self.streamBf16 and res.size % 8 == 0:
+                    # the residual stream in bf16, like every other activation: the sum is rounded once, to bf16
+                    rp, keep = self._operand(res)
+                    out = self._new(res.shape, "f32", "bf16")
+                    self._launch_held(ffi.EPI_RESIDUAL, aux=rp, out=out, out_dtype=BF16)
+                    del keep
+                    return out
+                if res.store == "f32":
+                    out = self._new(res.shape)
+                    rp = self._ptr(res)
+                    self._launch_held(ffi.EPI_RESIDUAL, aux=rp, out=out, out_dtype=F32)
+                    return out
         if a.store == b.store == "bf16" and tuple(a.shape) == tuple(b.shape):        # e.g. the three scattered parts of d(qkv)
             pa, pb = self._ptr(a), self._ptr(b)
             if (pa | pb) % 16 == 0:
@@ -394,24 +418,40 @@ class FastHipBackend(HipBackend):
         return self._view(a, a.shape)
 
     # ------------------------------------------------------------------ nn with bf16 storage
+    def _ln_bf16_ok(self, x: TensorData) -> bool:
+        dim = x.shape[-1] if x.shape else 0
+        return x.store == "bf16" and dim % 4 == 0 and 0 < dim <= 2048
+
     def layerNorm(self, x, weight, bias, eps) -> TensorData:
-        if x.store != "f32":
+        if x.store == "bf16" and not self._ln_bf16_ok(x):
+            self._f32(x)
+        if x.store not in ("f32", "bf16"):
             return super().layerNorm(x, weight, bias, eps)
         dim = x.shape[-1]
         if weight.size != dim or bias.size != dim:
             raise ValueError("layerNorm: weight/bias length must equal the last dimension")
         out = self._new(x.shape, "f32", "bf16")
-        check(self.lib.ah_layernorm(self._ptr(x), self._ptr(weight), self._ptr(bias), out._buf.ptr, x.size // max(1, dim), dim, eps, BF16, ffi.F32))
+        check(self.lib.ah_layernorm(self._ptr(x), self._ptr(weight), self._ptr(bias), out._buf.ptr, x.size // max(1, dim), dim, eps, BF16,
+                                    ffi.DTYPE_CODE[x.store]))
         return out
 
     def layerNormBackward(self, x, weight, gradOutput, eps) -> dict:
+        dim = x.shape[-1]
+        rows = x.size // max(1, dim)
+        if self._ln_bf16_ok(x) and rows > 0:
+            # the residual stream is kept in bf16: its gradient, which the tape adds dx to, is kept in bf16 as well
+            if gradOutput.store != "bf16":
+                gradOutput = self.castStore(gradOutput, "bf16")
+            gp = self._ptr(gradOutput)
+            dx, dw, db = self._new(x.shape, "f32", "bf16"), self._new(weight.shape), self._new(weight.shape)
+            check(self.lib.ah_layernorm_bwd(self._ptr(x), self._ptr(weight), gp, BF16, 0, 0, dx._buf.ptr, dw._buf.ptr, db._buf.ptr, rows, dim, eps, 0, BF16))
+            return {"dx": dx, "dw": dw, "db": db}
         if x.store != "f32":
             return super().layerNormBackward(x, weight, gradOutput, eps)
-        dim = x.shape[-1]
         gp = self._ptr(gradOutput)
         dx, dw, db = self._new(x.shape), self._new(weight.shape), self._new(weight.shape)
         check(self.lib.ah_layernorm_bwd(self._ptr(x), self._ptr(weight), gp, ffi.DTYPE_CODE[gradOutput.store], 0, dx._buf.ptr, 0, dw._buf.ptr,
-                                        db._buf.ptr, x.size // max(1, dim), dim, eps, 0))
+                                        db._buf.ptr, rows, dim, eps, 0, ffi.F32))
         return {"dx": dx, "dw": dw, "db": db}
 
     def crossEntropy(self, logits: TensorData, targets: TensorData) -> TensorData:
@@ -454,18 +494,43 @@ class FastHipBackend(HipBackend):
         return super().totalSumOfSquares(tensors)
 
     def adamwStep(self, params, grads, m, v, lr, beta1, beta2, eps, weightDecay, bc1, bc2, gradScale=1.0):
+        """Queued: the optimizer calls this once per parameter tensor with the same scalars (optimizers.ts:54-94); the updates of
+        a pass are launched together when the first of their tensors is read, written or released."""
         self._launch_held()
         self._f32(params, grads, m, v)
         if not (params.size == grads.size == m.size == v.size):
             raise ValueError("adamwStep: params, grads, m, v must have the same size")
+        key = (lr, beta1, beta2, eps, bc1, bc2, gradScale)
+        if self._adam_q and key != self._adam_key:
+            self._flush_adam()
         for t in (params, m, v):
             self._own(t)
-        pp = self._ptr(params)
+        ptrs = [self._ptr(t) for t in (params, grads, m, v)]    # (launches whatever still has to produce the gradient)
+        if not self._adam_q:
+            self._adam_key = key
+            self._adam_hyper(lr, beta1, beta2, eps, 0.0, bc1, bc2, gradScale)      # the device copy of the scalars, once per pass
         sh = getattr(params, "_shadow", None)
-        h, dev = self._adam_hyper(lr, beta1, beta2, eps, weightDecay, bc1, bc2, gradScale)
-        check(self.lib.ah_adamw(pp, self._ptr(grads), self._ptr(m), self._ptr(v), params.size, C.byref(h), dev, 0, sh.ptr if sh is not None else 0))
+        self._adam_q.append((*ptrs, sh.ptr if sh is not None else 0, params.size, weightDecay))
+        for b in (params._buf, grads._buf, m._buf, v._buf) + ((sh,) if sh is not None else ()):
+            b.refs += 1
+            self._adam_holds.append(b)
+            self._adam_bufs.add(id(b))
         for t in (params, m, v):
-            HipBackend._dirty(self, t)                          # host copies are stale; the shadow was refreshed by the kernel
+            HipBackend._dirty(self, t)                          # host copies are stale; the shadow is refreshed by the kernel
+        if len(self._adam_q) >= 16:                             # the device is usually idle here (the norm was just read back):
+            self._flush_adam()                                  # give it the first tensors while the host queues the rest
+
+    def _flush_adam(self):
+        q, self._adam_q = self._adam_q, []
+        if not q:
+            return
+        holds, self._adam_holds, self._adam_bufs = self._adam_holds, [], set()
+        lr, beta1, beta2, eps, bc1, bc2, gradScale = self._adam_key
+        h, dev = self._adam_hyper(lr, beta1, beta2, eps, 0.0, bc1, bc2, gradScale)
+        items = (ffi.AhAdamWItem * len(q))(*[ffi.AhAdamWItem(p, g, m, v, sh, n, wd, 0) for p, g, m, v, sh, n, wd in q])
+        check(self.lib.ah_adamw_list(items, len(q), C.byref(h), dev, 0))
+        for b in holds:
+            b.release()
 
     def lionStep(self, params, grads, m, *a, **kw):
         self._own(params), self._own(m)
@@ -486,9 +551,11 @@ class FastHipBackend(HipBackend):
     def flush(self):
         self._launch_held()
         self._launch_weight_grads()
+        self._flush_adam()
         super().flush()
 
     def syncGpu(self):
         self._launch_held()
         self._launch_weight_grads()
+        self._flush_adam()
         super().syncGpu()

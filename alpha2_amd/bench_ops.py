@@ -172,7 +172,7 @@ def bench_bandwidth(b: Bench):
     out16, dx, dx16, dw, db = b.alloc(rows * dim * 2), b.alloc(rows * dim * 4), b.alloc(rows * dim * 2), b.alloc(dim * 4), b.alloc(dim * 4)
     ms = b.time(lambda: ffi.check(lib.ah_layernorm(x, w, bias, out16, rows, dim, 1e-5, ffi.BF16, ffi.F32)))
     b.record("layernorm fwd 16384x768", ms, nbytes=rows * dim * 6, note="f32 in, bf16 out")
-    ms = b.time(lambda: ffi.check(lib.ah_layernorm_bwd(x, w, g16, ffi.BF16, res, dx, dx16, dw, db, rows, dim, 1e-5, 0)))
+    ms = b.time(lambda: ffi.check(lib.ah_layernorm_bwd(x, w, g16, ffi.BF16, res, dx, dx16, dw, db, rows, dim, 1e-5, 0, ffi.F32)))
     b.record("layernorm bwd 16384x768", ms, nbytes=rows * dim * 16, note="x f32, g bf16, + residual grad f32 -> dx f32 + bf16; dw, db")
     x16, res16 = b.randn(rows * dim, ffi.BF16, 1.0, 11), b.randn(rows * dim, ffi.BF16, 1.0, 12)
     part = b.alloc(int(lib.ah_layernorm_bwd_partials_bytes(rows, dim)))

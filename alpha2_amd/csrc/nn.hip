@@ -931,7 +931,7 @@ static int32_t ln_bwd_launch(ah_ptr x, ah_ptr w, ah_ptr grad_out, int32_t grad_d
   bool vec = dim % 4 == 0 && dim <= 2048 && x % sa == 0 && aligned16(w) && aligned16(dx) && (grad_out % 8 == 0) && (residual_grad % sa == 0) &&
              (dx_bf16 % 8 == 0) && (grad_dtype == AH_BF16 || aligned16(grad_out));
   if (stream_dtype == AH_BF16)
-    AH_ARG(vec && grad_dtype == AH_BF16 && dx_bf16, "ah_layernorm_bwd_deferred: a bf16 stream needs bf16 gradients, a bf16 dx and rows of 4 k <= 2048 aligned elements");
+    AH_ARG(vec && grad_dtype == AH_BF16 && dx_bf16, "ah_layernorm_bwd: a bf16 stream needs bf16 gradients, a bf16 dx and rows of 4 k <= 2048 aligned elements");
   else
     AH_ARG(dx != 0, "ah_layernorm_bwd: null dx");
   if (vec) {
@@ -955,21 +955,22 @@ static int32_t ln_bwd_launch(ah_ptr x, ah_ptr w, ah_ptr grad_out, int32_t grad_d
 }
 
 int32_t ah_layernorm_bwd(ah_ptr x, ah_ptr w, ah_ptr grad_out, int32_t grad_dtype, ah_ptr residual_grad, ah_ptr dx, ah_ptr dx_bf16,
-                         ah_ptr dw, ah_ptr db, int64_t rows, int64_t dim, float eps, int32_t accumulate) {
+                         ah_ptr dw, ah_ptr db, int64_t rows, int64_t dim, float eps, int32_t accumulate, int32_t stream_dtype) {
   AH_REQUIRE_READY();
   AH_ARG(grad_dtype == AH_F32 || grad_dtype == AH_BF16, "ah_layernorm_bwd: grad dtype must be f32 or bf16");
+  AH_ARG(stream_dtype == AH_F32 || stream_dtype == AH_BF16, "ah_layernorm_bwd: stream dtype must be f32 or bf16");
   if (dim == 0) return AH_OK;
   AH_ARG(dw && db, "ah_layernorm_bwd: null dw/db");
   if (rows == 0) {
     if (!accumulate) { int32_t rc = ah_fill_f32(dw, 0.f, (uint64_t)dim); if (rc) return rc; return ah_fill_f32(db, 0.f, (uint64_t)dim); }
     return AH_OK;
   }
-  AH_ARG(x && w && grad_out && dx, "ah_layernorm_bwd: null operand");
+  AH_ARG(x && w && grad_out && (dx || stream_dtype == AH_BF16), "ah_layernorm_bwd: null operand");
   AH_ARG(sizeof(float) * 2 * WPB * (size_t)dim <= 160 * 1024, "ah_layernorm_bwd: dim %lld too large for the LDS column accumulators", (long long)dim);
   const int nblk = ln_bwd_blocks(rows);
   float *part = (float *)scratch(sizeof(float) * 2 * (size_t)nblk * (size_t)dim);
   if (!part) return fail(AH_ERR_OOM, "ah_layernorm_bwd: no scratch");
-  int32_t rc = ln_bwd_launch(x, w, grad_out, grad_dtype, residual_grad, dx, dx_bf16, part, nblk, rows, dim, eps);
+  int32_t rc = ln_bwd_launch(x, w, grad_out, grad_dtype, residual_grad, dx, dx_bf16, part, nblk, rows, dim, eps, stream_dtype);
   if (rc) return rc;
   ah::launch_kernel(k_colsum_partials, dim3((unsigned)cdiv(dim, 32)), dim3(1024), 0, part, part + (size_t)nblk * dim, nblk, (int)dim,
                      dp<float>(dw), dp<float>(db), accumulate);

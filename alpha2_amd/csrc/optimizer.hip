@@ -57,6 +57,64 @@ __global__ void k_adamw(float *__restrict__ p, const float *__restrict__ g, floa
   }
 }
 
+// The same update for a LIST of tensors in one launch (the table is passed by value): block b works on one chunk of
+// AL_CHUNK elements of one tensor, found by bisection of the chunk offsets.  Element arithmetic = k_adamw's.
+constexpr int AL_MAX = 48;
+constexpr uint64_t AL_CHUNK = uint64_t(1) << 14;
+struct AdamList {
+  float *p[AL_MAX];
+  const float *g[AL_MAX];
+  float *m[AL_MAX], *v[AL_MAX];
+  uint16_t *shadow[AL_MAX];
+  uint64_t n[AL_MAX];
+  float wd[AL_MAX];
+  uint32_t first[AL_MAX + 1];
+  int count;
+};
+__global__ __launch_bounds__(TPB) void k_adamw_list(AdamList L, AhAdamW h, const AhAdamW *__restrict__ dev_h, const float *__restrict__ dev_scale) {
+  const uint32_t b = blockIdx.x;
+  int lo = 0, hi = L.count - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (L.first[mid] <= b) lo = mid; else hi = mid - 1;
+  }
+  if (dev_h) h = *dev_h;
+  h.weight_decay = L.wd[lo];
+  const float gs = h.grad_scale * (dev_scale ? dev_scale[0] : 1.0f);
+  if (!(fabsf(gs) <= 3.4028234e38f)) return;                      // "skip this step", as in k_adamw
+  float *p = L.p[lo], *m = L.m[lo], *v = L.v[lo];
+  const float *g = L.g[lo];
+  uint16_t *shadow = L.shadow[lo];
+  const uint64_t n = L.n[lo], c0 = (uint64_t)(b - L.first[lo]) * AL_CHUNK, c1 = c0 + AL_CHUNK < n ? c0 + AL_CHUNK : n;
+  uint64_t start = c0;
+  if (((((uintptr_t)p | (uintptr_t)g | (uintptr_t)m | (uintptr_t)v) & 15u) | ((uintptr_t)shadow & 7u)) == 0) {
+    const uint64_t q0 = c0 >> 2, q1 = c1 >> 2;
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    typedef unsigned u2 __attribute__((ext_vector_type(2)));
+    for (uint64_t i = q0 + threadIdx.x; i < q1; i += TPB) {
+      f4 pp = __builtin_nontemporal_load(reinterpret_cast<f4 *>(p) + i), gg = __builtin_nontemporal_load(reinterpret_cast<const f4 *>(g) + i);
+      f4 mm = __builtin_nontemporal_load(reinterpret_cast<f4 *>(m) + i), vv = __builtin_nontemporal_load(reinterpret_cast<f4 *>(v) + i);
+      float pa[4] = {pp.x, pp.y, pp.z, pp.w}, ma[4] = {mm.x, mm.y, mm.z, mm.w}, va[4] = {vv.x, vv.y, vv.z, vv.w};
+      adam_one(pa[0], gg.x, ma[0], va[0], h, gs); adam_one(pa[1], gg.y, ma[1], va[1], h, gs);
+      adam_one(pa[2], gg.z, ma[2], va[2], h, gs); adam_one(pa[3], gg.w, ma[3], va[3], h, gs);
+      pp = f4{pa[0], pa[1], pa[2], pa[3]}; mm = f4{ma[0], ma[1], ma[2], ma[3]}; vv = f4{va[0], va[1], va[2], va[3]};
+      __builtin_nontemporal_store(pp, reinterpret_cast<f4 *>(p) + i); __builtin_nontemporal_store(mm, reinterpret_cast<f4 *>(m) + i);
+      __builtin_nontemporal_store(vv, reinterpret_cast<f4 *>(v) + i);
+      if (shadow) {
+        u2 s; s.x = pack_bf16x2(pp.x, pp.y); s.y = pack_bf16x2(pp.z, pp.w);
+        __builtin_nontemporal_store(s, reinterpret_cast<u2 *>(shadow) + i);
+      }
+    }
+    start = q1 << 2;
+  }
+  for (uint64_t i = start + threadIdx.x; i < c1; i += TPB) {
+    float pp = p[i], mm = m[i], vv = v[i];
+    adam_one(pp, g[i], mm, vv, h, gs);
+    p[i] = pp; m[i] = mm; v[i] = vv;
+    if (shadow) shadow[i] = f32_to_bf16_bits(pp);
+  }
+}
+
 __global__ void k_clip_coef(const float *__restrict__ sumsq, float grad_scale, float clip, float *__restrict__ out) {
   if (threadIdx.x == 0 && blockIdx.x == 0) {
     float norm = sqrtf(sumsq[0]) * fabsf(grad_scale);
@@ -283,6 +341,39 @@ int32_t ah_adamw(ah_ptr p, ah_ptr g, ah_ptr m, ah_ptr v, uint64_t n, const AhAda
   ah::launch_kernel(k_adamw, dim3((unsigned)blocks), dim3(TPB), 0, dp<float>(p), dp<const float>(g), dp<float>(m),
                      dp<float>(v), n, *h, dp<const AhAdamW>(dev_hyper), dp<const float>(dev_scale), dp<uint16_t>(bf16_shadow), vec);
   AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+
+int32_t ah_adamw_list(const AhAdamWItem *items, int32_t count, const AhAdamW *h, ah_ptr dev_hyper, ah_ptr dev_scale) {
+  AH_REQUIRE_READY();
+  AH_ARG(h != nullptr, "ah_adamw_list: null hyper-parameters");
+  AH_ARG(count >= 0 && (count == 0 || items != nullptr), "ah_adamw_list: bad list");
+  for (int i = 0; i < count; i++)
+    AH_ARG(items[i].n == 0 || (items[i].p && items[i].g && items[i].m && items[i].v), "ah_adamw_list: null operand in item %d", i);
+  int i = 0;
+  while (i < count) {
+    AdamList L;
+    L.count = 0;
+    uint64_t nb = 0;
+    for (; i < count && L.count < AL_MAX; i++) {
+      const AhAdamWItem &it = items[i];
+      if (it.n == 0) continue;
+      const int k = L.count++;
+      L.p[k] = dp<float>(it.p); L.g[k] = dp<const float>(it.g); L.m[k] = dp<float>(it.m); L.v[k] = dp<float>(it.v);
+      L.shadow[k] = dp<uint16_t>(it.shadow); L.n[k] = it.n; L.wd[k] = it.weight_decay;
+      L.first[k] = (uint32_t)nb;
+      nb += (it.n + AL_CHUNK - 1) / AL_CHUNK;
+    }
+    if (L.count == 0) break;
+    AH_ARG(nb < (uint64_t(1) << 31), "ah_adamw_list: too many elements in one launch");
+    L.first[L.count] = (uint32_t)nb;
+    for (int k = L.count; k < AL_MAX; k++) {
+      L.p[k] = nullptr; L.g[k] = nullptr; L.m[k] = nullptr; L.v[k] = nullptr; L.shadow[k] = nullptr; L.n[k] = 0; L.wd[k] = 0.f;
+      L.first[k + 1] = (uint32_t)nb;
+    }
+    ah::launch_kernel(k_adamw_list, dim3((unsigned)nb), dim3(TPB), 0, L, *h, dp<const AhAdamW>(dev_hyper), dp<const float>(dev_scale));
+    AH_LAUNCH_CHECK();
+  }
   return AH_OK;
 }
 

@@ -60,6 +60,7 @@ struct Context {
   hipStream_t side = nullptr, cur = nullptr;      // side stream for ah_side_begin .. ah_side_end; cur = where launches go now
   hipEvent_t side_ev[2] = {nullptr, nullptr};     // main -> side ("start after this"), side -> main ("wait for the side work")
   bool side_used = false;
+  unsigned chunks_since_host_boundary = 0;        // step plans, RECORD: how many size-limited segments since the host last needed the stream
   hipDeviceProp_t prop;
   char err[512] = "";
   // allocator
@@ -251,7 +252,14 @@ void launch_raw(const void *func, dim3 grid, dim3 block, unsigned shmem, void **
     if (hipStreamGetCaptureInfo_v2(g.stream, &st, nullptr, nullptr, &deps, &ndeps) == hipSuccess &&
         st == hipStreamCaptureStatusActive && ndeps == 1) o.node = deps[0];
     else g.plan->broken = true;            // cannot name the node: this plan will not be replayed
-    if (sg.ops.size() >= step_chunk() && step_boundary("chunk") == AH_OK) (void)step_begin_capture();
+    // After a boundary the host made, the device is idle until the first chunk has been issued: chunks start small there
+    // (4, 8, 16, ... launches) and grow to the full size.
+    static const bool no_ramp = [] { const char *e = getenv("AH_STEP_RAMP"); return e && e[0] == '0'; }();
+    const size_t ramp = (!no_ramp && g.chunks_since_host_boundary < 3) ? (size_t(4) << g.chunks_since_host_boundary) : step_chunk();
+    if (sg.ops.size() >= (ramp < step_chunk() ? ramp : step_chunk()) && step_boundary("chunk") == AH_OK) {
+      g.chunks_since_host_boundary++;
+      (void)step_begin_capture();
+    }
     return;
   }
   // STEP_VERIFY
@@ -297,6 +305,7 @@ int32_t step_boundary(const char *what) {
   if (g.step_mode == STEP_RECORD) {
     if (g.plan->segs.back().ops.empty() && strcmp(what, "ah_step_end") != 0) {
       // nothing recorded since the last boundary: the host may touch the stream without a segment of its own
+      g.chunks_since_host_boundary = 0;
       if (g.step_capture_open) {
         g.step_capture_open = false;
         hipGraph_t junk = nullptr;
@@ -308,6 +317,7 @@ int32_t step_boundary(const char *what) {
     int32_t rc = step_close_segment(what);
     if (rc != AH_OK) { g.plan->broken = true; return rc; }
     g.plan->segs.emplace_back();
+    if (strcmp(what, "chunk") != 0) g.chunks_since_host_boundary = 0;
     return AH_OK;
   }
   StepSeg &sg = g.plan->segs[g.seg];
@@ -706,6 +716,7 @@ int32_t ah_step_begin(uint64_t key) {
   plan_destroy(pl);
   pl.segs.emplace_back();
   g.step_mode = STEP_RECORD;
+  g.chunks_since_host_boundary = 0;
   int32_t rc = step_begin_capture();
   if (rc != AH_OK) { g.step_mode = STEP_OFF; g.plans.erase(key); g.plan = nullptr; }
   return rc;

@@ -267,10 +267,12 @@ int32_t ah_layernorm(ah_ptr x, ah_ptr w, ah_ptr b, ah_ptr out, int64_t rows, int
                      int32_t out_dtype, int32_t x_dtype);
 /* dx (+= residual_grad when that handle is non-zero), dw, db.  dw/db are deterministic column sums;
  * accumulate != 0 adds them into existing dw/db (gradient accumulation). grad_out dtype f32 or bf16.
- * dx_bf16 (0 = none) also receives dx rounded to bf16, the operand of the next backward GEMMs. */
+ * dx_bf16 (0 = none) also receives dx rounded to bf16, the operand of the next backward GEMMs.
+ * stream_dtype = the type of x and residual_grad: AH_F32, or AH_BF16 for a residual stream kept in bf16 (then grad_out is
+ * bf16, dim % 4 == 0, dim <= 2048, dx_bf16 is required and dx may be 0). */
 int32_t ah_layernorm_bwd(ah_ptr x, ah_ptr w, ah_ptr grad_out, int32_t grad_dtype, ah_ptr residual_grad,
                          ah_ptr dx, ah_ptr dx_bf16, ah_ptr dw, ah_ptr db, int64_t rows, int64_t dim, float eps,
-                         int32_t accumulate);
+                         int32_t accumulate, int32_t stream_dtype);
 /* The same with the column sums put off: the per-block partial sums of dw and db go to `partials` (caller-owned, at
  * least ah_layernorm_bwd_partials_bytes(rows, dim) bytes, which is 0 before ah_init), and ONE later call of
  * ah_layernorm_colsums reduces those of many LayerNorms (the 2 L + 1 of a model's backward pass) in one launch instead of
@@ -386,6 +388,10 @@ typedef struct {
  * (grad_scale x dev_scale[0]) is not finite the call changes nothing (see ah_step_guard). */
 int32_t ah_adamw(ah_ptr p, ah_ptr g, ah_ptr m, ah_ptr v, uint64_t n, const AhAdamW *h, ah_ptr dev_hyper,
                  ah_ptr dev_scale, ah_ptr bf16_shadow);
+/* The same update for a list of tensors in one launch per 48 of them: what AdamW.stepParamEntries (optimizers.ts:54-94) does
+ * tensor by tensor.  h, dev_hyper and dev_scale as for ah_adamw; the weight decay is per item (the no-decay set). */
+typedef struct { ah_ptr p, g, m, v, shadow; uint64_t n; float weight_decay; int32_t reserved; } AhAdamWItem;
+int32_t ah_adamw_list(const AhAdamWItem *items, int32_t count, const AhAdamW *h, ah_ptr dev_hyper, ah_ptr dev_scale);
 /* out[0] = clip / (sqrt(sumsq[0]) * |grad_scale|) if that norm exceeds clip, else 1  (trainer.ts:1650-1656);
  * out[1] = the norm itself. */
 int32_t ah_clip_coef(ah_ptr sumsq, float grad_scale, float clip, ah_ptr out2);

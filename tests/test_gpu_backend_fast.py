@@ -64,9 +64,15 @@ def test_held_back_products_and_their_epilogues(FB):
     prod = FB.matmulTransposed(_td(x), _td(w))
     view = FB.reshape(prod, (2, M // 2, N))
     y = FB.add(_td(res.reshape(2, M // 2, N)), view)
-    assert y.store == "f32"
-    _close(y.data, res.reshape(-1) + pre.reshape(-1), "residual epilogue")
+    assert y.store == "bf16"                                   # the residual stream is a bf16 activation by default ...
+    _close(y.data, _bf16(res).reshape(-1) + pre.reshape(-1), "residual epilogue")
     _close(prod.data, pre, "the product itself, computed only now because somebody asked")
+    FB.streamBf16 = False                                      # ... and f32 on request
+    prod = FB.matmulTransposed(_td(x), _td(w))
+    y = FB.add(_td(res), prod)
+    FB.streamBf16 = True
+    assert y.store == "f32"
+    _close(y.data, res.reshape(-1) + pre.reshape(-1), "residual epilogue, f32 stream")
     # geluBackward(pre, matmul(g, w2))
     w2 = rs.randn(N, K) * 0.1                 # [N, K]: g [M, N] @ w2 -> [M, K]
     pre2 = FB.matmulTransposed(_td(x), _td(rs.randn(K, K) * 0.1))

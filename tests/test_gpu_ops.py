@@ -570,7 +570,7 @@ def test_layernorm_backward_with_column_sums_put_off(B):
         assert nbytes >= 8 * dim
         part = B.zeros((nbytes // 4,))
         keep += [xd, wd, gd, dx_, dw_, db_, dx2, dw2, db2, part]
-        ffi.check(lib.ah_layernorm_bwd(B._ptr(xd), B._ptr(wd), B._ptr(gd), ffi.F32, 0, B._ptr(dx_), 0, B._ptr(dw_), B._ptr(db_), rows, dim, 1e-5, 1))
+        ffi.check(lib.ah_layernorm_bwd(B._ptr(xd), B._ptr(wd), B._ptr(gd), ffi.F32, 0, B._ptr(dx_), 0, B._ptr(dw_), B._ptr(db_), rows, dim, 1e-5, 1, ffi.F32))
         ffi.check(lib.ah_layernorm_bwd_deferred(B._ptr(xd), B._ptr(wd), B._ptr(gd), ffi.F32, 0, B._ptr(dx2), 0, B._ptr(part), rows, dim, 1e-5, ffi.F32))
         jobs.append(ffi.AhColsumJob(B._ptr(part), B._ptr(dw2), B._ptr(db2), rows, dim, 1, 0))
         wants.append((dx_, dw_, db_, dx2, dw2, db2))
