@@ -54,6 +54,17 @@ class _HeldWeightGrad:
         self.into = None                  # (buffer, offset) of an existing gradient to accumulate into instead
 
 
+class _HeldLayerNormBwd:
+    """A layerNormBackward that has been asked for and not launched yet.  The tape's next call usually adds its dx to the gradient
+    already flowing along the residual stream (tape.ts:116-127): that gradient then becomes the kernel's own residual input
+    and the sum costs no pass of its own."""
+
+    def __init__(self, x_ptr, w_ptr, g_ptr, dx, dw, db, rows, dim, eps, holds):
+        self.x_ptr, self.w_ptr, self.g_ptr = x_ptr, w_ptr, g_ptr
+        self.outs = (dx._buf, dw._buf, db._buf)
+        self.rows, self.dim, self.eps, self.holds = rows, dim, eps, holds
+
+
 class FastHipBackend(HipBackend):
     name = "hip"
 
@@ -73,6 +84,9 @@ class FastHipBackend(HipBackend):
         self._adam_key = None
         self._adam_holds: List[_Buf] = []
         self._adam_bufs = set()          # id(_Buf) of every buffer a queued update reads or writes
+        self._held_ln: Optional[_HeldLayerNormBwd] = None
+        # dx tensors whose LayerNorm backward went straight into a sum and that were never written themselves: id(_Buf) -> recipe
+        self._ln_unwritten = {}
 
     # ------------------------------------------------------------------ storage helpers
     def _hold(self, *bufs):
@@ -97,6 +111,15 @@ class FastHipBackend(HipBackend):
         if self._adam_q and t._buf is not None and id(t._buf) in self._adam_bufs:
             self._flush_adam()
         if t._buf is not None:
+            if self._held_ln is not None and any(t._buf is b for b in self._held_ln.holds):
+                self._launch_ln()
+            elif self._ln_unwritten and id(t._buf) in self._ln_unwritten:
+                h = self._ln_unwritten.pop(id(t._buf))           # somebody reads the dx that only ever existed inside a sum
+                scratch = _Buf(self.lib, 8 * h.dim)
+                check(self.lib.ah_layernorm_bwd(h.x_ptr, h.w_ptr, h.g_ptr, BF16, 0, 0, h.outs[0].ptr, scratch.ptr, scratch.ptr + 4 * h.dim,
+                                                h.rows, h.dim, h.eps, 0, BF16))
+                scratch.release()
+                self._unhold(h.holds)
             if self._held is not None and t._buf is self._held.out_buf:
                 self._launch_held()
             elif self._wgrads and (self._is_queued(t._buf) or any(w.into is not None and w.into[0] is t._buf for w in self._wgrads)):
@@ -207,6 +230,8 @@ class FastHipBackend(HipBackend):
                 self._unhold(h.holds)
             elif self._orphans and id(buf) in self._orphans:
                 self._unhold(self._orphans.pop(id(buf)).holds)
+            elif self._ln_unwritten and id(buf) in self._ln_unwritten:
+                self._unhold(self._ln_unwritten.pop(id(buf)).holds)
             elif self._wgrads:
                 for i, w in enumerate(self._wgrads):
                     if buf is w.out_buf and w.into is None:
@@ -372,6 +397,18 @@ class FastHipBackend(HipBackend):
                 w.holds.append(a._buf)
                 self._dirty(a)
                 return
+        h = self._held_ln
+        if h is not None and b._buf is h.outs[0] and b._off == 0 and b.size == h.rows * h.dim and a.store == "bf16" and a.size == b.size \
+                and a._buf is not None and a._dev_valid and not any(a._buf is x for x in h.holds):
+            self._launch_held()
+            pa = self._ptr(a)
+            if self._held_ln is h and pa % 16 == 0:
+                buf = _Buf(self.lib, a.size * 2)                 # (never in place: `a` usually shares its buffer with a clone)
+                self._launch_ln(residual=pa, dx_ptr=buf.ptr)
+                a._buf.release()
+                a._buf, a._off = buf, 0
+                self._dirty(a)
+                return
         self._launch_held()
         self._ptr(a), self._ptr(b)                               # launches whatever still has to produce (or add into) them
         if a.store == b.store == "bf16" and a.size == b.size and a._dev_valid and (self._ptr(a) | self._ptr(b)) % 16 == 0:
@@ -442,9 +479,11 @@ class FastHipBackend(HipBackend):
             # the residual stream is kept in bf16: its gradient, which the tape adds dx to, is kept in bf16 as well
             if gradOutput.store != "bf16":
                 gradOutput = self.castStore(gradOutput, "bf16")
-            gp = self._ptr(gradOutput)
+            self._launch_ln()
+            gp, xp, wp = self._ptr(gradOutput), self._ptr(x), self._ptr(weight)
             dx, dw, db = self._new(x.shape, "f32", "bf16"), self._new(weight.shape), self._new(weight.shape)
-            check(self.lib.ah_layernorm_bwd(self._ptr(x), self._ptr(weight), gp, BF16, 0, 0, dx._buf.ptr, dw._buf.ptr, db._buf.ptr, rows, dim, eps, 0, BF16))
+            self._held_ln = _HeldLayerNormBwd(xp, wp, gp, dx, dw, db, rows, dim, eps,
+                                              self._hold(x._buf, weight._buf, gradOutput._buf, dx._buf, dw._buf, db._buf))
             return {"dx": dx, "dw": dw, "db": db}
         if x.store != "f32":
             return super().layerNormBackward(x, weight, gradOutput, eps)
@@ -453,6 +492,21 @@ class FastHipBackend(HipBackend):
         check(self.lib.ah_layernorm_bwd(self._ptr(x), self._ptr(weight), gp, ffi.DTYPE_CODE[gradOutput.store], 0, dx._buf.ptr, 0, dw._buf.ptr,
                                         db._buf.ptr, rows, dim, eps, 0, ffi.F32))
         return {"dx": dx, "dw": dw, "db": db}
+
+    def _launch_ln(self, residual: int = 0, dx_ptr: int = 0):
+        """Launches the held LayerNorm backward: plainly, or (residual, dx_ptr given) with its dx added to `residual` into dx_ptr."""
+        h, self._held_ln = self._held_ln, None
+        if h is None:
+            return
+        if not dx_ptr and all(b.refs == 1 for b in h.outs):     # every result was released unread
+            self._unhold(h.holds)
+            return
+        check(self.lib.ah_layernorm_bwd(h.x_ptr, h.w_ptr, h.g_ptr, BF16, residual, 0, dx_ptr or h.outs[0].ptr, h.outs[1].ptr, h.outs[2].ptr,
+                                        h.rows, h.dim, h.eps, 0, BF16))
+        if dx_ptr:                                               # the bare dx was not written: keep the recipe until its tensor is released
+            self._ln_unwritten[id(h.outs[0])] = h
+        else:
+            self._unhold(h.holds)
 
     def crossEntropy(self, logits: TensorData, targets: TensorData) -> TensorData:
         N, Cc = logits.shape
@@ -490,6 +544,7 @@ class FastHipBackend(HipBackend):
     # ------------------------------------------------------------------ optimizer
     def totalSumOfSquares(self, tensors: Sequence[TensorData]) -> TensorData:
         self._launch_held()
+        self._launch_ln()
         self._launch_weight_grads()
         return super().totalSumOfSquares(tensors)
 
@@ -550,12 +605,14 @@ class FastHipBackend(HipBackend):
 
     def flush(self):
         self._launch_held()
+        self._launch_ln()
         self._launch_weight_grads()
         self._flush_adam()
         super().flush()
 
     def syncGpu(self):
         self._launch_held()
+        self._launch_ln()
         self._launch_weight_grads()
         self._flush_adam()
         super().syncGpu()

@@ -216,3 +216,66 @@ def test_bf16_tensors_move_as_words_and_the_reference_flash_branch_stays_in_bf16
         assert abs(a.gradNorm - b.gradNorm) <= 5e-2 * a.gradNorm, (s, a.gradNorm, b.gradNorm)
     FB.enableStepGraphs(False)
     assert FB.stepStats()["replayed"] - before["replayed"] >= 4, (before, FB.stepStats(), FB.stepFallbackNotes)
+
+
+def test_layernorm_backward_is_held_until_its_dx_is_added_to_the_stream_gradient(FB):
+    """The tape's sequence after a LayerNorm on the residual stream (tape.ts:116-127): layerNormBackward, then addInplace of dx
+    into the gradient the residual add left on the stream, then clones of dw and db.  The sum comes out of the LayerNorm kernel
+    itself; it, dw and db must equal float64 numpy on the bf16-rounded operands, and the same calls in other orders (dx read
+    first, dx read after it went into the sum, everything released unread) must still give the plain results."""
+    rs = np.random.RandomState(11)
+    rows, dim, eps = 96, 128, 1e-5
+    x, w, g, acc = rs.randn(rows, dim), 1 + 0.1 * rs.randn(dim), rs.randn(rows, dim) * 0.3, rs.randn(rows, dim)
+    xb, gb, ab = _bf16(x).astype(np.float64), _bf16(g).astype(np.float64), _bf16(acc).astype(np.float64)
+    mean = xb.mean(1, keepdims=True)
+    rstd = 1 / np.sqrt(((xb - mean) ** 2).mean(1, keepdims=True) + eps)
+    xh = (xb - mean) * rstd
+    gw = gb * w.astype(np.float32).astype(np.float64)
+    dx = rstd * (gw - gw.mean(1, keepdims=True) - xh * (gw * xh).mean(1, keepdims=True))
+    dw, db = (gb * xh).sum(0), gb.sum(0)
+
+    def operands():
+        return (FB.castStore(_td(x), "bf16"), _td(w), FB.castStore(_td(g), "bf16"), FB.castStore(_td(acc), "bf16"))
+
+    # the tape's order: the sum is one launch, the clone keeps the old contents of the stream gradient
+    tx, tw, tg, ta = operands()
+    keep = FB.clone(ta)
+    r = FB.layerNormBackward(tx, tw, tg, eps)
+    assert FB._held_ln is not None
+    FB.addInplace(ta, r["dx"])
+    assert FB._held_ln is None and ta.store == "bf16"
+    gw_, gb_ = FB.clone(r["dw"]), FB.clone(r["db"])
+    _close(ta.data, ab + dx, "stream gradient + dx", 1e-2)
+    assert np.array_equal(keep.data, ab.astype(np.float32).reshape(keep.data.shape))
+    _close(gw_.data, dw, "dw", 1e-4)
+    _close(gb_.data, db, "db", 1e-4)
+    # dx itself was never written; a reader still gets it
+    _close(r["dx"].data, dx, "dx read after it went into the sum", 1e-2)
+    FB.releaseGpuTensor(r["dx"])
+    assert not FB._ln_unwritten
+
+    # dx read first: the plain kernel, then an ordinary add
+    tx, tw, tg, ta = operands()
+    r = FB.layerNormBackward(tx, tw, tg, eps)
+    _close(r["dx"].data, dx, "dx", 1e-2)
+    assert FB._held_ln is None
+    FB.addInplace(ta, r["dx"])
+    _close(ta.data, ab + dx, "stream gradient + dx, two launches", 1.5e-2)
+    _close(r["dw"].data, dw, "dw", 1e-4)
+
+    # a second LayerNorm backward while one is held launches the first
+    tx, tw, tg, ta = operands()
+    r1 = FB.layerNormBackward(tx, tw, tg, eps)
+    r2 = FB.layerNormBackward(tx, tw, tg, eps)
+    FB.addInplace(ta, r2["dx"])
+    _close(r1["dx"].data, dx, "first of two", 1e-2)
+    _close(ta.data, ab + dx, "second of two", 1e-2)
+    FB.releaseGpuTensor(r2["dx"])                              # (what the tape does with a gradient it has consumed)
+
+    # released unread: nothing is launched, nothing is left behind
+    tx, tw, tg, ta = operands()
+    r = FB.layerNormBackward(tx, tw, tg, eps)
+    for t in r.values():
+        FB.releaseGpuTensor(t)
+    FB.flush()
+    assert FB._held_ln is None and not FB._ln_unwritten
