@@ -133,7 +133,7 @@ SIGNATURES = {
     "ah_adamw": [u64, u64, u64, u64, u64, C.POINTER(AhAdamW), u64, u64, u64],
     "ah_clip_coef": [u64, f32, f32, u64],
     "ah_side_begin": [], "ah_side_end": [], "ah_side_join": [],
-    "ah_step_begin": [u64], "ah_step_end": [C.POINTER(C.c_int32)], "ah_step_reset": [u64],
+    "ah_step_begin": [u64], "ah_step_end": [C.POINTER(C.c_int32)], "ah_step_reset": [u64], "ah_step_kick": [],
     "ah_step_guard": [u64, u64, f32, f32, C.c_double, C.c_double, u64, u64, u64],
     "ah_lion": [u64, u64, u64, u64, C.POINTER(AhLion)], "ah_sgd": [u64, u64, u64, C.c_double, C.c_double],
     "ah_adafactor_2d": [u64, u64, u64, u64, i64, i64, C.POINTER(AhAdafactor)],

@@ -82,8 +82,10 @@ class FastHipBackend(HipBackend):
         # adamwStep calls of one optimizer pass, launched together (one kernel per 48 tensors) when anything needs their result
         self._adam_q: List[tuple] = []   # (p, g, m, v, shadow, n, weight decay) as device addresses
         self._adam_key = None
+        self._adam_flush_at = 1
         self._adam_holds: List[_Buf] = []
         self._adam_bufs = set()          # id(_Buf) of every buffer a queued update reads or writes
+        self._ssq_args = None            # (addresses, sizes, their ctypes arrays) of the last totalSumOfSquares call
         self._held_ln: Optional[_HeldLayerNormBwd] = None
         # dx tensors whose LayerNorm backward went straight into a sum and that were never written themselves: id(_Buf) -> recipe
         self._ln_unwritten = {}
@@ -546,6 +548,23 @@ class FastHipBackend(HipBackend):
         self._launch_held()
         self._launch_ln()
         self._launch_weight_grads()
+        self._flush_adam()
+        # The device is idle while this runs (the trainer has just read the loss back, trainer.ts:1247,1345-1349): with nothing
+        # pending and every gradient resident in f32, the addresses are read straight off the tensors, and the argument
+        # arrays of the last call are reused when the gradient set sits where it sat then.
+        if not self._orphans and not self._ln_unwritten:
+            try:
+                key = tuple([t._buf.ptr + t._off if t._dev_valid and t.store == "f32" else None for t in tensors])
+            except AttributeError:                              # a tensor without a device buffer
+                key = (None,)
+            if None not in key and len(key) > 0:
+                c = self._ssq_args
+                if c is None or c[0] != key or c[1] != [t.size for t in tensors]:
+                    sizes = [t.size for t in tensors]
+                    c = self._ssq_args = (key, sizes, (C.c_uint64 * len(key))(*key), (C.c_uint64 * len(key))(*sizes))
+                total = self._new((1,))
+                check(self.lib.ah_sum_sq_list(c[2], c[3], len(key), total._buf.ptr))
+                return total
         return super().totalSumOfSquares(tensors)
 
     def adamwStep(self, params, grads, m, v, lr, beta1, beta2, eps, weightDecay, bc1, bc2, gradScale=1.0):
@@ -562,6 +581,8 @@ class FastHipBackend(HipBackend):
             self._own(t)
         ptrs = [self._ptr(t) for t in (params, grads, m, v)]    # (launches whatever still has to produce the gradient)
         if not self._adam_q:
+            if key != self._adam_key:
+                self._adam_flush_at = 1                         # a new optimizer pass
             self._adam_key = key
             self._adam_hyper(lr, beta1, beta2, eps, 0.0, bc1, bc2, gradScale)      # the device copy of the scalars, once per pass
         sh = getattr(params, "_shadow", None)
@@ -572,8 +593,10 @@ class FastHipBackend(HipBackend):
             self._adam_bufs.add(id(b))
         for t in (params, m, v):
             HipBackend._dirty(self, t)                          # host copies are stale; the shadow is refreshed by the kernel
-        if len(self._adam_q) >= 16:                             # the device is usually idle here (the norm was just read back):
-            self._flush_adam()                                  # give it the first tensors while the host queues the rest
+        if len(self._adam_q) >= self._adam_flush_at:            # the device is usually idle here (the norm was just read back):
+            self._flush_adam()                                  # give it the first tensor at once, then 16 while the host queues
+            self._adam_flush_at = 16 if self._adam_flush_at == 1 else 48      # the rest, then a launch's full table at a time
+            check(self.lib.ah_step_kick())                      # (inside a step plan: launch now, do not wait for a full segment)
 
     def _flush_adam(self):
         q, self._adam_q = self._adam_q, []

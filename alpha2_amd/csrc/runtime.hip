@@ -317,7 +317,7 @@ int32_t step_boundary(const char *what) {
     int32_t rc = step_close_segment(what);
     if (rc != AH_OK) { g.plan->broken = true; return rc; }
     g.plan->segs.emplace_back();
-    if (strcmp(what, "chunk") != 0) g.chunks_since_host_boundary = 0;
+    if (strcmp(what, "chunk") != 0 && strcmp(what, "kick") != 0) g.chunks_since_host_boundary = 0;
     return AH_OK;
   }
   StepSeg &sg = g.plan->segs[g.seg];
@@ -748,6 +748,14 @@ int32_t ah_step_end(int32_t *out_how) {
   g.step_mode = STEP_OFF; g.plan = nullptr; g.step_capture_open = false;
   if (out_how) *out_how = how;
   return rc;
+}
+
+int32_t ah_step_kick(void) {
+  AH_REQUIRE_READY();
+  if (g.step_mode != STEP_RECORD && g.step_mode != STEP_VERIFY) return AH_OK;
+  int32_t rc = step_boundary("kick");
+  if (rc != AH_OK) return rc;
+  return step_resume();
 }
 
 int32_t ah_step_reset(uint64_t key) {

@@ -115,6 +115,12 @@ enum { AH_STEP_EAGER = 0, AH_STEP_RECORDED = 1, AH_STEP_REPLAYED = 2, AH_STEP_FE
 int32_t     ah_step_begin(uint64_t key);
 int32_t     ah_step_end(int32_t *out_how);
 int32_t     ah_step_reset(uint64_t key);          /* drop the plan of `key` */
+/* A hint from a caller that is about to spend host time before its next launches (e.g. between the first and the later
+ * adamwStep calls of an optimizer pass, packages/train/src/optimizers.ts:54-94): what has been issued since the last boundary
+ * becomes a segment of its own and is launched now instead of waiting for the segment to fill.  Part of the plan like any
+ * other boundary (a replay expects it at the same place); a no-op outside a step and when nothing has been issued.  The
+ * reference's counterpart is an early batchSubmit (helios_vk.c:4417). */
+int32_t     ah_step_kick(void);
 const char *ah_step_note(void);                    /* why the last step fell back ("" if it did not) */
 
 /* ---- a side stream (same priority) for work nothing depends on for a while, e.g. weight gradients, which only the

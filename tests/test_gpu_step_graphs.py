@@ -83,3 +83,35 @@ def test_per_step_scalars_and_dropout_seeds_follow_the_caller(B):
     assert len({x[3] for x in graph}) > 3                       # the schedule moved
     for n in pe:
         assert np.array_equal(pe[n], pg[n]), n
+
+
+def test_a_kick_is_a_boundary_of_the_plan(B):
+    """ah_step_kick launches what has been issued so far as a segment of its own: the same results as without it, expected at
+    the same place on replay (a step that kicks elsewhere falls back), and a no-op outside a step or with nothing issued."""
+    from alpha2_amd import TensorData
+    from alpha2_amd._ffi import check
+    x = TensorData((4096,), "f32", np.arange(4096, dtype=np.float32))
+    assert B.lib.ah_step_kick() == 0                                 # outside a step
+    B._ptr(x)                                                        # (uploaded before the plan, so every step issues the same calls)
+
+    def step(kick_after):
+        t = x
+        check(B.lib.ah_step_kick())                                  # nothing issued yet
+        for i in range(6):
+            t = B.scale(t, 1.5)
+            if i == kick_after:
+                check(B.lib.ah_step_kick())
+        return t
+
+    B.enableStepGraphs(True)
+    B.flush()
+    want = x.data * np.float32(1.5) ** 6
+    hows = []
+    for kick_after in (2, 2, 2, 4, 2, 2):
+        got = step(kick_after).data.copy()
+        B.flush()
+        hows.append(B.lastStepHow)
+        assert np.array_equal(got, want), kick_after               # (every product is exact in f32)
+    B.enableStepGraphs(False)
+    assert hows[0] == "recorded" and hows[1] == hows[2] == "replayed", hows
+    assert hows[3] == "fell-back" and hows[4] == "recorded" and hows[5] == "replayed", (hows, B.lastStepNote)
