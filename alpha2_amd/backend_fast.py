@@ -65,6 +65,20 @@ class _HeldLayerNormBwd:
         self.rows, self.dim, self.eps, self.holds = rows, dim, eps, holds
 
 
+class _HeldScatter:
+    """scatterSlice results that have been asked for and not written: column blocks of a [rows, cols] bf16 matrix that is zero
+    elsewhere.  The tape adds the three blocks of d(qkv) to one another (ops.ts:816-858, tape.ts:116-127): sums of held scatters
+    with disjoint columns are merged, and the matrix is written once, each block copied to its place."""
+
+    def __init__(self, rows, cols, parts, srcs, out):
+        self.rows, self.cols = rows, cols
+        self.parts = parts                  # [(source address, first column, width)]
+        self.srcs, self.out = srcs, out     # held buffers: the sources, the (unwritten) result
+
+    def disjoint(self, other) -> bool:
+        return all(c0 + w <= d0 or d0 + v <= c0 for _, c0, w in self.parts for _, d0, v in other.parts)
+
+
 class FastHipBackend(HipBackend):
     name = "hip"
 
@@ -86,6 +100,7 @@ class FastHipBackend(HipBackend):
         self._adam_holds: List[_Buf] = []
         self._adam_bufs = set()          # id(_Buf) of every buffer a queued update reads or writes
         self._ssq_args = None            # (addresses, sizes, their ctypes arrays) of the last totalSumOfSquares call
+        self._scatters = {}              # id(_Buf) of an unwritten scatterSlice result -> _HeldScatter
         self._held_ln: Optional[_HeldLayerNormBwd] = None
         # dx tensors whose LayerNorm backward went straight into a sum and that were never written themselves: id(_Buf) -> recipe
         self._ln_unwritten = {}
@@ -122,6 +137,8 @@ class FastHipBackend(HipBackend):
                                                 h.rows, h.dim, h.eps, 0, BF16))
                 scratch.release()
                 self._unhold(h.holds)
+            if self._scatters and id(t._buf) in self._scatters:
+                self._write_scatter(t._buf)
             if self._held is not None and t._buf is self._held.out_buf:
                 self._launch_held()
             elif self._wgrads and (self._is_queued(t._buf) or any(w.into is not None and w.into[0] is t._buf for w in self._wgrads)):
@@ -197,11 +214,36 @@ class FastHipBackend(HipBackend):
     def scatterSlice(self, grad: TensorData, origShape, starts, ends) -> TensorData:
         if grad.store != "bf16" or not grad.shape or grad.shape[-1] % 2 or origShape[-1] % 2 or starts[-1] % 2:
             return super().scatterSlice(grad, origShape, starts, ends)
+        if len(origShape) == 2 and len(grad.shape) == 2 and starts[0] == 0 and grad.shape[0] == origShape[0] and grad.size > 0 \
+                and starts[1] + grad.shape[1] <= origShape[1]:
+            gp = self._ptr(grad)                                # a column block of whole rows: held back
+            out = self._new(origShape, grad.dtype, "bf16")
+            grad._buf.refs += 1
+            out._buf.refs += 1
+            self._scatters[id(out._buf)] = _HeldScatter(origShape[0], origShape[1], [(gp, starts[1], grad.shape[1])], [grad._buf], out._buf)
+            return out
         halve = lambda xs: list(xs[:-1]) + [xs[-1] // 2]
         out = self._new(origShape, grad.dtype, "bf16")
         check(self.lib.ah_scatter_slice(self._ptr(grad), out._buf.ptr, len(origShape), ffi.shape_arr(halve(grad.shape)),
                                         ffi.shape_arr(halve(origShape)), ffi.shape_arr(halve(starts))))
         return out
+
+    def _write_scatter(self, buf):
+        h = self._scatters.pop(id(buf))
+        parts = sorted(h.parts, key=lambda p: p[1])
+        dst = ffi.shape_arr([h.rows, h.cols // 2])
+        covered = parts[0][1] == 0 and parts[-1][1] + parts[-1][2] == h.cols and all(a[1] + a[2] == b[1] for a, b in zip(parts, parts[1:]))
+        for i, (src, c0, w) in enumerate(parts):
+            blk = ffi.shape_arr([h.rows, w // 2])
+            if i == 0 and not covered:                          # the first block brings the zeros of everything that is no block
+                check(self.lib.ah_scatter_slice(src, buf.ptr, 2, blk, dst, ffi.shape_arr([0, c0 // 2])))
+            else:
+                check(self.lib.ah_cat_part(src, buf.ptr, 2, blk, dst, 1, c0 // 2))
+        self._unhold(h.srcs + [h.out])
+
+    def _drop_scatter(self, buf):
+        h = self._scatters.pop(id(buf))
+        self._unhold(h.srcs + [h.out])
 
     def _operand(self, t: TensorData):
         """Device address of `t` as a bf16 matrix operand, and the buffer that must outlive the launch."""
@@ -234,6 +276,8 @@ class FastHipBackend(HipBackend):
                 self._unhold(self._orphans.pop(id(buf)).holds)
             elif self._ln_unwritten and id(buf) in self._ln_unwritten:
                 self._unhold(self._ln_unwritten.pop(id(buf)).holds)
+            elif self._scatters and id(buf) in self._scatters:
+                self._drop_scatter(buf)
             elif self._wgrads:
                 for i, w in enumerate(self._wgrads):
                     if buf is w.out_buf and w.into is None:
@@ -242,7 +286,8 @@ class FastHipBackend(HipBackend):
                         break
 
     def _view(self, t: TensorData, shape, byte_off: int = 0) -> TensorData:
-        if t._buf is not None and t._dev_valid and (self._is_held(t) or id(t._buf) in self._orphans or self._is_queued(t._buf)):
+        if t._buf is not None and t._dev_valid and (self._is_held(t) or id(t._buf) in self._orphans or self._is_queued(t._buf)
+                                                    or id(t._buf) in self._scatters):
             v = TensorData(shape, t.dtype)                      # a view of a held-back product stays held back
             v.store, v._buf, v._off = t.store, t._buf, t._off + byte_off
             t._buf.refs += 1
@@ -397,6 +442,25 @@ class FastHipBackend(HipBackend):
                 w.into = (a._buf, a._off)                        # the grouped launch adds into `a`; `b` itself is never computed
                 a._buf.refs += 1
                 w.holds.append(a._buf)
+                self._dirty(a)
+                return
+        if self._scatters and a._buf is not None and b._buf is not None and a._buf is not b._buf:
+            sa, sb = self._scatters.get(id(a._buf)), self._scatters.get(id(b._buf))
+            if sa is not None and sb is not None and a._off == 0 and b._off == 0 and a.size == b.size == sa.rows * sa.cols \
+                    and (sa.rows, sa.cols) == (sb.rows, sb.cols) and a._dev_valid and sa.disjoint(sb):
+                for x in sb.srcs:
+                    x.refs += 1
+                if a._buf.refs > 2:                              # (its own name and the record's hold are two) shared with a clone:
+                    for x in sa.srcs:                            # the sum gets a buffer and a record of its own
+                        x.refs += 1
+                    nb = _Buf(self.lib, a.size * 2)
+                    nb.refs += 1
+                    self._scatters[id(nb)] = _HeldScatter(sa.rows, sa.cols, sa.parts + sb.parts, sa.srcs + sb.srcs, nb)
+                    a._buf.release()
+                    a._buf = nb
+                else:
+                    sa.parts = sa.parts + sb.parts
+                    sa.srcs = sa.srcs + sb.srcs
                 self._dirty(a)
                 return
         h = self._held_ln

@@ -279,3 +279,56 @@ def test_layernorm_backward_is_held_until_its_dx_is_added_to_the_stream_gradient
         FB.releaseGpuTensor(t)
     FB.flush()
     assert FB._held_ln is None and not FB._ln_unwritten
+
+
+def test_scattered_column_blocks_are_merged_before_they_are_written(FB):
+    """The backward of sliceQkv (ops.ts:816-858): three scatterSlice results, the first cloned and the others added in place
+    (tape.ts:116-127).  Held back, the three become one matrix written once; blocks that leave columns uncovered bring their
+    zeros; overlapping blocks and blocks read on their own take the ordinary route.  All exact: copies and zeros only."""
+    rs = np.random.RandomState(13)
+    rows, d = 48, 32
+    blocks = [_bf16(rs.randn(rows, d)) for _ in range(3)]
+    full = np.concatenate(blocks, axis=1)
+
+    def scatter(i, at=None):
+        c0 = d * i if at is None else at
+        return FB.scatterSlice(FB.castStore(_td(blocks[i]), "bf16"), (rows, 3 * d), [0, c0], [rows, c0 + d])
+
+    # the tape's sequence, last block first
+    s = scatter(2)
+    acc = FB.clone(s)
+    FB.releaseGpuTensor(s)
+    for i in (1, 0):
+        s = scatter(i)
+        FB.addInplace(acc, s)
+        FB.releaseGpuTensor(s)
+    assert len(FB._scatters) == 1                                  # one unwritten matrix, three blocks
+    assert np.array_equal(acc.data.reshape(rows, 3 * d), full)
+    assert not FB._scatters
+
+    # two of three blocks: the rest is zero; a clone taken in between keeps the single block
+    s = scatter(0)
+    acc = FB.clone(s)
+    s2 = scatter(2)
+    FB.addInplace(acc, s2)                                         # `s` still names the first buffer: the sum gets its own
+    want = full.copy()
+    want[:, d:2 * d] = 0
+    assert np.array_equal(acc.data.reshape(rows, 3 * d), want)
+    only0 = np.zeros_like(full)
+    only0[:, :d] = blocks[0]
+    assert np.array_equal(s.data.reshape(rows, 3 * d), only0)
+    only2 = np.zeros_like(full)
+    only2[:, 2 * d:] = blocks[2]
+    assert np.array_equal(s2.data.reshape(rows, 3 * d), only2)
+
+    # overlapping blocks are really added
+    a, b = scatter(0, at=0), scatter(1, at=d // 2)
+    acc = FB.clone(a)
+    FB.addInplace(acc, b)
+    want = np.zeros((rows, 3 * d), np.float32)
+    want[:, :d] += blocks[0]
+    want[:, d // 2:d // 2 + d] += blocks[1]
+    _close(acc.data, _bf16(want), "overlapping blocks", 1e-2)
+    for t in (a, b, acc, s, s2):
+        FB.releaseGpuTensor(t)
+    assert not FB._scatters
