@@ -1,5 +1,6 @@
 // Element-wise and data-movement kernels (HBM-bound; coalesced, float4 where alignment allows).
 #include "common.h"
+#include <cstring>
 
 using namespace ah;
 
@@ -451,7 +452,7 @@ int32_t ah_binary_broadcast(int32_t op, ah_ptr a, ah_ptr b, ah_ptr out, int32_t 
   AH_REQUIRE_READY();
   AH_ARG(op >= AH_ADD && op <= AH_DIV, "ah_binary_broadcast: bad op %d", op);
   AH_ARG(nd >= 0 && nd <= 6, "ah_binary_broadcast: nd %d > 6", nd);
-  Dims6 d; d.nd = nd;
+  Dims6 d; memset(&d, 0, sizeof d); d.nd = nd;      // (zeroed: see the Gather6 arguments below)
   for (int i = 0; i < nd; i++) { d.shape[i] = shape[i]; d.sa[i] = stride_a[i]; d.sb[i] = stride_b[i]; }
   uint64_t n = (uint64_t)prod(nd, shape);
   if (n == 0) return AH_OK;
@@ -704,7 +705,7 @@ int32_t ah_transpose(ah_ptr a, ah_ptr out, int32_t nd, const int64_t *shape, int
   }
   // out[i] over the transposed shape gathers from a with swapped strides
   int64_t st[6]; row_major_strides(nd, shape, st);
-  Gather6 g; g.nd = nd; g.offset = 0;
+  Gather6 g; memset(&g, 0, sizeof g); g.nd = nd; g.offset = 0;      // (zeroed: the unused dimensions and the padding are part of the argument a step plan compares)
   for (int i = 0; i < nd; i++) { g.shape[i] = shape[i]; g.stride[i] = st[i]; }
   { int64_t t = g.shape[d0]; g.shape[d0] = g.shape[d1]; g.shape[d1] = t; t = g.stride[d0]; g.stride[d0] = g.stride[d1]; g.stride[d1] = t; }
   ah::launch_kernel(k_gather, dim3(grid_for(n)), dim3(TPB), 0, dp<const uint32_t>(a), dp<uint32_t>(out), n, g);
@@ -716,7 +717,7 @@ int32_t ah_slice(ah_ptr a, ah_ptr out, int32_t nd, const int64_t *shape, const i
   AH_REQUIRE_READY();
   AH_ARG(nd >= 1 && nd <= 6, "ah_slice: nd %d out of range", nd);
   int64_t st[6]; row_major_strides(nd, shape, st);
-  Gather6 g; g.nd = nd; g.offset = 0;
+  Gather6 g; memset(&g, 0, sizeof g); g.nd = nd; g.offset = 0;      // (zeroed: the unused dimensions and the padding are part of the argument a step plan compares)
   for (int i = 0; i < nd; i++) {
     AH_ARG(starts[i] >= 0 && ends[i] <= shape[i] && starts[i] <= ends[i], "ah_slice: range [%lld,%lld) outside dim %d of size %lld",
            (long long)starts[i], (long long)ends[i], i, (long long)shape[i]);
@@ -734,7 +735,7 @@ int32_t ah_scatter_slice(ah_ptr grad, ah_ptr out, int32_t nd, const int64_t *gsh
   AH_REQUIRE_READY();
   AH_ARG(nd >= 1 && nd <= 6, "ah_scatter_slice: nd %d out of range", nd);
   int64_t st[6]; row_major_strides(nd, orig, st);
-  Gather6 g; g.nd = nd; g.offset = 0;
+  Gather6 g; memset(&g, 0, sizeof g); g.nd = nd; g.offset = 0;      // (zeroed: the unused dimensions and the padding are part of the argument a step plan compares)
   for (int i = 0; i < nd; i++) {
     AH_ARG(starts[i] >= 0 && starts[i] + gshape[i] <= orig[i], "ah_scatter_slice: slice does not fit dim %d", i);
     g.shape[i] = gshape[i]; g.stride[i] = st[i]; g.offset += starts[i] * st[i];
@@ -758,7 +759,7 @@ int32_t ah_cat_part(ah_ptr src, ah_ptr dst, int32_t nd, const int64_t *src_shape
   if (axis < 0) axis += nd;
   AH_ARG(axis >= 0 && axis < nd, "ah_cat_part: axis out of range");
   int64_t st[6]; row_major_strides(nd, dst_shape, st);
-  Gather6 g; g.nd = nd; g.offset = axis_offset * st[axis];
+  Gather6 g; memset(&g, 0, sizeof g); g.nd = nd; g.offset = axis_offset * st[axis];
   for (int i = 0; i < nd; i++) {
     if (i != axis) AH_ARG(src_shape[i] == dst_shape[i], "cat: shape mismatch at dim %d", i);
     g.shape[i] = src_shape[i]; g.stride[i] = st[i];
@@ -786,7 +787,7 @@ int32_t ah_slice_qkv(ah_ptr qkv, ah_ptr q, ah_ptr k, ah_ptr v, int64_t rows, int
 int32_t ah_broadcast(ah_ptr a, ah_ptr out, int32_t nd, const int64_t *out_shape, const int64_t *stride_a) {
   AH_REQUIRE_READY();
   AH_ARG(nd >= 0 && nd <= 6, "ah_broadcast: nd %d out of range", nd);
-  Gather6 g; g.nd = nd; g.offset = 0;
+  Gather6 g; memset(&g, 0, sizeof g); g.nd = nd; g.offset = 0;      // (zeroed: the unused dimensions and the padding are part of the argument a step plan compares)
   for (int i = 0; i < nd; i++) { g.shape[i] = out_shape[i]; g.stride[i] = stride_a[i]; }
   uint64_t n = (uint64_t)prod(nd, out_shape);
   if (n == 0) return AH_OK;
