@@ -249,30 +249,51 @@ __global__ void k_binary_bcast(const float *__restrict__ a, const float *__restr
   }
 }
 
-// generic strided gather: out[i] = src[offset + sum(coord_k * stride_k)] over `shape`
+// generic strided gather: out[i] = src[offset + sum(coord_k * stride_k)] over `shape`; strided scatter: dst[that] = src[i].
+// W is the unit moved (one 4-byte word, or four when the innermost dimension is contiguous on both sides and everything is a
+// multiple of four words: shape, strides and offset are then in units of W), I the integer type of the index arithmetic (32-bit
+// whenever every index fits: a 64-bit division is the most expensive thing in these kernels).
 struct Gather6 { int64_t shape[6]; int64_t stride[6]; int64_t offset; int nd; };
-__global__ void k_gather(const uint32_t *__restrict__ src, uint32_t *__restrict__ out, uint64_t n, Gather6 d) {
-  uint64_t tid = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x, stride = (uint64_t)gridDim.x * blockDim.x;
-  for (uint64_t i = tid; i < n; i += stride) {
-    uint64_t rem = i; int64_t s = d.offset;
-    for (int k = d.nd - 1; k >= 0; k--) {
-      uint64_t c = rem % (uint64_t)d.shape[k]; rem /= (uint64_t)d.shape[k];
-      s += (int64_t)c * d.stride[k];
-    }
-    out[i] = src[s];
+template <class W, class I, bool SCATTER>
+__global__ void k_move(const W *__restrict__ src, W *__restrict__ dst, uint64_t n, Gather6 d) {
+  const I total = (I)n, step = (I)((uint64_t)gridDim.x * blockDim.x);
+  I shp[6], str[6];
+#pragma unroll
+  for (int k = 0; k < 6; k++) { shp[k] = (I)d.shape[k]; str[k] = (I)d.stride[k]; }
+  for (I i = (I)(blockIdx.x * (uint64_t)blockDim.x + threadIdx.x); i < total; i += step) {
+    I rem = i, s = (I)d.offset;
+#pragma unroll
+    for (int k = 5; k >= 0; k--)
+      if (k < d.nd) {
+        const I q = rem / shp[k], c = rem - q * shp[k];
+        rem = q;
+        s += c * str[k];
+      }
+    if (SCATTER) dst[s] = src[i]; else dst[i] = src[s];
+    if (i + step < i) break;                                       // (the index type wrapped: i was the last one)
   }
 }
-// generic strided scatter: dst[offset + sum(coord_k*stride_k)] = src[i]
-__global__ void k_scatter(const uint32_t *__restrict__ src, uint32_t *__restrict__ dst, uint64_t n, Gather6 d) {
-  uint64_t tid = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x, stride = (uint64_t)gridDim.x * blockDim.x;
-  for (uint64_t i = tid; i < n; i += stride) {
-    uint64_t rem = i; int64_t s = d.offset;
-    for (int k = d.nd - 1; k >= 0; k--) {
-      uint64_t c = rem % (uint64_t)d.shape[k]; rem /= (uint64_t)d.shape[k];
-      s += (int64_t)c * d.stride[k];
-    }
-    dst[s] = src[i];
+// `g` describes the strided side; the other side is contiguous over g.shape.
+template <bool SCATTER>
+static void launch_move(const void *src, void *dst, uint64_t n, Gather6 g) {
+  const int nd = g.nd;
+  const uintptr_t both = (uintptr_t)src | (uintptr_t)dst;
+  bool vec = nd >= 1 && g.stride[nd - 1] == 1 && g.shape[nd - 1] % 4 == 0 && g.offset % 4 == 0 && (both & 15u) == 0;
+  for (int k = 0; vec && k < nd - 1; k++) vec = g.stride[k] % 4 == 0;
+  if (vec) {
+    g.shape[nd - 1] /= 4; g.offset /= 4; n /= 4;
+    for (int k = 0; k < nd - 1; k++) g.stride[k] /= 4;
   }
+  uint64_t reach = (uint64_t)g.offset;                             // largest index on the strided side
+  bool nonneg = g.offset >= 0;
+  for (int k = 0; k < nd; k++) { nonneg = nonneg && g.stride[k] >= 0; if (g.shape[k] > 0 && g.stride[k] > 0) reach += (uint64_t)(g.shape[k] - 1) * (uint64_t)g.stride[k]; }
+  const bool small = nonneg && n < (uint64_t(1) << 31) && reach < (uint64_t(1) << 31);
+  const dim3 grid(grid_for(n)), blk(TPB);
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+  if (vec && small) ah::launch_kernel((k_move<u32x4, uint32_t, SCATTER>), grid, blk, 0, (const u32x4 *)src, (u32x4 *)dst, n, g);
+  else if (vec) ah::launch_kernel((k_move<u32x4, uint64_t, SCATTER>), grid, blk, 0, (const u32x4 *)src, (u32x4 *)dst, n, g);
+  else if (small) ah::launch_kernel((k_move<uint32_t, uint32_t, SCATTER>), grid, blk, 0, (const uint32_t *)src, (uint32_t *)dst, n, g);
+  else ah::launch_kernel((k_move<uint32_t, uint64_t, SCATTER>), grid, blk, 0, (const uint32_t *)src, (uint32_t *)dst, n, g);
 }
 
 // 32x32 LDS-tiled transpose of the last two dims of [batch, R, C] (coalesced both ways)
@@ -708,7 +729,7 @@ int32_t ah_transpose(ah_ptr a, ah_ptr out, int32_t nd, const int64_t *shape, int
   Gather6 g; memset(&g, 0, sizeof g); g.nd = nd; g.offset = 0;      // (zeroed: the unused dimensions and the padding are part of the argument a step plan compares)
   for (int i = 0; i < nd; i++) { g.shape[i] = shape[i]; g.stride[i] = st[i]; }
   { int64_t t = g.shape[d0]; g.shape[d0] = g.shape[d1]; g.shape[d1] = t; t = g.stride[d0]; g.stride[d0] = g.stride[d1]; g.stride[d1] = t; }
-  ah::launch_kernel(k_gather, dim3(grid_for(n)), dim3(TPB), 0, dp<const uint32_t>(a), dp<uint32_t>(out), n, g);
+  launch_move<false>(dp<const void>(a), dp<void>(out), n, g);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
@@ -726,7 +747,7 @@ int32_t ah_slice(ah_ptr a, ah_ptr out, int32_t nd, const int64_t *shape, const i
   uint64_t n = (uint64_t)prod(nd, g.shape);
   if (n == 0) return AH_OK;
   AH_ARG(a && out, "ah_slice: null operand");
-  ah::launch_kernel(k_gather, dim3(grid_for(n)), dim3(TPB), 0, dp<const uint32_t>(a), dp<uint32_t>(out), n, g);
+  launch_move<false>(dp<const void>(a), dp<void>(out), n, g);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
@@ -747,7 +768,7 @@ int32_t ah_scatter_slice(ah_ptr grad, ah_ptr out, int32_t nd, const int64_t *gsh
   if (rc) return rc;
   if (n == 0) return AH_OK;
   AH_ARG(grad != 0, "ah_scatter_slice: null grad");
-  ah::launch_kernel(k_scatter, dim3(grid_for(n)), dim3(TPB), 0, dp<const uint32_t>(grad), dp<uint32_t>(out), n, g);
+  launch_move<true>(dp<const void>(grad), dp<void>(out), n, g);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
@@ -768,7 +789,7 @@ int32_t ah_cat_part(ah_ptr src, ah_ptr dst, int32_t nd, const int64_t *src_shape
   uint64_t n = (uint64_t)prod(nd, src_shape);
   if (n == 0) return AH_OK;
   AH_ARG(src && dst, "ah_cat_part: null operand");
-  ah::launch_kernel(k_scatter, dim3(grid_for(n)), dim3(TPB), 0, dp<const uint32_t>(src), dp<uint32_t>(dst), n, g);
+  launch_move<true>(dp<const void>(src), dp<void>(dst), n, g);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
@@ -792,7 +813,7 @@ int32_t ah_broadcast(ah_ptr a, ah_ptr out, int32_t nd, const int64_t *out_shape,
   uint64_t n = (uint64_t)prod(nd, out_shape);
   if (n == 0) return AH_OK;
   AH_ARG(a && out, "ah_broadcast: null operand");
-  ah::launch_kernel(k_gather, dim3(grid_for(n)), dim3(TPB), 0, dp<const uint32_t>(a), dp<uint32_t>(out), n, g);
+  launch_move<false>(dp<const void>(a), dp<void>(out), n, g);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
