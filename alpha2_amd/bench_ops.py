@@ -182,6 +182,16 @@ def bench_bandwidth(b: Bench):
     b.record("layernorm bwd 16384x768, bf16 stream", ms, nbytes=rows * dim * 8, note="x, g, residual grad bf16 -> dx bf16; partial dw, db (column sums put off)")
     b.release()
 
+    # data movement of the reference's flash-attention branch (gpt.ts:232-253) on bf16 storage, moved as 4-byte words
+    qkv16, q16 = b.randn(rows * 3 * dim, ffi.BF16), [b.alloc(rows * dim * 2) for _ in range(3)]
+    ms = b.time(lambda: ffi.check(lib.ah_slice_qkv(qkv16, q16[0], q16[1], q16[2], rows, dim // 2)))
+    b.record("sliceQkv 16384x2304 bf16", ms, nbytes=rows * 3 * dim * 4, note="three column blocks, one launch each")
+    tr = b.alloc(rows * dim * 2)
+    shp = ffi.shape_arr([16, 12, 1024, 32])
+    ms = b.time(lambda: ffi.check(lib.ah_transpose(q16[0], tr, 4, shp, 1, 2)))
+    b.record("transpose [16,12,1024,64] bf16, dims 1 and 2", ms, nbytes=rows * dim * 4, note="heads <-> positions, 128-byte rows kept whole")
+    b.release()
+
     h = b.randn(rows * F, ffi.F32)
     gh, oh = b.randn(rows * F, ffi.F32), b.alloc(rows * F * 4)
     ms = b.time(lambda: ffi.check(lib.ah_unary(ffi.GELU, h, oh, rows * F, 0.0, 0.0)))
