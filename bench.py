@@ -104,6 +104,10 @@ def main():
     if args.gpus != 1:
         print("bench.py: this build runs the step on ONE GPU; --gpus must be 1 (no multi-GPU path exists in this run)", file=sys.stderr)
         sys.exit(2)
+    if args.mode == "backend" and not args.no_step_graphs:
+        # a step plan takes up to five steps to settle: one eager step, one recorded, and - when the recorded step's buffers
+        # were not yet at their steady addresses - one replayed, one that falls back and one recorded again
+        args.warmup = max(args.warmup, 6)
 
     from alpha2_amd import FastHipBackend, HipBackend
     from alpha2_amd.model import ModelConfig
