@@ -89,6 +89,7 @@ class FastHipBackend(HipBackend):
         self.streamBf16 = stream_bf16
         self._held: Optional[_HeldGemm] = None
         self._wgrads: List[_HeldWeightGrad] = []
+        self._wq_out, self._wq_into = set(), set()   # id(_Buf) of the queued gradients' results / of the tensors they will be added into
         self._group = group_weight_grads
         self._plans = {}                 # descriptor tuple -> grouped plan id
         # products that became another op's epilogue and were never written themselves: computed only if somebody reads them
@@ -120,7 +121,7 @@ class FastHipBackend(HipBackend):
         return h is not None and t._buf is h.out_buf
 
     def _is_queued(self, buf) -> bool:
-        return any(buf is w.out_buf for w in self._wgrads)
+        return id(buf) in self._wq_out
 
     def _ptr(self, t: TensorData) -> int:
         if not t._dev_valid and t._buf is not None:
@@ -141,7 +142,7 @@ class FastHipBackend(HipBackend):
                 self._write_scatter(t._buf)
             if self._held is not None and t._buf is self._held.out_buf:
                 self._launch_held()
-            elif self._wgrads and (self._is_queued(t._buf) or any(w.into is not None and w.into[0] is t._buf for w in self._wgrads)):
+            elif self._wgrads and (id(t._buf) in self._wq_out or id(t._buf) in self._wq_into):
                 self._launch_weight_grads()
             elif self._orphans and id(t._buf) in self._orphans:
                 h = self._orphans.pop(id(t._buf))
@@ -282,6 +283,7 @@ class FastHipBackend(HipBackend):
                 for i, w in enumerate(self._wgrads):
                     if buf is w.out_buf and w.into is None:
                         del self._wgrads[i]
+                        self._wq_out.discard(id(buf))
                         self._unhold(w.holds)
                         break
 
@@ -391,12 +393,14 @@ class FastHipBackend(HipBackend):
         bp, bh = self._operand(b)
         out = self._new((K, N))
         self._wgrads.append(_HeldWeightGrad(ap, bp, out, K, N, M, self._hold(ah, bh, out._buf)))
+        self._wq_out.add(id(out._buf))
         if not self._group:
             self._launch_weight_grads()
         return out
 
     def _launch_weight_grads(self):
         ws, self._wgrads = self._wgrads, []
+        self._wq_out, self._wq_into = set(), set()
         descs = []
         for w in ws:
             if w.into is None and w.out_buf.refs == 1:          # released unread
@@ -436,14 +440,16 @@ class FastHipBackend(HipBackend):
             self._unhold(w.holds)
 
     def addInplace(self, a: TensorData, b: TensorData):
-        for w in self._wgrads:
-            if b._buf is w.out_buf and w.into is None and a.store == "f32" and a.size == b.size and a._buf is not None and a._dev_valid \
-                    and a._buf.refs == 1 and not self._is_queued(a._buf) and not any(o.into is not None and o.into[0] is a._buf for o in self._wgrads):
-                w.into = (a._buf, a._off)                        # the grouped launch adds into `a`; `b` itself is never computed
-                a._buf.refs += 1
-                w.holds.append(a._buf)
-                self._dirty(a)
-                return
+        if self._wgrads and b._buf is not None and id(b._buf) in self._wq_out:
+            for w in self._wgrads:
+                if b._buf is w.out_buf and w.into is None and a.store == "f32" and a.size == b.size and a._buf is not None and a._dev_valid \
+                        and a._buf.refs == 1 and id(a._buf) not in self._wq_out and id(a._buf) not in self._wq_into:
+                    w.into = (a._buf, a._off)                    # the grouped launch adds into `a`; `b` itself is never computed
+                    a._buf.refs += 1
+                    w.holds.append(a._buf)
+                    self._wq_into.add(id(a._buf))
+                    self._dirty(a)
+                    return
         if self._scatters and a._buf is not None and b._buf is not None and a._buf is not b._buf:
             sa, sb = self._scatters.get(id(a._buf)), self._scatters.get(id(b._buf))
             if sa is not None and sb is not None and a._off == 0 and b._off == 0 and a.size == b.size == sa.rows * sa.cols \
