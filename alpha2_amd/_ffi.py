@@ -80,7 +80,8 @@ class AhAdafactor(C.Structure):
 SIGNATURES = {
     "ah_init": [i32], "ah_shutdown": [], "ah_device_info": [C.POINTER(AhDeviceInfo)], "ah_sync": [],
     "ah_alloc": [u64, C.POINTER(u64)], "ah_free": [u64], "ah_upload": [u64, C.c_void_p, u64],
-    "ah_download": [C.c_void_p, u64, u64], "ah_copy": [u64, u64, u64], "ah_fill_f32": [u64, f32, u64],
+    "ah_download": [C.c_void_p, u64, u64], "ah_download_begin": [u64, u64, C.POINTER(u64)], "ah_download_end": [u64, C.c_void_p, u64],
+    "ah_copy": [u64, u64, u64], "ah_fill_f32": [u64, f32, u64],
     "ah_fill_i32": [u64, i32, u64], "ah_stats": [C.POINTER(AhStats)], "ah_reset_op_count": [], "ah_trim_pool": [],
     "ah_graph_begin": [], "ah_graph_end": [C.POINTER(u64)], "ah_graph_launch": [u64], "ah_graph_destroy": [u64],
     "ah_event_create": [C.POINTER(u64)], "ah_event_record": [u64], "ah_event_elapsed_ms": [u64, u64, C.POINTER(f32)],

@@ -151,6 +151,12 @@ class FastHipBackend(HipBackend):
         return super()._ptr(t)
 
     def _download(self, t: TensorData):
+        tk = getattr(t, "_early", None)
+        if tk:                                                  # its copy to the host was started when it was computed
+            t._early = None
+            out = np.empty(1, dtype=np.float32)
+            if t._dev_valid and t.store == "f32" and t.size == 1 and self.lib.ah_download_end(tk, out.ctypes.data_as(C.c_void_p), 4) == 0:
+                return out
         self._ptr(t)
         # the host is about to wait for the device: whatever is queued and will be needed anyway (the weight gradients once
         # backward has been issued) goes out first, so the device has work while the host reads and carries on
@@ -176,6 +182,7 @@ class FastHipBackend(HipBackend):
     def _dirty(self, t: TensorData):
         super()._dirty(t)
         t._shadow = None
+        t._early = None
 
     # ---- data movement on bf16 storage.  The kernels behind slice / transpose / scatter copy 4-byte words and never look
     # inside them, so a bf16 tensor whose innermost dimension is even and is left whole (or cut at even columns) is moved as
@@ -585,6 +592,11 @@ class FastHipBackend(HipBackend):
         out, lse = self._new(()), self._new((N,))
         check(self.lib.ah_cross_entropy(self._ptr(logits), ffi.DTYPE_CODE[logits.store], self._ptr(targets), out._buf.ptr, lse._buf.ptr, N, Cc))
         logits._ce_lse = lse
+        # The reference's trainer reads the loss after it has issued the whole backward pass (trainer.ts:1247): the copy to the
+        # host starts now, and reading it later waits for this copy only, not for the backward pass.
+        tk = C.c_uint64(0)
+        if self.lib.ah_download_begin(out._buf.ptr + out._off, 4, C.byref(tk)) == 0:
+            out._early = tk.value
         return out
 
     def crossEntropyBackward(self, logits, targets, gradOutput) -> TensorData:

@@ -54,6 +54,7 @@ struct StepPlan {
 };
 enum { STEP_OFF = 0, STEP_RECORD = 1, STEP_VERIFY = 2, STEP_EAGER = 3 };
 
+constexpr unsigned EARLY_SLOTS = 16, EARLY_SLOT_BYTES = 256;
 struct Context {
   bool inited = false;
   int device = -1;
@@ -85,6 +86,15 @@ struct Context {
   char *ring = nullptr;
   unsigned ring_next = 0;
   hipEvent_t ring_ev[2] = {nullptr, nullptr};
+  // read-backs started early (ah_download_begin): small pinned slots.  The copy runs on a stream of its own behind an event of
+  // the main stream, and the host waits for the copy's own event on that stream: an event of the main stream cannot be waited
+  // for while the main stream is capturing (step plans), one of another stream can.
+  char *early = nullptr;
+  hipStream_t early_stream = nullptr;
+  hipEvent_t early_ev[EARLY_SLOTS] = {}, early_done[EARLY_SLOTS] = {};
+  uint64_t early_id[EARLY_SLOTS] = {};
+  uint32_t early_bytes[EARLY_SLOTS] = {};
+  uint64_t early_next = 1;
   // step plans
   int step_mode = STEP_OFF;
   bool step_capture_open = false, step_fellback = false;
@@ -377,6 +387,14 @@ int32_t ah_init(int32_t device) {
   AH_HIP(hipHostMalloc((void **)&g.ring, RING_SLOTS * RING_SLOT_BYTES, hipHostMallocDefault));
   AH_HIP(hipEventCreateWithFlags(&g.ring_ev[0], hipEventDisableTiming));
   AH_HIP(hipEventCreateWithFlags(&g.ring_ev[1], hipEventDisableTiming));
+  AH_HIP(hipHostMalloc((void **)&g.early, EARLY_SLOTS * EARLY_SLOT_BYTES, hipHostMallocDefault));
+  AH_HIP(hipStreamCreateWithFlags(&g.early_stream, hipStreamNonBlocking));
+  for (unsigned i = 0; i < EARLY_SLOTS; i++) {
+    AH_HIP(hipEventCreateWithFlags(&g.early_ev[i], hipEventDisableTiming));
+    AH_HIP(hipEventCreateWithFlags(&g.early_done[i], hipEventDisableTiming));
+    g.early_id[i] = 0;
+  }
+  g.early_next = 1;
   g.device = device;
   { int32_t rc = static_partials_init(device); if (rc != AH_OK) return rc; }
   g.inited = true;
@@ -407,6 +425,13 @@ int32_t ah_shutdown(void) {
   if (g.ring) (void)hipHostFree(g.ring);
   if (g.ring_ev[0]) (void)hipEventDestroy(g.ring_ev[0]);
   if (g.ring_ev[1]) (void)hipEventDestroy(g.ring_ev[1]);
+  if (g.early) (void)hipHostFree(g.early);
+  for (unsigned i = 0; i < EARLY_SLOTS; i++) {
+    if (g.early_ev[i]) { (void)hipEventDestroy(g.early_ev[i]); g.early_ev[i] = nullptr; }
+    if (g.early_done[i]) { (void)hipEventDestroy(g.early_done[i]); g.early_done[i] = nullptr; }
+  }
+  if (g.early_stream) { (void)hipStreamDestroy(g.early_stream); g.early_stream = nullptr; }
+  g.early = nullptr;
   if (g.side) { (void)hipStreamSynchronize(g.side); (void)hipStreamDestroy(g.side); }
   if (g.side_ev[0]) (void)hipEventDestroy(g.side_ev[0]);
   if (g.side_ev[1]) (void)hipEventDestroy(g.side_ev[1]);
@@ -569,6 +594,38 @@ int32_t ah_download(void *host, ah_ptr src, uint64_t bytes) {
     memcpy(dst + off, g.pinned, chunk);
     off += chunk;
   }
+  return AH_OK;
+}
+
+int32_t ah_download_begin(ah_ptr src, uint64_t bytes, uint64_t *out_ticket) {
+  AH_REQUIRE_READY();
+  AH_ARG(out_ticket != nullptr, "ah_download_begin: null out_ticket");
+  *out_ticket = 0;
+  if (g.capturing) return fail(AH_ERR_STATE, "ah_download_begin: illegal while a graph is being captured");
+  AH_ARG(src != 0 && bytes > 0 && bytes <= EARLY_SLOT_BYTES, "ah_download_begin: 1..%u bytes", EARLY_SLOT_BYTES);
+  { int32_t rc = step_boundary("ah_download_begin"); if (rc != AH_OK) return rc; }
+  struct Resume { ~Resume() { (void)step_resume(); } } resume_capture_on_return;
+  const uint64_t id = g.early_next++;
+  const unsigned slot = (unsigned)(id % EARLY_SLOTS);
+  AH_HIP(hipEventRecord(g.early_ev[slot], g.stream));
+  AH_HIP(hipStreamWaitEvent(g.early_stream, g.early_ev[slot], 0));
+  AH_HIP(hipMemcpyAsync(g.early + slot * EARLY_SLOT_BYTES, dp<void>(src), bytes, hipMemcpyDeviceToHost, g.early_stream));
+  AH_HIP(hipEventRecord(g.early_done[slot], g.early_stream));
+  AH_HIP(hipStreamWaitEvent(g.stream, g.early_done[slot], 0));     // later work may overwrite `src`: it queues behind the copy
+  g.early_id[slot] = id;
+  g.early_bytes[slot] = (uint32_t)bytes;
+  *out_ticket = id;
+  return AH_OK;
+}
+
+int32_t ah_download_end(uint64_t ticket, void *host, uint64_t bytes) {
+  AH_REQUIRE_READY();
+  AH_ARG(host != nullptr, "ah_download_end: null host");
+  const unsigned slot = (unsigned)(ticket % EARLY_SLOTS);
+  if (ticket == 0 || g.early_id[slot] != ticket) return fail(AH_ERR_STATE, "ah_download_end: ticket %llu is no longer held (newer read-backs took its slot)", (unsigned long long)ticket);
+  AH_ARG(bytes == g.early_bytes[slot], "ah_download_end: %llu bytes asked, %u copied", (unsigned long long)bytes, g.early_bytes[slot]);
+  AH_HIP(hipEventSynchronize(g.early_done[slot]));
+  memcpy(host, g.early + slot * EARLY_SLOT_BYTES, bytes);
   return AH_OK;
 }
 

@@ -13,7 +13,7 @@
  *     byte offset is a valid operand (views).  Only handles returned by ah_alloc may be freed.
  *   - Tensors are row-major contiguous unless a leading-dimension argument says otherwise.
  *   - One caller thread.  All work is enqueued on one persistent HIP stream in call order;
- *     ah_sync, ah_download and ah_event_elapsed_ms are the only blocking calls.
+ *     ah_sync, ah_download, ah_download_end and ah_event_elapsed_ms are the only blocking calls.
  *   - dtype codes: AH_F32 activations/params/grads, AH_BF16 internal fast-mode storage,
  *     AH_I32 indices, AH_F16 storage-only cast target (the reference's Dtype has no bf16:
  *     packages/core/src/types.ts:6).
@@ -64,6 +64,15 @@ int32_t ah_alloc(uint64_t bytes, ah_ptr *out);
 int32_t ah_free(ah_ptr p);
 int32_t ah_upload(ah_ptr dst, const void *host, uint64_t bytes);      /* host buffer borrowed for the call only */
 int32_t ah_download(void *host, ah_ptr src, uint64_t bytes);          /* blocks until data has landed */
+/* A read-back of at most 256 bytes in two halves, for a value that exists long before the host looks at it (the loss of a
+ * step, which the reference's trainer reads after it has issued the whole backward pass, trainer.ts:1247): _begin queues the
+ * copy into a pinned slot behind the work issued so far and returns a ticket; _end waits for THAT copy only - not for what
+ * was issued after it - and hands the bytes over.  Sixteen tickets are held; an older one is refused (AH_ERR_STATE), and the
+ * caller reads with ah_download instead.  Inside a step plan _begin is a boundary like ah_download; _end is none.  The
+ * reference's counterpart is its lazy read-back against a timeline value (packages/helios/src/backend.ts:1143-1171,
+ * helios_vk.c waitTimeline). */
+int32_t ah_download_begin(ah_ptr src, uint64_t bytes, uint64_t *out_ticket);
+int32_t ah_download_end(uint64_t ticket, void *host, uint64_t bytes);
 int32_t ah_copy(ah_ptr dst, ah_ptr src, uint64_t bytes);              /* device to device */
 int32_t ah_fill_f32(ah_ptr dst, float value, uint64_t n);
 int32_t ah_fill_i32(ah_ptr dst, int32_t value, uint64_t n);

@@ -115,3 +115,54 @@ def test_a_kick_is_a_boundary_of_the_plan(B):
     B.enableStepGraphs(False)
     assert hows[0] == "recorded" and hows[1] == hows[2] == "replayed", hows
     assert hows[3] == "fell-back" and hows[4] == "recorded" and hows[5] == "replayed", (hows, B.lastStepNote)
+
+
+def test_an_early_read_back_waits_for_its_own_copy_only(B):
+    """ah_download_begin / ah_download_end: the value is the one the tensor held when the copy was queued, whatever is issued
+    (and overwrites the tensor) afterwards; a ticket whose slot has been taken by sixteen newer ones is refused; inside a step
+    plan the pair gives the same values on recorded and replayed steps."""
+    import ctypes as C
+    from alpha2_amd import TensorData
+    from alpha2_amd._ffi import check
+    lib = B.lib
+    x = TensorData((64,), "f32", np.arange(64, dtype=np.float32))
+    p = B._ptr(x)
+
+    def begin(ptr, nbytes):
+        tk = C.c_uint64(0)
+        check(lib.ah_download_begin(ptr, nbytes, C.byref(tk)))
+        return tk.value
+
+    def end(tk, n):
+        out = np.empty(n, np.float32)
+        rc = lib.ah_download_end(tk, out.ctypes.data_as(C.c_void_p), out.nbytes)
+        return rc, out
+
+    tk = begin(p + 16, 32)
+    B.scaleInplace(x, 3.0)                                          # queued behind the copy: must not show in it
+    big = B.scale(TensorData((1 << 22,), "f32", np.ones(1 << 22, np.float32)), 2.0)
+    rc, got = end(tk, 8)
+    assert rc == 0 and np.array_equal(got, np.arange(4, 12, dtype=np.float32))
+    assert np.array_equal(x.data, 3 * np.arange(64, dtype=np.float32)) and float(big.data[5]) == 2.0
+    old = begin(p, 4)
+    for _ in range(16):
+        last = begin(p, 4)
+    assert end(old, 1)[0] != 0                                      # sixteen newer tickets took its slot
+    rc, got = end(last, 1)
+    assert rc == 0 and got[0] == 0.0
+    assert lib.ah_download_end(last, got.ctypes.data_as(C.c_void_p), 8) != 0      # another size than was copied
+
+    B.enableStepGraphs(True)
+    B.flush()
+    vals, hows = [], []
+    for s in range(4):
+        t = B.scale(x, float(s + 1))
+        tk = begin(B._ptr(t) + 4, 4)
+        t2 = B.scale(t, 10.0)
+        rc, got = end(tk, 1)
+        vals.append((rc, float(got[0]), float(t2.data[1])))
+        B.flush()
+        hows.append(B.lastStepHow)
+    B.enableStepGraphs(False)
+    assert vals == [(0, 3.0 * (s + 1), 30.0 * (s + 1)) for s in range(4)], vals
+    assert hows[0] == "recorded" and hows[-1] == "replayed", hows
