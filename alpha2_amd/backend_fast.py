@@ -65,6 +65,17 @@ class _HeldLayerNormBwd:
         self.rows, self.dim, self.eps, self.holds = rows, dim, eps, holds
 
 
+class _HeldCrossEntropy:
+    """A crossEntropy that has been asked for and not launched: if the next call on its logits is crossEntropyBackward (the
+    last entry of the tape is the first one its backward pass visits, tape.ts:60-157), loss and gradient come out of one pass
+    over the logits instead of two."""
+
+    def __init__(self, logits_ptr, targets_ptr, logits_buf, out, lse, n, c, holds):
+        self.logits_ptr, self.targets_ptr, self.logits_buf = logits_ptr, targets_ptr, logits_buf
+        self.out, self.out_buf, self.lse_buf = out, out._buf, lse._buf      # (the tensor itself only to hand it its read-back ticket)
+        self.n, self.c, self.holds = n, c, holds
+
+
 class _HeldScatter:
     """scatterSlice results that have been asked for and not written: column blocks of a [rows, cols] bf16 matrix that is zero
     elsewhere.  The tape adds the three blocks of d(qkv) to one another (ops.ts:816-858, tape.ts:116-127): sums of held scatters
@@ -102,6 +113,7 @@ class FastHipBackend(HipBackend):
         self._adam_bufs = set()          # id(_Buf) of every buffer a queued update reads or writes
         self._ssq_args = None            # (addresses, sizes, their ctypes arrays) of the last totalSumOfSquares call
         self._scatters = {}              # id(_Buf) of an unwritten scatterSlice result -> _HeldScatter
+        self._held_ce: Optional[_HeldCrossEntropy] = None
         self._held_ln: Optional[_HeldLayerNormBwd] = None
         # dx tensors whose LayerNorm backward went straight into a sum and that were never written themselves: id(_Buf) -> recipe
         self._ln_unwritten = {}
@@ -140,6 +152,8 @@ class FastHipBackend(HipBackend):
                 self._unhold(h.holds)
             if self._scatters and id(t._buf) in self._scatters:
                 self._write_scatter(t._buf)
+            if self._held_ce is not None and any(t._buf is b for b in self._held_ce.holds):
+                self._launch_ce()
             if self._held is not None and t._buf is self._held.out_buf:
                 self._launch_held()
             elif self._wgrads and (id(t._buf) in self._wq_out or id(t._buf) in self._wq_into):
@@ -587,26 +601,60 @@ class FastHipBackend(HipBackend):
         else:
             self._unhold(h.holds)
 
-    def crossEntropy(self, logits: TensorData, targets: TensorData) -> TensorData:
-        N, Cc = logits.shape
-        out, lse = self._new(()), self._new((N,))
-        check(self.lib.ah_cross_entropy(self._ptr(logits), ffi.DTYPE_CODE[logits.store], self._ptr(targets), out._buf.ptr, lse._buf.ptr, N, Cc))
-        logits._ce_lse = lse
+    def _early_loss(self, out: TensorData):
         # The reference's trainer reads the loss after it has issued the whole backward pass (trainer.ts:1247): the copy to the
-        # host starts now, and reading it later waits for this copy only, not for the backward pass.
+        # host starts as soon as the loss exists, and reading it later waits for this copy only, not for the backward pass.
+        if out._buf is None:
+            return
         tk = C.c_uint64(0)
         if self.lib.ah_download_begin(out._buf.ptr + out._off, 4, C.byref(tk)) == 0:
             out._early = tk.value
+
+    def _launch_ce(self):
+        """The held cross-entropy on its own (somebody needs the loss, or touches its operands, before any backward call)."""
+        h, self._held_ce = self._held_ce, None
+        if h is None:
+            return
+        if not (h.out_buf.refs == 1 and h.lse_buf.refs == 1):     # (both released unread otherwise)
+            check(self.lib.ah_cross_entropy(h.logits_ptr, BF16, h.targets_ptr, h.out_buf.ptr, h.lse_buf.ptr, h.n, h.c))
+            if h.out._buf is h.out_buf:
+                self._early_loss(h.out)
+        self._unhold(h.holds)
+
+    def crossEntropy(self, logits: TensorData, targets: TensorData) -> TensorData:
+        N, Cc = logits.shape
+        out, lse = self._new(()), self._new((N,))
+        self._launch_ce()
+        lp, tp = self._ptr(logits), self._ptr(targets)
+        logits._ce_lse = lse
+        if logits.store == "bf16" and N > 0 and Cc > 0:
+            self._held_ce = _HeldCrossEntropy(lp, tp, logits._buf, out, lse, N, Cc, self._hold(logits._buf, targets._buf, out._buf, lse._buf))
+            return out
+        check(self.lib.ah_cross_entropy(lp, ffi.DTYPE_CODE[logits.store], tp, out._buf.ptr, lse._buf.ptr, N, Cc))
+        self._early_loss(out)
         return out
 
     def crossEntropyBackward(self, logits, targets, gradOutput) -> TensorData:
+        h = self._held_ce
+        if h is not None and logits._buf is h.logits_buf and logits.store == "bf16" and tuple(logits.shape) == (h.n, h.c) \
+                and gradOutput._buf is not None and not any(gradOutput._buf is b for b in h.holds):
+            gp = self._ptr(gradOutput)
+            if self._held_ce is h:                              # (still held: loss, gradient and LSE in one pass over the logits)
+                self._held_ce = None
+                out = self._new((h.n, h.c), "f32", "bf16")
+                check(self.lib.ah_cross_entropy_fwd_bwd(h.logits_ptr, BF16, h.targets_ptr, h.out_buf.ptr, h.lse_buf.ptr, gp, 1.0,
+                                                        out._buf.ptr, h.n, h.c))
+                if h.out._buf is h.out_buf:
+                    self._early_loss(h.out)
+                self._unhold(h.holds)
+                return out
         lse = getattr(logits, "_ce_lse", None)
         if lse is None or lse._buf is None or logits.store != "bf16":
             self._f32(logits)
             return super().crossEntropyBackward(logits, targets, gradOutput)
         N, Cc = logits.shape
         out = self._new((N, Cc), "f32", "bf16")
-        check(self.lib.ah_cross_entropy_bwd(self._ptr(logits), BF16, self._ptr(targets), lse._buf.ptr, self._ptr(gradOutput), 1.0,
+        check(self.lib.ah_cross_entropy_bwd(self._ptr(logits), BF16, self._ptr(targets), self._ptr(lse), self._ptr(gradOutput), 1.0,
                                             out._buf.ptr, N, Cc))
         return out
 
@@ -711,6 +759,7 @@ class FastHipBackend(HipBackend):
     def flush(self):
         self._launch_held()
         self._launch_ln()
+        self._launch_ce()
         self._launch_weight_grads()
         self._flush_adam()
         super().flush()
@@ -718,6 +767,7 @@ class FastHipBackend(HipBackend):
     def syncGpu(self):
         self._launch_held()
         self._launch_ln()
+        self._launch_ce()
         self._launch_weight_grads()
         self._flush_adam()
         super().syncGpu()

@@ -332,3 +332,50 @@ def test_scattered_column_blocks_are_merged_before_they_are_written(FB):
     for t in (a, b, acc, s, s2):
         FB.releaseGpuTensor(t)
     assert not FB._scatters
+
+
+def test_cross_entropy_is_held_until_its_backward_is_asked_for(FB):
+    """crossEntropy followed by crossEntropyBackward on the same bf16 logits (the tape's last entry, visited first by its
+    backward pass) is one pass over the logits: loss, LSE and gradient bit-identical to the two-kernel route; a loss that is
+    read first, and one that is released unread, take the plain forward (or nothing)."""
+    rs = np.random.RandomState(17)
+    N, V = 96, 512
+    logits = _bf16(rs.randn(N, V) * 2)
+    targets = rs.randint(0, V, N).astype(np.int32)
+    lf = logits.astype(np.float64)
+    m = lf.max(1, keepdims=True)
+    lse = (m + np.log(np.exp(lf - m).sum(1, keepdims=True)))[:, 0]
+    want_loss = float(np.mean(lse - lf[np.arange(N), targets]))
+    p = np.exp(lf - lse[:, None])
+    p[np.arange(N), targets] -= 1
+    want_grad = p / N * 0.5
+
+    from alpha2_amd import TensorData
+
+    def operands():
+        return FB.castStore(_td(logits), "bf16"), TensorData(targets.shape, "i32", targets), _td(np.float32(0.5).reshape(()))
+
+    # fused: nothing is launched by crossEntropy itself
+    lg, tg, g = operands()
+    loss = FB.crossEntropy(lg, tg)
+    assert FB._held_ce is not None
+    grad = FB.crossEntropyBackward(lg, tg, g)
+    assert FB._held_ce is None
+    fused_loss, fused_grad = float(loss.data[0]), grad.data.copy()
+    assert abs(fused_loss - want_loss) <= 1e-5 * abs(want_loss)
+    assert np.all(np.abs(fused_grad.reshape(N, V) - want_grad) <= 2.0 ** -8 * np.abs(want_grad) + 1e-9)      # a bf16 result
+
+    # the loss read first: forward alone, then the backward kernel; same bits
+    lg, tg, g = operands()
+    loss = FB.crossEntropy(lg, tg)
+    plain_loss = float(loss.data[0])
+    assert FB._held_ce is None
+    plain_grad = FB.crossEntropyBackward(lg, tg, g).data.copy()
+    assert plain_loss == fused_loss and np.array_equal(plain_grad, fused_grad)
+
+    # released unread
+    lg, tg, g = operands()
+    loss = FB.crossEntropy(lg, tg)
+    FB.releaseGpuTensor(loss)
+    FB.flush()
+    assert FB._held_ce is None
