@@ -58,9 +58,14 @@ __global__ void k_adamw(float *__restrict__ p, const float *__restrict__ g, floa
 }
 
 // The same update for a LIST of tensors in one launch (the table is passed by value): block b works on one chunk of
-// AL_CHUNK elements of one tensor, found by bisection of the chunk offsets.  Element arithmetic = k_adamw's.
+// AL_CHUNK elements of one tensor, found by bisection of the chunk offsets.  Element arithmetic = k_adamw's.  One float4 per
+// thread: measured on the 101 tensors of the 163 M-parameter model, 855 us per pass against 876 / 914 / 962 with 2 / 4 / 16
+// iterations per thread (k_adamw on one contiguous array: 864).
 constexpr int AL_MAX = 48;
-constexpr uint64_t AL_CHUNK = uint64_t(1) << 14;
+#ifndef AL_CHUNK_LOG2
+#define AL_CHUNK_LOG2 10
+#endif
+constexpr uint64_t AL_CHUNK = uint64_t(1) << AL_CHUNK_LOG2;
 struct AdamList {
   float *p[AL_MAX];
   const float *g[AL_MAX];

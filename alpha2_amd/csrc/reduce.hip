@@ -78,7 +78,10 @@ __global__ void k_partial_sum(const float *__restrict__ a, uint64_t n, double *_
 // stage 1 for a LIST of tensors in one launch: block b sums the squares of one 64 K-element chunk of one tensor (the table is
 // passed by value; a block finds its tensor by bisection of the chunk offsets).  The partition depends on the sizes only.
 constexpr int SL_MAX = 120;
-constexpr uint64_t SL_CHUNK = uint64_t(1) << 16;
+#ifndef SL_CHUNK_LOG2
+#define SL_CHUNK_LOG2 14
+#endif
+constexpr uint64_t SL_CHUNK = uint64_t(1) << SL_CHUNK_LOG2;
 struct SumList {
   const float *x[SL_MAX];
   uint64_t n[SL_MAX];
@@ -96,7 +99,7 @@ __global__ void k_sum_sq_list(SumList L, double *__restrict__ partial) {
   const float *a = L.x[lo];
   const uint64_t n = L.n[lo], c0 = (uint64_t)(b - L.first[lo]) * SL_CHUNK, c1 = c0 + SL_CHUNK < n ? c0 + SL_CHUNK : n;
   double s = 0;
-  if ((((uintptr_t)a) & 15u) == 0) {                 // chunk starts are multiples of 64 K elements: as aligned as the tensor
+  if ((((uintptr_t)a) & 15u) == 0) {                 // chunk starts are multiples of SL_CHUNK elements: as aligned as the tensor
     const uint64_t q0 = c0 >> 2, q1 = c1 >> 2;
     for (uint64_t i = q0 + threadIdx.x; i < q1; i += blockDim.x) {
       float4 v = reinterpret_cast<const float4 *>(a)[i];

@@ -234,7 +234,7 @@ int32_t ah_argmax(ah_ptr a, ah_ptr out_i32, int64_t outer, int64_t dim, int64_t 
 int32_t ah_sum_sq(ah_ptr x, uint64_t n, ah_ptr out);
 /* The same over a list of tensors as ONE number: Backend.totalSumOfSquares (interfaces.ts:145), which the trainer calls on
  * the whole gradient set (trainer.ts:1345-1349).  One launch per 120 tensors plus one for the final sum, instead of three per
- * tensor; the partition into partial sums (chunks of 65536 elements per tensor) depends on the sizes only. */
+ * tensor; the partition into partial sums (chunks of 16384 elements per tensor) depends on the sizes only. */
 int32_t ah_sum_sq_list(const ah_ptr *xs, const uint64_t *ns, int32_t count, ah_ptr out);
 /* ah_sum_sq for callers that cannot allocate (code under HIP graph capture, tight serving loops, harnesses that forbid
  * hipMalloc): it has no counterpart in the reference.  Same kernels, same partition and so bit-identical results, but the
