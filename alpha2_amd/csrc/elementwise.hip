@@ -10,7 +10,10 @@ constexpr int TPB = 256;
 
 inline int grid_for(uint64_t work_items) {
   int64_t blocks = cdiv((int64_t)work_items, TPB);
-  int64_t cap = (int64_t)num_cus() * 16;
+#ifndef GRID_CAP_PER_CU
+#define GRID_CAP_PER_CU 1024      // (measured: gelu forward / backward on 50 M elements 66 / 102 us, against 72 / 119 us with 16 blocks per CU striding over the array)
+#endif
+  int64_t cap = (int64_t)num_cus() * GRID_CAP_PER_CU;
   if (blocks > cap) blocks = cap;
   if (blocks < 1) blocks = 1;
   return (int)blocks;
