@@ -567,7 +567,7 @@ __device__ __forceinline__ void online_merge(float &m, float &s, float m2, float
 template <class T>
 __global__ void k_ce_fwd(const T *__restrict__ logits, const int32_t *__restrict__ targets, float *__restrict__ row_loss,
                          float *__restrict__ lse_out, int64_t c) {
-  __shared__ float shm[WPB], shs[WPB];
+  __shared__ float shm[16], shs[16];                    // one pair per wave of the block (up to 1024 threads)
   int64_t row = blockIdx.x;
   const T *p = logits + row * c;
   float m = -INFINITY, s = 0.f;
@@ -599,7 +599,7 @@ __global__ void k_ce_fwd(const T *__restrict__ logits, const int32_t *__restrict
   if (lane == 0) { shm[wv] = m; shs[wv] = s; }
   __syncthreads();
   if (threadIdx.x == 0) {
-    for (int k = 1; k < WPB; k++) online_merge(m, s, shm[k], shs[k]);
+    for (int k = 1; k < (int)(blockDim.x >> 6); k++) online_merge(m, s, shm[k], shs[k]);
     float lse = m + logf(s);
     int32_t t = targets[row];
     float picked = (t >= 0 && t < c) ? Io<T>::ld(p, t) : lse;     // an out-of-range target contributes 0 loss
@@ -673,11 +673,15 @@ __global__ void k_ce_bwd(const T *__restrict__ logits, const int32_t *__restrict
 // Forward and backward of the loss in ONE pass over bf16 logits: the block keeps its whole row in registers (up to
 // CE_CHUNKS 16-byte chunks per thread), so the logits are read once instead of twice.  Same per-thread order of the online
 // (max, sum) updates and the same expressions as k_ce_fwd / k_ce_bwd: results are bit-identical to that pair.
-constexpr int CE_CHUNKS = 25;            // 25 x 256 threads x 8 classes = 51200 classes per row
-__global__ __launch_bounds__(256) void k_ce_fwd_bwd(const uint16_t *__restrict__ logits, const int32_t *__restrict__ targets,
+#ifndef CE_TPB
+#define CE_TPB 512        // measured at 16384 x 50304: 636 us with 512 threads per row, 670 with 256, 793 with 1024
+#endif
+constexpr int CE_CHUNKS = (51200 / 8 + CE_TPB - 1) / CE_TPB;      // CE_CHUNKS x CE_TPB threads x 8 classes >= 51200 classes per row
+constexpr int CE_WPB = CE_TPB / 64;
+__global__ __launch_bounds__(CE_TPB) void k_ce_fwd_bwd(const uint16_t *__restrict__ logits, const int32_t *__restrict__ targets,
                                                     float *__restrict__ row_loss, float *__restrict__ lse_out, const float *__restrict__ g,
                                                     float g_mul, uint16_t *__restrict__ out, int64_t n, int64_t c) {
-  __shared__ float shm[WPB], shs[WPB], sh_lse;
+  __shared__ float shm[CE_WPB], shs[CE_WPB], sh_lse;
   const int64_t row = blockIdx.x;
   const uint16_t *p = logits + row * c;
   const int nvec = (int)(c >> 3);
@@ -685,7 +689,7 @@ __global__ __launch_bounds__(256) void k_ce_fwd_bwd(const uint16_t *__restrict__
   float m = -INFINITY, s = 0.f;
 #pragma unroll
   for (int k = 0; k < CE_CHUNKS; k++) {
-    const int j = threadIdx.x + k * 256;
+    const int j = threadIdx.x + k * CE_TPB;
     if (j < nvec) {
       typedef unsigned u4v __attribute__((ext_vector_type(4)));     // 1.65 GB read once and written once: non-temporal (-6 %)
       const u4v un = __builtin_nontemporal_load(reinterpret_cast<const u4v *>(p) + j);
@@ -709,7 +713,7 @@ __global__ __launch_bounds__(256) void k_ce_fwd_bwd(const uint16_t *__restrict__
   __syncthreads();
   const int32_t t = targets[row];
   if (threadIdx.x == 0) {
-    for (int k = 1; k < WPB; k++) online_merge(m, s, shm[k], shs[k]);
+    for (int k = 1; k < CE_WPB; k++) online_merge(m, s, shm[k], shs[k]);
     const float lse = m + logf(s);
     const float picked = (t >= 0 && t < c) ? bf16_bits_to_f32(p[t]) : lse;     // an out-of-range target contributes 0 loss
     row_loss[row] = lse - picked;
@@ -721,7 +725,7 @@ __global__ __launch_bounds__(256) void k_ce_fwd_bwd(const uint16_t *__restrict__
   uint16_t *q = out + row * c;
 #pragma unroll
   for (int k = 0; k < CE_CHUNKS; k++) {
-    const int j8 = threadIdx.x + k * 256;
+    const int j8 = threadIdx.x + k * CE_TPB;
     if (j8 < nvec) {
       uint32_t o[4];
       ce_grad8(r[k], l, scale, j8 == (t >> 3) ? (int)(t & 7) : -1, o);
@@ -1027,7 +1031,7 @@ int32_t ah_cross_entropy(ah_ptr logits, int32_t dtype, ah_ptr targets, ah_ptr lo
   if (dtype == AH_F32)
     ah::launch_kernel(k_ce_fwd<float>, dim3((unsigned)n), dim3(TPB), 0, dp<const float>(logits), dp<const int32_t>(targets), rows, dp<float>(lse_out), c);
   else
-    ah::launch_kernel(k_ce_fwd<uint16_t>, dim3((unsigned)n), dim3(TPB), 0, dp<const uint16_t>(logits), dp<const int32_t>(targets), rows, dp<float>(lse_out), c);
+    ah::launch_kernel(k_ce_fwd<uint16_t>, dim3((unsigned)n), dim3(CE_TPB), 0, dp<const uint16_t>(logits), dp<const int32_t>(targets), rows, dp<float>(lse_out), c);
   AH_LAUNCH_CHECK();
   ah::launch_kernel(k_mean_rows, dim3(1), dim3(TPB), 0, rows, n, dp<float>(loss_out));
   AH_LAUNCH_CHECK();
@@ -1067,14 +1071,14 @@ int32_t ah_cross_entropy_fwd_bwd(ah_ptr logits, int32_t dtype, ah_ptr targets, a
   AH_ARG(n > 0 && c > 0, "ah_cross_entropy_fwd_bwd: empty logits [%lld, %lld]", (long long)n, (long long)c);
   AH_ARG(logits && targets && lse_out && dlogits, "ah_cross_entropy_fwd_bwd: null operand");
   AH_ARG(n < (int64_t(1) << 31), "ah_cross_entropy_fwd_bwd: too many rows");
-  const bool one_pass = dtype == AH_BF16 && (c & 7) == 0 && (c >> 3) <= (int64_t)CE_CHUNKS * 256 && ((logits | dlogits) & 15u) == 0;
+  const bool one_pass = dtype == AH_BF16 && (c & 7) == 0 && (c >> 3) <= (int64_t)CE_CHUNKS * CE_TPB && ((logits | dlogits) & 15u) == 0;
   if (!one_pass) {                // rows that do not fit the registers of a block, f32 logits, odd alignments: the two kernels
     int32_t rc = ah_cross_entropy(logits, dtype, targets, loss_out, lse_out, n, c);
     return rc ? rc : ah_cross_entropy_bwd(logits, dtype, targets, lse_out, g_scalar, g_mul, dlogits, n, c);
   }
   float *rows = (float *)scratch(sizeof(float) * (size_t)n);
   if (!rows) return fail(AH_ERR_OOM, "ah_cross_entropy_fwd_bwd: no scratch");
-  ah::launch_kernel(k_ce_fwd_bwd, dim3((unsigned)n), dim3(256), 0, dp<const uint16_t>(logits), dp<const int32_t>(targets), rows,
+  ah::launch_kernel(k_ce_fwd_bwd, dim3((unsigned)n), dim3(CE_TPB), 0, dp<const uint16_t>(logits), dp<const int32_t>(targets), rows,
                      dp<float>(lse_out), dp<const float>(g_scalar), g_mul, dp<uint16_t>(dlogits), n, c);
   AH_LAUNCH_CHECK();
   ah::launch_kernel(k_mean_rows, dim3(1), dim3(TPB), 0, rows, n, dp<float>(loss_out));
