@@ -102,7 +102,7 @@ class FastHipBackend(HipBackend):
         self._wgrads: List[_HeldWeightGrad] = []
         self._wq_out, self._wq_into = set(), set()   # id(_Buf) of the queued gradients' results / of the tensors they will be added into
         self._group = group_weight_grads
-        self._plans = {}                 # descriptor tuple -> grouped plan id
+        self._plans = {}                 # (epilogue, shapes) -> grouped plan id
         # products that became another op's epilogue and were never written themselves: computed only if somebody reads them
         self._orphans = {}               # id(_Buf) -> _HeldGemm
         # adamwStep calls of one optimizer pass, launched together (one kernel per 48 tensors) when anything needs their result
@@ -432,17 +432,21 @@ class FastHipBackend(HipBackend):
         for epi in (ffi.EPI_NONE, ffi.EPI_ACCUM):
             part = [d for d in descs if d.epilogue == epi]
             if groupable and len(part) > 1:
-                key = tuple((d.a, d.b, d.c, d.m, d.n, d.k) for d in part)
+                # one plan per list of shapes; the gradients are new tensors every step, so its tables are rewritten every time
+                # (also when nothing moved: a step plan wants the same launches from every step)
+                key = (epi,) + tuple((d.m, d.n, d.k) for d in part)
                 plan = self._plans.get(key)
+                arr = (ffi.AhGemm * len(part))(*part)
                 if plan is None:
-                    if len(self._plans) >= 8:                   # buffers moved: old plans will not be asked for again
+                    if len(self._plans) >= 8:
                         for p in self._plans.values():
                             check(self.lib.ah_gemm_grouped_destroy(p))
                         self._plans = {}
-                    arr = (ffi.AhGemm * len(part))(*part)
                     pid = C.c_uint64()
                     check(self.lib.ah_gemm_grouped_plan(arr, len(part), C.byref(pid)))
                     plan = self._plans[key] = pid.value
+                else:
+                    check(self.lib.ah_gemm_grouped_update(plan, arr, len(part)))
                 timed = getattr(self, "_timed", None)
                 if timed is None:
                     check(self.lib.ah_gemm_grouped_run(plan, epi))

@@ -318,7 +318,14 @@ struct JoinPart { float *c; float *ws; int M, N; int64_t ldc; };
 struct GroupPlan {
   ah_ptr table; int count, blocks, layout, out_dtype; bool live;
   ah_ptr parts, ws; int nparts;
+  int ndescs; int64_t ws_bytes;        // what ah_gemm_grouped_update checks a new descriptor list against:
+  std::vector<int64_t> shape;          // m, n, k, lda, ldb, ldc of every problem
 };
+std::vector<int64_t> group_shape(const AhGemm *descs, int count) {
+  std::vector<int64_t> v;
+  for (int i = 0; i < count; i++) { const AhGemm &q = descs[i]; v.insert(v.end(), {q.m, q.n, q.k, q.lda, q.ldb, q.ldc}); }
+  return v;
+}
 std::vector<GroupPlan> g_plans;      // plan id = index + 1
 
 // C += ws, ws = 0 for every k-split problem of a grouped launch: block (x, y) walks the float4s of part y.  The workspace
@@ -366,53 +373,51 @@ std::vector<int> split_tail(const AhGemm *descs, int count, int64_t blocks) {
 
 extern "C" {
 
-int32_t ah_gemm_grouped_plan(const AhGemm *descs, int32_t count, uint64_t *plan_out) {
-  AH_REQUIRE_READY();
-  AH_ARG(descs != nullptr && plan_out != nullptr && count > 0 && count <= 4096, "ah_gemm_grouped_plan: bad descriptor list (count %d)", count);
-  std::vector<GemmGroupEntry> tab((size_t)count);
+// Validates a descriptor list and builds the launch's tables from it: `tab` (one entry per problem, the problems of a short last
+// round as two entries each at the end) and `parts` (what k_grouped_join adds to what).  The second halves write consecutive
+// pieces of a workspace that starts at ws_base (0 while only its size, *ws_bytes, is wanted).
+static int32_t grouped_tables(const char *who, const AhGemm *descs, int32_t count, ah_ptr ws_base, std::vector<GemmGroupEntry> &tab,
+                              std::vector<JoinPart> &parts, int64_t *blocks_out, int64_t *ws_bytes) {
+  AH_ARG(descs != nullptr && count > 0 && count <= 4096, "%s: bad descriptor list (count %d)", who, count);
+  tab.assign((size_t)count, GemmGroupEntry{});
+  parts.clear();
   int64_t blocks = 0;
   const int layout = descs[0].layout, out_dtype = descs[0].out_dtype;
-  AH_ARG(layout >= AH_GEMM_NN && layout <= AH_GEMM_TN, "ah_gemm_grouped_plan: bad layout %d", layout);
-  AH_ARG(out_dtype == AH_F32 || out_dtype == AH_BF16, "ah_gemm_grouped_plan: output must be f32 or bf16");
+  AH_ARG(layout >= AH_GEMM_NN && layout <= AH_GEMM_TN, "%s: bad layout %d", who, layout);
+  AH_ARG(out_dtype == AH_F32 || out_dtype == AH_BF16, "%s: output must be f32 or bf16", who);
   const bool akm = layout == AH_GEMM_TN, bkm = layout != AH_GEMM_NT;
   const int osz = out_dtype == AH_F32 ? 4 : 2;
   for (int i = 0; i < count; i++) {
     const AhGemm &q = descs[i];
     if (q.layout != layout || q.out_dtype != out_dtype || q.in_dtype != AH_BF16 || q.batch != 1 ||
         (q.epilogue != AH_EPI_NONE && q.epilogue != AH_EPI_ACCUM))
-      return fail(AH_ERR_UNSUPPORTED, "ah_gemm_grouped_plan: problem %d: a group shares one layout and output type, takes bf16 operands, "
-                                      "batch 1 and the NONE / ACCUM epilogues", i);
+      return fail(AH_ERR_UNSUPPORTED, "%s: problem %d: a group shares one layout and output type, takes bf16 operands, "
+                                      "batch 1 and the NONE / ACCUM epilogues", who, i);
     AH_ARG(q.m > 0 && q.n > 0 && q.k >= 64 && q.k % 64 == 0 && q.m < (1ll << 31) && q.n < (1ll << 31) && q.k < (1ll << 31),
-           "ah_gemm_grouped_plan: problem %d: extents m=%lld n=%lld k=%lld (k must be a positive multiple of 64)", i, (long long)q.m,
+           "%s: problem %d: extents m=%lld n=%lld k=%lld (k must be a positive multiple of 64)", who, i, (long long)q.m,
            (long long)q.n, (long long)q.k);
-    AH_ARG(q.a != 0 && q.b != 0 && q.c != 0, "ah_gemm_grouped_plan: problem %d: null operand", i);
+    AH_ARG(q.a != 0 && q.b != 0 && q.c != 0, "%s: problem %d: null operand", who, i);
     int64_t a_cols = akm ? q.m : q.k, b_cols = bkm ? q.n : q.k;
     AH_ARG(q.lda >= a_cols && q.ldb >= b_cols && q.ldc >= q.n, "matmul shape mismatch: problem %d: lda/ldb/ldc too small", i);
     bool ok = aligned16(q.a) && aligned16(q.b) && q.lda % 8 == 0 && q.ldb % 8 == 0 && (!akm || q.m % 8 == 0) && (!bkm || q.n % 8 == 0) &&
               (q.c % (4 * osz)) == 0 && q.ldc % 4 == 0;
-    AH_ARG(ok, "ah_gemm_grouped_plan: problem %d: operands need 16-byte aligned rows and a vector-aligned C", i);
+    AH_ARG(ok, "%s: problem %d: operands need 16-byte aligned rows and a vector-aligned C", who, i);
     int64_t a_span = (akm ? (int64_t)64 : q.m) * q.lda * 2, b_span = (bkm ? (int64_t)64 : q.n) * q.ldb * 2;
-    AH_ARG(a_span < (1ll << 32) && b_span < (1ll << 32), "ah_gemm_grouped_plan: problem %d: operand spans more than 4 GiB", i);
-    AH_ARG(q.ldc < (1 << 22), "ah_gemm_grouped_plan: problem %d: ldc %lld too large (128 rows of C must span less than 2 GiB)", i, (long long)q.ldc);
+    AH_ARG(a_span < (1ll << 32) && b_span < (1ll << 32), "%s: problem %d: operand spans more than 4 GiB", who, i);
+    AH_ARG(q.ldc < (1 << 22), "%s: problem %d: ldc %lld too large (128 rows of C must span less than 2 GiB)", who, i, (long long)q.ldc);
     GemmGroupEntry &e = tab[(size_t)i];
     e.a = dp<const void>(q.a); e.b = dp<const void>(q.b); e.c = dp<void>(q.c);
     e.M = (int)q.m; e.N = (int)q.n; e.K = (int)q.k; e.tile_start = (int)blocks;
     e.lda = q.lda; e.ldb = q.ldb; e.ldc = q.ldc;
     blocks += cdiv(q.m, 256) * cdiv(q.n, 256);
-    AH_ARG(blocks < (1ll << 31), "ah_gemm_grouped_plan: too many tiles");
+    AH_ARG(blocks < (1ll << 31), "%s: too many tiles", who);
   }
   // the problems that make up a short last round are cut in two along k: they move to the end of the table as pairs of
   // entries, the second of which writes the workspace
-  GroupPlan plan{0, count, (int)blocks, layout, out_dtype, true, 0, 0, 0};
   const std::vector<int> chosen = split_tail(descs, count, blocks);
-  std::vector<JoinPart> parts;
-  int32_t rc = AH_OK;
+  *ws_bytes = 0;
   if (!chosen.empty()) {
-    int64_t ws_bytes = 0;
-    for (int i : chosen) ws_bytes += descs[i].m * descs[i].n * 4;
-    rc = ah_alloc((size_t)ws_bytes, &plan.ws);
-    if (rc) return rc;
-    rc = ah_fill_f32(plan.ws, 0.f, (uint64_t)(ws_bytes / 4));         // the workspace is all zero between runs (see k_grouped_join)
+    for (int i : chosen) *ws_bytes += descs[i].m * descs[i].n * 4;
     std::vector<GemmGroupEntry> cut_tab;
     std::vector<bool> cut((size_t)count, false);
     for (int i : chosen) cut[(size_t)i] = true;
@@ -424,7 +429,7 @@ int32_t ah_gemm_grouped_plan(const AhGemm *descs, int32_t count, uint64_t *plan_
     };
     for (int i = 0; i < count; i++)
       if (!cut[(size_t)i]) push(tab[(size_t)i]);
-    char *ws = dp<char>(plan.ws);
+    char *ws = dp<char>(ws_base);
     for (int i : chosen) {
       GemmGroupEntry lo = tab[(size_t)i], hi = lo;
       lo.K = hi.K = lo.K / 2;
@@ -438,9 +443,27 @@ int32_t ah_gemm_grouped_plan(const AhGemm *descs, int32_t count, uint64_t *plan_
       push(hi);
     }
     tab.swap(cut_tab);
-    plan.count = (int)tab.size();
-    plan.blocks = (int)nblocks;
-    plan.nparts = (int)parts.size();
+    blocks = nblocks;
+  }
+  *blocks_out = blocks;
+  return AH_OK;
+}
+
+int32_t ah_gemm_grouped_plan(const AhGemm *descs, int32_t count, uint64_t *plan_out) {
+  AH_REQUIRE_READY();
+  AH_ARG(plan_out != nullptr, "ah_gemm_grouped_plan: null plan_out");
+  std::vector<GemmGroupEntry> tab;
+  std::vector<JoinPart> parts;
+  int64_t blocks = 0, ws_bytes = 0;
+  int32_t rc = grouped_tables("ah_gemm_grouped_plan", descs, count, 0, tab, parts, &blocks, &ws_bytes);      // sizes first
+  if (rc) return rc;
+  GroupPlan plan{0, (int)tab.size(), (int)blocks, descs[0].layout, descs[0].out_dtype, true, 0, 0, (int)parts.size(), count, ws_bytes,
+                 group_shape(descs, count)};
+  if (ws_bytes > 0) {
+    rc = ah_alloc((size_t)ws_bytes, &plan.ws);
+    if (rc) return rc;
+    rc = ah_fill_f32(plan.ws, 0.f, (uint64_t)(ws_bytes / 4));           // the workspace is all zero between runs (see k_grouped_join)
+    if (rc == AH_OK) rc = grouped_tables("ah_gemm_grouped_plan", descs, count, plan.ws, tab, parts, &blocks, &ws_bytes);
     if (rc == AH_OK) rc = ah_alloc(parts.size() * sizeof(JoinPart), &plan.parts);
     if (rc == AH_OK) rc = ah_upload(plan.parts, parts.data(), parts.size() * sizeof(JoinPart));
   }
@@ -455,6 +478,25 @@ int32_t ah_gemm_grouped_plan(const AhGemm *descs, int32_t count, uint64_t *plan_
   g_plans.push_back(plan);
   *plan_out = g_plans.size();
   return AH_OK;
+}
+
+int32_t ah_gemm_grouped_update(uint64_t plan, const AhGemm *descs, int32_t count) {
+  AH_REQUIRE_READY();
+  AH_ARG(plan >= 1 && plan <= g_plans.size() && g_plans[plan - 1].live, "ah_gemm_grouped_update: unknown plan %llu", (unsigned long long)plan);
+  const GroupPlan &p = g_plans[plan - 1];
+  std::vector<GemmGroupEntry> tab;
+  std::vector<JoinPart> parts;
+  int64_t blocks = 0, ws_bytes = 0;
+  int32_t rc = grouped_tables("ah_gemm_grouped_update", descs, count, p.ws, tab, parts, &blocks, &ws_bytes);
+  if (rc) return rc;
+  if (count != p.ndescs || descs[0].layout != p.layout || descs[0].out_dtype != p.out_dtype || (int)tab.size() != p.count ||
+      (int)blocks != p.blocks || (int)parts.size() != p.nparts || ws_bytes != p.ws_bytes || group_shape(descs, count) != p.shape)
+    return fail(AH_ERR_ARG, "ah_gemm_grouped_update: the problems do not have the shapes the plan was made for");
+  if (!parts.empty()) {
+    rc = ah_upload(p.parts, parts.data(), parts.size() * sizeof(JoinPart));
+    if (rc) return rc;
+  }
+  return ah_upload(p.table, tab.data(), tab.size() * sizeof(GemmGroupEntry));
 }
 
 int32_t ah_gemm_grouped_run(uint64_t plan, int32_t epilogue) {

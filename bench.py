@@ -105,9 +105,9 @@ def main():
         print("bench.py: this build runs the step on ONE GPU; --gpus must be 1 (no multi-GPU path exists in this run)", file=sys.stderr)
         sys.exit(2)
     if args.mode == "backend" and not args.no_step_graphs:
-        # a step plan takes up to five steps to settle: one eager step, one recorded, and - when the recorded step's buffers
-        # were not yet at their steady addresses - one replayed, one that falls back and one recorded again
-        args.warmup = max(args.warmup, 6)
+        # a step plan takes a few steps to settle: one eager step, one recorded, and a first replay that rewrites the nodes
+        # whose buffers were not yet at their steady addresses when the step was recorded
+        args.warmup = max(args.warmup, 4)
 
     from alpha2_amd import FastHipBackend, HipBackend
     from alpha2_amd.model import ModelConfig

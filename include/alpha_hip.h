@@ -360,6 +360,10 @@ int32_t ah_gemm(const AhGemm *g);
  * second kernel in a fixed order), which halves the cost of that round; ah_gemm_last_kernel then reports 2 slices. */
 int32_t ah_gemm_grouped_plan(const AhGemm *descs, int32_t count, uint64_t *plan_out);
 int32_t ah_gemm_grouped_run(uint64_t plan, int32_t epilogue);
+/* The same problems at other addresses (a caller whose gradient buffers are new tensors every step: the tape's weight
+ * gradients, packages/autograd/src/ops.ts:197-234): rewrites the plan's device tables from a descriptor list with the shapes
+ * the plan was made for, without allocating.  Two small uploads; a list of other shapes is refused. */
+int32_t ah_gemm_grouped_update(uint64_t plan, const AhGemm *descs, int32_t count);
 int32_t ah_gemm_grouped_destroy(uint64_t plan);
 /* Profiling aid (no counterpart in the reference): writes the name of the kernel the most recent ah_gemm call
  * launched, spelled as a profiler demangles it (e.g. "k_gemm_bf16<256, 256, 2, 4, false, false>"), and the number

@@ -1048,7 +1048,33 @@ def test_gemm_grouped_last_round_cut_in_two_along_k(B, shapes, K, cut):
         for out, want, (m, n) in zip(outs, wants, shapes):
             B._dirty(out)
             assert_close(out.data.reshape(m, n), run * want, rel=1e-4, what=f"ACCUM {m}x{n}")
+    # the same problems at other addresses (operands swapped in from fresh tensors, results into fresh tensors): the plan's
+    # tables are rewritten in place; a list of other shapes is refused
+    outs2, descs2 = [], []
+    for d, (m, n) in zip(descs, shapes):
+        src_g = TensorData((K, m), "f16", np.zeros(K * m, np.uint16))
+        src_x = TensorData((K, n), "f16", np.zeros(K * n, np.uint16))
+        ffi.check(B.lib.ah_copy(B._ptr(src_g), d.a, K * m * 2))
+        ffi.check(B.lib.ah_copy(B._ptr(src_x), d.b, K * n * 2))
+        out = B.zeros((m, n))
+        keep += [src_g, src_x]
+        outs2.append(out)
+        descs2.append(ffi.AhGemm(ffi.GEMM_TN, ffi.BF16, ffi.F32, ffi.EPI_NONE, m, n, K, m, n, n, 1, 0, 0, 0, B._ptr(src_g), B._ptr(src_x), B._ptr(out), 0))
+    arr2 = (ffi.AhGemm * len(descs2))(*descs2)
+    ffi.check(B.lib.ah_gemm_grouped_update(plan.value, arr2, len(descs2)))
+    ffi.check(B.lib.ah_gemm_grouped_run(plan.value, ffi.EPI_NONE))
+    for i, (out, (m, n)) in enumerate(zip(outs2, shapes)):
+        B._dirty(out)
+        assert np.array_equal(out.data.reshape(m, n), first[i]), f"{m}x{n}: after the update"
+    for out, want, (m, n) in zip(outs, wants, shapes):    # the old results were not touched by the run after the update
+        B._dirty(out)
+        assert_close(out.data.reshape(m, n), 3 * want, rel=1e-4, what=f"old C {m}x{n}")
+    other = (ffi.AhGemm * len(descs2))(*descs2)
+    other[0].k = K + 64
+    assert B.lib.ah_gemm_grouped_update(plan.value, other, len(descs2)) != 0 and b"shapes the plan was made for" in B.lib.ah_last_error()
+    assert B.lib.ah_gemm_grouped_update(plan.value, arr2, len(descs2) - 1) != 0
     ffi.check(B.lib.ah_gemm_grouped_destroy(plan.value))
+    assert B.lib.ah_gemm_grouped_update(plan.value, arr2, len(descs2)) != 0 and b"unknown plan" in B.lib.ah_last_error()
 
 
 # ---------------------------------------------------------------------------------------------- parity at the benchmark sizes
