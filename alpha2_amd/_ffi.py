@@ -128,6 +128,7 @@ SIGNATURES = {
     "ah_gemm": [C.POINTER(AhGemm)],
     "ah_gemm_grouped_plan": [C.POINTER(AhGemm), C.c_int32, C.POINTER(C.c_uint64)],
     "ah_gemm_grouped_run": [u64, i32],
+    "ah_gemm_grouped_run_sumsq": [u64, i32, u64],
     "ah_gemm_grouped_update": [u64, C.POINTER(AhGemm), C.c_int32],
     "ah_gemm_grouped_destroy": [u64],
     "ah_gemm_last_kernel": [C.c_char_p, C.c_int32, C.POINTER(C.c_int32)],

@@ -318,6 +318,7 @@ struct JoinPart { float *c; float *ws; int M, N; int64_t ldc; };
 struct GroupPlan {
   ah_ptr table; int count, blocks, layout, out_dtype; bool live;
   ah_ptr parts, ws; int nparts;
+  ah_ptr sumsq;                        // 4 floats per block of the launch, then JOIN_BLOCKS per k-split problem (ah_gemm_grouped_run_sumsq)
   int ndescs; int64_t ws_bytes;        // what ah_gemm_grouped_update checks a new descriptor list against:
   std::vector<int64_t> shape;          // m, n, k, lda, ldb, ldc of every problem
 };
@@ -331,10 +332,14 @@ std::vector<GroupPlan> g_plans;      // plan id = index + 1
 // C += ws, ws = 0 for every k-split problem of a grouped launch: block (x, y) walks the float4s of part y.  The workspace
 // is left all zero, so the second halves of an ACCUMULATING run (whose epilogue adds to what it finds) store into it just
 // as those of a plain run do.
-__global__ __launch_bounds__(256) void k_grouped_join(const JoinPart *__restrict__ parts) {
+constexpr int JOIN_BLOCKS = 128;     // blocks per k-split problem
+// With SUMSQ, block (x, y) also leaves the sum of the squares of the sums it stored in sumsq[JOIN_BLOCKS y + x].
+template <bool SUMSQ>
+__global__ __launch_bounds__(256) void k_grouped_join(const JoinPart *__restrict__ parts, float *__restrict__ sumsq) {
   const JoinPart p = parts[blockIdx.y];
   const int nq = p.N >> 2;
   const int64_t total = (int64_t)p.M * nq;
+  float ss = 0.f;
   for (int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x; q < total; q += (int64_t)gridDim.x * 256) {
     const int64_t row = q / nq;
     const int col = (int)(q - row * nq) * 4;
@@ -344,7 +349,29 @@ __global__ __launch_bounds__(256) void k_grouped_join(const JoinPart *__restrict
     v.x += w.x; v.y += w.y; v.z += w.z; v.w += w.w;
     *dst = v;
     *src = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (SUMSQ) ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
   }
+  if (SUMSQ) {
+    __shared__ float part[4];
+    ss = ah::wave_sum(ss);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    if (threadIdx.x == 0) sumsq[blockIdx.y * JOIN_BLOCKS + blockIdx.x] = (part[0] + part[1]) + (part[2] + part[3]);
+  }
+}
+
+// *inout += the sum of the n partial sums, added up in f64 in an order that depends on n only.
+__global__ __launch_bounds__(256) void k_grouped_sumsq_final(const float *__restrict__ partial, int n, float *__restrict__ inout) {
+  __shared__ double sh[256];
+  double t = 0.0;
+  for (int i = threadIdx.x; i < n; i += 256) t += (double)partial[i];
+  sh[threadIdx.x] = t;
+  __syncthreads();
+  for (int w = 128; w > 0; w >>= 1) {
+    if ((int)threadIdx.x < w) sh[threadIdx.x] += sh[threadIdx.x + w];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) *inout = (float)((double)*inout + sh[0]);
 }
 
 constexpr int GROUP_ROUND = 256;     // tiles that run at a time: one per CU
@@ -433,6 +460,7 @@ static int32_t grouped_tables(const char *who, const AhGemm *descs, int32_t coun
     for (int i : chosen) {
       GemmGroupEntry lo = tab[(size_t)i], hi = lo;
       lo.K = hi.K = lo.K / 2;
+      lo.partial = hi.partial = 1;
       hi.a = (const char *)lo.a + (akm ? (int64_t)lo.K * lo.lda : (int64_t)lo.K) * 2;
       hi.b = (const char *)lo.b + (bkm ? (int64_t)lo.K * lo.ldb : (int64_t)lo.K) * 2;
       hi.c = ws;
@@ -457,7 +485,7 @@ int32_t ah_gemm_grouped_plan(const AhGemm *descs, int32_t count, uint64_t *plan_
   int64_t blocks = 0, ws_bytes = 0;
   int32_t rc = grouped_tables("ah_gemm_grouped_plan", descs, count, 0, tab, parts, &blocks, &ws_bytes);      // sizes first
   if (rc) return rc;
-  GroupPlan plan{0, (int)tab.size(), (int)blocks, descs[0].layout, descs[0].out_dtype, true, 0, 0, (int)parts.size(), count, ws_bytes,
+  GroupPlan plan{0, (int)tab.size(), (int)blocks, descs[0].layout, descs[0].out_dtype, true, 0, 0, (int)parts.size(), 0, count, ws_bytes,
                  group_shape(descs, count)};
   if (ws_bytes > 0) {
     rc = ah_alloc((size_t)ws_bytes, &plan.ws);
@@ -469,7 +497,9 @@ int32_t ah_gemm_grouped_plan(const AhGemm *descs, int32_t count, uint64_t *plan_
   }
   if (rc == AH_OK) rc = ah_alloc(tab.size() * sizeof(GemmGroupEntry), &plan.table);
   if (rc == AH_OK) rc = ah_upload(plan.table, tab.data(), tab.size() * sizeof(GemmGroupEntry));
+  if (rc == AH_OK && plan.out_dtype == AH_F32) rc = ah_alloc(((size_t)blocks * 4 + parts.size() * JOIN_BLOCKS) * sizeof(float), &plan.sumsq);
   if (rc) {
+    if (plan.sumsq) ah_free(plan.sumsq);
     if (plan.ws) ah_free(plan.ws);
     if (plan.parts) ah_free(plan.parts);
     if (plan.table) ah_free(plan.table);
@@ -499,23 +529,41 @@ int32_t ah_gemm_grouped_update(uint64_t plan, const AhGemm *descs, int32_t count
   return ah_upload(p.table, tab.data(), tab.size() * sizeof(GemmGroupEntry));
 }
 
-int32_t ah_gemm_grouped_run(uint64_t plan, int32_t epilogue) {
+// The launches of a plan; with sumsq_inout also the sum of the squares of everything they leave in the C matrices.
+static int32_t grouped_run(const char *who, uint64_t plan, int32_t epilogue, ah_ptr sumsq_inout) {
   AH_REQUIRE_READY();
-  AH_ARG(plan >= 1 && plan <= g_plans.size() && g_plans[plan - 1].live, "ah_gemm_grouped_run: unknown plan %llu", (unsigned long long)plan);
+  AH_ARG(plan >= 1 && plan <= g_plans.size() && g_plans[plan - 1].live, "%s: unknown plan %llu", who, (unsigned long long)plan);
   const GroupPlan &p = g_plans[plan - 1];
-  AH_ARG(epilogue == AH_EPI_NONE || (epilogue == AH_EPI_ACCUM && p.out_dtype == AH_F32), "ah_gemm_grouped_run: epilogue %d is not provided for this plan", epilogue);
+  AH_ARG(epilogue == AH_EPI_NONE || (epilogue == AH_EPI_ACCUM && p.out_dtype == AH_F32), "%s: epilogue %d is not provided for this plan", who, epilogue);
+  const bool sums = sumsq_inout != 0;
+  if (sums && p.out_dtype != AH_F32) return fail(AH_ERR_UNSUPPORTED, "%s: the sum of squares is provided for f32 outputs", who);
   const GemmGroupEntry *tab = dp<const GemmGroupEntry>(p.table);
+  float *ss = sums ? dp<float>(p.sumsq) : nullptr;
   int32_t rc;
   switch (p.layout) {
-    case AH_GEMM_NT: rc = gemm_bf16_dma_nt_grouped(tab, p.count, p.blocks, epilogue, p.out_dtype); break;
-    case AH_GEMM_NN: rc = gemm_bf16_dma_nn_grouped(tab, p.count, p.blocks, epilogue, p.out_dtype); break;
-    default: rc = gemm_bf16_dma_tn_grouped(tab, p.count, p.blocks, epilogue, p.out_dtype);
+    case AH_GEMM_NT: rc = gemm_bf16_dma_nt_grouped(tab, p.count, p.blocks, epilogue, p.out_dtype, ss); break;
+    case AH_GEMM_NN: rc = gemm_bf16_dma_nn_grouped(tab, p.count, p.blocks, epilogue, p.out_dtype, ss); break;
+    default: rc = gemm_bf16_dma_tn_grouped(tab, p.count, p.blocks, epilogue, p.out_dtype, ss);
   }
-  if (rc != AH_OK || p.nparts == 0) return rc;
-  ah::launch_kernel(k_grouped_join, dim3(128, (unsigned)p.nparts), dim3(256), 0, dp<const JoinPart>(p.parts));
-  AH_LAUNCH_CHECK();
-  ah::note_gemm_split(2);
+  if (rc != AH_OK) return rc;
+  if (p.nparts > 0) {
+    if (sums) ah::launch_kernel(k_grouped_join<true>, dim3(JOIN_BLOCKS, (unsigned)p.nparts), dim3(256), 0, dp<const JoinPart>(p.parts), ss + (size_t)p.blocks * 4);
+    else ah::launch_kernel(k_grouped_join<false>, dim3(JOIN_BLOCKS, (unsigned)p.nparts), dim3(256), 0, dp<const JoinPart>(p.parts), (float *)nullptr);
+    AH_LAUNCH_CHECK();
+    ah::note_gemm_split(2);
+  }
+  if (sums) {
+    ah::launch_kernel(k_grouped_sumsq_final, dim3(1), dim3(256), 0, (const float *)ss, p.blocks * 4 + p.nparts * JOIN_BLOCKS, dp<float>(sumsq_inout));
+    AH_LAUNCH_CHECK();
+  }
   return AH_OK;
+}
+
+int32_t ah_gemm_grouped_run(uint64_t plan, int32_t epilogue) { return grouped_run("ah_gemm_grouped_run", plan, epilogue, 0); }
+
+int32_t ah_gemm_grouped_run_sumsq(uint64_t plan, int32_t epilogue, ah_ptr sumsq_inout) {
+  AH_ARG(sumsq_inout != 0 && sumsq_inout % 4 == 0, "ah_gemm_grouped_run_sumsq: sumsq_inout must be an f32 on the device");
+  return grouped_run("ah_gemm_grouped_run_sumsq", plan, epilogue, sumsq_inout);
 }
 
 int32_t ah_gemm_grouped_destroy(uint64_t plan) {
@@ -523,6 +571,8 @@ int32_t ah_gemm_grouped_destroy(uint64_t plan) {
   AH_ARG(plan >= 1 && plan <= g_plans.size() && g_plans[plan - 1].live, "ah_gemm_grouped_destroy: unknown plan %llu", (unsigned long long)plan);
   GroupPlan &p = g_plans[plan - 1];
   p.live = false;
+  if (p.sumsq) ah_free(p.sumsq);
+  p.sumsq = 0;
   if (p.nparts > 0) {
     ah_free(p.parts);
     ah_free(p.ws);
@@ -572,6 +622,7 @@ int32_t ah_gemm(const AhGemm *p) {
   ga.sa = q.stride_a; ga.sb = q.stride_b; ga.sc = q.stride_c;
   ga.epi = q.epilogue;
   ga.ksplit = (int)q.k; ga.nsplit = 1;
+  ga.sumsq = nullptr;
   int batch = (int)q.batch;
 
   // 4-wide epilogue accesses need 16-byte (f32) / 8-byte (bf16) aligned rows of C and aux

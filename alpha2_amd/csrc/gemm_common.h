@@ -10,6 +10,7 @@ struct GemmGroupEntry {
   const void *a, *b;
   void *c;
   int M, N, K, tile_start;      // tile_start: first block id of this problem
+  int partial, pad_;            // partial: what the entry stores is one half of a k-split product, not the final C
   int64_t lda, ldb, ldc;
 };
 
@@ -27,6 +28,7 @@ struct GemmArgs {
   int64_t sa, sb, sc;  // batch strides (elements)
   int epi;
   int ksplit, nsplit;  // split-K (bf16 direct kernel only): K elements per split, number of splits (1 = off)
+  float *sumsq;        // grouped launches that also sum the squares of what they store: the block's four slots (one per wave)
 };
 
 // Epilogue for 4 consecutive columns (col..col+3) of one row: the MFMA operands are swapped (acc = B-frag x A-frag)
@@ -147,9 +149,11 @@ struct EpiStage { char *p[4]; };
 // row past the end of C is then out of the descriptor's range, a lane in a column past the end is given an offset that
 // always is.  The loads run ahead: vmcnt retires in issue order, stores included, so the reads of pass p + DEPTH are issued
 // before the stores of pass p.  Requires N % 4 == 0 and 128 rows of C to span less than 2 GiB.
-template <int EPI, class OUT, int TM, int TN>
-__device__ __forceinline__ void store_tiles_lds(const GemmArgs &g, int64_t cbase, int row0, int col0, int lane, const f32x16 (&acc)[TM][TN],
-                                                const EpiStage &st) {
+// With SUMSQ the lane also adds up the squares of the values it stores (those the address unit drops count as zero) and
+// returns the sum.
+template <int EPI, class OUT, int TM, int TN, bool SUMSQ = false>
+__device__ __forceinline__ float store_tiles_lds(const GemmArgs &g, int64_t cbase, int row0, int col0, int lane, const f32x16 (&acc)[TM][TN],
+                                                 const EpiStage &st) {
   constexpr bool F32OUT = sizeof(OUT) == 4;
   constexpr int JP = F32OUT ? 1 : 2;                  // 32 x 32 tiles per pass: a row of the pass is 128 bytes of output
   constexpr int NJP = (TN + JP - 1) / JP, NPASS = TM * NJP;
@@ -175,6 +179,7 @@ __device__ __forceinline__ void store_tiles_lds(const GemmArgs &g, int64_t cbase
   for (int q = 0; q < 4; q++) wofs[q] = lr * 128 + (((2 * q + lk) ^ (lr & 7)) << 4);
 
   AuxT pre[DEPTH][8];
+  float ss = 0.f;
   // element offset (uniform) of the first row and column of iteration `it` of pass p, and this lane's part for the pass
   auto group_el = [&](int p, int it) -> int {
     const int i = p / NJP, j0 = (p % NJP) * JP, ns = TN - j0 < JP ? TN - j0 : JP;
@@ -237,6 +242,11 @@ __device__ __forceinline__ void store_tiles_lds(const GemmArgs &g, int64_t cbase
         for (int e = 0; e < 4; e++) v[e] = gelu_f(v[e]);
       }
       buffer_store4<EPI == EPI_PLAIN_STREAMED ? 2 : 0>(v[0], v[1], v[2], v[3], (OUT *)nullptr, buffer_window(c + ge * ES, (span - ge) * ES), le);
+      if (SUMSQ) {      // the address unit's own test: the lane's 4 elements end inside the window
+        const bool stored = le != OUTSIDE && (int)(ns == 2 ? lane_el2 : lane_el1) + 4 <= span - ge;
+        const float q = v[0] * v[0] + v[1] * v[1] + v[2] * v[2] + v[3] * v[3];
+        ss += stored ? q : 0.f;
+      }
     }
     __builtin_amdgcn_sched_barrier(0);
     if (READS && p + DEPTH < NPASS) {
@@ -244,6 +254,7 @@ __device__ __forceinline__ void store_tiles_lds(const GemmArgs &g, int64_t cbase
       __builtin_amdgcn_sched_barrier(0);
     }
   }
+  return ss;
 }
 
 // Stores a wave's TM x TN grid of 32x32 accumulators (C^T orientation: 4 consecutive registers = 4 consecutive columns).
@@ -272,8 +283,9 @@ int32_t splitk_reduce(const float *ws, float *c, int nsplit, int M, int N, int64
 int32_t gemm_bf16_dma_nt(const GemmArgs &ga, int batch, int out_dtype, int bn);
 int32_t gemm_bf16_dma_nn(const GemmArgs &ga, int batch, int out_dtype, int bn);
 int32_t gemm_bf16_dma_tn(const GemmArgs &ga, int batch, int out_dtype, int bn);
-int32_t gemm_bf16_dma_nt_grouped(const GemmGroupEntry *tab, int count, int blocks, int epi, int out_dtype);
-int32_t gemm_bf16_dma_nn_grouped(const GemmGroupEntry *tab, int count, int blocks, int epi, int out_dtype);
-int32_t gemm_bf16_dma_tn_grouped(const GemmGroupEntry *tab, int count, int blocks, int epi, int out_dtype);
+// sumsq (f32 outputs only, or null): 4 floats per block, the sums of the squares of what each wave stored as final values of C
+int32_t gemm_bf16_dma_nt_grouped(const GemmGroupEntry *tab, int count, int blocks, int epi, int out_dtype, float *sumsq);
+int32_t gemm_bf16_dma_nn_grouped(const GemmGroupEntry *tab, int count, int blocks, int epi, int out_dtype, float *sumsq);
+int32_t gemm_bf16_dma_tn_grouped(const GemmGroupEntry *tab, int count, int blocks, int epi, int out_dtype, float *sumsq);
 
 }  // namespace ah

@@ -360,6 +360,13 @@ int32_t ah_gemm(const AhGemm *g);
  * second kernel in a fixed order), which halves the cost of that round; ah_gemm_last_kernel then reports 2 slices. */
 int32_t ah_gemm_grouped_plan(const AhGemm *descs, int32_t count, uint64_t *plan_out);
 int32_t ah_gemm_grouped_run(uint64_t plan, int32_t epilogue);
+/* ah_gemm_grouped_run of an f32 plan that also adds, to the f32 at sumsq_inout, the sum of the squares of every value the
+ * run leaves in the C matrices (after ACCUM: of the accumulated values): the weight gradients' share of the norm that
+ * Backend.totalSumOfSquares (interfaces.ts:145; trainer.ts:1345-1349) computes by reading every gradient again.  The
+ * squares are taken in the epilogue, from the registers that are being stored, summed per wave in f32 and over the waves
+ * in f64 in an order that depends on the plan only (same result from run to run).  Four floats per 256 x 256 tile of
+ * scratch, which the plan owns. */
+int32_t ah_gemm_grouped_run_sumsq(uint64_t plan, int32_t epilogue, ah_ptr sumsq_inout);
 /* The same problems at other addresses (a caller whose gradient buffers are new tensors every step: the tape's weight
  * gradients, packages/autograd/src/ops.ts:197-234): rewrites the plan's device tables from a descriptor list with the shapes
  * the plan was made for, without allocating.  Two small uploads; a list of other shapes is refused. */

@@ -1008,6 +1008,70 @@ def test_gemm_grouped_matches_separate_products(B):
     assert B.lib.ah_gemm_grouped_plan(bad, 1, C.byref(plan)) != 0 and b"multiple of 64" in B.lib.ah_last_error()
 
 
+@pytest.mark.parametrize("shapes,K", [
+    ([(768, 768), (264, 520), (2304, 768), (8, 8), (1000, 256)], 640),      # ragged edges in both directions, every problem cut in two along k
+    ([(4096, 4096), (768, 768), (1280, 1792)], 256),                         # the last round is cut, the first problem is not
+    ([(3072, 3072), (768, 768)], 128),                                       # no cut
+])
+def test_gemm_grouped_sum_of_squares_of_what_it_stores(B, shapes, K):
+    """ah_gemm_grouped_run_sumsq leaves the same matrices as ah_gemm_grouped_run, bit for bit, and adds the sum of their
+    squares (after ACCUM: of the accumulated values) to the number it is given; the first problem's C is a column block
+    of a wider matrix, whose other columns are neither counted nor touched.  The same run twice gives the same number."""
+    import ctypes as C
+    from alpha2_amd import TensorData, _ffi as ffi
+    keep, descs, outs, lds = [], [], [], []
+    for i, (m, n) in enumerate(shapes):
+        gy, x = _bf16_round(rs.randn(K, m).astype(np.float32))[0], _bf16_round(rs.randn(K, n).astype(np.float32))[0]
+        tg, tx = TensorData(gy.shape, "f16", _bf16_round(gy)[1]), TensorData(x.shape, "f16", _bf16_round(x)[1])
+        ldc = n + 8 if i == 0 else n
+        out = TensorData((m, ldc), "f32", np.full(m * ldc, 7.0, np.float32))
+        keep += [tg, tx]
+        outs.append(out)
+        lds.append(ldc)
+        descs.append(ffi.AhGemm(ffi.GEMM_TN, ffi.BF16, ffi.F32, ffi.EPI_NONE, m, n, K, m, n, ldc, 1, 0, 0, 0, B._ptr(tg), B._ptr(tx), B._ptr(out), 0))
+    arr = (ffi.AhGemm * len(descs))(*descs)
+    plan = C.c_uint64()
+    ffi.check(B.lib.ah_gemm_grouped_plan(arr, len(descs), C.byref(plan)))
+
+    def read():
+        got = []
+        for out, (m, n), ldc in zip(outs, shapes, lds):
+            B._dirty(out)
+            full = out.data.reshape(m, ldc).copy()
+            assert np.all(full[:, n:] == 7.0), "columns outside C were written"
+            got.append(full[:, :n])
+        return got
+    ffi.check(B.lib.ah_gemm_grouped_run(plan.value, ffi.EPI_NONE))
+    plain = read()
+    ffi.check(B.lib.ah_gemm_grouped_run(plan.value, ffi.EPI_ACCUM))
+    plain2 = read()
+    for epi, want_c in ((ffi.EPI_NONE, plain), (ffi.EPI_ACCUM, plain2)):
+        numbers = []
+        for rep in range(2):
+            if epi == ffi.EPI_ACCUM:                                          # back to the state the accumulating run started from
+                ffi.check(B.lib.ah_gemm_grouped_run(plan.value, ffi.EPI_NONE))
+            acc = TensorData((1,), "f32", np.array([3.0], np.float32))
+            ffi.check(B.lib.ah_gemm_grouped_run_sumsq(plan.value, epi, B._ptr(acc)))
+            assert B.lastGemmKernel()[0].endswith(", true>")
+            got = read()
+            for g_, w_, (m, n) in zip(got, want_c, shapes):
+                assert np.array_equal(g_, w_), f"{m}x{n}: the matrices differ from ah_gemm_grouped_run's"
+            B._dirty(acc)
+            numbers.append(float(acc.data[0]))
+            want = 3.0 + sum(float((g_.astype(np.float64) ** 2).sum()) for g_ in got)
+            assert abs(numbers[-1] - want) <= 1e-5 * want, (epi, numbers[-1], want)
+        assert numbers[0] == numbers[1]
+    bf = B.zeros((64, 64))
+    tb = TensorData((64, 64), "f16", np.zeros(64 * 64, np.uint16))
+    d16 = (ffi.AhGemm * 1)(ffi.AhGemm(ffi.GEMM_TN, ffi.BF16, ffi.BF16, ffi.EPI_NONE, 64, 64, 64, 64, 64, 64, 1, 0, 0, 0, B._ptr(tb), B._ptr(tb), B._ptr(tb), 0))
+    p16 = C.c_uint64()
+    ffi.check(B.lib.ah_gemm_grouped_plan(d16, 1, C.byref(p16)))
+    assert B.lib.ah_gemm_grouped_run_sumsq(p16.value, ffi.EPI_NONE, B._ptr(bf)) != 0 and b"f32 outputs" in B.lib.ah_last_error()
+    assert B.lib.ah_gemm_grouped_run_sumsq(plan.value, ffi.EPI_NONE, 0) != 0
+    ffi.check(B.lib.ah_gemm_grouped_destroy(p16.value))
+    ffi.check(B.lib.ah_gemm_grouped_destroy(plan.value))
+
+
 @pytest.mark.parametrize("shapes,K,cut", [
     ([(4096, 4096), (768, 768), (1280, 1792)], 256, True),       # 256 + 9 + 35 tiles: the last round (44) is cut, the first problem is not
     ([(2048, 2048), (1280, 1792)], 320, False),                  # 64 + 35 tiles, k not a multiple of 128: nothing to cut
