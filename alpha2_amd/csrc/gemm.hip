@@ -360,18 +360,21 @@ __global__ __launch_bounds__(256) void k_grouped_join(const JoinPart *__restrict
   }
 }
 
-// *inout += the sum of the n partial sums, added up in f64 in an order that depends on n only.
+// *inout += the sum of the n partial sums (n a multiple of 4), added up in f64 in an order that depends on n only.
 __global__ __launch_bounds__(256) void k_grouped_sumsq_final(const float *__restrict__ partial, int n, float *__restrict__ inout) {
-  __shared__ double sh[256];
+  __shared__ double sh[4];
+  const float4 *p4 = reinterpret_cast<const float4 *>(partial);
+  const int n4 = n >> 2;
   double t = 0.0;
-  for (int i = threadIdx.x; i < n; i += 256) t += (double)partial[i];
-  sh[threadIdx.x] = t;
-  __syncthreads();
-  for (int w = 128; w > 0; w >>= 1) {
-    if ((int)threadIdx.x < w) sh[threadIdx.x] += sh[threadIdx.x + w];
-    __syncthreads();
+#pragma unroll 8
+  for (int i = threadIdx.x; i < n4; i += 256) {      // (unrolled: the loads of a thread are in flight together)
+    const float4 v = p4[i];
+    t += ((double)v.x + (double)v.y) + ((double)v.z + (double)v.w);
   }
-  if (threadIdx.x == 0) *inout = (float)((double)*inout + sh[0]);
+  t = ah::wave_sum_d(t);
+  if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = t;
+  __syncthreads();
+  if (threadIdx.x == 0) *inout = (float)((double)*inout + ((sh[0] + sh[1]) + (sh[2] + sh[3])));
 }
 
 constexpr int GROUP_ROUND = 256;     // tiles that run at a time: one per CU

@@ -48,7 +48,8 @@ class StepStats:
 
 class FusedTrainer:
     def __init__(self, backend: HipBackend, cfg: ModelConfig, tc: TrainConfig, batch: int, seed: int = 0, use_graph: bool = True,
-                 accum: int = 1, params: Optional[dict] = None, dw_groups: int = 1, stream: str = "bf16"):
+                 accum: int = 1, params: Optional[dict] = None, dw_groups: int = 1, stream: str = "bf16",
+                 norm_in_epilogue: bool = True):
         self.act = cfg.ffnActivation or "gelu"
         if self.act not in ("gelu", "silu", "relu", "swiglu", "universal", "kan_spline") or cfg.dropout != 0:
             raise ValueError("FusedTrainer schedules the gelu / silu / relu / swiglu / universal / kan_spline blocks without dropout; "
@@ -61,6 +62,7 @@ class FusedTrainer:
             raise ValueError("FusedTrainer needs head_dim in {32,64,128}, nEmbd and ffnDim multiples of 64, vocab multiple of 8")
         self.BT = batch * self.T
         self.dw_groups = max(1, min(int(dw_groups), self.L))
+        self._want_norm_in_epilogue = bool(norm_in_epilogue)
         # The residual stream x and the gradient that flows back along it: f32, or bf16 like every other activation
         # ("bf16": the residual epilogues and the LayerNorm kernels move half the bytes; each add into the stream then rounds
         # to 8 bits, as in any all-bf16-activation step)
@@ -208,9 +210,29 @@ class FusedTrainer:
                 plan = C.c_uint64()
                 check(self.lib.ah_gemm_grouped_plan(arr, len(g_), C.byref(plan)))
                 self._dw_plans.append(plan.value)
+        # With one launch, its epilogue squares and sums the gradients it stores (ah_gemm_grouped_run_sumsq), so the norm
+        # only has to read what that launch does not write: the stretches of the gradient arena between its outputs
+        # (embeddings, LayerNorm and activation coefficients; the arena's padding is zero and stays zero).
+        self._norm_in_epilogue = self._want_norm_in_epilogue and n == 1 and self._dw_plans is not None
+        self._norm_done = False                   # the backward pass of this step has left the norm's square in self.sumsq
+        if self._norm_in_epilogue:
+            written = sorted((d.c, d.m * d.n * 4) for d in self._dw_descs)
+            gaps, at = [], self.G
+            for start, nbytes in written + [(self.G + self.nparam * 4, 0)]:
+                assert start >= at
+                if start > at:
+                    gaps.append((at, (start - at) // 4))
+                at = start + nbytes
+            self._norm_rest = ((C.c_uint64 * len(gaps))(*[a_ for a_, _ in gaps]), (C.c_uint64 * len(gaps))(*[n_ for _, n_ in gaps]), len(gaps))
 
-    def _weight_grads(self, epilogue: int, k: int):
-        """Run k of the weight gradients (all of them when dw_groups = 1)."""
+    def _weight_grads(self, epilogue: int, k: int, sumsq: int = 0):
+        """Run k of the weight gradients (all of them when dw_groups = 1); with sumsq, the sum of the squares of the gradients
+        the run leaves is added to that device float."""
+        def run():
+            if sumsq:
+                check(self.lib.ah_gemm_grouped_run_sumsq(self._dw_plans[k], epilogue, sumsq))
+            else:
+                check(self.lib.ah_gemm_grouped_run(self._dw_plans[k], epilogue))
         side = self.dw_groups > 1 and self._timed is None
         if side:
             check(self.lib.ah_side_begin())
@@ -219,11 +241,11 @@ class FusedTrainer:
                 for d in self._dw_group_descs[k]:
                     self._gemm(d.layout, d.a, d.b, d.c, d.m, d.n, d.k, d.lda, d.ldb, d.ldc, F32, epilogue)
             elif self._timed is None:
-                check(self.lib.ah_gemm_grouped_run(self._dw_plans[k], epilogue))
+                run()
             else:
                 e0, e1 = self.B._event(), self.B._event()
                 check(self.lib.ah_event_record(e0))
-                check(self.lib.ah_gemm_grouped_run(self._dw_plans[k], epilogue))
+                run()
                 check(self.lib.ah_event_record(e1))
                 kernel, nsplit = self.B.lastGemmKernel()
                 self._timed.append({"kind": "gemm", "kernel": kernel, "nsplit": nsplit, "layout": ffi.GEMM_TN, "m": 0, "n": 0, "k": self.BT,
@@ -290,7 +312,7 @@ class FusedTrainer:
             self._timed.append({"kind": "flash_bwd" if bwd else "flash_fwd", "flops": fl, "e0": t0, "e1": t1})
 
     # ------------------------------------------------------------------ the step
-    def _forward_backward(self, first_micro: bool, micro: int = 0):
+    def _forward_backward(self, first_micro: bool, micro: int = 0, last_micro: bool = True):
         self.tok, self.tgt = self.toks[micro], self.tgts[micro]
         lib, BT, Cc, Fd, V, L = self.lib, self.BT, self.C, self.F, self.V, self.L
         NN, NT, TN = ffi.GEMM_NN, ffi.GEMM_NT, ffi.GEMM_TN
@@ -360,20 +382,28 @@ class FusedTrainer:
         jobs = (ffi.AhColsumJob * len(self._ln_jobs))(*[
             ffi.AhColsumJob(part, self.g(name + ".weight"), self.g(name + ".bias"), BT, Cc, acc, 0) for name, part in self._ln_jobs])
         check(lib.ah_layernorm_colsums(jobs, len(self._ln_jobs)))
-        if self.dw_groups == 1:
-            self._weight_grads(wepi, 0)
         if self._index_bytes:
             check(lib.ah_embedding_bwd_indexed(self.tok_index[micro], self.dx[cur], self.g("wte"), BT, Cc, V, acc))
         else:
             check(lib.ah_embedding_bwd(self.tok, self.dx[cur], self.g("wte"), BT, Cc, V, acc))
         check(lib.ah_pos_embedding_bwd(self.dx[cur], self.g("wpe"), self.batch, self.T, Cc, acc))
+        if self.dw_groups == 1:
+            if last_micro and self._norm_in_epilogue:     # the norm of the step's gradient: the other gradients first, the launch adds its own
+                xs, ns, count = self._norm_rest
+                check(lib.ah_sum_sq_list(xs, ns, count, self.sumsq))
+                self._weight_grads(wepi, 0, self.sumsq)
+                self._norm_done = True
+            else:
+                self._weight_grads(wepi, 0)
         if self.dw_groups > 1:                    # the next micro-step overwrites the operands, the optimizer reads the results
             check(lib.ah_side_join())
 
     def _optimizer(self):
         lib, tc = self.lib, self.tc
         split = self.off["_split"]
-        check(lib.ah_sum_sq(self.G, self.nparam, self.sumsq))               # arena padding is zero and stays zero
+        if not self._norm_done:
+            check(lib.ah_sum_sq(self.G, self.nparam, self.sumsq))           # arena padding is zero and stays zero
+        self._norm_done = False
         # clip coefficient, non-finite guard and the bias corrections, all on the device (trainer.ts:1248-1262,1495-1522,1650-1656)
         check(lib.ah_step_guard(self.sumsq, self.loss, 1.0 / self.accum, tc.gradClip, tc.beta1, tc.beta2, self.guard, self.hyper, self.clip))
         h = ffi.AhAdamW(tc.lr, tc.beta1, tc.beta2, tc.eps, tc.weightDecay, 1.0, 1.0, 1.0 / self.accum)
@@ -387,7 +417,7 @@ class FusedTrainer:
 
     def _whole_step(self):
         for m in range(self.accum):               # gradients of the micro-steps are summed in place; scaled once in the optimizer
-            self._forward_backward(m == 0, m)
+            self._forward_backward(m == 0, m, m == self.accum - 1)
         self._optimizer()
 
     def _upload_batch(self, inputs: TensorData, targets: TensorData, ti: int, tt: int):

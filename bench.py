@@ -93,6 +93,8 @@ def main():
     ap.add_argument("--mode", choices=["fast", "backend", "parity"], default="fast")
     ap.add_argument("--no-step-graphs", action="store_true", help="backend mode: issue every launch eagerly")
     ap.add_argument("--dw-groups", type=int, default=1, help="fast mode: weight-gradient GEMMs in this many runs on a second stream")
+    ap.add_argument("--norm-over-arena", action="store_true", help="fast mode, for comparison: take the gradient norm by reading the whole gradient "
+                    "arena again instead of summing the weight gradients' squares in the epilogue of the launch that stores them")
     ap.add_argument("--stream", choices=["f32", "bf16"], default="bf16", help="fast mode: storage type of the residual stream and its gradient")
     ap.add_argument("--attention", choices=["heads", "reference-flash", "unfused"], default="heads",
                     help="backend / parity mode: which attention branch of the model runs (reference-flash = the op sequence of the "
@@ -140,7 +142,8 @@ def main():
             return runner.step([(B.reshape(x, x.shape), B.reshape(y, y.shape)) for x, y in pick])
     else:
         from alpha2_amd.fused import FusedTrainer
-        runner = FusedTrainer(B, cfg, tc, BATCH, seed=0, accum=accum, dw_groups=args.dw_groups, stream=args.stream)
+        runner = FusedTrainer(B, cfg, tc, BATCH, seed=0, accum=accum, dw_groups=args.dw_groups, stream=args.stream,
+                              norm_in_epilogue=not args.norm_over_arena)
         dtype = "bf16"
         ids = [runner.add_batch(x, y) for x, y in micro]                   # resident in HBM before the timed region
         cursor = [0]
@@ -216,6 +219,8 @@ def main():
         out["config"]["step_plans"] = step_stats
     if args.mode == "fast" and args.dw_groups > 1:
         out["config"]["dw_groups"] = args.dw_groups
+    if args.mode == "fast" and args.norm_over_arena:
+        out["config"]["norm"] = "over the arena"
     if args.mode == "fast":
         out["config"]["residual_stream"] = args.stream
     if not args.no_cpu:

@@ -157,9 +157,10 @@ def test_fused_step_with_a_non_finite_gradient_is_skipped_on_the_device(B):
         t.step()
     before = {n: a.param(n) for n in ("wte", "layer.0.mlp.fc1", "lnF.weight")}
     m_before = a.stateDict()["buffers"]["layer.0.mlp.fc1.m"].data.copy()
-    # poison: run forward/backward, then put an Inf into the gradient arena before the optimizer part
+    # poison: run forward/backward, then put an Inf into the gradient arena before the optimizer part (as a micro-step that is
+    # not the last: the norm is then taken by the optimizer part, over the arena as it finds it)
     a._write_hyper()
-    a._forward_backward(True, 0)
+    a._forward_backward(True, 0, last_micro=False)
     inf = np.array([np.inf], np.float32)
     ffi_check = __import__("alpha2_amd._ffi", fromlist=["check"]).check
     ffi_check(B.lib.ah_upload(a.g("layer.0.mlp.fc1") + 40, inf.ctypes.data_as(C.c_void_p), 4))
@@ -222,6 +223,44 @@ def test_fused_step_is_bit_identical_from_run_to_run(B):
 
 @pytest.mark.parametrize("graph", [False, True])
 @pytest.mark.parametrize("accum", [1, 2])
+def test_gradient_norm_from_the_weight_gradient_epilogue(B, graph, accum):
+    """By default the grouped weight-gradient launch of the last micro-step squares and sums what it stores, and only the
+    other gradients are read again for the norm.  Against a trainer that reads the whole gradient arena: the gradients are
+    the same bits, the norm agrees to f32 rounding (another order of the same sum), the parameters after four steps to a
+    rounding of the clip coefficient; and the reported norm is the norm of the arena the step left."""
+    import ctypes as C
+    from alpha2_amd import TensorData, _ffi as ffi
+    from alpha2_amd.fused import FusedTrainer
+    from alpha2_amd.model import ModelConfig
+    from alpha2_amd.train import TrainConfig, syntheticBatch
+    mk = lambda fold: FusedTrainer(B, ModelConfig(**CFG), TrainConfig(iters=6, gradAccumSteps=accum), 4, seed=0, use_graph=graph,
+                                   accum=accum, norm_in_epilogue=fold)
+    one, two = mk(True), mk(False)
+    assert one._norm_in_epilogue and not two._norm_in_epilogue
+    batches = [syntheticBatch(3 + m, 4, 64, 256) for m in range(accum)]
+    i1, i2 = [one.add_batch(*b) for b in batches], [two.add_batch(*b) for b in batches]
+    for s in range(4):
+        one.step(i1 if accum > 1 else i1[0])
+        two.step(i2 if accum > 1 else i2[0])
+        if s == 0:
+            for name in ("wte", "wpe", "lmHead", "layer.0.attn.wqkv", "layer.1.mlp.fc2", "layer.1.ln1.weight", "lnF.bias"):
+                assert np.array_equal(one.grad(name), two.grad(name)), name
+    for a, b in zip(one.history(0, 4), two.history(0, 4)):
+        assert abs(a.loss - b.loss) <= 1e-6 * abs(b.loss) and abs(a.gradNorm - b.gradNorm) <= 1e-5 * b.gradNorm, (a, b)
+    assert one.history(0, 1)[0].loss == two.history(0, 1)[0].loss
+    for name in ("wte", "lmHead", "layer.0.attn.wqkv", "layer.1.mlp.fc2", "layer.1.ln1.weight"):
+        assert np.allclose(one.param(name), two.param(name), rtol=0, atol=1e-6), name
+    arena = TensorData((1,), "f32", np.zeros(1, np.float32))
+    ffi.check(B.lib.ah_sum_sq(one.G, one.nparam, B._ptr(arena)))
+    B._dirty(arena)
+    want = math.sqrt(float(arena.data[0])) / accum
+    got = one.history(3, 1)[0].gradNorm
+    assert abs(got - want) <= 1e-5 * want, (got, want)
+    one.close(), two.close()
+
+
+@pytest.mark.parametrize("graph", [False, True])
+@pytest.mark.parametrize("accum", [1, 2])
 def test_weight_gradients_on_the_side_stream_give_the_same_step(B, graph, accum):
     """dw_groups = 2 launches the weight-gradient GEMMs of the upper layer beside the backward kernels of the lower one on
     a second stream; every product keeps its own kernel configuration, so the step must not change by a bit."""
@@ -229,7 +268,7 @@ def test_weight_gradients_on_the_side_stream_give_the_same_step(B, graph, accum)
     from alpha2_amd.model import ModelConfig
     from alpha2_amd.train import TrainConfig, syntheticBatch
     mk = lambda groups: FusedTrainer(B, ModelConfig(**CFG), TrainConfig(iters=6, gradAccumSteps=accum), 4, seed=0, use_graph=graph,
-                                     accum=accum, dw_groups=groups)
+                                     accum=accum, dw_groups=groups, norm_in_epilogue=False)      # (both sum the norm over the arena)
     one, two = mk(1), mk(2)
     batches = [syntheticBatch(3 + m, 4, 64, 256) for m in range(accum)]
     i1, i2 = [one.add_batch(*b) for b in batches], [two.add_batch(*b) for b in batches]
