@@ -420,6 +420,10 @@ class FastHipBackend(HipBackend):
         return out
 
     def _launch_weight_grads(self):
+        self._run_weight_grads(*self._take_weight_grads())
+
+    def _take_weight_grads(self):
+        """Empties the queue: (the queued products, [(epilogue, descriptors, as one grouped launch?)])."""
         ws, self._wgrads = self._wgrads, []
         self._wq_out, self._wq_into = set(), set()
         descs = []
@@ -429,9 +433,17 @@ class FastHipBackend(HipBackend):
             dst, epi = (w.out_buf.ptr + w.out_off, ffi.EPI_NONE) if w.into is None else (w.into[0].ptr + w.into[1], ffi.EPI_ACCUM)
             descs.append(ffi.AhGemm(ffi.GEMM_TN, BF16, F32, epi, w.m, w.n, w.k, w.m, w.n, w.n, 1, 0, 0, 0, w.g_ptr, w.x_ptr, dst, 0))
         groupable = all(d.k % 64 == 0 and d.m % 8 == 0 and d.n % 8 == 0 for d in descs)
+        parts = []
         for epi in (ffi.EPI_NONE, ffi.EPI_ACCUM):
             part = [d for d in descs if d.epilogue == epi]
-            if groupable and len(part) > 1:
+            if part:
+                parts.append((epi, part, groupable and len(part) > 1))
+        return ws, parts
+
+    def _run_weight_grads(self, ws, parts, sumsq: int = 0):
+        """Launches them; with sumsq, the grouped launches add the sum of the squares of what they leave to that device float."""
+        for epi, part, grouped in parts:
+            if grouped:
                 # one plan per list of shapes; the gradients are new tensors every step, so its tables are rewritten every time
                 # (also when nothing moved: a step plan wants the same launches from every step)
                 key = (epi,) + tuple((d.m, d.n, d.k) for d in part)
@@ -447,13 +459,19 @@ class FastHipBackend(HipBackend):
                     plan = self._plans[key] = pid.value
                 else:
                     check(self.lib.ah_gemm_grouped_update(plan, arr, len(part)))
+
+                def run():
+                    if sumsq:
+                        check(self.lib.ah_gemm_grouped_run_sumsq(plan, epi, sumsq))
+                    else:
+                        check(self.lib.ah_gemm_grouped_run(plan, epi))
                 timed = getattr(self, "_timed", None)
                 if timed is None:
-                    check(self.lib.ah_gemm_grouped_run(plan, epi))
+                    run()
                 else:
                     e0, e1 = self._event(), self._event()
                     check(self.lib.ah_event_record(e0))
-                    check(self.lib.ah_gemm_grouped_run(plan, epi))
+                    run()
                     check(self.lib.ah_event_record(e1))
                     kernel, nsplit = self.lastGemmKernel()
                     timed.append({"kind": "gemm", "kernel": kernel, "nsplit": nsplit, "layout": ffi.GEMM_TN, "dtype": BF16, "m": 0, "n": 0,
@@ -681,25 +699,49 @@ class FastHipBackend(HipBackend):
     def totalSumOfSquares(self, tensors: Sequence[TensorData]) -> TensorData:
         self._launch_held()
         self._launch_ln()
-        self._launch_weight_grads()
-        self._flush_adam()
         # The device is idle while this runs (the trainer has just read the loss back, trainer.ts:1247,1345-1349): with nothing
         # pending and every gradient resident in f32, the addresses are read straight off the tensors, and the argument
         # arrays of the last call are reused when the gradient set sits where it sat then.
-        if not self._orphans and not self._ln_unwritten:
+        def addresses():
+            if self._orphans or self._ln_unwritten:
+                return (None,)
             try:
-                key = tuple([t._buf.ptr + t._off if t._dev_valid and t.store == "f32" else None for t in tensors])
+                return tuple([t._buf.ptr + t._off if t._dev_valid and t.store == "f32" else None for t in tensors])
             except AttributeError:                              # a tensor without a device buffer
-                key = (None,)
-            if None not in key and len(key) > 0:
-                c = self._ssq_args
-                if c is None or c[0] != key or c[1] != [t.size for t in tensors]:
-                    sizes = [t.size for t in tensors]
-                    c = self._ssq_args = (key, sizes, (C.c_uint64 * len(key))(*key), (C.c_uint64 * len(key))(*sizes))
-                total = self._new((1,))
-                check(self.lib.ah_sum_sq_list(c[2], c[3], len(key), total._buf.ptr))
-                return total
+                return (None,)
+        if self._wgrads and not self._adam_q:
+            # The queued weight gradients are about to be computed by grouped launches: let those sum the squares of what
+            # they store, and read only the other gradients again.  Every result of such a launch must be one of the listed
+            # tensors, whole; otherwise the launches run as they are and the list is read as usual.
+            key = addresses()
+            if None not in key and len(set(key)) == len(key):
+                ws, parts = self._take_weight_grads()
+                covered = {d.c: d.m * d.n for _, part, grouped in parts if grouped for d in part}
+                listed = {k: t.size for k, t in zip(key, tensors)}
+                if covered and all(listed.get(a) == n for a, n in covered.items()):
+                    total = self._new((1,))
+                    rest = [(k, t.size) for k, t in zip(key, tensors) if k not in covered]
+                    if rest:
+                        self._sum_sq_list(tuple(k for k, _ in rest), [n for _, n in rest], total._buf.ptr)
+                    else:
+                        check(self.lib.ah_fill_f32(total._buf.ptr, 0.0, 1))
+                    self._run_weight_grads(ws, parts, total._buf.ptr)
+                    return total
+                self._run_weight_grads(ws, parts)
+        self._launch_weight_grads()
+        self._flush_adam()
+        key = addresses()
+        if None not in key and len(key) > 0:
+            total = self._new((1,))
+            self._sum_sq_list(key, [t.size for t in tensors], total._buf.ptr)
+            return total
         return super().totalSumOfSquares(tensors)
+
+    def _sum_sq_list(self, ptrs, sizes, out: int):
+        c = self._ssq_args
+        if c is None or c[0] != ptrs or c[1] != sizes:
+            c = self._ssq_args = (ptrs, sizes, (C.c_uint64 * len(ptrs))(*ptrs), (C.c_uint64 * len(ptrs))(*sizes))
+        check(self.lib.ah_sum_sq_list(c[2], c[3], len(ptrs), out))
 
     def adamwStep(self, params, grads, m, v, lr, beta1, beta2, eps, weightDecay, bc1, bc2, gradScale=1.0):
         """Queued: the optimizer calls this once per parameter tensor with the same scalars (optimizers.ts:54-94); the updates of

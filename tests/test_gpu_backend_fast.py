@@ -99,6 +99,7 @@ def test_weight_gradients_are_grouped_and_accumulate_in_place(FB):
         FB.releaseGpuTensor(o)
     total = FB.totalSumOfSquares(grads)                         # the trainer's gradient norm reads them: one grouped launch
     assert len(FB._wgrads) == 0
+    assert FB.lastGemmKernel()[0].endswith(", true>")           # ... which squares and sums what it stores: nothing is read again
     assert abs(float(total.data[0]) - sum(float((w ** 2).sum()) for w in wants)) <= 1e-3 * sum(float((w ** 2).sum()) for w in wants)
     for gr, w in zip(grads, wants):
         _close(gr.data, w, "grouped weight gradient", tol=1e-3)
@@ -109,6 +110,24 @@ def test_weight_gradients_are_grouped_and_accumulate_in_place(FB):
         FB.releaseGpuTensor(o)
     for gr, w in zip(grads, wants):
         _close(gr.data, 2 * w, "accumulated weight gradient", tol=1e-3)
+    # the norm over queued products and other tensors: the launch sums its own, the others are read
+    sq = [float((w ** 2).sum()) for w in wants]
+    o = [FB.matmulTransposedA(_td(g), _td(x)) for g, x in zip(gs, xs)]
+    extra = FB.scale(_td(np.arange(10.0)), 1.0)                 # (resident on the device, as the trainer's gradients are)
+    got = float(FB.totalSumOfSquares([o[0], extra, o[1], o[2]]).data[0])
+    assert FB.lastGemmKernel()[0].endswith(", true>") and abs(got - (sum(sq) + 285.0)) <= 1e-3 * (sum(sq) + 285.0)
+    # a queued product that the list does not name must not count: the launches run as they are, the list is read
+    o = [FB.matmulTransposedA(_td(g), _td(x)) for g, x in zip(gs, xs)]
+    got = float(FB.totalSumOfSquares([o[0], o[2]]).data[0])
+    assert FB.lastGemmKernel()[0].endswith(", false>") and abs(got - (sq[0] + sq[2])) <= 1e-3 * (sq[0] + sq[2])
+    _close(o[1].data, wants[1], "the product outside the list", tol=1e-3)
+    # accumulating launches count the accumulated values
+    o2 = [FB.matmulTransposedA(_td(g), _td(x)) for g, x in zip(gs, xs)]
+    for gr, x in zip(grads, o2):
+        FB.addInplace(gr, x)
+        FB.releaseGpuTensor(x)
+    got = float(FB.totalSumOfSquares(grads).data[0])
+    assert FB.lastGemmKernel()[0].endswith(", true>") and abs(got - 9 * sum(sq)) <= 1e-3 * 9 * sum(sq)
 
 
 def test_clone_is_copy_on_write(FB):
