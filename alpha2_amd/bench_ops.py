@@ -1,7 +1,7 @@
 """Per-op microbenchmarks on the shapes of the training step, in the manner of the reference's scripts/bench-ops.ts
 (3 warm-up calls, then the mean of `iters` calls; TFLOP/s = flops / time, GB/s = algorithmic bytes / time):
 
-    python -m alpha2_amd.bench_ops [--iters 10] [--only gemm|flash|bandwidth|epilogue] [--json]
+    python -m alpha2_amd.bench_ops [--iters 10] [--only gemm|flash|bandwidth|ceiling|epilogue] [--json]
 
 * GEMM: C = A B^T and both backward products, M = 16384 (batch x context), K = 768, N in {768, 2304, 3072, 50304},
   bf16 operands with fp32 accumulation and fp32 throughout; flops 2 M N K (scripts/bench-ops.ts:302,328).
@@ -13,6 +13,8 @@
   (scripts/bench-ops.ts:652,673).
 * Bandwidth-bound ops at the GPT-2-small step's sizes: LayerNorm forward / backward, GELU forward / backward, fused
   cross-entropy forward + backward, embedding gather / scatter-add, sum of squares, AdamW; bytes = the algorithmic minimum.
+* The matrix pipes alone (`ah_probe_mfma_bf16`: independent 32x32x16 bf16 MFMAs on registers, no memory traffic), on zeros and
+  on operands whose bits toggle, for one short launch and sustained: what the part's power limit leaves of the published peak.
 
 Every call goes through the C ABI; timing is by HIP events on the library's stream.  Peaks used for the last column:
 2.5 PFLOP/s (bf16 MFMA), 157.3 TFLOP/s (fp32 MFMA), 8 TB/s (HBM).
@@ -240,15 +242,55 @@ def bench_bandwidth(b: Bench):
     b.release()
 
 
+def bench_ceiling(b: Bench):
+    """What the matrix pipes sustain with nothing else going on (operands in registers), by how long they are kept busy and by
+    what the operands hold; the rate of the last line is the ceiling a bf16 GEMM on real data can be read against."""
+    lib = b.lib
+    fl = C.c_double()
+
+    def run(name, waves, iters, launches, random_ops, note=""):
+        ffi.check(lib.ah_probe_mfma_bf16(waves, 100, random_ops, C.byref(fl)))       # (first launch of a kernel: code upload)
+        ffi.check(lib.ah_sync())
+        e0, e1 = b.B._event(), b.B._event()
+        ffi.check(lib.ah_event_record(e0))
+        for _ in range(launches):
+            ffi.check(lib.ah_probe_mfma_bf16(waves, iters, random_ops, C.byref(fl)))
+        ffi.check(lib.ah_event_record(e1))
+        ms = C.c_float()
+        ffi.check(lib.ah_event_elapsed_ms(e0, e1, C.byref(ms)))
+        for e in (e0, e1):
+            ffi.check(lib.ah_event_destroy(e))
+        b.record(name, ms.value / launches, flops=fl.value, note=note)
+    run("mfma bf16, zeros, 100 x 3 ms", 1, 30000, 100, 0, "registers only, no memory traffic: the published dense peak")
+    run("mfma bf16, random, 1 x 0.15 ms", 1, 1000, 1, 1, "operands whose bits toggle; one short launch after an idle device")
+    run("mfma bf16, random, 1 x 4 ms", 1, 30000, 1, 1, "the length of the step's weight-gradient launch")
+    run("mfma bf16, random, 100 x 4 ms", 1, 30000, 100, 1, "sustained: what the power limit allows the matrix pipes alone")
+    run("mfma bf16, random, 100 x 4 ms, 2 waves", 2, 15000, 100, 1, "two waves per SIMD: the same")
+    # the other side of it: the library's GEMM on operands that toggle nothing (the power limit does not bind, the clock stays
+    # up), which shows what the kernel's own structure - its traffic through L2 and LDS - allows; compare the rows of the
+    # same shapes in the GEMM section, which run on random operands
+    M, K, N = 16384, 768, 50304
+    a, w, g = b.randn(M * K, ffi.BF16, 0.0), b.randn(N * K, ffi.BF16, 0.0), b.randn(M * N, ffi.BF16, 0.0)
+    c_fwd, c_da, c_db = b.alloc(M * N * 2), b.alloc(M * K * 2), b.alloc(N * K * 4)
+    for label, layout, (m, n, k, lda, ldb, ldc), (pa, pb, pc), out in (
+            ("fwd  C=A.B^T", ffi.GEMM_NT, (M, N, K, K, K, N), (a, w, c_fwd), ffi.BF16),
+            ("dA   G.B", ffi.GEMM_NN, (M, K, N, N, K, K), (g, w, c_da), ffi.BF16),
+            ("dB   G^T.A", ffi.GEMM_TN, (N, K, M, N, K, K), (g, a, c_db), ffi.F32)):
+        d = ffi.AhGemm(layout, ffi.BF16, out, ffi.EPI_NONE, m, n, k, lda, ldb, ldc, 1, 0, 0, 0, pa, pb, pc, 0)
+        ms = b.time(lambda: ffi.check(lib.ah_gemm(C.byref(d))))
+        b.record(f"gemm bf16 N={N} {label}, zeros", ms, flops=2.0 * M * N * K, note="all-zero operands")
+    b.release()
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser(description=__doc__.split("\n")[0])
     ap.add_argument("--iters", type=int, default=10)
-    ap.add_argument("--only", choices=["gemm", "flash", "bandwidth", "epilogue"])
+    ap.add_argument("--only", choices=["gemm", "flash", "bandwidth", "ceiling", "epilogue"])
     ap.add_argument("--json", action="store_true", help="also print one JSON line with every row")
     args = ap.parse_args(argv)
     b = Bench(args.iters)
     print(f"{'op':34s} {'time':>13s} {'rate':>16s} {'peak':>7s}")
-    for name, fn in (("gemm", bench_gemm), ("flash", bench_flash), ("bandwidth", bench_bandwidth)):
+    for name, fn in (("gemm", bench_gemm), ("flash", bench_flash), ("bandwidth", bench_bandwidth), ("ceiling", bench_ceiling)):
         if args.only in (None, name):
             fn(b)
     if args.only == "epilogue":

@@ -15,7 +15,7 @@ OBJ = os.path.join(CSRC, "build")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIB_DIR, "libalpha_hip.so")
 SOURCES = ["runtime", "elementwise", "reduce", "nn", "optimizer", "gemm", "gemm_bf16", "gemm_bf16_dma_nt", "gemm_bf16_dma_nn",
-           "gemm_bf16_dma_tn", "attention", "attention_bf16"]
+           "gemm_bf16_dma_tn", "attention", "attention_bf16", "probe"]
 # -packed-fp32-ops off: the compiler must not form v_pk_*_f32 from ordinary float code on this target.
 FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          "-Wno-unused-command-line-argument"]

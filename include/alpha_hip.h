@@ -376,6 +376,14 @@ int32_t ah_gemm_grouped_destroy(uint64_t plan);
  * launched, spelled as a profiler demangles it (e.g. "k_gemm_bf16<256, 256, 2, 4, false, false>"), and the number
  * of split-K slices it used (1 = none; > 1 means a k_splitk_reduce launch followed). */
 int32_t ah_gemm_last_kernel(char *name, int32_t capacity, int32_t *nsplit);
+/* Measurement aid (no counterpart in the reference; the nearest is the flop accounting of scripts/bench-ops.ts:302-328, which
+ * prices GEMMs against a peak): ONE launch in which every SIMD of the device runs waves_per_simd (1-4) waves that each issue
+ * iters (1-200000) x 8 independent 32x32x16 bf16 MFMAs on operands held in registers: no LDS, no memory traffic.
+ * random_operands != 0: operands of the size of activations and weights with pseudo-random bits; 0: all zeros.  *flops_out (host,
+ * may be null) = the flops of the launch.  Timed by the caller with ah_event_*: with zeros the part runs at its published
+ * dense peak, with operands whose bits toggle at what its power limit sustains, which is the ceiling a GEMM on real data
+ * can be read against. */
+int32_t ah_probe_mfma_bf16(int32_t waves_per_simd, int32_t iters, int32_t random_operands, double *flops_out);
 
 /* ---- fused causal flash attention.  Backend.flashAttention / flashAttentionBackward
  *      (interfaces.ts:127-135; kernel semantics packages/helios/src/kernels/attention.ts:1-586):

@@ -1249,3 +1249,19 @@ def test_flash_attention_microbench_shapes(B, bwd_variant, T, cap):
     assert_close(sel(g["dQ"]), dq.reshape(3, T, D), rel=rel, what="dQ", **loose(dq))
     assert_close(sel(g["dK"]), dk.reshape(3, T, D), rel=rel, what="dK", **loose(dk))
     assert_close(sel(g["dV"]), dv.reshape(3, T, D), rel=rel, what="dV", **loose(dv))
+
+
+def test_mfma_probe_runs_and_refuses_sizes_outside_its_range(B):
+    """The measurement aid launches and finishes (every wave runs a counted loop), reports the flops of its launch, and
+    refuses iteration counts and wave counts beyond its stated range."""
+    import ctypes as C
+    from alpha2_amd import _ffi as ffi
+    fl = C.c_double()
+    for random_ops in (0, 1):
+        ffi.check(B.lib.ah_probe_mfma_bf16(2, 50, random_ops, C.byref(fl)))
+    ffi.check(B.lib.ah_sync())
+    info = ffi.AhDeviceInfo()
+    ffi.check(B.lib.ah_device_info(C.byref(info)))
+    assert fl.value == info.compute_units * 2 * 4 * 50 * 8 * 2.0 * 32 * 32 * 16
+    assert B.lib.ah_probe_mfma_bf16(5, 50, 1, None) != 0 and b"1-4 waves" in B.lib.ah_last_error()
+    assert B.lib.ah_probe_mfma_bf16(1, 200001, 1, None) != 0
