@@ -1251,6 +1251,34 @@ def test_flash_attention_microbench_shapes(B, bwd_variant, T, cap):
     assert_close(sel(g["dV"]), dv.reshape(3, T, D), rel=rel, what="dV", **loose(dv))
 
 
+@pytest.mark.parametrize("K", [128, 192])      # every problem cut in two along k (the joining kernel sums) / none cut (the epilogue sums)
+def test_gemm_grouped_sum_of_squares_is_not_finite_when_a_product_is_not(B, K):
+    """The trainer skips a step whose gradient norm is not finite (trainer.ts:1248,1495-1522): an Inf or a NaN that a weight-gradient
+    product stores must reach the sum its launch takes, also from the last row of a ragged tile."""
+    import ctypes as C
+    import math
+    from alpha2_amd import TensorData, _ffi as ffi
+    for bad in (np.inf, np.nan):
+        keep, descs = [], []
+        for m, n, poison in ((256, 256, False), (264, 520, True), (512, 256, False)):
+            gy, x = _bf16_round(rs.randn(K, m).astype(np.float32))[0], _bf16_round(rs.randn(K, n).astype(np.float32))[0]
+            if poison:
+                gy[5, m - 1] = bad                                            # reaches row m - 1 of C, in the ragged edge tile
+            tg, tx = TensorData(gy.shape, "f16", _bf16_round(gy)[1]), TensorData(x.shape, "f16", _bf16_round(x)[1])
+            out = B.zeros((m, n))
+            keep += [tg, tx, out]
+            descs.append(ffi.AhGemm(ffi.GEMM_TN, ffi.BF16, ffi.F32, ffi.EPI_NONE, m, n, K, m, n, n, 1, 0, 0, 0, B._ptr(tg), B._ptr(tx), B._ptr(out), 0))
+        arr = (ffi.AhGemm * len(descs))(*descs)
+        plan = C.c_uint64()
+        ffi.check(B.lib.ah_gemm_grouped_plan(arr, len(descs), C.byref(plan)))
+        acc = TensorData((1,), "f32", np.array([0.0], np.float32))
+        ffi.check(B.lib.ah_gemm_grouped_run_sumsq(plan.value, ffi.EPI_NONE, B._ptr(acc)))
+        assert B.lastGemmKernel()[1] == (2 if K % 128 == 0 else 1)
+        B._dirty(acc)
+        assert not math.isfinite(float(acc.data[0])), (bad, float(acc.data[0]))
+        ffi.check(B.lib.ah_gemm_grouped_destroy(plan.value))
+
+
 def test_mfma_probe_runs_and_refuses_sizes_outside_its_range(B):
     """The measurement aid launches and finishes (every wave runs a counted loop), reports the flops of its launch, and
     refuses iteration counts and wave counts beyond its stated range."""
