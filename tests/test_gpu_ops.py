@@ -759,6 +759,42 @@ def test_adamw_vs_oracle_and_reference_gradscale_identity(B, golden):
     assert np.max(np.abs(run(False) - run(True))) < 1e-7
 
 
+def test_clip_coefficient_on_the_device_and_its_use_by_adamw(B):
+    """ah_clip_coef against the trainer's rule (trainer.ts:1650-1656: norm = sqrt(sum of squares) x |gradScale|; the
+    coefficient is clip / norm above the clip value, 1 at or below it, and clipping is off at clip <= 0), and an AdamW step
+    that takes the coefficient from the device against the same step with the coefficient folded into gradScale on the host."""
+    import ctypes as C
+    import math
+    from alpha2_amd import TensorData, _ffi as ffi
+    out = B.zeros((2,))
+    for sumsq, scale, clip in ((16.0, 0.5, 1.0), (16.0, -0.5, 1.0), (0.25, 1.0, 1.0), (1.0, 1.0, 1.0), (9.0, 1.0, 0.0), (0.0, 1.0, 1.0)):
+        ss = TensorData((1,), "f32", np.array([sumsq], np.float32))
+        ffi.check(B.lib.ah_clip_coef(B._ptr(ss), scale, clip, B._ptr(out)))
+        B._dirty(out)
+        norm = math.sqrt(sumsq) * abs(scale)
+        want = clip / norm if clip > 0 and norm > clip else 1.0
+        assert abs(float(out.data[0]) - want) <= 2e-7 * want and abs(float(out.data[1]) - norm) <= 2e-7 * max(norm, 1.0), (sumsq, scale, clip, out.data)
+    assert B.lib.ah_clip_coef(0, 1.0, 1.0, B._ptr(out)) != 0 and b"null operand" in B.lib.ah_last_error()
+    n = 4099
+    p0, g = rs.randn(n).astype(np.float32), rs.randn(n).astype(np.float32)
+    ssq = TensorData((1,), "f32", np.array([float((g.astype(np.float64) ** 2).sum())], np.float32))
+    ffi.check(B.lib.ah_clip_coef(B._ptr(ssq), 0.5, 1.0, B._ptr(out)))
+    B._dirty(out)
+    coef = float(out.data[0])
+    assert coef < 1.0
+    h = ffi.AhAdamW(3e-4, 0.9, 0.95, 1e-8, 0.1, 0.1, 0.05, 0.5)
+    pa, ma, va = dev(B, p0), dev(B, np.zeros(n, np.float32)), dev(B, np.zeros(n, np.float32))
+    gt = dev(B, g)
+    ffi.check(B.lib.ah_adamw(B._ptr(pa), B._ptr(gt), B._ptr(ma), B._ptr(va), n, C.byref(h), 0, B._ptr(out), 0))
+    for t in (pa, ma, va):
+        B._dirty(t)
+    pb, mb, vb = dev(B, p0), dev(B, np.zeros(n, np.float32)), dev(B, np.zeros(n, np.float32))
+    B.adamwStep(pb, dev(B, g), mb, vb, 3e-4, 0.9, 0.95, 1e-8, 0.1, 0.1, 0.05, float(np.float32(0.5) * np.float32(coef)))
+    assert_close(pa.data, pb.data, rel=1e-6, what="adamw with the device coefficient: p")
+    assert_close(ma.data, mb.data, rel=1e-6, what="adamw with the device coefficient: m")
+    assert_close(va.data, vb.data, rel=1e-6, what="adamw with the device coefficient: v")
+
+
 def test_graph_capture_replays_match_eager(B):
     import ctypes as C
     from alpha2_amd import _ffi as ffi
