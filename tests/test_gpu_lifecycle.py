@@ -1,0 +1,48 @@
+"""ah_init / ah_shutdown through the C ABI, in a process of its own (shutting the library down would pull the device
+memory from under the other tests' backend): work, shut down, every call then refused with AH_ERR_STATE until the
+library is initialised again, work again with nothing left over from the first life."""
+import os
+import subprocess
+import sys
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+SCRIPT = r"""
+import ctypes as C
+import numpy as np
+from alpha2_amd import _ffi as ffi
+lib = ffi.load()
+assert lib.ah_shutdown() == 0                                   # before any init: nothing to do
+p = C.c_uint64()
+assert lib.ah_alloc(64, C.byref(p)) == 3 and b"ah_init" in lib.ah_last_error()       # AH_ERR_STATE
+x = np.arange(1000, dtype=np.float32)
+got = np.zeros(1, np.float32)
+for life in range(2):
+    ffi.check(lib.ah_init(0))
+    ffi.check(lib.ah_init(0))                                   # a second init of the same device is accepted
+    s = ffi.AhStats()
+    ffi.check(lib.ah_stats(C.byref(s)))
+    assert s.live_allocs == 0, (life, s.live_allocs)
+    px, out = C.c_uint64(), C.c_uint64()
+    ffi.check(lib.ah_alloc(x.nbytes, C.byref(px)))
+    ffi.check(lib.ah_alloc(16, C.byref(out)))
+    ffi.check(lib.ah_upload(px.value, x.ctypes.data_as(C.c_void_p), x.nbytes))
+    ffi.check(lib.ah_sum_sq(px.value, x.size, out.value))
+    ffi.check(lib.ah_sum_sq_static(px.value, x.size, out.value + 4))             # its per-device array is found again after a shutdown
+    two = np.zeros(2, np.float32)
+    ffi.check(lib.ah_download(two.ctypes.data_as(C.c_void_p), out.value, 8))
+    assert two[0] == two[1] == np.float32(float((x.astype(np.float64) ** 2).sum())), two
+    assert lib.ah_shutdown() == 0                               # frees what the caller left allocated
+    assert lib.ah_sum_sq(px.value, x.size, out.value) == 3
+    assert lib.ah_free(px.value) == 3
+print("lifecycle ok")
+"""
+
+
+def test_shutdown_and_a_second_life():
+    env = dict(os.environ, PYTHONPATH=ROOT + os.pathsep + os.environ.get("PYTHONPATH", ""))
+    r = subprocess.run([sys.executable, "-c", SCRIPT], capture_output=True, text=True, cwd=ROOT, env=env, timeout=100)
+    assert r.returncode == 0 and "lifecycle ok" in r.stdout, r.stdout[-2000:] + r.stderr[-2000:]
