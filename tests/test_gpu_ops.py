@@ -1329,3 +1329,27 @@ def test_mfma_probe_runs_and_refuses_sizes_outside_its_range(B):
     assert fl.value == info.compute_units * 2 * 4 * 50 * 8 * 2.0 * 32 * 32 * 16
     assert B.lib.ah_probe_mfma_bf16(5, 50, 1, None) != 0 and b"1-4 waves" in B.lib.ah_last_error()
     assert B.lib.ah_probe_mfma_bf16(1, 200001, 1, None) != 0
+
+
+def test_the_extras_the_trainer_calls_on_a_gpu_backend(B):
+    """resetStepOps / gpuOpsThisStep and purgeBufferPools, which the reference trainer calls when the backend has them
+    (trainer.ts:1003-1032,1915,1956): the launch counter restarts and counts, and purging the pool frees every cached block
+    without touching live tensors."""
+    x = dev(B, rs.randn(1000).astype(np.float32))
+    B.resetStepOps()
+    assert B.gpuOpsThisStep == 0
+    tmp = [B.scale(x, float(i)) for i in range(1, 6)]
+    assert B.gpuOpsThisStep >= 5
+    want = [t.data.copy() for t in tmp]
+    keep = tmp.pop()
+    for t in tmp:
+        B.releaseGpuTensor(t)
+    B.syncGpu()
+    assert B.gpuMemStats()["bufferPoolEntries"] >= 4
+    live = B.gpuMemStats()["liveAllocs"]
+    B.purgeBufferPools()
+    st = B.gpuMemStats()
+    assert st["bufferPoolEntries"] == 0 and st["bufferPoolBytes"] == 0 and st["liveAllocs"] == live
+    B._dirty(keep)
+    assert np.array_equal(keep.data, want[-1])                  # a live tensor is where it was
+    assert_close(B.scale(x, 2.0).data, 2 * x.data, what="an op after the purge")

@@ -74,6 +74,34 @@ def test_a_step_that_deviates_falls_back_and_the_plan_is_recorded_again(B):
     assert after["replayed"] - before["replayed"] >= 3
 
 
+def test_resetting_the_plan_makes_the_next_bracketed_step_record_again(B):
+    """resetStepPlan forgets the recorded plan: refused while a step is open, and after it the next bracketed step is recorded
+    anew and the following ones replay it - with the numbers of eager execution all along."""
+    from alpha2_amd._ffi import AlphaHipError
+    from alpha2_amd.train import syntheticBatch
+    eager, _, _ = _run(B, False, steps=9)
+    tr = _trainer(B)
+    got = []
+
+    def go(lo, hi):
+        for s in range(lo, hi):
+            r = tr.step([syntheticBatch(40 + s, 4, 32, 96)])
+            got.append((r.loss, r.gradNorm, r.clipCoef, r.lr))
+    B.enableStepGraphs(True)
+    go(0, 4)
+    with pytest.raises(AlphaHipError, match="while a step is open"):
+        B.resetStepPlan()
+    B.enableStepGraphs(False)
+    a = B.stepStats()
+    B.resetStepPlan()
+    B.enableStepGraphs(True)
+    go(4, 9)
+    B.enableStepGraphs(False)
+    b = B.stepStats()
+    assert b["recorded"] - a["recorded"] == 1 and b["replayed"] - a["replayed"] >= 2 and b["fellBack"] == a["fellBack"], (a, b, B.lastStepNote)
+    assert got == eager
+
+
 def test_per_step_scalars_and_dropout_seeds_follow_the_caller(B):
     """Learning rate, bias corrections, the clip coefficient and the dropout seed change every step: they are kernel
     arguments, rewritten in the graph nodes, not frozen at recording time."""
