@@ -216,7 +216,7 @@ int32_t ah_sum_axis(ah_ptr a, ah_ptr out, int64_t outer, int64_t dim, int64_t in
   int64_t lines = outer * inner;
   if (lines == 0) return AH_OK;
   AH_ARG(a && out, "ah_sum_axis: null operand");
-  if (dim == 0) return ah_fill_f32(out, 0.f, (uint64_t)lines);
+  if (dim == 0) return ah_fill_f32(out, mean ? NAN : 0.f, (uint64_t)lines);      // a sum of no terms; its mean is 0 / 0 (cpu_ref.ts:325-330)
   if (inner > 1 && lines >= 4096) {
     ah::launch_kernel(k_sum_strided, dim3((unsigned)cdiv(lines, TPB)), dim3(TPB), 0, dp<const float>(a),
                        dp<float>(out), outer, dim, inner, mean);
@@ -231,7 +231,7 @@ int32_t ah_sum_axis(ah_ptr a, ah_ptr out, int64_t outer, int64_t dim, int64_t in
 static int32_t full_reduce(ah_ptr a, uint64_t n, ah_ptr out, double div, int sq, const char *who) {
   AH_REQUIRE_READY();
   AH_ARG(out != 0, "%s: null out", who);
-  if (n == 0) return ah_fill_f32(out, 0.f, 1);
+  if (n == 0) return ah_fill_f32(out, div == 0.0 ? NAN : 0.f, 1);      // the mean of nothing is 0 / 0 (cpu_ref.ts:317-320)
   AH_ARG(a != 0, "%s: null input", who);
   int nb = partial_blocks(n);
   double *partial = (double *)scratch(sizeof(double) * (size_t)nb);

@@ -188,7 +188,9 @@ void orc_sum_axis(const float *a, const int64_t *shape, int nd, int ax, float *o
   int64_t strides[ORC_MAX_DIMS];
   shape_strides(shape, nd, strides);
   int64_t dim = shape[ax], axs = strides[ax];
-  int64_t outer = shape_size(shape, nd) / dim;
+  int64_t outer = 1;                          /* the other dimensions' product (cpu_ref.ts:272-280): an empty reduced axis gives */
+  for (int d = 0; d < nd; d++)                /* one zero per output (mean: 0 / 0), and no division by its length here        */
+    if (d != ax) outer *= shape[d];
   /* output flat index -> coords over the non-reduced dims (row-major), as flatToMulti does */
   for (int64_t i = 0; i < outer; i++) {
     int64_t rem = i, base = 0;
@@ -280,7 +282,9 @@ void orc_softmax(const float *a, const int64_t *shape, int nd, int ax, float *ou
   int64_t strides[ORC_MAX_DIMS];
   shape_strides(shape, nd, strides);
   int64_t dim = shape[ax], axs = strides[ax];
-  int64_t outer = shape_size(shape, nd) / dim;
+  int64_t outer = 1;                          /* the other dimensions' product (cpu_ref.ts:272-280): an empty reduced axis gives */
+  for (int d = 0; d < nd; d++)                /* one zero per output (mean: 0 / 0), and no division by its length here        */
+    if (d != ax) outer *= shape[d];
   for (int64_t o = 0; o < outer; o++) {
     int64_t rem = o, base = 0;
     for (int d = nd - 1; d >= 0; d--) {
@@ -306,7 +310,9 @@ void orc_log_softmax(const float *a, const int64_t *shape, int nd, int ax, float
   int64_t strides[ORC_MAX_DIMS];
   shape_strides(shape, nd, strides);
   int64_t dim = shape[ax], axs = strides[ax];
-  int64_t outer = shape_size(shape, nd) / dim;
+  int64_t outer = 1;                          /* the other dimensions' product (cpu_ref.ts:272-280): an empty reduced axis gives */
+  for (int d = 0; d < nd; d++)                /* one zero per output (mean: 0 / 0), and no division by its length here        */
+    if (d != ax) outer *= shape[d];
   for (int64_t o = 0; o < outer; o++) {
     int64_t rem = o, base = 0;
     for (int d = nd - 1; d >= 0; d--) {
@@ -412,7 +418,9 @@ void orc_argmax(const float *a, const int64_t *shape, int nd, int ax, int32_t *o
   int64_t strides[ORC_MAX_DIMS];
   shape_strides(shape, nd, strides);
   int64_t dim = shape[ax], axs = strides[ax];
-  int64_t outer = shape_size(shape, nd) / dim;
+  int64_t outer = 1;                          /* the other dimensions' product (cpu_ref.ts:272-280): an empty reduced axis gives */
+  for (int d = 0; d < nd; d++)                /* one zero per output (mean: 0 / 0), and no division by its length here        */
+    if (d != ax) outer *= shape[d];
   for (int64_t o = 0; o < outer; o++) {
     int64_t rem = o, base = 0;
     for (int d = nd - 1; d >= 0; d--) {

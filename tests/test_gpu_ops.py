@@ -288,6 +288,41 @@ def test_empty_tensors(B):
     assert B.sum(dev(B, np.zeros((0,), np.float32))).data[0] == 0.0
 
 
+def test_empty_extents_give_what_the_cpu_path_gives(B):
+    """Tensors with an extent of zero through the ops of the step: the shapes and values of the reference's CPU loops
+    (an empty sum is 0, an empty mean 0 / 0 = NaN, a product over an empty k is all zeros), no launch of an empty grid."""
+    z = lambda *shape: np.zeros(shape, np.float32)
+    cases = {
+        "matmul, no rows": lambda X, t: X.matmul(t(z(0, 5)), t(np.ones((5, 3), np.float32))),
+        "matmul, empty k": lambda X, t: X.matmul(t(z(4, 0)), t(z(0, 3))),
+        "matmul, no columns": lambda X, t: X.matmul(t(np.ones((4, 5), np.float32)), t(z(5, 0))),
+        "transpose": lambda X, t: X.transpose(t(z(0, 3)), 0, 1),
+        "layerNorm": lambda X, t: X.layerNorm(t(z(0, 8)), t(np.ones(8, np.float32)), t(z(8)), 1e-5),
+        "softmax": lambda X, t: X.softmax(t(z(0, 8))),
+        "sum over an empty axis": lambda X, t: X.sum(t(z(3, 0)), 1),
+        "sum along an axis of an empty tensor": lambda X, t: X.sum(t(z(0, 8)), 0),
+        "mean over an empty axis": lambda X, t: X.mean(t(z(3, 0)), 1),
+        "mean of nothing": lambda X, t: X.mean(t(z(0))),
+        "scale": lambda X, t: X.scale(t(z(0, 2)), 2.0),
+        "argmax": lambda X, t: X.argmax(t(z(0, 4)), -1),
+        "slice to nothing": lambda X, t: X.slice(t(np.ones((4, 4), np.float32)), [0, 2], [4, 2]),
+    }
+    for name, fn in cases.items():
+        got, want = fn(B, lambda a: dev(B, a)), fn(O, orc)
+        assert tuple(got.shape) == tuple(want.shape), (name, got.shape, want.shape)
+        assert np.array_equal(np.asarray(got.data).reshape(-1)[:shape_size_of(want)], np.asarray(want.data).reshape(-1)[:shape_size_of(want)], equal_nan=True), (name, got.data, want.data)
+    emb = B.embedding(dev(B, np.ones((5, 4), np.float32)), dev(B, np.zeros((0,), np.int32), "i32"))
+    assert tuple(emb.shape) == (0, 4) and emb.data.size == 0
+    assert float(B.totalSumOfSquares([]).data[0]) == 0.0 and float(B.sumOfSquares(dev(B, z(0))).data[0]) == 0.0
+
+
+def shape_size_of(t):
+    n = 1
+    for d in t.shape:
+        n *= d
+    return n
+
+
 def test_broadcast_binary_and_errors(B):
     a, b = rs.randn(2, 1, 4).astype(np.float32), (rs.randn(3, 1) + 3).astype(np.float32)
     for name in ("add", "sub", "mul", "div"):

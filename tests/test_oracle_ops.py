@@ -353,3 +353,16 @@ def test_dropout_hash_differs_from_u32_wrapping_beyond_2_to_53():
     limit = 2 ** 53 // 2246822519
     assert all(py_dropout_hash(42, 3, i) == wrap(42, 3, i) for i in list(range(2000)) + list(range(limit - 2000, limit - 8)))
     assert sum(py_dropout_hash(42, 3, i) != wrap(42, 3, i) for i in range(limit + 10, limit + 2010)) > 500
+
+
+def test_sum_and_mean_over_an_empty_axis():
+    """cpu_ref.ts:272-308: one output per combination of the other dimensions, each the sum of no terms; mean divides it by
+    the axis length, 0 / 0 (cpu_ref.ts:325-330)."""
+    z = ref.f32(np.zeros((3, 0), np.float32))
+    s = B.sum(z, 1)
+    assert s.shape == (3,) and np.array_equal(s.data[:3], np.zeros(3, np.float32))
+    m = B.mean(z, 1)
+    assert m.shape == (3,) and np.all(np.isnan(m.data[:3]))
+    s0 = B.sum(ref.f32(np.zeros((0, 8), np.float32)), 0)
+    assert s0.shape == (8,) and np.array_equal(s0.data[:8], np.zeros(8, np.float32))
+    assert np.isnan(B.mean(ref.f32(np.zeros((0,), np.float32))).data[0])
