@@ -36,7 +36,7 @@ struct UnOp {
       case AH_SQRT: return sqrtf(x);
       case AH_POW: return powf(x, p0);
       case AH_SCALE: return x * p0;
-      case AH_CLAMP: return fmaxf(p0, fminf(p1, x));
+      case AH_CLAMP: { const float m = p1 < x ? p1 : x; return p0 > m ? p0 : m; }      // max(lo, min(hi, x)) with JS's NaN: NaN stays NaN (cpu_ref.ts:358-360)
       case AH_GELU: return gelu_f(x);
       case AH_RELU: return x > 0.f ? x : 0.f;
       case AH_SILU: return x / (1.0f + expf(-x));

@@ -553,10 +553,12 @@ __global__ __launch_bounds__(256) void k_layernorm_bwd_vec(const X *__restrict__
 }
 
 // ---------------------------------------------------------------- softmax cross-entropy
-// exp(v - m) as one fused multiply-add into the bare base-2 exponential, with neg_m_l2 = -m log2(e) (the vector paths of
-// the three kernels below use the same form, so their results agree bit for bit)
+// exp(v - m) through the bare base-2 exponential (the vector paths of the three kernels below use the same form, so their
+// results agree bit for bit).  The difference is taken first, as the reference takes it (cpu_ref.ts:493-563): folded into
+// one multiply-add, v log2(e) - m log2(e), the rounding of the second product is an error of |m| 2^-24 in the exponent -
+// nothing at |m| < 100, a wrong loss for logits of 1e6, an infinite one at 1e30.
 constexpr float CE_LOG2E = 1.4426950408889634f;
-__device__ __forceinline__ float exp_minus(float v, float neg_m_l2) { return __builtin_amdgcn_exp2f(fmaf(v, CE_LOG2E, neg_m_l2)); }
+__device__ __forceinline__ float exp_minus(float v, float m) { return __builtin_amdgcn_exp2f((v - m) * CE_LOG2E); }
 __device__ __forceinline__ void online_merge(float &m, float &s, float m2, float s2) {
   float nm = fmaxf(m, m2);
   if (nm == -INFINITY) { m = nm; s = 0.f; return; }
@@ -585,9 +587,8 @@ __global__ void k_ce_fwd(const T *__restrict__ logits, const int32_t *__restrict
 #pragma unroll
     for (int i = 1; i < VW; i++) vm = fmaxf(vm, v[i]);
     if (vm > m) { s *= __expf(m - vm); m = vm; }
-    const float nm = -m * CE_LOG2E;
 #pragma unroll
-    for (int i = 0; i < VW; i++) s += exp_minus(v[i], nm);
+    for (int i = 0; i < VW; i++) s += exp_minus(v[i], m);
   }
   for (int64_t j = nvec * VW + threadIdx.x; j < c; j += blockDim.x) {
     float v = Io<T>::ld(p, j);
@@ -633,11 +634,10 @@ __global__ void k_mean_rows(const float *__restrict__ v, int64_t n, float *__res
 __device__ __forceinline__ void ce_grad8(const uint4 &u, float lse, float scale, int hot, uint32_t (&o)[4]) {
   const uint32_t in[4] = {u.x, u.y, u.z, u.w};
   float e[8];
-  const float nl = -lse * CE_LOG2E;
 #pragma unroll
   for (int i = 0; i < 4; i++) {
-    e[2 * i] = exp_minus(bf16_bits_to_f32(in[i] & 0xffff), nl);
-    e[2 * i + 1] = exp_minus(bf16_bits_to_f32(in[i] >> 16), nl);
+    e[2 * i] = exp_minus(bf16_bits_to_f32(in[i] & 0xffff), lse);
+    e[2 * i + 1] = exp_minus(bf16_bits_to_f32(in[i] >> 16), lse);
   }
   if (hot >= 0) {
 #pragma unroll
@@ -701,9 +701,8 @@ __global__ __launch_bounds__(CE_TPB) void k_ce_fwd_bwd(const uint16_t *__restric
 #pragma unroll
       for (int i = 1; i < 8; i++) vm = fmaxf(vm, v[i]);
       if (vm > m) { s *= __expf(m - vm); m = vm; }
-      const float nm = -m * CE_LOG2E;
 #pragma unroll
-      for (int i = 0; i < 8; i++) s += exp_minus(v[i], nm);
+      for (int i = 0; i < 8; i++) s += exp_minus(v[i], m);
     }
   }
 #pragma unroll

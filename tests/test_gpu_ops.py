@@ -678,6 +678,61 @@ def test_cross_entropy_one_pass_equals_forward_then_backward(B, n, c, dtype):
     assert np.all(np.abs(dl - wantg) <= np.abs(wantg) * (half + 1e-4) + 1e-9), "ce.dlogits"
 
 
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("scale", [1e3, 1e5, 1e30])
+def test_cross_entropy_with_logits_far_from_zero(B, dtype, scale):
+    """The reference takes exp(x - max) of the difference (cpu_ref.ts:493-563), so the loss of a row does not depend on
+    where the row sits: logits of the size of 1e3, 1e5 or 1e30 (rows with a clear winner, with ties, and rows shifted as a
+    whole) must give the oracle's loss.  (An exponent formed as x log2(e) - max log2(e) in one fused multiply-add is off by
+    |max| 2^-24: visible from 1e5, infinite at 1e30.)  The gradient is checked to 1e-4 where an f32 log-sum-exp, which is
+    what the backward kernels are handed, still resolves it: rows up to 1e3 (half an ulp of 1e3 is 3e-5); at 1e5 to 2 % of a
+    row's mass; at 1e30, where log(sum) vanishes beside the maximum in f32 (the reference keeps the two apart in f64), only
+    that it is finite."""
+    from alpha2_amd import _ffi as ffi
+    code = ffi.DTYPE_CODE[dtype]
+    n, c = 6, 64
+    base = rs.randn(n, c).astype(np.float32)
+    lg = base.copy()
+    lg[0] *= scale                                   # spread over the whole range: one clear winner
+    lg[1] = scale + base[1]                          # a row shifted as a whole
+    lg[2] = -scale + 3 * base[2]
+    lg[3] = 0.0; lg[3, 5] = scale; lg[3, 9] = scale   # a tie at the top
+    lg[4] = scale * np.sign(base[4])                 # half the row at +scale, half at -scale
+    lg[5] = base[5]                                  # an ordinary row beside them
+    tg = np.array([int(np.argmax(lg[0])), 3, 7, 5, int(np.argmin(lg[4])), 1], np.int32)
+    src = B.castStore(dev(B, lg), dtype)
+    seen = np.array(src.data, dtype=np.float32).reshape(n, c)
+    tgd = dev(B, tg, "i32")
+    for entry in ("pair", "one"):
+        loss, lse, dl = B._new(()), B._new((n,)), B._new((n, c), "f32", dtype)
+        if entry == "pair":
+            ffi.check(B.lib.ah_cross_entropy(B._ptr(src), code, B._ptr(tgd), B._ptr(loss), B._ptr(lse), n, c))
+            ffi.check(B.lib.ah_cross_entropy_bwd(B._ptr(src), code, B._ptr(tgd), B._ptr(lse), 0, 1.0, B._ptr(dl), n, c))
+        else:
+            ffi.check(B.lib.ah_cross_entropy_fwd_bwd(B._ptr(src), code, B._ptr(tgd), B._ptr(loss), B._ptr(lse), 0, 1.0, B._ptr(dl), n, c))
+        B._dirty(dl)
+        want = O.crossEntropy(orc(seen), orc(tg)).data
+        want = float(np.asarray(want).reshape(-1)[0])
+        assert np.isfinite(want) and abs(float(np.asarray(loss.data).reshape(-1)[0]) - want) <= 1e-5 * abs(want) + 1e-6, (entry, loss.data, want)
+        wantg = ref.cross_entropy_backward(orc(seen), orc(tg), 1.0).data.reshape(n, c)
+        half = 2.0 ** -8 if dtype == "bf16" else 0.0
+        got = np.array(dl.data, dtype=np.float32).reshape(n, c)
+        if scale <= 1e3:
+            assert np.all(np.abs(got - wantg) <= np.abs(wantg) * (half + 1e-4) + 1e-7), (entry, np.abs(got - wantg).max())
+        elif scale <= 1e5:
+            assert np.all(np.isfinite(got)) and np.all(np.abs(got.sum(axis=1)) <= 2e-2 / n) and np.all(got[np.arange(n), tg] <= 0), entry
+            assert np.all(np.abs(got - wantg) <= 2e-2 / n), (entry, np.abs(got - wantg).max())      # probabilities within 2 % of the row's mass
+        else:
+            assert np.all(np.isfinite(got)), entry
+
+
+def test_clamp_keeps_nan(B):
+    """max(lo, min(hi, x)) in the reference's arithmetic (cpu_ref.ts:358-360): Math.min / Math.max return NaN for a NaN."""
+    x = np.array([np.nan, -3.0, 0.5, 7.0, np.inf, -np.inf], np.float32)
+    got, want = B.clamp(dev(B, x), -1.0, 2.0).data, O.clamp(orc(x), -1.0, 2.0).data
+    assert np.isnan(got[0]) and np.isnan(want[0]) and np.array_equal(got[1:], want[1:]) and np.array_equal(got[1:], [-1.0, 0.5, 2.0, 2.0, -1.0])
+
+
 @pytest.mark.parametrize("M,K,N", [(2, 2, 2), (33, 19, 47), (64, 64, 64), (128, 128, 128), (256, 256, 256), (1024, 128, 384), (130, 515, 257)])
 def test_gemm_f32_all_layouts(B, M, K, N):
     a, b = rs.randn(M, K).astype(np.float32), rs.randn(K, N).astype(np.float32)
