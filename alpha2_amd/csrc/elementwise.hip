@@ -48,8 +48,11 @@ struct UnBwd {
   int op; float p0, p1;
   __device__ __forceinline__ float operator()(float x, float g) const {
     switch (op) {
-      case AH_GELU_BWD: return g * gelu_grad_f(x);
-      case AH_RELU_BWD: return x > 0.f ? g : 0.f;
+      // gelu' is 1 / 0 beyond +-40 to the last bit; evaluated there, x^3 does not overflow f32 as it would from 7e12 on (the
+      // reference computes in f64, ops.ts:401-419).  NaN and the infinities go through as they are (the reference's formula
+      // gives NaN for both: 0 x inf).
+      case AH_GELU_BWD: { const float ax = fabsf(x); return g * gelu_grad_f(ax > 40.f && ax <= 3.402823466e38f ? copysignf(40.f, x) : x); }
+      case AH_RELU_BWD: return g * (x > 0.f ? 1.f : 0.f);       // a product with the mask, as the reference forms it (ops.ts:280-290): an infinite g at x <= 0 is NaN
       case AH_SILU_BWD: { float s = 1.0f / (1.0f + expf(-x)); return g * (s * (1.0f + x * (1.0f - s))); }
       case AH_CLAMP_BWD: return (x > p0 && x < p1) ? g : 0.f;
       default: { float t = tanhf(x / p0); return g * (1.0f - t * t); }   // AH_SOFTCAP_BWD

@@ -726,6 +726,24 @@ def test_cross_entropy_with_logits_far_from_zero(B, dtype, scale):
             assert np.all(np.isfinite(got)), entry
 
 
+def test_unary_backward_formulas_at_the_ends_of_the_range(B):
+    """Where f32 arithmetic and the reference's f64 could part ways: gelu' of huge inputs (x^3 overflows f32 from 7e12 on; the
+    derivative is 1 or 0 there, and 0 x inf = NaN at the infinities themselves, ops.ts:401-419), and relu's backward as a
+    product with the 0 / 1 mask (ops.ts:280-290: an infinite gradient where the input was not positive is NaN, not 0)."""
+    x = np.array([1e13, -1e13, 3.4e38, -3.4e38, 50.0, -50.0, np.inf, -np.inf, np.nan, 0.5], np.float32)
+    for gval in (1.0, -2.5, np.inf):
+        g = np.full(x.shape, gval, np.float32)
+        got, want = B.geluBackward(dev(B, x), dev(B, g)).data, ref.gelu_backward(orc(x), orc(g)).data
+        assert np.array_equal(np.isnan(got), np.isnan(want)), (gval, got, want)
+        ok = ~np.isnan(want)
+        assert np.allclose(got[ok], want[ok], rtol=1e-5, atol=1e-30), (gval, got, want)
+    xr = np.array([1.0, 0.0, -1.0, -0.0, np.nan, 2.0], np.float32)
+    gr = np.array([np.inf, np.inf, -np.inf, 3.0, 1.0, np.nan], np.float32)
+    got, want = B.reluBackward(dev(B, xr), dev(B, gr)).data, ref.relu_backward(orc(xr), orc(gr)).data
+    assert np.array_equal(np.isnan(got), np.isnan(want)) and np.array_equal(got[~np.isnan(want)], want[~np.isnan(want)]), (got, want)
+    assert np.isinf(got[0]) and np.isnan(got[1]) and np.isnan(got[2]) and got[3] == 0.0
+
+
 def test_clamp_keeps_nan(B):
     """max(lo, min(hi, x)) in the reference's arithmetic (cpu_ref.ts:358-360): Math.min / Math.max return NaN for a NaN."""
     x = np.array([np.nan, -3.0, 0.5, 7.0, np.inf, -np.inf], np.float32)
