@@ -673,6 +673,23 @@ int32_t ah_gemm(const AhGemm *p) {
   }
 
   AH_ARG(q.k % 8 == 0, "ah_gemm: bf16 contraction length %lld must be a multiple of 8", (long long)q.k);
+  ah_ptr zeros = 0;
+  if (q.k == 0) {
+    // A product over an empty contraction is all zeros (cpu_ref.ts:166-258 sums no terms), and the epilogue applies to that.
+    // It runs as an A B^T product with k = 64 whose operand rows all alias one stretch of 64 zeros (leading dimensions and
+    // batch strides 0), so every output type, epilogue and batch goes through the kernels it always goes through.
+    const uint64_t zbytes = 64 * 2;
+    int32_t rz = ah_alloc(zbytes, &zeros);
+    if (rz) return rz;
+    rz = ah_fill_i32(zeros, 0, zbytes / 4);
+    if (rz) { ah_free(zeros); return rz; }
+    ga.a = ga.b = dp<const void>(zeros);
+    ga.lda = ga.ldb = 0; ga.sa = ga.sb = 0;
+    ga.K = 64; ga.ksplit = 64;
+    int32_t rc0 = vec_c ? ah::gemm_bf16_direct(ga, AH_GEMM_NT, batch, q.out_dtype) : run_bf16_nt(ga, batch, q.out_dtype, vec_c);
+    int32_t rf = ah_free(zeros);      // stream-ordered: reusable only by later work
+    return rc0 ? rc0 : rf;
+  }
   {
     // direct kernel: every operand row (k-contiguous) or row group (k-major) must be 16-byte addressable
     bool akm = q.layout == AH_GEMM_TN, bkm = q.layout != AH_GEMM_NT;

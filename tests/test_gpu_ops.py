@@ -975,6 +975,39 @@ def _raw_gemm(B, layout, a, b, m, n, k, in_dtype, out_dtype, epi=0, aux=None, c_
     return out, aux_out
 
 
+@pytest.mark.parametrize("m,n", [(256, 192), (37, 20), (5, 3)])
+def test_gemm_over_an_empty_contraction(B, m, n):
+    """k = 0: the product is all zeros (cpu_ref.ts:166-258 sums no terms) and the epilogue applies to that, for bf16 operands in
+    every layout (leading dimensions at their minimum, 0 columns or 0 rows of operand) as for f32 ones: NONE writes zeros
+    over what was there, ACCUM leaves C, RESIDUAL copies the residual, GELU gives gelu(0) = 0 with a zero pre-activation."""
+    import ctypes as C
+    from alpha2_amd import TensorData, _ffi as ffi
+    c0, res = rs.randn(m, n).astype(np.float32), rs.randn(m, n).astype(np.float32)
+    for in_dtype in (ffi.BF16, ffi.F32):
+        for layout in (ffi.GEMM_NN, ffi.GEMM_NT, ffi.GEMM_TN):
+            dummy = TensorData((64,), "f32", np.ones(64, np.float32))          # never read: the operands have no elements
+            lda = {ffi.GEMM_NN: 0, ffi.GEMM_NT: 0, ffi.GEMM_TN: m}[layout]
+            ldb = {ffi.GEMM_NN: n, ffi.GEMM_NT: 0, ffi.GEMM_TN: n}[layout]
+            cases = [(ffi.F32, ffi.EPI_NONE, None, np.zeros((m, n), np.float32)), (ffi.F32, ffi.EPI_ACCUM, None, c0), (ffi.F32, ffi.EPI_RESIDUAL, res, res)]
+            if in_dtype == ffi.BF16:
+                cases += [(ffi.BF16, ffi.EPI_NONE, None, np.zeros((m, n), np.float32)), (ffi.BF16, ffi.EPI_RESIDUAL, res, _bf16_round(res)[0]),
+                          (ffi.BF16, ffi.EPI_GELU, np.ones((m, n), np.float32), np.zeros((m, n), np.float32))]
+            for out_dtype, epi, aux, want in cases:
+                store = lambda arr: (TensorData(arr.shape, "f16", _bf16_round(arr)[1]) if out_dtype == ffi.BF16 else TensorData(arr.shape, "f32", arr.copy()))
+                tc = store(c0)
+                taux = store(aux) if aux is not None else None
+                g = ffi.AhGemm(layout, in_dtype, out_dtype, epi, m, n, 0, lda, ldb, n, 1, 0, 0, 0, B._ptr(dummy), B._ptr(dummy), B._ptr(tc),
+                               B._ptr(taux) if taux is not None else 0)
+                ffi.check(B.lib.ah_gemm(C.byref(g)))
+                B._dirty(tc)
+                got = ((tc.data.astype(np.uint32) << 16).view(np.float32) if out_dtype == ffi.BF16 else tc.data).reshape(m, n)
+                exp = _bf16_round(want)[0] if out_dtype == ffi.BF16 else want
+                assert np.array_equal(got, exp), (in_dtype, layout, out_dtype, epi)
+                if epi == ffi.EPI_GELU:
+                    B._dirty(taux)
+                    assert not np.any(taux.data), "pre-activation of an empty product"
+
+
 @pytest.mark.parametrize("in_bf16,out_bf16", [(False, False), (True, False), (True, True)])
 @pytest.mark.parametrize("M,N,K", [(128, 128, 64), (256, 384, 96), (300, 200, 72), (1024, 768, 256)])
 def test_gemm_layouts_epilogues_dtypes(B, in_bf16, out_bf16, M, N, K):
