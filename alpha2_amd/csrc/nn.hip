@@ -1022,7 +1022,8 @@ int32_t ah_cross_entropy(ah_ptr logits, int32_t dtype, ah_ptr targets, ah_ptr lo
   AH_REQUIRE_READY();
   AH_ARG(dtype == AH_F32 || dtype == AH_BF16, "ah_cross_entropy: logits dtype must be f32 or bf16");
   AH_ARG(loss_out != 0, "ah_cross_entropy: null loss_out");
-  AH_ARG(n > 0 && c > 0, "ah_cross_entropy: empty logits [%lld, %lld]", (long long)n, (long long)c);
+  AH_ARG(n >= 0 && c >= 0, "ah_cross_entropy: negative extent [%lld, %lld]", (long long)n, (long long)c);
+  if (n == 0 || c == 0) return ah_fill_f32(loss_out, NAN, 1);      // a mean over no rows (0 / 0), or of entries that do not exist (cpu_ref.ts:543-563)
   AH_ARG(logits && targets, "ah_cross_entropy: null operand");
   AH_ARG(n < (int64_t(1) << 31), "ah_cross_entropy: too many rows");
   float *rows = (float *)scratch(sizeof(float) * (size_t)n);
@@ -1067,7 +1068,8 @@ int32_t ah_cross_entropy_fwd_bwd(ah_ptr logits, int32_t dtype, ah_ptr targets, a
   AH_REQUIRE_READY();
   AH_ARG(dtype == AH_F32 || dtype == AH_BF16, "ah_cross_entropy_fwd_bwd: logits dtype must be f32 or bf16");
   AH_ARG(loss_out != 0, "ah_cross_entropy_fwd_bwd: null loss_out");
-  AH_ARG(n > 0 && c > 0, "ah_cross_entropy_fwd_bwd: empty logits [%lld, %lld]", (long long)n, (long long)c);
+  AH_ARG(n >= 0 && c >= 0, "ah_cross_entropy_fwd_bwd: negative extent [%lld, %lld]", (long long)n, (long long)c);
+  if (n == 0 || c == 0) return ah_fill_f32(loss_out, NAN, 1);      // as ah_cross_entropy; there is no gradient to write
   AH_ARG(logits && targets && lse_out && dlogits, "ah_cross_entropy_fwd_bwd: null operand");
   AH_ARG(n < (int64_t(1) << 31), "ah_cross_entropy_fwd_bwd: too many rows");
   const bool one_pass = dtype == AH_BF16 && (c & 7) == 0 && (c >> 3) <= (int64_t)CE_CHUNKS * CE_TPB && ((logits | dlogits) & 15u) == 0;

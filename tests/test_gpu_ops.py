@@ -314,6 +314,10 @@ def test_empty_extents_give_what_the_cpu_path_gives(B):
     emb = B.embedding(dev(B, np.ones((5, 4), np.float32)), dev(B, np.zeros((0,), np.int32), "i32"))
     assert tuple(emb.shape) == (0, 4) and emb.data.size == 0
     assert float(B.totalSumOfSquares([]).data[0]) == 0.0 and float(B.sumOfSquares(dev(B, z(0))).data[0]) == 0.0
+    # the loss over no rows is a mean of nothing (cpu_ref.ts:543-563), its gradient has no entries
+    no_rows, no_targets = dev(B, z(0, 8)), dev(B, np.zeros(0, np.int32), "i32")
+    assert np.isnan(B.crossEntropy(no_rows, no_targets).data).all() and np.isnan(O.crossEntropy(orc(z(0, 8)), orc(np.zeros(0, np.int32))).data).all()
+    assert tuple(B.crossEntropyBackward(no_rows, no_targets, dev(B, np.ones((), np.float32))).shape) == (0, 8)
 
 
 def shape_size_of(t):
