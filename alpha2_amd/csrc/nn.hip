@@ -18,10 +18,10 @@ __global__ void k_embedding(const float *__restrict__ w, const int32_t *__restri
   if (row >= n_idx) return;
   int lane = threadIdx.x & 63;
   int64_t r = idx[row];
-  bool ok = r >= 0 && r < vocab;                 // an out-of-range id yields a zero row instead of a fault
-  const float *src = w + (ok ? r : 0) * dim;
+  bool ok = r >= 0 && r < vocab;                 // an out-of-range id yields a row of NaN, as reading past the weight array
+  const float *src = w + (ok ? r : 0) * dim;     // does in the reference's loop (cpu_ref.ts:364-385), and no fault
   OUT *dst = out + row * dim;
-  for (int64_t j = lane; j < dim; j += 64) Io<OUT>::st(dst, j, ok ? src[j] : 0.f);
+  for (int64_t j = lane; j < dim; j += 64) Io<OUT>::st(dst, j, ok ? src[j] : NAN);
 }
 template <class OUT>
 __global__ void k_embedding_tok_pos(const float *__restrict__ wte, const float *__restrict__ wpe, const int32_t *__restrict__ tok,
@@ -36,12 +36,12 @@ __global__ void k_embedding_tok_pos(const float *__restrict__ wte, const float *
   if ((dim & 3) == 0) {
     for (int64_t j = lane; j < (dim >> 2); j += 64) {
       float4 u = reinterpret_cast<const float4 *>(a)[j], v = reinterpret_cast<const float4 *>(b)[j];
-      if (!ok) u = make_float4(0, 0, 0, 0);
+      if (!ok) u = make_float4(NAN, NAN, NAN, NAN);      // (as k_embedding: what the reference's loop reads past the array)
       if constexpr (sizeof(OUT) == 4) reinterpret_cast<float4 *>(dst)[j] = make_float4(u.x + v.x, u.y + v.y, u.z + v.z, u.w + v.w);
       else reinterpret_cast<uint2 *>(dst)[j] = make_uint2(pack_bf16x2(u.x + v.x, u.y + v.y), pack_bf16x2(u.z + v.z, u.w + v.w));
     }
   } else {
-    for (int64_t j = lane; j < dim; j += 64) Io<OUT>::st(dst, j, (ok ? a[j] : 0.f) + b[j]);
+    for (int64_t j = lane; j < dim; j += 64) Io<OUT>::st(dst, j, (ok ? a[j] : NAN) + b[j]);
   }
 }
 // scatter-add with hardware f32 atomics (the reference's GPU kernel uses CAS-loop atomics:

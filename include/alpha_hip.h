@@ -249,6 +249,8 @@ int32_t ah_softmax_bwd(ah_ptr s, ah_ptr g, ah_ptr out, int64_t rows, int64_t dim
 /* ---- nn.  Backend.embedding / embeddingBackward (cpu_ref.ts:364-385; ops.ts:491-507),
  *      layerNorm / layerNormBackward (cpu_ref.ts:387-420; ops.ts:509-571),
  *      crossEntropy / crossEntropyBackward (cpu_ref.ts:543-563; ops.ts:702-729). ---- */
+/* out[i] = weight[idx[i]]; an id outside [0, vocab) gives a row of NaN, which is what the reference's loop stores when it
+ * reads past the weight array (cpu_ref.ts:364-385), and no access outside the array is made. */
 int32_t ah_embedding(ah_ptr weight, ah_ptr idx_i32, ah_ptr out, int64_t n_idx, int64_t dim, int64_t vocab,
                      int32_t out_dtype);
 /* out[i] = wte[tok[i]] + wpe[i % T]  -- tok+pos embedding and the add of gpt.ts:362-379 in one pass */

@@ -209,10 +209,11 @@ void orc_sum_axis(const float *a, const int64_t *shape, int nd, int ax, float *o
 }
 
 /* embedding: cpu_ref.ts:364-385 */
-void orc_embedding(const float *w, int64_t dim, const int32_t *idx, int64_t n, float *out) {
+void orc_embedding(const float *w, int64_t dim, int64_t vocab, const int32_t *idx, int64_t n, float *out) {
   for (int64_t i = 0; i < n; i++) {
     int64_t src = (int64_t)idx[i] * dim, dst = i * dim;
-    for (int64_t d = 0; d < dim; d++) out[dst + d] = w[src + d];
+    /* an element outside the weight array reads as undefined and is stored as NaN (typed-array semantics of the loop) */
+    for (int64_t d = 0; d < dim; d++) out[dst + d] = (src + d >= 0 && src + d < vocab * dim) ? w[src + d] : NAN;
   }
 }
 /* embedding backward (scatter-add, sequential in index order): packages/autograd/src/ops.ts:495-505 */
@@ -221,8 +222,11 @@ void orc_embedding_bwd(const int32_t *idx, int64_t n, const float *g, int64_t di
   memset(grad, 0, sizeof(float) * (size_t)(vocab * dim));
   for (int64_t i = 0; i < n; i++) {
     int64_t r = idx[i];
-    for (int64_t d = 0; d < dim; d++)
-      grad[r * dim + d] = (float)((double)grad[r * dim + d] + (double)g[i * dim + d]); /* Float32Array += */
+    for (int64_t d = 0; d < dim; d++) {
+      int64_t f = r * dim + d;
+      if (f < 0 || f >= vocab * dim) continue;    /* a store past either end of a typed array is dropped */
+      grad[f] = (float)((double)grad[f] + (double)g[i * dim + d]); /* Float32Array += */
+    }
   }
 }
 

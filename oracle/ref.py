@@ -267,7 +267,7 @@ class CpuRef:
         n = indices.data.size
         out = np.empty(n * dim, dtype=np.float32)
         idx = np.ascontiguousarray(indices.data, dtype=np.int32)
-        lib().orc_embedding(_fp(weight.data), _n(dim), _fp(idx), _n(n), _fp(out))
+        lib().orc_embedding(_fp(weight.data), _n(dim), _n(weight.shape[0]), _fp(idx), _n(n), _fp(out))
         return TD(tuple(indices.shape) + (dim,), "f32", out)
 
     def layerNorm(self, x: TD, weight: TD, bias: TD, eps: float) -> TD:

@@ -748,6 +748,28 @@ def test_unary_backward_formulas_at_the_ends_of_the_range(B):
     assert np.isinf(got[0]) and np.isnan(got[1]) and np.isnan(got[2]) and got[3] == 0.0
 
 
+def test_embedding_of_an_id_outside_the_table_is_a_row_of_nan(B):
+    """The reference's gather reads weight[id * dim + d] from a typed array: past either end that is undefined, stored as NaN
+    (cpu_ref.ts:364-385).  The device gives the same rows (also from the fused token + position gather) without touching
+    memory outside the table; the backward pass skips such ids, as a store past a typed array's end is dropped (ops.ts:491-507)."""
+    import ctypes as C
+    from alpha2_amd import _ffi as ffi
+    w = rs.randn(6, 8).astype(np.float32)
+    ids = np.array([0, 5, 6, -1, 3, 1 << 20, -(1 << 20)], np.int32)
+    got, want = B.embedding(dev(B, w), dev(B, ids, "i32")).data.reshape(len(ids), 8), O.embedding(orc(w), orc(ids)).data.reshape(len(ids), 8)
+    assert np.array_equal(got, want, equal_nan=True)
+    assert np.isnan(got[[2, 3, 5, 6]]).all() and np.array_equal(got[[0, 1, 4]], w[[0, 5, 3]])
+    wpe = rs.randn(len(ids), 8).astype(np.float32)
+    out = B._new((len(ids), 8))
+    tw, tp, ti = dev(B, w), dev(B, wpe), dev(B, ids, "i32")
+    ffi.check(B.lib.ah_embedding_tok_pos(B._ptr(tw), B._ptr(tp), B._ptr(ti), B._ptr(out), len(ids), len(ids), 8, 6, ffi.F32))
+    B._dirty(out)
+    both = out.data.reshape(len(ids), 8)
+    assert np.isnan(both[[2, 3, 5, 6]]).all() and np.array_equal(both[[0, 1, 4]], (w[[0, 5, 3]] + wpe[[0, 1, 4]]))
+    g = rs.randn(len(ids), 8).astype(np.float32)
+    assert_close(B.embeddingBackward(dev(B, ids, "i32"), dev(B, g), 6).data, ref.embedding_backward(orc(ids), orc(g), 6).data, what="embedding backward with ids outside")
+
+
 def test_clamp_keeps_nan(B):
     """max(lo, min(hi, x)) in the reference's arithmetic (cpu_ref.ts:358-360): Math.min / Math.max return NaN for a NaN."""
     x = np.array([np.nan, -3.0, 0.5, 7.0, np.inf, -np.inf], np.float32)

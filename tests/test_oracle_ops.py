@@ -366,3 +366,15 @@ def test_sum_and_mean_over_an_empty_axis():
     s0 = B.sum(ref.f32(np.zeros((0, 8), np.float32)), 0)
     assert s0.shape == (8,) and np.array_equal(s0.data[:8], np.zeros(8, np.float32))
     assert np.isnan(B.mean(ref.f32(np.zeros((0,), np.float32))).data[0])
+
+
+def test_embedding_with_ids_outside_the_table():
+    """cpu_ref.ts:364-385 reads weight[id * dim + d] from a typed array: undefined past either end, stored as NaN; the backward
+    loop's store past the end is dropped (ops.ts:491-507).  No access outside the arrays on this side either."""
+    w = np.arange(12, dtype=np.float32).reshape(3, 4)
+    ids = np.array([2, 3, -1, 0], np.int32)
+    out = B.embedding(ref.f32(w), ref.i32(ids)).data.reshape(4, 4)
+    assert np.array_equal(out[[0, 3]], w[[2, 0]]) and np.isnan(out[[1, 2]]).all()
+    g = np.ones((4, 4), np.float32)
+    gw = ref.embedding_backward(ref.i32(ids), ref.f32(g), 3).data.reshape(3, 4)
+    assert np.array_equal(gw, np.array([[1] * 4, [0] * 4, [1] * 4], np.float32))
