@@ -348,6 +348,8 @@ class FastHipBackend(HipBackend):
         M, K, N = a.shape[0], a.shape[1], b.shape[0]
         if b.shape[1] != K:
             raise ValueError(f"matmul shape mismatch: [{a.shape}] x [{b.shape}]^T")
+        if K % 8:                                               # the bf16 kernels contract in 16-byte pieces: such a product runs in f32
+            return super().matmulTransposed(a, b)
         return self._hold_gemm(ffi.GEMM_NT, a, b, (M, N), M, N, K, K, K)
 
     def matmul(self, a: TensorData, b: TensorData) -> TensorData:
@@ -356,6 +358,8 @@ class FastHipBackend(HipBackend):
         M, K, N = a.shape[0], a.shape[1], b.shape[1]
         if b.shape[0] != K:
             raise ValueError(f"matmul shape mismatch: [{a.shape}] x [{b.shape}]")
+        if K % 8:
+            return super().matmul(a, b)
         return self._hold_gemm(ffi.GEMM_NN, a, b, (M, N), M, N, K, K, N)
 
     def gelu(self, a: TensorData) -> TensorData:
@@ -410,6 +414,8 @@ class FastHipBackend(HipBackend):
         M, K, N = a.shape[0], a.shape[1], b.shape[1]
         if b.shape[0] != M:
             raise ValueError(f"matmul shape mismatch: [{a.shape}]^T x [{b.shape}]")
+        if M % 8:                                               # (the contraction runs over the rows here)
+            return super().matmulTransposedA(a, b)
         ap, ah = self._operand(a)
         bp, bh = self._operand(b)
         out = self._new((K, N))

@@ -398,3 +398,26 @@ def test_cross_entropy_is_held_until_its_backward_is_asked_for(FB):
     FB.releaseGpuTensor(loss)
     FB.flush()
     assert FB._held_ce is None
+
+
+@pytest.mark.parametrize("cfg", [
+    dict(vocabSize=7, blockSize=1, nLayer=1, nEmbd=8, nHead=1),                              # one token per row, a vocabulary of 7
+    dict(vocabSize=33, blockSize=3, nLayer=2, nEmbd=12, nHead=3),                            # head size 4, nothing a multiple of 8
+    dict(vocabSize=96, blockSize=5, nLayer=1, nEmbd=64, nHead=2),                            # 5 or 15 tokens: the weight gradients contract over them
+    dict(vocabSize=50, blockSize=17, nLayer=1, nEmbd=32, nHead=1, ffnActivation="swiglu"),
+])
+@pytest.mark.parametrize("batch,accum", [(1, 1), (3, 2)])
+def test_shapes_the_bf16_kernels_do_not_take_run_in_f32_behind_the_interface(FB, cfg, batch, accum):
+    """A caller of the interface picks any model shape: products whose contraction length is not a multiple of 8 (the bf16
+    kernels load 16 bytes at a time) run through the f32 kernels instead of being refused, head sizes without a flash
+    kernel through the unfused chain; two steps track the oracle as every other shape does."""
+    from alpha2_amd.model import ModelConfig
+    from alpha2_amd.train import TrainConfig, Trainer, syntheticBatch
+    tr = Trainer(FB, ModelConfig(**cfg), TrainConfig(iters=4, gradAccumSteps=accum), seed=2)
+    orc = rm.Trainer(rm.ModelConfig(**cfg), rm.TrainConfig(iters=4, gradAccumSteps=accum), seed=2)
+    for s in range(2):
+        bs = [syntheticBatch(9 + 2 * s + m, batch, cfg["blockSize"], cfg["vocabSize"]) for m in range(accum)]
+        ob = [rm.synthetic_batch(9 + 2 * s + m, batch, cfg["blockSize"], cfg["vocabSize"]) for m in range(accum)]
+        r, o = tr.step(bs), orc.step(ob)
+        assert abs(r.loss - o.loss) <= 2e-2 * abs(o.loss), (s, r.loss, o.loss)
+        assert abs(r.gradNorm - o.gradNorm) <= 1e-1 * o.gradNorm, (s, r.gradNorm, o.gradNorm)
