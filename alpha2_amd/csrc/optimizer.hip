@@ -211,7 +211,7 @@ __global__ __launch_bounds__(256) void k_af_vrmean(const float *__restrict__ vr,
   double s = 0;
   for (int64_t r = threadIdx.x; r < rows; r += blockDim.x) s += (double)vr[r];
   s = block_sum_f64(s, sh);
-  if (threadIdx.x == 0) { double mean = s * (1.0 / (double)rows); ws[0] = 1.0 / (mean > eps ? mean : eps); }
+  if (threadIdx.x == 0) { double mean = s * (1.0 / (double)rows); ws[0] = 1.0 / ((mean > eps || mean != mean) ? mean : eps); }      // Math.max(mean, eps): a NaN stays one (optimizers.ts:450)
 }
 __device__ __forceinline__ double af_denom(const float *vr, const float *vc, int64_t r, int64_t c, double inv_vr_mean, double eps) {
   double d = sqrt((double)vr[r] * inv_vr_mean) * sqrt((double)vc[c]);
@@ -245,7 +245,8 @@ __global__ void k_af_step_scale(const double *__restrict__ part, int nblk, uint6
     double s = 0;
     for (int b = 0; b < nblk; b++) s += part[b];
     double rms = sqrt(s / (double)(n > 1 ? n : 1));
-    double den = h.clip_threshold > 0 ? (rms / h.clip_threshold > 1.0 ? rms / h.clip_threshold : 1.0) : 1.0;
+    const double q = rms / h.clip_threshold;
+    double den = h.clip_threshold > 0 ? ((q > 1.0 || q != q) ? q : 1.0) : 1.0;      // Math.max(1, rms / clip): a NaN stays one (optimizers.ts:466,499)
     ws[1] = h.lr / den;
   }
 }

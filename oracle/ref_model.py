@@ -761,6 +761,11 @@ class Lion:
         return {"step": self._step, "buffers": {name + ".m": TD((m.size,), "f32", m.copy()) for name, m in self.m.items()}}
 
 
+def _js_max(a: float, b: float) -> float:
+    """Math.max: NaN if either argument is NaN (Python's max keeps whichever argument the comparison does not displace)."""
+    return float("nan") if (a != a or b != b) else max(a, b)
+
+
 class Adafactor:
     """optimizers.ts:349-543."""
 
@@ -793,7 +798,7 @@ class Adafactor:
                 vr[r] = np.float32(beta2 * float(vr[r]) + (1 - beta2) * (_seq_sum(g2[r]) * (1 / cols)) + eps)
             for c in range(cols):
                 vc[c] = np.float32(beta2 * float(vc[c]) + (1 - beta2) * (_seq_sum(g2[:, c]) * (1 / rows)) + eps)
-            vr_mean = max(_seq_sum(vr) * (1 / rows), eps)
+            vr_mean = _js_max(_seq_sum(vr) * (1 / rows), eps)
             r_scale = np.sqrt(vr.astype(np.float64) * (1 / vr_mean))
             denom = np.maximum(eps, r_scale[:, None] * np.sqrt(vc.astype(np.float64))[None, :]).reshape(-1)
         else:                                                        # optimizers.ts:478-500
@@ -804,7 +809,7 @@ class Adafactor:
             denom = np.sqrt(v.astype(np.float64))
         upd = g / denom
         rms = math.sqrt(_seq_sum(upd * upd) / max(1, size))
-        clip_den = max(1.0, rms / self.clip) if self.clip > 0 else 1.0
+        clip_den = _js_max(1.0, rms / self.clip) if self.clip > 0 else 1.0
         step_scale = lr / clip_den
         flat = p.reshape(-1)
         if wd > 0:

@@ -156,6 +156,43 @@ def test_adafactor_kernels_match_the_host_loops(B, shape):
         np.testing.assert_allclose(dd[key].data, od[key].data, rtol=1e-6, atol=0)
 
 
+def test_adafactor_with_a_gradient_that_is_not_finite_poisons_the_whole_tensor():
+    """Math.max(1, rms / clip) is NaN when the update's RMS is (optimizers.ts:465-466,498-499), and the step scale with it:
+    one NaN or infinite gradient entry makes every parameter of the tensor NaN, in both branches (Python's max would keep 1)."""
+    for shape in ((6,), (2, 3)):
+        p = np.arange(1, 7, dtype=np.float32)
+        g = np.array([0.1, -0.2, np.nan, 0.3, 0.4, -0.5], dtype=np.float32)
+        M.Adafactor(lr=1e-2, beta2=0.99, eps=1e-30, clipThreshold=1.0, weightDecay=0.0).stepParamEntries(_entries(p, g, shape))
+        assert np.isnan(p).all(), (shape, p)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(12,), (3, 4)])
+def test_optimizer_kernels_on_gradients_at_the_ends_of_the_range(B, shape):
+    """Infinite, NaN, denormal and largest-finite gradient entries through two steps of each optimizer: the device gives what the
+    host loops give, NaN for NaN (sign(NaN), Math.max with a NaN) included."""
+    from alpha2_amd import TensorData
+    from alpha2_amd.optimizers import Adafactor, Lion, SGD
+    p0 = np.array([1.0, -2.0, 0.5, 3.0, 0.0, -0.0, 1e-30, 1e30, 7.0, -7.0, 2.0, 2.0], np.float32)
+    g0 = np.array([np.inf, -np.inf, np.nan, 0.0, -0.0, 1e-45, 3.4e38, -3.4e38, 1e-20, -1e-20, 1.0, -1.0], np.float32)
+    makers = (("lion", lambda: M.Lion(lr=3e-3, beta1=0.9, beta2=0.95, weightDecay=0.1), lambda: Lion(B, lr=3e-3, beta1=0.9, beta2=0.95, weightDecay=0.1)),
+              ("sgd", lambda: M.SGD(0.05), lambda: SGD(B, 0.05)),
+              ("adafactor", lambda: M.Adafactor(lr=1e-2, beta2=0.99, eps=1e-30, clipThreshold=1.0, weightDecay=0.05),
+               lambda: Adafactor(B, lr=1e-2, beta2=0.99, eps=1e-30, clipThreshold=1.0, weightDecay=0.05)))
+    for name, mk_o, mk_d in makers:
+        for g in (g0, np.where(np.isfinite(g0), g0, 1.0).astype(np.float32)):
+            want, o, d = p0.copy(), mk_o(), mk_d()
+            ent = _dev_entries(B, p0, g, shape)
+            for k in range(2):
+                o.stepParamEntries(_entries(want, g, shape), 0.5)
+                ent[0][1].grad = TensorData(shape, "f32", g.copy())
+                d.stepParamEntries(ent, 0.5)
+            got = np.asarray(ent[0][1].data.data).reshape(-1)
+            assert np.array_equal(np.isnan(got), np.isnan(want)), (name, got, want)
+            ok = ~np.isnan(want)
+            np.testing.assert_allclose(got[ok], want[ok], rtol=2e-6, atol=1e-37, err_msg=name)
+
+
 @pytest.mark.gpu
 def test_optimizer_registry_and_state_round_trip(B):
     from alpha2_amd import TensorData
