@@ -47,11 +47,12 @@ class _HeldGemm:
 
 
 class _HeldWeightGrad:
-    __slots__ = ("g_ptr", "x_ptr", "out_buf", "out_off", "m", "n", "k", "holds", "into")
+    __slots__ = ("g_ptr", "x_ptr", "out_buf", "out_off", "m", "n", "k", "holds", "into", "add_after")
 
     def __init__(self, g_ptr, x_ptr, out, m, n, k, holds):
         self.g_ptr, self.x_ptr, self.out_buf, self.out_off, self.m, self.n, self.k, self.holds = g_ptr, x_ptr, out._buf, out._off, m, n, k, holds
         self.into = None                  # (buffer, offset) of an existing gradient to accumulate into instead
+        self.add_after = None             # set at launch: the same, when the product had to be computed into its own tensor
 
 
 class _HeldLayerNormBwd:
@@ -429,13 +430,19 @@ class FastHipBackend(HipBackend):
         self._run_weight_grads(*self._take_weight_grads())
 
     def _take_weight_grads(self):
-        """Empties the queue: (the queued products, [(epilogue, descriptors, as one grouped launch?)])."""
+        """Empties the queue: (the queued products, [(epilogue, descriptors, as one grouped launch?)]).  A product that was
+        re-targeted to accumulate into an existing gradient (addInplace) while its own tensor is still alive - the tape
+        releases it at once, another caller may not - is computed into its own tensor after all, and added from there:
+        its entry in ws carries the sum still to be made."""
         ws, self._wgrads = self._wgrads, []
         self._wq_out, self._wq_into = set(), set()
         descs = []
         for w in ws:
+            w.add_after = None
             if w.into is None and w.out_buf.refs == 1:          # released unread
                 continue
+            if w.into is not None and w.out_buf.refs > 1:       # (the queue's own hold is one reference)
+                w.add_after, w.into = w.into, None
             dst, epi = (w.out_buf.ptr + w.out_off, ffi.EPI_NONE) if w.into is None else (w.into[0].ptr + w.into[1], ffi.EPI_ACCUM)
             descs.append(ffi.AhGemm(ffi.GEMM_TN, BF16, F32, epi, w.m, w.n, w.k, w.m, w.n, w.n, 1, 0, 0, 0, w.g_ptr, w.x_ptr, dst, 0))
         groupable = all(d.k % 64 == 0 and d.m % 8 == 0 and d.n % 8 == 0 for d in descs)
@@ -486,13 +493,16 @@ class FastHipBackend(HipBackend):
                 for d in part:
                     check(self.lib.ah_gemm(C.byref(d)))
         for w in ws:
+            if w.add_after is not None:
+                check(self.lib.ah_add_inplace(w.add_after[0].ptr + w.add_after[1], w.out_buf.ptr + w.out_off, w.m * w.n))
             self._unhold(w.holds)
 
     def addInplace(self, a: TensorData, b: TensorData):
         if self._wgrads and b._buf is not None and id(b._buf) in self._wq_out:
             for w in self._wgrads:
                 if b._buf is w.out_buf and w.into is None and a.store == "f32" and a.size == b.size and a._buf is not None and a._dev_valid \
-                        and a._buf.refs == 1 and id(a._buf) not in self._wq_out and id(a._buf) not in self._wq_into:
+                        and a._buf.refs == 1 and id(a._buf) not in self._wq_out and id(a._buf) not in self._wq_into \
+                        and not any(a._buf is x for x in w.holds):      # (`a` may be an operand of the very product: it cannot be written while it is read)
                     w.into = (a._buf, a._off)                    # the grouped launch adds into `a`; `b` itself is never computed
                     a._buf.refs += 1
                     w.holds.append(a._buf)
@@ -724,7 +734,7 @@ class FastHipBackend(HipBackend):
                 ws, parts = self._take_weight_grads()
                 covered = {d.c: d.m * d.n for _, part, grouped in parts if grouped for d in part}
                 listed = {k: t.size for k, t in zip(key, tensors)}
-                if covered and all(listed.get(a) == n for a, n in covered.items()):
+                if covered and all(listed.get(a) == n for a, n in covered.items()) and not any(w.add_after is not None for w in ws):
                     total = self._new((1,))
                     rest = [(k, t.size) for k, t in zip(key, tensors) if k not in covered]
                     if rest:

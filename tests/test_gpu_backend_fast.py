@@ -421,3 +421,62 @@ def test_shapes_the_bf16_kernels_do_not_take_run_in_f32_behind_the_interface(FB,
         r, o = tr.step(bs), orc.step(ob)
         assert abs(r.loss - o.loss) <= 2e-2 * abs(o.loss), (s, r.loss, o.loss)
         assert abs(r.gradNorm - o.gradNorm) <= 1e-1 * o.gradNorm, (s, r.gradNorm, o.gradNorm)
+
+
+def test_a_product_added_into_a_gradient_is_still_its_tensors_value_when_that_is_kept(FB):
+    """addInplace(acc, product) makes a queued weight gradient accumulate into `acc` and skips the product's own tensor, which
+    the tape releases at once (tape.ts:116-127).  A caller that keeps it must find the product in it all the same, and the sum
+    in `acc`."""
+    rs = np.random.RandomState(12)
+    g, x, a0 = rs.randn(64, 32) * 0.3, rs.randn(64, 48) * 0.5, rs.randn(32, 48)
+    want = _bf16(g).astype(np.float64).T @ _bf16(x).astype(np.float64)
+    acc = FB.scale(_td(a0), 1.0)
+    out = FB.matmulTransposedA(_td(g), _td(x))
+    FB.addInplace(acc, out)                                      # `out` is not released
+    kept = FB.matmulTransposedA(_td(g), _td(x))                  # a second one, released as the tape does
+    FB.addInplace(acc, kept)
+    FB.releaseGpuTensor(kept)
+    _close(out.data, want, "the product whose tensor was kept", tol=1e-3)
+    _close(acc.data, a0 + 2 * want, "the sum", tol=1e-3)
+
+
+def test_random_op_programs_give_what_eager_execution_gives(FB):
+    """Random programs over a pool of [16, 16] tensors - products of all three kinds, gelu and its backward, sums, in-place
+    sums and scalings, copy-on-write clones, releases, reads and norms in any order - on the fast backend (held products,
+    queued gradients, shared buffers) against the same programs on the eager f32 backend.  A slip of the lazy machinery (a
+    stale buffer, a sum made twice, a product never computed) is a difference of the size of the values; bf16 storage a few
+    percent of it."""
+    from alpha2_amd import HipBackend, TensorData
+    HB, N = HipBackend(0), 16
+    kinds = ["mmT", "mm", "mmTA", "gelu", "geluB", "add", "addI", "scale", "scaleI", "clone", "release", "read", "ssq", "relu"]
+    probs = [.14, .08, .08, .08, .05, .1, .08, .04, .04, .09, .07, .09, .03, .03]
+
+    def run(Bk, init, ops):
+        pool, reads = [TensorData((N, N), "f32", v.copy()) for v in init], []
+        for kind, i, j, sc in ops:
+            a, b = pool[i % len(pool)], pool[j % len(pool)]
+            if kind == "mmT": pool.append(Bk.matmulTransposed(a, b))
+            elif kind == "mm": pool.append(Bk.matmul(a, b))
+            elif kind == "mmTA": pool.append(Bk.matmulTransposedA(a, b))
+            elif kind == "gelu": pool.append(Bk.gelu(a))
+            elif kind == "geluB": pool.append(Bk.geluBackward(a, b))
+            elif kind == "relu": pool.append(Bk.relu(a))
+            elif kind == "add": pool.append(Bk.add(a, b))
+            elif kind == "addI" and a is not b: Bk.addInplace(a, b)
+            elif kind == "scale": pool.append(Bk.scale(a, sc))
+            elif kind == "scaleI": Bk.scaleInplace(a, sc * 0.7)
+            elif kind == "clone": pool.append(Bk.clone(a))
+            elif kind == "release" and len(pool) > 2: Bk.releaseGpuTensor(pool.pop(i % len(pool)))
+            elif kind == "read": reads.append(np.array(a.data, dtype=np.float32).reshape(-1).copy())
+            elif kind == "ssq": reads.append(np.array(Bk.totalSumOfSquares([a, b] if a is not b else [a]).data, dtype=np.float32).reshape(-1).copy())
+        reads += [np.array(t.data, dtype=np.float32).reshape(-1).copy() for t in pool]
+        Bk.syncGpu()
+        return reads
+    for seed in range(120):
+        rs = np.random.RandomState(seed)
+        init = [rs.randn(N, N).astype(np.float32) * 0.25 for _ in range(4)]
+        ops = [(str(rs.choice(kinds, p=probs)), int(rs.randint(0, 1 << 30)), int(rs.randint(0, 1 << 30)), float(rs.uniform(0.5, 1.5))) for _ in range(60)]
+        for k, (got, want) in enumerate(zip(run(FB, init, ops), run(HB, init, ops))):
+            fin = np.isfinite(want)
+            size = float(np.abs(want[fin]).max()) if fin.any() else 1.0
+            assert got.shape == want.shape and float(np.abs(got[fin] - want[fin]).max(initial=0)) <= 0.1 * size + 1e-3, (seed, k, size)
