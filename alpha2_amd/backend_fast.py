@@ -727,14 +727,16 @@ class FastHipBackend(HipBackend):
                 return (None,)
         if self._wgrads and not self._adam_q:
             # The queued weight gradients are about to be computed by grouped launches: let those sum the squares of what
-            # they store, and read only the other gradients again.  Every result of such a launch must be one of the listed
-            # tensors, whole; otherwise the launches run as they are and the list is read as usual.
+            # they store, and read only the other gradients again.  Every queued product must then go out in a grouped launch
+            # (one that runs on its own would be read by the list before it is computed) and every result must be one of the
+            # listed tensors, whole; otherwise the launches run as they are and the list is read as usual.
             key = addresses()
             if None not in key and len(set(key)) == len(key):
                 ws, parts = self._take_weight_grads()
                 covered = {d.c: d.m * d.n for _, part, grouped in parts if grouped for d in part}
                 listed = {k: t.size for k, t in zip(key, tensors)}
-                if covered and all(listed.get(a) == n for a, n in covered.items()) and not any(w.add_after is not None for w in ws):
+                if covered and all(grouped for _, _, grouped in parts) and all(listed.get(a) == n for a, n in covered.items()) \
+                        and not any(w.add_after is not None for w in ws):
                     total = self._new((1,))
                     rest = [(k, t.size) for k, t in zip(key, tensors) if k not in covered]
                     if rest:
@@ -778,6 +780,13 @@ class FastHipBackend(HipBackend):
             self._adam_key = key
             self._adam_hyper(lr, beta1, beta2, eps, 0.0, bc1, bc2, gradScale)      # the device copy of the scalars, once per pass
         sh = getattr(params, "_shadow", None)
+        if sh is not None and self._orphans:
+            # a product whose plain result was never written (its epilogue went elsewhere) and whose tensor is still alive
+            # would be computed later from this shadow, which the update rewrites in place: compute it from the old weights now
+            for key in [k for k, h in self._orphans.items() if any(b is sh for b in h.holds)]:
+                h = self._orphans.pop(key)
+                self._gemm(h.layout, h.a_ptr, h.b_ptr, h.out_ptr, h.m, h.n, h.k, h.lda, h.ldb, h.n, in_dtype=BF16, out_dtype=BF16)
+                self._unhold(h.holds)
         self._adam_q.append((*ptrs, sh.ptr if sh is not None else 0, params.size, weightDecay))
         for b in (params._buf, grads._buf, m._buf, v._buf) + ((sh,) if sh is not None else ()):
             b.refs += 1

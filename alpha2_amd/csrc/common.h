@@ -18,10 +18,13 @@ int32_t     hip_fail(hipError_t e, const char *what);
 void        count_op();
 int         num_cus();
 // Scratch for two-stage reductions: a library-owned device buffer of at least `bytes` bytes that stays
-// valid until the next call that asks for scratch on the same stream (calls are stream-ordered).
+// valid until the next call that asks for scratch on the same stream (calls are stream-ordered).  There is ONE buffer,
+// ordered by the main stream: between ah_side_begin and ah_side_end it is refused (nullptr), as is growing it while a
+// graph or step plan exists.
 void       *scratch(size_t bytes);
 int         current_device();                     // the device ah_init was called with
 int32_t     static_partials_init(int device);     // reduce.hip: device address of its static scratch array (called by ah_init)
+void        gemm_plans_forget();                  // gemm.hip: every grouped-GEMM plan id becomes unknown (called by ah_shutdown)
 
 // Every kernel of the library is launched through launch_kernel(): the arguments are converted to the kernel's parameter
 // types and handed, as an array of pointers to them, to launch_raw (runtime.hip).  Outside a step plan that is

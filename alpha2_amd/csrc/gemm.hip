@@ -327,7 +327,13 @@ std::vector<int64_t> group_shape(const AhGemm *descs, int count) {
   for (int i = 0; i < count; i++) { const AhGemm &q = descs[i]; v.insert(v.end(), {q.m, q.n, q.k, q.lda, q.ldb, q.ldc}); }
   return v;
 }
-std::vector<GroupPlan> g_plans;      // plan id = index + 1
+std::vector<GroupPlan> g_plans;      // plan id = g_plan_base + index + 1
+uint64_t g_plan_base = 0;            // ids handed out in earlier lives of the library (before an ah_shutdown): never valid again
+GroupPlan *find_plan(uint64_t id) {
+  if (id <= g_plan_base || id - g_plan_base > g_plans.size()) return nullptr;
+  GroupPlan &p = g_plans[id - g_plan_base - 1];
+  return p.live ? &p : nullptr;
+}
 
 // C += ws, ws = 0 for every k-split problem of a grouped launch: block (x, y) walks the float4s of part y.  The workspace
 // is left all zero, so the second halves of an ACCUMULATING run (whose epilogue adds to what it finds) store into it just
@@ -400,6 +406,14 @@ std::vector<int> split_tail(const AhGemm *descs, int count, int64_t blocks) {
   return chosen;
 }
 }  // namespace
+
+namespace ah {
+// ah_shutdown frees every device allocation, the plans' tables and workspaces among them: their ids must stop working.
+void gemm_plans_forget() {
+  g_plan_base += g_plans.size();
+  g_plans.clear();
+}
+}  // namespace ah
 
 extern "C" {
 
@@ -509,14 +523,14 @@ int32_t ah_gemm_grouped_plan(const AhGemm *descs, int32_t count, uint64_t *plan_
     return rc;
   }
   g_plans.push_back(plan);
-  *plan_out = g_plans.size();
+  *plan_out = g_plan_base + g_plans.size();
   return AH_OK;
 }
 
 int32_t ah_gemm_grouped_update(uint64_t plan, const AhGemm *descs, int32_t count) {
   AH_REQUIRE_READY();
-  AH_ARG(plan >= 1 && plan <= g_plans.size() && g_plans[plan - 1].live, "ah_gemm_grouped_update: unknown plan %llu", (unsigned long long)plan);
-  const GroupPlan &p = g_plans[plan - 1];
+  AH_ARG(find_plan(plan) != nullptr, "ah_gemm_grouped_update: unknown plan %llu", (unsigned long long)plan);
+  const GroupPlan &p = *find_plan(plan);
   std::vector<GemmGroupEntry> tab;
   std::vector<JoinPart> parts;
   int64_t blocks = 0, ws_bytes = 0;
@@ -535,8 +549,8 @@ int32_t ah_gemm_grouped_update(uint64_t plan, const AhGemm *descs, int32_t count
 // The launches of a plan; with sumsq_inout also the sum of the squares of everything they leave in the C matrices.
 static int32_t grouped_run(const char *who, uint64_t plan, int32_t epilogue, ah_ptr sumsq_inout) {
   AH_REQUIRE_READY();
-  AH_ARG(plan >= 1 && plan <= g_plans.size() && g_plans[plan - 1].live, "%s: unknown plan %llu", who, (unsigned long long)plan);
-  const GroupPlan &p = g_plans[plan - 1];
+  AH_ARG(find_plan(plan) != nullptr, "%s: unknown plan %llu", who, (unsigned long long)plan);
+  const GroupPlan &p = *find_plan(plan);
   AH_ARG(epilogue == AH_EPI_NONE || (epilogue == AH_EPI_ACCUM && p.out_dtype == AH_F32), "%s: epilogue %d is not provided for this plan", who, epilogue);
   const bool sums = sumsq_inout != 0;
   if (sums && p.out_dtype != AH_F32) return fail(AH_ERR_UNSUPPORTED, "%s: the sum of squares is provided for f32 outputs", who);
@@ -571,8 +585,8 @@ int32_t ah_gemm_grouped_run_sumsq(uint64_t plan, int32_t epilogue, ah_ptr sumsq_
 
 int32_t ah_gemm_grouped_destroy(uint64_t plan) {
   AH_REQUIRE_READY();
-  AH_ARG(plan >= 1 && plan <= g_plans.size() && g_plans[plan - 1].live, "ah_gemm_grouped_destroy: unknown plan %llu", (unsigned long long)plan);
-  GroupPlan &p = g_plans[plan - 1];
+  AH_ARG(find_plan(plan) != nullptr, "ah_gemm_grouped_destroy: unknown plan %llu", (unsigned long long)plan);
+  GroupPlan &p = *find_plan(plan);
   p.live = false;
   if (p.sumsq) ah_free(p.sumsq);
   p.sumsq = 0;

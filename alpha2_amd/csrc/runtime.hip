@@ -135,10 +135,12 @@ int32_t hip_fail(hipError_t e, const char *what) {
   return AH_ERR_HIP;
 }
 void *scratch(size_t bytes) {
+  if (g.cur != g.stream) return nullptr;      // side-stream work would race with main-stream users of the one buffer
   if (bytes <= g.scratch_bytes) return g.scratch;
-  // Growing scratch is only legal while no graph exists or is being captured (a graph replays into the addresses it
-  // was captured with); ah_init sizes it for every reduction this library launches, so this branch is a safety net.
-  if (g.capturing || !g.graphs.empty()) return nullptr;
+  // Growing scratch is only legal while no graph or step plan exists or is being captured (their nodes replay into the
+  // addresses they were recorded with, and a capturing stream cannot be synchronised); ah_init sizes it for every
+  // reduction this library launches, so this branch is a safety net.  Callers fail with AH_ERR_OOM on nullptr.
+  if (g.capturing || !g.graphs.empty() || !g.plans.empty() || g.step_capture_open || g.step_mode != STEP_OFF) return nullptr;
   (void)hipStreamSynchronize(g.stream);
   if (g.scratch) (void)hipFree(g.scratch);
   g.scratch = nullptr; g.scratch_bytes = 0;
@@ -153,10 +155,7 @@ constexpr size_t STEP_UPLOAD_MAX = size_t(16) << 20;     // larger uploads insid
 // A segment is closed after this many launches even when the host does not need the stream: on replay the graph of a
 // chunk is launched as soon as its last launch has been verified, so the device works on chunk k while the host is still
 // issuing (verifying) chunk k+1 -- the overlap eager execution has, at graph-launch cost.
-size_t step_chunk() {
-  static const size_t n = [] { const char *e = getenv("AH_STEP_CHUNK"); long v = e ? atol(e) : 0; return v > 0 ? (size_t)v : (size_t)32; }();
-  return n;
-}
+constexpr size_t STEP_CHUNK = 32;
 
 __global__ void k_step_copy(char *__restrict__ dst, const char *__restrict__ src, uint64_t bytes) {
   uint64_t tid = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x, stride = (uint64_t)gridDim.x * blockDim.x;
@@ -267,9 +266,8 @@ void launch_raw(const void *func, dim3 grid, dim3 block, unsigned shmem, void **
     else g.plan->broken = true;            // cannot name the node: this plan will not be replayed
     // After a boundary the host made, the device is idle until the first chunk has been issued: chunks start small there
     // (4, 8, 16, ... launches) and grow to the full size.
-    static const bool no_ramp = [] { const char *e = getenv("AH_STEP_RAMP"); return e && e[0] == '0'; }();
-    const size_t ramp = (!no_ramp && g.chunks_since_host_boundary < 3) ? (size_t(4) << g.chunks_since_host_boundary) : step_chunk();
-    if (sg.ops.size() >= (ramp < step_chunk() ? ramp : step_chunk()) && step_boundary("chunk") == AH_OK) {
+    const size_t chunk = g.chunks_since_host_boundary < 3 ? (size_t(4) << g.chunks_since_host_boundary) : STEP_CHUNK;
+    if (sg.ops.size() >= chunk && step_boundary("chunk") == AH_OK) {
       g.chunks_since_host_boundary++;
       (void)step_begin_capture();
     }
@@ -280,11 +278,8 @@ void launch_raw(const void *func, dim3 grid, dim3 block, unsigned shmem, void **
   if (g.op < sg.ops.size() && same_launch(sg.ops[g.op], func, grid, block, shmem, sizes, nargs)) {
     StepOp &o = sg.ops[g.op];
     bool differ = false;
-    static const bool debug = getenv("AH_STEP_DEBUG") != nullptr;
     for (int i = 0; i < nargs; i++)
       if (memcmp(o.blob.data() + o.off[i], args[i], sizes[i]) != 0) {
-        if (debug) fprintf(stderr, "[ah step] seg %zu launch %zu %s: argument %d (%u bytes) differs\n", g.seg, g.op,
-                           hipKernelNameRefByPtr(func, g.stream), i, sizes[i]);
         memcpy(o.blob.data() + o.off[i], args[i], sizes[i]);
         differ = true;
       }
@@ -408,6 +403,7 @@ int32_t ah_shutdown(void) {
   (void)hipStreamSynchronize(g.stream);
   for (auto &kv : g.plans) plan_destroy(kv.second);
   g.plans.clear();
+  gemm_plans_forget();
   for (auto &kv : g.graphs) {
     if (kv.second.exec) (void)hipGraphExecDestroy(kv.second.exec);
     if (kv.second.graph) (void)hipGraphDestroy(kv.second.graph);

@@ -144,9 +144,19 @@ def transformerBlock(ctx: Ctx, x: Variable, layer: dict, cfg: ModelConfig, Bt: i
     else:
         qF, kF, vF = ag.sliceQkv(ctx, qkv)
         q, k, v = (ag.reshape(ctx, t, [Bt, T, Cc]) for t in (qF, kF, vF))
-        if cfg.attention == "reference-flash" and ag._has(Bk, "flashAttention") and D in (32, 64, 128):
+        if cfg.attention == "reference-flash" and ag._has(Bk, "flashAttention"):
             qFA, kFA, vFA = (ag.reshape(ctx, t, [Bt * H, T, D]) for t in (q, k, v))
-            att = ag.flashAttention(ctx, qFA, kFA, vFA, T, scl, cap)
+            if D in (32, 64, 128):
+                att = ag.flashAttention(ctx, qFA, kFA, vFA, T, scl, cap)
+            else:
+                # a head size without a fused kernel: the same function of the same slabs, op by op (no dropout on the
+                # attention weights: this branch has none, gpt.ts:247-254)
+                scores = ag.scale(ctx, ag.matmul(ctx, qFA, ag.transpose(ctx, kFA, 1, 2)), scl)
+                if cap > 0:
+                    scores = ag.softCap(ctx, scores, cap)
+                masked = Variable(Bk.maskedFill(scores.data, mask, -1e9), True)
+                ctx.tape.record(masked, [scores], lambda g, B, rel, n: [B.maskedFill(g, mask, 0)])
+                att = ag.matmul(ctx, ag.softmax(ctx, masked, -1), vFA)
             concat = ag.reshape(ctx, ag.transpose(ctx, ag.reshape(ctx, att, [Bt, H, T, D]), 1, 2), [Bt * T, Cc])
         else:
             qH, kH, vH = (ag.transpose(ctx, ag.reshape(ctx, t, [Bt, T, H, D]), 1, 2) for t in (q, k, v))

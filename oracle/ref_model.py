@@ -5,6 +5,11 @@ Restatement of the reference's host-side training step as it runs on its CPU bac
   * differentiable ops + CPU fallbacks  packages/autograd/src/ops.ts:99-974
   * initGPT / transformerBlock / gptForward (the NON-flash branch cpu_ref takes)
                                         packages/model/src/gpt.ts:73-151, 220-333, 344-427
+  * the flash branch of transformerBlock (ModelConfig.attention = "reference-flash": what an unchanged gpt.ts runs on a
+    backend that offers flashAttention)  packages/model/src/gpt.ts:247-254, with the op's contract
+                                        (packages/core/src/interfaces.ts:127-135) restated in closed form, forward and
+                                        backward, per [T, D] slab; pinned in tests/test_oracle_model.py against PyTorch
+                                        float64 autograd (whole model, and the op alone against torch's fused routine)
   * AdamW.stepParamEntries              packages/train/src/optimizers.ts:54-115
   * sample(): token selection + loop     packages/train/src/sample.ts:36-198 (pinned in tests/test_sample.py by hand-worked
                                         distributions with scripted rng draws)
@@ -384,6 +389,9 @@ class ModelConfig:
     ffnDim: Optional[int] = None
     softCap: Optional[float] = None
     activationGraph: Optional[dict] = None
+    # which branch of gpt.ts:246-280 the block takes: "heads" = the one for a backend WITHOUT flashAttention (cpu_ref,
+    # :255-279), "reference-flash" = the one for a backend WITH it (:247-254), restated with materialised attention
+    attention: str = "heads"
 
 
 def _init_weight(rng: SeededRng, shape, std) -> Variable:
@@ -468,8 +476,54 @@ def _eval_activation_graph(ctx, x, node):
     raise ValueError(f"activation graph node {kind!r}")
 
 
+def flash_attention_forward(q: np.ndarray, k: np.ndarray, v: np.ndarray, scl: float, cap: float):
+    """Backend.flashAttention (interfaces.ts:127-135): q, k, v [B*H, T, D] -> output [B*H, T, D] and the log-sum-exp of
+    every row [B*H, T].  Per [T, D] slab: scores = scl * q k^T, then tanh(s / cap) * cap when cap > 0
+    (helios/src/kernels/attention.ts:427-437: the hyperbolic tangent itself, not the clamped-exponential form the
+    autograd fallback composes, ops.ts:329-340), keys after the query masked out, softmax, times v.  f32 in and out,
+    f64 inside (cpu_ref's convention); the whole [T, T] matrix is materialised."""
+    q64, k64, v64 = (np.asarray(x, np.float64) for x in (q, k, v))
+    T = q64.shape[1]
+    s = scl * (q64 @ k64.transpose(0, 2, 1))
+    th = np.tanh(s / cap) if cap > 0 else None
+    c = th * cap if cap > 0 else s
+    future = np.triu(np.ones((T, T), dtype=bool), 1)
+    c = np.where(future[None], -np.inf, c)
+    mx = c.max(-1, keepdims=True)
+    e = np.exp(c - mx)
+    den = e.sum(-1, keepdims=True)
+    p = e / den
+    return (p @ v64), (mx + np.log(den))[..., 0], p, th
+
+
+def flash_attention_backward(q, k, v, do, scl: float, cap: float):
+    """Backend.flashAttentionBackward (interfaces.ts:131-135), closed form: dV = P^T dO; dP = dO V^T;
+    d(capped scores) = P * (dP - rowsum(dP * P)); through the cap: * (1 - tanh^2); dQ = scl * dS K; dK = scl * dS^T Q."""
+    q64, k64, v64, do64 = (np.asarray(x, np.float64) for x in (q, k, v, do))
+    _, _, p, th = flash_attention_forward(q, k, v, scl, cap)
+    dv = p.transpose(0, 2, 1) @ do64
+    dp = do64 @ v64.transpose(0, 2, 1)
+    dc = p * (dp - (dp * p).sum(-1, keepdims=True))
+    ds = dc * (1.0 - th * th) if cap > 0 else dc
+    return scl * (ds @ k64), scl * (ds.transpose(0, 2, 1) @ q64), dv
+
+
+def flashAttention(ctx, q, k, v, T, scl, cap):
+    """ops.ts:741-770: records Backend.flashAttention with Backend.flashAttentionBackward as its gradient.  cpu_ref has
+    neither (ops.ts:746 throws); the two functions above restate the contract."""
+    shp = q.data.shape
+    qa, ka, va = (x.data.data.reshape(shp) for x in (q, k, v))
+    out = flash_attention_forward(qa, ka, va, scl, cap)[0]
+
+    def bw(g, B, n):
+        dq, dk, dv = flash_attention_backward(qa, ka, va, g.data.reshape(shp), scl, cap)
+        return [TD(shp, "f32", x.astype(np.float32).reshape(-1)) for x in (dq, dk, dv)]
+    return _record(ctx, TD(shp, "f32", out.astype(np.float32).reshape(-1)), [q, k, v], bw)
+
+
 def _transformer_block(ctx, x, layer, cfg: ModelConfig, Bt, T, mask: TD, training):
-    """gpt.ts:220-333, the branch taken when backend.flashAttention is absent (cpu_ref)."""
+    """gpt.ts:220-333.  cfg.attention picks the branch of :246-280: "heads" is the one taken when backend.flashAttention
+    is absent (cpu_ref), "reference-flash" the one taken when it is present."""
     H, Cc = cfg.nHead, cfg.nEmbd
     D = Cc // H
     ln1 = layerNorm(ctx, x, layer["ln1"]["weight"], layer["ln1"]["bias"], 1e-5)
@@ -479,6 +533,8 @@ def _transformer_block(ctx, x, layer, cfg: ModelConfig, Bt, T, mask: TD, trainin
     k = reshape(ctx, kF, [Bt, T, Cc])
     v = reshape(ctx, vF, [Bt, T, Cc])
     cap = cfg.softCap if cfg.softCap is not None else 30.0
+    if cfg.attention == "reference-flash":
+        return _block_tail(ctx, x, layer, cfg, Bt, T, training, _flash_branch(ctx, q, k, v, cfg, Bt, T, cap))
     qH = transpose(ctx, reshape(ctx, q, [Bt, T, H, D]), 1, 2)
     kH = transpose(ctx, reshape(ctx, k, [Bt, T, H, D]), 1, 2)
     vH = transpose(ctx, reshape(ctx, v, [Bt, T, H, D]), 1, 2)
@@ -490,6 +546,25 @@ def _transformer_block(ctx, x, layer, cfg: ModelConfig, Bt, T, mask: TD, trainin
     att = softmax(ctx, masked, -1)
     out = matmul(ctx, dropout(ctx, att, cfg.dropout, training), vH)
     concat = reshape(ctx, transpose(ctx, out, 1, 2), [Bt * T, Cc])
+    return _block_tail(ctx, x, layer, cfg, Bt, T, training, concat)
+
+
+def _flash_branch(ctx, q, k, v, cfg: ModelConfig, Bt, T, cap):
+    """gpt.ts:247-254: [B, T, C] is re-read as [B*H, T, D] WITHOUT moving heads next to the batch (slab j of batch entry b
+    is rows j*T/H .. (j+1)*T/H of that entry, each row cut into H pieces of D), attention runs per slab, and the result
+    [B, H, T, D] is transposed (1, 2) and flattened to [B*T, C]."""
+    H, Cc = cfg.nHead, cfg.nEmbd
+    D = Cc // H
+    qFA = reshape(ctx, q, [Bt * H, T, D])
+    kFA = reshape(ctx, k, [Bt * H, T, D])
+    vFA = reshape(ctx, v, [Bt * H, T, D])
+    out = flashAttention(ctx, qFA, kFA, vFA, T, 1 / math.sqrt(D), cap)
+    return reshape(ctx, transpose(ctx, reshape(ctx, out, [Bt, H, T, D]), 1, 2), [Bt * T, Cc])
+
+
+def _block_tail(ctx, x, layer, cfg: ModelConfig, Bt, T, training, concat):
+    """gpt.ts:281-333: output projection, residual, LayerNorm, MLP, residual."""
+    Cc = cfg.nEmbd
     proj = reshape(ctx, matmulTransposed(ctx, concat, layer["attn"]["wo"]), [Bt, T, Cc])
     x = residualDropoutAdd(ctx, x, proj, cfg.dropout, training)
 

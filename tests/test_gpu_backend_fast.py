@@ -130,6 +130,52 @@ def test_weight_gradients_are_grouped_and_accumulate_in_place(FB):
     assert FB.lastGemmKernel()[0].endswith(", true>") and abs(got - 9 * sum(sq)) <= 1e-3 * 9 * sum(sq)
 
 
+def test_gradient_norm_with_one_accumulating_and_several_fresh_weight_gradients(FB):
+    """One queued product re-targeted by addInplace (a shared weight: a part of one descriptor, launched on its own) beside
+    fresh ones (a grouped launch): the norm must see the accumulated gradient after its product has run, as eager execution
+    (every product launched when it is asked for) does."""
+    rs = np.random.RandomState(16)
+    T = 256
+    gs = [rs.randn(T, m) * 0.2 for m in (64, 128, 192, 64)]
+    xs = [rs.randn(T, n) * 0.5 for n in (128, 64, 128, 128)]
+    wants = [_bf16(g).astype(np.float64).T @ _bf16(x).astype(np.float64) for g, x in zip(gs, xs)]
+    got = []
+    for group in (True, False):
+        FB._group = group
+        try:
+            shared = FB.clone(FB.matmulTransposedA(_td(gs[3]), _td(xs[3])))       # the first use's gradient, resident
+            FB.syncGpu()
+            fresh = [FB.matmulTransposedA(_td(g), _td(x)) for g, x in zip(gs[:3], xs[:3])]
+            again = FB.matmulTransposedA(_td(gs[3]), _td(xs[3]))                  # the second use: added into the first
+            FB.addInplace(shared, again)
+            FB.releaseGpuTensor(again)
+            got.append(float(FB.totalSumOfSquares(fresh + [shared]).data[0]))
+            _close(shared.data, 2 * wants[3], "gradient of the shared weight", tol=1e-3)
+        finally:
+            FB._group = True
+    want = sum(float((w ** 2).sum()) for w in wants[:3]) + float(((2 * wants[3]) ** 2).sum())
+    assert abs(got[0] - want) <= 1e-3 * want and abs(got[1] - want) <= 1e-3 * want, (got, want)
+
+
+def test_a_product_kept_past_the_optimizer_step_is_of_the_weights_it_was_asked_with(FB):
+    """A product whose epilogue took its place (x W^T + residual) is only a recipe while its own tensor is unread; the recipe
+    names the weight's bf16 shadow, which adamwStep rewrites in place: read after the update, the tensor must still be the
+    product with the weights of the time of the call (what eager execution, and the reference's backends, give)."""
+    rs = np.random.RandomState(21)
+    x, w, res = _bf16(rs.randn(64, 128) * 0.5), _bf16(rs.randn(256, 128) * 0.1), _bf16(rs.randn(64, 256))
+    W = _td(w)
+    prod = FB.matmulTransposed(FB.castStore(_td(x), "bf16"), W)
+    out = FB.add(FB.castStore(_td(res), "bf16"), prod)              # the residual epilogue: `prod` itself is not written
+    g = _td(np.ones_like(w))
+    m, v = _td(np.zeros_like(w)), _td(np.zeros_like(w))
+    FB.adamwStep(W, g, m, v, 0.5, 0.9, 0.95, 1e-8, 0.0, 0.1, 0.05, 1.0)
+    FB.syncGpu()
+    want = x.astype(np.float64) @ w.astype(np.float64).T
+    assert np.max(np.abs(W.data.reshape(w.shape) - w)) > 0.1      # the weights did move
+    _close(prod.data, want, "the product read after the update", tol=1e-2)
+    _close(out.data, want + res, "its residual sum", tol=1e-2)
+
+
 def test_clone_is_copy_on_write(FB):
     a = _td(np.arange(8.0))
     c = FB.clone(a)
@@ -138,6 +184,42 @@ def test_clone_is_copy_on_write(FB):
     d = FB.clone(c)
     FB.scaleInplace(c, 2.0)
     assert np.array_equal(d.data, np.arange(8.0) + 1) and np.array_equal(c.data, 2 * (np.arange(8.0) + 1))
+
+
+@pytest.mark.parametrize("graphs", [False, True])
+def test_reference_flash_branch_on_the_fast_backend_tracks_its_oracle_over_50_steps(FB, graphs):
+    """The branch an unchanged gpt.ts takes on a backend with flashAttention (gpt.ts:247-254), run by the generic trainer on
+    the fast backend (bf16 words moved by sliceQkv / transpose, the three scatterSlice results of the backward pass merged),
+    against the oracle's restatement of that branch: loss within 2e-2 relative at every one of 50 steps, eagerly and replayed
+    from a step plan, the two bit-identical."""
+    from alpha2_amd.model import ModelConfig
+    from alpha2_amd.train import TrainConfig, Trainer, syntheticBatch
+    steps = 50
+    cfg = dict(CFG, attention="reference-flash")
+    tr = Trainer(FB, ModelConfig(**cfg), TrainConfig(iters=steps), seed=3)
+    orc = rm.Trainer(rm.ModelConfig(**cfg), rm.TrainConfig(iters=steps), seed=3)
+    for t in (tr, orc):                             # attention weights large enough that the slab wiring shows in the loss
+        for n, v in t.entries:
+            if n.endswith("attn.wqkv"):
+                v.data.data = v.data.data * 8
+    FB.enableStepGraphs(graphs)
+    before = FB.stepStats()
+    losses = []
+    for s in range(steps):
+        r = tr.step([syntheticBatch(50 + s, 4, 64, 256)])
+        o = orc.step([rm.synthetic_batch(50 + s, 4, 64, 256)])
+        assert math.isfinite(r.loss) and abs(r.loss - o.loss) <= 2e-2 * abs(o.loss), (s, r.loss, o.loss)
+        assert abs(r.gradNorm - o.gradNorm) <= 5e-2 * o.gradNorm and abs(r.lr - o.lr) < 1e-15, (s, r.gradNorm, o.gradNorm)
+        losses.append((r.loss, r.gradNorm))
+    FB.enableStepGraphs(False)
+    fn = test_reference_flash_branch_on_the_fast_backend_tracks_its_oracle_over_50_steps
+    if graphs:
+        assert FB.stepStats()["replayed"] - before["replayed"] >= steps - 4, (before, FB.stepStats(), FB.lastStepNote)
+        fn.graph_losses = losses
+    else:
+        fn.eager_losses = losses
+    if hasattr(fn, "graph_losses") and hasattr(fn, "eager_losses"):
+        assert fn.graph_losses == fn.eager_losses
 
 
 @pytest.mark.parametrize("graphs", [False, True])

@@ -23,7 +23,9 @@ def _both(B, cfg_kw, tc_kw, seed=0):
     from alpha2_amd.model import ModelConfig
     from alpha2_amd.train import TrainConfig, Trainer
     dev = Trainer(B, ModelConfig(**cfg_kw), TrainConfig(**tc_kw), seed=seed)
-    orc = rm.Trainer(rm.ModelConfig(**{k: v for k, v in cfg_kw.items() if k != "attention"}),
+    # the oracle knows the two branches of gpt.ts:246-280; "unfused" is the product's op-by-op form of the heads branch
+    okw = dict(cfg_kw, attention="reference-flash" if cfg_kw.get("attention") == "reference-flash" else "heads")
+    orc = rm.Trainer(rm.ModelConfig(**okw),
                      rm.TrainConfig(**{k: v for k, v in tc_kw.items() if k in rm.TrainConfig.__dataclass_fields__}), seed=seed)
     for (n1, v1), (n2, v2) in zip(dev.entries, orc.entries):        # same names, same order, same initial values
         assert n1 == n2 and np.array_equal(v1.data.data, v2.data.data), n1
@@ -161,22 +163,51 @@ def test_activation_checkpointing_matches_plain(B):
         assert_close(b, a, rel=1e-5)
 
 
-def test_reference_flash_layout_is_exposed_and_differs(B):
-    """The reference reshapes [B,T,C] -> [B*H,T,D] without a head transpose when a backend exposes flashAttention
-    (gpt.ts:248-254); that path is available as attention="reference-flash" and is NOT the cpu_ref function."""
+@pytest.mark.parametrize("kw", [dict(), dict(softCap=0.0), dict(nHead=4, ffnActivation="swiglu", softCap=2.0),
+                                dict(nEmbd=128, nHead=4, softCap=2.0)])        # (the third: head size 16, no fused kernel)
+def test_reference_flash_branch_matches_its_oracle(B, kw):
+    """What an unchanged gpt.ts runs on a backend that offers flashAttention (gpt.ts:247-254: [B, T, C] re-read as
+    [B*H, T, D] slabs without a head transpose, flashAttention per slab, transpose (1, 2) back) against the oracle's
+    restatement of that branch: logits, loss and every gradient at the fp32 bar, with the attention weights made large
+    enough that the wiring of slabs matters; it is not the cpu_ref function (checked against the heads branch)."""
     from alpha2_amd.autograd import Tape
-    from alpha2_amd.model import ModelConfig, gptForward, initGPT
-    from alpha2_amd.rng import SeededRng
+    from alpha2_amd.model import gptForward
     from alpha2_amd.train import syntheticBatch
-    losses = {}
-    for mode in ("heads", "reference-flash"):
-        cfg = ModelConfig(vocabSize=50, blockSize=16, nLayer=2, nEmbd=64, nHead=2, attention=mode)
-        params = initGPT(cfg, B, SeededRng(4))
-        for l in params["layers"]:
-            l["attn"]["wqkv"].data.data = l["attn"]["wqkv"].data.data * 20        # make attention matter
-        inp, tgt = syntheticBatch(8, 2, 16, 50)
-        losses[mode] = float(gptForward(cfg, params, B, Tape(), inp, tgt, True)["loss"].data.data[0])
-    assert math.isfinite(losses["reference-flash"]) and abs(losses["heads"] - losses["reference-flash"]) > 1e-6
+    cfg = dict(dict(vocabSize=61, blockSize=24, nLayer=2, nEmbd=64, nHead=2, attention="reference-flash"), **kw)
+    dev, orc = _both(B, cfg, dict(iters=1), seed=4)
+    for (n, v), (_, ov) in zip(dev.entries, orc.entries):
+        if n.endswith("attn.wqkv"):
+            v.data.data = v.data.data * 20
+            ov.data.data *= 20
+    inp, tgt = syntheticBatch(3, 3, 24, 61)
+    oi, ot = rm.synthetic_batch(3, 3, 24, 61)
+    tape, otape = Tape(), rm.Tape()
+    r = gptForward(dev.cfg, dev.params, B, tape, inp, tgt, True)
+    ologits, oloss = rm.gptForward(orc.cfg, orc.params, orc.B, otape, oi, ot, True)
+    assert_close(r["logits"].data.data, ologits.data.data, what="logits")
+    assert_close(r["loss"].data.data, oloss.data.data, what="loss")
+    tape.backward(r["loss"], B)
+    otape.backward(oloss, orc.B)
+    for (n, v), (_, ov) in zip(dev.entries, orc.entries):
+        assert_close(v.grad.data, ov.grad.data, what=f"grad {n}")
+    hcfg = rm.ModelConfig(**dict(cfg, attention="heads", softCap=cfg.get("softCap") or 30.0))
+    _, hloss = rm.gptForward(hcfg, orc.params, orc.B, rm.Tape(), oi, ot, True)
+    assert abs(float(hloss.data.data[0]) - float(oloss.data.data[0])) > 1e-4
+
+
+def test_reference_flash_branch_training_steps_with_dropout_match_oracle(B):
+    """The same branch through the trainer: 6 steps with two micro-steps and dropout 0.1, which in this branch has two
+    sites per layer (the residual branches; no dropout on the attention weights, gpt.ts:247-254 against :276)."""
+    from alpha2_amd.train import syntheticBatch
+    cfg = dict(vocabSize=96, blockSize=32, nLayer=2, nEmbd=64, nHead=2, dropout=0.1, attention="reference-flash")
+    dev, orc = _both(B, cfg, dict(iters=6, gradAccumSteps=2, seed=7), seed=2)
+    for s in range(6):
+        bs = [syntheticBatch(300 + 2 * s + m, 4, 32, 96) for m in range(2)]
+        obs = [rm.synthetic_batch(300 + 2 * s + m, 4, 32, 96) for m in range(2)]
+        r, o = dev.step(bs), orc.step(obs)
+        assert abs(r.loss - o.loss) <= 1e-3 * abs(o.loss), (s, r.loss, o.loss)
+        assert abs(r.gradNorm - o.gradNorm) <= 1e-3 * o.gradNorm, (s, r.gradNorm, o.gradNorm)
+    assert (dev.dropoutRng.counter, orc.dropoutRng.counter) == (4, 4)
 
 
 @pytest.mark.parametrize("N,Bt,T,packed", [(5000, 8, 128, False), (129, 2, 128, False), (1000, 4, 64, True), (10, 3, 7, True),

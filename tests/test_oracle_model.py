@@ -102,7 +102,7 @@ def _composed_closed_form(h):
     return 0.5 * (F.silu(h) * (h * h)) + (F.relu(h) * g(h) + (-0.3 * h + 0.25 * g(h)))
 
 
-def _torch_forward(cfg, P, tokens, targets, cap=30.0, masks=None):
+def _torch_forward(cfg, P, tokens, targets, cap=30.0, masks=None, flash=False):
     """The same network in PyTorch float64 (library ops; independent of the oracle's loops).  `masks`: per layer the
     dropout masks of the attention weights and of the two residual branches, in the order the model draws them."""
     Bt, T = tokens.shape
@@ -114,14 +114,26 @@ def _torch_forward(cfg, P, tokens, targets, cap=30.0, masks=None):
         g = lambda s: P[f"layer.{i}.{s}"]
         h = F.layer_norm(x, (Cc,), g("ln1.weight"), g("ln1.bias"), 1e-5)
         qkv = h.reshape(Bt * T, Cc) @ g("attn.wqkv").T
-        q, k, v = [t.reshape(Bt, T, H, D).transpose(1, 2) for t in qkv.split(Cc, dim=1)]
-        s = (q @ k.transpose(2, 3)) / math.sqrt(D)
-        s = cap * torch.tanh(s / cap)
-        s = s.masked_fill(mask, -1e9)
-        w = torch.softmax(s, -1)
-        if masks is not None:
-            w = w * masks[i][0].reshape(w.shape)
-        a = w @ v
+        if flash:
+            # gpt.ts:247-254: the three [B*T, C] matrices re-read as [B*H, T, D] slabs as they lie in memory (no head
+            # transpose), causal soft-capped attention per slab (library routine; no dropout on the weights in this
+            # branch), then [B, H, T, D] -> transpose(1, 2) -> [B*T, C]
+            q, k, v = [t.contiguous().reshape(Bt * H, T, D) for t in qkv.split(Cc, dim=1)]
+            bias = torch.zeros(T, T, dtype=torch.float64).masked_fill(mask, float("-inf"))
+            s = (q @ k.transpose(1, 2)) / math.sqrt(D)
+            s = (cap * torch.tanh(s / cap) if cap > 0 else s) + bias       # a cap of 0 switches it off (interfaces.ts:127-135)
+            a = (torch.softmax(s, -1) @ v).reshape(Bt, H, T, D)
+            if cap == 0:        # plain causal attention: the library's fused routine must agree
+                assert torch.allclose(a, F.scaled_dot_product_attention(q, k, v, is_causal=True).reshape(Bt, H, T, D), atol=1e-9)
+        else:
+            q, k, v = [t.reshape(Bt, T, H, D).transpose(1, 2) for t in qkv.split(Cc, dim=1)]
+            s = (q @ k.transpose(2, 3)) / math.sqrt(D)
+            s = cap * torch.tanh(s / cap)
+            s = s.masked_fill(mask, -1e9)
+            w = torch.softmax(s, -1)
+            if masks is not None:
+                w = w * masks[i][0].reshape(w.shape)
+            a = w @ v
         proj = (a.transpose(1, 2).reshape(Bt * T, Cc) @ g("attn.wo").T).reshape(Bt, T, Cc)
         x = x + (proj * masks[i][1].reshape(proj.shape) if masks is not None else proj)
         h = F.layer_norm(x, (Cc,), g("ln2.weight"), g("ln2.bias"), 1e-5).reshape(Bt * T, Cc)
@@ -152,9 +164,10 @@ def _torch_forward(cfg, P, tokens, targets, cap=30.0, masks=None):
     return logits, F.cross_entropy(logits, targets.reshape(-1))
 
 
-def _check_model(act, seed, dropout=0.0):
+def _check_model(act, seed, dropout=0.0, attention="heads", cap=None):
     cfg = rm.ModelConfig(vocabSize=29, blockSize=12, nLayer=2, nEmbd=16, nHead=4, ffnActivation=act, dropout=dropout,
-                         activationGraph=COMPOSED_GRAPH if act == "composed" else None)
+                         activationGraph=COMPOSED_GRAPH if act == "composed" else None, attention=attention, softCap=cap)
+    flash = attention == "reference-flash"
     Bm = ref.CpuRef()
     params = rm.initGPT(cfg, Bm, ref.SeededRng(seed))
     entries = rm.collectParamEntries(params)
@@ -171,13 +184,18 @@ def _check_model(act, seed, dropout=0.0):
         from tests.util import py_dropout_mask
         drng = rm.DropoutRng(77)
         sizes = [3 * 4 * 12 * 12, 3 * 12 * 16, 3 * 12 * 16]
-        masks = [[torch.tensor(py_dropout_mask(77, 3 * l + j, dropout, range(n)).astype(np.float64)) for j, n in enumerate(sizes)]
-                 for l in range(cfg.nLayer)]
+        if flash:       # no dropout on the attention weights in this branch: two sites per layer, the counter follows
+            masks = [[None] + [torch.tensor(py_dropout_mask(77, 2 * l + j, dropout, range(n)).astype(np.float64))
+                               for j, n in enumerate(sizes[1:])] for l in range(cfg.nLayer)]
+        else:
+            masks = [[torch.tensor(py_dropout_mask(77, 3 * l + j, dropout, range(n)).astype(np.float64)) for j, n in enumerate(sizes)]
+                     for l in range(cfg.nLayer)]
     logits, loss = rm.gptForward(cfg, params, Bm, tape, inp, tgt, True, drng)
     tape.backward(loss, Bm)
     P = {n: torch.tensor(v.data.data.astype(np.float64)).reshape(v.data.shape).requires_grad_() for n, v in entries}
     tl, tloss = _torch_forward(cfg, P, torch.tensor(inp.data.astype(np.int64)).reshape(3, 12),
-                               torch.tensor(tgt.data.astype(np.int64)).reshape(3, 12), masks=masks)
+                               torch.tensor(tgt.data.astype(np.int64)).reshape(3, 12), masks=masks, flash=flash,
+                               cap=30.0 if cap is None else cap)      # gpt.ts:244: config.softCap ?? 30
     tloss.backward()
     assert abs(float(loss.data.data[0]) - tloss.item()) < 2e-6
     assert np.max(np.abs(logits.data.data - tl.detach().numpy().reshape(-1))) < 2e-6
@@ -203,6 +221,61 @@ def test_full_model_forward_backward_vs_torch_f64_composed_activation():
 def test_full_model_forward_backward_vs_torch_f64_with_dropout():
     """Dropout 0.2 at the three sites of every layer, masks from the independently restated hash."""
     _check_model("gelu", 6, dropout=0.2)
+
+
+@pytest.mark.parametrize("cap,mag", [(30.0, 1.0), (0.0, 1.0), (2.0, 6.0)])
+def test_flash_attention_contract_vs_torch_f64(cap, mag):
+    """The oracle's closed forms for Backend.flashAttention / flashAttentionBackward (interfaces.ts:127-135) against PyTorch
+    float64 autograd through the materialised definition, incl. scores far into the cap's flat part (where the composed
+    clamped-exponential form of ops.ts:329-340 overflows its f32 denominator and is NOT what the fused op computes), and
+    against torch's own fused causal attention when the cap is off."""
+    rs = np.random.RandomState(5)
+    BH, T, D = 3, 19, 8
+    q, k, v, do = (rs.randn(BH, T, D).astype(np.float32) * mag for _ in range(4))
+    scl = 1 / math.sqrt(D)
+    out, lse, _, _ = rm.flash_attention_forward(q, k, v, scl, cap)
+    dq, dk, dv = rm.flash_attention_backward(q, k, v, do, scl, cap)
+    Q, K, V = (torch.tensor(x.astype(np.float64)).requires_grad_() for x in (q, k, v))
+    s = (Q @ K.transpose(1, 2)) * scl
+    if cap > 0:
+        s = cap * torch.tanh(s / cap)
+    s = s.masked_fill(torch.triu(torch.ones(T, T, dtype=torch.bool), 1), float("-inf"))
+    o = torch.softmax(s, -1) @ V
+    o.backward(torch.tensor(do.astype(np.float64)))
+    assert np.max(np.abs(out - o.detach().numpy())) < 1e-12 and np.max(np.abs(lse - torch.logsumexp(s, -1).detach().numpy())) < 1e-12
+    for got, want in ((dq, Q.grad), (dk, K.grad), (dv, V.grad)):
+        assert np.max(np.abs(got - want.numpy())) < 1e-10 * (1 + float(want.abs().max()))
+    if cap == 0:
+        assert torch.allclose(o, F.scaled_dot_product_attention(Q, K, V, is_causal=True), atol=1e-12)
+    # recorded on the tape (ops.ts:741-770): f32 in and out
+    tape = rm.Tape()
+    ctx = rm.Ctx(tape, ref.CpuRef())
+    qv, kv, vv = (rm.Variable(ref.TD((BH, T, D), "f32", x.reshape(-1).copy()), True) for x in (q, k, v))
+    ov = rm.flashAttention(ctx, qv, kv, vv, T, scl, cap)
+    tape.backward(ov, ref.CpuRef(), ref.TD((BH, T, D), "f32", do.reshape(-1).copy()))
+    assert ov.data.data.dtype == np.float32 and np.array_equal(ov.data.data, out.astype(np.float32).reshape(-1))
+    assert np.array_equal(qv.grad.data, dq.astype(np.float32).reshape(-1)) and np.array_equal(vv.grad.data, dv.astype(np.float32).reshape(-1))
+
+
+def test_flash_branch_of_the_block_vs_torch_f64():
+    """gpt.ts:247-254, the branch an unchanged model takes on a backend with flashAttention: slabs cut from [B, T, C]
+    without a head transpose.  It is a different function from the heads branch (checked), with the default cap, with a cap
+    low enough to bend the scores, with the cap switched off (where torch's fused attention routine is compared too), and
+    with dropout (two sites per layer here)."""
+    _check_model("gelu", 0, attention="reference-flash")
+    _check_model("gelu", 1, attention="reference-flash", cap=0.7)
+    _check_model("swiglu", 2, attention="reference-flash", cap=0.0)
+    _check_model("gelu", 6, dropout=0.2, attention="reference-flash")
+    losses = []
+    for att in ("heads", "reference-flash"):
+        cfg = rm.ModelConfig(vocabSize=29, blockSize=12, nLayer=2, nEmbd=16, nHead=4, attention=att)
+        Bm = ref.CpuRef()
+        params = rm.initGPT(cfg, Bm, ref.SeededRng(0))
+        for _, v in rm.collectParamEntries(params):
+            v.data.data *= 8
+        inp, tgt = rm.synthetic_batch(1, 3, 12, 29)
+        losses.append(float(rm.gptForward(cfg, params, Bm, rm.Tape(), inp, tgt)[1].data.data[0]))
+    assert abs(losses[0] - losses[1]) > 1e-4
 
 
 def test_dropout_is_off_when_not_training_and_masks_follow_the_step_seed():
