@@ -456,18 +456,22 @@ class FusedTrainer:
                     self._bufs.remove(b)
         self._batches = []
 
-    def _use_batch(self, i, micro: int = 0):
-        """Copy stored batch i into the resident slot of micro-step `micro` (a sequence fills slots 0, 1, ...)."""
+    def _use_batch(self, i, micro: int = 0, reindex: bool = False):
+        """Copy stored batch i into the resident slot of micro-step `micro` (a sequence fills slots 0, 1, ...).  `reindex`:
+        build the slot's scatter-add index from its ids again instead of copying the one made when the batch was stored
+        (what a loop that feeds a new batch every step pays: the sort of the ids is then part of the step)."""
         if isinstance(i, (list, tuple)):
             if len(i) != self.accum:
                 raise ValueError(f"need {self.accum} batch indices, one per micro-step")
             for m, bi in enumerate(i):
-                self._use_batch(bi, m)
+                self._use_batch(bi, m, reindex)
             return
         ti, tt, ix = self._batches[i]
         check(self.lib.ah_copy(self.toks[micro], ti, self.BT * 4))
         check(self.lib.ah_copy(self.tgts[micro], tt, self.BT * 4))
-        if ix:
+        if ix and reindex:
+            check(self.lib.ah_embedding_index(self.toks[micro], self.BT, self.V, self.tok_index[micro]))
+        elif ix:
             check(self.lib.ah_copy(self.tok_index[micro], ix, self._index_bytes))
         self._have_batch = True
 
@@ -486,12 +490,12 @@ class FusedTrainer:
         check(self.lib.ah_upload(self.hyper, C.byref(v), 4))
         return lr
 
-    def step(self, batch_index=None) -> int:
+    def step(self, batch_index=None, reindex: bool = False) -> int:
         """Enqueue one optimizer step (no host synchronisation); returns the step index whose loss / grad-norm can be
         read later with history().  `batch_index`: a stored batch, or with gradient accumulation a sequence of `accum`
-        stored batches (micro-steps run in that order); None keeps the resident ones."""
+        stored batches (micro-steps run in that order); None keeps the resident ones.  `reindex`: see _use_batch."""
         if batch_index is not None:
-            self._use_batch(batch_index)
+            self._use_batch(batch_index, reindex=reindex)
         elif not self._have_batch:
             raise RuntimeError("no batch set")
         self._write_hyper()

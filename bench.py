@@ -2,7 +2,7 @@
 """Headline benchmark: training tokens/s of the GPT-2-small-shape step (vocab 50304, d 768, 12 layers, 12 heads,
 ctx 1024, batch 16; forward + backward + AdamW with gradient clipping) on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--mode fast|backend|parity] [--no-cpu] [--workload gpt2-small|gpt-350m]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--mode fast|backend|parity] [--no-cpu] [--no-extra] [--workload gpt2-small|gpt-350m]
 
 `--mode fast` (default) is the hand-scheduled step (FusedTrainer); `--mode backend` runs the generic tape-driven Trainer -- one
 `Backend` call per op, host-side loss / norm / clip, exactly the call structure of the reference trainer -- on FastHipBackend
@@ -12,8 +12,13 @@ segments); `--mode parity` runs the same Trainer on the fp32 kernels.
 The default workload is the one the metric is quoted on; `--workload gpt-350m` runs the 350M-shape step (d 1024, 24 layers,
 16 heads, batch 8 with 4 accumulated micro-steps, whole step in one hipGraph) and reports it the same way.
 
+After the headline measurement the default invocation also times, each in a child process of its own once the parent has
+released its device memory, the path the reference's trainer would take -- `--mode backend` with the model's own attention
+wiring (`--attention reference-flash`, gpt.ts:247-254) and with true multi-head attention (`heads`) -- and the 350M-shape
+workload, and adds them to the line as `backend_mode` and `workload_350m` (`--no-extra` leaves them out).
+
 Prints ONE JSON line.  `value` is tokens/s with parameters, optimizer state and the token batch already resident in
-HBM.  `roofline` is for the dominant kernel, the MFMA GEMM instantiation that does the most arithmetic in a step (which is
+HBM; the scatter-add index of the token embedding's gradient (a sort of the batch's ids) is built inside the timed steps.  `roofline` is for the dominant kernel, the MFMA GEMM instantiation that does the most arithmetic in a step (which is
 also the one with the largest summed duration; going by arithmetic keeps the choice the same from run to run):
 2*M*N*K of its launches divided by their summed durations, each launch bracketed by HIP events on the library's
 stream (`all_gemm` gives the same over every GEMM launch of the step).  `cpu_baseline` times the CPU oracle
@@ -100,6 +105,7 @@ def main():
                     help="backend / parity mode: which attention branch of the model runs (reference-flash = the op sequence of the "
                          "reference's flash branch, gpt.ts:232-253; unfused = its CPU branch)")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-extra", action="store_true", help="only the headline measurement: no backend-mode and no 350M-shape runs")
     ap.add_argument("--cpu-tokens", type=int, default=32)
     ap.add_argument("--workload", choices=sorted(WORKLOADS), default="gpt2-small")
     args = ap.parse_args()
@@ -151,7 +157,8 @@ def main():
         def one_step():
             pick = [ids[(cursor[0] + m) % ring] for m in range(accum)]
             cursor[0] += accum
-            return runner.step(pick if accum > 1 else pick[0])             # two 64 KB device-to-device copies, then the graph
+            # two 64 KB device-to-device copies and the sort of the ids for the embedding gradient, then the graph
+            return runner.step(pick if accum > 1 else pick[0], reindex=True)
 
     losses = []
     for _ in range(args.warmup):
@@ -223,9 +230,44 @@ def main():
         out["config"]["norm"] = "over the arena"
     if args.mode == "fast":
         out["config"]["residual_stream"] = args.stream
+        out["index_us_outside_timed_region"] = 0.0      # the id sort of every batch runs inside the timed steps
+    if args.mode == "fast" and args.workload == "gpt2-small" and not args.no_extra:
+        runner.close()
+        del runner
+        B.purgeBufferPools()
+        out.update(extra_runs(args))
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(model, args.cpu_tokens)
     print(json.dumps(out))
+
+
+def extra_runs(args) -> dict:
+    """The same steps through the reference's call structure (generic Trainer on FastHipBackend, step plans) with both
+    attention wirings, and the 350M-shape workload: each a child process running this file, its JSON line parsed."""
+    import subprocess
+
+    def child(*flags):
+        cmd = [sys.executable, os.path.abspath(__file__), "--steps", str(args.steps), "--warmup", str(args.warmup), "--no-cpu", "--no-extra", *flags]
+        try:
+            r = subprocess.run(cmd, capture_output=True, text=True, timeout=600, cwd=ROOT)
+            line = [l for l in r.stdout.splitlines() if l.startswith("{")]
+            if r.returncode != 0 or not line:
+                return {"error": (r.stderr or r.stdout)[-300:]}
+            return json.loads(line[-1])
+        except Exception as e:                                   # a failed extra run must not cost the headline line
+            return {"error": repr(e)[:300]}
+    ref, heads, big = (child("--mode", "backend", "--attention", "reference-flash"), child("--mode", "backend", "--attention", "heads"),
+                       child("--workload", "gpt-350m"))
+    res = {"backend_mode": {"ms_per_step": heads.get("ms_per_step"), "ms_per_step_reference_flash": ref.get("ms_per_step"),
+                            "step_plans": (heads.get("config") or {}).get("step_plans"),
+                            "step_plans_reference_flash": (ref.get("config") or {}).get("step_plans"),
+                            "what": "generic tape-driven Trainer, one Backend call per op, on FastHipBackend with step plans; same model, batches and steps"},
+           "workload_350m": {"ms_per_step": big.get("ms_per_step"), "tokens_per_s": big.get("value"), "mfu": big.get("mfu_vs_bf16_dense_peak"),
+                             "what": (big.get("config") or {}).get("workload")}}
+    for k, v in (("backend_mode", heads), ("backend_mode", ref), ("workload_350m", big)):
+        if "error" in v:
+            res[k].setdefault("errors", []).append(v["error"])
+    return res
 
 
 def _timed(B, one_step):

@@ -9,6 +9,7 @@ properties that do not need the CPU oracle, which would take hours at these size
   (micro-batch gradients are summed and scaled by 1/K once: trainer.ts:1164-1273);
 * clipping: after a step whose gradient norm exceeded the clip, clipCoef * gradNorm == clip (trainer.ts:1650-1656).
 """
+import gc
 import math
 
 import numpy as np
@@ -116,3 +117,44 @@ def test_gpt2_small_shape_fifty_steps_on_fresh_batches_with_loss_tracked(B):
     # predecessors -- and a transformer learns that.  50 steps of a fresh model get well below the initial 10.98 either way.
     assert hg[-1].loss < 8.0 and min(h.loss for h in hg) > 3.0, [h.loss for h in hg]
     graph.close(), eager.close()
+
+
+@pytest.mark.parametrize("attention", ["reference-flash", "heads"])
+def test_gpt2_small_shape_through_the_backend_interface_under_step_plans(attention):
+    """The path the reference's trainer takes (trainer.ts:1188-1273,1761-1784: tape-driven, one Backend call per op, loss and
+    norm read back on the host) at the GPT-2-small shape on the bf16 backend: the initial loss has its closed form, the
+    first bracketed step is recorded and every later one replayed without falling back, and the replayed steps give bit
+    for bit what eager issue of the same calls gives.  `reference-flash` is the model's own wiring (gpt.ts:247-254)."""
+    from alpha2_amd import FastHipBackend
+    from alpha2_amd.model import ModelConfig
+    from alpha2_amd.train import TrainConfig, Trainer, zipfBatches
+    steps = 7
+    batches = zipfBatches(4, steps, 16, 1024, 50304)
+    runs = {}
+    for graphs in (True, False):
+        FB = FastHipBackend(0)
+        FB.resetStepPlan()
+        tr = Trainer(FB, ModelConfig(**SMALL, attention=attention), TrainConfig(iters=50, batchSize=16), seed=0)
+        FB.enableStepGraphs(graphs)
+        before = FB.stepStats()
+        out = []
+        for s in range(steps):
+            x, y = batches[s]
+            r = tr.step([(x, y)])
+            assert math.isfinite(r.loss) and math.isfinite(r.gradNorm), (graphs, s)
+            if r.gradNorm > 1.0:
+                assert abs(r.clipCoef * r.gradNorm - 1.0) < 1e-5, s
+            out.append((r.loss, r.gradNorm))
+        FB.enableStepGraphs(False)
+        after = FB.stepStats()
+        if graphs:
+            assert after["recorded"] - before["recorded"] == 1 and after["fellBack"] - before["fellBack"] == 0, (before, after, FB.stepFallbackNotes)
+            assert after["replayed"] - before["replayed"] >= steps - 2, (before, after)
+        runs[graphs] = out
+        del tr, r
+        gc.collect()                                      # parameters and moments go back to the pool (the buffers' finalisers)
+        FB.resetStepPlan()
+        FB.purgeBufferPools()
+    assert abs(runs[True][0][0] - _expected_initial_loss(SMALL)) < 0.08, runs[True][0]
+    assert runs[True] == runs[False]
+    assert runs[True][-1][0] < runs[True][0][0]
