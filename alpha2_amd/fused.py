@@ -49,8 +49,12 @@ class StepStats:
 class FusedTrainer:
     def __init__(self, backend: HipBackend, cfg: ModelConfig, tc: TrainConfig, batch: int, seed: int = 0, use_graph: bool = True,
                  accum: int = 1, params: Optional[dict] = None, dw_groups: int = 1, stream: str = "bf16",
-                 norm_in_epilogue: bool = True):
+                 norm_in_epilogue: bool = True, index_in_step: bool = False):
         self.act = cfg.ffnActivation or "gelu"
+        # index_in_step: the scatter-add index of the token embedding's gradient (a sort of the micro-batch's ids) is built
+        # inside every step, on the side stream beside the forward pass, instead of once when a batch is stored: what a loop
+        # pays that feeds a new batch every step
+        self.index_in_step = bool(index_in_step)
         if self.act not in ("gelu", "silu", "relu", "swiglu", "universal", "kan_spline") or cfg.dropout != 0:
             raise ValueError("FusedTrainer schedules the gelu / silu / relu / swiglu / universal / kan_spline blocks without dropout; "
                              "use train.Trainer for composed activations and dropout")
@@ -319,6 +323,10 @@ class FusedTrainer:
         acc = 0 if first_micro else 1
         wepi = ffi.EPI_NONE if first_micro else ffi.EPI_ACCUM
         SD = self.SD
+        if self._index_bytes and self.index_in_step:      # one workgroup's work: beside the forward pass, joined before its use
+            check(lib.ah_side_begin())
+            check(lib.ah_embedding_index(self.tok, BT, V, self.tok_index[micro]))
+            check(lib.ah_side_end())
         check(lib.ah_embedding_tok_pos(self.p("wte"), self.p("wpe"), self.tok, self.x[0], BT, self.T, Cc, V, SD))
         for l in range(L):
             pre = f"layer.{l}."
@@ -383,6 +391,8 @@ class FusedTrainer:
             ffi.AhColsumJob(part, self.g(name + ".weight"), self.g(name + ".bias"), BT, Cc, acc, 0) for name, part in self._ln_jobs])
         check(lib.ah_layernorm_colsums(jobs, len(self._ln_jobs)))
         if self._index_bytes:
+            if self.index_in_step:
+                check(lib.ah_side_join())
             check(lib.ah_embedding_bwd_indexed(self.tok_index[micro], self.dx[cur], self.g("wte"), BT, Cc, V, acc))
         else:
             check(lib.ah_embedding_bwd(self.tok, self.dx[cur], self.g("wte"), BT, Cc, V, acc))
@@ -432,7 +442,7 @@ class FusedTrainer:
         """Upload one [B, T] token batch straight into the resident slot of micro-step `micro` (nothing is retained: a loop
         that feeds a fresh batch every step allocates nothing); step() trains on the resident slots until they change."""
         self._upload_batch(inputs, targets, self.toks[micro], self.tgts[micro])
-        if self._index_bytes:
+        if self._index_bytes and not self.index_in_step:
             check(self.lib.ah_embedding_index(self.toks[micro], self.BT, self.V, self.tok_index[micro]))
         self._have_batch = True
 
@@ -442,7 +452,7 @@ class FusedTrainer:
         ti, tt = self._alloc(n), self._alloc(n)
         self._upload_batch(inputs, targets, ti, tt)
         ix = 0
-        if self._index_bytes:
+        if self._index_bytes and not self.index_in_step:
             ix = self._alloc(self._index_bytes)
             check(self.lib.ah_embedding_index(ti, self.BT, self.V, ix))
         self._batches.append((ti, tt, ix))
@@ -456,22 +466,18 @@ class FusedTrainer:
                     self._bufs.remove(b)
         self._batches = []
 
-    def _use_batch(self, i, micro: int = 0, reindex: bool = False):
-        """Copy stored batch i into the resident slot of micro-step `micro` (a sequence fills slots 0, 1, ...).  `reindex`:
-        build the slot's scatter-add index from its ids again instead of copying the one made when the batch was stored
-        (what a loop that feeds a new batch every step pays: the sort of the ids is then part of the step)."""
+    def _use_batch(self, i, micro: int = 0):
+        """Copy stored batch i into the resident slot of micro-step `micro` (a sequence fills slots 0, 1, ...)."""
         if isinstance(i, (list, tuple)):
             if len(i) != self.accum:
                 raise ValueError(f"need {self.accum} batch indices, one per micro-step")
             for m, bi in enumerate(i):
-                self._use_batch(bi, m, reindex)
+                self._use_batch(bi, m)
             return
         ti, tt, ix = self._batches[i]
         check(self.lib.ah_copy(self.toks[micro], ti, self.BT * 4))
         check(self.lib.ah_copy(self.tgts[micro], tt, self.BT * 4))
-        if ix and reindex:
-            check(self.lib.ah_embedding_index(self.toks[micro], self.BT, self.V, self.tok_index[micro]))
-        elif ix:
+        if ix:
             check(self.lib.ah_copy(self.tok_index[micro], ix, self._index_bytes))
         self._have_batch = True
 
@@ -490,12 +496,12 @@ class FusedTrainer:
         check(self.lib.ah_upload(self.hyper, C.byref(v), 4))
         return lr
 
-    def step(self, batch_index=None, reindex: bool = False) -> int:
+    def step(self, batch_index=None) -> int:
         """Enqueue one optimizer step (no host synchronisation); returns the step index whose loss / grad-norm can be
         read later with history().  `batch_index`: a stored batch, or with gradient accumulation a sequence of `accum`
-        stored batches (micro-steps run in that order); None keeps the resident ones.  `reindex`: see _use_batch."""
+        stored batches (micro-steps run in that order); None keeps the resident ones."""
         if batch_index is not None:
-            self._use_batch(batch_index, reindex=reindex)
+            self._use_batch(batch_index)
         elif not self._have_batch:
             raise RuntimeError("no batch set")
         self._write_hyper()

@@ -137,8 +137,8 @@ const char *ah_step_note(void);                    /* why the last step fell bac
  *      everything issued on the main stream so far; the main stream carries on at once.  ah_side_join makes the main stream
  *      wait for all side work.  Legal inside ah_graph_begin .. ah_graph_end (the fork and join become graph edges; join
  *      before ah_graph_end) and a no-op inside a step plan.  Allocation and frees stay ordered on the main stream: buffers
- *      that side work reads or writes must not be freed before ah_side_join.  Only ah_gemm (without its split-K path) and
- *      ah_gemm_grouped_run / _run_sumsq may be issued between ah_side_begin and ah_side_end: the entry points that work
+ *      that side work reads or writes must not be freed before ah_side_join.  Only ah_gemm (without its split-K path),
+ *      ah_gemm_grouped_run / _run_sumsq and ah_embedding_index may be issued between ah_side_begin and ah_side_end: the entry points that work
  *      through the library's one scratch buffer (the reductions, ah_layernorm_bwd, ah_cross_entropy*, ah_channel_act_bwd,
  *      the Adafactor steps) are refused there (AH_ERR_OOM, "no scratch"), and those that take a workspace
  *      from the pool (ah_embedding_bwd, the one-pass flash backward, split-K products) would have it handed back to the

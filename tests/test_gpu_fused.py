@@ -19,11 +19,11 @@ def B():
     return HipBackend(0)
 
 
-def _make(B, tc_kw, use_graph, seed=0, batch=4):
+def _make(B, tc_kw, use_graph, seed=0, batch=4, **kw):
     from alpha2_amd.fused import FusedTrainer
     from alpha2_amd.model import ModelConfig
     from alpha2_amd.train import TrainConfig
-    return FusedTrainer(B, ModelConfig(**CFG), TrainConfig(**tc_kw), batch, seed=seed, use_graph=use_graph)
+    return FusedTrainer(B, ModelConfig(**CFG), TrainConfig(**tc_kw), batch, seed=seed, use_graph=use_graph, **kw)
 
 
 def test_fused_step_gradients_and_update_match_oracle(B):
@@ -219,6 +219,25 @@ def test_fused_step_is_bit_identical_from_run_to_run(B):
         assert np.array_equal(other[2], runs[0][2])
         for n, v in runs[0][1].items():
             assert np.array_equal(other[1][n], v), n
+
+
+@pytest.mark.parametrize("graph", [False, True])
+def test_sorting_the_ids_inside_the_step_gives_the_same_bits(B, graph):
+    """index_in_step: the scatter-add index of the token embedding's gradient is built in every step, on the side stream
+    beside the forward pass (a fork and a join of the captured graph), instead of once when the batch is stored: same index,
+    so the same bits, with two micro-steps as well."""
+    from alpha2_amd.fused import FusedTrainer
+    from alpha2_amd.model import ModelConfig
+    from alpha2_amd.train import TrainConfig, syntheticBatch
+    runs = []
+    for in_step in (False, True):
+        ft = FusedTrainer(B, ModelConfig(**CFG), TrainConfig(iters=4, gradAccumSteps=2), 4, seed=9, use_graph=graph, accum=2, index_in_step=in_step)
+        ids = [ft.add_batch(*syntheticBatch(400 + s, 4, 64, 256)) for s in range(6)]
+        for s in range(3):
+            ft.step([ids[2 * s], ids[2 * s + 1]])
+        runs.append(([(x.loss, x.gradNorm) for x in ft.history(0, 3)], ft.param("wte"), ft.grad("wte")))
+        ft.close()
+    assert runs[0][0] == runs[1][0] and np.array_equal(runs[0][1], runs[1][1]) and np.array_equal(runs[0][2], runs[1][2])
 
 
 @pytest.mark.parametrize("graph", [False, True])
