@@ -231,6 +231,12 @@ def main():
     if args.mode == "fast":
         out["config"]["residual_stream"] = args.stream
         out["index_us_outside_timed_region"] = 0.0      # the id sort of every batch is part of the captured step
+    if args.mode == "fast":
+        # the ceiling under the power limit, measured here and now: 10 launches of ~4 ms each way
+        probe = mfma_probe(B)
+        out["mfma_sustained"] = dict(probe, what="matrix pipes alone, operands in registers, 10 x ~4 ms (ah_probe_mfma_bf16)")
+        out["roofline"]["frac_of_sustained"] = achieved / probe["toggling_operands_tflops"]
+        out["mfu_vs_sustained"] = out["step_tflops"] / probe["toggling_operands_tflops"]
     if args.mode == "fast" and args.workload == "gpt2-small" and not args.no_extra:
         runner.close()
         del runner
@@ -239,6 +245,29 @@ def main():
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(model, args.cpu_tokens)
     print(json.dumps(out))
+
+
+def mfma_probe(B) -> dict:
+    """What the matrix pipes alone sustain in this process on this box (ah_probe_mfma_bf16: independent 32x32x16 bf16 MFMAs
+    on registers, no memory traffic): on all-zero operands the part runs at its published peak, on operands whose bits toggle
+    at what its power limit leaves, which is the ceiling a GEMM on real data can be read against."""
+    import ctypes as C
+    from alpha2_amd import _ffi as ffi
+    lib, fl, out = B.lib, C.c_double(), {}
+    for name, rnd in (("zero_operands_tflops", 0), ("toggling_operands_tflops", 1)):
+        ffi.check(lib.ah_probe_mfma_bf16(1, 100, rnd, C.byref(fl)))
+        ffi.check(lib.ah_sync())
+        e0, e1 = B._event(), B._event()
+        ffi.check(lib.ah_event_record(e0))
+        for _ in range(10):
+            ffi.check(lib.ah_probe_mfma_bf16(1, 30000, rnd, C.byref(fl)))
+        ffi.check(lib.ah_event_record(e1))
+        ms = C.c_float()
+        ffi.check(lib.ah_event_elapsed_ms(e0, e1, C.byref(ms)))
+        for e in (e0, e1):
+            ffi.check(lib.ah_event_destroy(e))
+        out[name] = fl.value * 10 / (ms.value * 1e-3) / 1e12
+    return out
 
 
 def extra_runs(args) -> dict:
