@@ -126,6 +126,7 @@ SIGNATURES = {
     "ah_cross_entropy_bwd": [u64, i32, u64, u64, u64, f32, u64, i64, i64],
     "ah_cross_entropy_fwd_bwd": [u64, i32, u64, u64, u64, u64, f32, u64, i64, i64],
     "ah_gemm": [C.POINTER(AhGemm)],
+    "ah_gemm_planes": [C.POINTER(AhGemm), i64, i64, i64, i64, i32],
     "ah_gemm_grouped_plan": [C.POINTER(AhGemm), C.c_int32, C.POINTER(C.c_uint64)],
     "ah_gemm_grouped_run": [u64, i32],
     "ah_gemm_grouped_run_sumsq": [u64, i32, u64],

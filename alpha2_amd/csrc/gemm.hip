@@ -605,6 +605,50 @@ int32_t ah_gemm_last_kernel(char *name, int32_t capacity, int32_t *nsplit) {
   return AH_OK;
 }
 
+int32_t ah_gemm_planes(const AhGemm *p, int64_t c_plane_cols, int64_t c_plane_stride, int64_t a_plane_k, int64_t a_plane_stride, int32_t dry_run) {
+  AH_REQUIRE_READY();
+  AH_ARG(p != nullptr, "ah_gemm_planes: null descriptor");
+  const AhGemm &q = *p;
+  AH_ARG(q.layout == AH_GEMM_NN || q.layout == AH_GEMM_NT, "ah_gemm_planes: layout NN or NT (A row-major [m, k])");
+  AH_ARG(c_plane_cols >= 0 && a_plane_k >= 0 && (c_plane_cols > 0 || a_plane_k > 0), "ah_gemm_planes: no planes given");
+  AH_ARG(q.m > 0 && q.n > 0 && q.k > 0 && q.m < (1ll << 31) && q.n < (1ll << 31) && q.k < (1ll << 31), "ah_gemm_planes: bad extent");
+  AH_ARG(q.a != 0 && q.b != 0 && q.c != 0, "ah_gemm_planes: null operand");
+  if (q.in_dtype != AH_BF16 || q.out_dtype != AH_BF16 || q.epilogue != AH_EPI_NONE || q.batch != 1)
+    return fail(AH_ERR_UNSUPPORTED, "ah_gemm_planes: one plain product of bf16 operands with a bf16 result");
+  const bool bkm = q.layout == AH_GEMM_NN;
+  if (c_plane_cols > 0) {
+    AH_ARG(q.n % c_plane_cols == 0 && q.ldc >= c_plane_cols && c_plane_stride % 4 == 0,
+           "ah_gemm_planes: n = %lld is not whole planes of %lld columns, or ldc / the plane stride do not fit", (long long)q.n, (long long)c_plane_cols);
+  } else {
+    AH_ARG(q.ldc >= q.n, "matmul shape mismatch: ldc %lld too small for n=%lld", (long long)q.ldc, (long long)q.n);
+  }
+  if (a_plane_k > 0) {
+    AH_ARG(q.k % a_plane_k == 0 && q.k / a_plane_k <= 3 && q.lda >= a_plane_k && a_plane_stride % 8 == 0,
+           "ah_gemm_planes: k = %lld is not 1 to 3 whole planes of %lld, or lda / the plane stride do not fit", (long long)q.k, (long long)a_plane_k);
+  } else {
+    AH_ARG(q.lda >= q.k, "matmul shape mismatch: lda %lld too small for k=%lld", (long long)q.lda, (long long)q.k);
+  }
+  AH_ARG(q.ldb >= (bkm ? q.n : q.k), "matmul shape mismatch: ldb %lld too small", (long long)q.ldb);
+  // what the large-tile kernel asks of its operands (the checks ah_gemm makes before it takes that kernel)
+  const bool fits = aligned16(q.a) && aligned16(q.b) && q.lda % 8 == 0 && q.ldb % 8 == 0 && (!bkm || q.n % 8 == 0) && q.k % 64 == 0 &&
+                    q.c % 8 == 0 && q.ldc % 4 == 0 && (a_plane_k == 0 || a_plane_k % 64 == 0) && (c_plane_cols == 0 || c_plane_cols % 128 == 0);
+  GemmArgs ga;
+  ga.a = dp<const void>(q.a); ga.b = dp<const void>(q.b); ga.c = dp<void>(q.c);
+  ga.aux = nullptr; ga.aux_out = nullptr;
+  ga.M = (int)q.m; ga.N = (int)q.n; ga.K = (int)q.k;
+  ga.lda = q.lda; ga.ldb = q.ldb; ga.ldc = q.ldc;
+  ga.sa = ga.sb = ga.sc = 0;
+  ga.epi = AH_EPI_NONE;
+  ga.ksplit = (int)q.k; ga.nsplit = 1;
+  ga.sumsq = nullptr;
+  if (c_plane_cols > 0) { ga.c_plane_n = (int)c_plane_cols; ga.c_plane_adj = c_plane_stride - c_plane_cols; }
+  if (a_plane_k > 0) { ga.a_plane_tiles = (int)(a_plane_k / 64); ga.a_plane_adj = (a_plane_stride - a_plane_k) * 2; }
+  if (!fits || !ah::gemm_bf16_takes_large_tile(ga, q.layout))
+    return fail(AH_ERR_UNSUPPORTED, "ah_gemm_planes: m=%lld n=%lld k=%lld does not run on the large-tile kernel", (long long)q.m, (long long)q.n, (long long)q.k);
+  if (dry_run) return AH_OK;
+  return ah::gemm_bf16_direct(ga, q.layout, 1, AH_BF16);
+}
+
 int32_t ah_gemm(const AhGemm *p) {
   AH_REQUIRE_READY();
   AH_ARG(p != nullptr, "ah_gemm: null descriptor");

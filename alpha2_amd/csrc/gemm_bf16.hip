@@ -235,33 +235,44 @@ int32_t launch(const GemmArgs &ga, int batch, int out_dtype) {
   return AH_OK;
 }
 
+// Large outputs go to the kernel fed by global->LDS loads (gemm_bf16_dma.inc): half the L2 traffic and a third of the
+// LDS traffic per flop of the 128x128 tile.  It holds one block per CU, so what matters is how evenly the tiles fill
+// whole rounds of CUs: take 256 x 256, 256 x 192 or 256 x 128 tiles, whichever wastes least of its last round, and keep the
+// 128x128 tile of this file (two blocks per CU, finer grain) when neither fills 70 %.  Returns the tile width, 0 = the
+// 128x128 kernel.  A product with planes only gets tile widths that divide a plane of C, and always gets one.
+int pick_large_tile(const GemmArgs &ga, int batch, bool akm, bool bkm) {
+  if (!(ga.M >= 256 && ga.N >= 128 && ga.ldc < (1 << 22))) return 0;      // (its epilogue addresses 128 rows of C with 31-bit byte offsets)
+  const int64_t cus = num_cus(), per = (int64_t)batch * ga.nsplit;
+  auto fill = [&](int bn) {
+    if (ga.c_plane_n > 0 && ga.c_plane_n % bn != 0) return 0.0;
+    int64_t t = cdiv(ga.M, 256) * cdiv(ga.N, bn) * per;
+    double useful = (double)ga.N / (double)(cdiv(ga.N, bn) * bn);        // columns of edge tiles that exist
+    return useful * (double)t / (double)(cdiv(t, cus) * cus);
+  };
+  // (narrower tiles read more from LDS per flop: measured ~3 % and ~8 % slower per flop than the 256-wide one; with two
+  // k-major operands, whose transposing LDS reads run at half rate, the 128-wide tile is ~35 % slower per flop)
+  double f256 = ga.N >= 256 ? fill(256) : 0.0, f192 = 0.97 * fill(192), f128 = (akm && bkm ? 0.65 : 0.92) * fill(128);
+  int bn = f256 >= f192 && f256 >= f128 ? 256 : f192 >= f128 ? 192 : 128;
+  const double best = bn == 256 ? f256 : bn == 192 ? f192 : f128;
+  if (ga.c_plane_n > 0 || ga.a_plane_adj != 0) return best > 0.0 ? bn : 0;      // planes exist on this kernel only: taken however few tiles there are
+  return best >= 0.7 ? bn : 0;
+}
+
 template <bool AKM, bool BKM>
 int32_t run(const GemmArgs &ga, int batch, int out_dtype) {
-  // Large outputs go to the kernel fed by global->LDS loads (gemm_bf16_dma.inc): half the L2 traffic and a third of the
-  // LDS traffic per flop of the 128x128 tile.  It holds one block per CU, so what matters is how evenly the tiles fill
-  // whole rounds of CUs: take 256 x 256, 256 x 192 or 256 x 128 tiles, whichever wastes least of its last round, and keep the
-  // 128x128 tile of this file (two blocks per CU, finer grain) when neither fills 70 %.
-  if (ga.M >= 256 && ga.N >= 128 && ga.ldc < (1 << 22)) {      // (its epilogue addresses 128 rows of C with 31-bit byte offsets)
-    const int64_t cus = num_cus(), per = (int64_t)batch * ga.nsplit;
-    auto fill = [&](int bn) {
-      int64_t t = cdiv(ga.M, 256) * cdiv(ga.N, bn) * per;
-      double useful = (double)ga.N / (double)(cdiv(ga.N, bn) * bn);        // columns of edge tiles that exist
-      return useful * (double)t / (double)(cdiv(t, cus) * cus);
-    };
-    // (narrower tiles read more from LDS per flop: measured ~3 % and ~8 % slower per flop than the 256-wide one; with two
-    // k-major operands, whose transposing LDS reads run at half rate, the 128-wide tile is ~35 % slower per flop)
-    double f256 = ga.N >= 256 ? fill(256) : 0.0, f192 = 0.97 * fill(192), f128 = (AKM && BKM ? 0.65 : 0.92) * fill(128);
-    int bn = f256 >= f192 && f256 >= f128 ? 256 : f192 >= f128 ? 192 : 128;
-
-    if ((bn == 256 ? f256 : bn == 192 ? f192 : f128) >= 0.7)
-      return AKM ? gemm_bf16_dma_tn(ga, batch, out_dtype, bn) : BKM ? gemm_bf16_dma_nn(ga, batch, out_dtype, bn) : gemm_bf16_dma_nt(ga, batch, out_dtype, bn);
-  }
+  const int bn = pick_large_tile(ga, batch, AKM, BKM);
+  if (bn) return AKM ? gemm_bf16_dma_tn(ga, batch, out_dtype, bn) : BKM ? gemm_bf16_dma_nn(ga, batch, out_dtype, bn) : gemm_bf16_dma_nt(ga, batch, out_dtype, bn);
+  if (ga.c_plane_n > 0 || ga.a_plane_adj != 0) return fail(AH_ERR_UNSUPPORTED, "ah_gemm_planes: this shape does not run on the large-tile kernel");
   return launch<128, 128, 2, 2, AKM, BKM>(ga, batch, out_dtype);
 }
 
 }  // namespace
 
 namespace ah {
+
+bool gemm_bf16_takes_large_tile(const GemmArgs &ga, int layout) {
+  return pick_large_tile(ga, 1, layout == AH_GEMM_TN, layout != AH_GEMM_NT) != 0;
+}
 
 // Preconditions (checked by the caller): K % 64 == 0; operands 16-byte aligned with lda/ldb/strides % 8 == 0;
 // M % 8 == 0 (N % 8 == 0) when A (B) is k-major; C/aux rows vector-aligned; a provided epilogue/output combination.

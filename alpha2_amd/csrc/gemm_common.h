@@ -29,6 +29,11 @@ struct GemmArgs {
   int epi;
   int ksplit, nsplit;  // split-K (bf16 direct kernel only): K elements per split, number of splits (1 = off)
   float *sumsq;        // grouped launches that also sum the squares of what they store: the block's four slots (one per wave)
+  // Planes (the large-tile bf16 kernel with a k-contiguous A only; off by default).  C: columns [p n, (p + 1) n) with
+  // n = c_plane_n live c_plane_adj ELEMENTS further per p than in one [M, ldc] matrix.  A: k-tiles [p t, (p + 1) t) with
+  // t = a_plane_tiles live a_plane_adj BYTES further per p than in one [M, lda] matrix (p <= 2).
+  int c_plane_n = 0, a_plane_tiles = 1 << 28;
+  int64_t c_plane_adj = 0, a_plane_adj = 0;
 };
 
 // Epilogue for 4 consecutive columns (col..col+3) of one row: the MFMA operands are swapped (acc = B-frag x A-frag)
@@ -276,6 +281,7 @@ __device__ __forceinline__ void store_tiles(const GemmArgs &g, int64_t cbase, in
 
 // gemm_bf16.hip
 int32_t gemm_bf16_direct(const GemmArgs &ga, int layout, int batch, int out_dtype);
+bool gemm_bf16_takes_large_tile(const GemmArgs &ga, int layout);       // would gemm_bf16_direct run it on the 256-row tile kernel (batch 1)
 // c[M][N] (leading dimension ldc) = (accumulate ? c : 0) + sum over the nsplit slices of ws[nsplit][M][N], in fixed order; M N % 4 == 0
 int32_t splitk_reduce(const float *ws, float *c, int nsplit, int M, int N, int64_t ldc, bool accumulate);
 // gemm_bf16_dma_{nt,nn,tn}.hip: 256 x bn tiles (bn = 256 or 192) fed by direct global->LDS loads (same preconditions as the

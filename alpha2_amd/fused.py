@@ -65,6 +65,19 @@ class FusedTrainer:
         if self.D not in (32, 64, 128) or self.C % 8 or self.F % 64 or self.C % 64 or self.V % 8:
             raise ValueError("FusedTrainer needs head_dim in {32,64,128}, nEmbd and ffnDim multiples of 64, vocab multiple of 8")
         self.BT = batch * self.T
+        # Which function the attention sub-layer computes: "heads" = multi-head attention on the columns of the [BT, 3C] projection;
+        # "reference-flash" = what gpt.ts:247-254 computes on a backend with flashAttention: q, k, v cut out of the projection
+        # as contiguous [BT, C] matrices and re-read as [B H, T, D] slabs without a head transpose.  Here the projection writes
+        # the three matrices itself and its backward reads the three gradients where the attention kernel leaves them
+        # (ah_gemm_planes), so the wiring moves no data.
+        if cfg.attention not in ("heads", "reference-flash"):
+            raise ValueError("FusedTrainer computes attention with the fused kernel: attention must be 'heads' or 'reference-flash'")
+        self.slabs = cfg.attention == "reference-flash"
+        if self.slabs:
+            probe = ffi.AhGemm(ffi.GEMM_NT, BF16, BF16, ffi.EPI_NONE, self.BT, 3 * self.C, self.C, self.C, self.C, self.C, 1, 0, 0, 0, 256, 256, 256, 0)
+            if self.lib.ah_gemm_planes(C.byref(probe), self.C, self.BT * self.C, 0, 0, 1) != 0:
+                raise ValueError("FusedTrainer with attention='reference-flash' needs a shape that ah_gemm_planes takes: "
+                                 + self.lib.ah_last_error().decode("utf-8", "replace"))
         self.dw_groups = max(1, min(int(dw_groups), self.L))
         self._want_norm_in_epilogue = bool(norm_in_epilogue)
         # The residual stream x and the gradient that flows back along it: f32, or bf16 like every other activation
@@ -181,13 +194,16 @@ class FusedTrainer:
         soon as backward has passed its lowest layer, beside the backward kernels of the layers below."""
         BT, Cc, Fd, V, TN = self.BT, self.C, self.F, self.V, ffi.GEMM_TN     # (swiglu: d[gate; up] is one [2F, C] product)
 
-        def desc(dy, x, gname, m, n):
-            return ffi.AhGemm(TN, BF16, F32, ffi.EPI_NONE, m, n, BT, m, n, n, 1, 0, 0, 0, dy, x, self.g(gname), 0)
+        def desc(dy, x, gname, m, n, row0=0):
+            return ffi.AhGemm(TN, BF16, F32, ffi.EPI_NONE, m, n, BT, m, n, n, 1, 0, 0, 0, dy, x, self.g(gname) + row0 * n * 4, 0)
 
         def layer(l):
             pre = f"layer.{l}."
-            return [desc(self.dy_fc2[l], self.hact[l], pre + self.w2, Cc, Fd), desc(self.dh[l], self.ln2[l], pre + self.w1, self.Fin, Cc),
-                    desc(self.dy_wo[l], self.att[l], pre + "attn.wo", Cc, Cc), desc(self.dqkv[l], self.ln1[l], pre + "attn.wqkv", 3 * Cc, Cc)]
+            d = [desc(self.dy_fc2[l], self.hact[l], pre + self.w2, Cc, Fd), desc(self.dh[l], self.ln2[l], pre + self.w1, self.Fin, Cc),
+                 desc(self.dy_wo[l], self.att[l], pre + "attn.wo", Cc, Cc)]
+            if self.slabs:      # dq, dk, dv lie apart as [BT, C] matrices: rows [p C, (p + 1) C) of the [3C, C] gradient each
+                return d + [desc(self.dqkv[l] + p * BT * Cc * 2, self.ln1[l], pre + "attn.wqkv", Cc, Cc, p * Cc) for p in range(3)]
+            return d + [desc(self.dqkv[l], self.ln1[l], pre + "attn.wqkv", 3 * Cc, Cc)]
         n = self.dw_groups
         bounds = [self.L - (self.L * (k + 1)) // n for k in range(n)]          # lowest layer of run k (run n-1 ends at layer 0)
         self._dw_after_layer = {}                                                # layer whose backward completes run k -> k
@@ -278,14 +294,20 @@ class FusedTrainer:
     def g(self, name: str) -> int:
         return self.G + self.off[name] * 4
 
-    def _gemm(self, layout, a, b, c, m, n, k, lda, ldb, ldc, out=BF16, epi=ffi.EPI_NONE, aux=0):
+    def _gemm(self, layout, a, b, c, m, n, k, lda, ldb, ldc, out=BF16, epi=ffi.EPI_NONE, aux=0, c_planes=None, a_planes=None):
+        """One product; c_planes / a_planes = (extent, stride) of the planes C's columns / A's contraction lie in."""
         g = ffi.AhGemm(layout, BF16, out, epi, m, n, k, lda, ldb, ldc, 1, 0, 0, 0, a, b, c, aux)
+        if c_planes or a_planes:
+            cp, ap = c_planes or (0, 0), a_planes or (0, 0)
+            run = lambda: check(self.lib.ah_gemm_planes(C.byref(g), cp[0], cp[1], ap[0], ap[1], 0))
+        else:
+            run = lambda: check(self.lib.ah_gemm(C.byref(g)))
         if self._timed is None:
-            check(self.lib.ah_gemm(C.byref(g)))
+            run()
             return
         e0, e1 = self.B._event(), self.B._event()
         check(self.lib.ah_event_record(e0))
-        check(self.lib.ah_gemm(C.byref(g)))
+        run()
         check(self.lib.ah_event_record(e1))
         kernel, nsplit = self.B.lastGemmKernel()
         self._timed.append({"kind": "gemm", "kernel": kernel, "nsplit": nsplit, "layout": layout, "m": m, "n": n, "k": k,
@@ -295,15 +317,18 @@ class FusedTrainer:
         Cc, T, D = self.C, self.T, self.D
         f = ffi.AhFlash()
         f.dtype, f.batch, f.heads, f.seq, f.head_dim = BF16, self.batch, self.H, T, D
+        # where q, k, v (and their gradients) of (batch b, head h, position t) lie: in columns h D .. of row b T + t of the
+        # [BT, 3C] projection, or -- slabs -- in row t of slab b H + h of a contiguous [BT, C] matrix read as [B H, T, D]
+        sb, sh, st, nxt = (T * Cc, T * D, D, self.BT * Cc * 2) if self.slabs else (T * 3 * Cc, D, 3 * Cc, Cc * 2)
         for nm in ("q", "k", "v"):
-            setattr(f, nm + "_sb", T * 3 * Cc), setattr(f, nm + "_sh", D), setattr(f, nm + "_st", 3 * Cc)
-        f.o_sb, f.o_sh, f.o_st = T * Cc, D, Cc
+            setattr(f, nm + "_sb", sb), setattr(f, nm + "_sh", sh), setattr(f, nm + "_st", st)
+        f.o_sb, f.o_sh, f.o_st = T * Cc, D, Cc            # (the slabs' result transposed back, gpt.ts:254, is this same layout)
         f.scale, f.soft_cap = 1 / math.sqrt(D), self.cap
         q = self.qkv[l]
-        f.q, f.k, f.v, f.o, f.lse = q, q + Cc * 2, q + 2 * Cc * 2, self.att[l], self.lse[l]
+        f.q, f.k, f.v, f.o, f.lse = q, q + nxt, q + 2 * nxt, self.att[l], self.lse[l]
         if bwd:
             d = self.dqkv[l]
-            f.d_o, f.dq, f.dk, f.dv = self.datt, d, d + Cc * 2, d + 2 * Cc * 2
+            f.d_o, f.dq, f.dk, f.dv = self.datt, d, d + nxt, d + 2 * nxt
         t0 = None
         if self._timed is not None:
             t0 = self.B._event()
@@ -331,7 +356,10 @@ class FusedTrainer:
         for l in range(L):
             pre = f"layer.{l}."
             check(lib.ah_layernorm(self.x[l], self.p(pre + "ln1.weight"), self.p(pre + "ln1.bias"), self.ln1[l], BT, Cc, 1e-5, BF16, SD))
-            self._gemm(NT, self.ln1[l], self.p(pre + "attn.wqkv", True), self.qkv[l], BT, 3 * Cc, Cc, Cc, Cc, 3 * Cc)
+            if self.slabs:
+                self._gemm(NT, self.ln1[l], self.p(pre + "attn.wqkv", True), self.qkv[l], BT, 3 * Cc, Cc, Cc, Cc, Cc, c_planes=(Cc, BT * Cc))
+            else:
+                self._gemm(NT, self.ln1[l], self.p(pre + "attn.wqkv", True), self.qkv[l], BT, 3 * Cc, Cc, Cc, Cc, 3 * Cc)
             self._flash(l, False)
             self._gemm(NT, self.att[l], self.p(pre + "attn.wo", True), self.xmid[l], BT, Cc, Cc, Cc, Cc, Cc, SD, ffi.EPI_RESIDUAL, self.x[l])
             check(lib.ah_layernorm(self.xmid[l], self.p(pre + "ln2.weight"), self.p(pre + "ln2.bias"), self.ln2[l], BT, Cc, 1e-5, BF16, SD))
@@ -380,7 +408,10 @@ class FusedTrainer:
             # attention: x_mid = x_in + wo(attn(wqkv(ln1(x_in))))
             self._gemm(NN, self.dy_wo[l], self.p(pre + "attn.wo", True), self.datt, BT, Cc, Cc, Cc, Cc, Cc)
             self._flash(l, True)
-            self._gemm(NN, self.dqkv[l], self.p(pre + "attn.wqkv", True), self.dlnb, BT, Cc, 3 * Cc, 3 * Cc, Cc, Cc)
+            if self.slabs:
+                self._gemm(NN, self.dqkv[l], self.p(pre + "attn.wqkv", True), self.dlnb, BT, Cc, 3 * Cc, Cc, Cc, Cc, a_planes=(Cc, BT * Cc))
+            else:
+                self._gemm(NN, self.dqkv[l], self.p(pre + "attn.wqkv", True), self.dlnb, BT, Cc, 3 * Cc, 3 * Cc, Cc, Cc)
             check(lib.ah_layernorm_bwd_deferred(self.x[l], self.p(pre + "ln1.weight"), self.dlnb, BF16, self.dx[cur] if f32s else self.dy_wo[l],
                                                 self.dx[cur ^ 1] if f32s else (self.dx[0] if l == 0 else 0),      # the embeddings take their gradient in f32
                                                 self.dy_fc2[l - 1] if l > 0 else self.dxb0, self._ln_part[pre + "ln1"], BT, Cc, 1e-5, SD))

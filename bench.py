@@ -102,8 +102,8 @@ def main():
                     "arena again instead of summing the weight gradients' squares in the epilogue of the launch that stores them")
     ap.add_argument("--stream", choices=["f32", "bf16"], default="bf16", help="fast mode: storage type of the residual stream and its gradient")
     ap.add_argument("--attention", choices=["heads", "reference-flash", "unfused"], default="heads",
-                    help="backend / parity mode: which attention branch of the model runs (reference-flash = the op sequence of the "
-                         "reference's flash branch, gpt.ts:232-253; unfused = its CPU branch)")
+                    help="which attention branch of the model runs (reference-flash = what the reference's flash branch computes, "
+                         "gpt.ts:232-253; heads = multi-head attention; unfused = its CPU branch, backend / parity mode only)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="only the headline measurement: no backend-mode and no 350M-shape runs")
     ap.add_argument("--cpu-tokens", type=int, default=32)
@@ -207,7 +207,7 @@ def main():
         "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": f"synthetic (Zipf s=1.1 token ids, seed {tok_seed}; random-init N(0,0.02) weights, seed 0)",
         "config": {"workload": describe,
                    "tokens_per_step": tokens, "mode": args.mode, "loss_first_step": loss_first, "loss_last_step": loss_last,
-                   **({"attention": args.attention} if args.mode != "fast" else {})},
+                   "attention": args.attention},
         # model flops per second against the dense bf16 MFMA peak: by the reference's (non-causal) attention count, and with
         # the causal half of the attention products only
         "step_tflops": flops / (ms * 1e-3) / 1e12, "mfu_vs_bf16_dense_peak": flops / (ms * 1e-3) / 1e12 / PEAK["bf16"],

@@ -355,6 +355,19 @@ typedef struct {
   ah_ptr  a, b, c, aux;
 } AhGemm;
 int32_t ah_gemm(const AhGemm *g);
+/* ah_gemm with one operand in planes, so that a fused projection needs no copy around it.  Replaces the data movement of
+ * Backend.sliceQkv (interfaces.ts:117; ops.ts:816-840: the [rows, 3C] product cut into three contiguous [rows, C]
+ * tensors) and of the three Backend.scatterSlice results added up in its backward (interfaces.ts:121; ops.ts:826-834):
+ *   c_plane_cols > 0: columns [p c_plane_cols, (p + 1) c_plane_cols) of C are stored as the [m, c_plane_cols] matrix at
+ *     c + p * c_plane_stride (elements) with row stride ldc: the product writes q, k and v where sliceQkv would put them;
+ *   a_plane_k > 0: columns [p a_plane_k, (p + 1) a_plane_k) of the row-major A [m, k] are read from the [m, a_plane_k] matrix
+ *     at a + p * a_plane_stride with row stride lda (1 to 3 planes): the product reads dq, dk, dv where flash attention's
+ *     backward leaves them, as if scattered into one [rows, 3C] gradient and added.
+ * One plain product (layout NN or NT, bf16 operands and result, batch 1) on the 256-row tile kernel: m >= 256, n >= 128,
+ * k and a_plane_k % 64 == 0, c_plane_cols % 128 == 0, operands 16-byte aligned with lda, ldb % 8 == 0; anything else returns
+ * AH_ERR_UNSUPPORTED and the caller moves the data instead.  dry_run != 0 only answers (AH_OK / AH_ERR_UNSUPPORTED), nothing is launched. */
+int32_t ah_gemm_planes(const AhGemm *g, int64_t c_plane_cols, int64_t c_plane_stride, int64_t a_plane_k, int64_t a_plane_stride,
+                       int32_t dry_run);
 /* Grouped GEMM: several independent problems of ONE layout in one launch (256x256 tiles of all problems share the
  * grid, so small outputs with a long contraction fill the chip without split-K).  Used for the weight gradients
  * dW_i = G_i^T X_i of all layers at the end of backward; the reference computes them one matmul at a time

@@ -64,6 +64,7 @@ export const lib = dlopen(process.env.ALPHA_HIP_LIB ?? "libalpha_hip.so", {
   ah_gemm_grouped_run_sumsq:       { args: [u64, i32, u64], returns: i32 },
   ah_gemm_grouped_update:          { args: [u64, ptr, i32], returns: i32 },
   ah_gemm_last_kernel:             { args: [ptr, i32, ptr], returns: i32 },
+  ah_gemm_planes:                  { args: [ptr, i64, i64, i64, i64, i32], returns: i32 },
   ah_graph_begin:                  { args: [], returns: i32 },
   ah_graph_destroy:                { args: [u64], returns: i32 },
   ah_graph_end:                    { args: [ptr], returns: i32 },

@@ -39,7 +39,8 @@ def _expected_initial_loss(cfg):
     return math.log(cfg["vocabSize"]) + 0.5 * 0.02 ** 2 * cfg["nEmbd"]
 
 
-@pytest.mark.parametrize("name,cfg,batch,accum,seed", [("gpt2-small", SMALL, 16, 1, 4), ("350m", M350, 8, 4, 5)])
+@pytest.mark.parametrize("name,cfg,batch,accum,seed", [("gpt2-small", SMALL, 16, 1, 4), ("350m", M350, 8, 4, 5),
+                                                       ("gpt2-small-slabs", dict(SMALL, attention="reference-flash"), 16, 1, 4)])
 def test_full_size_step_properties(B, name, cfg, batch, accum, seed):
     from alpha2_amd.train import zipfBatch
     steps = 6                                             # past the spike that the first warm-up steps make

@@ -19,17 +19,24 @@ def B():
     return HipBackend(0)
 
 
-def _make(B, tc_kw, use_graph, seed=0, batch=4, **kw):
+def _make(B, tc_kw, use_graph, seed=0, batch=4, attention="heads", **kw):
     from alpha2_amd.fused import FusedTrainer
     from alpha2_amd.model import ModelConfig
     from alpha2_amd.train import TrainConfig
-    return FusedTrainer(B, ModelConfig(**CFG), TrainConfig(**tc_kw), batch, seed=seed, use_graph=use_graph, **kw)
+    return FusedTrainer(B, ModelConfig(**CFG, attention=attention), TrainConfig(**tc_kw), batch, seed=seed, use_graph=use_graph, **kw)
 
 
-def test_fused_step_gradients_and_update_match_oracle(B):
+# "heads": multi-head attention (the oracle's CPU branch, gpt.ts:255-279); "reference-flash": the slabs an unchanged gpt.ts
+# hands to flashAttention (gpt.ts:247-254), which the fused step wires without moving data (ah_gemm_planes)
+ATTENTION = ["heads", "reference-flash"]
+
+
+@pytest.mark.parametrize("attention", ATTENTION)
+def test_fused_step_gradients_and_update_match_oracle(B, attention):
     from alpha2_amd.train import syntheticBatch
-    ft = _make(B, dict(iters=1), use_graph=False)
-    orc = rm.Trainer(rm.ModelConfig(**CFG), rm.TrainConfig(iters=1), seed=0)
+    ft = _make(B, dict(iters=1), use_graph=False, attention=attention)
+    assert ft.slabs == (attention == "reference-flash")
+    orc = rm.Trainer(rm.ModelConfig(**CFG, attention=attention), rm.TrainConfig(iters=1), seed=0)
     for name, v in orc.entries:
         assert np.array_equal(ft.param(name), v.data.data), name          # same initial parameters, bit for bit
     ft.set_batch(*syntheticBatch(1, 4, 64, 256))
@@ -59,13 +66,14 @@ def test_fused_step_gradients_and_update_match_oracle(B):
         assert np.sqrt(np.mean(d * d)) <= 0.35 * 3e-4, name               # and mostly in the same direction as the oracle
 
 
-def test_fused_loss_parity_over_steps_graph_replay(B):
+@pytest.mark.parametrize("attention", ATTENTION)
+def test_fused_loss_parity_over_steps_graph_replay(B, attention):
     from alpha2_amd.train import syntheticBatch
     steps = 50
     tc = dict(iters=steps)
-    ft = _make(B, tc, use_graph=True, seed=3)
-    eager = _make(B, tc, use_graph=False, seed=3)
-    orc = rm.Trainer(rm.ModelConfig(**CFG), rm.TrainConfig(iters=steps), seed=3)
+    ft = _make(B, tc, use_graph=True, seed=3, attention=attention)
+    eager = _make(B, tc, use_graph=False, seed=3, attention=attention)
+    orc = rm.Trainer(rm.ModelConfig(**CFG, attention=attention), rm.TrainConfig(iters=steps), seed=3)
     ids = [ft.add_batch(*syntheticBatch(50 + s, 4, 64, 256)) for s in range(steps)]
     for s in range(steps):
         eager.add_batch(*syntheticBatch(50 + s, 4, 64, 256))
@@ -85,7 +93,8 @@ def test_fused_loss_parity_over_steps_graph_replay(B):
     ft.close(), eager.close()
 
 
-def test_fused_gradient_accumulation_matches_oracle(B):
+@pytest.mark.parametrize("attention", ATTENTION)
+def test_fused_gradient_accumulation_matches_oracle(B, attention):
     """Two micro-batches per optimizer step: summed gradients scaled once, reported loss = mean of the micro losses
     (trainer.ts:1164-1273); graph replay and eager execution agree."""
     from alpha2_amd.fused import FusedTrainer
@@ -93,9 +102,9 @@ def test_fused_gradient_accumulation_matches_oracle(B):
     from alpha2_amd.train import TrainConfig, syntheticBatch
     steps, K = 6, 2
     tc = dict(iters=steps, gradAccumSteps=K)
-    mk = lambda graph: FusedTrainer(B, ModelConfig(**CFG), TrainConfig(**tc), 4, seed=5, use_graph=graph, accum=K)
+    mk = lambda graph: FusedTrainer(B, ModelConfig(**CFG, attention=attention), TrainConfig(**tc), 4, seed=5, use_graph=graph, accum=K)
     ft, eager = mk(True), mk(False)
-    orc = rm.Trainer(rm.ModelConfig(**CFG), rm.TrainConfig(iters=steps, gradAccumSteps=K), seed=5)
+    orc = rm.Trainer(rm.ModelConfig(**CFG, attention=attention), rm.TrainConfig(iters=steps, gradAccumSteps=K), seed=5)
     for s in range(steps):
         seeds = [300 + K * s + m for m in range(K)]
         ids = [ft.add_batch(*syntheticBatch(sd, 4, 64, 256)) for sd in seeds]

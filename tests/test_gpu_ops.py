@@ -1406,6 +1406,74 @@ def test_gemm_microbench_shapes_forward_and_both_backward(B, N, in_dtype):
         lib.ah_free(p)
 
 
+@pytest.mark.parametrize("M,Cc", [(16384, 768), (4096, 768), (8192, 1024)])
+def test_gemm_with_an_operand_in_planes_equals_the_product_around_copies(B, M, Cc):
+    """ah_gemm_planes: the fused qkv projection writing q, k, v as three contiguous [M, C] matrices (what sliceQkv,
+    ops.ts:816-840, makes of the [M, 3C] product) and the input gradient read from dq, dk, dv lying apart (what three
+    scatterSlice results added up, ops.ts:826-834, would hold as one [M, 3C] matrix): bit for bit the ordinary products
+    of the same operands, which are checked against float64 on sampled rows."""
+    import ctypes as C
+    from alpha2_amd import _ffi as ffi
+    lib = B.lib
+    rng = np.random.default_rng(11)
+
+    def bits(shape, std):
+        x = (rng.standard_normal(shape, dtype=np.float32) * np.float32(std)).view(np.uint32)
+        x += np.uint32(0x7FFF) + ((x >> np.uint32(16)) & np.uint32(1))
+        return (x >> np.uint32(16)).astype(np.uint16)
+    f64 = lambda u: (u.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+    live = []
+
+    def up(u):
+        p = C.c_uint64()
+        ffi.check(lib.ah_alloc(max(u.nbytes, 16), C.byref(p)))
+        ffi.check(lib.ah_upload(p.value, u.ctypes.data_as(C.c_void_p), u.nbytes))
+        live.append(p.value)
+        return p.value
+
+    def down(ptr, shape):
+        out = np.empty(shape, np.uint16)
+        ffi.check(lib.ah_download(out.ctypes.data_as(C.c_void_p), ptr, out.nbytes))
+        return out
+    x, w, g = bits((M, Cc), 1.0), bits((3 * Cc, Cc), 0.02), bits((M, 3 * Cc), 0.5)
+    px, pw, pg = up(x), up(w), up(g)
+    pg_planes = up(np.ascontiguousarray(g.reshape(M, 3, Cc).transpose(1, 0, 2)))            # [3][M][C]
+    c1, c2 = up(np.zeros((M, 3 * Cc), np.uint16)), up(np.full((3, M, Cc), 0x7FC0, np.uint16))
+    d1, d2 = up(np.zeros((M, Cc), np.uint16)), up(np.full((M, Cc), 0x7FC0, np.uint16))
+    BF = ffi.BF16
+    # forward: [M, C] x [3C, C]^T
+    fwd = ffi.AhGemm(ffi.GEMM_NT, BF, BF, ffi.EPI_NONE, M, 3 * Cc, Cc, Cc, Cc, 3 * Cc, 1, 0, 0, 0, px, pw, c1, 0)
+    ffi.check(lib.ah_gemm(C.byref(fwd)))
+    fwd.ldc, fwd.c = Cc, c2
+    ffi.check(lib.ah_gemm_planes(C.byref(fwd), Cc, M * Cc, 0, 0, 1))                          # asked first, nothing launched
+    assert (down(c2, (8,)) == 0x7FC0).all()
+    ffi.check(lib.ah_gemm_planes(C.byref(fwd), Cc, M * Cc, 0, 0, 0))
+    assert B.lastGemmKernel()[0].startswith("k_gemm_bf16_dma_planes<false, false")
+    whole, planes = down(c1, (M, 3 * Cc)), down(c2, (3, M, Cc))
+    for p in range(3):
+        assert np.array_equal(planes[p], whole[:, p * Cc:(p + 1) * Cc]), p
+    rows = np.sort(rng.choice(M, 16, replace=False))
+    assert_close(f64(whole[rows]), f64(x[rows]) @ f64(w).T, rel=1e-2, what="qkv rows")         # (bf16 result: half an ulp is 2^-9)
+    # input gradient: [M, 3C] x [3C, C]
+    bwd = ffi.AhGemm(ffi.GEMM_NN, BF, BF, ffi.EPI_NONE, M, Cc, 3 * Cc, 3 * Cc, Cc, Cc, 1, 0, 0, 0, pg, pw, d1, 0)
+    ffi.check(lib.ah_gemm(C.byref(bwd)))
+    bwd.lda, bwd.a, bwd.c = Cc, pg_planes, d2
+    ffi.check(lib.ah_gemm_planes(C.byref(bwd), 0, 0, Cc, M * Cc, 0))
+    assert B.lastGemmKernel()[0].startswith("k_gemm_bf16_dma_planes<false, true")
+    whole, planes = down(d1, (M, Cc)), down(d2, (M, Cc))
+    assert np.array_equal(whole, planes)
+    assert_close(f64(planes[rows]), f64(g[rows]) @ f64(w), rel=1e-2, what="dx rows")
+    # what it does not take is refused with a reason and nothing is launched
+    small = ffi.AhGemm(ffi.GEMM_NT, BF, BF, ffi.EPI_NONE, 128, 3 * Cc, Cc, Cc, Cc, Cc, 1, 0, 0, 0, px, pw, c2, 0)
+    assert lib.ah_gemm_planes(C.byref(small), Cc, 128 * Cc, 0, 0, 1) == 5
+    f32out = ffi.AhGemm(ffi.GEMM_NT, BF, ffi.F32, ffi.EPI_NONE, M, 3 * Cc, Cc, Cc, Cc, Cc, 1, 0, 0, 0, px, pw, c2, 0)
+    assert lib.ah_gemm_planes(C.byref(f32out), Cc, M * Cc, 0, 0, 0) == 5
+    ragged = ffi.AhGemm(ffi.GEMM_NT, BF, BF, ffi.EPI_NONE, M, 3 * Cc, Cc, Cc, Cc, Cc, 1, 0, 0, 0, px, pw, c2, 0)
+    assert lib.ah_gemm_planes(C.byref(ragged), Cc - 64, M * Cc, 0, 0, 0) == 2
+    for p in live:
+        lib.ah_free(p)
+
+
 @pytest.mark.parametrize("BH,T,D", [(20, 384, 64), (60, 2048, 128)])
 @pytest.mark.parametrize("store", ["bf16", "f32"])
 def test_flash_attention_heads_are_independent_of_how_blocks_are_dealt_out(B, store, BH, T, D):
