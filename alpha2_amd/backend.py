@@ -108,6 +108,7 @@ class HipBackend:
         self.lastStepHow, self.lastStepNote = "eager", ""
         self.stepFallbackNotes: List[str] = []
         self._hyper_dev, self._hyper_key = None, None
+        self.planeProducts = 0                 # products issued through ah_gemm_planes (an operand in planes, no copy around it)
         self.flashBackwardVariant = 0          # AhFlash.bwd_variant for the bf16 backward kernels (1: one pass over the scores)
 
     # ------------------------------------------------------------------ residency helpers
@@ -319,15 +320,18 @@ class HipBackend:
     def div(self, a, b): return self._binary(ffi.DIV, a, b)
 
     def _gemm(self, layout, a_ptr, b_ptr, c_ptr, m, n, k, lda, ldb, ldc, batch=1, sa=0, sb=0, sc=0, in_dtype=ffi.F32,
-              out_dtype=ffi.F32, epilogue=ffi.EPI_NONE, aux=0):
+              out_dtype=ffi.F32, epilogue=ffi.EPI_NONE, aux=0, planes=None):
+        """planes = (c_plane_cols, c_plane_stride, a_plane_k, a_plane_stride): the product goes through ah_gemm_planes."""
         g = ffi.AhGemm(layout, in_dtype, out_dtype, epilogue, m, n, k, lda, ldb, ldc, batch, sa, sb, sc, a_ptr, b_ptr, c_ptr, aux)
+        run = (lambda: check(self.lib.ah_gemm(C.byref(g)))) if planes is None else (lambda: check(self.lib.ah_gemm_planes(C.byref(g), *planes, 0)))
+        self.planeProducts += planes is not None
         timed = getattr(self, "_timed", None)
         if timed is None:
-            check(self.lib.ah_gemm(C.byref(g)))
+            run()
             return
         e0, e1 = self._event(), self._event()
         check(self.lib.ah_event_record(e0))
-        check(self.lib.ah_gemm(C.byref(g)))
+        run()
         check(self.lib.ah_event_record(e1))
         kernel, nsplit = self.lastGemmKernel()
         timed.append({"kind": "gemm", "kernel": kernel, "nsplit": nsplit, "layout": layout, "dtype": in_dtype, "m": m, "n": n, "k": k,

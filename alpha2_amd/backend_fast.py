@@ -35,11 +35,14 @@ BF16, F32 = ffi.BF16, ffi.F32
 class _HeldGemm:
     """A product whose launch is held back by one call.  It holds a reference on its operands' buffers and on its output
     buffer until it is launched (or dropped, when nobody but this record still refers to the output)."""
-    __slots__ = ("layout", "a_ptr", "b_ptr", "out_buf", "out_off", "m", "n", "k", "lda", "ldb", "holds")
+    __slots__ = ("layout", "a_ptr", "b_ptr", "out_buf", "out_off", "m", "n", "k", "lda", "ldb", "holds", "a_planes")
 
     def __init__(self, layout, a_ptr, b_ptr, out, m, n, k, lda, ldb, holds):
         self.layout, self.a_ptr, self.b_ptr, self.out_buf, self.out_off = layout, a_ptr, b_ptr, out._buf, out._off
         self.m, self.n, self.k, self.lda, self.ldb, self.holds = m, n, k, lda, ldb, holds
+        # A lies in planes (an unwritten sum of scatterSlice results): (columns per plane, elements from plane to plane), a_ptr
+        # the first plane, lda its row stride
+        self.a_planes = None
 
     @property
     def out_ptr(self) -> int:
@@ -47,10 +50,12 @@ class _HeldGemm:
 
 
 class _HeldWeightGrad:
-    __slots__ = ("g_ptr", "x_ptr", "out_buf", "out_off", "m", "n", "k", "holds", "into", "add_after")
+    __slots__ = ("g_ptr", "x_ptr", "out_buf", "out_off", "m", "n", "k", "holds", "into", "add_after", "planes", "dst")
 
     def __init__(self, g_ptr, x_ptr, out, m, n, k, holds):
         self.g_ptr, self.x_ptr, self.out_buf, self.out_off, self.m, self.n, self.k, self.holds = g_ptr, x_ptr, out._buf, out._off, m, n, k, holds
+        self.planes = None                # G lies in planes: (columns per plane, bytes from plane to plane); one problem per plane
+        self.dst = None                   # set at launch: where the product (all of its problems) is written
         self.into = None                  # (buffer, offset) of an existing gradient to accumulate into instead
         self.add_after = None             # set at launch: the same, when the product had to be computed into its own tensor
 
@@ -114,6 +119,7 @@ class FastHipBackend(HipBackend):
         self._adam_bufs = set()          # id(_Buf) of every buffer a queued update reads or writes
         self._ssq_args = None            # (addresses, sizes, their ctypes arrays) of the last totalSumOfSquares call
         self._scatters = {}              # id(_Buf) of an unwritten scatterSlice result -> _HeldScatter
+        self._planes_ok = {}             # (layout, m, n, k, plane extents) -> does ah_gemm_planes take it
         self._held_ce: Optional[_HeldCrossEntropy] = None
         self._held_ln: Optional[_HeldLayerNormBwd] = None
         # dx tensors whose LayerNorm backward went straight into a sum and that were never written themselves: id(_Buf) -> recipe
@@ -161,7 +167,7 @@ class FastHipBackend(HipBackend):
                 self._launch_weight_grads()
             elif self._orphans and id(t._buf) in self._orphans:
                 h = self._orphans.pop(id(t._buf))
-                self._gemm(h.layout, h.a_ptr, h.b_ptr, h.out_ptr, h.m, h.n, h.k, h.lda, h.ldb, h.n, in_dtype=BF16, out_dtype=BF16)
+                self._run_held(h, h.out_ptr)
                 self._unhold(h.holds)
         return super()._ptr(t)
 
@@ -203,11 +209,44 @@ class FastHipBackend(HipBackend):
     # inside them, so a bf16 tensor whose innermost dimension is even and is left whole (or cut at even columns) is moved as
     # the tensor of half that width: q, k, v and the head transposes of the reference's attention branch (gpt.ts:232-253) stay
     # in bf16 instead of being widened to f32 first.
+    def _takes_planes(self, layout, m, n, k, lda, ldb, ldc, c_planes=(0, 0), a_planes=(0, 0)) -> bool:
+        key = (layout, m, n, k, lda, ldb, ldc, c_planes, a_planes)
+        ok = self._planes_ok.get(key)
+        if ok is None:                                          # asked once per shape: nothing is launched
+            g = ffi.AhGemm(layout, BF16, BF16, ffi.EPI_NONE, m, n, k, lda, ldb, ldc, 1, 0, 0, 0, 256, 256, 256, 0)
+            ok = self._planes_ok[key] = self.lib.ah_gemm_planes(C.byref(g), *c_planes, *a_planes, 1) == 0
+        return ok
+
+    def _plane_views(self, count: int, shape) -> list:
+        """`count` bf16 tensors of one shape that lie one behind the other in one allocation."""
+        n = shapeSize(shape)
+        buf = _Buf(self.lib, count * n * 2)
+        buf.refs = count
+        out = []
+        for p in range(count):
+            v = TensorData(shape, "f32")
+            v.store, v._buf, v._off, v._dev_valid, v._backend = "bf16", buf, p * n * 2, True, self
+            out.append(v)
+        return out
+
     def sliceQkv(self, a: TensorData):
         rows, c3 = a.shape
         d = c3 // 3
         if a.store != "bf16" or d % 2 or c3 != 3 * d:
             return super().sliceQkv(a)
+        h = self._held
+        if h is not None and a._buf is h.out_buf and a._off == h.out_off and h.layout == ffi.GEMM_NT and h.a_planes is None \
+                and (h.m, h.n) == (rows, c3) and self._takes_planes(ffi.GEMM_NT, h.m, h.n, h.k, h.lda, h.ldb, d, c_planes=(d, rows * d)):
+            # the projection is still to be launched: it writes q, k and v as three matrices itself (ah_gemm_planes)
+            self._held = None
+            q, k, v = self._plane_views(3, (rows, d))
+            self._gemm(ffi.GEMM_NT, h.a_ptr, h.b_ptr, q._buf.ptr, h.m, h.n, h.k, h.lda, h.ldb, d, in_dtype=BF16, out_dtype=BF16,
+                       planes=(d, rows * d, 0, 0))
+            if h.out_buf.refs > 1:
+                self._orphans[id(h.out_buf)] = h                # the [rows, 3d] product itself was not written: keep the recipe
+            else:
+                self._unhold(h.holds)
+            return [q, k, v]
         q, k, v = (self._new((rows, d), "f32", "bf16") for _ in range(3))
         check(self.lib.ah_slice_qkv(self._ptr(a), q._buf.ptr, k._buf.ptr, v._buf.ptr, rows, d // 2))
         return [q, k, v]
@@ -328,12 +367,44 @@ class FastHipBackend(HipBackend):
             self._unhold(h.holds)
             return
         dst = h.out_ptr if out is None else out._buf.ptr + out._off
-        self._gemm(h.layout, h.a_ptr, h.b_ptr, dst, h.m, h.n, h.k, h.lda, h.ldb, h.n, in_dtype=BF16, out_dtype=out_dtype,
-                   epilogue=epilogue, aux=aux)
+        self._run_held(h, dst, epilogue, aux, out_dtype)
         if out is not None and epilogue != ffi.EPI_GELU and h.out_buf.refs > 1:
             self._orphans[id(h.out_buf)] = h                    # the plain product was not written: keep the recipe
         else:
             self._unhold(h.holds)
+
+    def _run_held(self, h: _HeldGemm, dst: int, epilogue=ffi.EPI_NONE, aux: int = 0, out_dtype=BF16):
+        if h.a_planes is not None:
+            if epilogue == ffi.EPI_NONE and out_dtype == BF16:
+                self._gemm(h.layout, h.a_ptr, h.b_ptr, dst, h.m, h.n, h.k, h.lda, h.ldb, h.n, in_dtype=BF16, out_dtype=BF16,
+                           planes=(0, 0) + h.a_planes)
+                return
+            # an epilogue (or an f32 result) wants A as one matrix: the planes are copied side by side first
+            w, step = h.a_planes
+            whole = _Buf(self.lib, h.m * h.k * 2)
+            for p in range(h.k // w):
+                check(self.lib.ah_cat_part(h.a_ptr + p * step * 2, whole.ptr, 2, ffi.shape_arr([h.m, w // 2]), ffi.shape_arr([h.m, h.k // 2]), 1, p * w // 2))
+            self._gemm(h.layout, whole.ptr, h.b_ptr, dst, h.m, h.n, h.k, h.k, h.ldb, h.n, in_dtype=BF16, out_dtype=out_dtype,
+                       epilogue=epilogue, aux=aux)
+            whole.release()                                      # (stream-ordered: reusable only by later work)
+            return
+        self._gemm(h.layout, h.a_ptr, h.b_ptr, dst, h.m, h.n, h.k, h.lda, h.ldb, h.n, in_dtype=BF16, out_dtype=out_dtype,
+                   epilogue=epilogue, aux=aux)
+
+    def _scatter_planes(self, t: TensorData):
+        """`t` as an unwritten sum of scatterSlice results (the three parts of d(qkv), ops.ts:826-834) whose sources are equally
+        wide, cover every column and lie equally far apart: (first source, columns each, bytes apart, count, record)."""
+        if not self._scatters or t._buf is None or t._off != 0 or not t._dev_valid:
+            return None
+        h = self._scatters.get(id(t._buf))
+        if h is None or tuple(t.shape) != (h.rows, h.cols) or not 2 <= len(h.parts) <= 3:
+            return None
+        parts = sorted(h.parts, key=lambda p: p[1])
+        w, step = parts[0][2], parts[1][0] - parts[0][0]
+        if any(p[2] != w or p[1] != i * w or p[0] != parts[0][0] + i * step for i, p in enumerate(parts)) or w * len(parts) != h.cols \
+                or step <= 0 or step % 16 or parts[0][0] % 16:
+            return None
+        return parts[0][0], w, step, len(parts), h
 
     def _hold_gemm(self, layout, a: TensorData, b: TensorData, oshape, m, n, k, lda, ldb) -> TensorData:
         self._launch_held()
@@ -361,6 +432,17 @@ class FastHipBackend(HipBackend):
             raise ValueError(f"matmul shape mismatch: [{a.shape}] x [{b.shape}]")
         if K % 8:
             return super().matmul(a, b)
+        sp = self._scatter_planes(a)
+        if sp is not None and self._takes_planes(ffi.GEMM_NN, M, N, K, sp[1], N, N, a_planes=(sp[1], sp[2] // 2)):
+            # dX of the fused projection: the three gradients are read where they lie, their sum is never written
+            base, w, step, _, rec = sp
+            self._launch_held()
+            bp, bh = self._operand(b)
+            out = self._new((M, N), "f32", "bf16")
+            h = _HeldGemm(ffi.GEMM_NN, base, bp, out, M, N, K, w, N, self._hold(*rec.srcs, bh, out._buf))
+            h.a_planes = (w, step // 2)
+            self._held = h
+            return out
         return self._hold_gemm(ffi.GEMM_NN, a, b, (M, N), M, N, K, K, N)
 
     def gelu(self, a: TensorData) -> TensorData:
@@ -417,6 +499,16 @@ class FastHipBackend(HipBackend):
             raise ValueError(f"matmul shape mismatch: [{a.shape}]^T x [{b.shape}]")
         if M % 8:                                               # (the contraction runs over the rows here)
             return super().matmulTransposedA(a, b)
+        sp = self._scatter_planes(a) if self._group and M % 64 == 0 and N % 8 == 0 else None
+        if sp is not None and sp[1] % 8 == 0:
+            # dW of the fused projection: one problem of the grouped launch per gradient, each writing its rows of dW
+            bp, bh = self._operand(b)
+            out = self._new((K, N))
+            wg = _HeldWeightGrad(sp[0], bp, out, K, N, M, self._hold(*sp[4].srcs, bh, out._buf))
+            wg.planes = (sp[1], sp[2])
+            self._wgrads.append(wg)
+            self._wq_out.add(id(out._buf))
+            return out
         ap, ah = self._operand(a)
         bp, bh = self._operand(b)
         out = self._new((K, N))
@@ -438,13 +530,20 @@ class FastHipBackend(HipBackend):
         self._wq_out, self._wq_into = set(), set()
         descs = []
         for w in ws:
-            w.add_after = None
+            w.add_after, w.dst = None, None
             if w.into is None and w.out_buf.refs == 1:          # released unread
                 continue
             if w.into is not None and w.out_buf.refs > 1:       # (the queue's own hold is one reference)
                 w.add_after, w.into = w.into, None
             dst, epi = (w.out_buf.ptr + w.out_off, ffi.EPI_NONE) if w.into is None else (w.into[0].ptr + w.into[1], ffi.EPI_ACCUM)
-            descs.append(ffi.AhGemm(ffi.GEMM_TN, BF16, F32, epi, w.m, w.n, w.k, w.m, w.n, w.n, 1, 0, 0, 0, w.g_ptr, w.x_ptr, dst, 0))
+            w.dst = dst
+            if w.planes is None:
+                descs.append(ffi.AhGemm(ffi.GEMM_TN, BF16, F32, epi, w.m, w.n, w.k, w.m, w.n, w.n, 1, 0, 0, 0, w.g_ptr, w.x_ptr, dst, 0))
+            else:
+                cols, step = w.planes
+                for p in range(w.m // cols):
+                    descs.append(ffi.AhGemm(ffi.GEMM_TN, BF16, F32, epi, cols, w.n, w.k, cols, w.n, w.n, 1, 0, 0, 0, w.g_ptr + p * step, w.x_ptr,
+                                            dst + p * cols * w.n * 4, 0))
         groupable = all(d.k % 64 == 0 and d.m % 8 == 0 and d.n % 8 == 0 for d in descs)
         parts = []
         for epi in (ffi.EPI_NONE, ffi.EPI_ACCUM):
@@ -704,7 +803,17 @@ class FastHipBackend(HipBackend):
     def flashAttentionBackward(self, Q, K, V, O, dO, lse, T, scale, softCap) -> dict:
         if not (Q.store == K.store == V.store == O.store == dO.store):
             self._words(Q, K, V, O, dO)
-        return super().flashAttentionBackward(Q, K, V, O, dO, lse, T, scale, softCap)
+        if Q.store != "bf16":
+            return super().flashAttentionBackward(Q, K, V, O, dO, lse, T, scale, softCap)
+        # the three gradients one behind the other in one allocation: what consumes their scattered sum (the projection's dX
+        # and dW products) can then read them in place
+        f = self._flash_desc(Q, K, V, T, scale, softCap)
+        f.dtype = BF16
+        f.q, f.k, f.v, f.o, f.lse, f.d_o = self._ptr(Q), self._ptr(K), self._ptr(V), self._ptr(O), self._ptr(lse), self._ptr(dO)
+        dQ, dK, dV = self._plane_views(3, Q.shape)
+        f.dq, f.dk, f.dv = dQ._buf.ptr + dQ._off, dK._buf.ptr + dK._off, dV._buf.ptr + dV._off
+        check(self.lib.ah_flash_bwd(C.byref(f)))
+        return {"dQ": dQ, "dK": dK, "dV": dV}
 
     def attentionQkvBackward(self, qkv, out, dOut, lse, Bt, T, nHead, scale, softCap) -> TensorData:
         if not (qkv.store == out.store == dOut.store):
@@ -733,7 +842,7 @@ class FastHipBackend(HipBackend):
             key = addresses()
             if None not in key and len(set(key)) == len(key):
                 ws, parts = self._take_weight_grads()
-                covered = {d.c: d.m * d.n for _, part, grouped in parts if grouped for d in part}
+                covered = {w.dst: w.m * w.n for w in ws if w.dst is not None} if all(grouped for _, _, grouped in parts) else {}
                 listed = {k: t.size for k, t in zip(key, tensors)}
                 if covered and all(grouped for _, _, grouped in parts) and all(listed.get(a) == n for a, n in covered.items()) \
                         and not any(w.add_after is not None for w in ws):
@@ -785,7 +894,7 @@ class FastHipBackend(HipBackend):
             # would be computed later from this shadow, which the update rewrites in place: compute it from the old weights now
             for key in [k for k, h in self._orphans.items() if any(b is sh for b in h.holds)]:
                 h = self._orphans.pop(key)
-                self._gemm(h.layout, h.a_ptr, h.b_ptr, h.out_ptr, h.m, h.n, h.k, h.lda, h.ldb, h.n, in_dtype=BF16, out_dtype=BF16)
+                self._run_held(h, h.out_ptr)
                 self._unhold(h.holds)
         self._adam_q.append((*ptrs, sh.ptr if sh is not None else 0, params.size, weightDecay))
         for b in (params._buf, grads._buf, m._buf, v._buf) + ((sh,) if sh is not None else ()):

@@ -4,7 +4,9 @@ ctx 1024, batch 16; forward + backward + AdamW with gradient clipping) on one MI
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--mode fast|backend|parity] [--no-cpu] [--no-extra] [--workload gpt2-small|gpt-350m]
 
-`--mode fast` (default) is the hand-scheduled step (FusedTrainer); `--mode backend` runs the generic tape-driven Trainer -- one
+`--mode fast` (default) is the hand-scheduled step (FusedTrainer) of the function an unchanged gpt.ts computes on a backend
+with flashAttention (`--attention reference-flash`, gpt.ts:247-254: q, k, v re-read as [B H, T, D] slabs without a head
+transpose; `--attention heads` = multi-head attention on the columns of the projection instead); `--mode backend` runs the generic tape-driven Trainer -- one
 `Backend` call per op, host-side loss / norm / clip, exactly the call structure of the reference trainer -- on FastHipBackend
 (bf16 storage, fused epilogues and grouped weight gradients behind the interface, steps replayed as recorded hipGraph
 segments); `--mode parity` runs the same Trainer on the fp32 kernels.
@@ -14,8 +16,8 @@ The default workload is the one the metric is quoted on; `--workload gpt-350m` r
 
 After the headline measurement the default invocation also times, each in a child process of its own once the parent has
 released its device memory, the path the reference's trainer would take -- `--mode backend` with the model's own attention
-wiring (`--attention reference-flash`, gpt.ts:247-254) and with true multi-head attention (`heads`) -- and the 350M-shape
-workload, and adds them to the line as `backend_mode` and `workload_350m` (`--no-extra` leaves them out).
+wiring and with multi-head attention (`heads`) --, the 350M-shape workload and the headline step with `heads`, and adds them
+to the line as `backend_mode`, `workload_350m` and `fused_step_heads_attention` (`--no-extra` leaves them out).
 
 Prints ONE JSON line.  `value` is tokens/s with parameters, optimizer state and the token batch already resident in
 HBM; the scatter-add index of the token embedding's gradient (a sort of the batch's ids) is built inside the timed steps.  `roofline` is for the dominant kernel, the MFMA GEMM instantiation that does the most arithmetic in a step (which is
@@ -101,7 +103,7 @@ def main():
     ap.add_argument("--norm-over-arena", action="store_true", help="fast mode, for comparison: take the gradient norm by reading the whole gradient "
                     "arena again instead of summing the weight gradients' squares in the epilogue of the launch that stores them")
     ap.add_argument("--stream", choices=["f32", "bf16"], default="bf16", help="fast mode: storage type of the residual stream and its gradient")
-    ap.add_argument("--attention", choices=["heads", "reference-flash", "unfused"], default="heads",
+    ap.add_argument("--attention", choices=["heads", "reference-flash", "unfused"], default="reference-flash",
                     help="which attention branch of the model runs (reference-flash = what the reference's flash branch computes, "
                          "gpt.ts:232-253; heads = multi-head attention; unfused = its CPU branch, backend / parity mode only)")
     ap.add_argument("--no-cpu", action="store_true")
@@ -287,13 +289,16 @@ def extra_runs(args) -> dict:
             return {"error": repr(e)[:300]}
     ref, heads, big = (child("--mode", "backend", "--attention", "reference-flash"), child("--mode", "backend", "--attention", "heads"),
                        child("--workload", "gpt-350m"))
-    res = {"backend_mode": {"ms_per_step": heads.get("ms_per_step"), "ms_per_step_reference_flash": ref.get("ms_per_step"),
+    fused_heads = child("--attention", "heads")
+    res = {"fused_step_heads_attention": {"ms_per_step": fused_heads.get("ms_per_step"),
+                                          "what": "the headline step with multi-head attention on the columns of the projection instead of the reference's slabs"},
+           "backend_mode": {"ms_per_step": heads.get("ms_per_step"), "ms_per_step_reference_flash": ref.get("ms_per_step"),
                             "step_plans": (heads.get("config") or {}).get("step_plans"),
                             "step_plans_reference_flash": (ref.get("config") or {}).get("step_plans"),
                             "what": "generic tape-driven Trainer, one Backend call per op, on FastHipBackend with step plans; same model, batches and steps"},
            "workload_350m": {"ms_per_step": big.get("ms_per_step"), "tokens_per_s": big.get("value"), "mfu": big.get("mfu_vs_bf16_dense_peak"),
                              "what": (big.get("config") or {}).get("workload")}}
-    for k, v in (("backend_mode", heads), ("backend_mode", ref), ("workload_350m", big)):
+    for k, v in (("backend_mode", heads), ("backend_mode", ref), ("workload_350m", big), ("fused_step_heads_attention", fused_heads)):
         if "error" in v:
             res[k].setdefault("errors", []).append(v["error"])
     return res

@@ -203,7 +203,7 @@ def test_reference_flash_branch_on_the_fast_backend_tracks_its_oracle_over_50_st
             if n.endswith("attn.wqkv"):
                 v.data.data = v.data.data * 8
     FB.enableStepGraphs(graphs)
-    before = FB.stepStats()
+    before, planes_before = FB.stepStats(), FB.planeProducts
     losses = []
     for s in range(steps):
         r = tr.step([syntheticBatch(50 + s, 4, 64, 256)])
@@ -212,6 +212,9 @@ def test_reference_flash_branch_on_the_fast_backend_tracks_its_oracle_over_50_st
         assert abs(r.gradNorm - o.gradNorm) <= 5e-2 * o.gradNorm and abs(r.lr - o.lr) < 1e-15, (s, r.gradNorm, o.gradNorm)
         losses.append((r.loss, r.gradNorm))
     FB.enableStepGraphs(False)
+    # at this shape the fused projection writes q, k, v in place of sliceQkv's copies and its backward reads dq, dk, dv where
+    # they lie (ah_gemm_planes): two such products per layer and step
+    assert FB.planeProducts - planes_before == 2 * cfg["nLayer"] * steps, (FB.planeProducts, planes_before)
     fn = test_reference_flash_branch_on_the_fast_backend_tracks_its_oracle_over_50_steps
     if graphs:
         assert FB.stepStats()["replayed"] - before["replayed"] >= steps - 4, (before, FB.stepStats(), FB.lastStepNote)
@@ -433,6 +436,72 @@ def test_scattered_column_blocks_are_merged_before_they_are_written(FB):
     for t in (a, b, acc, s, s2):
         FB.releaseGpuTensor(t)
     assert not FB._scatters
+
+
+def test_the_fused_projection_and_its_backward_take_their_operands_in_planes(FB):
+    """sliceQkv of a projection that has not been launched yet makes the projection write q, k, v itself, and the backward
+    products of the projection read dq, dk, dv where flashAttentionBackward leaves them instead of a written sum of three
+    scatterSlice results (ops.ts:816-858, 197-234).  Same numbers as the route around copies, to an ulp of the bf16 results
+    (at this size the ordinary route runs another kernel) and to f32 summation order for the weight gradient."""
+    rs = np.random.RandomState(17)
+    rows, d = 512, 128
+    x, w = _bf16(rs.randn(rows, d)), _bf16(rs.randn(3 * d, d) * 0.1)
+    X, W = FB.castStore(_td(x), "bf16"), _td(w)
+    n0 = FB.planeProducts
+    # forward
+    plain = FB.matmulTransposed(X, W).data.reshape(rows, 3 * d).copy()                 # read at once: written as one matrix
+    held = FB.matmulTransposed(X, W)
+    q, k, v = FB.sliceQkv(held)
+    assert FB.planeProducts == n0 + 1 and q._buf is k._buf is v._buf
+    for i, t in enumerate((q, k, v)):
+        assert t.store == "bf16"
+        _close(t.data.reshape(rows, d), plain[:, i * d:(i + 1) * d], f"plane {i}", 4e-3)         # (another kernel at this size: an ulp of bf16 here and there)
+        _close(t.data.reshape(rows, d), _bf16(x.astype(np.float64) @ w[i * d:(i + 1) * d].astype(np.float64).T), f"plane {i} vs f64", 4e-3)
+    assert np.array_equal(held.data.reshape(rows, 3 * d), plain)                        # the product itself, asked for after all
+    # backward: gradients as flashAttentionBackward allocates them (one behind the other), scattered and summed by the tape
+    gs = [_bf16(rs.randn(rows, d)) for _ in range(3)]
+
+    def summed(planes: bool):
+        if planes:
+            ts = FB._plane_views(3, (rows, d))
+            for t, g in zip(ts, gs):
+                bits = (g.view(np.uint32) >> 16).astype(np.uint16)
+                ffi.check(FB.lib.ah_upload(t._buf.ptr + t._off, bits.ctypes.data_as(C.c_void_p), bits.nbytes))
+        else:
+            ts = [FB.castStore(_td(g), "bf16") for g in gs]
+        sc = [FB.scatterSlice(t, (rows, 3 * d), [0, i * d], [rows, (i + 1) * d]) for i, t in enumerate(ts)]
+        acc = FB.clone(sc[2])
+        for i in (1, 0):
+            FB.addInplace(acc, sc[i])
+        for t in sc + ts:
+            FB.releaseGpuTensor(t)
+        return acc
+    import ctypes as C
+    from alpha2_amd import _ffi as ffi
+    res = FB.castStore(_td(_bf16(rs.randn(rows, d))), "bf16")
+    outs = {}
+    for planes in (False, True):
+        n1 = FB.planeProducts
+        g = summed(planes)
+        dx = FB.matmul(g, W)
+        dw = FB.matmulTransposedA(g, X)
+        other = FB.matmulTransposedA(FB.castStore(_td(gs[0]), "bf16"), X)               # a second queued product: the launch is grouped
+        dxv, dwv, ov = dx.data.reshape(rows, d).copy(), dw.data.reshape(3 * d, d).copy(), other.data.copy()
+        assert FB.planeProducts - n1 == (1 if planes else 0)
+        assert (id(g._buf) in FB._scatters) == planes                                    # with planes the sum is still unwritten
+        with_res = FB.add(res, FB.matmul(g, W)).data.reshape(rows, d).copy()            # an epilogue wants the operand whole
+        gv = g.data.reshape(rows, 3 * d).copy()
+        outs[planes] = (dxv, dwv, ov, with_res, gv)
+        for t in (g, dx, dw, other):
+            FB.releaseGpuTensor(t)
+        assert not FB._scatters
+    _close(outs[True][0], outs[False][0], "dX from planes", 4e-3)
+    _close(outs[True][3], outs[False][3], "dX + residual", 4e-3)
+    assert np.array_equal(outs[True][4], np.concatenate(gs, axis=1)) and np.array_equal(outs[False][4], outs[True][4])
+    assert np.array_equal(outs[True][2], outs[False][2])
+    _close(outs[True][1], outs[False][1], "dW from planes", 1e-6)
+    _close(outs[True][1], np.concatenate(gs, axis=1).astype(np.float64).T @ x.astype(np.float64), "dW", 1e-5)
+    _close(outs[True][0], _bf16(np.concatenate(gs, axis=1).astype(np.float64) @ w.astype(np.float64)), "dX", 4e-3)
 
 
 def test_cross_entropy_is_held_until_its_backward_is_asked_for(FB):
