@@ -99,6 +99,7 @@ SIGNATURES = {
     "ah_silu_mul": [u64, u64, u64, u64], "ah_silu_mul_bwd": [u64, u64, u64, u64, u64, u64],
     "ah_residual_dropout_add": [u64, u64, u64, u64, u64],
     "ah_dropout_mask": [u64, u64, i32, i32, C.c_double],
+    "ah_dropout_apply": [u64, i32, u64, u64, i32, u64, u64, i32, C.c_double],
     "ah_masked_fill": [u64, u64, u64, u64, u64, f32], "ah_causal_mask": [u64, i64],
     "ah_cast": [u64, i32, u64, i32, u64], "ah_check_finite": [u64, u64, u64],
     "ah_transpose": [u64, u64, i32, p_i64, i32, i32],

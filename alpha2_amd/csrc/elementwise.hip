@@ -391,6 +391,52 @@ __global__ void k_dropout_mask(float *__restrict__ out, uint64_t n, int32_t seed
     out[i] = ((double)h * (1.0 / 4294967296.0) > p) ? keep : 0.f;
   }
 }
+// out = (residual or 0) + x * mask, the mask of k_dropout_mask made on the fly from a seed that lives in device memory: four
+// consecutive elements per thread (8- or 16-byte accesses), the tail one at a time.
+__device__ __forceinline__ float drop_keep(double base, uint64_t i, double p, float keep) {
+#pragma clang fp contract(off)
+  double sum = base + (double)i * 2246822519.0;
+  uint32_t h = (uint32_t)(int64_t)sum;
+  h = (h ^ (h >> 16)) * 0x85ebca6bu;
+  h = (h ^ (h >> 13)) * 0xc2b2ae35u;
+  h = h ^ (h >> 16);
+  return ((double)h * (1.0 / 4294967296.0) > p) ? keep : 0.f;
+}
+__device__ __forceinline__ void ld4(const float *p, uint64_t i, float (&v)[4]) { float4 t = *reinterpret_cast<const float4 *>(p + i); v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w; }
+__device__ __forceinline__ void ld4(const uint16_t *p, uint64_t i, float (&v)[4]) {
+  uint2 t = *reinterpret_cast<const uint2 *>(p + i);
+  v[0] = bf16_bits_to_f32(t.x & 0xffffu); v[1] = bf16_bits_to_f32(t.x >> 16); v[2] = bf16_bits_to_f32(t.y & 0xffffu); v[3] = bf16_bits_to_f32(t.y >> 16);
+}
+__device__ __forceinline__ void st4(float *p, uint64_t i, const float (&v)[4]) { *reinterpret_cast<float4 *>(p + i) = make_float4(v[0], v[1], v[2], v[3]); }
+__device__ __forceinline__ void st4(uint16_t *p, uint64_t i, const float (&v)[4]) { *reinterpret_cast<uint2 *>(p + i) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])); }
+__device__ __forceinline__ float ld1(const float *p, uint64_t i) { return p[i]; }
+__device__ __forceinline__ float ld1(const uint16_t *p, uint64_t i) { return bf16_bits_to_f32(p[i]); }
+__device__ __forceinline__ void st1(float *p, uint64_t i, float v) { p[i] = v; }
+__device__ __forceinline__ void st1(uint16_t *p, uint64_t i, float v) { p[i] = f32_to_bf16_bits(v); }
+template <class X, class O>
+__global__ void k_dropout_apply(const X *__restrict__ x, const O *__restrict__ residual, O *__restrict__ out, uint64_t n, const int32_t *__restrict__ seed,
+                                int32_t counter, double p, float keep, int vec) {
+#pragma clang fp contract(off)
+  const uint64_t tid = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x, stride = (uint64_t)gridDim.x * blockDim.x;
+  const double base = (double)seed[0] + (double)counter * 2654435761.0;
+  const uint64_t n4 = vec ? n >> 2 : 0;
+  for (uint64_t q = tid; q < n4; q += stride) {
+    const uint64_t i = q << 2;
+    float v[4], r[4] = {0.f, 0.f, 0.f, 0.f};
+    ld4(x, i, v);
+    if (residual) ld4(residual, i, r);
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      const float m = v[e] * drop_keep(base, i + e, p, keep);
+      r[e] = residual ? r[e] + m : m;               // (no residual: the product itself, the sign of a zero included)
+    }
+    st4(out, i, r);
+  }
+  for (uint64_t i = (n4 << 2) + tid; i < n; i += stride) {
+    const float m = ld1(x, i) * drop_keep(base, i, p, keep);
+    st1(out, i, residual ? ld1(residual, i) + m : m);
+  }
+}
 __global__ void k_masked_fill(const float *__restrict__ a, const float *__restrict__ mask, float *__restrict__ out,
                               uint64_t n, uint64_t mask_n, float value) {
   uint64_t tid = blockIdx.x * (uint64_t)blockDim.x + threadIdx.x, stride = (uint64_t)gridDim.x * blockDim.x;
@@ -669,6 +715,31 @@ int32_t ah_dropout_mask(ah_ptr out, uint64_t n, int32_t seed, int32_t counter, d
   AH_ARG(n <= (1ull << 32), "ah_dropout_mask: at most 2^32 elements (the hash sum must stay below 2^63)");
   ah::launch_kernel(k_dropout_mask, dim3(grid_for(n)), dim3(TPB), 0, dp<float>(out), n, seed, counter, p,
                      (float)(1.0 / (1.0 - p)));
+  AH_LAUNCH_CHECK();
+  return AH_OK;
+}
+int32_t ah_dropout_apply(ah_ptr x, int32_t x_dtype, ah_ptr residual, ah_ptr out, int32_t out_dtype, uint64_t n, ah_ptr seed_i32,
+                         int32_t counter, double p) {
+  AH_REQUIRE_READY();
+  if (n == 0) return AH_OK;
+  AH_ARG(x != 0 && out != 0 && seed_i32 != 0, "ah_dropout_apply: null operand");
+  AH_ARG((x_dtype == AH_F32 || x_dtype == AH_BF16) && (out_dtype == AH_F32 || out_dtype == AH_BF16), "ah_dropout_apply: f32 or bf16 operands");
+  AH_ARG(p >= 0.0 && p < 1.0, "ah_dropout_apply: p must be in [0,1)");
+  AH_ARG(n <= (1ull << 32), "ah_dropout_apply: at most 2^32 elements (the hash sum must stay below 2^63)");
+  const int xs = x_dtype == AH_F32 ? 4 : 2, os = out_dtype == AH_F32 ? 4 : 2;
+  AH_ARG(x % xs == 0 && out % os == 0 && residual % os == 0 && seed_i32 % 4 == 0, "ah_dropout_apply: misaligned operand");
+  const int vec = x % (4 * xs) == 0 && out % (4 * os) == 0 && residual % (4 * os) == 0;
+  const float keep = (float)(1.0 / (1.0 - p));
+  const dim3 grid(grid_for(vec ? n / 4 + 1 : n)), blk(TPB);
+  const int32_t *seed = dp<const int32_t>(seed_i32);
+  if (x_dtype == AH_F32 && out_dtype == AH_F32)
+    ah::launch_kernel(k_dropout_apply<float, float>, grid, blk, 0, dp<const float>(x), dp<const float>(residual), dp<float>(out), n, seed, counter, p, keep, vec);
+  else if (x_dtype == AH_F32)
+    ah::launch_kernel(k_dropout_apply<float, uint16_t>, grid, blk, 0, dp<const float>(x), dp<const uint16_t>(residual), dp<uint16_t>(out), n, seed, counter, p, keep, vec);
+  else if (out_dtype == AH_F32)
+    ah::launch_kernel(k_dropout_apply<uint16_t, float>, grid, blk, 0, dp<const uint16_t>(x), dp<const float>(residual), dp<float>(out), n, seed, counter, p, keep, vec);
+  else
+    ah::launch_kernel(k_dropout_apply<uint16_t, uint16_t>, grid, blk, 0, dp<const uint16_t>(x), dp<const uint16_t>(residual), dp<uint16_t>(out), n, seed, counter, p, keep, vec);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }

@@ -6,7 +6,12 @@ replayed every step.
 Differences from the op-by-op path are layout and fusion only; the arithmetic is the same function:
   * tok+pos embedding and their add are one kernel; the residual adds are GEMM epilogues; GELU (+ saved
     pre-activation) and its derivative are GEMM epilogues; attention reads Q, K, V in place out of the [BT, 3C]
-    projection and writes merged heads;
+    projection and writes merged heads (attention="heads"), or -- attention="reference-flash", the function gpt.ts:247-254
+    computes on a backend with flashAttention -- the projection writes q, k, v as three [BT, C] matrices that are read as
+    [B H, T, D] slabs, and its backward reads the three gradients where the attention kernel leaves them;
+  * dropout (reference-flash wiring only): the two residualDropoutAdd of a block become one pass each over the projection
+    with the mask made on the fly, and so do the two mask multiplies of their backward; the seed of a step's masks is read
+    from device memory, so the captured graph draws new masks at every replay;
   * every activation is bf16, by default the residual stream and the gradient flowing back along it too (stream="f32"
     keeps those two in f32: 3 % slower, losses equal to 1e-4 relative);
   * parameters, gradients and Adam moments each live in ONE arena ordered [decayed | not decayed], so the gradient
@@ -37,6 +42,11 @@ def _align(n: int, a: int = 64) -> int:
     return (n + a - 1) // a * a
 
 
+def _i32(x: int) -> int:
+    x &= 0xFFFFFFFF
+    return x - (1 << 32) if x >> 31 else x
+
+
 @dataclass
 class StepStats:
     loss: float
@@ -55,9 +65,15 @@ class FusedTrainer:
         # inside every step, on the side stream beside the forward pass, instead of once when a batch is stored: what a loop
         # pays that feeds a new batch every step
         self.index_in_step = bool(index_in_step)
-        if self.act not in ("gelu", "silu", "relu", "swiglu", "universal", "kan_spline") or cfg.dropout != 0:
-            raise ValueError("FusedTrainer schedules the gelu / silu / relu / swiglu / universal / kan_spline blocks without dropout; "
-                             "use train.Trainer for composed activations and dropout")
+        if self.act not in ("gelu", "silu", "relu", "swiglu", "universal", "kan_spline"):
+            raise ValueError("FusedTrainer schedules the gelu / silu / relu / swiglu / universal / kan_spline blocks; "
+                             "use train.Trainer for composed activations")
+        # Dropout: the two residualDropoutAdd of a block (gpt.ts:281,332), the only places the model's flash branch drops
+        # anything.  The multi-head wiring stands for the CPU branch, which also drops attention weights (gpt.ts:276): the fused
+        # attention kernel has no such thing, so dropout goes with the reference's own wiring only.
+        self.drop = float(cfg.dropout)
+        if not 0.0 <= self.drop < 1.0 or (self.drop > 0 and cfg.attention != "reference-flash"):
+            raise ValueError("FusedTrainer applies dropout (0 <= p < 1) with attention='reference-flash' only; use train.Trainer otherwise")
         self.B, self.lib, self.cfg, self.tc = backend, backend.lib, cfg, tc
         self.batch, self.T, self.accum, self.use_graph = batch, cfg.blockSize, accum, use_graph
         self.C, self.H, self.L, self.V, self.F = cfg.nEmbd, cfg.nHead, cfg.nLayer, cfg.vocabSize, ffn_dim(cfg)
@@ -169,6 +185,14 @@ class FusedTrainer:
         self.dh = [a(BT * self.Fin * 2) for _ in range(self.L)]
         self.dqkv = [a(BT * 3 * Cc * 2) for _ in range(self.L)]
         self.dxb0 = a(BT * Cc * 2)                # grad of the embedding output in bf16 (written by the last LayerNorm backward, unused)
+        if self.drop > 0:
+            # a projection before its mask (one at a time), the masked output gradients of the two projections per layer (the
+            # operands of their dX and dW products; the unmasked ones stay the residual stream's gradient), and the seed of every
+            # micro-step's masks, which the host writes before each step
+            self.proj = a(BT * Cc * 2)
+            self.dproj_fc2 = [a(BT * Cc * 2) for _ in range(self.L)]
+            self.dproj_wo = [a(BT * Cc * 2) for _ in range(self.L)]
+            self.seed_dev = a(4 * self.accum)
         self.loss, self.sumsq, self.clip = a(4), a(4), a(16)         # clip: coefficient (NaN = skip), norm, skipped flag
         self.loss_micro = a(4)
         self.hyper = a(ffi.C.sizeof(ffi.AhAdamW))
@@ -199,8 +223,9 @@ class FusedTrainer:
 
         def layer(l):
             pre = f"layer.{l}."
-            d = [desc(self.dy_fc2[l], self.hact[l], pre + self.w2, Cc, Fd), desc(self.dh[l], self.ln2[l], pre + self.w1, self.Fin, Cc),
-                 desc(self.dy_wo[l], self.att[l], pre + "attn.wo", Cc, Cc)]
+            dyf, dyw = (self.dproj_fc2[l], self.dproj_wo[l]) if self.drop > 0 else (self.dy_fc2[l], self.dy_wo[l])
+            d = [desc(dyf, self.hact[l], pre + self.w2, Cc, Fd), desc(self.dh[l], self.ln2[l], pre + self.w1, self.Fin, Cc),
+                 desc(dyw, self.att[l], pre + "attn.wo", Cc, Cc)]
             if self.slabs:      # dq, dk, dv lie apart as [BT, C] matrices: rows [p C, (p + 1) C) of the [3C, C] gradient each
                 return d + [desc(self.dqkv[l] + p * BT * Cc * 2, self.ln1[l], pre + "attn.wqkv", Cc, Cc, p * Cc) for p in range(3)]
             return d + [desc(self.dqkv[l], self.ln1[l], pre + "attn.wqkv", 3 * Cc, Cc)]
@@ -313,6 +338,11 @@ class FusedTrainer:
         self._timed.append({"kind": "gemm", "kernel": kernel, "nsplit": nsplit, "layout": layout, "m": m, "n": n, "k": k,
                             "flops": 2.0 * m * n * k, "e0": e0, "e1": e1})
 
+    def _dropout(self, x: int, residual: int, out: int, out_dtype: int, micro: int, counter: int):
+        """out = residual + x * mask (residual 0: the mask multiply of the backward pass); x bf16, mask number `counter` of the
+        micro-step (ops.ts:25-82), its seed read from device memory when the kernel runs."""
+        check(self.lib.ah_dropout_apply(x, BF16, residual, out, out_dtype, self.BT * self.C, self.seed_dev + 4 * micro, counter, self.drop))
+
     def _flash(self, l: int, bwd: bool):
         Cc, T, D = self.C, self.T, self.D
         f = ffi.AhFlash()
@@ -361,7 +391,11 @@ class FusedTrainer:
             else:
                 self._gemm(NT, self.ln1[l], self.p(pre + "attn.wqkv", True), self.qkv[l], BT, 3 * Cc, Cc, Cc, Cc, 3 * Cc)
             self._flash(l, False)
-            self._gemm(NT, self.att[l], self.p(pre + "attn.wo", True), self.xmid[l], BT, Cc, Cc, Cc, Cc, Cc, SD, ffi.EPI_RESIDUAL, self.x[l])
+            if self.drop > 0:
+                self._gemm(NT, self.att[l], self.p(pre + "attn.wo", True), self.proj, BT, Cc, Cc, Cc, Cc, Cc)
+                self._dropout(self.proj, self.x[l], self.xmid[l], SD, micro, 2 * l)
+            else:
+                self._gemm(NT, self.att[l], self.p(pre + "attn.wo", True), self.xmid[l], BT, Cc, Cc, Cc, Cc, Cc, SD, ffi.EPI_RESIDUAL, self.x[l])
             check(lib.ah_layernorm(self.xmid[l], self.p(pre + "ln2.weight"), self.p(pre + "ln2.bias"), self.ln2[l], BT, Cc, 1e-5, BF16, SD))
             if self.act == "gelu":
                 self._gemm(NT, self.ln2[l], self.p(pre + "mlp.fc1", True), self.hact[l], BT, Fd, Cc, Cc, Cc, Fd, BF16, ffi.EPI_GELU_GRAD, self.hgrad[l])
@@ -372,7 +406,11 @@ class FusedTrainer:
                     check(lib.ah_swiglu(BF16, self.hpre[l], self.hact[l], BT, Fd))
                 else:
                     check(lib.ah_channel_act(BF16, self.hpre[l], self._coef_handles(l, self.p), self._act_mask, self.hact[l], BT, Fd))
-            self._gemm(NT, self.hact[l], self.p(pre + self.w2, True), self.x[l + 1], BT, Cc, Fd, Fd, Fd, Cc, SD, ffi.EPI_RESIDUAL, self.xmid[l])
+            if self.drop > 0:
+                self._gemm(NT, self.hact[l], self.p(pre + self.w2, True), self.proj, BT, Cc, Fd, Fd, Fd, Cc)
+                self._dropout(self.proj, self.xmid[l], self.x[l + 1], SD, micro, 2 * l + 1)
+            else:
+                self._gemm(NT, self.hact[l], self.p(pre + self.w2, True), self.x[l + 1], BT, Cc, Fd, Fd, Fd, Cc, SD, ffi.EPI_RESIDUAL, self.xmid[l])
         check(lib.ah_layernorm(self.x[L], self.p("lnF.weight"), self.p("lnF.bias"), self.lnf, BT, Cc, 1e-5, BF16, SD))
         self._gemm(NT, self.lnf, self.p("lmHead", True), self.logits, BT, V, Cc, Cc, Cc, V)
         # loss and dlogits (in place) from one read of the logits
@@ -392,10 +430,14 @@ class FusedTrainer:
         for l in reversed(range(L)):
             pre = f"layer.{l}."
             # MLP: x_out = x_mid + fc2(gelu(fc1(ln2(x_mid))))
+            dyf = self.dy_fc2[l]
+            if self.drop > 0:                      # the projection's own gradient is the stream's times the mask it was dropped with
+                dyf = self.dproj_fc2[l]
+                self._dropout(self.dy_fc2[l], 0, dyf, BF16, micro, 2 * l + 1)
             if self.act == "gelu":
-                self._gemm(NN, self.dy_fc2[l], self.p(pre + "mlp.fc2", True), self.dh[l], BT, Fd, Cc, Cc, Fd, Fd, BF16, ffi.EPI_MUL_AUX, self.hgrad[l])
+                self._gemm(NN, dyf, self.p(pre + "mlp.fc2", True), self.dh[l], BT, Fd, Cc, Cc, Fd, Fd, BF16, ffi.EPI_MUL_AUX, self.hgrad[l])
             else:
-                self._gemm(NN, self.dy_fc2[l], self.p(pre + self.w2, True), self.dact, BT, Fd, Cc, Cc, Fd, Fd)
+                self._gemm(NN, dyf, self.p(pre + self.w2, True), self.dact, BT, Fd, Cc, Cc, Fd, Fd)
                 if self.act == "swiglu":
                     check(lib.ah_swiglu_bwd(BF16, self.hpre[l], self.dact, self.dh[l], BT, Fd))
                 else:
@@ -406,7 +448,11 @@ class FusedTrainer:
                                                 self.dx[cur ^ 1] if f32s else 0, self.dy_wo[l], self._ln_part[pre + "ln2"], BT, Cc, 1e-5, SD))
             cur ^= f32s
             # attention: x_mid = x_in + wo(attn(wqkv(ln1(x_in))))
-            self._gemm(NN, self.dy_wo[l], self.p(pre + "attn.wo", True), self.datt, BT, Cc, Cc, Cc, Cc, Cc)
+            dyw = self.dy_wo[l]
+            if self.drop > 0:
+                dyw = self.dproj_wo[l]
+                self._dropout(self.dy_wo[l], 0, dyw, BF16, micro, 2 * l)
+            self._gemm(NN, dyw, self.p(pre + "attn.wo", True), self.datt, BT, Cc, Cc, Cc, Cc, Cc)
             self._flash(l, True)
             if self.slabs:
                 self._gemm(NN, self.dqkv[l], self.p(pre + "attn.wqkv", True), self.dlnb, BT, Cc, 3 * Cc, Cc, Cc, Cc, a_planes=(Cc, BT * Cc))
@@ -525,6 +571,9 @@ class FusedTrainer:
         lr = lrAt(self.tc, self.stepIdx)
         v = C.c_float(lr)
         check(self.lib.ah_upload(self.hyper, C.byref(v), 4))
+        if self.drop > 0:                          # the masks of this step's micro-steps (trainer.ts:1169,1202), as int32 like `seed | 0`
+            seeds = (C.c_int32 * self.accum)(*[_i32(self.tc.seed + self.stepIdx * 1000 + m) for m in range(self.accum)])
+            check(self.lib.ah_upload(self.seed_dev, seeds, 4 * self.accum))
         return lr
 
     def step(self, batch_index=None) -> int:

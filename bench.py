@@ -289,7 +289,7 @@ def extra_runs(args) -> dict:
             return {"error": repr(e)[:300]}
     ref, heads, big = (child("--mode", "backend", "--attention", "reference-flash"), child("--mode", "backend", "--attention", "heads"),
                        child("--workload", "gpt-350m"))
-    fused_heads = child("--attention", "heads")
+    fused_heads, big_heads = child("--attention", "heads"), child("--workload", "gpt-350m", "--attention", "heads")
     res = {"fused_step_heads_attention": {"ms_per_step": fused_heads.get("ms_per_step"),
                                           "what": "the headline step with multi-head attention on the columns of the projection instead of the reference's slabs"},
            "backend_mode": {"ms_per_step": heads.get("ms_per_step"), "ms_per_step_reference_flash": ref.get("ms_per_step"),
@@ -297,8 +297,10 @@ def extra_runs(args) -> dict:
                             "step_plans_reference_flash": (ref.get("config") or {}).get("step_plans"),
                             "what": "generic tape-driven Trainer, one Backend call per op, on FastHipBackend with step plans; same model, batches and steps"},
            "workload_350m": {"ms_per_step": big.get("ms_per_step"), "tokens_per_s": big.get("value"), "mfu": big.get("mfu_vs_bf16_dense_peak"),
+                             "ms_per_step_heads_attention": big_heads.get("ms_per_step"),
                              "what": (big.get("config") or {}).get("workload")}}
-    for k, v in (("backend_mode", heads), ("backend_mode", ref), ("workload_350m", big), ("fused_step_heads_attention", fused_heads)):
+    for k, v in (("backend_mode", heads), ("backend_mode", ref), ("workload_350m", big), ("workload_350m", big_heads),
+                 ("fused_step_heads_attention", fused_heads)):
         if "error" in v:
             res[k].setdefault("errors", []).append(v["error"])
     return res

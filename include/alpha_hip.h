@@ -205,6 +205,13 @@ int32_t ah_residual_dropout_add(ah_ptr residual, ah_ptr projected, ah_ptr mask, 
  * reference's CPU path, DropoutRng.hash (packages/autograd/src/ops.ts:74-81), reproduced bit for bit for every index: its
  * first line is evaluated in doubles before the cut to 32 bits.  n <= 2^32. */
 int32_t ah_dropout_mask(ah_ptr out, uint64_t n, int32_t seed, int32_t counter, double p);
+/* Backend.residualDropoutAdd and the mask multiply of its backward (ops.ts:616-686) with the mask of ah_dropout_mask made on
+ * the fly instead of stored: out[i] = (residual ? residual[i] : 0) + x[i] * mask(seed, counter, p)[i].  The seed is read from
+ * device memory (one int32) when the kernel runs, so a captured step draws new masks at every replay: the host writes the
+ * step's seed there before it launches the step (trainer.ts:1169,1202: seed + 1000 step + micro-step; counter = the mask's
+ * place in the forward pass, ops.ts:25-82).  x is f32 or bf16; residual and out share out_dtype (f32 or bf16). */
+int32_t ah_dropout_apply(ah_ptr x, int32_t x_dtype, ah_ptr residual, ah_ptr out, int32_t out_dtype, uint64_t n, ah_ptr seed_i32,
+                         int32_t counter, double p);
 /* Backend.maskedFill with the mask tiled by i % mask_n (cpu_ref.ts:891-911) */
 int32_t ah_masked_fill(ah_ptr a, ah_ptr mask, ah_ptr out, uint64_t n, uint64_t mask_n, float value);
 /* Backend.causalMask (cpu_ref.ts:880-889) */

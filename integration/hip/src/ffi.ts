@@ -41,6 +41,7 @@ export const lib = dlopen(process.env.ALPHA_HIP_LIB ?? "libalpha_hip.so", {
   ah_download:                     { args: [ptr, u64, u64], returns: i32 },
   ah_download_begin:               { args: [u64, u64, ptr], returns: i32 },
   ah_download_end:                 { args: [u64, ptr, u64], returns: i32 },
+  ah_dropout_apply:                { args: [u64, i32, u64, u64, i32, u64, u64, i32, f64], returns: i32 },
   ah_dropout_mask:                 { args: [u64, u64, i32, i32, f64], returns: i32 },
   ah_embedding:                    { args: [u64, u64, u64, i64, i64, i64, i32], returns: i32 },
   ah_embedding_bwd:                { args: [u64, u64, u64, i64, i64, i64, i32], returns: i32 },

@@ -93,6 +93,65 @@ def test_fused_loss_parity_over_steps_graph_replay(B, attention):
     ft.close(), eager.close()
 
 
+@pytest.mark.parametrize("accum", [1, 2])
+def test_fused_step_with_dropout_matches_oracle(B, accum):
+    """dropout 0.25 in the two residualDropoutAdd of every block (gpt.ts:281,332) on the reference's flash-branch wiring: masks
+    from DropoutRng's counter hash (ops.ts:25-82), reseeded per step and micro-step (trainer.ts:1169,1202), made on the fly from
+    a seed in device memory, so a replayed graph draws new masks every step.  Against the oracle: gradients of the first step,
+    then the loss of 12 steps; graph replay = eager."""
+    from alpha2_amd.fused import FusedTrainer
+    from alpha2_amd.model import ModelConfig
+    from alpha2_amd.train import TrainConfig, syntheticBatch
+    cfg = dict(CFG, attention="reference-flash", dropout=0.25)
+    steps = 12
+    tc = dict(iters=steps, gradAccumSteps=accum, seed=77)
+    mk = lambda graph: FusedTrainer(B, ModelConfig(**cfg), TrainConfig(**tc), 4, seed=6, use_graph=graph, accum=accum)
+    ft, eager = mk(True), mk(False)
+    orc = rm.Trainer(rm.ModelConfig(**cfg), rm.TrainConfig(**tc), seed=6)
+    nodrop = rm.Trainer(rm.ModelConfig(**dict(cfg, dropout=0.0)), rm.TrainConfig(**tc), seed=6)
+    differs = 0
+    for s in range(steps):
+        seeds = [900 + accum * s + m for m in range(accum)]
+        ids = [ft.add_batch(*syntheticBatch(sd, 4, 64, 256)) for sd in seeds]
+        ide = [eager.add_batch(*syntheticBatch(sd, 4, 64, 256)) for sd in seeds]
+        ft.step(ids if accum > 1 else ids[0])
+        eager.step(ide if accum > 1 else ide[0])
+        ob = [rm.synthetic_batch(sd, 4, 64, 256) for sd in seeds]
+        o, o0 = orc.step(ob), nodrop.step(ob)
+        hg, he = ft.history(s, 1)[0], eager.history(s, 1)[0]
+        assert abs(hg.loss - o.loss) <= 2e-2 * abs(o.loss), (s, hg.loss, o.loss)
+        assert abs(hg.gradNorm - o.gradNorm) <= 4e-2 * o.gradNorm, (s, hg.gradNorm, o.gradNorm)
+        assert hg.loss == he.loss and hg.gradNorm == he.gradNorm, (s, hg, he)
+        differs += abs(o.loss - o0.loss) > 1e-3 * abs(o0.loss)
+    assert differs >= 3                                   # the masks matter at this size: the comparison is not vacuous
+    ft.close(), eager.close()
+
+
+def test_fused_dropout_gradients_match_oracle_and_other_wirings_are_refused(B):
+    from alpha2_amd.fused import FusedTrainer
+    from alpha2_amd.model import ModelConfig
+    from alpha2_amd.train import TrainConfig, syntheticBatch
+    cfg = dict(CFG, attention="reference-flash", dropout=0.2)
+    with pytest.raises(ValueError, match="reference-flash"):
+        FusedTrainer(B, ModelConfig(**dict(cfg, attention="heads")), TrainConfig(iters=1), 4)
+    ft = FusedTrainer(B, ModelConfig(**cfg), TrainConfig(iters=1, seed=5), 4, seed=1, use_graph=False)
+    orc = rm.Trainer(rm.ModelConfig(**cfg), rm.TrainConfig(iters=1, seed=5), seed=1)
+    ft.set_batch(*syntheticBatch(3, 4, 64, 256))
+    ob = rm.synthetic_batch(3, 4, 64, 256)
+    orc.dropoutRng.reset(5 + 0 * 1000 + 0, 0)             # the masks of step 0, micro-step 0 (trainer.ts:1169,1202)
+    _, oloss = rm.gptForward(orc.cfg, orc.params, orc.B, orc.tape, ob[0], ob[1], True, dropoutRng=orc.dropoutRng)
+    orc.tape.backward(oloss, orc.B)
+    ograds = {n: v.grad.data.copy() for n, v in orc.entries}
+    ft.step()
+    st = ft.history(0, 1)[0]
+    assert abs(st.loss - float(oloss.data.data[0])) <= 2e-2 * abs(float(oloss.data.data[0]))
+    for name, g in ograds.items():
+        got, w = ft.grad(name).astype(np.float64), g.astype(np.float64)
+        cos = float(got @ w / (np.linalg.norm(got) * np.linalg.norm(w) + 1e-300))
+        assert cos > 0.995 and abs(np.linalg.norm(got) / np.linalg.norm(w) - 1) < 3e-2, (name, cos)
+    ft.close()
+
+
 @pytest.mark.parametrize("attention", ATTENTION)
 def test_fused_gradient_accumulation_matches_oracle(B, attention):
     """Two micro-batches per optimizer step: summed gradients scaled once, reported loss = mean of the micro losses

@@ -142,6 +142,56 @@ def test_dropout_mask_equals_the_cpu_path_for_every_index(B):
         B.dropoutMask([4], 1, 0, 1.0)
 
 
+@pytest.mark.parametrize("n", [1, 7, 4096, 1_000_003])
+def test_dropout_applied_from_a_seed_in_device_memory_equals_mask_then_multiply_add(B, n):
+    """ah_dropout_apply against the reference's own sequence (ops.ts:616-686: dropoutMask, then residual + projected * mask, and
+    grad * mask in backward) with DropoutRng's CPU-path mask: f32 in and out exactly; bf16 operands to the one rounding of the
+    result; a new seed written to the same device word gives the other mask without anything else changing."""
+    import ctypes as C
+    from alpha2_amd import _ffi as ffi
+    lib = B.lib
+    r = np.random.RandomState(n % 1000)
+    x, res = r.randn(n).astype(np.float32), r.randn(n).astype(np.float32)
+    bits = lambda a: (lambda u: ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16))(a.view(np.uint32).astype(np.uint64))
+    widen = lambda h: (h.astype(np.uint32) << 16).view(np.float32)
+    live = []
+
+    def up(a):
+        p = C.c_uint64()
+        ffi.check(lib.ah_alloc(max(a.nbytes, 16), C.byref(p)))
+        ffi.check(lib.ah_upload(p.value, a.ctypes.data_as(C.c_void_p), a.nbytes))
+        live.append(p.value)
+        return p.value
+
+    def down(ptr, dtype):
+        out = np.empty(n, dtype)
+        ffi.check(lib.ah_download(out.ctypes.data_as(C.c_void_p), ptr, out.nbytes))
+        return out
+    seed_dev = up(np.array([0], np.int32))
+    xf, rf, xb, rb = up(x), up(res), up(bits(x)), up(bits(res))
+    of, ob = up(np.zeros(n, np.float32)), up(np.zeros(n, np.uint16))
+    for seed, counter, p in ((42, 0, 0.1), (-7 + 3 * 1000 + 1, 5, 0.5)):
+        ffi.check(lib.ah_upload(seed_dev, np.array([seed], np.int32).ctypes.data_as(C.c_void_p), 4))
+        mask = ref.dropout_mask(seed, counter, p, n)
+        ffi.check(lib.ah_dropout_apply(xf, ffi.F32, rf, of, ffi.F32, n, seed_dev, counter, p))
+        assert np.array_equal(down(of, np.float32), res + x * mask)
+        ffi.check(lib.ah_dropout_apply(xf, ffi.F32, 0, of, ffi.F32, n, seed_dev, counter, p))                  # backward: no residual
+        assert np.array_equal(down(of, np.float32), x * mask)
+        ffi.check(lib.ah_dropout_apply(xb, ffi.BF16, rb, ob, ffi.BF16, n, seed_dev, counter, p))
+        assert np.array_equal(down(ob, np.uint16), bits(widen(bits(res)) + widen(bits(x)) * mask))
+        ffi.check(lib.ah_dropout_apply(xb, ffi.BF16, rf, of, ffi.F32, n, seed_dev, counter, p))
+        assert np.array_equal(down(of, np.float32), res + widen(bits(x)) * mask)
+        ffi.check(lib.ah_dropout_apply(xf, ffi.F32, 0, ob, ffi.BF16, n, seed_dev, counter, p))
+        assert np.array_equal(down(ob, np.uint16), bits(x * mask))
+        if n > 8:                                                   # operands that are not 16-byte aligned take the one-at-a-time path
+            ffi.check(lib.ah_dropout_apply(xb + 2, ffi.BF16, rb + 2, ob + 2, ffi.BF16, n - 1, seed_dev, counter, p))
+            assert np.array_equal(down(ob, np.uint16)[1:], bits(widen(bits(res))[1:] + widen(bits(x))[1:] * mask[:-1]))
+    assert lib.ah_dropout_apply(xf, ffi.F32, 0, of, ffi.F32, n, seed_dev, 0, 1.0) == 2
+    assert lib.ah_dropout_apply(xf, ffi.F32, 0, of, ffi.F32, n, 0, 0, 0.5) == 2
+    for p_ in live:
+        lib.ah_free(p_)
+
+
 @pytest.mark.parametrize("rows,cols", [(1, 4), (37, 24), (130, 260), (1000, 512)])
 def test_channel_activation_mixtures_match_the_composed_ops(B, rows, cols):
     """channelAct / channelActBackward (one pass) against the oracle running the chain of ops the reference records for its
