@@ -24,14 +24,14 @@ constexpr int WAVES = 4;   // 4 waves x 32 owned rows = 128 rows per block
 
 __device__ __forceinline__ float softcap_fwd(float s, float cap, float inv_cap) { return cap > 0.f ? tanhf(s * inv_cap) * cap : s; }
 
-// cooperative load of a [32 x D] f32 tile (rows row0.., zero beyond `rows`) into LDS with pitch D+1
+// cooperative load of a [32 x D] f32 tile (rows row0.., zero beyond `rows` and beyond feature hd) into LDS with pitch D+1
 template <int D>
-__device__ __forceinline__ void load_tile_f32(float *s, const float *__restrict__ base, int64_t st, int row0, int rows, float mul) {
+__device__ __forceinline__ void load_tile_f32(float *s, const float *__restrict__ base, int64_t st, int row0, int rows, float mul, int hd) {
   constexpr int P = D + 1, V4 = D / 4;
   for (int c = threadIdx.x; c < BC * V4; c += blockDim.x) {
     int r = c / V4, d4 = c % V4;
     float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (row0 + r < rows) x = *reinterpret_cast<const float4 *>(base + (int64_t)(row0 + r) * st + d4 * 4);
+    if (row0 + r < rows && d4 * 4 < hd) x = *reinterpret_cast<const float4 *>(base + (int64_t)(row0 + r) * st + d4 * 4);
     float *p = s + r * P + d4 * 4;
     p[0] = x.x * mul; p[1] = x.y * mul; p[2] = x.z * mul; p[3] = x.w * mul;
   }
@@ -55,7 +55,7 @@ __global__ __launch_bounds__(256) void k_flash_fwd_f32(FlashArgs a) {
 
   float qreg[D / 2];                                  // Q[qi][2i + lk] * scale
 #pragma unroll
-  for (int i = 0; i < D / 2; i++) qreg[i] = qi < a.T ? Q[(int64_t)qi * a.q_st + 2 * i + lk] * a.scale : 0.f;
+  for (int i = 0; i < D / 2; i++) qreg[i] = qi < a.T && 2 * i + lk < a.hd ? Q[(int64_t)qi * a.q_st + 2 * i + lk] * a.scale : 0.f;
 
   f32x16 o[DB];
 #pragma unroll
@@ -67,8 +67,8 @@ __global__ __launch_bounds__(256) void k_flash_fwd_f32(FlashArgs a) {
   int q_block_end = min(a.T, (xblk + 1) * (WAVES * 32));   // causal: keys < q_block_end
   for (int kv0 = 0; kv0 < q_block_end; kv0 += BC) {
     __syncthreads();
-    load_tile_f32<D>(Ks, K, a.k_st, kv0, a.T, 1.0f);
-    load_tile_f32<D>(Vs, V, a.v_st, kv0, a.T, 1.0f);
+    load_tile_f32<D>(Ks, K, a.k_st, kv0, a.T, 1.0f, a.hd);
+    load_tile_f32<D>(Vs, V, a.v_st, kv0, a.T, 1.0f, a.hd);
     __syncthreads();
     if (kv0 > q0 + 31) continue;                      // whole tile is in this wave's future (uniform per wave)
     f32x16 s;
@@ -115,7 +115,7 @@ __global__ __launch_bounds__(256) void k_flash_fwd_f32(FlashArgs a) {
 #pragma unroll
       for (int j = 0; j < 4; j++) {
         float4 w = make_float4(o[d][4 * j] * inv_l, o[d][4 * j + 1] * inv_l, o[d][4 * j + 2] * inv_l, o[d][4 * j + 3] * inv_l);
-        *reinterpret_cast<float4 *>(O + 32 * d + 8 * j + 4 * lk) = w;
+        if (32 * d + 8 * j + 4 * lk < a.hd) *reinterpret_cast<float4 *>(O + 32 * d + 8 * j + 4 * lk) = w;
       }
     if (lk == 0) a.lse[((int64_t)b * a.H + h) * a.T + qi] = m + logf(l);
   }
@@ -132,7 +132,7 @@ __global__ void k_flash_delta_f32(FlashArgs a) {
   const float *O = (const float *)a.o + b * a.o_sb + h * a.o_sh + (int64_t)t * a.o_st;
   const float *dO = (const float *)a.d_o + b * a.o_sb + h * a.o_sh + (int64_t)t * a.o_st;
   float s = 0.f;
-  for (int d = lane; d < D; d += 64) s += O[d] * dO[d];
+  for (int d = lane; d < a.hd; d += 64) s += O[d] * dO[d];
   s = wave_sum(s);
   if (lane == 0) a.delta[row] = s;
 }
@@ -157,8 +157,8 @@ __global__ __launch_bounds__(256) void k_flash_dq_f32(FlashArgs a) {
   float qreg[D / 2], doreg[D / 2];
 #pragma unroll
   for (int i = 0; i < D / 2; i++) {
-    qreg[i] = live ? Q[(int64_t)qi * a.q_st + 2 * i + lk] * a.scale : 0.f;
-    doreg[i] = live ? dO[(int64_t)qi * a.o_st + 2 * i + lk] : 0.f;
+    qreg[i] = live && 2 * i + lk < a.hd ? Q[(int64_t)qi * a.q_st + 2 * i + lk] * a.scale : 0.f;
+    doreg[i] = live && 2 * i + lk < a.hd ? dO[(int64_t)qi * a.o_st + 2 * i + lk] : 0.f;
   }
   int64_t srow = ((int64_t)b * a.H + h) * a.T + qi;
   float lse = live ? a.lse[srow] : 0.f, delta = live ? a.delta[srow] : 0.f;
@@ -172,8 +172,8 @@ __global__ __launch_bounds__(256) void k_flash_dq_f32(FlashArgs a) {
   int q_block_end = min(a.T, (xblk + 1) * (WAVES * 32));
   for (int kv0 = 0; kv0 < q_block_end; kv0 += BC) {
     __syncthreads();
-    load_tile_f32<D>(Ks, K, a.k_st, kv0, a.T, 1.0f);
-    load_tile_f32<D>(Vs, V, a.v_st, kv0, a.T, 1.0f);
+    load_tile_f32<D>(Ks, K, a.k_st, kv0, a.T, 1.0f, a.hd);
+    load_tile_f32<D>(Vs, V, a.v_st, kv0, a.T, 1.0f, a.hd);
     __syncthreads();
     if (kv0 > q0 + 31) continue;
     f32x16 s, dp;
@@ -207,7 +207,8 @@ __global__ __launch_bounds__(256) void k_flash_dq_f32(FlashArgs a) {
     for (int d = 0; d < DB; d++)
 #pragma unroll
       for (int j = 0; j < 4; j++)
-        *reinterpret_cast<float4 *>(dQ + 32 * d + 8 * j + 4 * lk) = make_float4(dq[d][4 * j], dq[d][4 * j + 1], dq[d][4 * j + 2], dq[d][4 * j + 3]);
+        if (32 * d + 8 * j + 4 * lk < a.hd)
+          *reinterpret_cast<float4 *>(dQ + 32 * d + 8 * j + 4 * lk) = make_float4(dq[d][4 * j], dq[d][4 * j + 1], dq[d][4 * j + 2], dq[d][4 * j + 3]);
   }
 }
 
@@ -230,8 +231,8 @@ __global__ __launch_bounds__(256) void k_flash_dkv_f32(FlashArgs a) {
   float kreg[D / 2], vreg[D / 2];
 #pragma unroll
   for (int i = 0; i < D / 2; i++) {
-    kreg[i] = live ? K[(int64_t)kvi * a.k_st + 2 * i + lk] : 0.f;
-    vreg[i] = live ? V[(int64_t)kvi * a.v_st + 2 * i + lk] : 0.f;
+    kreg[i] = live && 2 * i + lk < a.hd ? K[(int64_t)kvi * a.k_st + 2 * i + lk] : 0.f;
+    vreg[i] = live && 2 * i + lk < a.hd ? V[(int64_t)kvi * a.v_st + 2 * i + lk] : 0.f;
   }
   f32x16 dk[DB], dv[DB];
 #pragma unroll
@@ -242,8 +243,8 @@ __global__ __launch_bounds__(256) void k_flash_dkv_f32(FlashArgs a) {
   int64_t srow0 = ((int64_t)b * a.H + h) * a.T;
   for (int q0 = kv_blk0; q0 < a.T; q0 += BC) {        // causal: queries at or after this block's first key
     __syncthreads();
-    load_tile_f32<D>(Qs, Q, a.q_st, q0, a.T, a.scale);
-    load_tile_f32<D>(dOs, dO, a.o_st, q0, a.T, 1.0f);
+    load_tile_f32<D>(Qs, Q, a.q_st, q0, a.T, a.scale, a.hd);
+    load_tile_f32<D>(dOs, dO, a.o_st, q0, a.T, 1.0f, a.hd);
     if (threadIdx.x < BC) {
       int qi = q0 + threadIdx.x;
       Ls[threadIdx.x] = qi < a.T ? a.lse[srow0 + qi] : 0.f;
@@ -286,6 +287,7 @@ __global__ __launch_bounds__(256) void k_flash_dkv_f32(FlashArgs a) {
     for (int d = 0; d < DB; d++)
 #pragma unroll
       for (int j = 0; j < 4; j++) {
+        if (32 * d + 8 * j + 4 * lk >= a.hd) continue;
         *reinterpret_cast<float4 *>(dK + 32 * d + 8 * j + 4 * lk) = make_float4(dk[d][4 * j], dk[d][4 * j + 1], dk[d][4 * j + 2], dk[d][4 * j + 3]);
         *reinterpret_cast<float4 *>(dV + 32 * d + 8 * j + 4 * lk) = make_float4(dv[d][4 * j], dv[d][4 * j + 1], dv[d][4 * j + 2], dv[d][4 * j + 3]);
       }
@@ -295,7 +297,7 @@ __global__ __launch_bounds__(256) void k_flash_dkv_f32(FlashArgs a) {
 int32_t check(const AhFlash *f, bool bwd, FlashArgs &a) {
   AH_ARG(f != nullptr, "flash attention: null descriptor");
   AH_ARG(f->dtype == AH_F32 || f->dtype == AH_BF16, "flash attention: dtype %d must be f32 or bf16", f->dtype);
-  AH_ARG(f->head_dim == 32 || f->head_dim == 64 || f->head_dim == 128, "flash attention: head_dim %d not in {32, 64, 128}", f->head_dim);
+  AH_ARG(f->head_dim >= 8 && f->head_dim <= 128 && f->head_dim % 8 == 0, "flash attention: head_dim %d is not a multiple of 8 from 8 to 128", f->head_dim);
   AH_ARG(f->batch >= 0 && f->heads >= 0 && f->seq >= 0, "flash attention: negative extent");
   AH_ARG((int64_t)f->batch * f->heads <= 65535, "flash attention: batch*heads %lld exceeds 65535", (long long)f->batch * f->heads);
   AH_ARG(f->q && f->k && f->v && f->o && f->lse, "flash attention: null operand");
@@ -313,7 +315,7 @@ int32_t check(const AhFlash *f, bool bwd, FlashArgs &a) {
   a.o = dp<void>(f->o); a.lse = dp<float>(f->lse);
   a.d_o = dp<const void>(f->d_o); a.dq = dp<void>(f->dq); a.dk = dp<void>(f->dk); a.dv = dp<void>(f->dv);
   a.delta = nullptr; a.variant = f->bwd_variant;
-  a.B = f->batch; a.H = f->heads; a.T = f->seq;
+  a.B = f->batch; a.H = f->heads; a.T = f->seq; a.hd = f->head_dim;
   a.q_sb = f->q_sb; a.q_sh = f->q_sh; a.q_st = f->q_st;
   a.k_sb = f->k_sb; a.k_sh = f->k_sh; a.k_st = f->k_st;
   a.v_sb = f->v_sb; a.v_sh = f->v_sh; a.v_st = f->v_st;
@@ -356,8 +358,9 @@ int32_t ah_flash_fwd(const AhFlash *f) {
   int32_t rc = check(f, false, a);
   if (rc) return rc;
   if (a.B * a.H == 0 || a.T == 0) return AH_OK;
-  if (f->dtype == AH_BF16) return flash_fwd_bf16(a, f->head_dim);
-  switch (f->head_dim) {
+  const int tile_d = f->head_dim <= 32 ? 32 : f->head_dim <= 64 ? 64 : 128;      // the kernels' head size: the features beyond head_dim are zeros
+  if (f->dtype == AH_BF16) return flash_fwd_bf16(a, tile_d);
+  switch (tile_d) {
     case 32: return run_fwd<32>(a);
     case 64: return run_fwd<64>(a);
     default: return run_fwd<128>(a);
@@ -370,8 +373,9 @@ int32_t ah_flash_bwd(const AhFlash *f) {
   int32_t rc = check(f, true, a);
   if (rc) return rc;
   if (a.B * a.H == 0 || a.T == 0) return AH_OK;
-  if (f->dtype == AH_BF16) return flash_bwd_bf16(a, f->head_dim);
-  switch (f->head_dim) {
+  const int tile_d = f->head_dim <= 32 ? 32 : f->head_dim <= 64 ? 64 : 128;
+  if (f->dtype == AH_BF16) return flash_bwd_bf16(a, tile_d);
+  switch (tile_d) {
     case 32: return run_bwd<32>(a);
     case 64: return run_bwd<64>(a);
     default: return run_bwd<128>(a);

@@ -50,13 +50,14 @@ __device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_ex
 __device__ __forceinline__ float rcp_fast(float x) { return __builtin_amdgcn_rcpf(x); }
 
 // global -> registers: rows [row0, row0+64) of a [T][D] operand with row stride st (elements); rows >= T read as zero
-template <int D>
-__device__ __forceinline__ void tile_load(const uint16_t *__restrict__ base, int64_t st, int row0, int T, u32x4 (&v)[Geo<D>::CHUNKS]) {
+// (PAD: the tensors' head size hd is smaller than D; features hd .. D - 1 read as zero)
+template <int D, bool PAD = false>
+__device__ __forceinline__ void tile_load(const uint16_t *__restrict__ base, int64_t st, int row0, int T, u32x4 (&v)[Geo<D>::CHUNKS], int hd = D) {
 #pragma unroll
   for (int i = 0; i < Geo<D>::CHUNKS; i++) {
     int c = threadIdx.x + 256 * i, r = c / (D / 8), c8 = c % (D / 8);
     u32x4 x = {0u, 0u, 0u, 0u};
-    if (row0 + r < T) x = *reinterpret_cast<const u32x4 *>(base + (int64_t)(row0 + r) * st + c8 * 8);
+    if (row0 + r < T && (!PAD || c8 * 8 < hd)) x = *reinterpret_cast<const u32x4 *>(base + (int64_t)(row0 + r) * st + c8 * 8);
     v[i] = x;
   }
 }
@@ -91,25 +92,25 @@ __device__ __forceinline__ bf16x8 acc_to_b(const f32x16 &s, int m) {
   return r;
 }
 // this lane's row of a [T][D] operand as B fragments (k = d): one 16-byte global load per 16 features
-template <int D>
-__device__ __forceinline__ void row_frags(const uint16_t *__restrict__ base, int64_t st, int row, bool live, int lane, bf16x8 (&f)[D / 16]) {
+template <int D, bool PAD = false>
+__device__ __forceinline__ void row_frags(const uint16_t *__restrict__ base, int64_t st, int row, bool live, int lane, bf16x8 (&f)[D / 16], int hd = D) {
 #pragma unroll
   for (int ks = 0; ks < D / 16; ks++) {
     u32x4 x = {0u, 0u, 0u, 0u};
-    if (live) x = *reinterpret_cast<const u32x4 *>(base + (int64_t)row * st + ks * 16 + (lane >> 5) * 8);
+    if (live && (!PAD || ks * 16 + (lane >> 5) * 8 < hd)) x = *reinterpret_cast<const u32x4 *>(base + (int64_t)row * st + ks * 16 + (lane >> 5) * 8);
     f[ks] = __builtin_bit_cast(bf16x8, x);
   }
 }
 // O^T-style accumulators (rows = features 32db + 8j + 4h + r, column = owned row) -> bf16 row-major store
-template <int D>
-__device__ __forceinline__ void store_rows(uint16_t *__restrict__ dst, const f32x16 (&acc)[D / 32], float mul, int lane) {
+template <int D, bool PAD = false>
+__device__ __forceinline__ void store_rows(uint16_t *__restrict__ dst, const f32x16 (&acc)[D / 32], float mul, int lane, int hd = D) {
   int lk = lane >> 5;
 #pragma unroll
   for (int db = 0; db < D / 32; db++)
 #pragma unroll
     for (int j = 0; j < 4; j++) {
       uint2 w = make_uint2(pack_bf16x2(acc[db][4 * j] * mul, acc[db][4 * j + 1] * mul), pack_bf16x2(acc[db][4 * j + 2] * mul, acc[db][4 * j + 3] * mul));
-      *reinterpret_cast<uint2 *>(dst + 32 * db + 8 * j + 4 * lk) = w;
+      if (!PAD || 32 * db + 8 * j + 4 * lk < hd) *reinterpret_cast<uint2 *>(dst + 32 * db + 8 * j + 4 * lk) = w;
     }
 }
 
@@ -117,8 +118,8 @@ __device__ __forceinline__ void store_rows(uint16_t *__restrict__ dst, const f32
 // Launch bounds ask for at least two (three) waves per SIMD at head sizes up to 64: besides the occupancy this keeps the
 // register budget at 256 (170), where the compiler uses the VGPR form of MFMA and no accumulator ever has to be copied
 // between AGPRs and VGPRs for the softmax arithmetic.
-template <int D, bool CAPPED>
-__global__ __launch_bounds__(256, D <= 64 ? 3 : 1) void k_flash_fwd_bf16(FlashArgs a) {
+template <int D, bool CAPPED, bool PAD>
+__device__ __forceinline__ void flash_fwd_bf16_body(const FlashArgs &a) {
   constexpr int DB = D / 32, KS = D / 16;
   __shared__ __attribute__((aligned(16))) uint16_t Ks[2][Geo<D>::ELEMS], Vs[2][Geo<D>::ELEMS];
   int bh, xblk;
@@ -135,7 +136,7 @@ __global__ __launch_bounds__(256, D <= 64 ? 3 : 1) void k_flash_fwd_bf16(FlashAr
   const float ic2 = CAPPED ? -1.0f / (2.0f * a.cap * LOG2E) : 0.f;      // 1 / c2, c2 = -2 cap log2(e): p = 2^(c2 r)
 
   bf16x8 qf[KS];
-  row_frags<D>(Q, a.q_st, qi, qi < a.T, lane, qf);
+  row_frags<D, PAD>(Q, a.q_st, qi, qi < a.T, lane, qf, a.hd);
   f32x16 o[DB];
 #pragma unroll
   for (int d = 0; d < DB; d++)
@@ -154,16 +155,16 @@ __global__ __launch_bounds__(256, D <= 64 ? 3 : 1) void k_flash_fwd_bf16(FlashAr
   int kv_end = min(a.T, (qblk + 1) * 128);                         // causal: keys < kv_end
   int ntile = (kv_end + ST - 1) / ST;
   u32x4 rk[Geo<D>::CHUNKS], rv[Geo<D>::CHUNKS];
-  tile_load<D>(K, a.k_st, 0, a.T, rk);
-  tile_load<D>(V, a.v_st, 0, a.T, rv);
+  tile_load<D, PAD>(K, a.k_st, 0, a.T, rk, a.hd);
+  tile_load<D, PAD>(V, a.v_st, 0, a.T, rv, a.hd);
   tile_store<D>(Ks[0], rk);
   tile_store<D>(Vs[0], rv);
   __syncthreads();
   for (int it = 0; it < ntile; it++) {
     int cur = it & 1;
     if (it + 1 < ntile) {
-      tile_load<D>(K, a.k_st, (it + 1) * ST, a.T, rk);
-      tile_load<D>(V, a.v_st, (it + 1) * ST, a.T, rv);
+      tile_load<D, PAD>(K, a.k_st, (it + 1) * ST, a.T, rk, a.hd);
+      tile_load<D, PAD>(V, a.v_st, (it + 1) * ST, a.T, rv, a.hd);
     }
     if (CAPPED && it * ST + ST - 1 <= q0) {
       // Both 32-key halves of the tile lie entirely below this wave's diagonal (no masking, which is most tiles): run
@@ -272,11 +273,16 @@ __global__ __launch_bounds__(256, D <= 64 ? 3 : 1) void k_flash_fwd_bf16(FlashAr
   if (CAPPED) { l += __shfl_xor(l, 32, 64); l_rnd = lacc[0]; } else l_rnd = l;
   if (qi < a.T) {
     float inv_l = l_rnd > 0.f ? 1.0f / l_rnd : 0.f;
-    store_rows<D>((uint16_t *)a.o + b * a.o_sb + h * a.o_sh + (int64_t)qi * a.o_st, o, inv_l, lane);
+    store_rows<D, PAD>((uint16_t *)a.o + b * a.o_sb + h * a.o_sh + (int64_t)qi * a.o_st, o, inv_l, lane, a.hd);
     // natural-log LSE: the constant maximum is the cap itself; the running maximum is held in base 2
     if (lk == 0) a.lse[((int64_t)b * a.H + h) * a.T + qi] = (CAPPED ? a.cap : m * (1.0f / LOG2E)) + __logf(l);
   }
 }
+template <int D, bool CAPPED>
+__global__ __launch_bounds__(256, D <= 64 ? 3 : 1) void k_flash_fwd_bf16(FlashArgs a) { flash_fwd_bf16_body<D, CAPPED, false>(a); }
+// the same for tensors whose head size is smaller than D
+template <int D, bool CAPPED>
+__global__ __launch_bounds__(256, D <= 64 ? 3 : 1) void k_flash_fwd_bf16_padded(FlashArgs a) { flash_fwd_bf16_body<D, CAPPED, true>(a); }
 
 // Per-score backward arithmetic shared by the dQ and dK/dV kernels.  s = raw q.k, dpd = dO.v - delta (the dP accumulator
 // starts at -delta = -rowsum(dO*O), so the subtraction rides on the MFMA), krow = (max - lse) in base 2 (max = cap when
@@ -297,8 +303,8 @@ __device__ __forceinline__ float score_bwd(float s, float dpd, float krow, float
 }
 
 // ------------------------------------------------------------------------------------------ dQ (and delta)
-template <int D, bool CAPPED>
-__global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void k_flash_dq_bf16(FlashArgs a) {
+template <int D, bool CAPPED, bool PAD>
+__device__ __forceinline__ void flash_dq_bf16_body(const FlashArgs &a) {
   constexpr int DB = D / 32, KS = D / 16;
   __shared__ __attribute__((aligned(16))) uint16_t Ks[2][Geo<D>::ELEMS], Vs[2][Geo<D>::ELEMS];
   int bh, xblk;
@@ -316,14 +322,14 @@ __global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void k_flash_dq_bf16(FlashArg
   const float c2 = -2.0f * a.cap * LOG2E;
   bool live = qi < a.T;
   bf16x8 qf[KS], dof[KS];
-  row_frags<D>(Q, a.q_st, qi, live, lane, qf);
-  row_frags<D>(dO, a.o_st, qi, live, lane, dof);
+  row_frags<D, PAD>(Q, a.q_st, qi, live, lane, qf, a.hd);
+  row_frags<D, PAD>(dO, a.o_st, qi, live, lane, dof, a.hd);
   int64_t srow = ((int64_t)b * a.H + h) * a.T + qi;
   // delta = rowsum(dO * O): each half-wave holds half of the row's features; also published for the dK/dV kernel
   float delta = 0.f;
   {
     bf16x8 of[KS];
-    row_frags<D>(O, a.o_st, qi, live, lane, of);
+    row_frags<D, PAD>(O, a.o_st, qi, live, lane, of, a.hd);
 #pragma unroll
     for (int ks = 0; ks < KS; ks++)
 #pragma unroll
@@ -341,16 +347,16 @@ __global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void k_flash_dq_bf16(FlashArg
   int kv_end = min(a.T, (qblk + 1) * 128);
   int ntile = (kv_end + ST - 1) / ST;
   u32x4 rk[Geo<D>::CHUNKS], rv[Geo<D>::CHUNKS];
-  tile_load<D>(K, a.k_st, 0, a.T, rk);
-  tile_load<D>(V, a.v_st, 0, a.T, rv);
+  tile_load<D, PAD>(K, a.k_st, 0, a.T, rk, a.hd);
+  tile_load<D, PAD>(V, a.v_st, 0, a.T, rv, a.hd);
   tile_store<D>(Ks[0], rk);
   tile_store<D>(Vs[0], rv);
   __syncthreads();
   for (int it = 0; it < ntile; it++) {
     int cur = it & 1;
     if (it + 1 < ntile) {
-      tile_load<D>(K, a.k_st, (it + 1) * ST, a.T, rk);
-      tile_load<D>(V, a.v_st, (it + 1) * ST, a.T, rv);
+      tile_load<D, PAD>(K, a.k_st, (it + 1) * ST, a.T, rk, a.hd);
+      tile_load<D, PAD>(V, a.v_st, (it + 1) * ST, a.T, rv, a.hd);
     }
 #pragma unroll
     for (int sub = 0; sub < ST / 32; sub++) {
@@ -392,12 +398,17 @@ __global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void k_flash_dq_bf16(FlashArg
     }
     __syncthreads();
   }
-  if (live) store_rows<D>((uint16_t *)a.dq + b * a.q_sb + h * a.q_sh + (int64_t)qi * a.q_st, dq, CAPPED ? 4.0f * a.scale : a.scale, lane);
+  if (live) store_rows<D, PAD>((uint16_t *)a.dq + b * a.q_sb + h * a.q_sh + (int64_t)qi * a.q_st, dq, CAPPED ? 4.0f * a.scale : a.scale, lane, a.hd);
 }
+template <int D, bool CAPPED>
+__global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void k_flash_dq_bf16(FlashArgs a) { flash_dq_bf16_body<D, CAPPED, false>(a); }
+// the same for tensors whose head size is smaller than D
+template <int D, bool CAPPED>
+__global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void k_flash_dq_bf16_padded(FlashArgs a) { flash_dq_bf16_body<D, CAPPED, true>(a); }
 
 // ------------------------------------------------------------------------------------------ dK, dV
-template <int D, bool CAPPED>
-__global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void k_flash_dkv_bf16(FlashArgs a) {
+template <int D, bool CAPPED, bool PAD>
+__device__ __forceinline__ void flash_dkv_bf16_body(const FlashArgs &a) {
   constexpr int DB = D / 32, KS = D / 16;
   __shared__ __attribute__((aligned(16))) uint16_t Qs[2][Geo<D>::ELEMS], dOs[2][Geo<D>::ELEMS];
   __shared__ __attribute__((aligned(16))) float Ls[2][ST], Ds[2][ST];      // per streamed query: (max - lse) in base 2; -delta
@@ -415,8 +426,8 @@ __global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void k_flash_dkv_bf16(FlashAr
   const float lse_max = CAPPED ? a.cap : 0.f;
   bool live = kvi < a.T;
   bf16x8 kf[KS], vf[KS];
-  row_frags<D>(K, a.k_st, kvi, live, lane, kf);
-  row_frags<D>(V, a.v_st, kvi, live, lane, vf);
+  row_frags<D, PAD>(K, a.k_st, kvi, live, lane, kf, a.hd);
+  row_frags<D, PAD>(V, a.v_st, kvi, live, lane, vf, a.hd);
   f32x16 dk[DB], dv[DB];
 #pragma unroll
   for (int d = 0; d < DB; d++)
@@ -436,8 +447,8 @@ __global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void k_flash_dkv_bf16(FlashAr
       rd = qi < a.T ? -a.delta[srow0 + qi] : 0.f;
     }
   };
-  tile_load<D>(Q, a.q_st, q_first, a.T, rq);
-  tile_load<D>(dO, a.o_st, q_first, a.T, rdo);
+  tile_load<D, PAD>(Q, a.q_st, q_first, a.T, rq, a.hd);
+  tile_load<D, PAD>(dO, a.o_st, q_first, a.T, rdo, a.hd);
   load_stats(q_first);
   tile_store<D>(Qs[0], rq);
   tile_store<D>(dOs[0], rdo);
@@ -446,8 +457,8 @@ __global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void k_flash_dkv_bf16(FlashAr
   for (int it = 0; it < ntile; it++) {
     int cur = it & 1;
     if (it + 1 < ntile) {
-      tile_load<D>(Q, a.q_st, q_first + (it + 1) * ST, a.T, rq);
-      tile_load<D>(dO, a.o_st, q_first + (it + 1) * ST, a.T, rdo);
+      tile_load<D, PAD>(Q, a.q_st, q_first + (it + 1) * ST, a.T, rq, a.hd);
+      tile_load<D, PAD>(dO, a.o_st, q_first + (it + 1) * ST, a.T, rdo, a.hd);
       load_stats(q_first + (it + 1) * ST);
     }
 #pragma unroll
@@ -507,10 +518,15 @@ __global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void k_flash_dkv_bf16(FlashAr
     __syncthreads();
   }
   if (live) {
-    store_rows<D>((uint16_t *)a.dk + b * a.k_sb + h * a.k_sh + (int64_t)kvi * a.k_st, dk, CAPPED ? 4.0f * a.scale : a.scale, lane);
-    store_rows<D>((uint16_t *)a.dv + b * a.v_sb + h * a.v_sh + (int64_t)kvi * a.v_st, dv, 1.0f, lane);
+    store_rows<D, PAD>((uint16_t *)a.dk + b * a.k_sb + h * a.k_sh + (int64_t)kvi * a.k_st, dk, CAPPED ? 4.0f * a.scale : a.scale, lane, a.hd);
+    store_rows<D, PAD>((uint16_t *)a.dv + b * a.v_sb + h * a.v_sh + (int64_t)kvi * a.v_st, dv, 1.0f, lane, a.hd);
   }
 }
+template <int D, bool CAPPED>
+__global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void k_flash_dkv_bf16(FlashArgs a) { flash_dkv_bf16_body<D, CAPPED, false>(a); }
+// the same for tensors whose head size is smaller than D
+template <int D, bool CAPPED>
+__global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void k_flash_dkv_bf16_padded(FlashArgs a) { flash_dkv_bf16_body<D, CAPPED, true>(a); }
 
 // ------------------------------------------------------------------------------------------ backward, one pass over the scores
 // The dQ / dK,dV pair above evaluates every probability and every score gradient twice, and that per-score arithmetic is what
@@ -744,7 +760,8 @@ __global__ __launch_bounds__(256) void k_flash_dq_reduce(FlashArgs a, const floa
 template <int D, bool CAPPED>
 int32_t run_fwd(const FlashArgs &a) {
   dim3 grid((unsigned)cdiv(a.T, 128), (unsigned)(a.B * a.H));
-  ah::launch_kernel((k_flash_fwd_bf16<D, CAPPED>), grid, dim3(256), 0, a);
+  if (a.hd == D) ah::launch_kernel((k_flash_fwd_bf16<D, CAPPED>), grid, dim3(256), 0, a);
+  else ah::launch_kernel((k_flash_fwd_bf16_padded<D, CAPPED>), grid, dim3(256), 0, a);
   AH_LAUNCH_CHECK();
   return AH_OK;
 }
@@ -767,7 +784,7 @@ int32_t run_bwd_fused(FlashArgs &a) {
 template <int D, bool CAPPED>
 int32_t run_bwd(FlashArgs &a) {
   if constexpr (D <= 64) {
-    if (a.variant == 1 || flash_bwd_one_pass()) return run_bwd_fused<D, CAPPED>(a);
+    if (a.hd == D && (a.variant == 1 || flash_bwd_one_pass())) return run_bwd_fused<D, CAPPED>(a);      // (the one-pass kernel takes whole head sizes only)
   }
   int64_t rows = (int64_t)a.B * a.H * a.T;
   ah_ptr delta = 0;
@@ -775,9 +792,11 @@ int32_t run_bwd(FlashArgs &a) {
   if (rc) return rc;
   a.delta = dp<float>(delta);
   dim3 grid((unsigned)cdiv(a.T, 128), (unsigned)(a.B * a.H));
-  ah::launch_kernel((k_flash_dq_bf16<D, CAPPED>), grid, dim3(256), 0, a);      // also writes delta
+  if (a.hd == D) ah::launch_kernel((k_flash_dq_bf16<D, CAPPED>), grid, dim3(256), 0, a);      // also writes delta
+  else ah::launch_kernel((k_flash_dq_bf16_padded<D, CAPPED>), grid, dim3(256), 0, a);
   AH_LAUNCH_CHECK();
-  ah::launch_kernel((k_flash_dkv_bf16<D, CAPPED>), grid, dim3(256), 0, a);
+  if (a.hd == D) ah::launch_kernel((k_flash_dkv_bf16<D, CAPPED>), grid, dim3(256), 0, a);
+  else ah::launch_kernel((k_flash_dkv_bf16_padded<D, CAPPED>), grid, dim3(256), 0, a);
   AH_LAUNCH_CHECK();
   return ah_free(delta);
 }

@@ -12,6 +12,7 @@ struct FlashArgs {
   void *dq, *dk, *dv;
   float *delta;            // [B, H, T] rowsum(dO * O)
   int B, H, T;
+  int hd;                  // head size of the tensors; the kernels' D is the next of {32, 64, 128}, features hd .. D - 1 read as zero and are not stored
   int64_t q_sb, q_sh, q_st, k_sb, k_sh, k_st, v_sb, v_sh, v_st, o_sb, o_sh, o_st;
   float scale, cap;
   int variant;             // AhFlash::bwd_variant

@@ -78,8 +78,8 @@ class FusedTrainer:
         self.batch, self.T, self.accum, self.use_graph = batch, cfg.blockSize, accum, use_graph
         self.C, self.H, self.L, self.V, self.F = cfg.nEmbd, cfg.nHead, cfg.nLayer, cfg.vocabSize, ffn_dim(cfg)
         self.D = self.C // self.H
-        if self.D not in (32, 64, 128) or self.C % 8 or self.F % 64 or self.C % 64 or self.V % 8:
-            raise ValueError("FusedTrainer needs head_dim in {32,64,128}, nEmbd and ffnDim multiples of 64, vocab multiple of 8")
+        if not (8 <= self.D <= 128 and self.D % 8 == 0) or self.C % 8 or self.F % 64 or self.C % 64 or self.V % 8:
+            raise ValueError("FusedTrainer needs a head size that is a multiple of 8 up to 128, nEmbd and ffnDim multiples of 64, vocab multiple of 8")
         self.BT = batch * self.T
         # Which function the attention sub-layer computes: "heads" = multi-head attention on the columns of the [BT, 3C] projection;
         # "reference-flash" = what gpt.ts:247-254 computes on a backend with flashAttention: q, k, v cut out of the projection

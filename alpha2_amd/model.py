@@ -130,6 +130,11 @@ def clearForwardCache():
     _pos_cache.clear()
 
 
+def flashHeadSize(d: int) -> bool:
+    """Head sizes the fused attention kernels take: multiples of 8 up to 128 (others run the same function op by op)."""
+    return 8 <= d <= 128 and d % 8 == 0
+
+
 def transformerBlock(ctx: Ctx, x: Variable, layer: dict, cfg: ModelConfig, Bt: int, T: int, mask, training: bool) -> Variable:
     """gpt.ts:220-333."""
     H, Cc = cfg.nHead, cfg.nEmbd
@@ -139,14 +144,14 @@ def transformerBlock(ctx: Ctx, x: Variable, layer: dict, cfg: ModelConfig, Bt: i
     qkv = ag.matmulTransposed(ctx, ag.reshape(ctx, ln1, [Bt * T, Cc]), layer["attn"]["wqkv"])
     cap = cfg.softCap if cfg.softCap is not None else 30.0
     scl = 1 / math.sqrt(D)
-    if cfg.attention == "heads" and cfg.dropout == 0 and ag._has(Bk, "attentionQkv") and D in (32, 64, 128):
+    if cfg.attention == "heads" and cfg.dropout == 0 and ag._has(Bk, "attentionQkv") and flashHeadSize(D):
         concat = ag.causalSelfAttention(ctx, qkv, Bt, T, H, scl, cap)
     else:
         qF, kF, vF = ag.sliceQkv(ctx, qkv)
         q, k, v = (ag.reshape(ctx, t, [Bt, T, Cc]) for t in (qF, kF, vF))
         if cfg.attention == "reference-flash" and ag._has(Bk, "flashAttention"):
             qFA, kFA, vFA = (ag.reshape(ctx, t, [Bt * H, T, D]) for t in (q, k, v))
-            if D in (32, 64, 128):
+            if flashHeadSize(D):
                 att = ag.flashAttention(ctx, qFA, kFA, vFA, T, scl, cap)
             else:
                 # a head size without a fused kernel: the same function of the same slabs, op by op (no dropout on the
@@ -218,7 +223,7 @@ def gptForward(cfg: ModelConfig, params: dict, backend, tape: Tape, tokens: Tens
         _pos_cache[key] = pos
     x = ag.add(ctx, tok, ag.embedding(ctx, params["wpe"], pos))
     mask = None
-    if cfg.attention == "unfused" or cfg.dropout != 0 or not ag._has(backend, "attentionQkv") or cfg.nEmbd // cfg.nHead not in (32, 64, 128):
+    if cfg.attention == "unfused" or cfg.dropout != 0 or not ag._has(backend, "attentionQkv") or not flashHeadSize(cfg.nEmbd // cfg.nHead):
         mask = _mask_cache.get((id(backend), T))
         if mask is None:
             mask = backend.causalMask(T)

@@ -418,7 +418,8 @@ int32_t ah_probe_mfma_bf16(int32_t waves_per_simd, int32_t iters, int32_t random
  *      O = P V; LSE = m + log(l).  Element (b, h, t, d) of Q lives at q + b*q_sb + h*q_sh + t*q_st + d
  *      (same strides for K, V; o_* for O and dO; dq/dk/dv use the q strides), so both the reference's
  *      [B*H, T, D] contract and a [B*T, 3C] QKV projection read in place are expressible.
- *      LSE is [B, H, T] f32.  head_dim in {32, 64, 128}. ---- */
+ *      LSE is [B, H, T] f32.  head_dim: a multiple of 8 from 8 to 128 (the kernels are built for 32, 64 and 128; another size
+ *      runs the next larger one with the missing features read as zeros and never stored). ---- */
 typedef struct {
   int32_t dtype;             /* AH_F32 (fp32 MFMA) or AH_BF16 */
   int32_t batch, heads, seq, head_dim;

@@ -93,6 +93,25 @@ def test_fused_loss_parity_over_steps_graph_replay(B, attention):
     ft.close(), eager.close()
 
 
+@pytest.mark.parametrize("attention", ATTENTION)
+def test_fused_step_with_head_size_16_tracks_the_oracle(B, attention):
+    """nEmbd 128 with 8 heads, as in the reference's small domains (packages/core/src/domains.ts:30-31): the attention kernels of
+    size 32 run with half their features read as zeros; 10 steps against the oracle, both wirings."""
+    from alpha2_amd.fused import FusedTrainer
+    from alpha2_amd.model import ModelConfig
+    from alpha2_amd.train import TrainConfig, syntheticBatch
+    cfg = dict(CFG, nHead=8, attention=attention)
+    ft = FusedTrainer(B, ModelConfig(**cfg), TrainConfig(iters=10), 4, seed=2)
+    orc = rm.Trainer(rm.ModelConfig(**cfg), rm.TrainConfig(iters=10), seed=2)
+    for s in range(10):
+        ft.step(ft.add_batch(*syntheticBatch(20 + s, 4, 64, 256)))
+        o = orc.step([rm.synthetic_batch(20 + s, 4, 64, 256)])
+        h = ft.history(s, 1)[0]
+        assert abs(h.loss - o.loss) <= 2e-2 * abs(o.loss), (s, h.loss, o.loss)
+        assert abs(h.gradNorm - o.gradNorm) <= 3e-2 * o.gradNorm, (s, h.gradNorm, o.gradNorm)
+    ft.close()
+
+
 @pytest.mark.parametrize("accum", [1, 2])
 def test_fused_step_with_dropout_matches_oracle(B, accum):
     """dropout 0.25 in the two residualDropoutAdd of every block (gpt.ts:281,332) on the reference's flash-branch wiring: masks

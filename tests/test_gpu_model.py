@@ -32,12 +32,14 @@ def _both(B, cfg_kw, tc_kw, seed=0):
     return dev, orc
 
 
-@pytest.mark.parametrize("attention", ["heads", "unfused"])
-def test_forward_backward_grads_match_oracle(B, attention):
+@pytest.mark.parametrize("attention,heads", [("heads", 2), ("unfused", 4), ("heads", 4), ("heads", 8)])
+def test_forward_backward_grads_match_oracle(B, attention, heads):
+    """Head sizes 32, 16 (unfused), 16 and 8 through the fused kernel (the reference's small domains have 128 / 8 and 64 / 4:
+    packages/core/src/domains.ts): the kernels of size 32 with the missing features read as zeros."""
     from alpha2_amd.autograd import Tape
     from alpha2_amd.model import gptForward
     from alpha2_amd.train import syntheticBatch
-    cfg = dict(vocabSize=61, blockSize=24, nLayer=2, nEmbd=64, nHead=2 if attention == "heads" else 4, attention=attention)
+    cfg = dict(vocabSize=61, blockSize=24, nLayer=2, nEmbd=64, nHead=heads, attention=attention)
     dev, orc = _both(B, cfg, dict(iters=1))
     inp, tgt = syntheticBatch(3, 3, 24, 61)
     oi, ot = rm.synthetic_batch(3, 3, 24, 61)
@@ -164,7 +166,7 @@ def test_activation_checkpointing_matches_plain(B):
 
 
 @pytest.mark.parametrize("kw", [dict(), dict(softCap=0.0), dict(nHead=4, ffnActivation="swiglu", softCap=2.0),
-                                dict(nEmbd=128, nHead=4, softCap=2.0)])        # (the third: head size 16, no fused kernel)
+                                dict(nEmbd=128, nHead=4, softCap=2.0), dict(nEmbd=96, nHead=8, softCap=30.0)])      # (head sizes 32, 32, 16, 32 and 12: the last has no fused kernel)
 def test_reference_flash_branch_matches_its_oracle(B, kw):
     """What an unchanged gpt.ts runs on a backend that offers flashAttention (gpt.ts:247-254: [B, T, C] re-read as
     [B*H, T, D] slabs without a head transpose, flashAttention per slab, transpose (1, 2) back) against the oracle's

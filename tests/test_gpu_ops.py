@@ -899,7 +899,8 @@ def _oracle_attention(q, k, v, do, scale, cap):
     return out.data.data, lse, qv.grad.data, kv.grad.data, vv.grad.data
 
 
-@pytest.mark.parametrize("BH,T,D,cap", [(2, 64, 32, 30.0), (3, 100, 64, 0.0), (2, 129, 64, 30.0), (1, 256, 128, 30.0), (2, 1, 32, 0.0)])
+@pytest.mark.parametrize("BH,T,D,cap", [(2, 64, 32, 30.0), (3, 100, 64, 0.0), (2, 129, 64, 30.0), (1, 256, 128, 30.0), (2, 1, 32, 0.0),
+                                        (3, 130, 16, 30.0), (2, 70, 8, 0.0), (2, 97, 48, 2.0), (1, 200, 96, 30.0)])      # (the last four: sizes between the kernels')
 def test_flash_attention_f32_vs_materialised(B, BH, T, D, cap):
     q, k, v, do = (rs.randn(BH, T, D).astype(np.float32) for _ in range(4))
     scale = 1 / math.sqrt(D)
@@ -1153,11 +1154,14 @@ def bwd_variant(request, B):
 
 
 @pytest.mark.parametrize("BH,T,D,cap", [(2, 64, 32, 30.0), (3, 100, 64, 0.0), (2, 129, 64, 30.0), (2, 320, 64, 30.0), (1, 256, 128, 30.0), (2, 1, 64, 0.0),
-                                        (3, 700, 64, 30.0), (2, 513, 32, 0.0)])
+                                        (3, 700, 64, 30.0), (2, 513, 32, 0.0),
+                                        (3, 200, 16, 30.0), (2, 70, 8, 0.0), (3, 130, 48, 0.0), (2, 96, 80, 30.0), (1, 150, 120, 2.0)])
 def test_flash_attention_bf16_vs_materialised(B, bwd_variant, BH, T, D, cap):
     """bf16 operands, fp32 accumulation.  Inputs are bf16-exact so the oracle sees the same numbers; the kernel rounds P and
     dS to bf16 before the second product and its outputs to bf16, so the bar is bf16 resolution (2^-7 of the tensor scale).
-    T = 700 and 513 give the one-pass kernel several 256-key blocks with a ragged last one."""
+    T = 700 and 513 give the one-pass kernel several 256-key blocks with a ragged last one.  Head sizes 16, 8, 48, 80 and 120 run
+    the kernels of the next size up (32, 64, 128) with the missing features read as zeros and never stored: the tensors here
+    are exactly [BH, T, D], so a store past a row's end would land in the next row and show."""
     q, k, v, do = (_bf16_round(rs.randn(BH, T, D).astype(np.float32))[0] for _ in range(4))
     scale = 1 / math.sqrt(D)
     want_o, want_lse, dq, dk, dv = _oracle_attention(q, k, v, do, scale, cap)
