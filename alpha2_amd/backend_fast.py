@@ -7,8 +7,9 @@ packages/train/src/trainer.ts:1188-1273,1761-1784).  Behind the interface:
     outputs, their gradients); the residual stream, parameters, gradients of parameters and optimizer state stay f32;
   * every 2-D parameter has a bf16 shadow that `adamwStep` refreshes in the same pass (the MFMA operand of the next step);
   * a linear layer's product is held back by ONE call, so that the op the reference issues next can become its epilogue:
-        gelu(matmulTransposed(x, W))                   -> AH_EPI_GELU      (ops.ts:426-487 issues exactly these two calls)
-        geluBackward(pre, matmul(g, W))                -> AH_EPI_GELU_BWD
+        gelu(matmulTransposed(x, W))                   -> AH_EPI_GELU_GRAD (ops.ts:426-487 issues exactly these two calls): the
+                                                          launch saves gelu'(pre) and leaves pre itself as a recipe
+        geluBackward(pre, matmul(g, W))                -> AH_EPI_MUL_AUX with that derivative (AH_EPI_GELU_BWD from a written pre)
         add(x, reshape(matmulTransposed(h, W)))        -> AH_EPI_RESIDUAL  (gpt.ts:280-281,331-332 via residualDropoutAdd)
     anything else that touches the held-back product simply launches it as it is;
   * weight gradients dW = G^T X (matmulTransposedA) are held back until something reads one of them (in the trainer: the
@@ -35,7 +36,7 @@ BF16, F32 = ffi.BF16, ffi.F32
 class _HeldGemm:
     """A product whose launch is held back by one call.  It holds a reference on its operands' buffers and on its output
     buffer until it is launched (or dropped, when nobody but this record still refers to the output)."""
-    __slots__ = ("layout", "a_ptr", "b_ptr", "out_buf", "out_off", "m", "n", "k", "lda", "ldb", "holds", "a_planes")
+    __slots__ = ("layout", "a_ptr", "b_ptr", "out_buf", "out_off", "m", "n", "k", "lda", "ldb", "holds", "a_planes", "gelu_grad")
 
     def __init__(self, layout, a_ptr, b_ptr, out, m, n, k, lda, ldb, holds):
         self.layout, self.a_ptr, self.b_ptr, self.out_buf, self.out_off = layout, a_ptr, b_ptr, out._buf, out._off
@@ -43,6 +44,9 @@ class _HeldGemm:
         # A lies in planes (an unwritten sum of scatterSlice results): (columns per plane, elements from plane to plane), a_ptr
         # the first plane, lda its row stride
         self.a_planes = None
+        # gelu was asked of this product: its derivative at the product's values, saved by the launch that made the activation
+        # (a buffer of the record's own, released with it); the product itself was not written
+        self.gelu_grad = None
 
     @property
     def out_ptr(self) -> int:
@@ -99,8 +103,11 @@ class _HeldScatter:
 class FastHipBackend(HipBackend):
     name = "hip"
 
-    def __init__(self, device: int = 0, group_weight_grads: bool = True, stream_bf16: bool = True):
+    def __init__(self, device: int = 0, group_weight_grads: bool = True, stream_bf16: bool = True, gelu_saves_derivative: bool = True):
         super().__init__(device)
+        # gelu of a held-back product saves gelu'(pre) for the backward product's epilogue (one multiply per element there); False:
+        # it saves the pre-activation itself, as the reference's matmulTransposedGelu contract reads, and backward evaluates gelu'
+        self.geluSavesDerivative = gelu_saves_derivative
         # the residual stream (the running sum the residual adds produce) and the gradient flowing back along it are stored in
         # bf16 like every other activation; False keeps both in f32
         self.streamBf16 = stream_bf16
@@ -446,13 +453,29 @@ class FastHipBackend(HipBackend):
         return self._hold_gemm(ffi.GEMM_NN, a, b, (M, N), M, N, K, K, N)
 
     def gelu(self, a: TensorData) -> TensorData:
-        if self._is_held(a) and self._held.layout == ffi.GEMM_NT:
+        h = self._held
+        if self._is_held(a) and h.layout == ffi.GEMM_NT and not self.geluSavesDerivative:
             out = self._new(a.shape, "f32", "bf16")             # `a` receives the pre-activation, as the caller expects
             self._launch_held(ffi.EPI_GELU, aux=a._buf.ptr + a._off, out=out)
+            return out
+        if self._is_held(a) and h.layout == ffi.GEMM_NT and h.a_planes is None and a._off == h.out_off:
+            # One launch gives gelu(product) and gelu'(product); the derivative is what backward needs (geluBackward multiplies
+            # by it), so it is what is saved.  `a` itself, the pre-activation the caller may still read (ops.ts:426-487), is not
+            # written: the record stays as its recipe and computes it if anybody asks.
+            out = self._new(a.shape, "f32", "bf16")
+            h.gelu_grad = _Buf(self.lib, a.size * 2)
+            h.holds.append(h.gelu_grad)
+            self._launch_held(ffi.EPI_GELU_GRAD, aux=h.gelu_grad.ptr, out=out)
             return out
         return super().gelu(a)
 
     def geluBackward(self, x: TensorData, g: TensorData) -> TensorData:
+        rec = self._orphans.get(id(x._buf)) if self._orphans and x._buf is not None else None
+        if rec is not None and rec.gelu_grad is not None and self._is_held(g) and x.store == "bf16" and x.shape == g.shape \
+                and x._off == rec.out_off and self._held.a_planes is None:
+            out = self._new(g.shape, "f32", "bf16")             # g * gelu'(x) with the saved derivative: one multiply per element
+            self._launch_held(ffi.EPI_MUL_AUX, aux=rec.gelu_grad.ptr, out=out)
+            return out
         if self._is_held(g) and x.store == "bf16" and x.shape == g.shape and not self._is_held(x):
             pre = self._ptr(x)
             out = self._new(g.shape, "f32", "bf16")
