@@ -100,6 +100,27 @@ class _HeldScatter:
         return all(c0 + w <= d0 or d0 + v <= c0 for _, c0, w in self.parts for _, d0, v in other.parts)
 
 
+class _HeldFlash:
+    """A flashAttention that has been asked for and not launched (gpt.ts:247-254 reshapes its result to [B, H, T, D] and
+    transposes (1, 2) next: launched from that transpose, the kernel writes the transposed layout itself through its output
+    strides).  Afterwards the record says where the result lies: `twin` = (buffer, B, H) of the [B, T, H, D] copy while the
+    [B H, T, D] tensor the caller holds is still unwritten (it is written from the twin if anybody reads it)."""
+    __slots__ = ("q", "k", "v", "o_buf", "lse_buf", "BH", "T", "D", "scale", "cap", "holds", "twin", "launched")
+
+    def __init__(self, q, k, v, o_buf, lse_buf, BH, T, D, scale, cap, holds):
+        self.q, self.k, self.v, self.o_buf, self.lse_buf, self.BH, self.T, self.D = q, k, v, o_buf, lse_buf, BH, T, D
+        self.scale, self.cap, self.holds, self.twin, self.launched = scale, cap, holds, None, False
+
+
+class _LazyTranspose:
+    """transpose(1, 2) of a 4-D bf16 tensor that has been asked for and not written: in the backward pass of the slab wiring its
+    consumer is flashAttentionBackward, which reads the source through strides instead."""
+    __slots__ = ("src_ptr", "src_shape", "out_buf", "holds")
+
+    def __init__(self, src_ptr, src_shape, out_buf, holds):
+        self.src_ptr, self.src_shape, self.out_buf, self.holds = src_ptr, tuple(src_shape), out_buf, holds
+
+
 class FastHipBackend(HipBackend):
     name = "hip"
 
@@ -127,6 +148,9 @@ class FastHipBackend(HipBackend):
         self._ssq_args = None            # (addresses, sizes, their ctypes arrays) of the last totalSumOfSquares call
         self._scatters = {}              # id(_Buf) of an unwritten scatterSlice result -> _HeldScatter
         self._planes_ok = {}             # (layout, m, n, k, plane extents) -> does ah_gemm_planes take it
+        # unwritten results whose making is still open: id(_Buf) -> _HeldFlash (under its output's and its LSE's buffer) or _LazyTranspose
+        self._lazy = {}
+        self._pending_flash: Optional[_HeldFlash] = None
         self._held_ce: Optional[_HeldCrossEntropy] = None
         self._held_ln: Optional[_HeldLayerNormBwd] = None
         # dx tensors whose LayerNorm backward went straight into a sum and that were never written themselves: id(_Buf) -> recipe
@@ -166,6 +190,8 @@ class FastHipBackend(HipBackend):
                 self._unhold(h.holds)
             if self._scatters and id(t._buf) in self._scatters:
                 self._write_scatter(t._buf)
+            if self._lazy and id(t._buf) in self._lazy:
+                self._materialise(t._buf)
             if self._held_ce is not None and any(t._buf is b for b in self._held_ce.holds):
                 self._launch_ce()
             if self._held is not None and t._buf is self._held.out_buf:
@@ -265,6 +291,17 @@ class FastHipBackend(HipBackend):
             return super().transpose(a, dim0, dim1)
         ns = list(a.shape)
         ns[d0], ns[d1] = a.shape[d1], a.shape[d0]
+        if nd == 4 and (d0, d1) == (1, 2) and a._buf is not None and a._dev_valid and a.size > 0:
+            rec = self._lazy.get(id(a._buf))
+            if isinstance(rec, _HeldFlash) and not rec.launched and a._buf is rec.o_buf and a._off == 0 \
+                    and a.shape[0] * a.shape[1] == rec.BH and (a.shape[2], a.shape[3]) == (rec.T, rec.D):
+                out = self._new(ns, a.dtype, "bf16")            # the attention kernel writes [B, T, H, D] itself
+                self._launch_flash(rec, twin=(out._buf, a.shape[0], a.shape[1]))
+                return out
+            src = self._ptr(a)                                  # (whatever still has to produce `a` runs now)
+            out = self._new(ns, a.dtype, "bf16")
+            self._lazy[id(out._buf)] = _LazyTranspose(src, a.shape, out._buf, self._hold(a._buf, out._buf))
+            return out
         half = list(a.shape)
         half[-1] //= 2
         out = self._new(ns, a.dtype, "bf16")
@@ -347,6 +384,8 @@ class FastHipBackend(HipBackend):
                 self._unhold(self._ln_unwritten.pop(id(buf)).holds)
             elif self._scatters and id(buf) in self._scatters:
                 self._drop_scatter(buf)
+            elif self._lazy and id(buf) in self._lazy:
+                self._drop_lazy(buf)
             elif self._wgrads:
                 for i, w in enumerate(self._wgrads):
                     if buf is w.out_buf and w.into is None:
@@ -357,7 +396,7 @@ class FastHipBackend(HipBackend):
 
     def _view(self, t: TensorData, shape, byte_off: int = 0) -> TensorData:
         if t._buf is not None and t._dev_valid and (self._is_held(t) or id(t._buf) in self._orphans or self._is_queued(t._buf)
-                                                    or id(t._buf) in self._scatters):
+                                                    or id(t._buf) in self._scatters or id(t._buf) in self._lazy):
             v = TensorData(shape, t.dtype)                      # a view of a held-back product stays held back
             v.store, v._buf, v._off = t.store, t._buf, t._off + byte_off
             t._buf.refs += 1
@@ -690,6 +729,7 @@ class FastHipBackend(HipBackend):
 
     def _own(self, t: TensorData):
         """Before an in-place write: give `t` a buffer nobody else shares."""
+        self._launch_flash()                                    # (a pending attention reads its operands as they are now)
         if t._buf is not None and t._buf.refs > 1 and t._dev_valid:
             n = t.size * ffi.DTYPE_BYTES[t.store]
             buf = _Buf(self.lib, n)
@@ -821,7 +861,85 @@ class FastHipBackend(HipBackend):
     def flashAttention(self, Q, K, V, T, scale, softCap) -> dict:
         if not (Q.store == K.store == V.store):
             self._words(Q, K, V)
-        return super().flashAttention(Q, K, V, T, scale, softCap)
+        if Q.store != "bf16" or Q.size == 0 or len(Q.shape) != 3 or Q.shape[2] % 8 or not 8 <= Q.shape[2] <= 128:
+            return super().flashAttention(Q, K, V, T, scale, softCap)      # (also what the library refuses: it says so at once)
+        self._flash_desc(Q, K, V, T, scale, softCap)            # (the shape checks)
+        self._launch_flash()
+        BH, _, D = Q.shape
+        q, k, v = self._ptr(Q), self._ptr(K), self._ptr(V)
+        out, lse = self._new(Q.shape, "f32", "bf16"), self._new((BH, T))
+        rec = _HeldFlash(q, k, v, out._buf, lse._buf, BH, T, D, scale, softCap, self._hold(Q._buf, K._buf, V._buf, out._buf, lse._buf))
+        self._lazy[id(out._buf)] = self._lazy[id(lse._buf)] = self._pending_flash = rec
+        return {"output": out, "lse": lse}
+
+    def _flash_strides(self, f: ffi.AhFlash, B: int, H: int, T: int, D: int, o_heads: bool):
+        """q, k, v (and their gradients) as [B H, T, D] slabs; o (and dO) as slabs too, or as [B, T, H, D]."""
+        f.batch, f.heads, f.seq, f.head_dim = B, H, T, D
+        for nm in ("q", "k", "v", "o"):
+            setattr(f, nm + "_sb", H * T * D), setattr(f, nm + "_sh", T * D), setattr(f, nm + "_st", D)
+        if o_heads:
+            f.o_sb, f.o_sh, f.o_st = T * H * D, D, H * D
+
+    def _launch_flash(self, rec: Optional[_HeldFlash] = None, twin=None):
+        """Launches the pending attention: into the [B H, T, D] tensor the caller holds, or -- twin = (buffer, B, H) -- as
+        [B, T, H, D] into that buffer, leaving the caller's tensor unwritten."""
+        rec = rec or self._pending_flash
+        if rec is None or rec.launched:
+            return
+        if self._pending_flash is rec:
+            self._pending_flash = None
+        self._lazy.pop(id(rec.lse_buf), None)
+        if twin is None and rec.o_buf.refs == 1 and rec.lse_buf.refs == 1:      # both results released unread
+            self._lazy.pop(id(rec.o_buf), None)
+            rec.launched = True
+            self._unhold(rec.holds)
+            return
+        f = ffi.AhFlash()
+        f.dtype, f.scale, f.soft_cap, f.bwd_variant = BF16, rec.scale, rec.cap, self.flashBackwardVariant
+        f.q, f.k, f.v, f.lse = rec.q, rec.k, rec.v, rec.lse_buf.ptr
+        if twin is None:
+            self._flash_strides(f, rec.BH, 1, rec.T, rec.D, False)
+            f.o = rec.o_buf.ptr
+        else:
+            self._flash_strides(f, twin[1], twin[2], rec.T, rec.D, True)
+            f.o = twin[0].ptr
+        check(self.lib.ah_flash_fwd(C.byref(f)))
+        rec.launched = True
+        self._unhold(rec.holds)
+        rec.holds = []
+        if twin is None:
+            self._lazy.pop(id(rec.o_buf), None)
+        else:                                                   # the caller's tensor now stands for "the twin, transposed back"
+            rec.twin = twin
+            rec.holds = self._hold(rec.o_buf, twin[0])
+
+    def _materialise(self, buf):
+        rec = self._lazy.get(id(buf))
+        if isinstance(rec, _HeldFlash):
+            if not rec.launched:
+                self._launch_flash(rec)
+            elif buf is rec.o_buf and rec.twin is not None:     # somebody reads the slabs after all: transposed back from the twin
+                tb, B, H = rec.twin
+                self._lazy.pop(id(buf), None)
+                check(self.lib.ah_transpose(tb.ptr, buf.ptr, 4, ffi.shape_arr([B, rec.T, H, rec.D // 2]), 1, 2))
+                self._unhold(rec.holds)
+        elif isinstance(rec, _LazyTranspose):
+            self._lazy.pop(id(buf), None)
+            half = list(rec.src_shape)
+            half[-1] //= 2
+            check(self.lib.ah_transpose(rec.src_ptr, buf.ptr, 4, ffi.shape_arr(half), 1, 2))
+            self._unhold(rec.holds)
+
+    def _drop_lazy(self, buf):
+        """`buf` has been released by everybody but its record."""
+        rec = self._lazy.get(id(buf))
+        if isinstance(rec, _HeldFlash) and not rec.launched:
+            if rec.o_buf.refs == 1 and rec.lse_buf.refs == 1:   # (its other result may still be read: then it has to be computed)
+                self._launch_flash(rec)
+            return
+        self._lazy.pop(id(buf), None)
+        if rec is not None:
+            self._unhold(rec.holds)
 
     def flashAttentionBackward(self, Q, K, V, O, dO, lse, T, scale, softCap) -> dict:
         if not (Q.store == K.store == V.store == O.store == dO.store):
@@ -832,7 +950,17 @@ class FastHipBackend(HipBackend):
         # and dW products) can then read them in place
         f = self._flash_desc(Q, K, V, T, scale, softCap)
         f.dtype = BF16
-        f.q, f.k, f.v, f.o, f.lse, f.d_o = self._ptr(Q), self._ptr(K), self._ptr(V), self._ptr(O), self._ptr(lse), self._ptr(dO)
+        orec = self._lazy.get(id(O._buf)) if O._buf is not None else None
+        drec = self._lazy.get(id(dO._buf)) if dO._buf is not None else None
+        if isinstance(orec, _HeldFlash) and orec.twin is not None and isinstance(drec, _LazyTranspose) and O._off == 0 and dO._off == 0 \
+                and O._buf is orec.o_buf and drec.src_shape == (orec.twin[1], T, orec.twin[2], Q.shape[2]):
+            # the forward result exists as [B, T, H, D] and so does its gradient (the transposes around the slabs were never
+            # run): the kernels read both through strides
+            self._flash_strides(f, orec.twin[1], orec.twin[2], T, Q.shape[2], True)
+            f.q, f.k, f.v, f.lse = self._ptr(Q), self._ptr(K), self._ptr(V), self._ptr(lse)
+            f.o, f.d_o = orec.twin[0].ptr, drec.src_ptr
+        else:
+            f.q, f.k, f.v, f.o, f.lse, f.d_o = self._ptr(Q), self._ptr(K), self._ptr(V), self._ptr(O), self._ptr(lse), self._ptr(dO)
         dQ, dK, dV = self._plane_views(3, Q.shape)
         f.dq, f.dk, f.dv = dQ._buf.ptr + dQ._off, dK._buf.ptr + dK._off, dV._buf.ptr + dV._off
         check(self.lib.ah_flash_bwd(C.byref(f)))
@@ -961,6 +1089,7 @@ class FastHipBackend(HipBackend):
 
     def flush(self):
         self._launch_held()
+        self._launch_flash()
         self._launch_ln()
         self._launch_ce()
         self._launch_weight_grads()
@@ -969,6 +1098,7 @@ class FastHipBackend(HipBackend):
 
     def syncGpu(self):
         self._launch_held()
+        self._launch_flash()
         self._launch_ln()
         self._launch_ce()
         self._launch_weight_grads()

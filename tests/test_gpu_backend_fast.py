@@ -524,6 +524,58 @@ def test_the_fused_projection_and_its_backward_take_their_operands_in_planes(FB)
     _close(outs[True][0], _bf16(np.concatenate(gs, axis=1).astype(np.float64) @ w.astype(np.float64)), "dX", 4e-3)
 
 
+def test_the_transposes_around_the_slabs_become_strides_of_the_attention_kernels(FB):
+    """gpt.ts:247-254 reshapes flashAttention's [B H, T, D] result to [B, H, T, D] and transposes (1, 2); its backward transposes the
+    incoming gradient the other way and hands it to flashAttentionBackward.  Held back, neither transpose runs: the forward kernel
+    writes [B, T, H, D] through its output strides and the backward kernels read O and dO in that layout.  Bit for bit what the
+    calls give when every result is read at once (which launches each op on its own), and the slab-shaped result is still right
+    when somebody reads it afterwards."""
+    rs = np.random.RandomState(23)
+    Bt, H, T, D = 3, 4, 96, 32
+    q, k, v = (_bf16(rs.randn(Bt * H, T, D)) for _ in range(3))
+    g = _bf16(rs.randn(Bt, T, H, D))
+    scale, cap = 1 / math.sqrt(D), 30.0
+
+    def run(eager: bool):
+        Q, K, V, G = (FB.castStore(_td(x), "bf16") for x in (q, k, v, g))
+        r = FB.flashAttention(Q, K, V, T, scale, cap)
+        O, lse = r["output"], r["lse"]
+        if eager:
+            O.data
+        O4 = FB.reshape(O, (Bt, H, T, D))
+        Ot = FB.transpose(O4, 1, 2)
+        fwd = Ot.data.reshape(Bt, T, H, D).copy()
+        gT = FB.transpose(G, 1, 2)
+        if eager:
+            gT.data
+        g3 = FB.reshape(gT, (Bt * H, T, D))
+        d = FB.flashAttentionBackward(Q, K, V, O, g3, lse, T, scale, cap)
+        grads = [d[n].data.copy() for n in ("dQ", "dK", "dV")]
+        lazy_left = len(FB._lazy)
+        slab = O.data.reshape(Bt * H, T, D).copy()
+        lsev = lse.data.copy()
+        for t in (O, O4, lse, Ot, gT, g3, Q, K, V, G, d["dQ"], d["dK"], d["dV"]):
+            FB.releaseGpuTensor(t)
+        return fwd, grads, slab, lsev, lazy_left
+    e, l = run(True), run(False)
+    assert e[4] == 0 and l[4] == 2                               # lazily: O stands for its transposed twin, the gradient's transpose was never written
+    assert not FB._lazy
+    assert np.array_equal(e[0], l[0]) and np.array_equal(e[2], l[2]) and np.array_equal(e[3], l[3])
+    assert np.array_equal(l[0], l[2].reshape(Bt, H, T, D).transpose(0, 2, 1, 3))
+    for a, b in zip(e[1], l[1]):
+        assert np.array_equal(a, b)
+    # a result nobody transposes is launched as it is when it is read; one nobody reads is never launched
+    Q, K, V = (FB.castStore(_td(x), "bf16") for x in (q, k, v))
+    r = FB.flashAttention(Q, K, V, T, scale, cap)
+    assert np.array_equal(r["output"].data.reshape(Bt * H, T, D), e[2]) and not FB._lazy
+    r = FB.flashAttention(Q, K, V, T, scale, cap)
+    FB.releaseGpuTensor(r["output"])
+    assert np.array_equal(r["lse"].data, e[3])                   # (its other result is still wanted)
+    r = FB.flashAttention(Q, K, V, T, scale, cap)
+    FB.releaseGpuTensor(r["output"]), FB.releaseGpuTensor(r["lse"])
+    assert not FB._lazy and FB._pending_flash is None
+
+
 def test_cross_entropy_is_held_until_its_backward_is_asked_for(FB):
     """crossEntropy followed by crossEntropyBackward on the same bf16 logits (the tape's last entry, visited first by its
     backward pass) is one pass over the logits: loss, LSE and gradient bit-identical to the two-kernel route; a loss that is
