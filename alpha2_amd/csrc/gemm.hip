@@ -619,11 +619,13 @@ int32_t ah_gemm_planes(const AhGemm *p, int64_t c_plane_cols, int64_t c_plane_st
   if (c_plane_cols > 0) {
     AH_ARG(q.n % c_plane_cols == 0 && q.ldc >= c_plane_cols && c_plane_stride % 4 == 0,
            "ah_gemm_planes: n = %lld is not whole planes of %lld columns, or ldc / the plane stride do not fit", (long long)q.n, (long long)c_plane_cols);
+    AH_ARG(q.n == c_plane_cols || c_plane_stride >= (q.m - 1) * q.ldc + c_plane_cols,
+           "ah_gemm_planes: planes of C %lld elements apart overlap (m = %lld rows of stride %lld)", (long long)c_plane_stride, (long long)q.m, (long long)q.ldc);
   } else {
     AH_ARG(q.ldc >= q.n, "matmul shape mismatch: ldc %lld too small for n=%lld", (long long)q.ldc, (long long)q.n);
   }
   if (a_plane_k > 0) {
-    AH_ARG(q.k % a_plane_k == 0 && q.k / a_plane_k <= 3 && q.lda >= a_plane_k && a_plane_stride % 8 == 0,
+    AH_ARG(q.k % a_plane_k == 0 && q.k / a_plane_k <= 3 && q.lda >= a_plane_k && a_plane_stride % 8 == 0 && a_plane_stride >= 0,
            "ah_gemm_planes: k = %lld is not 1 to 3 whole planes of %lld, or lda / the plane stride do not fit", (long long)q.k, (long long)a_plane_k);
   } else {
     AH_ARG(q.lda >= q.k, "matmul shape mismatch: lda %lld too small for k=%lld", (long long)q.lda, (long long)q.k);

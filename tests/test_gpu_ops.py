@@ -1525,6 +1525,7 @@ def test_gemm_with_an_operand_in_planes_equals_the_product_around_copies(B, M, C
     assert lib.ah_gemm_planes(C.byref(f32out), Cc, M * Cc, 0, 0, 0) == 5
     ragged = ffi.AhGemm(ffi.GEMM_NT, BF, BF, ffi.EPI_NONE, M, 3 * Cc, Cc, Cc, Cc, Cc, 1, 0, 0, 0, px, pw, c2, 0)
     assert lib.ah_gemm_planes(C.byref(ragged), Cc - 64, M * Cc, 0, 0, 0) == 2
+    assert lib.ah_gemm_planes(C.byref(ragged), Cc, M * Cc - 8, 0, 0, 0) == 2 and b"overlap" in lib.ah_last_error()
     for p in live:
         lib.ah_free(p)
 
