@@ -230,6 +230,31 @@ def test_fused_checkpoint_resume(B, tmp_path):
     a.close(), b.close()
 
 
+def test_fused_resume_with_dropout_draws_the_masks_of_the_uninterrupted_run(B, tmp_path):
+    """The masks of a step depend on its index (trainer.ts:1169: seed + 1000 step): a run resumed at step 3 must drop what the
+    uninterrupted run drops from step 3 on."""
+    from alpha2_amd.fused import FusedTrainer
+    from alpha2_amd.model import ModelConfig
+    from alpha2_amd.train import TrainConfig, syntheticBatch
+    cfg = ModelConfig(**CFG, attention="reference-flash", dropout=0.2)
+    mk = lambda seed: FusedTrainer(B, cfg, TrainConfig(iters=6, seed=9), 4, seed=seed, use_graph=True)
+    a = mk(6)
+    ids = [a.add_batch(*syntheticBatch(800 + s, 4, 64, 256)) for s in range(6)]
+    for s in range(3):
+        a.step(ids[s])
+    path = str(tmp_path / "drop.alph")
+    a.saveCheckpoint(path)
+    b = mk(11)
+    idb = [b.add_batch(*syntheticBatch(800 + s, 4, 64, 256)) for s in range(6)]
+    assert b.loadCheckpoint(path)["step"] == 3
+    for s in range(3, 6):
+        a.step(ids[s])
+        b.step(idb[s])
+    for x, y in zip(a.history(3, 3), b.history(3, 3)):
+        assert abs(x.loss - y.loss) <= 1e-4 * abs(x.loss) and abs(x.gradNorm - y.gradNorm) <= 1e-3 * x.gradNorm, (x, y)
+    a.close(), b.close()
+
+
 def test_fused_step_with_a_non_finite_gradient_is_skipped_on_the_device(B):
     """The reference trainer skips the optimizer call when the loss or the gradient norm is not finite
     (trainer.ts:1248-1262,1495-1522).  The fast path takes that decision on the device: parameters, moments, the bf16
