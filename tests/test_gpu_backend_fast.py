@@ -628,6 +628,10 @@ def test_cross_entropy_is_held_until_its_backward_is_asked_for(FB):
     dict(vocabSize=33, blockSize=3, nLayer=2, nEmbd=12, nHead=3),                            # head size 4, nothing a multiple of 8
     dict(vocabSize=96, blockSize=5, nLayer=1, nEmbd=64, nHead=2),                            # 5 or 15 tokens: the weight gradients contract over them
     dict(vocabSize=50, blockSize=17, nLayer=1, nEmbd=32, nHead=1, ffnActivation="swiglu"),
+    # the reference's own attention wiring at shapes the plane products do not take (fewer than 256 rows; C not a multiple of 128):
+    # sliceQkv and the scattered sum move the data, the transposes around the slabs are still the attention kernels' strides
+    dict(vocabSize=96, blockSize=16, nLayer=2, nEmbd=64, nHead=2, attention="reference-flash"),
+    dict(vocabSize=64, blockSize=96, nLayer=1, nEmbd=192, nHead=8, attention="reference-flash"),       # (3 x 96 = 288 rows, C = 192, head size 24)
 ])
 @pytest.mark.parametrize("batch,accum", [(1, 1), (3, 2)])
 def test_shapes_the_bf16_kernels_do_not_take_run_in_f32_behind_the_interface(FB, cfg, batch, accum):
