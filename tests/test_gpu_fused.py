@@ -112,8 +112,8 @@ def test_fused_step_with_head_size_16_tracks_the_oracle(B, attention):
     ft.close()
 
 
-@pytest.mark.parametrize("accum", [1, 2])
-def test_fused_step_with_dropout_matches_oracle(B, accum):
+@pytest.mark.parametrize("accum,stream", [(1, "bf16"), (2, "bf16"), (2, "f32")])
+def test_fused_step_with_dropout_matches_oracle(B, accum, stream):
     """dropout 0.25 in the two residualDropoutAdd of every block (gpt.ts:281,332) on the reference's flash-branch wiring: masks
     from DropoutRng's counter hash (ops.ts:25-82), reseeded per step and micro-step (trainer.ts:1169,1202), made on the fly from
     a seed in device memory, so a replayed graph draws new masks every step.  Against the oracle: gradients of the first step,
@@ -124,7 +124,7 @@ def test_fused_step_with_dropout_matches_oracle(B, accum):
     cfg = dict(CFG, attention="reference-flash", dropout=0.25)
     steps = 12
     tc = dict(iters=steps, gradAccumSteps=accum, seed=77)
-    mk = lambda graph: FusedTrainer(B, ModelConfig(**cfg), TrainConfig(**tc), 4, seed=6, use_graph=graph, accum=accum)
+    mk = lambda graph: FusedTrainer(B, ModelConfig(**cfg), TrainConfig(**tc), 4, seed=6, use_graph=graph, accum=accum, stream=stream)
     ft, eager = mk(True), mk(False)
     orc = rm.Trainer(rm.ModelConfig(**cfg), rm.TrainConfig(**tc), seed=6)
     nodrop = rm.Trainer(rm.ModelConfig(**dict(cfg, dropout=0.0)), rm.TrainConfig(**tc), seed=6)
