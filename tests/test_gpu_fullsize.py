@@ -27,12 +27,12 @@ def B():
     return HipBackend(0)
 
 
-def _trainer(B, cfg, batch, accum, graph):
+def _trainer(B, cfg, batch, accum, graph, **kw):
     from alpha2_amd.fused import FusedTrainer
     from alpha2_amd.model import ModelConfig
     from alpha2_amd.train import TrainConfig
     return FusedTrainer(B, ModelConfig(**cfg), TrainConfig(iters=50, batchSize=batch, gradAccumSteps=accum), batch, seed=0,
-                        use_graph=graph, accum=accum)
+                        use_graph=graph, accum=accum, **kw)
 
 
 def _expected_initial_loss(cfg):
@@ -83,15 +83,17 @@ def test_accumulating_one_batch_four_times_equals_one_micro_step(B):
     one.close(), four.close()
 
 
-def test_gpt2_small_shape_fifty_steps_on_fresh_batches_with_loss_tracked(B):
-    """The 50-step run of the GPT-2-small-shape configuration: every step a batch it has not seen (Zipf s = 1.1 token ids),
+@pytest.mark.parametrize("attention", ["heads", "reference-flash"])
+def test_gpt2_small_shape_fifty_steps_on_fresh_batches_with_loss_tracked(B, attention):
+    """The 50-step run of the GPT-2-small-shape configuration (with multi-head attention and with the reference's own wiring): every step a batch it has not seen (Zipf s = 1.1 token ids),
     the whole step replayed from the captured graph, loss tracked on the device.  Properties that need no oracle run:
     every loss and norm is finite; graph replay equals eager execution of the same kernels at sampled steps; the loss
     falls from ln V + 0.02^2 C / 2 and its 5-step mean never rises by more than 0.05 once the warm-up is over; the learning rate follows the schedule; clipCoef * gradNorm = clip whenever the
     norm exceeds the clip."""
     from alpha2_amd.train import TrainConfig, lrAt, zipfBatches
     steps, sample = 50, (0, 1, 7, 23, 49)
-    graph, eager = _trainer(B, SMALL, 16, 1, True), _trainer(B, SMALL, 16, 1, False)
+    cfg = dict(SMALL, attention=attention)
+    graph, eager = _trainer(B, cfg, 16, 1, True, index_in_step=True), _trainer(B, cfg, 16, 1, False, index_in_step=True)
     batches = zipfBatches(4, steps, 16, 1024, 50304)                 # 50 batches cut from the one stream of seed 4
     ig = [graph.add_batch(*b) for b in batches]
     for s in range(steps):
@@ -118,6 +120,28 @@ def test_gpt2_small_shape_fifty_steps_on_fresh_batches_with_loss_tracked(B):
     # predecessors -- and a transformer learns that.  50 steps of a fresh model get well below the initial 10.98 either way.
     assert hg[-1].loss < 8.0 and min(h.loss for h in hg) > 3.0, [h.loss for h in hg]
     graph.close(), eager.close()
+
+
+def test_gpt2_small_shape_with_dropout_replays_what_eager_execution_gives(B):
+    """Dropout 0.1 at full size on the reference's wiring: the captured step reads each step's seed from device memory, so its
+    replays must give what eager execution of the same steps gives, every step with masks of its own (the loss of a step
+    replayed with the previous step's seed would differ)."""
+    from alpha2_amd.train import zipfBatches
+    steps = 6
+    cfg = dict(SMALL, attention="reference-flash", dropout=0.1)
+    graph, eager = _trainer(B, cfg, 16, 1, True), _trainer(B, cfg, 16, 1, False)
+    plain = _trainer(B, dict(cfg, dropout=0.0), 16, 1, True)
+    b = zipfBatches(4, 1, 16, 1024, 50304)[0]
+    ig, ie, ip = graph.add_batch(*b), eager.add_batch(*b), plain.add_batch(*b)
+    for _ in range(steps):                                # the SAME batch every step: only the masks change from step to step
+        graph.step(ig), eager.step(ie), plain.step(ip)
+    hg, he, hp = graph.history(0, steps), eager.history(0, steps), plain.history(0, steps)
+    assert abs(hg[0].loss - _expected_initial_loss(SMALL)) < 0.08
+    for s in range(steps):
+        assert math.isfinite(hg[s].loss) and abs(hg[s].loss - he[s].loss) <= 1e-4 * abs(he[s].loss), (s, hg[s].loss, he[s].loss)
+        assert abs(hg[s].gradNorm - he[s].gradNorm) <= 2e-3 * he[s].gradNorm
+    assert hg[-1].loss < hg[0].loss and abs(hg[-1].loss - hp[-1].loss) > 1e-4 * hp[-1].loss       # dropout did something
+    graph.close(), eager.close(), plain.close()
 
 
 @pytest.mark.parametrize("attention", ["reference-flash", "heads"])
