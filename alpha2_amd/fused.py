@@ -59,8 +59,19 @@ class StepStats:
 class FusedTrainer:
     def __init__(self, backend: HipBackend, cfg: ModelConfig, tc: TrainConfig, batch: int, seed: int = 0, use_graph: bool = True,
                  accum: int = 1, params: Optional[dict] = None, dw_groups: int = 1, stream: str = "bf16",
-                 norm_in_epilogue: bool = True, index_in_step: bool = False):
+                 norm_in_epilogue: bool = True, index_in_step: bool = False, micro_per_pass: int = 1):
         self.act = cfg.ffnActivation or "gelu"
+        # micro_per_pass = P: the `accum` micro-steps of an optimizer step (trainer.ts:1164-1273: one forward + backward each,
+        # gradients summed, the mean of their losses reported) run P at a time as one pass over P x batch sequences.  A pass's
+        # loss is the mean of its micro-steps' losses and its gradient their mean, so the step's numbers are the same; what
+        # changes is that the products of a pass have P times the rows (at 8 x 1024 rows a 256-row tile kernel has one tile per
+        # CU and nothing to overlap its epilogue with).  Batches are still stored and named one micro-batch at a time.
+        self.per_pass = int(micro_per_pass)
+        if self.per_pass < 1 or accum % self.per_pass:
+            raise ValueError(f"micro_per_pass = {micro_per_pass} must divide the {accum} micro-steps of a step")
+        self.micro_batch, self.micro_steps = batch, accum
+        batch, accum = batch * self.per_pass, accum // self.per_pass      # from here on: a pass and the number of passes
+        index_in_step = index_in_step or self.per_pass > 1         # (an index stored with one micro-batch does not cover a pass)
         # index_in_step: the scatter-add index of the token embedding's gradient (a sort of the micro-batch's ids) is built
         # inside every step, on the side stream beside the forward pass, instead of once when a batch is stored: what a loop
         # pays that feeds a new batch every step
@@ -81,6 +92,7 @@ class FusedTrainer:
         if not (8 <= self.D <= 128 and self.D % 8 == 0) or self.C % 8 or self.F % 64 or self.C % 64 or self.V % 8:
             raise ValueError("FusedTrainer needs a head size that is a multiple of 8 up to 128, nEmbd and ffnDim multiples of 64, vocab multiple of 8")
         self.BT = batch * self.T
+        self.BTm = self.micro_batch * self.T
         # Which function the attention sub-layer computes: "heads" = multi-head attention on the columns of the [BT, 3C] projection;
         # "reference-flash" = what gpt.ts:247-254 computes on a backend with flashAttention: q, k, v cut out of the projection
         # as contiguous [BT, C] matrices and re-read as [B H, T, D] slabs without a head transpose.  Here the projection writes
@@ -192,7 +204,7 @@ class FusedTrainer:
             self.proj = a(BT * Cc * 2)
             self.dproj_fc2 = [a(BT * Cc * 2) for _ in range(self.L)]
             self.dproj_wo = [a(BT * Cc * 2) for _ in range(self.L)]
-            self.seed_dev = a(4 * self.accum)
+            self.seed_dev = a(4 * self.micro_steps)
         self.loss, self.sumsq, self.clip = a(4), a(4), a(16)         # clip: coefficient (NaN = skip), norm, skipped flag
         self.loss_micro = a(4)
         self.hyper = a(ffi.C.sizeof(ffi.AhAdamW))
@@ -341,7 +353,10 @@ class FusedTrainer:
     def _dropout(self, x: int, residual: int, out: int, out_dtype: int, micro: int, counter: int):
         """out = residual + x * mask (residual 0: the mask multiply of the backward pass); x bf16, mask number `counter` of the
         micro-step (ops.ts:25-82), its seed read from device memory when the kernel runs."""
-        check(self.lib.ah_dropout_apply(x, BF16, residual, out, out_dtype, self.BT * self.C, self.seed_dev + 4 * micro, counter, self.drop))
+        n, rs = self.BTm * self.C, 4 if out_dtype == F32 else 2
+        for seg in range(self.per_pass):                              # every micro-batch of the pass with the seed of its own micro-step
+            check(self.lib.ah_dropout_apply(x + seg * n * 2, BF16, residual + seg * n * rs if residual else 0, out + seg * n * rs, out_dtype, n,
+                                            self.seed_dev + 4 * (micro * self.per_pass + seg), counter, self.drop))
 
     def _flash(self, l: int, bwd: bool):
         Cc, T, D = self.C, self.T, self.D
@@ -508,24 +523,25 @@ class FusedTrainer:
         self._optimizer()
 
     def _upload_batch(self, inputs: TensorData, targets: TensorData, ti: int, tt: int):
-        n = self.BT * 4
+        n = self.BTm * 4
         a, b = np.ascontiguousarray(inputs.data, dtype=np.int32), np.ascontiguousarray(targets.data, dtype=np.int32)
-        if a.size != self.BT or b.size != self.BT:
-            raise ValueError(f"batch must be [{self.batch}, {self.T}]")
+        if a.size != self.BTm or b.size != self.BTm:
+            raise ValueError(f"batch must be [{self.micro_batch}, {self.T}]")
         check(self.lib.ah_upload(ti, a.ctypes.data_as(C.c_void_p), n))
         check(self.lib.ah_upload(tt, b.ctypes.data_as(C.c_void_p), n))
 
     def set_batch(self, inputs: TensorData, targets: TensorData, micro: int = 0):
         """Upload one [B, T] token batch straight into the resident slot of micro-step `micro` (nothing is retained: a loop
         that feeds a fresh batch every step allocates nothing); step() trains on the resident slots until they change."""
-        self._upload_batch(inputs, targets, self.toks[micro], self.tgts[micro])
+        at = (micro % self.per_pass) * self.BTm * 4             # micro-step `micro` is slot micro % P of pass micro // P
+        self._upload_batch(inputs, targets, self.toks[micro // self.per_pass] + at, self.tgts[micro // self.per_pass] + at)
         if self._index_bytes and not self.index_in_step:
             check(self.lib.ah_embedding_index(self.toks[micro], self.BT, self.V, self.tok_index[micro]))
         self._have_batch = True
 
     def add_batch(self, inputs: TensorData, targets: TensorData) -> int:
         """Store a batch on the device for later steps (step(batch_index)); stored batches live until drop_batches()."""
-        n = self.BT * 4
+        n = self.BTm * 4
         ti, tt = self._alloc(n), self._alloc(n)
         self._upload_batch(inputs, targets, ti, tt)
         ix = 0
@@ -546,14 +562,15 @@ class FusedTrainer:
     def _use_batch(self, i, micro: int = 0):
         """Copy stored batch i into the resident slot of micro-step `micro` (a sequence fills slots 0, 1, ...)."""
         if isinstance(i, (list, tuple)):
-            if len(i) != self.accum:
-                raise ValueError(f"need {self.accum} batch indices, one per micro-step")
+            if len(i) != self.micro_steps:
+                raise ValueError(f"need {self.micro_steps} batch indices, one per micro-step")
             for m, bi in enumerate(i):
                 self._use_batch(bi, m)
             return
         ti, tt, ix = self._batches[i]
-        check(self.lib.ah_copy(self.toks[micro], ti, self.BT * 4))
-        check(self.lib.ah_copy(self.tgts[micro], tt, self.BT * 4))
+        at = (micro % self.per_pass) * self.BTm * 4
+        check(self.lib.ah_copy(self.toks[micro // self.per_pass] + at, ti, self.BTm * 4))
+        check(self.lib.ah_copy(self.tgts[micro // self.per_pass] + at, tt, self.BTm * 4))
         if ix:
             check(self.lib.ah_copy(self.tok_index[micro], ix, self._index_bytes))
         self._have_batch = True
@@ -572,8 +589,8 @@ class FusedTrainer:
         v = C.c_float(lr)
         check(self.lib.ah_upload(self.hyper, C.byref(v), 4))
         if self.drop > 0:                          # the masks of this step's micro-steps (trainer.ts:1169,1202), as int32 like `seed | 0`
-            seeds = (C.c_int32 * self.accum)(*[_i32(self.tc.seed + self.stepIdx * 1000 + m) for m in range(self.accum)])
-            check(self.lib.ah_upload(self.seed_dev, seeds, 4 * self.accum))
+            seeds = (C.c_int32 * self.micro_steps)(*[_i32(self.tc.seed + self.stepIdx * 1000 + m) for m in range(self.micro_steps)])
+            check(self.lib.ah_upload(self.seed_dev, seeds, 4 * self.micro_steps))
         return lr
 
     def step(self, batch_index=None) -> int:

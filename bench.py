@@ -110,6 +110,9 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="only the headline measurement: no backend-mode and no 350M-shape runs")
     ap.add_argument("--cpu-tokens", type=int, default=32)
     ap.add_argument("--workload", choices=sorted(WORKLOADS), default="gpt2-small")
+    ap.add_argument("--micro-per-pass", type=int, default=1,
+                    help="fast mode, workloads with accumulated micro-steps: run this many micro-steps as one pass over their micro-batches "
+                         "(FusedTrainer(micro_per_pass=...): the step's loss, gradient and update are the same numbers)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs the step on ONE GPU; --gpus must be 1 (no multi-GPU path exists in this run)", file=sys.stderr)
@@ -151,7 +154,7 @@ def main():
     else:
         from alpha2_amd.fused import FusedTrainer
         runner = FusedTrainer(B, cfg, tc, BATCH, seed=0, accum=accum, dw_groups=args.dw_groups, stream=args.stream,
-                              norm_in_epilogue=not args.norm_over_arena, index_in_step=True)
+                              norm_in_epilogue=not args.norm_over_arena, index_in_step=True, micro_per_pass=args.micro_per_pass)
         dtype = "bf16"
         ids = [runner.add_batch(x, y) for x, y in micro]                   # resident in HBM before the timed region
         cursor = [0]
@@ -209,7 +212,7 @@ def main():
         "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": f"synthetic (Zipf s=1.1 token ids, seed {tok_seed}; random-init N(0,0.02) weights, seed 0)",
         "config": {"workload": describe,
                    "tokens_per_step": tokens, "mode": args.mode, "loss_first_step": loss_first, "loss_last_step": loss_last,
-                   "attention": args.attention},
+                   "attention": args.attention, **({"micro_per_pass": args.micro_per_pass} if args.micro_per_pass != 1 else {})},
         # model flops per second against the dense bf16 MFMA peak: by the reference's (non-causal) attention count, and with
         # the causal half of the attention products only
         "step_tflops": flops / (ms * 1e-3) / 1e12, "mfu_vs_bf16_dense_peak": flops / (ms * 1e-3) / 1e12 / PEAK["bf16"],
@@ -290,6 +293,7 @@ def extra_runs(args) -> dict:
     ref, heads, big = (child("--mode", "backend", "--attention", "reference-flash"), child("--mode", "backend", "--attention", "heads"),
                        child("--workload", "gpt-350m"))
     fused_heads, big_heads = child("--attention", "heads"), child("--workload", "gpt-350m", "--attention", "heads")
+    big_pairs = child("--workload", "gpt-350m", "--micro-per-pass", "2")
     res = {"fused_step_heads_attention": {"ms_per_step": fused_heads.get("ms_per_step"),
                                           "what": "the headline step with multi-head attention on the columns of the projection instead of the reference's slabs"},
            "backend_mode": {"ms_per_step": heads.get("ms_per_step"), "ms_per_step_reference_flash": ref.get("ms_per_step"),
@@ -298,8 +302,12 @@ def extra_runs(args) -> dict:
                             "what": "generic tape-driven Trainer, one Backend call per op, on FastHipBackend with step plans; same model, batches and steps"},
            "workload_350m": {"ms_per_step": big.get("ms_per_step"), "tokens_per_s": big.get("value"), "mfu": big.get("mfu_vs_bf16_dense_peak"),
                              "ms_per_step_heads_attention": big_heads.get("ms_per_step"),
+                             # the same step with its four micro-steps run two to a pass (same loss, gradient and update:
+                             # tests/test_gpu_fullsize.py): a pass then has 16384 rows for its products instead of 8192
+                             "micro_steps_two_to_a_pass": {"ms_per_step": big_pairs.get("ms_per_step"), "tokens_per_s": big_pairs.get("value"),
+                                                           "mfu": big_pairs.get("mfu_vs_bf16_dense_peak")},
                              "what": (big.get("config") or {}).get("workload")}}
-    for k, v in (("backend_mode", heads), ("backend_mode", ref), ("workload_350m", big), ("workload_350m", big_heads),
+    for k, v in (("backend_mode", heads), ("backend_mode", ref), ("workload_350m", big), ("workload_350m", big_heads), ("workload_350m", big_pairs),
                  ("fused_step_heads_attention", fused_heads)):
         if "error" in v:
             res[k].setdefault("errors", []).append(v["error"])

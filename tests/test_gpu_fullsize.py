@@ -122,6 +122,27 @@ def test_gpt2_small_shape_fifty_steps_on_fresh_batches_with_loss_tracked(B, atte
     graph.close(), eager.close()
 
 
+def test_350m_micro_steps_in_pairs_give_the_numbers_of_four_separate_micro_steps(B):
+    """350M shape, batch 8 x 4 accumulated micro-steps: run as two passes of two micro-batches (`micro_per_pass = 2`) the step
+    must report the loss and the gradient norm of the four separate micro-steps and make their update."""
+    from alpha2_amd.train import zipfBatches
+    steps = 3
+    four, pairs = _trainer(B, M350, 8, 4, True), _trainer(B, M350, 8, 4, True, micro_per_pass=2)
+    batches = zipfBatches(5, 4 * steps, 8, 1024, 50304)
+    i4, ip = [four.add_batch(*b) for b in batches], [pairs.add_batch(*b) for b in batches]
+    for s in range(steps):
+        four.step(i4[4 * s:4 * s + 4])
+        pairs.step(ip[4 * s:4 * s + 4])
+    h4, hp = four.history(0, steps), pairs.history(0, steps)
+    assert abs(h4[0].loss - _expected_initial_loss(M350)) < 0.08
+    for s in range(steps):
+        assert abs(h4[s].loss - hp[s].loss) <= 2e-5 * abs(h4[s].loss), (s, h4[s].loss, hp[s].loss)
+        assert abs(h4[s].gradNorm - hp[s].gradNorm) <= 2e-3 * h4[s].gradNorm, (s, h4[s].gradNorm, hp[s].gradNorm)
+    for pname in ("wte", "layer.23.attn.wqkv", "layer.0.mlp.fc2", "lmHead", "lnF.weight"):
+        assert np.max(np.abs(four.param(pname) - pairs.param(pname))) <= 2.5 * steps * 3e-4, pname
+    four.close(), pairs.close()
+
+
 def test_gpt2_small_shape_with_dropout_replays_what_eager_execution_gives(B):
     """Dropout 0.1 at full size on the reference's wiring: the captured step reads each step's seed from device memory, so its
     replays must give what eager execution of the same steps gives, every step with masks of its own (the loss of a step

@@ -199,6 +199,42 @@ def test_fused_gradient_accumulation_matches_oracle(B, attention):
     ft.close(), eager.close()
 
 
+@pytest.mark.parametrize("dropout", [0.0, 0.2])
+@pytest.mark.parametrize("K,P", [(2, 2), (4, 2), (4, 4)])
+def test_micro_steps_run_several_to_a_pass_give_the_numbers_of_one_at_a_time(B, K, P, dropout):
+    """`micro_per_pass`: the K micro-steps of a step (trainer.ts:1164-1273) run P at a time as one pass over P micro-batches.  The
+    reported loss (mean of the micro-step losses), the gradient norm and the update must be those of the oracle's K separate
+    micro-steps -- with dropout too, every micro-batch of a pass drawing the masks of its own micro-step (trainer.ts:1202) --
+    and those of the same trainer running them one at a time."""
+    from alpha2_amd.fused import FusedTrainer
+    from alpha2_amd.model import ModelConfig
+    from alpha2_amd.train import TrainConfig, syntheticBatch
+    cfg = dict(CFG, attention="reference-flash", dropout=dropout)
+    steps = 5
+    tc = dict(iters=steps, gradAccumSteps=K, seed=21)
+    mk = lambda per, graph: FusedTrainer(B, ModelConfig(**cfg), TrainConfig(**tc), 4, seed=8, use_graph=graph, accum=K, micro_per_pass=per)
+    merged, eager, single = mk(P, True), mk(P, False), mk(1, True)
+    assert (merged.batch, merged.accum, merged.micro_steps) == (4 * P, K // P, K)
+    orc = rm.Trainer(rm.ModelConfig(**cfg), rm.TrainConfig(**tc), seed=8)
+    for s in range(steps):
+        seeds = [500 + K * s + m for m in range(K)]
+        ids = [[t.add_batch(*syntheticBatch(sd, 4, 64, 256)) for sd in seeds] for t in (merged, eager, single)]
+        for t, i in zip((merged, eager, single), ids):
+            t.step(i)
+        o = orc.step([rm.synthetic_batch(sd, 4, 64, 256) for sd in seeds])
+        hm, he, h1 = (t.history(s, 1)[0] for t in (merged, eager, single))
+        assert abs(hm.loss - o.loss) <= 2e-2 * abs(o.loss) and abs(hm.gradNorm - o.gradNorm) <= 4e-2 * o.gradNorm, (s, hm, o.loss, o.gradNorm)
+        assert abs(hm.loss - h1.loss) <= 2e-3 * abs(h1.loss) and abs(hm.gradNorm - h1.gradNorm) <= 1e-2 * h1.gradNorm, (s, hm, h1)
+        assert hm.loss == he.loss and hm.gradNorm == he.gradNorm, (s, hm, he)
+    for name in ("wte", "layer.1.attn.wqkv", "layer.0.mlp.fc2", "lmHead"):
+        assert np.max(np.abs(merged.param(name) - single.param(name))) <= 2.5 * steps * 3e-4, name      # (AdamW moves an entry by about lr per step)
+    with pytest.raises(ValueError, match="one per micro-step"):
+        merged.step([0] * (K - 1))
+    with pytest.raises(ValueError, match="must divide"):
+        FusedTrainer(B, ModelConfig(**cfg), TrainConfig(**tc), 4, accum=K, micro_per_pass=3)
+    merged.close(), eager.close(), single.close()
+
+
 def test_fused_checkpoint_resume(B, tmp_path):
     """The fast path writes and reads the same file format; a resumed run (graph captured after the load) follows the
     uninterrupted one, and the generic trainer accepts the file too."""
