@@ -111,6 +111,15 @@ def bench_gemm(b: Bench):
                 ms = b.time(lambda: ffi.check(b.lib.ah_gemm(C.byref(d))))
                 kern, nsplit = b.B.lastGemmKernel()
                 b.record(f"gemm {dname} N={N} {label}", ms, flops=flops, dtype=dname, note=f"{kern}" + (f" split-K x{nsplit}" if nsplit > 1 else ""))
+            if dt == ffi.BF16 and N == 2304:
+                # the fused q, k, v projection under the reference's attention wiring (gpt.ts:239-254): result columns / the
+                # contraction in three planes instead of sliceQkv's copies and the written sum of three scatterSlice results
+                d = ffi.AhGemm(ffi.GEMM_NT, dt, dt, ffi.EPI_NONE, M, N, K, K, K, K, 1, 0, 0, 0, a, w, c_fwd, 0)
+                ms = b.time(lambda: ffi.check(b.lib.ah_gemm_planes(C.byref(d), K, M * K, 0, 0, 0)))
+                b.record("gemm bf16 N=2304 fwd, q k v as planes", ms, flops=flops, dtype=dname, note=b.B.lastGemmKernel()[0])
+                d2 = ffi.AhGemm(ffi.GEMM_NN, dt, dt, ffi.EPI_NONE, M, K, N, K, K, K, 1, 0, 0, 0, g, w, c_da, 0)
+                ms = b.time(lambda: ffi.check(b.lib.ah_gemm_planes(C.byref(d2), 0, 0, K, M * K, 0)))
+                b.record("gemm bf16 N=2304 dA, dq dk dv as planes", ms, flops=flops, dtype=dname, note=b.B.lastGemmKernel()[0])
             b.release()
 
 
@@ -192,6 +201,13 @@ def bench_bandwidth(b: Bench):
     shp = ffi.shape_arr([16, 12, 1024, 32])
     ms = b.time(lambda: ffi.check(lib.ah_transpose(q16[0], tr, 4, shp, 1, 2)))
     b.record("transpose [16,12,1024,64] bf16, dims 1 and 2", ms, nbytes=rows * dim * 4, note="heads <-> positions, 128-byte rows kept whole")
+    # residualDropoutAdd and the mask multiply of its backward with the mask made on the fly (no mask tensor): bf16 stream
+    seed = b.alloc(4)
+    ffi.check(lib.ah_fill_i32(seed, 42, 1))
+    ms = b.time(lambda: ffi.check(lib.ah_dropout_apply(q16[0], ffi.BF16, q16[1], q16[2], ffi.BF16, rows * dim, seed, 3, 0.1)))
+    b.record("dropout: residual + x * mask 16384x768 bf16", ms, nbytes=rows * dim * 6, note="mask from the counter hash, seed in device memory")
+    ms = b.time(lambda: ffi.check(lib.ah_dropout_apply(q16[0], ffi.BF16, 0, q16[2], ffi.BF16, rows * dim, seed, 3, 0.1)))
+    b.record("dropout: x * mask 16384x768 bf16", ms, nbytes=rows * dim * 4)
     b.release()
 
     h = b.randn(rows * F, ffi.F32)
