@@ -23,6 +23,7 @@
 #include "attention_common.h"
 #include <cstdlib>
 #include <cstring>
+#include <type_traits>
 
 using namespace ah;
 
@@ -324,6 +325,13 @@ __device__ __forceinline__ void flash_dq_bf16_body(const FlashArgs &a) {
   bf16x8 qf[KS], dof[KS];
   row_frags<D, PAD>(Q, a.q_st, qi, live, lane, qf, a.hd);
   row_frags<D, PAD>(dO, a.o_st, qi, live, lane, dof, a.hd);
+  // the first key tile is asked for before delta is worked out, so that the two waits for memory are one
+  u32x4 rk[Geo<D>::CHUNKS], rv[Geo<D>::CHUNKS];
+  auto load_tile = [&](int row0) {
+    tile_load<D, PAD>(K, a.k_st, row0, a.T, rk, a.hd);
+    tile_load<D, PAD>(V, a.v_st, row0, a.T, rv, a.hd);
+  };
+  load_tile(0);
   int64_t srow = ((int64_t)b * a.H + h) * a.T + qi;
   // delta = rowsum(dO * O): each half-wave holds half of the row's features; also published for the dK/dV kernel
   float delta = 0.f;
@@ -346,18 +354,87 @@ __device__ __forceinline__ void flash_dq_bf16_body(const FlashArgs &a) {
 
   int kv_end = min(a.T, (qblk + 1) * 128);
   int ntile = (kv_end + ST - 1) / ST;
-  u32x4 rk[Geo<D>::CHUNKS], rv[Geo<D>::CHUNKS];
-  tile_load<D, PAD>(K, a.k_st, 0, a.T, rk, a.hd);
-  tile_load<D, PAD>(V, a.v_st, 0, a.T, rv, a.hd);
   tile_store<D>(Ks[0], rk);
   tile_store<D>(Vs[0], rv);
   __syncthreads();
-  for (int it = 0; it < ntile; it++) {
-    int cur = it & 1;
-    if (it + 1 < ntile) {
-      tile_load<D, PAD>(K, a.k_st, (it + 1) * ST, a.T, rk, a.hd);
-      tile_load<D, PAD>(V, a.v_st, (it + 1) * ST, a.T, rv, a.hd);
+  int it = 0;
+  // The key tiles that lie wholly below the diagonal of every wave of the block (no masking, no wave skips any) run as a
+  // software pipeline inside each wave: while the vector unit works through the scores of one 32 x 32 sub-tile, the matrix
+  // pipe computes S and dP of the next one, and dQ of a sub-tile is accumulated a step later, from K^T fragments read while
+  // its tile was current.  One wave issues in order, so the products are placed between groups of scores by hand
+  // (sched_barrier keeps the compiler from regrouping them): a dependent MFMA never waits for its predecessor with the
+  // vector unit idle, which is what two waves per SIMD could not cover in the tile-at-a-time loop below.
+  if constexpr (D <= 64) {
+    const int n_full = min(ntile, 2 * qblk);
+    if (n_full > 0) {
+      constexpr int SC = 16 / KS;                                  // scores of the previous sub-tile behind each pair of products
+      f32x16 sA, dpA, sB, dpB, zero16, negd;
+      bf16x8 ktA[2][DB], ktB[2][DB];
+#pragma unroll
+      for (int e = 0; e < 16; e++) { zero16[e] = 0.f; negd[e] = -delta; }
+      auto scores = [&](f32x16 &sp, f32x16 &dpp, int e0) {
+#pragma unroll
+        for (int e = e0; e < e0 + SC; e++) {
+          float ds;
+          score_bwd<CAPPED>(sp[e], dpp[e], krow, c1, c2, ds);
+          sp[e] = ds;
+        }
+      };
+      // products of sub-tile (cur, sub) into (sn, dpn, ktn); scores and dQ of the previous sub-tile (sp, dpp, ktp)
+      auto step = [&](auto have_prev, int cur, int sub, f32x16 &sn, f32x16 &dpn, bf16x8 (&ktn)[2][DB], f32x16 &sp, f32x16 &dpp, bf16x8 (&ktp)[2][DB]) {
+        constexpr bool PREV = decltype(have_prev)::value;
+        bf16x8 kfr[KS], vfr[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) { kfr[ks] = tile_frag<D>(Ks[cur], sub * 32, ks, lane); vfr[ks] = tile_frag<D>(Vs[cur], sub * 32, ks, lane); }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+          if constexpr (PREV) scores(sp, dpp, ks * SC);
+          __builtin_amdgcn_sched_barrier(0);
+          sn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfr[ks], qf[ks], ks == 0 ? zero16 : sn, 0, 0, 0);
+          dpn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfr[ks], dof[ks], ks == 0 ? negd : dpn, 0, 0, 0);       // dP - delta
+          if constexpr (PREV) if ((ks + 1) * SC == 8 + SC) {       // scores 0..7 were finished one group ago
+            bf16x8 b0 = acc_to_b(sp, 0);
+#pragma unroll
+            for (int d = 0; d < DB; d++) dq[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ktp[0][d], b0, dq[d], 0, 0, 0);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        if constexpr (PREV) {
+          bf16x8 b1 = acc_to_b(sp, 1);
+#pragma unroll
+          for (int d = 0; d < DB; d++) dq[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ktp[1][d], b1, dq[d], 0, 0, 0);
+        }
+#pragma unroll
+        for (int m = 0; m < 2; m++)
+#pragma unroll
+          for (int d = 0; d < DB; d++) ktn[m][d] = tile_frag_t<D>(Ks[cur], sub * 32, m, d, lane);
+        __builtin_amdgcn_sched_barrier(0);
+      };
+      for (; it < n_full; it++) {
+        int cur = it & 1;
+        load_tile((it + 1) * ST);                                   // it + 1 < ntile: the diagonal tiles follow
+        if (it == 0) step(std::false_type{}, cur, 0, sA, dpA, ktA, sB, dpB, ktB);
+        else step(std::true_type{}, cur, 0, sA, dpA, ktA, sB, dpB, ktB);
+        step(std::true_type{}, cur, 1, sB, dpB, ktB, sA, dpA, ktA);
+        tile_store<D>(Ks[cur ^ 1], rk);
+        tile_store<D>(Vs[cur ^ 1], rv);
+        __syncthreads();
+      }
+      // the last sub-tile's scores and dQ
+#pragma unroll
+      for (int g = 0; g < KS; g++) scores(sB, dpB, g * SC);
+      bf16x8 b0 = acc_to_b(sB, 0), b1 = acc_to_b(sB, 1);
+#pragma unroll
+      for (int d = 0; d < DB; d++) {
+        dq[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ktB[0][d], b0, dq[d], 0, 0, 0);
+        dq[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ktB[1][d], b1, dq[d], 0, 0, 0);
+      }
     }
+  }
+  for (; it < ntile; it++) {
+    int cur = it & 1;
+    if (it + 1 < ntile) load_tile((it + 1) * ST);
 #pragma unroll
     for (int sub = 0; sub < ST / 32; sub++) {
       int kv0 = it * ST + sub * 32;
