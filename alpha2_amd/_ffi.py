@@ -135,6 +135,7 @@ SIGNATURES = {
     "ah_gemm_grouped_destroy": [u64],
     "ah_gemm_last_kernel": [C.c_char_p, C.c_int32, C.POINTER(C.c_int32)],
     "ah_probe_mfma_bf16": [i32, i32, i32, C.POINTER(C.c_double)],
+    "ah_probe_issue": [i32, i32, i32, C.POINTER(C.c_double)],
     "ah_flash_fwd": [C.POINTER(AhFlash)], "ah_flash_bwd": [C.POINTER(AhFlash)],
     "ah_adamw": [u64, u64, u64, u64, u64, C.POINTER(AhAdamW), u64, u64, u64],
     "ah_clip_coef": [u64, f32, f32, u64],

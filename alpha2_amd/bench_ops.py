@@ -1,7 +1,7 @@
 """Per-op microbenchmarks on the shapes of the training step, in the manner of the reference's scripts/bench-ops.ts
 (3 warm-up calls, then the mean of `iters` calls; TFLOP/s = flops / time, GB/s = algorithmic bytes / time):
 
-    python -m alpha2_amd.bench_ops [--iters 10] [--only gemm|flash|bandwidth|ceiling|epilogue] [--json]
+    python -m alpha2_amd.bench_ops [--iters 10] [--only gemm|flash|bandwidth|ceiling|epilogue|issue] [--json]
 
 * GEMM: C = A B^T and both backward products, M = 16384 (batch x context), K = 768, N in {768, 2304, 3072, 50304},
   bf16 operands with fp32 accumulation and fp32 throughout; flops 2 M N K (scripts/bench-ops.ts:302,328).
@@ -15,6 +15,9 @@
   cross-entropy forward + backward, embedding gather / scatter-add, sum of squares, AdamW; bytes = the algorithmic minimum.
 * The matrix pipes alone (`ah_probe_mfma_bf16`: independent 32x32x16 bf16 MFMAs on registers, no memory traffic), on zeros and
   on operands whose bits toggle, for one short launch and sustained: what the part's power limit leaves of the published peak.
+* `--only issue` (not part of the default run): what one SIMD issues per nanosecond (`ah_probe_issue`: v_fma_f32, v_exp_f32, a
+  mix of the two, an MFMA alone and with vector work behind it, at one, two and four waves per SIMD): the figures the
+  attention kernels, whose time goes to per-score vector instructions, are read against.
 
 Every call goes through the C ABI; timing is by HIP events on the library's stream.  Peaks used for the last column:
 2.5 PFLOP/s (bf16 MFMA), 157.3 TFLOP/s (fp32 MFMA), 8 TB/s (HBM).
@@ -298,13 +301,42 @@ def bench_ceiling(b: Bench):
     b.release()
 
 
+def bench_issue(b: Bench):
+    """Time per group of instructions on one SIMD (`ah_probe_issue`), by how many waves share the SIMD."""
+    lib = b.lib
+    n = C.c_double()
+    kinds = ((0, "v_fma_f32"), (1, "v_exp_f32"), (2, "v_exp_f32 + 3 v_fma_f32"), (3, "mfma 32x32x16 bf16"),
+             (4, "mfma 32x32x16 bf16 + 8 v_fma_f32"), (5, "mfma 32x32x16 bf16 + 16 v_fma_f32"))
+    print(f"{'group of instructions':40s} {'waves/SIMD':>10s} {'ns per group per SIMD':>22s}")
+    for kind, name in kinds:
+        for waves in ((1, 2, 4) if kind < 3 else (1, 2)):
+            ffi.check(lib.ah_probe_issue(kind, waves, 100, C.byref(n)))          # (first launch of a kernel: code upload)
+            ffi.check(lib.ah_sync())
+            e0, e1 = b.B._event(), b.B._event()
+            ffi.check(lib.ah_event_record(e0))
+            ffi.check(lib.ah_probe_issue(kind, waves, 20000, C.byref(n)))
+            ffi.check(lib.ah_event_record(e1))
+            ms = C.c_float()
+            ffi.check(lib.ah_event_elapsed_ms(e0, e1, C.byref(ms)))
+            for e in (e0, e1):
+                ffi.check(lib.ah_event_destroy(e))
+            ns = ms.value * 1e6 / n.value
+            b.rows.append({"op": f"issue: {name}", "waves_per_simd": waves, "ns_per_group": ns})
+            print(f"{name:40s} {waves:10d} {ns:22.2f}", flush=True)
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser(description=__doc__.split("\n")[0])
     ap.add_argument("--iters", type=int, default=10)
-    ap.add_argument("--only", choices=["gemm", "flash", "bandwidth", "ceiling", "epilogue"])
+    ap.add_argument("--only", choices=["gemm", "flash", "bandwidth", "ceiling", "epilogue", "issue"])
     ap.add_argument("--json", action="store_true", help="also print one JSON line with every row")
     args = ap.parse_args(argv)
     b = Bench(args.iters)
+    if args.only == "issue":
+        bench_issue(b)
+        if args.json:
+            print(json.dumps(b.rows))
+        return 0
     print(f"{'op':34s} {'time':>13s} {'rate':>16s} {'peak':>7s}")
     for name, fn in (("gemm", bench_gemm), ("flash", bench_flash), ("bandwidth", bench_bandwidth), ("ceiling", bench_ceiling)):
         if args.only in (None, name):

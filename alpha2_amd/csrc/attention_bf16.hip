@@ -49,6 +49,9 @@ bool flash_bwd_one_pass() {
 
 __device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float rcp_fast(float x) { return __builtin_amdgcn_rcpf(x); }
+// First statement of a block that only the tiles on the diagonal need (masking): with it the compiler keeps the block behind a
+// branch the other tiles skip, where it would otherwise turn a cheap block into selects that every tile executes.
+__device__ __forceinline__ void keep_branch() { asm volatile("; rare path" ::: "memory"); }
 
 // global -> registers: rows [row0, row0+64) of a [T][D] operand with row stride st (elements); rows >= T read as zero
 // (PAD: the tensors' head size hd is smaller than D; features hd .. D - 1 read as zero)
@@ -226,15 +229,17 @@ __device__ __forceinline__ void flash_fwd_bf16_body(const FlashArgs &a) {
         } else {
           float tmax = -INFINITY;
 #pragma unroll
-          for (int e = 0; e < 16; e++) {
-            float x = s[e] * c1;
-            if (edge) {
+          for (int e = 0; e < 16; e++) s[e] *= c1;
+          if (edge) {
+            keep_branch();
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
               int kv = kv0 + 8 * (e >> 2) + 4 * lk + (e & 3);
-              x = (kv > qi || kv >= a.T) ? -INFINITY : x;
+              s[e] = (kv > qi || kv >= a.T) ? -INFINITY : s[e];
             }
-            s[e] = x;
-            tmax = fmaxf(tmax, x);
           }
+#pragma unroll
+          for (int e = 0; e < 16; e++) tmax = fmaxf(tmax, s[e]);
           tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
           float m_new = fmaxf(m, tmax);
           float m_use = m_new == -INFINITY ? 0.f : m_new;

@@ -43,7 +43,67 @@ __global__ __launch_bounds__(256) void k_probe_mfma_bf16(float *out, int iters) 
     for (int e = 0; e < 16; e++) s += c[j][e];
   if (s == 12345.678f) out[threadIdx.x & 63] = s;
 }
+
+// Issue rates of one SIMD.  Every wave runs `iters` x 32 groups of instructions on eight independent register chains (no
+// memory traffic, the guarded store is never taken); a group is KIND 0: one v_fma_f32, 1: one v_exp_f32, 2: one v_exp_f32 and
+// three v_fma_f32, 3: one 32x32x16 bf16 MFMA (two accumulators alternate), 4 / 5: that MFMA followed by 8 / 16 v_fma_f32.
+// Inline assembly, so that the compiler neither merges nor reorders what is being timed.
+template <int KIND>
+__global__ __launch_bounds__(1024) void k_probe_issue(float *out, int iters, float a, float b) {
+  float x[8];
+#pragma unroll
+  for (int i = 0; i < 8; i++) x[i] = 0.001f * (float)(threadIdx.x + i);
+  f32x16 acc0, acc1;
+  bf16x8 fa, fb;
+#pragma unroll
+  for (int e = 0; e < 16; e++) { acc0[e] = 0.f; acc1[e] = 0.f; }
+#pragma unroll
+  for (int i = 0; i < 8; i++) { fa[i] = (__bf16)(0.01f * (float)(threadIdx.x & 63)); fb[i] = (__bf16)(0.02f * (float)i); }
+  for (int it = 0; it < iters; it++) {
+#pragma unroll
+    for (int g = 0; g < 32; g++) {
+      if (KIND == 0) asm volatile("v_fma_f32 %0, %0, %1, %2" : "+v"(x[g & 7]) : "v"(a), "v"(b));
+      if (KIND == 1 || KIND == 2) asm volatile("v_exp_f32 %0, %0" : "+v"(x[g & 7]));
+      if (KIND == 2) {
+#pragma unroll
+        for (int i = 1; i < 4; i++) asm volatile("v_fma_f32 %0, %0, %1, %2" : "+v"(x[(g + 2 * i) & 7]) : "v"(a), "v"(b));
+      }
+      if (KIND >= 3) {
+        if (g & 1) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc1) : "v"(fa), "v"(fb));
+        else asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc0) : "v"(fa), "v"(fb));
+#pragma unroll
+        for (int i = 0; i < (KIND == 4 ? 8 : KIND == 5 ? 16 : 0); i++) asm volatile("v_fma_f32 %0, %0, %1, %2" : "+v"(x[i & 7]) : "v"(a), "v"(b));
+      }
+    }
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; i++) s += x[i];
+#pragma unroll
+  for (int e = 0; e < 16; e++) s += acc0[e] + acc1[e];
+  if (s == 12345.678f) out[threadIdx.x & 63] = s;
+}
 }  // namespace
+
+extern "C" int32_t ah_probe_issue(int32_t kind, int32_t waves_per_simd, int32_t iters, double *groups_per_simd_out) {
+  AH_REQUIRE_READY();
+  AH_ARG(kind >= 0 && kind <= 5 && waves_per_simd >= 1 && waves_per_simd <= (kind >= 3 ? 2 : 4) && iters >= 1 && iters <= 200000,
+         "ah_probe_issue: kind 0-5, 1-4 waves per SIMD (1-2 with an MFMA in the group), 1-200000 iterations");
+  float *out = (float *)scratch(256);
+  if (out == nullptr) return fail(AH_ERR_OOM, "ah_probe_issue: no scratch");
+  const dim3 grid((unsigned)num_cus()), block((unsigned)(256 * waves_per_simd));       // one workgroup per CU, its waves spread over the four SIMDs
+  switch (kind) {
+    case 0: ah::launch_kernel(k_probe_issue<0>, grid, block, 0, out, (int)iters, 0.999f, 0.001f); break;
+    case 1: ah::launch_kernel(k_probe_issue<1>, grid, block, 0, out, (int)iters, 0.999f, 0.001f); break;
+    case 2: ah::launch_kernel(k_probe_issue<2>, grid, block, 0, out, (int)iters, 0.999f, 0.001f); break;
+    case 3: ah::launch_kernel(k_probe_issue<3>, grid, block, 0, out, (int)iters, 0.999f, 0.001f); break;
+    case 4: ah::launch_kernel(k_probe_issue<4>, grid, block, 0, out, (int)iters, 0.999f, 0.001f); break;
+    default: ah::launch_kernel(k_probe_issue<5>, grid, block, 0, out, (int)iters, 0.999f, 0.001f); break;
+  }
+  AH_LAUNCH_CHECK();
+  if (groups_per_simd_out) *groups_per_simd_out = (double)iters * 32.0 * waves_per_simd;
+  return AH_OK;
+}
 
 extern "C" int32_t ah_probe_mfma_bf16(int32_t waves_per_simd, int32_t iters, int32_t random_operands, double *flops_out) {
   AH_REQUIRE_READY();

@@ -411,6 +411,14 @@ int32_t ah_gemm_last_kernel(char *name, int32_t capacity, int32_t *nsplit);
  * dense peak, with operands whose bits toggle at what its power limit sustains, which is the ceiling a GEMM on real data
  * can be read against. */
 int32_t ah_probe_mfma_bf16(int32_t waves_per_simd, int32_t iters, int32_t random_operands, double *flops_out);
+/* Measurement aid (no counterpart in the reference): ONE launch in which every SIMD of the device runs waves_per_simd waves that
+ * each issue iters (1-200000) x 32 groups of instructions on registers (no memory traffic).  kind 0: a group is one v_fma_f32;
+ * 1: one v_exp_f32; 2: one v_exp_f32 and three v_fma_f32; 3: one 32x32x16 bf16 MFMA; 4 / 5: that MFMA followed by 8 / 16
+ * v_fma_f32.  waves_per_simd 1-4 (1-2 with an MFMA in the group).  *groups_per_simd_out (host, may be null) = groups issued on
+ * each SIMD.  Timed by the caller with ah_event_*: the time per group says what one wave alone can issue, what several waves
+ * issue together, and how much of the vector work fits beside an MFMA -- the figures the attention kernels, which are bound
+ * by per-score vector instructions, are read against. */
+int32_t ah_probe_issue(int32_t kind, int32_t waves_per_simd, int32_t iters, double *groups_per_simd_out);
 
 /* ---- fused causal flash attention.  Backend.flashAttention / flashAttentionBackward
  *      (interfaces.ts:127-135; kernel semantics packages/helios/src/kernels/attention.ts:1-586):

@@ -80,6 +80,7 @@ export const lib = dlopen(process.env.ALPHA_HIP_LIB ?? "libalpha_hip.so", {
   ah_lion:                         { args: [u64, u64, u64, u64, ptr], returns: i32 },
   ah_masked_fill:                  { args: [u64, u64, u64, u64, u64, f32], returns: i32 },
   ah_pos_embedding_bwd:            { args: [u64, u64, i64, i64, i64, i32], returns: i32 },
+  ah_probe_issue:                  { args: [i32, i32, i32, ptr], returns: i32 },
   ah_probe_mfma_bf16:              { args: [i32, i32, i32, ptr], returns: i32 },
   ah_reset_op_count:               { args: [], returns: i32 },
   ah_residual_dropout_add:         { args: [u64, u64, u64, u64, u64], returns: i32 },

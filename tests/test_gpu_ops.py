@@ -1622,6 +1622,23 @@ def test_mfma_probe_runs_and_refuses_sizes_outside_its_range(B):
     assert B.lib.ah_probe_mfma_bf16(1, 200001, 1, None) != 0
 
 
+def test_issue_probe_runs_and_refuses_sizes_outside_its_range(B):
+    """The issue-rate aid launches and finishes for every kind of group (every wave runs a counted loop), reports the groups
+    issued per SIMD, and refuses kinds, wave counts and iteration counts beyond its stated range."""
+    import ctypes as C
+    from alpha2_amd import _ffi as ffi
+    n = C.c_double()
+    for kind in range(6):
+        for waves in ((1, 4) if kind < 3 else (1, 2)):
+            ffi.check(B.lib.ah_probe_issue(kind, waves, 20, C.byref(n)))
+            assert n.value == 20 * 32 * waves
+    ffi.check(B.lib.ah_sync())
+    assert B.lib.ah_probe_issue(6, 1, 20, None) != 0 and b"kind 0-5" in B.lib.ah_last_error()
+    assert B.lib.ah_probe_issue(3, 3, 20, None) != 0
+    assert B.lib.ah_probe_issue(0, 5, 20, None) != 0
+    assert B.lib.ah_probe_issue(0, 1, 200001, None) != 0
+
+
 def test_the_extras_the_trainer_calls_on_a_gpu_backend(B):
     """resetStepOps / gpuOpsThisStep and purgeBufferPools, which the reference trainer calls when the backend has them
     (trainer.ts:1003-1032,1915,1956): the launch counter restarts and counts, and purging the pool frees every cached block
