@@ -23,7 +23,6 @@
 #include "attention_common.h"
 #include <cstdlib>
 #include <cstring>
-#include <type_traits>
 
 using namespace ah;
 
@@ -290,10 +289,10 @@ __global__ __launch_bounds__(256, D <= 64 ? 3 : 1) void k_flash_fwd_bf16(FlashAr
 template <int D, bool CAPPED>
 __global__ __launch_bounds__(256, D <= 64 ? 3 : 1) void k_flash_fwd_bf16_padded(FlashArgs a) { flash_fwd_bf16_body<D, CAPPED, true>(a); }
 
-// Per-score backward arithmetic shared by the dQ and dK/dV kernels.  s = raw q.k, dpd = dO.v - delta (the dP accumulator
-// starts at -delta = -rowsum(dO*O), so the subtraction rides on the MFMA), krow = (max - lse) in base 2 (max = cap when
-// CAPPED, else 0).  Returns p and writes ds WITHOUT the constant factor (scale, and 4 for tanh' when CAPPED), which the
-// caller applies to its accumulators once.
+// Per-score backward arithmetic shared by the dQ and dK/dV kernels.  s = raw q.k, dpd = dO.v - delta with delta =
+// rowsum(dO*O) (in dK/dV the dP accumulator starts at -delta, so the subtraction rides on the MFMA; dQ subtracts it per score),
+// krow = (max - lse) in base 2 (max = cap when CAPPED, else 0).  Returns p and writes ds WITHOUT the constant factor (scale,
+// and 4 for tanh' when CAPPED), which the caller applies to its accumulators once.
 template <bool CAPPED>
 __device__ __forceinline__ float score_bwd(float s, float dpd, float krow, float c1, float c2, float &ds) {
   float p;
@@ -332,11 +331,8 @@ __device__ __forceinline__ void flash_dq_bf16_body(const FlashArgs &a) {
   row_frags<D, PAD>(dO, a.o_st, qi, live, lane, dof, a.hd);
   // the first key tile is asked for before delta is worked out, so that the two waits for memory are one
   u32x4 rk[Geo<D>::CHUNKS], rv[Geo<D>::CHUNKS];
-  auto load_tile = [&](int row0) {
-    tile_load<D, PAD>(K, a.k_st, row0, a.T, rk, a.hd);
-    tile_load<D, PAD>(V, a.v_st, row0, a.T, rv, a.hd);
-  };
-  load_tile(0);
+  tile_load<D, PAD>(K, a.k_st, 0, a.T, rk, a.hd);
+  tile_load<D, PAD>(V, a.v_st, 0, a.T, rv, a.hd);
   int64_t srow = ((int64_t)b * a.H + h) * a.T + qi;
   // delta = rowsum(dO * O): each half-wave holds half of the row's features; also published for the dK/dV kernel
   float delta = 0.f;
@@ -362,91 +358,19 @@ __device__ __forceinline__ void flash_dq_bf16_body(const FlashArgs &a) {
   tile_store<D>(Ks[0], rk);
   tile_store<D>(Vs[0], rv);
   __syncthreads();
-  int it = 0;
-  // The key tiles that lie wholly below the diagonal of every wave of the block (no masking, no wave skips any) run as a
-  // software pipeline inside each wave: while the vector unit works through the scores of one 32 x 32 sub-tile, the matrix
-  // pipe computes S and dP of the next one, and dQ of a sub-tile is accumulated a step later, from K^T fragments read while
-  // its tile was current.  One wave issues in order, so the products are placed between groups of scores by hand
-  // (sched_barrier keeps the compiler from regrouping them): a dependent MFMA never waits for its predecessor with the
-  // vector unit idle, which is what two waves per SIMD could not cover in the tile-at-a-time loop below.
-  if constexpr (D <= 64) {
-    const int n_full = min(ntile, 2 * qblk);
-    if (n_full > 0) {
-      constexpr int SC = 16 / KS;                                  // scores of the previous sub-tile behind each pair of products
-      f32x16 sA, dpA, sB, dpB, zero16, negd;
-      bf16x8 ktA[2][DB], ktB[2][DB];
-#pragma unroll
-      for (int e = 0; e < 16; e++) { zero16[e] = 0.f; negd[e] = -delta; }
-      auto scores = [&](f32x16 &sp, f32x16 &dpp, int e0) {
-#pragma unroll
-        for (int e = e0; e < e0 + SC; e++) {
-          float ds;
-          score_bwd<CAPPED>(sp[e], dpp[e], krow, c1, c2, ds);
-          sp[e] = ds;
-        }
-      };
-      // products of sub-tile (cur, sub) into (sn, dpn, ktn); scores and dQ of the previous sub-tile (sp, dpp, ktp)
-      auto step = [&](auto have_prev, int cur, int sub, f32x16 &sn, f32x16 &dpn, bf16x8 (&ktn)[2][DB], f32x16 &sp, f32x16 &dpp, bf16x8 (&ktp)[2][DB]) {
-        constexpr bool PREV = decltype(have_prev)::value;
-        bf16x8 kfr[KS], vfr[KS];
-#pragma unroll
-        for (int ks = 0; ks < KS; ks++) { kfr[ks] = tile_frag<D>(Ks[cur], sub * 32, ks, lane); vfr[ks] = tile_frag<D>(Vs[cur], sub * 32, ks, lane); }
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int ks = 0; ks < KS; ks++) {
-          if constexpr (PREV) scores(sp, dpp, ks * SC);
-          __builtin_amdgcn_sched_barrier(0);
-          sn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfr[ks], qf[ks], ks == 0 ? zero16 : sn, 0, 0, 0);
-          dpn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfr[ks], dof[ks], ks == 0 ? negd : dpn, 0, 0, 0);       // dP - delta
-          if constexpr (PREV) if ((ks + 1) * SC == 8 + SC) {       // scores 0..7 were finished one group ago
-            bf16x8 b0 = acc_to_b(sp, 0);
-#pragma unroll
-            for (int d = 0; d < DB; d++) dq[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ktp[0][d], b0, dq[d], 0, 0, 0);
-          }
-          __builtin_amdgcn_sched_barrier(0);
-        }
-        if constexpr (PREV) {
-          bf16x8 b1 = acc_to_b(sp, 1);
-#pragma unroll
-          for (int d = 0; d < DB; d++) dq[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ktp[1][d], b1, dq[d], 0, 0, 0);
-        }
-#pragma unroll
-        for (int m = 0; m < 2; m++)
-#pragma unroll
-          for (int d = 0; d < DB; d++) ktn[m][d] = tile_frag_t<D>(Ks[cur], sub * 32, m, d, lane);
-        __builtin_amdgcn_sched_barrier(0);
-      };
-      for (; it < n_full; it++) {
-        int cur = it & 1;
-        load_tile((it + 1) * ST);                                   // it + 1 < ntile: the diagonal tiles follow
-        if (it == 0) step(std::false_type{}, cur, 0, sA, dpA, ktA, sB, dpB, ktB);
-        else step(std::true_type{}, cur, 0, sA, dpA, ktA, sB, dpB, ktB);
-        step(std::true_type{}, cur, 1, sB, dpB, ktB, sA, dpA, ktA);
-        tile_store<D>(Ks[cur ^ 1], rk);
-        tile_store<D>(Vs[cur ^ 1], rv);
-        __syncthreads();
-      }
-      // the last sub-tile's scores and dQ
-#pragma unroll
-      for (int g = 0; g < KS; g++) scores(sB, dpB, g * SC);
-      bf16x8 b0 = acc_to_b(sB, 0), b1 = acc_to_b(sB, 1);
-#pragma unroll
-      for (int d = 0; d < DB; d++) {
-        dq[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ktB[0][d], b0, dq[d], 0, 0, 0);
-        dq[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ktB[1][d], b1, dq[d], 0, 0, 0);
-      }
-    }
-  }
-  for (; it < ntile; it++) {
+  for (int it = 0; it < ntile; it++) {
     int cur = it & 1;
-    if (it + 1 < ntile) load_tile((it + 1) * ST);
+    if (it + 1 < ntile) {
+      tile_load<D, PAD>(K, a.k_st, (it + 1) * ST, a.T, rk, a.hd);
+      tile_load<D, PAD>(V, a.v_st, (it + 1) * ST, a.T, rv, a.hd);
+    }
 #pragma unroll
     for (int sub = 0; sub < ST / 32; sub++) {
       int kv0 = it * ST + sub * 32;
       if (kv0 <= q0 + 31) {
         f32x16 s, dp;
 #pragma unroll
-        for (int e = 0; e < 16; e++) { s[e] = 0.f; dp[e] = -delta; }       // this lane's column is one query: dP - delta
+        for (int e = 0; e < 16; e++) { s[e] = 0.f; dp[e] = 0.f; }
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) {
           s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tile_frag<D>(Ks[cur], sub * 32, ks, lane), qf[ks], s, 0, 0, 0);     // S^T[kv, q]
@@ -456,7 +380,7 @@ __device__ __forceinline__ void flash_dq_bf16_body(const FlashArgs &a) {
 #pragma unroll
         for (int e = 0; e < 16; e++) {
           float ds;
-          score_bwd<CAPPED>(s[e], dp[e], krow, c1, c2, ds);
+          score_bwd<CAPPED>(s[e], dp[e] - delta, krow, c1, c2, ds);       // this lane's column is one query
           s[e] = ds;
         }
         if (edge) {
@@ -482,11 +406,16 @@ __device__ __forceinline__ void flash_dq_bf16_body(const FlashArgs &a) {
   }
   if (live) store_rows<D, PAD>((uint16_t *)a.dq + b * a.q_sb + h * a.q_sh + (int64_t)qi * a.q_st, dq, CAPPED ? 4.0f * a.scale : a.scale, lane, a.hd);
 }
+// Three waves per SIMD at head sizes up to 64 (170 registers): these kernels are bound by what the vector unit issues, and a
+// third wave keeps it fed while another waits for memory, a barrier or an MFMA chain.  That is why delta is subtracted per
+// score above instead of riding on the dP product as its starting value: the 16 registers that held it bought the third wave
+// (two waves with the products of the next sub-tile pipelined between the scores of the current one: 170 against 166 us for
+// the backward pass of a layer at B = 16, H = 12, T = 1024; 174 before either).
 template <int D, bool CAPPED>
-__global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void k_flash_dq_bf16(FlashArgs a) { flash_dq_bf16_body<D, CAPPED, false>(a); }
+__global__ __launch_bounds__(256, D <= 64 ? 3 : 1) void k_flash_dq_bf16(FlashArgs a) { flash_dq_bf16_body<D, CAPPED, false>(a); }
 // the same for tensors whose head size is smaller than D
 template <int D, bool CAPPED>
-__global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void k_flash_dq_bf16_padded(FlashArgs a) { flash_dq_bf16_body<D, CAPPED, true>(a); }
+__global__ __launch_bounds__(256, D <= 64 ? 3 : 1) void k_flash_dq_bf16_padded(FlashArgs a) { flash_dq_bf16_body<D, CAPPED, true>(a); }
 
 // ------------------------------------------------------------------------------------------ dK, dV
 template <int D, bool CAPPED, bool PAD>
@@ -604,11 +533,12 @@ __device__ __forceinline__ void flash_dkv_bf16_body(const FlashArgs &a) {
     store_rows<D, PAD>((uint16_t *)a.dv + b * a.v_sb + h * a.v_sh + (int64_t)kvi * a.v_st, dv, 1.0f, lane, a.hd);
   }
 }
+// (two waves per SIMD at head size 64: 212 registers, of which the two output accumulators are 64; three at head size 32)
 template <int D, bool CAPPED>
-__global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void k_flash_dkv_bf16(FlashArgs a) { flash_dkv_bf16_body<D, CAPPED, false>(a); }
+__global__ __launch_bounds__(256, D <= 32 ? 3 : D <= 64 ? 2 : 1) void k_flash_dkv_bf16(FlashArgs a) { flash_dkv_bf16_body<D, CAPPED, false>(a); }
 // the same for tensors whose head size is smaller than D
 template <int D, bool CAPPED>
-__global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void k_flash_dkv_bf16_padded(FlashArgs a) { flash_dkv_bf16_body<D, CAPPED, true>(a); }
+__global__ __launch_bounds__(256, D <= 32 ? 3 : D <= 64 ? 2 : 1) void k_flash_dkv_bf16_padded(FlashArgs a) { flash_dkv_bf16_body<D, CAPPED, true>(a); }
 
 // ------------------------------------------------------------------------------------------ backward, one pass over the scores
 // The dQ / dK,dV pair above evaluates every probability and every score gradient twice, and that per-score arithmetic is what
