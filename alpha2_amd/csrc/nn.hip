@@ -911,16 +911,15 @@ int32_t ah_layernorm(ah_ptr x, ah_ptr w, ah_ptr b, ah_ptr out, int64_t rows, int
   return out_dtype == AH_F32 ? launch_ln<float, float>(x, w, b, out, rows, dim, eps) : launch_ln<uint16_t, float>(x, w, b, out, rows, dim, eps);
 }
 
-#ifndef LNB_ROWS
-#define LNB_ROWS 8
-#endif
-#ifndef LNB_CAP
-#define LNB_CAP 2
-#endif
-// blocks of a LayerNorm-backward launch = rows of its partial column sums
-static int ln_bwd_blocks(int64_t rows) {
-  int64_t nblk = cdiv(rows, WPB * LNB_ROWS);      // >= 8 rows per wave amortises the partial write
-  int64_t cap = (int64_t)num_cus() * LNB_CAP;
+// Blocks of a LayerNorm-backward launch = rows of its partial column sums; a function of the shape alone, because the caller
+// sizes the partials by it (ah_layernorm_bwd_partials_bytes) and the column sums walk them.  The kernel is bound by the latency of
+// a row's loads (a wave has one row in flight beyond the one it reduces), so as many blocks as stay resident together, and no
+// more: a block beyond that runs alone in a second round.  Resident blocks per CU by registers, the least over the stream and
+// gradient types of a row length: 4 up to 512 elements, 3 up to 768, 2 beyond (16384 x 768: 21.3 us with two blocks per CU of
+// eight rows a wave, 19.5 with three of five or six, 24.4 with four; 8192 x 1024: 22.0 -> 16.1 us).
+static int ln_bwd_blocks(int64_t rows, int64_t dim) {
+  int64_t nblk = cdiv(rows, WPB * 4);             // >= 4 rows per wave amortise the partial write
+  int64_t cap = (int64_t)num_cus() * (dim <= 512 ? 4 : dim <= 768 ? 3 : 2);
   if (nblk > cap) nblk = cap;
   return nblk < 1 ? 1 : (int)nblk;
 }
@@ -970,7 +969,7 @@ int32_t ah_layernorm_bwd(ah_ptr x, ah_ptr w, ah_ptr grad_out, int32_t grad_dtype
   }
   AH_ARG(x && w && grad_out && (dx || stream_dtype == AH_BF16), "ah_layernorm_bwd: null operand");
   AH_ARG(sizeof(float) * 2 * WPB * (size_t)dim <= 160 * 1024, "ah_layernorm_bwd: dim %lld too large for the LDS column accumulators", (long long)dim);
-  const int nblk = ln_bwd_blocks(rows);
+  const int nblk = ln_bwd_blocks(rows, dim);
   float *part = (float *)scratch(sizeof(float) * 2 * (size_t)nblk * (size_t)dim);
   if (!part) return fail(AH_ERR_OOM, "ah_layernorm_bwd: no scratch");
   int32_t rc = ln_bwd_launch(x, w, grad_out, grad_dtype, residual_grad, dx, dx_bf16, part, nblk, rows, dim, eps, stream_dtype);
@@ -983,7 +982,7 @@ int32_t ah_layernorm_bwd(ah_ptr x, ah_ptr w, ah_ptr grad_out, int32_t grad_dtype
 
 int64_t ah_layernorm_bwd_partials_bytes(int64_t rows, int64_t dim) {
   if (rows <= 0 || dim <= 0 || !ready()) return 0;
-  return (int64_t)sizeof(float) * 2 * ln_bwd_blocks(rows) * dim;
+  return (int64_t)sizeof(float) * 2 * ln_bwd_blocks(rows, dim) * dim;
 }
 
 int32_t ah_layernorm_bwd_deferred(ah_ptr x, ah_ptr w, ah_ptr grad_out, int32_t grad_dtype, ah_ptr residual_grad, ah_ptr dx, ah_ptr dx_bf16,
@@ -995,7 +994,7 @@ int32_t ah_layernorm_bwd_deferred(ah_ptr x, ah_ptr w, ah_ptr grad_out, int32_t g
   AH_ARG(x && w && grad_out && (dx || stream_dtype == AH_BF16) && partials, "ah_layernorm_bwd_deferred: null operand");
   AH_ARG(partials % 4 == 0, "ah_layernorm_bwd_deferred: partials must be aligned to 4 bytes");
   AH_ARG(sizeof(float) * 2 * WPB * (size_t)dim <= 160 * 1024, "ah_layernorm_bwd_deferred: dim %lld too large for the LDS column accumulators", (long long)dim);
-  return ln_bwd_launch(x, w, grad_out, grad_dtype, residual_grad, dx, dx_bf16, dp<float>(partials), ln_bwd_blocks(rows), rows, dim, eps, stream_dtype);
+  return ln_bwd_launch(x, w, grad_out, grad_dtype, residual_grad, dx, dx_bf16, dp<float>(partials), ln_bwd_blocks(rows, dim), rows, dim, eps, stream_dtype);
 }
 
 int32_t ah_layernorm_colsums(const AhColsumJob *jobs, int32_t count) {
@@ -1009,7 +1008,7 @@ int32_t ah_layernorm_colsums(const AhColsumJob *jobs, int32_t count) {
       const AhColsumJob &q = jobs[first + i];
       AH_ARG(q.rows > 0 && q.dim > 0 && q.dim < (1ll << 31), "ah_layernorm_colsums: job %d: empty input [%lld, %lld]", first + i, (long long)q.rows, (long long)q.dim);
       AH_ARG(q.partials && q.dw && q.db, "ah_layernorm_colsums: job %d: null operand", first + i);
-      tab.j[i] = ColsumJob{dp<const float>(q.partials), dp<float>(q.dw), dp<float>(q.db), ln_bwd_blocks(q.rows), (int)q.dim, q.accumulate, 0};
+      tab.j[i] = ColsumJob{dp<const float>(q.partials), dp<float>(q.dw), dp<float>(q.db), ln_bwd_blocks(q.rows, q.dim), (int)q.dim, q.accumulate, 0};
       if (q.dim > max_dim) max_dim = q.dim;
     }
     ah::launch_kernel(k_colsum_partials_batched, dim3((unsigned)cdiv(max_dim, 32), (unsigned)n), dim3(1024), 0, tab);
